@@ -1,0 +1,77 @@
+/*
+ * llmq.h -- C ABI of libllmq_hip.so, the gfx950 (MI355X) kernels behind llm-quant's
+ * `mode="kernel"` path.
+ *
+ * Every entry point
+ *   - takes plain device pointers, sizes and a stream; no torch or HIP C++ types,
+ *   - launches on the given stream and returns without synchronising or reading back,
+ *     so a caller may record it into a HIP graph,
+ *   - allocates nothing (callers own inputs, outputs and workspaces),
+ *   - returns 0 on success, otherwise a hipError_t value (1 = invalid argument); the text
+ *     for the most recent failure on the calling thread is llmq_last_error().
+ *
+ * The reference (pjh5672/llm-quant) binds its kernels as a torch extension in
+ * llmquant/cuda/csrc/fake_quant.cpp:21-51; the functions below are what that binding's
+ * four ops reduce to once tensor checks and allocation are peeled off, plus the ops the
+ * reference still runs as PyTorch chains (activation quant, W4A8 GEMM, KV-cache quant and
+ * decode attention).
+ */
+#ifndef LLMQ_H
+#define LLMQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* A hipStream_t, passed as an opaque pointer so this header needs no HIP include. */
+typedef void* llmq_stream_t;
+
+/* Element type of activations / outputs. Values are stable: they are part of the ABI. */
+enum llmq_dtype { LLMQ_F32 = 0, LLMQ_F16 = 1, LLMQ_BF16 = 2 };
+
+/* Weight storage. INT8: one code per byte, [N, G, gs]. INT4_PACKED: two codes per byte,
+ * [N, G, gs/2], each code biased by +8, even k in the low nibble -- the bytes
+ * llmquant/packing/packing.py:20-33 writes to disk. */
+enum llmq_wformat { LLMQ_W_INT8 = 8, LLMQ_W_INT4_PACKED = 4 };
+
+#define LLMQ_GEMV_MAX_ROWS 4
+
+int llmq_abi_version(void);
+const char* llmq_last_error(void);
+
+/* Fused symmetric RTN quantize-dequantize over contiguous groups of the last axis.
+ * Replaces fake_quant_group (llmquant/cuda/csrc/fake_quant.cu:88-139), bit-exact with
+ * fake_quantize (llmquant/core/quant_ops.py:26-37):
+ *   scale = max(amax(|x|)/qmax, 1e-8); q = clamp(rint(x/scale), -qmax-1, qmax); out = q*scale
+ * x, out: n_groups*group_size elements of `dtype`; scale_or_null: n_groups fp32 or NULL.
+ * num_bits in [2, 8]. */
+int llmq_fake_quant_group(const void* x, void* out, float* scale_or_null, int64_t n_groups,
+                          int group_size, int num_bits, int dtype, llmq_stream_t stream);
+
+/* Same arithmetic, but emits the integer codes instead of the dequantized values:
+ * codes int8 [n_groups*group_size] (pack4 == 0) or nibble-packed uint8
+ * [n_groups*group_size/2] (pack4 != 0, num_bits <= 4), scale fp32 [n_groups].
+ * This is compute_scale + quantize (llmquant/core/observers.py:74-98,
+ * llmquant/core/quant_ops.py:13-19) as one pass: the activation quantizer of the A8 path
+ * (llmquant/quantizers/real.py:89-90). */
+int llmq_quant_group_codes(const void* x, void* codes, float* scale, int64_t n_groups,
+                           int group_size, int num_bits, int pack4, int dtype,
+                           llmq_stream_t stream);
+
+/* Weight-only quantized GEMV, out[m, n] = sum_g wscale[sr(n), g] * sum_{k in g} x[m, k]*q[n, g, k]
+ * with sr(n) = n / out_group when out_group > 0, else n. fp32 accumulation, result cast
+ * to `dtype`. Replaces wq_gemv (llmquant/cuda/csrc/wq_gemv.cu:134-185).
+ * x: [M, G*gs] `dtype`; qweight: see llmq_wformat; wscale: fp32 [scale_rows, G];
+ * out: [M, N] `dtype`. Any M >= 0 (rows are processed LLMQ_GEMV_MAX_ROWS at a time).
+ * gs must be a multiple of 4 (int8) or 8 (packed int4). */
+int llmq_wq_gemv(const void* x, const void* qweight, const float* wscale, void* out, int M,
+                 int N, int G, int gs, int out_group, int wformat, int dtype,
+                 llmq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLMQ_H */

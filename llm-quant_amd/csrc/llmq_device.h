@@ -1,0 +1,141 @@
+// Device-side helpers shared by the gfx950 kernels: element conversion with the rounding
+// the parity contract fixes (round-to-nearest-even everywhere), 128-bit vector access,
+// wave64 reductions, and the host-side error plumbing of the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/llmq.h"
+
+namespace llmq {
+
+constexpr int kWave = 64;
+constexpr float kScaleEps = 1e-8f;  // SCALE_EPS, llmquant/core/observers.py:5
+
+struct bf16_t { uint16_t bits; };
+struct f16_t { _Float16 v; };
+
+// ---- scalar conversions -----------------------------------------------------------------
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(f16_t v) { return static_cast<float>(v.v); }
+__device__ __forceinline__ float to_float(bf16_t v) {
+  return __builtin_bit_cast(float, static_cast<uint32_t>(v.bits) << 16);
+}
+
+__device__ __forceinline__ uint16_t bf16_bits_rne(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;  // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<uint16_t>(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ T from_float(float f);
+template <> __device__ __forceinline__ float from_float<float>(float f) { return f; }
+// fp32 -> fp16, round-to-nearest-even (v_cvt_f16_f32). The empty asm keeps the compiler from
+// folding a preceding multiply into v_fma_mixlo_f16, which adds +0 and so turns a -0 product
+// into +0.
+__device__ __forceinline__ _Float16 f16_rne(float f) {
+  asm volatile("" : "+v"(f));
+  return static_cast<_Float16>(f);
+}
+template <> __device__ __forceinline__ f16_t from_float<f16_t>(float f) { return f16_t{f16_rne(f)}; }
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
+  return bf16_t{bf16_bits_rne(f)};
+}
+
+// ---- 128-bit access ---------------------------------------------------------------------
+struct alignas(16) u32x4 { uint32_t x, y, z, w; };
+struct alignas(8) u32x2 { uint32_t x, y; };
+
+__device__ __forceinline__ u32x4 load16(const void* p) {
+  return *reinterpret_cast<const u32x4*>(p);
+}
+__device__ __forceinline__ void store16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+
+// A 16-byte packet of T, unpacked to fp32 and back.
+template <typename T> struct Pack;
+template <> struct Pack<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void unpack(u32x4 r, float* f) {
+    f[0] = __builtin_bit_cast(float, r.x); f[1] = __builtin_bit_cast(float, r.y);
+    f[2] = __builtin_bit_cast(float, r.z); f[3] = __builtin_bit_cast(float, r.w);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* f) {
+    return u32x4{__builtin_bit_cast(uint32_t, f[0]), __builtin_bit_cast(uint32_t, f[1]),
+                 __builtin_bit_cast(uint32_t, f[2]), __builtin_bit_cast(uint32_t, f[3])};
+  }
+};
+template <> struct Pack<bf16_t> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void unpack(u32x4 r, float* f) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+      f[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* f) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      w[i] = static_cast<uint32_t>(bf16_bits_rne(f[2 * i])) |
+             (static_cast<uint32_t>(bf16_bits_rne(f[2 * i + 1])) << 16);
+    }
+    return u32x4{w[0], w[1], w[2], w[3]};
+  }
+};
+template <> struct Pack<f16_t> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void unpack(u32x4 r, float* f) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w[i] & 0xffffu)));
+      f[2 * i + 1] = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w[i] >> 16)));
+    }
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* f) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint16_t lo = __builtin_bit_cast(uint16_t, f16_rne(f[2 * i]));
+      const uint16_t hi = __builtin_bit_cast(uint16_t, f16_rne(f[2 * i + 1]));
+      w[i] = static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
+    }
+    return u32x4{w[0], w[1], w[2], w[3]};
+  }
+};
+
+// ---- wave64 reductions ------------------------------------------------------------------
+// Butterfly over the low `width` lanes of each aligned lane group (width a power of two).
+template <int WIDTH> __device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+  for (int off = WIDTH / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+// ---- the quantizer, one element ------------------------------------------------------------
+// compute_scale (llmquant/core/observers.py:94-98): true IEEE division, then the eps floor.
+__device__ __forceinline__ float scale_from_amax(float amax, float qmax) {
+  return fmaxf(amax / qmax, kScaleEps);
+}
+// quantize (llmquant/core/quant_ops.py:13-19): divide, round half to even, clamp.
+__device__ __forceinline__ float quant_code(float v, float scale, float qmin, float qmax) {
+  return fminf(fmaxf(rintf(v / scale), qmin), qmax);
+}
+
+}  // namespace llmq
+
+// ---- host-side error plumbing -----------------------------------------------------------------
+namespace llmq_host {
+void set_error(const char* fmt, ...);
+int fail_invalid(const char* fmt, ...);   // records the text, returns hipErrorInvalidValue
+int check_launch(const char* what);       // hipGetLastError() -> 0 or the error, text recorded
+}  // namespace llmq_host

@@ -1,0 +1,81 @@
+"""Finding, building and loading the gfx950 kernels.
+
+Counterpart of llmquant/cuda/build.py in the reference, minus the JIT: the kernels are
+compiled ahead of time, in-tree, by the Makefile one directory up (hipcc cross-compiles
+gfx950 without a GPU), and this module only loads the result:
+
+  libllmq_hip.so      the C ABI (include/llmq.h): kernels, plain pointers, a stream
+  llmq_torch_ext.so   ATen/pybind layer exporting fake_quant_group, wq_gemv, ... on top of it
+
+There is no fallback. If the extension is missing it is built; if that fails, or there is
+no GPU, load_extension() raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import functools
+import importlib.util
+import pathlib
+import subprocess
+
+HERE = pathlib.Path(__file__).resolve().parent
+PACKAGE_ROOT = HERE.parent.parent  # the directory holding the Makefile and csrc/
+CAPI_PATH = HERE / "libllmq_hip.so"
+EXT_PATH = HERE / "llmq_torch_ext.so"
+EXT_NAME = "llmq_torch_ext"
+
+
+def build_extension(verbose: bool = False) -> None:
+    """Compile both libraries for gfx950 with the in-tree Makefile. Always recompiles."""
+    cmd = ["make", "-C", str(PACKAGE_ROOT), "-B", "-j8", "all"]
+    result = subprocess.run(cmd, capture_output=not verbose, text=True)
+    if result.returncode != 0:
+        tail = "" if verbose else (result.stdout or "")[-2000:] + (result.stderr or "")[-4000:]
+        raise RuntimeError(f"building the HIP kernels failed ({' '.join(cmd)}):\n{tail}")
+
+
+def import_extension():
+    """Load the prebuilt torch extension (no GPU needed just to load it)."""
+    import torch  # noqa: F401  -- brings in libtorch and the HIP runtime the extension links to
+
+    if not EXT_PATH.exists() or not CAPI_PATH.exists():
+        raise RuntimeError(
+            f"the HIP kernels are not built: {EXT_PATH} is missing. "
+            f"Run `make -C {PACKAGE_ROOT}` (or __graft_entry__.build())."
+        )
+    spec = importlib.util.spec_from_file_location(EXT_NAME, str(EXT_PATH))
+    module = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(module)
+    return module
+
+
+@functools.lru_cache(maxsize=1)
+def load_extension(verbose: bool = False):
+    """The extension module, loaded once per process. Raises without a GPU."""
+    import torch
+
+    if not torch.cuda.is_available():
+        raise RuntimeError("CUDA is not available; the kernels need a GPU to run")
+    if not EXT_PATH.exists() or not CAPI_PATH.exists():
+        build_extension(verbose)
+    return import_extension()
+
+
+@functools.lru_cache(maxsize=1)
+def load_capi() -> ctypes.CDLL:
+    """The C ABI library through ctypes, with argument types declared. Loading needs no GPU."""
+    import torch  # noqa: F401  -- so libamdhip64 resolves to the copy torch already loaded
+
+    if not CAPI_PATH.exists():
+        raise RuntimeError(f"{CAPI_PATH} is missing; run `make -C {PACKAGE_ROOT} capi`")
+    lib = ctypes.CDLL(str(CAPI_PATH))
+    c_int, c_i64, c_p, c_f = ctypes.c_int, ctypes.c_int64, ctypes.c_void_p, ctypes.c_float
+    lib.llmq_abi_version.restype = c_int
+    lib.llmq_last_error.restype = ctypes.c_char_p
+    lib.llmq_fake_quant_group.argtypes = [c_p, c_p, c_p, c_i64, c_int, c_int, c_int, c_p]
+    lib.llmq_quant_group_codes.argtypes = [c_p, c_p, c_p, c_i64, c_int, c_int, c_int, c_int, c_p]
+    lib.llmq_wq_gemv.argtypes = [c_p, c_p, c_p, c_p] + [c_int] * 7 + [c_p]
+    for name in ("llmq_fake_quant_group", "llmq_quant_group_codes", "llmq_wq_gemv"):
+        getattr(lib, name).restype = c_int
+    return lib

@@ -1,0 +1,110 @@
+"""mode="kernel": integer weights read straight from HBM by the gfx950 kernels.
+
+API mirror of llmquant/quantizers/kernel.py (KernelQuantLinear, pad_activation,
+KERNEL_MAX_ROWS), with one storage change: 4-bit weights live in HBM as the nibble-packed
+bytes the file format holds -- [N, G, gs/2] uint8 -- instead of one code per int8 byte, so
+a decode step streams half the bytes. `qweight` still hands back the canonical int8
+[N, G, gs] tensor for anything that wants the reference's view of the layer.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from llmquant.core.observers import group_view, pad_to_group
+from llmquant.core.scheme import QuantizationScheme
+from llmquant.hip.build import load_extension
+from llmquant.packing.packing import pack_int4, unpack_int4
+from llmquant.quantizers.real import quantize_weight
+
+#: up to this many activation rows the GEMV kernel runs; above it the weight is dequantized
+#: once and a dense matmul takes over
+KERNEL_MAX_ROWS = 4
+
+
+def pad_activation(flat: torch.Tensor, args) -> torch.Tensor:
+    """Zero-pad an activation into the same groups its weight was cut into (per head when the
+    reduction axis carries heads)."""
+    if not args.head_dim:
+        return pad_to_group(flat, args.group_size)
+    *lead, k = flat.shape
+    heads = flat.reshape(*lead, k // args.head_dim, args.head_dim)
+    return pad_to_group(heads, args.group_size).flatten(-2)
+
+
+class KernelQuantLinear(nn.Module):
+    """Linear over a canonical quantized weight: [N, groups, group_size] codes with padding
+    and head splits already applied, plus fp32 scales [scale_rows, groups]."""
+
+    def __init__(self, qweight, wscale, bias, scheme: QuantizationScheme, in_features: int):
+        super().__init__()
+        bits = scheme.weights.num_bits
+        if qweight.dtype == torch.uint8:
+            if bits != 4:
+                raise ValueError("a uint8 (nibble-packed) weight needs a 4-bit scheme")
+            stored = qweight.contiguous()
+            group_size = stored.shape[2] * 2
+        elif bits == 4:
+            stored = pack_int4(qweight)
+            group_size = qweight.shape[2]
+        else:
+            stored = qweight.contiguous()
+            group_size = qweight.shape[2]
+        self.register_buffer("qdata", stored)      # what the kernel reads
+        self.register_buffer("wscale", wscale.contiguous())  # [scale_rows, groups] fp32
+        self.bias = bias
+        self.scheme = scheme
+        self.out_features = stored.shape[0]
+        self.in_features = in_features                       # the layer's real width
+        self.padded_in_features = stored.shape[1] * group_size  # the canonical, padded one
+        self.out_group = scheme.weights.out_group or 0
+        self._packed = stored.dtype == torch.uint8
+        self._needs_padding = self.in_features != self.padded_in_features
+        self._weight_args = scheme.weights
+        # looked up once: a decode step runs ~113 of these modules
+        self._ext = load_extension()
+        self._gemv = self._ext.wq_gemv
+
+    @classmethod
+    def from_linear(cls, linear: nn.Linear, scheme: QuantizationScheme):
+        if scheme.weights is None:
+            raise ValueError("the kernel path needs a weight scheme; bf16 weights stay nn.Linear")
+        args = scheme.weights
+        codes, scale = quantize_weight(linear.weight.detach(), args)
+        canonical = group_view(codes, args.group_size, args.head_dim).contiguous()
+        scales = scale.reshape(-1, canonical.shape[1]).contiguous().float()
+        return cls(canonical, scales, linear.bias, scheme, linear.in_features)
+
+    @property
+    def qweight(self) -> torch.Tensor:
+        """Canonical int8 codes [N, groups, group_size] (unpacked on demand for 4-bit)."""
+        return unpack_int4(self.qdata) if self._packed else self.qdata
+
+    @property
+    def _broadcast_scale(self) -> torch.Tensor:
+        """[N, groups, 1] fp32: every row's scales, tiles expanded."""
+        repeat = self.out_features // self.wscale.shape[0]
+        return self.wscale.repeat_interleave(repeat, dim=0).unsqueeze(-1)
+
+    def _dequantized_weight(self, dtype):
+        """[out, padded_in] in the activation dtype, rebuilt per call and never cached."""
+        return (self.qweight * self._broadcast_scale).to(dtype).reshape(self.out_features, -1)
+
+    def forward(self, x):
+        rows = x.reshape(-1, x.shape[-1])
+        if self._needs_padding:
+            rows = pad_activation(rows, self._weight_args)
+        if rows.shape[0] <= KERNEL_MAX_ROWS:
+            out = self._gemv(rows, self.qdata, self.wscale, self.out_group)
+        else:
+            out = rows @ self._dequantized_weight(rows.dtype).T
+        if self.bias is not None:
+            out = out + self.bias.to(out.dtype)
+        return out.reshape(*x.shape[:-1], self.out_features).to(x.dtype)
+
+    def extra_repr(self):
+        a = self.scheme.input_activations
+        return (f"in_features={self.in_features}, out_features={self.out_features}, "
+                f"w{self.scheme.weights.num_bits}a{a.num_bits if a else 16}, "
+                f"group_size={self.scheme.weights.group_size}")
