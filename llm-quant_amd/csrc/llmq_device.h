@@ -138,4 +138,11 @@ namespace llmq_host {
 void set_error(const char* fmt, ...);
 int fail_invalid(const char* fmt, ...);   // records the text, returns hipErrorInvalidValue
 int check_launch(const char* what);       // hipGetLastError() -> 0 or the error, text recorded
+
+bool gemv_force_alu();
+// Matrix-core GEMV (wq_gemv_mfma.hip): whether it can take a problem, and its launch.
+bool gemv_mfma_supported(const void* x, const void* qw, const float* ws, int M, int G, int gs,
+                         int wformat);
+int gemv_mfma_launch(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
+                     int out_group, int wformat, int dtype, hipStream_t stream);
 }  // namespace llmq_host

@@ -18,6 +18,10 @@
 // Codes are converted with v_cvt_f32_ubyte*, which wants unsigned bytes: int8 is XORed
 // with 0x80 (code + 128) and int4 nibbles are used as stored (code + 8); the bias comes
 // back out as  bias * sum_{k in lane} x[k], computed once per x slice, not per row.
+#include <stdlib.h>
+
+#include <type_traits>
+
 #include "llmq_device.h"
 
 namespace {
@@ -272,6 +276,14 @@ int launch_typed(const void* x, const void* qw, const float* ws, void* out, int 
     const int rows = M - m0 < kRows ? M - m0 : kRows;
     const T* xm = static_cast<const T*>(x) + static_cast<int64_t>(m0) * k_total;
     T* om = static_cast<T*>(out) + static_cast<int64_t>(m0) * N;
+    if (llmq_host::gemv_mfma_supported(xm, qw, ws, rows, G, gs, BITS == 8 ? LLMQ_W_INT8 : LLMQ_W_INT4_PACKED) &&
+        !llmq_host::gemv_force_alu()) {
+      const int dtype = sizeof(T) == 4 ? LLMQ_F32 : (std::is_same<T, f16_t>::value ? LLMQ_F16 : LLMQ_BF16);
+      if (int rc = llmq_host::gemv_mfma_launch(xm, qw, ws, om, rows, N, G, out_group,
+                                               BITS == 8 ? LLMQ_W_INT8 : LLMQ_W_INT4_PACKED, dtype, stream))
+        return rc;
+      continue;
+    }
     if (!chunked) {
       const dim3 g((N + 3) / 4), b(256);
       hipLaunchKernelGGL((wq_gemv_scalar_kernel<T, BITS>), g, b, 0, stream, xm,
@@ -310,6 +322,18 @@ int launch_bits(const void* x, const void* qw, const float* ws, void* out, int M
 }
 
 }  // namespace
+
+namespace llmq_host {
+// LLMQ_GEMV_ALU=1 in the environment routes every GEMV to the vector-ALU kernel (used by the
+// tests to cover that kernel on shapes the matrix-core kernel would otherwise take).
+bool gemv_force_alu() {
+  static const bool forced = [] {
+    const char* v = getenv("LLMQ_GEMV_ALU");
+    return v != nullptr && v[0] == '1';
+  }();
+  return forced;
+}
+}  // namespace llmq_host
 
 extern "C" int llmq_wq_gemv(const void* x, const void* qweight, const float* wscale, void* out,
                             int M, int N, int G, int gs, int out_group, int wformat, int dtype,

@@ -1,0 +1,379 @@
+// Weight-only quantized GEMV on the int8 matrix core (v_mfma_i32_16x16x64_i8), gfx950.
+//
+//   out[m, n] = sum_g wscale[sr(n), g] * sum_{k in g} x[m, k] * q[n, g, k]        (group = 128)
+//
+// Decode reads every weight once and does two flops per code, so the kernel is judged by
+// how close it gets to streaming the codes at HBM rate. Converting codes to floats on the
+// vector ALU costs 2-3 instructions per code, which at 8 TB/s is more than the ALU has.
+// Here the codes go to the matrix core as they are:
+//
+//   * int8 codes are MFMA operand bytes straight out of the 128-bit load: no conversion.
+//   * packed int4: `w & 0x0f0f0f0f` and `(w >> 4) & 0x0f0f0f0f` are the even-k and odd-k
+//     codes (+8) as bytes: three ALU instructions per eight codes. The +8 comes back out
+//     as -8 * sum_k xdigit[k], a per-group constant that rides in as the MFMA's C operand.
+//   * the activation is made an integer once per workgroup: per (row, group) a power-of-two
+//     scale 2^-sh brings the group's abs-max into [2^21, 2^22), x*2^sh is rounded to an
+//     integer and split into three signed base-256 digits. Scaling by a power of two is
+//     exact and a bf16/fp16 element within 2^13 / 2^10 of its group's abs-max is carried
+//     without any rounding; smaller ones round at 2^-22 of the abs-max, i.e. at fp32
+//     resolution. The integer dot products are exact; the only fp32 roundings left are
+//     the per-group scale multiply and the sum over groups.
+//
+// MFMA mapping. One instruction multiplies a 16 x 64 A tile by a 64 x 16 B tile. B holds
+// 16 weight rows (lane l: row l%16, sixteen consecutive code bytes of k-block l/16), so a
+// 128-bit load per lane IS the operand and a wave-load covers 16 rows x 64 contiguous
+// bytes. A holds the activation digits, row i = 4*digit + m (m < 4 activation rows), read
+// from LDS once per workgroup and kept in registers. The int32 result has lane l holding
+// weight row l%16 and A rows 4*(l/16)..+3, i.e. lane block q = l/16 owns digit q for
+// m = 0..3: digits are recombined by scaling block q with 256^q in fp32.
+//
+// Work split: a workgroup owns 16 weight rows at a time and all of K; wave w owns groups
+// 4w..4w+3 (so K = 2048 -> 4 waves, 8192 -> 16 waves). Per row tile a wave issues 8 (int8)
+// or 4 (int4) 128-bit loads per lane plus one 128-bit load of its four scales, the next
+// tile's loads being issued before the current tile's epilogue. Partial sums meet in LDS.
+#include "llmq_device.h"
+
+namespace {
+
+using namespace llmq;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+constexpr int kGroup = 128;
+constexpr int kGW = 4;       // groups per wave
+constexpr int kDigits = 3;
+constexpr int kTileRows = 16;
+constexpr int kPlanePad = 16;
+
+struct MfmaArgs {
+  const void* x;
+  const uint8_t* qw;
+  const float* ws;
+  void* out;
+  int N, G, out_group;
+  int n_tiles;
+  int row_bytes;  // bytes of one weight row
+};
+
+template <typename T> __device__ __forceinline__ void load8(const T* p, float* f) {
+  if constexpr (Pack<T>::N == 8) {
+    Pack<T>::unpack(load16(p), f);
+  } else {
+    Pack<T>::unpack(load16(p), f);
+    Pack<T>::unpack(load16(p + 4), f + 4);
+  }
+}
+
+__device__ __forceinline__ int row16_sum(int v) {
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+// LDS carve-up, shared by host (size) and device (offsets).
+struct LdsLayout {
+  int plane;     // bytes of one digit plane of one activation row
+  int dig_off, cx_off, csum_off, part_off, total;
+  __host__ __device__ LdsLayout(int M, int G, int wk, bool need_csum) {
+    plane = G * kGroup + kPlanePad;
+    dig_off = 0;
+    cx_off = (kDigits * M * plane + 15) & ~15;
+    csum_off = cx_off + M * G * 4;
+    part_off = csum_off + (need_csum ? kDigits * M * G * 4 : 0);
+    part_off = (part_off + 15) & ~15;
+    total = part_off + 2 * wk * kDigits * M * kTileRows * 4;
+  }
+};
+
+template <typename T, int BITS, int M, int MAXT>
+__global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wv = tid / kWave;
+  const int wk = blockDim.x / kWave;
+  const int G = a.G;
+  const LdsLayout L(M, G, wk, BITS == 4);
+  int8_t* dig = reinterpret_cast<int8_t*>(smem + L.dig_off);
+  float* cxs = reinterpret_cast<float*>(smem + L.cx_off);
+  int* csum = reinterpret_cast<int*>(smem + L.csum_off);
+  float* part = reinterpret_cast<float*>(smem + L.part_off);
+
+  const int j = lane & 15;    // weight row within the tile (B column / D column)
+  const int blk = lane >> 4;  // k-block of the operand; digit block of the result
+  const int g0 = wv * kGW;
+
+  // ---- weight / scale loads of one row tile -------------------------------------------------
+  constexpr int kLoads = BITS == 8 ? 2 * kGW : kGW;
+  v4i b[kLoads];
+  float sc[kGW];
+  auto issue_loads = [&](int tile) {
+    const int n = min(tile * kTileRows + j, a.N - 1);  // rows past the end: loaded, not stored
+    const uint8_t* row = a.qw + static_cast<int64_t>(n) * a.row_bytes;
+#pragma unroll
+    for (int gi = 0; gi < kGW; ++gi) {
+      if (g0 + gi < G) {
+        if constexpr (BITS == 8) {
+          const uint8_t* p = row + (g0 + gi) * kGroup + blk * 16;
+          b[2 * gi] = *reinterpret_cast<const v4i*>(p);
+          b[2 * gi + 1] = *reinterpret_cast<const v4i*>(p + 64);
+        } else {
+          b[gi] = *reinterpret_cast<const v4i*>(row + (g0 + gi) * (kGroup / 2) + blk * 16);
+        }
+      }
+    }
+    const int srow = a.out_group > 0 ? n / a.out_group : n;
+    const float* sp = a.ws + static_cast<int64_t>(srow) * G + g0;
+    if ((G & 3) == 0) {
+      const u32x4 s4 = load16(sp);  // g0 is a multiple of 4 and so is G: aligned, in range
+      sc[0] = __builtin_bit_cast(float, s4.x); sc[1] = __builtin_bit_cast(float, s4.y);
+      sc[2] = __builtin_bit_cast(float, s4.z); sc[3] = __builtin_bit_cast(float, s4.w);
+    } else {
+#pragma unroll
+      for (int gi = 0; gi < kGW; ++gi) sc[gi] = g0 + gi < G ? sp[gi] : 0.0f;
+    }
+  };
+
+  int tile = blockIdx.x;
+  if (tile < a.n_tiles) issue_loads(tile);  // in flight while the activation is prepared
+
+  // ---- phase 1: activation -> integer digits in LDS, whole workgroup ------------------------
+  {
+    const T* __restrict__ x = static_cast<const T*>(a.x);
+    const int items = M * G * 16;  // 8 elements each; 16 consecutive items are one group
+    for (int base = 0; base < items; base += blockDim.x) {
+      const int item = base + tid;
+      const bool active = item < items;
+      const int tq = item & 15;
+      const int mg = active ? item >> 4 : 0;  // m * G + g
+      const int m = mg / G, g = mg - m * G;
+      float f[8];
+      if (active) {
+        load8<T>(x + static_cast<int64_t>(m) * G * kGroup + g * kGroup + tq * 8, f);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = 0.0f;
+      }
+      float amax = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(f[e]));
+      amax = group_max<16>(amax);
+      const int ebits = static_cast<int>((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xffu);
+      const int sh = 148 - ebits;  // amax * 2^sh in [2^21, 2^22)
+      uint32_t packed[kDigits][2] = {};
+      int dsum[kDigits] = {};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int xi = amax > 0.0f ? static_cast<int>(rintf(ldexpf(f[e], sh))) : 0;
+        const int d0 = static_cast<int8_t>(xi);
+        const int t1 = (xi - d0) >> 8;
+        const int d1 = static_cast<int8_t>(t1);
+        const int d2 = (t1 - d1) >> 8;
+        const int d[kDigits] = {d0, d1, d2};
+#pragma unroll
+        for (int q = 0; q < kDigits; ++q) {
+          dsum[q] += d[q];
+          // int8: bytes in element order. int4: even elements first (they meet the low
+          // nibbles), odd elements second.
+          const int slot = BITS == 8 ? e : (e >> 1) + 4 * (e & 1);
+          packed[q][slot >> 2] |= (static_cast<uint32_t>(d[q]) & 0xffu) << (8 * (slot & 3));
+        }
+      }
+      if (active) {
+#pragma unroll
+        for (int q = 0; q < kDigits; ++q) {
+          int8_t* plane = dig + (q * M + m) * L.plane + g * kGroup;
+          if constexpr (BITS == 8) {
+            *reinterpret_cast<u32x2*>(plane + tq * 8) = u32x2{packed[q][0], packed[q][1]};
+          } else {
+            // element k = 32*kb + 2*t + p lives at  p*64 + kb*16 + t
+            const int kb = tq >> 2, t0 = (tq & 3) * 4;
+            *reinterpret_cast<uint32_t*>(plane + kb * 16 + t0) = packed[q][0];
+            *reinterpret_cast<uint32_t*>(plane + 64 + kb * 16 + t0) = packed[q][1];
+          }
+        }
+      }
+      if constexpr (BITS == 4) {
+#pragma unroll
+        for (int q = 0; q < kDigits; ++q) {
+          const int s = row16_sum(dsum[q]);
+          if (active && tq == 0) csum[(q * M + m) * G + g] = s;
+        }
+      }
+      if (active && tq == 0) cxs[mg] = amax > 0.0f ? ldexpf(1.0f, -sh) : 0.0f;
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 2: this wave's operands and constants, into registers --------------------------
+  v4i afrag[kGW][2];
+  float fscale[kGW][M];  // 2^-sh * 256^digit of the result block this lane sits in
+  v4i cinit[kGW];
+  {
+    const int q = j >> 2, m = j & 3;  // A row j = 4*digit + m
+    const float digit_weight = blk == 0 ? 1.0f : (blk == 1 ? 256.0f : 65536.0f);
+#pragma unroll
+    for (int gi = 0; gi < kGW; ++gi) {
+      const int g = g0 + gi;
+      const bool ok = g < G;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        afrag[gi][s] = v4i{0, 0, 0, 0};
+        if (ok && q < kDigits && m < M) {
+          afrag[gi][s] = *reinterpret_cast<const v4i*>(dig + (q * M + m) * L.plane + g * kGroup + s * 64 + blk * 16);
+        }
+      }
+      cinit[gi] = v4i{0, 0, 0, 0};
+#pragma unroll
+      for (int r = 0; r < M; ++r) {
+        fscale[gi][r] = (ok && blk < kDigits) ? cxs[r * G + g] * digit_weight : 0.0f;
+        if constexpr (BITS == 4) {
+          if (ok && blk < kDigits) cinit[gi][r] = -8 * csum[(blk * M + r) * G + g];
+        }
+      }
+    }
+  }
+
+  // ---- phase 3: stream row tiles -----------------------------------------------------------
+  T* __restrict__ out = static_cast<T*>(a.out);
+  int buf = 0;
+  for (; tile < a.n_tiles; tile += gridDim.x) {
+    v4i d[kGW];
+#pragma unroll
+    for (int gi = 0; gi < kGW; ++gi) {
+      d[gi] = cinit[gi];
+      if (g0 + gi < G) {
+        if constexpr (BITS == 8) {
+          d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][0], b[2 * gi], d[gi], 0, 0, 0);
+          d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], b[2 * gi + 1], d[gi], 0, 0, 0);
+        } else {
+          const v4i lo = b[gi] & 0x0f0f0f0f;
+          const v4i hi = (b[gi] >> 4) & 0x0f0f0f0f;
+          d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][0], lo, d[gi], 0, 0, 0);
+          d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], hi, d[gi], 0, 0, 0);
+        }
+      }
+    }
+    float s_now[kGW];
+#pragma unroll
+    for (int gi = 0; gi < kGW; ++gi) s_now[gi] = sc[gi];
+    const int next = tile + gridDim.x;
+    if (next < a.n_tiles) issue_loads(next);
+
+    float acc[M];
+#pragma unroll
+    for (int r = 0; r < M; ++r) acc[r] = 0.0f;
+#pragma unroll
+    for (int gi = 0; gi < kGW; ++gi) {
+      if (g0 + gi < G) {
+#pragma unroll
+        for (int r = 0; r < M; ++r) {
+          acc[r] = fmaf(static_cast<float>(d[gi][r]), s_now[gi] * fscale[gi][r], acc[r]);
+        }
+      }
+    }
+    float* pbuf = part + buf * wk * kDigits * M * kTileRows;
+    if (blk < kDigits) {
+#pragma unroll
+      for (int r = 0; r < M; ++r) pbuf[((wv * kDigits + blk) * M + r) * kTileRows + j] = acc[r];
+    }
+    __syncthreads();
+    if (tid < M * kTileRows) {
+      const int r = tid >> 4, jj = tid & 15;
+      float total = 0.0f;
+      for (int w = 0; w < wk; ++w) {
+#pragma unroll
+        for (int q = kDigits - 1; q >= 0; --q) total += pbuf[((w * kDigits + q) * M + r) * kTileRows + jj];
+      }
+      const int n = tile * kTileRows + jj;
+      if (n < a.N) out[static_cast<int64_t>(r) * a.N + n] = from_float<T>(total);
+    }
+    buf ^= 1;
+  }
+}
+
+constexpr int kLdsDefault = 64 * 1024;   // dynamic LDS a kernel may use without opting in
+constexpr int kLdsMax = 160 * 1024;      // LDS of one gfx950 CU
+
+template <typename T, int BITS, int M, int MAXT>
+int launch_one(const MfmaArgs& a, int wk, int grid, int lds, hipStream_t stream) {
+  auto kernel = wq_gemv_mfma_kernel<T, BITS, M, MAXT>;
+  if (lds > kLdsDefault) {
+    static bool raised = false;  // per instantiation; worst case two threads both set it
+    if (!raised) {
+      const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax);
+      if (err != hipSuccess) {
+        llmq_host::set_error("raising the LDS limit failed: %s", hipGetErrorString(err));
+        return static_cast<int>(err);
+      }
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(wk * kWave), lds, stream, a);
+  return llmq_host::check_launch("wq_gemv_mfma_kernel");
+}
+
+template <typename T, int BITS, int M>
+int launch_m(const MfmaArgs& a, int wk, int grid, int lds, hipStream_t stream) {
+  if (wk <= 4) return launch_one<T, BITS, M, 256>(a, wk, grid, lds, stream);
+  if (wk <= 8) return launch_one<T, BITS, M, 512>(a, wk, grid, lds, stream);
+  return launch_one<T, BITS, M, 1024>(a, wk, grid, lds, stream);
+}
+
+template <typename T, int BITS>
+int launch_typed(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
+                 int out_group, hipStream_t stream) {
+  MfmaArgs a{};
+  a.x = x; a.qw = static_cast<const uint8_t*>(qw); a.ws = ws; a.out = out;
+  a.N = N; a.G = G; a.out_group = out_group;
+  a.n_tiles = (N + kTileRows - 1) / kTileRows;
+  a.row_bytes = G * kGroup * BITS / 8;
+  const int wk = (G + kGW - 1) / kGW;
+  const LdsLayout L(M, G, wk, BITS == 4);
+  // resident workgroups: up to 2048 threads per CU and the LDS they need
+  int per_cu = 2048 / (wk * kWave);
+  const int by_lds = kLdsMax / L.total;
+  if (per_cu > by_lds) per_cu = by_lds;
+  if (per_cu < 1) per_cu = 1;
+  int grid = 256 * per_cu;
+  if (grid > a.n_tiles) grid = a.n_tiles;
+  switch (M) {
+    case 1: return launch_m<T, BITS, 1>(a, wk, grid, L.total, stream);
+    case 2: return launch_m<T, BITS, 2>(a, wk, grid, L.total, stream);
+    case 3: return launch_m<T, BITS, 3>(a, wk, grid, L.total, stream);
+    default: return launch_m<T, BITS, 4>(a, wk, grid, L.total, stream);
+  }
+}
+
+}  // namespace
+
+namespace llmq_host {
+
+// Whether the matrix-core GEMV can take this problem (else the caller uses the ALU kernel).
+bool gemv_mfma_supported(const void* x, const void* qw, const float* ws, int M, int G, int gs,
+                         int wformat) {
+  if (gs != kGroup || G < 1 || G > 16 * kGW || M < 1 || M > 4) return false;
+  if (wformat != LLMQ_W_INT8 && wformat != LLMQ_W_INT4_PACKED) return false;
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(qw) |
+                         reinterpret_cast<uintptr_t>(ws);
+  if (bits & 15u) return false;
+  const int wk = (G + kGW - 1) / kGW;
+  return LdsLayout(M, G, wk, wformat == LLMQ_W_INT4_PACKED).total <= kLdsMax - 1024;
+}
+
+int gemv_mfma_launch(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
+                     int out_group, int wformat, int dtype, hipStream_t stream) {
+#define LLMQ_DISPATCH(T)                                                                     \
+  (wformat == LLMQ_W_INT8 ? launch_typed<T, 8>(x, qw, ws, out, M, N, G, out_group, stream)   \
+                          : launch_typed<T, 4>(x, qw, ws, out, M, N, G, out_group, stream))
+  switch (dtype) {
+    case LLMQ_F32: return LLMQ_DISPATCH(float);
+    case LLMQ_F16: return LLMQ_DISPATCH(f16_t);
+    case LLMQ_BF16: return LLMQ_DISPATCH(bf16_t);
+  }
+#undef LLMQ_DISPATCH
+  return fail_invalid("x must be float32, float16 or bfloat16, got dtype code %d", dtype);
+}
+
+}  // namespace llmq_host
