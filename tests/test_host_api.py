@@ -1,0 +1,315 @@
+"""The host-side package (llm-quant_amd/llmquant) behaves like the reference's API: the facts the
+reference's CPU tests assert (tests/test_quantization.py, test_grouping.py, test_real_quant.py,
+test_packing.py, test_kv_cache.py, test_config.py), re-asserted on this implementation, plus
+agreement of its PyTorch arithmetic with the numpy oracle."""
+
+import json
+import struct
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import llmq_oracle as oracle
+from llmquant import QuantConfig, QuantizationModifier, oneshot
+from llmquant.core import QuantizationArgs, preset_name_to_scheme
+from llmquant.core.layout import WeightLayout, layout_for
+from llmquant.core.observers import compute_scale, group_view, pad_to_group, ungroup
+from llmquant.core.quant_ops import fake_quantize, quantize
+from llmquant.core.scheme import GROUP_SIZE, PRESET_SCHEMES, QuantizationScheme
+from llmquant.packing import (pack_int4, pack_weight, read_header, read_packed, unpack_int4,
+                              unpack_weight, write_packed)
+from llmquant.packing.format import ALIGNMENT, MAGIC
+from llmquant.quantizers import (AVAILABLE_MODES, KERNEL_MAX_ROWS, FakeQuantCache, FakeQuantLinear,
+                                 RealQuantLinear, exact_fp32_matmul, make_cache_factory, pad_activation,
+                                 quant_linear_for, quantize_weight)
+
+HEADS, HEAD_DIM, K = 32, 64, 2048
+
+
+# ---- schemes and config -----------------------------------------------------------------------------
+
+def test_scheme_validation_and_presets():
+    with pytest.raises(ValueError, match="requires a positive group_size"):
+        QuantizationArgs(num_bits=4, strategy="group")
+    with pytest.raises(ValueError, match="only valid for strategy"):
+        QuantizationArgs(num_bits=4, strategy="channel", group_size=128)
+    assert set(PRESET_SCHEMES) == {"W4A8", "W8A8", "W4A16", "W8A16"}
+    assert preset_name_to_scheme("w4a8").weights.num_bits == 4
+    assert preset_name_to_scheme("W8A8").input_activations.dynamic
+    assert preset_name_to_scheme("W4A16").input_activations is None
+    with pytest.raises(ValueError):
+        preset_name_to_scheme("W3A8")
+    with pytest.raises(Exception):
+        preset_name_to_scheme("W4A8").weights.num_bits = 8  # frozen
+
+
+def test_config_axes_refusals_and_label():
+    from llmquant.core.config import normalize_dtype
+
+    assert [normalize_dtype(v) for v in (None, "bf16", "INT4", " int8 ")] == ["bf16", "bf16", "int4", "int8"]
+    with pytest.raises(ValueError, match="unknown dtype"):
+        normalize_dtype("fp8")
+    cfg = QuantConfig(attn_weight="int8", mlp_weight="int4", head_weight="int8", kv_cache="int8")
+    assert cfg.describe() == "attn-int8_mlp-int4_head-int8_act-bf16_kv-int8_g128"
+    assert cfg.kv_cache_bits == 8 and QuantConfig().kv_cache_bits is None
+    assert cfg.scheme("mlp_weight").weights.num_bits == 4 and QuantConfig().scheme("attn_weight") is None
+    assert QuantConfig(attn_weight="int4", activation="int8").scheme("attn_weight").input_activations.num_bits == 8
+    for bad in (dict(kv_cache="int4"), dict(head_weight="int4"), dict(activation="int4"), dict(group_size=0)):
+        with pytest.raises(ValueError):
+            QuantConfig(**bad)
+    with pytest.raises(ValueError, match="unknown target"):
+        cfg.scheme("kv_cache")
+    recipe = cfg.to_modifier(mode="kernel")
+    assert recipe.mode == "kernel" and recipe.kv_cache_bits == 8 and recipe.scheme is None
+
+
+class TinyConfig:
+    num_hidden_layers = 1
+    num_attention_heads = 2
+    num_key_value_heads = 2
+    hidden_size = K
+    head_dim = HEAD_DIM
+
+
+class TinyLlama(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.config = TinyConfig()
+        self.model = nn.Module()
+        self.model.layers = nn.ModuleList([nn.Module()])
+        layer = self.model.layers[0]
+        layer.self_attn = nn.Module()
+        layer.self_attn.q_proj = nn.Linear(K, 256, bias=False)
+        layer.self_attn.o_proj = nn.Linear(K, 256, bias=False)
+        layer.mlp = nn.Module()
+        layer.mlp.down_proj = nn.Linear(K, 256, bias=False)
+        self.lm_head = nn.Linear(K, GROUP_SIZE, bias=False)
+
+
+def test_routing_by_name():
+    recipe = QuantConfig(attn_weight="int4", mlp_weight="int4", activation="int8").to_modifier()
+    recipe.resolve(TinyLlama())
+    assert recipe.head_dim == HEAD_DIM
+    o = recipe.scheme_for("model.layers.0.self_attn.o_proj")
+    q = recipe.scheme_for("model.layers.0.self_attn.q_proj")
+    mlp = recipe.scheme_for("model.layers.0.mlp.down_proj")
+    assert o.weights.head_dim == HEAD_DIM and o.input_activations.head_dim == HEAD_DIM
+    assert q.weights.head_dim is None and q.weights.out_group == HEAD_DIM and mlp.weights.head_dim is None
+    assert mlp.weights.out_group is None and recipe.scheme_for("lm_head") is None
+    fused = recipe.scheme_for("model.layers.0.self_attn.qkv_proj")
+    assert fused.weights.out_group == HEAD_DIM
+    off = QuantConfig(attn_weight="int8", qkv_out_scale_per_head=False).to_modifier()
+    off.head_dim = HEAD_DIM
+    assert off.scheme_for("model.layers.0.self_attn.q_proj").weights.out_group is None
+    fixed = QuantizationModifier(attn_scheme="W4A16", head_dim=8)
+    assert fixed.resolve(TinyLlama()).head_dim == 8
+
+
+def test_apply_swaps_modules_per_mode():
+    class Tiny(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.proj = nn.Linear(GROUP_SIZE, 8, bias=False)
+            self.lm_head = nn.Linear(GROUP_SIZE, 4, bias=False)
+
+    model = QuantizationModifier(scheme="W4A8").apply(Tiny())
+    assert isinstance(model.proj, FakeQuantLinear) and isinstance(model.lm_head, nn.Linear)
+    model = QuantizationModifier(scheme="W4A8", lm_head_scheme="W8A8").apply(Tiny())
+    assert isinstance(model.lm_head, FakeQuantLinear) and model.lm_head.scheme.weights.num_bits == 8
+    model = oneshot(Tiny(), QuantizationModifier(scheme="W8A16", mode="real"))
+    assert isinstance(model.proj, RealQuantLinear)
+    assert AVAILABLE_MODES == {"fake", "real", "kernel"}
+    with pytest.raises(ValueError, match="unsupported mode"):
+        quant_linear_for("int3")
+    full = oneshot(TinyLlama(), QuantConfig(attn_weight="int8", mlp_weight="int4", head_weight="int8").to_modifier("real"))
+    assert full.model.layers[0].self_attn.o_proj.scheme.weights.head_dim == HEAD_DIM
+    assert full.lm_head.scheme.weights.num_bits == 8
+
+
+def test_kernel_mode_fails_loudly_without_a_gpu():
+    if torch.cuda.is_available():
+        pytest.skip("this is the no-GPU behaviour")
+    from llmquant.hip import load_extension
+    from llmquant.quantizers import KernelQuantLinear
+
+    with pytest.raises(RuntimeError, match="CUDA is not available"):
+        load_extension()
+    with pytest.raises(RuntimeError, match="CUDA is not available"):
+        KernelQuantLinear.from_linear(nn.Linear(128, 8, bias=False), preset_name_to_scheme("W8A16"))
+    with pytest.raises(ValueError, match="needs a weight scheme"):
+        KernelQuantLinear.from_linear(nn.Linear(128, 8), QuantizationScheme(weights=None, input_activations=None))
+
+
+# ---- layout ---------------------------------------------------------------------------------------------
+
+def test_layout_geometry():
+    o = layout_for(2048, 2048, QuantizationArgs(4, "group", group_size=128, head_dim=64))
+    assert (o.padded_in, o.in_groups, o.scale_rows, o.num_scales) == (4096, 32, 2048, 2048 * 32)
+    q = layout_for(2048, 2048, QuantizationArgs(8, "group", group_size=128, out_group=64))
+    assert (q.padded_out, q.scale_rows, q.in_groups) == (4096, 32, 16)
+    plain = WeightLayout(100, 300, 128)
+    assert (plain.padded_in, plain.padded_out, plain.weight_bytes(4)) == (384, 128, 384 * 128 // 2)
+    fused = layout_for((32 + 64) * 96, 3072, QuantizationArgs(8, "group", group_size=128, out_group=96))
+    assert fused.padded_out == 96 * 128 and fused.scale_rows == 96
+    with pytest.raises(ValueError, match="not a multiple of head_dim"):
+        WeightLayout(out_features=9217, in_features=3072, group_size=128, out_head_dim=96)
+    assert plain.bits_per_real_element(4, 4) > 4
+
+
+# ---- the PyTorch arithmetic equals the oracle's -----------------------------------------------------------
+
+@pytest.mark.parametrize("dtype,tag", [(torch.float32, "f32"), (torch.bfloat16, "bf16"), (torch.float16, "f16")])
+@pytest.mark.parametrize("kwargs", [dict(), dict(head_dim=64), dict(out_group=16)])
+def test_fake_quantize_equals_the_oracle(dtype, tag, kwargs):
+    torch.manual_seed(0)
+    x = (torch.randn(40, 320) * 2).to(dtype)
+    for bits in (4, 8):
+        args = QuantizationArgs(bits, "group", group_size=128, **kwargs)
+        got = fake_quantize(x, args)
+        want = oracle.fake_quantize(x.float().numpy(), bits, tag, "group", 128, **kwargs)
+        assert got.dtype == dtype and np.array_equal(got.float().numpy(), want)
+        assert np.array_equal(compute_scale(x, args).numpy(), oracle.compute_scale(x.float().numpy(), bits, "group", 128, **kwargs))
+
+
+def test_known_answers_hold_for_the_torch_form():
+    assert quantize(torch.tensor([0.5, 1.5, 2.5, -0.5]), torch.tensor(1.0), preset_name_to_scheme("W8A8").input_activations).tolist() == [0.0, 2.0, 2.0, -0.0]
+    x = torch.zeros(1, 128)
+    x[0, 0] = 6.2982625961
+    args = QuantizationArgs(4, "group", group_size=128)
+    assert torch.equal(compute_scale(x, args).flatten(), (x.abs().amax() / torch.tensor(7.0)).flatten())
+    w = torch.randn(8, 256)
+    assert torch.equal(fake_quantize(w, QuantizationArgs(4, "channel")), fake_quantize(w, QuantizationArgs(4, "group", group_size=256)))
+    x = torch.randn(4, 64)
+    assert torch.equal(fake_quantize(x, QuantizationArgs(4, "group", group_size=128)), fake_quantize(x, QuantizationArgs(4, "group", group_size=64)))
+    for k, padded in [(128, 128), (100, 128), (129, 256)]:
+        assert pad_to_group(torch.randn(3, k), 128).shape[-1] == padded
+    for k, hd in [(K, None), (K, HEAD_DIM), (100, None)]:
+        x = torch.randn(2, k)
+        assert torch.equal(ungroup(group_view(x, 128, hd), x.shape, 128, hd), x)
+    with pytest.raises(ValueError, match="not a multiple of head_dim"):
+        group_view(torch.randn(2, 100), 128, 64)
+
+
+@pytest.mark.parametrize("name", ["W8A16", "W8A8", "W4A16", "W4A8"])
+@pytest.mark.parametrize("kwargs", [dict(), dict(head_dim=64), dict(out_group=16)])
+def test_real_mode_module_equals_the_oracle(name, kwargs):
+    """RealQuantLinear on CPU against oracle.real_linear: equality for A8 (integer sums are
+    exact), float noise for A16 (the in-group fp32 summation order is the BLAS's)."""
+    from dataclasses import replace
+
+    torch.manual_seed(0)
+    linear = nn.Linear(512, 96, bias=True)
+    base = preset_name_to_scheme(name)
+    act = base.input_activations
+    if act is not None and "head_dim" in kwargs:
+        act = replace(act, head_dim=kwargs["head_dim"])
+    scheme = QuantizationScheme(weights=replace(base.weights, **kwargs), input_activations=act)
+    x = torch.randn(5, 512) * 2
+    got = RealQuantLinear.from_linear(linear, scheme)(x).detach().numpy()
+    canonical, scales = oracle.canonical_weight(linear.weight.detach().numpy(), base.weights.num_bits, 128, **kwargs)
+    padded = oracle.pad_activation(x.numpy(), 128, kwargs.get("head_dim"))
+    want = oracle.real_linear(padded, canonical, scales, "f32", kwargs.get("out_group"),
+                              8 if base.input_activations else None, linear.bias.detach().numpy())
+    if base.input_activations:
+        assert np.array_equal(got, want)
+    else:
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-6
+    q, scale = quantize_weight(linear.weight.detach(), scheme.weights)
+    assert q.dtype == torch.int8 and np.array_equal(q.numpy(), oracle.quantize_weight(linear.weight.detach().numpy(), base.weights.num_bits, 128, **kwargs)[0])
+
+
+def test_real_mode_module_behaviour():
+    linear = nn.Linear(512, 64, bias=True)
+    nn.init.constant_(linear.bias, 1.5)
+    module = RealQuantLinear.from_linear(linear, preset_name_to_scheme("W8A16"))
+    assert torch.allclose(module(torch.zeros(3, 512)), linear.bias.expand(3, 64))
+    assert module(torch.randn(2, 5, 512)).shape == (2, 5, 64)
+    with pytest.raises(ValueError, match="real quant needs a weight scheme"):
+        RealQuantLinear.from_linear(linear, QuantizationScheme(weights=None, input_activations=None))
+    before = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = True
+    try:
+        with exact_fp32_matmul():
+            assert torch.backends.cuda.matmul.allow_tf32 is False
+        assert torch.backends.cuda.matmul.allow_tf32 is True
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = before
+    assert KERNEL_MAX_ROWS == 4
+    flat = torch.randn(3, K)
+    assert pad_activation(flat, QuantizationArgs(8, "group", group_size=128, head_dim=64)).shape == (3, 2 * K)
+    assert pad_activation(torch.randn(3, 100), QuantizationArgs(8, "group", group_size=128)).shape == (3, 128)
+
+
+# ---- packing and the file format ---------------------------------------------------------------------------
+
+def test_nibble_packing():
+    assert int(pack_int4(torch.tensor([[-3, 5]], dtype=torch.int8))[0, 0]) == 0xD5
+    values = torch.arange(-8, 8, dtype=torch.int8).repeat(4, 1)
+    assert torch.equal(unpack_int4(pack_int4(values)), values)
+    assert pack_weight(values, 4).numel() * 2 == values.numel()
+    assert torch.equal(unpack_weight(pack_weight(values, 8), 8), values)
+    rnd = torch.randint(-8, 8, (7, 3, 64), dtype=torch.int8)
+    assert np.array_equal(pack_int4(rnd).numpy(), oracle.pack_int4(rnd.numpy()))
+    for bad in (9, -9):
+        with pytest.raises(ValueError, match=r"must be in \[-8, 7\]"):
+            pack_int4(torch.tensor([[bad, 0]], dtype=torch.int8))
+    with pytest.raises(ValueError, match="must be even"):
+        pack_int4(torch.zeros(1, 3, dtype=torch.int8))
+    for bits in (2, 16):
+        with pytest.raises(ValueError, match="unsupported num_bits"):
+            pack_weight(torch.zeros(2, 2, dtype=torch.int8), bits)
+        with pytest.raises(ValueError, match="unsupported num_bits"):
+            unpack_weight(torch.zeros(2, 2, dtype=torch.uint8), bits)
+
+
+def test_file_round_trip_alignment_and_rejections(tmp_path):
+    tensors = {
+        "packed": torch.randint(0, 255, (4, 8), dtype=torch.uint8),
+        "codes": torch.randint(-128, 127, (3, 5), dtype=torch.int8),
+        "scale": torch.rand(4, 2),
+        "norm": torch.randn(16).to(torch.bfloat16),
+    }
+    path = write_packed(tmp_path / "sub" / "w.bin", tensors, {"model_id": "test"})
+    restored, meta = read_packed(path)
+    assert meta["model_id"] == "test" and list(restored) == list(tensors)
+    for name, tensor in tensors.items():
+        assert restored[name].dtype == tensor.dtype and torch.equal(restored[name], tensor), name
+    for entry in read_header(path)["tensors"].values():
+        assert entry["offset"] % ALIGNMENT == 0
+    # byte-for-byte what the oracle's statement of the format produces
+    as_np = {n: (str(t.dtype).removeprefix("torch."), t.view(torch.uint16).numpy() if t.dtype == torch.bfloat16 else t.numpy())
+             for n, t in tensors.items()}
+    assert path.read_bytes() == oracle.packed_file_bytes(as_np, {"model_id": "test"})
+    foreign = tmp_path / "not-ours.bin"
+    foreign.write_bytes(b"SOMETHING" + b"\0" * 64)
+    with pytest.raises(ValueError, match="not a llmquant weight file"):
+        read_header(foreign)
+    header = json.dumps({"version": 999, "meta": {}, "tensors": {}}).encode()
+    future = tmp_path / "future.bin"
+    future.write_bytes(MAGIC + struct.pack("<Q", len(header)) + header)
+    with pytest.raises(ValueError, match="unsupported file version"):
+        read_header(future)
+    empty = write_packed(tmp_path / "empty.bin", {}, {"model_id": "none"})
+    assert read_packed(empty) == ({}, {"model_id": "none"})
+
+
+# ---- KV cache (fake mode) -------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_fake_quant_cache(bits):
+    torch.manual_seed(0)
+    shape = (1, 2, 5, HEAD_DIM)
+    keys, values = torch.randn(*shape), torch.randn(*shape)
+    cache = FakeQuantCache(bits)
+    ck, cv = cache.update(keys, values, 0)
+    args = QuantizationArgs(bits, "group", group_size=128, dynamic=True)
+    assert torch.equal(ck, fake_quantize(keys, args)) and torch.equal(cv, fake_quantize(values, args))
+    assert torch.equal(ck, fake_quantize(keys, QuantizationArgs(bits, "group", group_size=HEAD_DIM)))
+    assert not torch.equal(ck, keys) and cache._args(keys).group_size == 128
+    kept = ck.clone()
+    more = torch.randn(1, 2, 2, HEAD_DIM)
+    all_k, _ = cache.update(more, more.clone(), 0)
+    assert all_k.shape[2] == 7 and torch.equal(all_k[:, :, :5], kept)  # old tokens are not re-quantized
+    assert make_cache_factory(None) is None and isinstance(make_cache_factory(bits)(), FakeQuantCache)
