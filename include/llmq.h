@@ -71,6 +71,46 @@ int llmq_wq_gemv(const void* x, const void* qweight, const float* wscale, void* 
                  int N, int G, int gs, int out_group, int wformat, int dtype,
                  llmq_stream_t stream);
 
+/* KV cache, one layer. Codes are [kv_heads, t_max, head_dim] int8 (bits == 8) or
+ * [kv_heads, t_max, head_dim/2] nibble-packed uint8 (bits == 4); scales are fp32
+ * [kv_heads, t_max]: one scale per token per head, which is what FakeQuantCache's
+ * group-128 rule gives for head_dim <= 128 (llmquant/quantizers/fake.py:39-55).
+ *
+ * llmq_kv_append quantizes `n_new` tokens of K and V ([kv_heads, n_new, head_dim] `dtype`,
+ * token stride given in elements so a [heads, T, D] view of a larger tensor works) and
+ * writes them at positions *pos_dev .. *pos_dev + n_new - 1, where pos_dev is a device
+ * int32 (read by the kernel, never by the host). When dq_k / dq_v are non-NULL the
+ * dequantized values (dtype)(q*scale) are also written there ([kv_heads, n_new, head_dim]),
+ * which is what FakeQuantCache.update hands back to attention during prefill. */
+int llmq_kv_append(const void* k_new, const void* v_new, int64_t head_stride,
+                   int64_t token_stride, void* k_codes, void* v_codes, float* k_scale,
+                   float* v_scale, void* dq_k_or_null, void* dq_v_or_null,
+                   const int32_t* pos_dev, int n_new, int kv_heads, int head_dim, int t_max,
+                   int bits, int dtype, llmq_stream_t stream);
+
+/* Dequantize positions 0 .. n_tokens-1 of one layer's cache to [kv_heads, n_tokens, head_dim]
+ * `dtype`: (dtype)(code * scale), the tensor FakeQuantCache.update returns
+ * (llmquant/quantizers/fake.py:52-55) when attention is not run by the fused decode kernel. */
+int llmq_kv_dequant(const void* codes, const float* scale, void* out, int kv_heads, int head_dim,
+                    int t_max, int n_tokens, int bits, int dtype, llmq_stream_t stream);
+
+/* Single-token grouped-query attention over the quantized cache: for each query head h
+ * (kv head h / (q_heads/kv_heads)), softmax(q_h . K^T * sm_scale) V over tokens
+ * 0 .. *len_dev - 1, with K and V dequantized on read as (dtype)(code*scale) to keep the
+ * rounding point of FakeQuantCache. Scores and softmax in fp32.
+ * q: [q_heads, head_dim] `dtype`; out: [q_heads, head_dim] `dtype`.
+ * head_dim 64 or 128; q_heads / kv_heads in {1, 2, 4, 8}.
+ * workspace: at least llmq_kv_decode_workspace_floats(q_heads, head_dim, t_max) floats, zeroed once
+ * by the caller before first use (it holds arrival counters that each launch leaves at zero);
+ * launches that share a workspace must not overlap. There is no counterpart kernel in the
+ * reference: it runs HF attention over the dequantized bf16 cache (llmquant/quantizers/fake.py:39-55). */
+size_t llmq_kv_decode_workspace_floats(int q_heads, int head_dim, int t_max);
+int llmq_kv_decode_attention(const void* q, const void* k_codes, const void* v_codes,
+                             const float* k_scale, const float* v_scale, void* out,
+                             float* workspace, const int32_t* len_dev, float sm_scale,
+                             int q_heads, int kv_heads, int head_dim, int t_max, int bits,
+                             int dtype, llmq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,436 @@
+// Quantized KV cache for decode, gfx950: quantize-on-append, dequantize-on-read inside
+// single-token grouped-query attention.
+//
+// What is stored is what FakeQuantCache (llmquant/quantizers/fake.py:39-55) computes and then
+// throws away: the integer codes and the one fp32 scale per (token, head) that its group-128
+// rule yields for head_dim <= 128. Reading a cached element back gives (dtype)(code * scale),
+// the very value the reference keeps in its bf16 cache, so attention sees the same K and V;
+// only the bytes in HBM differ: head_dim (+4) per token-head instead of 2*head_dim.
+//
+// Layout, one layer: codes [kv_heads, t_max, head_dim] int8 (8 bit) or
+// [kv_heads, t_max, head_dim/2] nibble-packed uint8 (4 bit, +8 bias, even index low), scales
+// [kv_heads, t_max] fp32. The write position and the valid length live on the device, so a
+// decode step is the same sequence of launches every token and can be replayed from a graph.
+#include "llmq_device.h"
+
+namespace {
+
+using namespace llmq;
+
+// ---- append -------------------------------------------------------------------------------------
+// One wave per (tensor, head, token): lane l holds elements l and l + 64 of the head vector.
+template <typename T, int BITS>
+__global__ __launch_bounds__(256) void kv_append_kernel(
+    const T* __restrict__ k_new, const T* __restrict__ v_new, const int64_t head_stride,
+    const int64_t token_stride, uint8_t* __restrict__ k_codes, uint8_t* __restrict__ v_codes,
+    float* __restrict__ k_scale, float* __restrict__ v_scale, T* __restrict__ dq_k, T* __restrict__ dq_v,
+    const int32_t* __restrict__ pos_dev, const int n_new, const int kv_heads, const int head_dim,
+    const int t_max) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
+  const int64_t per_tensor = static_cast<int64_t>(kv_heads) * n_new;
+  if (wave >= 2 * per_tensor) return;  // whole waves leave together; no barrier follows
+  const bool is_v = wave >= per_tensor;
+  const int64_t idx = is_v ? wave - per_tensor : wave;
+  const int head = static_cast<int>(idx / n_new);
+  const int tok = static_cast<int>(idx - static_cast<int64_t>(head) * n_new);
+  const int pos = pos_dev[0] + tok;
+  if (pos < 0 || pos >= t_max) return;
+
+  const T* src = (is_v ? v_new : k_new) + head * head_stride + tok * token_stride;
+  const float qmax = static_cast<float>((1 << (BITS - 1)) - 1);
+  const float qmin = -qmax - 1.0f;
+  float f[2];
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    const int d = lane + e * kWave;
+    f[e] = d < head_dim ? to_float(src[d]) : 0.0f;
+  }
+  float amax = fmaxf(fabsf(f[0]), fabsf(f[1]));
+  amax = group_max<kWave>(amax);
+  const float scale = scale_from_amax(amax, qmax);
+  const int64_t slot = static_cast<int64_t>(head) * t_max + pos;
+  if (lane == 0) (is_v ? v_scale : k_scale)[slot] = scale;
+  uint8_t* codes = is_v ? v_codes : k_codes;
+  T* dq = is_v ? dq_v : dq_k;
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    const int d = lane + e * kWave;
+    const float q = quant_code(f[e], scale, qmin, qmax);
+    if (dq != nullptr && d < head_dim) {
+      dq[(static_cast<int64_t>(head) * n_new + tok) * head_dim + d] = from_float<T>(q * scale);
+    }
+    const int code = static_cast<int>(q);
+    if constexpr (BITS == 8) {
+      if (d < head_dim) codes[slot * head_dim + d] = static_cast<uint8_t>(code);
+    } else {
+      // pair the even lane's code with its odd neighbour's
+      const int mine = (code + 8) & 0xf;
+      const int other = __shfl_xor(mine, 1, kWave);
+      if ((lane & 1) == 0 && d < head_dim) {
+        codes[slot * (head_dim / 2) + d / 2] = static_cast<uint8_t>(mine | (other << 4));
+      }
+    }
+  }
+}
+
+// ---- dequantize a range of the cache (what update() hands back outside of decode) ---------------
+template <typename T, int BITS>
+__global__ __launch_bounds__(256) void kv_dequant_kernel(
+    const uint8_t* __restrict__ codes, const float* __restrict__ scale, T* __restrict__ out,
+    const int kv_heads, const int head_dim, const int t_max, const int n_tokens) {
+  const int64_t total = static_cast<int64_t>(kv_heads) * n_tokens * head_dim;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int d = static_cast<int>(i % head_dim);
+    const int64_t ht = i / head_dim;
+    const int t = static_cast<int>(ht % n_tokens);
+    const int h = static_cast<int>(ht / n_tokens);
+    const int64_t slot = static_cast<int64_t>(h) * t_max + t;
+    int code;
+    if constexpr (BITS == 8) {
+      code = static_cast<int8_t>(codes[slot * head_dim + d]);
+    } else {
+      const uint8_t byte = codes[slot * (head_dim / 2) + d / 2];
+      code = static_cast<int>((d & 1) ? (byte >> 4) : (byte & 0xf)) - 8;
+    }
+    out[i] = from_float<T>(static_cast<float>(code) * scale[slot]);
+  }
+}
+
+// ---- decode attention ------------------------------------------------------------------------------
+// Grid (splits, kv_heads). A workgroup owns one kv head and a fixed slice of token positions,
+// and serves all `REP` query heads of that kv head, so codes are read once. Inside a wave a
+// quad of lanes shares a token: lane (tk = lane / 4, dq = lane % 4) loads a quarter of the
+// token's K row and V row (16-byte loads; 16 tokens = 1 KiB contiguous per wave-load for
+// head_dim 64 int8). Every quad runs its own online softmax over its tokens (no cross-lane
+// traffic in the loop besides the 2-step quad sum of the score); quads, waves and finally
+// splits are merged with the usual (max, sum, weighted output) rule. The last workgroup of a
+// kv head to arrive (device counter, reset by that workgroup) merges the splits and writes
+// the output, so the whole attention is one launch.
+constexpr int kAttnThreads = 256;
+constexpr int kAttnWaves = kAttnThreads / kWave;
+constexpr int kTokPerIter = 16;  // tokens one wave handles per step (a quad per token)
+
+template <typename T> __device__ __forceinline__ float round_through(float v);
+template <> __device__ __forceinline__ float round_through<float>(float v) { return v; }
+template <> __device__ __forceinline__ float round_through<bf16_t>(float v) {
+  return __builtin_bit_cast(float, static_cast<uint32_t>(bf16_bits_rne(v)) << 16);
+}
+template <> __device__ __forceinline__ float round_through<f16_t>(float v) {
+  return static_cast<float>(f16_rne(v));
+}
+
+// 16 (DPL = 16) codes of one token quarter as floats
+template <int BITS, int DPL>
+__device__ __forceinline__ void load_codes(const uint8_t* row, int dq, float* c) {
+  if constexpr (BITS == 8) {
+#pragma unroll
+    for (int p = 0; p < DPL / 16; ++p) {
+      const u32x4 w = load16(row + dq * DPL + p * 16);
+      const uint32_t d[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) c[p * 16 + 4 * i + b] = static_cast<float>(static_cast<int8_t>(d[i] >> (8 * b)));
+    }
+  } else {
+#pragma unroll
+    for (int p = 0; p < DPL / 16; ++p) {
+      const u32x2 w = *reinterpret_cast<const u32x2*>(row + (dq * DPL + p * 16) / 2);
+      const uint32_t d[2] = {w.x, w.y};
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int b = 0; b < 8; ++b) c[p * 16 + 8 * i + b] = static_cast<float>(static_cast<int>((d[i] >> (4 * b)) & 0xfu) - 8);
+    }
+  }
+}
+
+template <typename T, int BITS, int D, int REP>
+__global__ __launch_bounds__(kAttnThreads) void kv_decode_attn_kernel(
+    const T* __restrict__ q, const uint8_t* __restrict__ k_codes, const uint8_t* __restrict__ v_codes,
+    const float* __restrict__ k_scale, const float* __restrict__ v_scale, T* __restrict__ out,
+    float* __restrict__ ws_part, int* __restrict__ ws_count, const int32_t* __restrict__ len_dev,
+    const float sm_scale_log2, const int t_max, const int chunk) {
+  constexpr int DPL = D / 4;           // head-dim elements per lane
+  constexpr int ROWB = BITS == 8 ? D : D / 2;
+  constexpr int REC = D + 2;           // floats per partial record: max, sum, weighted output
+  __shared__ float s_rec[kAttnWaves][REP][REC];
+  __shared__ int s_last;
+
+  const int split = blockIdx.x, n_splits = gridDim.x, kvh = blockIdx.y;
+  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+  const int tk = lane >> 2, dq = lane & 3;
+  const int len = min(len_dev[0], t_max);
+  const int t_begin = split * chunk, t_end = min(t_begin + chunk, len);
+
+  // this lane's quarter of each query head, pre-scaled so exp2 can be used
+  float qf[REP][DPL];
+#pragma unroll
+  for (int h = 0; h < REP; ++h)
+#pragma unroll
+    for (int i = 0; i < DPL; ++i)
+      qf[h][i] = to_float(q[(static_cast<int64_t>(kvh) * REP + h) * D + dq * DPL + i]) * sm_scale_log2;
+
+  float m[REP], l[REP], o[REP][DPL];
+#pragma unroll
+  for (int h = 0; h < REP; ++h) {
+    m[h] = -INFINITY;
+    l[h] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) o[h][i] = 0.0f;
+  }
+
+  const uint8_t* kbase = k_codes + static_cast<int64_t>(kvh) * t_max * ROWB;
+  const uint8_t* vbase = v_codes + static_cast<int64_t>(kvh) * t_max * ROWB;
+  const float* ksc = k_scale + static_cast<int64_t>(kvh) * t_max;
+  const float* vsc = v_scale + static_cast<int64_t>(kvh) * t_max;
+  for (int t0 = t_begin + wv * kTokPerIter; t0 < t_end; t0 += kAttnWaves * kTokPerIter) {
+    const int t = t0 + tk;
+    const bool ok = t < t_end;
+    const int tc = ok ? t : t_end - 1;  // clamp: loads stay in range, result dropped
+    float kc[DPL], vc[DPL];
+    load_codes<BITS, DPL>(kbase + static_cast<int64_t>(tc) * ROWB, dq, kc);
+    load_codes<BITS, DPL>(vbase + static_cast<int64_t>(tc) * ROWB, dq, vc);
+    const float ks = ksc[tc], vs = vsc[tc];
+    float s[REP];
+#pragma unroll
+    for (int h = 0; h < REP; ++h) s[h] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+      const float kd = round_through<T>(kc[i] * ks);  // the value the reference's cache holds
+#pragma unroll
+      for (int h = 0; h < REP; ++h) s[h] = fmaf(qf[h][i], kd, s[h]);
+    }
+#pragma unroll
+    for (int h = 0; h < REP; ++h) {
+      s[h] += __shfl_xor(s[h], 1, kWave);
+      s[h] += __shfl_xor(s[h], 2, kWave);
+    }
+    if (ok) {
+      float p[REP];
+#pragma unroll
+      for (int h = 0; h < REP; ++h) {
+        const float m_new = fmaxf(m[h], s[h]);
+        const float corr = exp2f(m[h] - m_new);  // exp2f(-inf) == 0 on the first token
+        p[h] = exp2f(s[h] - m_new);
+        l[h] = l[h] * corr + p[h];
+        m[h] = m_new;
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) o[h][i] *= corr;
+      }
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        const float vd = round_through<T>(vc[i] * vs);
+#pragma unroll
+        for (int h = 0; h < REP; ++h) o[h][i] = fmaf(p[h], vd, o[h][i]);
+      }
+    }
+  }
+
+  // ---- merge the 16 quads of the wave (lanes with the same dq): xor 4, 8, 16, 32 -------------------
+#pragma unroll
+  for (int off = 4; off < kWave; off <<= 1) {
+#pragma unroll
+    for (int h = 0; h < REP; ++h) {
+      const float m_o = __shfl_xor(m[h], off, kWave);
+      const float l_o = __shfl_xor(l[h], off, kWave);
+      const float m_new = fmaxf(m[h], m_o);
+      const float a = m[h] == -INFINITY ? 0.0f : exp2f(m[h] - m_new);
+      const float b = m_o == -INFINITY ? 0.0f : exp2f(m_o - m_new);
+      l[h] = l[h] * a + l_o * b;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        const float o_o = __shfl_xor(o[h][i], off, kWave);
+        o[h][i] = o[h][i] * a + o_o * b;
+      }
+      m[h] = m_new;
+    }
+  }
+  if (tk == 0) {
+#pragma unroll
+    for (int h = 0; h < REP; ++h) {
+      if (dq == 0) {
+        s_rec[wv][h][0] = m[h];
+        s_rec[wv][h][1] = l[h];
+      }
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) s_rec[wv][h][2 + dq * DPL + i] = o[h][i];
+    }
+  }
+  __syncthreads();
+
+  // ---- merge the waves; thread (h, d) for d < D ------------------------------------------------------
+  float* my_part = ws_part + ((static_cast<int64_t>(kvh) * n_splits + split) * REP) * REC;
+  for (int item = threadIdx.x; item < REP * D; item += kAttnThreads) {
+    const int h = item / D, d = item % D;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kAttnWaves; ++w) mm = fmaxf(mm, s_rec[w][h][0]);
+    float ll = 0.0f, oo = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kAttnWaves; ++w) {
+      const float a = s_rec[w][h][0] == -INFINITY ? 0.0f : exp2f(s_rec[w][h][0] - mm);
+      ll += s_rec[w][h][1] * a;
+      oo += s_rec[w][h][2 + d] * a;
+    }
+    my_part[h * REC + 2 + d] = oo;
+    if (d == 0) {
+      my_part[h * REC] = mm;
+      my_part[h * REC + 1] = ll;
+    }
+  }
+
+  // ---- last workgroup of this kv head merges the splits ------------------------------------------------
+  __threadfence();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int arrived = atomicAdd(&ws_count[kvh], 1);
+    s_last = arrived == n_splits - 1;
+  }
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
+  const float* parts = ws_part + static_cast<int64_t>(kvh) * n_splits * REP * REC;
+  for (int item = threadIdx.x; item < REP * D; item += kAttnThreads) {
+    const int h = item / D, d = item % D;
+    float mm = -INFINITY;
+    for (int s2 = 0; s2 < n_splits; ++s2) mm = fmaxf(mm, parts[(s2 * REP + h) * REC]);
+    float ll = 0.0f, oo = 0.0f;
+    for (int s2 = 0; s2 < n_splits; ++s2) {
+      const float ms = parts[(s2 * REP + h) * REC];
+      const float a = ms == -INFINITY ? 0.0f : exp2f(ms - mm);
+      ll += parts[(s2 * REP + h) * REC + 1] * a;
+      oo += parts[(s2 * REP + h) * REC + 2 + d] * a;
+    }
+    out[(static_cast<int64_t>(kvh) * REP + h) * D + d] = from_float<T>(ll > 0.0f ? oo / ll : 0.0f);
+  }
+  if (threadIdx.x == 0) ws_count[kvh] = 0;  // ready for the next launch
+}
+
+int splits_for(int t_max) {
+  int s = (t_max + 63) / 64;
+  if (s > 64) s = 64;
+  return s < 1 ? 1 : s;
+}
+
+template <typename T, int BITS, int D>
+int launch_attn_rep(int rep, dim3 grid, hipStream_t stream, const T* q, const uint8_t* kc,
+                    const uint8_t* vc, const float* ks, const float* vs, T* out, float* part, int* count,
+                    const int32_t* len_dev, float scale_log2, int t_max, int chunk) {
+#define LLMQ_ATTN(R)                                                                            \
+  case R:                                                                                       \
+    hipLaunchKernelGGL((kv_decode_attn_kernel<T, BITS, D, R>), grid, dim3(kAttnThreads), 0, stream, q, kc, \
+                       vc, ks, vs, out, part, count, len_dev, scale_log2, t_max, chunk);        \
+    break;
+  switch (rep) {
+    LLMQ_ATTN(1) LLMQ_ATTN(2) LLMQ_ATTN(4) LLMQ_ATTN(8)
+    default:
+      return llmq_host::fail_invalid("q_heads / kv_heads must be 1, 2, 4 or 8, got %d", rep);
+  }
+#undef LLMQ_ATTN
+  return llmq_host::check_launch("kv_decode_attn_kernel");
+}
+
+}  // namespace
+
+extern "C" size_t llmq_kv_decode_workspace_floats(int q_heads, int head_dim, int t_max) {
+  // partial records, then one int32 counter per head (sized by q_heads >= kv_heads)
+  return static_cast<size_t>(q_heads) * splits_for(t_max) * (head_dim + 2) + q_heads;
+}
+
+extern "C" int llmq_kv_append(const void* k_new, const void* v_new, int64_t head_stride,
+                              int64_t token_stride, void* k_codes, void* v_codes, float* k_scale,
+                              float* v_scale, void* dq_k_or_null, void* dq_v_or_null,
+                              const int32_t* pos_dev, int n_new, int kv_heads, int head_dim, int t_max,
+                              int bits, int dtype, llmq_stream_t stream) {
+  if (bits != 8 && bits != 4) return llmq_host::fail_invalid("KV cache bits must be 8 or 4, got %d", bits);
+  if (head_dim < 2 || head_dim > 128 || (head_dim & 1))
+    return llmq_host::fail_invalid("head_dim must be even and in [2, 128], got %d", head_dim);
+  if (n_new < 0 || kv_heads < 0 || t_max < 0) return llmq_host::fail_invalid("negative size");
+  if (n_new == 0 || kv_heads == 0) return 0;
+  if (!k_new || !v_new || !k_codes || !v_codes || !k_scale || !v_scale || !pos_dev)
+    return llmq_host::fail_invalid("null tensor pointer");
+  const int64_t waves = 2LL * kv_heads * n_new;
+  const dim3 grid(static_cast<unsigned>((waves + 3) / 4)), block(256);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define LLMQ_APPEND(T, B)                                                                       \
+  hipLaunchKernelGGL((kv_append_kernel<T, B>), grid, block, 0, s, static_cast<const T*>(k_new), \
+                     static_cast<const T*>(v_new), head_stride, token_stride,                   \
+                     static_cast<uint8_t*>(k_codes), static_cast<uint8_t*>(v_codes), k_scale, v_scale, \
+                     static_cast<T*>(dq_k_or_null), static_cast<T*>(dq_v_or_null), pos_dev, n_new, \
+                     kv_heads, head_dim, t_max)
+  switch (dtype) {
+    case LLMQ_F32: if (bits == 8) LLMQ_APPEND(float, 8); else LLMQ_APPEND(float, 4); break;
+    case LLMQ_F16: if (bits == 8) LLMQ_APPEND(f16_t, 8); else LLMQ_APPEND(f16_t, 4); break;
+    case LLMQ_BF16: if (bits == 8) LLMQ_APPEND(bf16_t, 8); else LLMQ_APPEND(bf16_t, 4); break;
+    default: return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+  }
+#undef LLMQ_APPEND
+  return llmq_host::check_launch("kv_append_kernel");
+}
+
+extern "C" int llmq_kv_dequant(const void* codes, const float* scale, void* out, int kv_heads,
+                               int head_dim, int t_max, int n_tokens, int bits, int dtype,
+                               llmq_stream_t stream) {
+  if (bits != 8 && bits != 4) return llmq_host::fail_invalid("KV cache bits must be 8 or 4, got %d", bits);
+  if (n_tokens < 0 || n_tokens > t_max) return llmq_host::fail_invalid("n_tokens %d outside [0, %d]", n_tokens, t_max);
+  const int64_t total = static_cast<int64_t>(kv_heads) * n_tokens * head_dim;
+  if (total == 0) return 0;
+  if (!codes || !scale || !out) return llmq_host::fail_invalid("null tensor pointer");
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  const dim3 grid(static_cast<unsigned>(blocks)), block(256);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define LLMQ_DQ(T, B)                                                                           \
+  hipLaunchKernelGGL((kv_dequant_kernel<T, B>), grid, block, 0, s, static_cast<const uint8_t*>(codes), \
+                     scale, static_cast<T*>(out), kv_heads, head_dim, t_max, n_tokens)
+  switch (dtype) {
+    case LLMQ_F32: if (bits == 8) LLMQ_DQ(float, 8); else LLMQ_DQ(float, 4); break;
+    case LLMQ_F16: if (bits == 8) LLMQ_DQ(f16_t, 8); else LLMQ_DQ(f16_t, 4); break;
+    case LLMQ_BF16: if (bits == 8) LLMQ_DQ(bf16_t, 8); else LLMQ_DQ(bf16_t, 4); break;
+    default: return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+  }
+#undef LLMQ_DQ
+  return llmq_host::check_launch("kv_dequant_kernel");
+}
+
+extern "C" int llmq_kv_decode_attention(const void* q, const void* k_codes, const void* v_codes,
+                                        const float* k_scale, const float* v_scale, void* out,
+                                        float* workspace, const int32_t* len_dev, float sm_scale,
+                                        int q_heads, int kv_heads, int head_dim, int t_max, int bits,
+                                        int dtype, llmq_stream_t stream) {
+  if (bits != 8 && bits != 4) return llmq_host::fail_invalid("KV cache bits must be 8 or 4, got %d", bits);
+  if (head_dim != 64 && head_dim != 128) return llmq_host::fail_invalid("head_dim must be 64 or 128, got %d", head_dim);
+  if (kv_heads <= 0 || q_heads <= 0 || q_heads % kv_heads) return llmq_host::fail_invalid("q_heads %d must be a positive multiple of kv_heads %d", q_heads, kv_heads);
+  if (t_max <= 0) return llmq_host::fail_invalid("t_max must be positive, got %d", t_max);
+  if (!q || !k_codes || !v_codes || !k_scale || !v_scale || !out || !workspace || !len_dev)
+    return llmq_host::fail_invalid("null tensor pointer");
+  if ((reinterpret_cast<uintptr_t>(k_codes) | reinterpret_cast<uintptr_t>(v_codes)) & 15u)
+    return llmq_host::fail_invalid("cache code pointers must be 16-byte aligned");
+  const int rep = q_heads / kv_heads;
+  const int splits = splits_for(t_max);
+  const int chunk = (t_max + splits - 1) / splits;
+  float* part = workspace;
+  int* count = reinterpret_cast<int*>(workspace + static_cast<size_t>(q_heads) * splits * (head_dim + 2));
+  const dim3 grid(splits, kv_heads);
+  const float scale_log2 = sm_scale * 1.4426950408889634f;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint8_t* kc = static_cast<const uint8_t*>(k_codes);
+  const uint8_t* vc = static_cast<const uint8_t*>(v_codes);
+#define LLMQ_GO(T, B, D)                                                                        \
+  return launch_attn_rep<T, B, D>(rep, grid, s, static_cast<const T*>(q), kc, vc, k_scale, v_scale, \
+                                  static_cast<T*>(out), part, count, len_dev, scale_log2, t_max, chunk)
+#define LLMQ_BD(T)                                                                              \
+  if (bits == 8) { if (head_dim == 64) LLMQ_GO(T, 8, 64); else LLMQ_GO(T, 8, 128); }            \
+  else { if (head_dim == 64) LLMQ_GO(T, 4, 64); else LLMQ_GO(T, 4, 128); }
+  switch (dtype) {
+    case LLMQ_F32: LLMQ_BD(float)
+    case LLMQ_F16: LLMQ_BD(f16_t)
+    case LLMQ_BF16: LLMQ_BD(bf16_t)
+  }
+#undef LLMQ_BD
+#undef LLMQ_GO
+  return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+}

@@ -136,6 +136,118 @@ at::Tensor wq_gemv(const at::Tensor& x, const at::Tensor& qweight, const at::Ten
   return out;
 }
 
+// ---- quantized KV cache -------------------------------------------------------------------------------
+// Cache tensors of one layer: codes [kv_heads, t_max, head_dim] int8 or [kv_heads, t_max,
+// head_dim / 2] uint8, scales [kv_heads, t_max] fp32. `position` is a device int32 tensor.
+
+struct CacheGeometry {
+  int kv_heads, t_max, head_dim, bits;
+};
+
+CacheGeometry cache_geometry(const at::Tensor& codes, const at::Tensor& scale, const char* what) {
+  TORCH_CHECK(codes.is_cuda() && scale.is_cuda(), what, " cache tensors must be CUDA");
+  TORCH_CHECK(codes.dim() == 3 && codes.is_contiguous(), what, " codes must be contiguous [kv_heads, t_max, head_dim]");
+  const bool packed = codes.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || codes.scalar_type() == at::kChar, what, " codes must be int8, or uint8 for 4-bit");
+  TORCH_CHECK(scale.scalar_type() == at::kFloat && scale.is_contiguous() && scale.dim() == 2 &&
+                  scale.size(0) == codes.size(0) && scale.size(1) == codes.size(1),
+              what, " scales must be contiguous float32 [kv_heads, t_max]");
+  return {static_cast<int>(codes.size(0)), static_cast<int>(codes.size(1)),
+          static_cast<int>(packed ? codes.size(2) * 2 : codes.size(2)), packed ? 4 : 8};
+}
+
+void check_position(const at::Tensor& position) {
+  TORCH_CHECK(position.is_cuda() && position.scalar_type() == at::kInt && position.numel() >= 1,
+              "position must be a CUDA int32 tensor");
+}
+
+// key / value: [kv_heads, n_new, head_dim] views (last axis contiguous, both with the same
+// strides). Returns the dequantized new tokens when asked, else two empty tensors.
+std::tuple<at::Tensor, at::Tensor> kv_append(const at::Tensor& key, const at::Tensor& value,
+                                             at::Tensor& k_codes, at::Tensor& v_codes, at::Tensor& k_scale,
+                                             at::Tensor& v_scale, const at::Tensor& position,
+                                             bool return_dequantized) {
+  TORCH_CHECK(key.is_cuda() && value.is_cuda(), "key and value must be CUDA tensors");
+  TORCH_CHECK(key.dim() == 3 && value.sizes() == key.sizes() && value.strides() == key.strides() &&
+                  key.scalar_type() == value.scalar_type(),
+              "key and value must be [kv_heads, n_new, head_dim] with equal shapes, strides and dtypes");
+  TORCH_CHECK(key.stride(2) == 1 || key.size(2) == 1, "the head_dim axis must be contiguous");
+  const int dtype = dtype_code(key, "key");
+  const CacheGeometry g = cache_geometry(k_codes, k_scale, "key");
+  const CacheGeometry gv = cache_geometry(v_codes, v_scale, "value");
+  TORCH_CHECK(g.kv_heads == gv.kv_heads && g.t_max == gv.t_max && g.head_dim == gv.head_dim && g.bits == gv.bits,
+              "key and value caches differ in geometry");
+  TORCH_CHECK(key.size(0) == g.kv_heads && key.size(2) == g.head_dim, "key is [", key.size(0), ", ",
+              key.size(1), ", ", key.size(2), "] but the cache holds ", g.kv_heads, " heads of ", g.head_dim);
+  check_position(position);
+  const int64_t n_new = key.size(1);
+  at::Tensor dq_k = at::empty({0}, key.options()), dq_v = at::empty({0}, key.options());
+  if (return_dequantized) {
+    dq_k = at::empty({g.kv_heads, n_new, g.head_dim}, key.options());
+    dq_v = at::empty({g.kv_heads, n_new, g.head_dim}, key.options());
+  }
+  if (n_new == 0) return std::make_tuple(dq_k, dq_v);
+  const c10::OptionalDeviceGuard guard(at::device_of(key));
+  check_rc(llmq_kv_append(key.const_data_ptr(), value.const_data_ptr(), key.stride(0), key.stride(1),
+                          k_codes.mutable_data_ptr(), v_codes.mutable_data_ptr(),
+                          k_scale.mutable_data_ptr<float>(), v_scale.mutable_data_ptr<float>(),
+                          return_dequantized ? dq_k.mutable_data_ptr() : nullptr,
+                          return_dequantized ? dq_v.mutable_data_ptr() : nullptr,
+                          position.const_data_ptr<int32_t>(), static_cast<int>(n_new), g.kv_heads,
+                          g.head_dim, g.t_max, g.bits, dtype, current_stream(key)),
+           "kv_append");
+  return std::make_tuple(dq_k, dq_v);
+}
+
+at::Tensor kv_dequant(const at::Tensor& codes, const at::Tensor& scale, int64_t n_tokens,
+                      at::ScalarType out_dtype) {
+  const CacheGeometry g = cache_geometry(codes, scale, "cache");
+  TORCH_CHECK(n_tokens >= 0 && n_tokens <= g.t_max, "n_tokens ", n_tokens, " outside [0, ", g.t_max, "]");
+  auto out = at::empty({g.kv_heads, n_tokens, g.head_dim}, codes.options().dtype(out_dtype));
+  const int dtype = dtype_code(out, "output dtype");
+  if (out.numel() == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(codes));
+  check_rc(llmq_kv_dequant(codes.const_data_ptr(), scale.const_data_ptr<float>(), out.mutable_data_ptr(),
+                           g.kv_heads, g.head_dim, g.t_max, static_cast<int>(n_tokens), g.bits, dtype,
+                           current_stream(codes)),
+           "kv_dequant");
+  return out;
+}
+
+int64_t kv_decode_workspace_floats(int64_t q_heads, int64_t head_dim, int64_t t_max) {
+  return static_cast<int64_t>(llmq_kv_decode_workspace_floats(static_cast<int>(q_heads),
+                                                              static_cast<int>(head_dim),
+                                                              static_cast<int>(t_max)));
+}
+
+// query: [q_heads, head_dim]; length: device int32, tokens valid in the cache. Returns [q_heads, head_dim].
+at::Tensor kv_decode_attention(const at::Tensor& query, const at::Tensor& k_codes, const at::Tensor& v_codes,
+                               const at::Tensor& k_scale, const at::Tensor& v_scale, at::Tensor& workspace,
+                               const at::Tensor& length, double sm_scale) {
+  TORCH_CHECK(query.is_cuda(), "query must be a CUDA tensor");
+  TORCH_CHECK(query.dim() == 2 && query.is_contiguous(), "query must be contiguous [q_heads, head_dim]");
+  const int dtype = dtype_code(query, "query");
+  const CacheGeometry g = cache_geometry(k_codes, k_scale, "key");
+  const CacheGeometry gv = cache_geometry(v_codes, v_scale, "value");
+  TORCH_CHECK(g.kv_heads == gv.kv_heads && g.t_max == gv.t_max && g.head_dim == gv.head_dim && g.bits == gv.bits,
+              "key and value caches differ in geometry");
+  TORCH_CHECK(query.size(1) == g.head_dim, "query head_dim ", query.size(1), " != cache head_dim ", g.head_dim);
+  const int q_heads = static_cast<int>(query.size(0));
+  check_position(length);
+  TORCH_CHECK(workspace.is_cuda() && workspace.scalar_type() == at::kFloat && workspace.is_contiguous() &&
+                  workspace.numel() >= kv_decode_workspace_floats(q_heads, g.head_dim, g.t_max),
+              "workspace must be a contiguous CUDA float32 tensor of at least kv_decode_workspace_floats() elements");
+  auto out = at::empty_like(query);
+  const c10::OptionalDeviceGuard guard(at::device_of(query));
+  check_rc(llmq_kv_decode_attention(query.const_data_ptr(), k_codes.const_data_ptr(), v_codes.const_data_ptr(),
+                                    k_scale.const_data_ptr<float>(), v_scale.const_data_ptr<float>(),
+                                    out.mutable_data_ptr(), workspace.mutable_data_ptr<float>(),
+                                    length.const_data_ptr<int32_t>(), static_cast<float>(sm_scale), q_heads,
+                                    g.kv_heads, g.head_dim, g.t_max, g.bits, dtype, current_stream(query)),
+           "kv_decode_attention");
+  return out;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -148,5 +260,17 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("wq_gemv", &wq_gemv,
         "Weight-only quantized matmul for a few rows: int8 or packed-int4 weight (HIP, gfx950)",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0);
+  m.def("kv_append", &kv_append,
+        "Quantize new K/V tokens into one layer's cache at the device-side position",
+        py::arg("key"), py::arg("value"), py::arg("k_codes"), py::arg("v_codes"), py::arg("k_scale"),
+        py::arg("v_scale"), py::arg("position"), py::arg("return_dequantized") = false);
+  m.def("kv_dequant", &kv_dequant, "Dequantize the first n_tokens of one layer's cache",
+        py::arg("codes"), py::arg("scale"), py::arg("n_tokens"), py::arg("out_dtype"));
+  m.def("kv_decode_workspace_floats", &kv_decode_workspace_floats, py::arg("q_heads"),
+        py::arg("head_dim"), py::arg("t_max"));
+  m.def("kv_decode_attention", &kv_decode_attention,
+        "Single-token GQA attention reading the quantized cache",
+        py::arg("query"), py::arg("k_codes"), py::arg("v_codes"), py::arg("k_scale"), py::arg("v_scale"),
+        py::arg("workspace"), py::arg("length"), py::arg("sm_scale"));
   m.def("abi_version", []() { return llmq_abi_version(); });
 }

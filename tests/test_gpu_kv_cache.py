@@ -1,0 +1,213 @@
+"""Quantized KV cache kernels against the CPU oracle: append (codes and scales bit-exact, as
+FakeQuantCache's arithmetic gives them), dequantize-on-read, and the fused single-token GQA
+attention (rel-L2 <= 1e-2 for bf16 outputs, <= 1e-3 for fp32, against float64 softmax attention
+over the (dtype)(code*scale) values; that attention arithmetic is not pinned by the reference,
+which delegates it to HF transformers)."""
+
+import pathlib
+
+import numpy as np
+import pytest
+import torch
+
+import llmq_oracle as oracle
+from conftest import rel_l2, tag_of, to_np
+
+pytestmark = pytest.mark.gpu
+GOLD = pathlib.Path(__file__).resolve().parent / "golden" / "kv_case.npz"
+
+
+@pytest.fixture(scope="module")
+def ext():
+    from llmquant.hip import load_extension
+
+    return load_extension()
+
+
+def new_cache(kv_heads, t_max, d, bits, dev="cuda"):
+    width = d if bits == 8 else d // 2
+    dt = torch.int8 if bits == 8 else torch.uint8
+    return dict(k_codes=torch.zeros(kv_heads, t_max, width, dtype=dt, device=dev),
+                v_codes=torch.zeros(kv_heads, t_max, width, dtype=dt, device=dev),
+                k_scale=torch.zeros(kv_heads, t_max, device=dev), v_scale=torch.zeros(kv_heads, t_max, device=dev))
+
+
+def append(ext, cache, k, v, pos, dq=False):
+    position = torch.tensor([pos], dtype=torch.int32, device="cuda")
+    return ext.kv_append(k, v, cache["k_codes"], cache["v_codes"], cache["k_scale"], cache["v_scale"], position, dq)
+
+
+def codes_np(t, bits):
+    a = t.cpu().numpy()
+    return oracle.unpack_int4(a) if bits == 4 else a
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_golden_case(ext, bits):
+    g = np.load(GOLD)
+    k = torch.from_numpy(g["k"].copy()).view(torch.bfloat16).cuda()
+    v = torch.from_numpy(g["v"].copy()).view(torch.bfloat16).cuda()
+    q = torch.from_numpy(g["q"].copy()).view(torch.bfloat16).cuda()
+    kv_heads, t, d = k.shape
+    cache = new_cache(kv_heads, 64, d, bits)
+    append(ext, cache, k, v, 0)
+    assert np.array_equal(codes_np(cache["k_codes"], bits)[:, :t], g[f"k_codes{bits}"])
+    assert np.array_equal(codes_np(cache["v_codes"], bits)[:, :t], g[f"v_codes{bits}"])
+    assert np.array_equal(to_np(cache["k_scale"])[:, :t], g[f"k_scale{bits}"])
+    assert np.array_equal(to_np(cache["v_scale"])[:, :t], g[f"v_scale{bits}"])
+    ws = torch.zeros(ext.kv_decode_workspace_floats(q.shape[0], d, 64), device="cuda")
+    length = torch.tensor([t], dtype=torch.int32, device="cuda")
+    out = ext.kv_decode_attention(q, cache["k_codes"], cache["v_codes"], cache["k_scale"], cache["v_scale"], ws,
+                                  length, d ** -0.5)
+    assert rel_l2(to_np(out), g[f"attn{bits}"]) <= 1e-2
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("d", [64, 128])
+def test_append_matches_the_oracle_and_fake_quant(ext, bits, dtype, d):
+    """Prefill-shaped append: [kv_heads, T, D] taken as a strided view of [T, kv_heads, D]
+    (how HF lays out projected keys), codes + scales + returned dequantized values."""
+    torch.manual_seed(0)
+    kv_heads, t = 8, 45
+    k = (torch.randn(t, kv_heads, d) * 2).to(dtype).cuda().transpose(0, 1)
+    v = torch.randn(t, kv_heads, d).to(dtype).cuda().transpose(0, 1)
+    assert not k.is_contiguous()
+    cache = new_cache(kv_heads, 64, d, bits)
+    dq_k, dq_v = append(ext, cache, k, v, 3, dq=True)
+    for name, src, dq in (("k", k, dq_k), ("v", v, dq_v)):
+        want_codes, want_scale = oracle.kv_quant(to_np(src), bits)
+        assert np.array_equal(codes_np(cache[f"{name}_codes"], bits)[:, 3:3 + t], want_codes)
+        assert np.array_equal(to_np(cache[f"{name}_scale"])[:, 3:3 + t], want_scale)
+        want_dq = oracle.fake_quantize(to_np(src), bits, tag_of(dtype), "group", 128)  # FakeQuantCache's rule
+        assert dq.dtype == dtype and np.array_equal(to_np(dq).view(np.uint32), want_dq.view(np.uint32))
+        assert np.all(to_np(cache[f"{name}_scale"])[:, :3] == 0) and np.all(to_np(cache[f"{name}_scale"])[:, 3 + t:] == 0)
+    # dequantize-on-read of the stored range gives the same values back
+    got = ext.kv_dequant(cache["k_codes"], cache["k_scale"], 3 + t, dtype)
+    assert np.array_equal(to_np(got)[:, 3:], to_np(dq_k))
+
+
+def test_old_tokens_are_not_requantized(ext):
+    torch.manual_seed(0)
+    cache = new_cache(2, 16, 64, 4)
+    first = torch.randn(2, 3, 64, device="cuda", dtype=torch.bfloat16)
+    append(ext, cache, first, first.clone(), 0)
+    kept = {k: v.clone() for k, v in cache.items()}
+    second = torch.randn(2, 2, 64, device="cuda", dtype=torch.bfloat16) * 10
+    append(ext, cache, second, second.clone(), 3)
+    for name in cache:
+        assert torch.equal(cache[name][:, :3], kept[name][:, :3])
+        assert not torch.equal(cache[name][:, 3:5], kept[name][:, 3:5])
+    # positions past the end of the cache are dropped, not written out of bounds
+    append(ext, cache, second, second.clone(), 15)
+    assert torch.equal(cache["k_codes"][:, :3], kept["k_codes"][:, :3])
+
+
+def attention_case(ext, bits, dtype, q_heads, kv_heads, d, t_max, length, seed=0):
+    torch.manual_seed(seed)
+    channel = torch.exp(0.5 * torch.randn(d))
+    k = (torch.randn(kv_heads, length, d) * channel).to(dtype).cuda()
+    v = (torch.randn(kv_heads, length, d) * channel).to(dtype).cuda()
+    q = torch.randn(q_heads, d).to(dtype).cuda()
+    cache = new_cache(kv_heads, t_max, d, bits)
+    append(ext, cache, k, v, 0)
+    ws = torch.zeros(ext.kv_decode_workspace_floats(q_heads, d, t_max), device="cuda")
+    len_dev = torch.tensor([length], dtype=torch.int32, device="cuda")
+    out = ext.kv_decode_attention(q, cache["k_codes"], cache["v_codes"], cache["k_scale"], cache["v_scale"], ws,
+                                  len_dev, d ** -0.5)
+    tag = tag_of(dtype)
+    kq, ks = oracle.kv_quant(to_np(k), bits)
+    vq, vs = oracle.kv_quant(to_np(v), bits)
+    want = oracle.gqa_decode_attention(to_np(q), oracle.kv_dequant(kq, ks, tag), oracle.kv_dequant(vq, vs, tag),
+                                       d ** -0.5, "f32")
+    return out, want, (cache, ws, len_dev, q)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("length", [1, 15, 64, 777, 2049])
+def test_decode_attention_llama_1b_geometry(ext, bits, length):
+    """BASELINE config 4: 32 query heads, 8 kv heads, head_dim 64, context up to 2048 + 1."""
+    out, want, _ = attention_case(ext, bits, torch.bfloat16, 32, 8, 64, 2049, length)
+    assert out.shape == (32, 64) and out.dtype == torch.bfloat16
+    assert rel_l2(to_np(out), want) <= 1e-2
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-3), (torch.float16, 1e-2)])
+@pytest.mark.parametrize("q_heads,kv_heads,d", [(8, 8, 64), (16, 8, 128), (32, 8, 128), (8, 1, 64)])
+def test_decode_attention_other_geometries(ext, dtype, tol, q_heads, kv_heads, d):
+    out, want, _ = attention_case(ext, 8, dtype, q_heads, kv_heads, d, 300, 211, seed=1)
+    assert rel_l2(to_np(out), want) <= tol
+    if dtype == torch.float32:
+        assert rel_l2(to_np(out), want) <= 1e-5  # fp32 throughout: only summation order differs
+
+
+def test_cost_tracks_valid_length_and_repeat_launches_agree(ext):
+    """Entries beyond `length` are ignored whatever they hold, and the arrival counters are
+    left clean: a second launch on the same workspace gives the same bits."""
+    out, want, (cache, ws, len_dev, q) = attention_case(ext, 8, torch.bfloat16, 32, 8, 64, 1024, 100, seed=2)
+    cache["k_codes"][:, 100:] = 127
+    cache["k_scale"][:, 100:] = 1e6
+    cache["v_codes"][:, 100:] = -128
+    cache["v_scale"][:, 100:] = 1e6
+    again = ext.kv_decode_attention(q, cache["k_codes"], cache["v_codes"], cache["k_scale"], cache["v_scale"], ws,
+                                    len_dev, 64 ** -0.5)
+    assert torch.equal(out, again)
+    assert rel_l2(to_np(again), want) <= 1e-2
+
+
+def test_graph_replay_follows_the_device_length(ext):
+    """Append + attend captured once, replayed while position/length advance on the device;
+    every replay must equal the eager result at that length."""
+    torch.manual_seed(3)
+    kv_heads, q_heads, d, t_max = 8, 32, 64, 256
+    cache = new_cache(kv_heads, t_max, d, 8)
+    ws = torch.zeros(ext.kv_decode_workspace_floats(q_heads, d, t_max), device="cuda")
+    prefix = torch.randn(kv_heads, 50, d, device="cuda", dtype=torch.bfloat16)
+    append(ext, cache, prefix, prefix.flip(1).contiguous(), 0)
+    pos = torch.tensor([50], dtype=torch.int32, device="cuda")
+    length = torch.tensor([51], dtype=torch.int32, device="cuda")
+    k1 = torch.zeros(kv_heads, 1, d, device="cuda", dtype=torch.bfloat16)
+    v1 = torch.zeros_like(k1)
+    q = torch.zeros(q_heads, d, device="cuda", dtype=torch.bfloat16)
+
+    def step():
+        ext.kv_append(k1, v1, cache["k_codes"], cache["v_codes"], cache["k_scale"], cache["v_scale"], pos, False)
+        return ext.kv_decode_attention(q, cache["k_codes"], cache["v_codes"], cache["k_scale"], cache["v_scale"], ws,
+                                       length, d ** -0.5)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        k1.normal_(); v1.normal_(); q.normal_()
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = step()
+    for i in range(5):
+        k1.normal_(); v1.normal_(); q.normal_()
+        pos.fill_(50 + i); length.fill_(51 + i)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        eager = step()  # same inputs, same position: rewrites the same slot with the same codes
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), i
+
+
+def test_argument_checks(ext):
+    cache = new_cache(2, 16, 64, 8)
+    k = torch.randn(2, 1, 64, device="cuda", dtype=torch.bfloat16)
+    pos = torch.tensor([0], dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="position must be a CUDA int32"):
+        ext.kv_append(k, k, cache["k_codes"], cache["v_codes"], cache["k_scale"], cache["v_scale"], pos.long(), False)
+    with pytest.raises(RuntimeError, match="cache holds"):
+        ext.kv_append(k[:1], k[:1], cache["k_codes"], cache["v_codes"], cache["k_scale"], cache["v_scale"], pos, False)
+    q = torch.randn(8, 64, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="workspace must be"):
+        ext.kv_decode_attention(q, cache["k_codes"], cache["v_codes"], cache["k_scale"], cache["v_scale"],
+                                torch.zeros(4, device="cuda"), pos, 0.125)
+    ws = torch.zeros(ext.kv_decode_workspace_floats(6, 64, 16), device="cuda")
+    with pytest.raises(RuntimeError, match="multiple of kv_heads|must be 1, 2, 4 or 8"):
+        ext.kv_decode_attention(q[:6], cache["k_codes"], cache["v_codes"], cache["k_scale"], cache["v_scale"], ws, pos, 0.125)
