@@ -1,0 +1,146 @@
+"""Replaying a captured decode step (API of llmquant/runtime/graph_decode.py).
+
+Two decoders share one interface (prefill / capture / step / logits / max_len):
+
+  GraphedDecoder    any HF causal LM over a transformers StaticCache, the arrangement the
+                    reference measures bf16 and weight-only runs with: eager prefill, warmup
+                    on a side stream, one captured step, replay
+  KernelDecoder     the kernel path with the integer KV cache (LlamaKernelRuntime): the case
+                    the reference cannot graph, because its quantized cache is a growing
+                    DynamicCache (graph_decode.py:40-43)
+
+`graphed_generate` picks between them; both are used for the bf16-vs-quantized comparison so
+neither side is credited with the graph alone.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from llmquant.runtime.llama_decode import WARMUP_CALLS, LlamaKernelRuntime
+
+__all__ = ["GraphedDecoder", "KernelDecoder", "WARMUP_CALLS", "can_graph", "graphed_generate"]
+
+
+def _on_gpu(model) -> bool:
+    if not torch.cuda.is_available():
+        return False
+    first = next(model.parameters(), None)
+    return first is not None and first.device.type == "cuda"
+
+
+def can_graph(model, cache_factory=None) -> bool:
+    """Whether a graphed decode is possible for this model and cache choice.
+
+    A PyTorch-side quantized cache (FakeQuantCache factory) still cannot be captured; the
+    kernel cache can, and is requested with `kv_bits` on graphed_generate instead of a factory.
+    """
+    if cache_factory is not None:
+        return False
+    return _on_gpu(model)
+
+
+class GraphedDecoder:
+    """One captured HF decode step over a StaticCache sized exactly to the run (attention
+    costs the allocated length, and warmup/capture calls consume slots that are rewound)."""
+
+    def __init__(self, model, prompt_tokens: int, new_tokens: int):
+        from transformers import StaticCache
+
+        self.model = model
+        self.device = next(model.parameters()).device
+        self.max_len = prompt_tokens + new_tokens + WARMUP_CALLS + 1
+        self.cache = StaticCache(config=model.config, max_batch_size=1, max_cache_len=self.max_len,
+                                 device=self.device, dtype=next(model.parameters()).dtype)
+        self.token = torch.zeros(1, 1, dtype=torch.long, device=self.device)
+        self.position = torch.zeros(1, dtype=torch.long, device=self.device)
+        self.graph = None
+        self.logits = None
+
+    def _forward_token(self):
+        return self.model(self.token, past_key_values=self.cache, use_cache=True,
+                          position_ids=self.position.unsqueeze(0))
+
+    @torch.no_grad()
+    def prefill(self, input_ids):
+        out = self.model(input_ids, past_key_values=self.cache, use_cache=True)
+        return out.logits[:, -1:].argmax(-1)
+
+    def _rewind(self, to: int):
+        for layer in self.cache.layers:
+            cursor = getattr(layer, "cumulative_length", None)
+            if isinstance(cursor, torch.Tensor):
+                cursor.fill_(to)
+
+    @torch.no_grad()
+    def capture(self, position: int):
+        self.position.fill_(position)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(WARMUP_CALLS):
+                self._forward_token()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            out = self._forward_token()
+        self.logits = out.logits
+        self._rewind(position)
+
+    @torch.no_grad()
+    def step(self, token, position: int):
+        self.token.copy_(token.reshape(1, 1))
+        self.position.fill_(position)
+        self.graph.replay()
+        return self.logits[:, -1:].argmax(-1)
+
+
+class KernelDecoder:
+    """Same interface over LlamaKernelRuntime and the integer KV cache."""
+
+    def __init__(self, model, prompt_tokens: int, new_tokens: int, kv_bits: int = 8):
+        self.max_len = prompt_tokens + new_tokens + 1
+        self.runtime = LlamaKernelRuntime(model, self.max_len, kv_bits)
+        self.graph = None
+
+    @property
+    def logits(self):
+        return self.runtime.logits
+
+    def prefill(self, input_ids):
+        return self.runtime.prefill(input_ids).reshape(1, 1)
+
+    def capture(self, position: int, token=None):
+        self.runtime.capture(self.runtime.token if token is None else token, position)
+        self.graph = self.runtime.graph
+
+    def step(self, token=None, position: int | None = None):
+        # the previous step already left its argmax and the advanced position on the device;
+        # explicit arguments re-seed them (used when a caller rewinds or substitutes a token)
+        if token is not None and position is not None and position != self.runtime.cache.get_seq_length():
+            self.runtime._set_step_inputs(token, position)
+        return self.runtime.step().reshape(1, 1)
+
+
+@torch.no_grad()
+def graphed_generate(model, input_ids, max_new_tokens: int, kv_bits: int | None = None):
+    """Greedy generation with the decode step replayed; None if it cannot be graphed. Returns
+    the full sequence like model.generate(..., do_sample=False). With kv_bits the integer KV
+    cache and the kernel runtime are used (Llama-architecture models)."""
+    if not can_graph(model):
+        return None
+    prompt = input_ids.shape[1]
+    if kv_bits is not None:
+        runtime = LlamaKernelRuntime(model, prompt + max_new_tokens + 1, kv_bits)
+        return runtime.generate(input_ids, max_new_tokens, use_graph=True)
+    decoder = GraphedDecoder(model, prompt, max_new_tokens)
+    nxt = decoder.prefill(input_ids)
+    out = [nxt]
+    if max_new_tokens > 1:
+        decoder.token.copy_(nxt.reshape(1, 1))
+        decoder.capture(prompt)
+        for i in range(1, max_new_tokens):
+            nxt = decoder.step(nxt, prompt + i - 1)
+            out.append(nxt)
+    return torch.cat([input_ids, *out], dim=1)
