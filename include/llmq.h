@@ -71,6 +71,16 @@ int llmq_wq_gemv(const void* x, const void* qweight, const float* wscale, void* 
                  int N, int G, int gs, int out_group, int wformat, int dtype,
                  llmq_stream_t stream);
 
+/* Integer GEMM with per-group scales on both operands (the A8 branch of
+ * RealQuantLinear.forward, llmquant/quantizers/real.py:76-103):
+ *   out[m, n] = sum over g, in order, of  float(sum_k a[m,g,k]*q[n,g,k]) * sw[sr(n), g] * sx[m, g]
+ * each group's term rounded to fp32 after every multiply and added sequentially, then
+ * bias (fp32, nullable) added and the sum cast to `dtype`. gs must be 128.
+ * a: int8 [M, G*128]; sx: fp32 [M, G]; qweight/wscale as for llmq_wq_gemv. */
+int llmq_wq_gemm_a8(const int8_t* a, const float* sx, const void* qweight, const float* wscale,
+                    const float* bias_or_null, void* out, int M, int N, int G, int gs,
+                    int out_group, int wformat, int dtype, llmq_stream_t stream);
+
 /* KV cache, one layer. Codes are [kv_heads, t_max, head_dim] int8 (bits == 8) or
  * [kv_heads, t_max, head_dim/2] nibble-packed uint8 (bits == 4); scales are fp32
  * [kv_heads, t_max]: one scale per token per head, which is what FakeQuantCache's

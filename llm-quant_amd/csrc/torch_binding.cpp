@@ -136,6 +136,48 @@ at::Tensor wq_gemv(const at::Tensor& x, const at::Tensor& qweight, const at::Ten
   return out;
 }
 
+// Integer GEMM: a int8 [M, K], sx fp32 [M, G]; qweight / wscale as for wq_gemv; optional fp32 or
+// half-width bias (converted to fp32 here, as RealQuantLinear adds bias.float()).
+at::Tensor wq_gemm_a8(const at::Tensor& a, const at::Tensor& sx, const at::Tensor& qweight,
+                      const at::Tensor& wscale, const c10::optional<at::Tensor>& bias, int64_t out_group,
+                      at::ScalarType out_dtype) {
+  TORCH_CHECK(a.is_cuda() && sx.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "all tensors must be CUDA");
+  TORCH_CHECK(a.scalar_type() == at::kChar && a.dim() == 2, "a must be int8 [M, K]");
+  TORCH_CHECK(sx.scalar_type() == at::kFloat && sx.dim() == 2, "sx must be float32 [M, groups]");
+  TORCH_CHECK(qweight.dim() == 3, "qweight must be [N, groups, group_size], got ", qweight.dim(), "D");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 2, "wscale must be float32 [scale_rows, groups]");
+  const auto ac = a.contiguous();
+  const auto sxc = sx.contiguous();
+  const auto wc = qweight.contiguous();
+  const auto sc = wscale.contiguous();
+  const int64_t M = ac.size(0), N = wc.size(0), groups = wc.size(1);
+  const int64_t group_size = packed ? wc.size(2) * 2 : wc.size(2);
+  TORCH_CHECK(group_size == 128, "the integer GEMM needs group_size 128, got ", group_size);
+  TORCH_CHECK(ac.size(1) == groups * group_size, "a last dim ", ac.size(1), " does not match qweight ",
+              groups, "x", group_size);
+  TORCH_CHECK(sxc.size(0) == M && sxc.size(1) == groups, "sx must be [", M, ", ", groups, "]");
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  TORCH_CHECK(sc.size(0) == scale_rows && sc.size(1) == groups, "wscale must be [", scale_rows, ", ", groups, "]");
+  at::Tensor bias_f;
+  if (bias.has_value() && bias->defined()) {
+    TORCH_CHECK(bias->numel() == N, "bias must have ", N, " elements");
+    bias_f = bias->to(at::kFloat).contiguous();
+  }
+  auto out = at::empty({M, N}, ac.options().dtype(out_dtype));
+  const int dtype = dtype_code(out, "output dtype");
+  if (M == 0 || N == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(ac));
+  check_rc(llmq_wq_gemm_a8(ac.const_data_ptr<int8_t>(), sxc.const_data_ptr<float>(), wc.const_data_ptr(),
+                           sc.const_data_ptr<float>(), bias_f.defined() ? bias_f.const_data_ptr<float>() : nullptr,
+                           out.mutable_data_ptr(), static_cast<int>(M), static_cast<int>(N),
+                           static_cast<int>(groups), static_cast<int>(group_size), static_cast<int>(out_group),
+                           packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype, current_stream(ac)),
+           "wq_gemm_a8");
+  return out;
+}
+
 // ---- quantized KV cache -------------------------------------------------------------------------------
 // Cache tensors of one layer: codes [kv_heads, t_max, head_dim] int8 or [kv_heads, t_max,
 // head_dim / 2] uint8, scales [kv_heads, t_max] fp32. `position` is a device int32 tensor.
@@ -260,6 +302,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("wq_gemv", &wq_gemv,
         "Weight-only quantized matmul for a few rows: int8 or packed-int4 weight (HIP, gfx950)",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0);
+  m.def("wq_gemm_a8", &wq_gemm_a8,
+        "Integer GEMM: int8 activations x int4/int8 group-quantized weights, real-mode rounding order",
+        py::arg("a"), py::arg("sx"), py::arg("qweight"), py::arg("wscale"), py::arg("bias") = py::none(),
+        py::arg("out_group") = 0, py::arg("out_dtype") = at::kBFloat16);
   m.def("kv_append", &kv_append,
         "Quantize new K/V tokens into one layer's cache at the device-side position",
         py::arg("key"), py::arg("value"), py::arg("k_codes"), py::arg("v_codes"), py::arg("k_scale"),

@@ -1,0 +1,252 @@
+// Integer prefill GEMM on the int8 matrix core (v_mfma_i32_32x32x32_i8), gfx950: int8
+// activations (quantized per token x group) times int4 / int8 group-quantized weights.
+//
+//   out[m, n] = sum over groups g, in order, of  ((float)(sum_k a[m,g,k] * q[n,g,k]) * sw[sr(n),g]) * sx[m,g]
+//
+// This is the A8 branch of RealQuantLinear.forward (llmquant/quantizers/real.py:76-103) with
+// its rounding points kept: the group's integer sum is exact (128 * 127 * 127 < 2^24), it is
+// converted to fp32, multiplied by the weight scale, then by the activation scale, then added
+// to the running fp32 total -- four separately rounded operations, in group order. The file is
+// built with -ffp-contract=off so no multiply-add is fused; results equal the reference's
+// real mode bit for bit.
+//
+// Shape. A workgroup (4 waves) owns a 128 x 128 output tile and walks K one group (128) at a
+// time. Activations [M, K] int8 and weights [N, K(/2)] are staged in LDS, weights unpacked
+// there to signed int8 in natural k order (packed int4: nibble - 8 computed four at a time
+// with a borrow-free byte subtract, even/odd nibbles re-interleaved with v_perm). Each wave
+// computes a 64 x 64 quadrant as 2 x 2 MFMA tiles of 32 x 32 (A = activations, rows m;
+// B = weights, columns n), 4 k-slabs of 32 per group. The next group's global loads are in
+// flight while the current one is multiplied. After each group the int32 accumulators go
+// through the scale epilogue above and are cleared.
+#include "llmq_device.h"
+
+namespace {
+
+using namespace llmq;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int kBM = 128, kBN = 128, kGroup = 128;
+constexpr int kThreads = 256;
+constexpr int kRowStride = kGroup + 16;  // bytes; padding keeps 16-byte reads off the same banks
+
+struct GemmArgs {
+  const int8_t* a;     // [M, G*128]
+  const float* sx;     // [M, G]
+  const uint8_t* qw;   // [N, G, 128] int8 or [N, G, 64] packed
+  const float* sw;     // [scale_rows, G]
+  const float* bias;   // [N] or null
+  void* out;           // [M, N]
+  int M, N, G, out_group;
+};
+
+// four codes (bytes, value + 8 in 0..15) -> four signed bytes (value), no borrow between bytes
+__device__ __forceinline__ uint32_t unbias4(uint32_t u) {
+  return ((u | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+}
+
+template <typename T, int BITS>
+__global__ __launch_bounds__(kThreads) void wq_gemm_a8_kernel(const GemmArgs g) {
+  __shared__ __attribute__((aligned(16))) int8_t s_a[2][kBM * kRowStride];
+  __shared__ __attribute__((aligned(16))) int8_t s_b[2][kBN * kRowStride];
+  __shared__ __attribute__((aligned(16))) float s_sx[2][kBM];
+  __shared__ __attribute__((aligned(16))) float s_sw[2][kBN];
+
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int wm = wv >> 1, wn = wv & 1;  // quadrant of the tile
+  const int m0 = blockIdx.y * kBM, n0 = blockIdx.x * kBN;
+  const int64_t k_total = static_cast<int64_t>(g.G) * kGroup;
+  const int64_t w_row_bytes = BITS == 8 ? k_total : k_total / 2;
+
+  // ---- staging: who loads what ------------------------------------------------------------------
+  // A tile: 128 rows x 128 B = 1024 16-byte packets, 4 per thread. Thread t: packets t + 256*i:
+  // row = p / 8, piece = p % 8.
+  // B tile int8: same. B tile int4: 128 rows x 64 B = 512 packets, 2 per thread: row = p / 4.
+  constexpr int kAPackets = 4;
+  constexpr int kBPackets = BITS == 8 ? 4 : 2;
+  u32x4 ra[kAPackets], rb[kBPackets];
+  float r_sx = 0.0f, r_sw = 0.0f;
+
+  auto load_group = [&](int grp) {
+#pragma unroll
+    for (int i = 0; i < kAPackets; ++i) {
+      const int p = tid + kThreads * i;
+      const int row = min(m0 + (p >> 3), g.M - 1);
+      ra[i] = load16(g.a + static_cast<int64_t>(row) * k_total + static_cast<int64_t>(grp) * kGroup + (p & 7) * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < kBPackets; ++i) {
+      const int p = tid + kThreads * i;
+      if constexpr (BITS == 8) {
+        const int row = min(n0 + (p >> 3), g.N - 1);
+        rb[i] = load16(g.qw + static_cast<int64_t>(row) * w_row_bytes + static_cast<int64_t>(grp) * kGroup + (p & 7) * 16);
+      } else {
+        const int row = min(n0 + (p >> 2), g.N - 1);
+        rb[i] = load16(g.qw + static_cast<int64_t>(row) * w_row_bytes + static_cast<int64_t>(grp) * (kGroup / 2) + (p & 3) * 16);
+      }
+    }
+    if (tid < kBM) {
+      r_sx = g.sx[static_cast<int64_t>(min(m0 + tid, g.M - 1)) * g.G + grp];
+    } else {
+      const int n = min(n0 + tid - kBM, g.N - 1);
+      r_sw = g.sw[static_cast<int64_t>(g.out_group > 0 ? n / g.out_group : n) * g.G + grp];
+    }
+  };
+  auto store_group = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < kAPackets; ++i) {
+      const int p = tid + kThreads * i;
+      store16(&s_a[buf][(p >> 3) * kRowStride + (p & 7) * 16], ra[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < kBPackets; ++i) {
+      const int p = tid + kThreads * i;
+      if constexpr (BITS == 8) {
+        store16(&s_b[buf][(p >> 3) * kRowStride + (p & 7) * 16], rb[i]);
+      } else {
+        // 16 packed bytes = 32 codes -> 32 signed bytes in natural k order
+        const uint32_t w[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
+        uint32_t o[8];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const uint32_t lo = unbias4(w[d] & 0x0f0f0f0fu);         // codes k = 8d + {0,2,4,6}
+          const uint32_t hi = unbias4((w[d] >> 4) & 0x0f0f0f0fu);  // codes k = 8d + {1,3,5,7}
+          // bytes (lo0, hi0, lo1, hi1) and (lo2, hi2, lo3, hi3); v_perm selects from {hi:lo}
+          o[2 * d] = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
+          o[2 * d + 1] = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
+        }
+        int8_t* dst = &s_b[buf][(p >> 2) * kRowStride + (p & 3) * 32];
+        store16(dst, u32x4{o[0], o[1], o[2], o[3]});
+        store16(dst + 16, u32x4{o[4], o[5], o[6], o[7]});
+      }
+    }
+    if (tid < kBM) s_sx[buf][tid] = r_sx; else s_sw[buf][tid - kBM] = r_sw;
+  };
+
+  float acc[2][2][16];
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
+
+  load_group(0);
+  store_group(0);
+  __syncthreads();
+
+  const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
+  for (int grp = 0; grp < g.G; ++grp) {
+    const int buf = grp & 1;
+    if (grp + 1 < g.G) load_group(grp + 1);  // in flight during the MFMAs below
+
+    v16i d[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) d[mi][ni][r] = 0;
+#pragma unroll
+    for (int ks = 0; ks < kGroup / 32; ++ks) {
+      v4i fa[2], fb[2];
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) {
+        fa[mi] = *reinterpret_cast<const v4i*>(&s_a[buf][(wm * 64 + mi * 32 + frag_row) * kRowStride + ks * 32 + frag_k]);
+      }
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) {
+        fb[ni] = *reinterpret_cast<const v4i*>(&s_b[buf][(wn * 64 + ni * 32 + frag_row) * kRowStride + ks * 32 + frag_k]);
+      }
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+          d[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[mi], fb[ni], d[mi][ni], 0, 0, 0);
+    }
+
+    // scale epilogue: result register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4,
+    // column lane%32
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni) {
+      const float sw = s_sw[buf][wn * 64 + ni * 32 + (lane & 31)];
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) {
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          // four consecutive rows: one 128-bit LDS read of their activation scales
+          const int row = wm * 64 + mi * 32 + 8 * r4 + 4 * (lane >> 5);
+          const u32x4 s4 = *reinterpret_cast<const u32x4*>(&s_sx[buf][row]);
+          const float sx4[4] = {__builtin_bit_cast(float, s4.x), __builtin_bit_cast(float, s4.y),
+                                __builtin_bit_cast(float, s4.z), __builtin_bit_cast(float, s4.w)};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float f = static_cast<float>(d[mi][ni][4 * r4 + i]);
+            f = f * sw;
+            f = f * sx4[i];
+            acc[mi][ni][4 * r4 + i] = acc[mi][ni][4 * r4 + i] + f;
+          }
+        }
+      }
+    }
+
+    if (grp + 1 < g.G) store_group(buf ^ 1);  // nobody reads that buffer any more: see barrier below
+    __syncthreads();
+  }
+
+  T* __restrict__ out = static_cast<T*>(g.out);
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    const int n = n0 + wn * 64 + ni * 32 + (lane & 31);
+    const float b = (g.bias != nullptr && n < g.N) ? g.bias[n] : 0.0f;
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (m < g.M && n < g.N) {
+          const float v = g.bias != nullptr ? acc[mi][ni][r] + b : acc[mi][ni][r];
+          out[static_cast<int64_t>(m) * g.N + n] = from_float<T>(v);
+        }
+      }
+    }
+  }
+}
+
+template <typename T>
+int launch_typed(const GemmArgs& g, int wformat, hipStream_t stream) {
+  const dim3 grid((g.N + kBN - 1) / kBN, (g.M + kBM - 1) / kBM), block(kThreads);
+  if (wformat == LLMQ_W_INT8) {
+    hipLaunchKernelGGL((wq_gemm_a8_kernel<T, 8>), grid, block, 0, stream, g);
+  } else {
+    hipLaunchKernelGGL((wq_gemm_a8_kernel<T, 4>), grid, block, 0, stream, g);
+  }
+  return llmq_host::check_launch("wq_gemm_a8_kernel");
+}
+
+}  // namespace
+
+extern "C" int llmq_wq_gemm_a8(const int8_t* a, const float* sx, const void* qweight,
+                               const float* wscale, const float* bias_or_null, void* out, int M,
+                               int N, int G, int gs, int out_group, int wformat, int dtype,
+                               llmq_stream_t stream) {
+  if (M < 0 || N < 0 || G < 0) return llmq_host::fail_invalid("negative dimension M=%d N=%d G=%d", M, N, G);
+  if (gs != kGroup) return llmq_host::fail_invalid("the integer GEMM needs group_size 128, got %d", gs);
+  if (out_group < 0) return llmq_host::fail_invalid("out_group must be >= 0, got %d", out_group);
+  if (wformat != LLMQ_W_INT8 && wformat != LLMQ_W_INT4_PACKED)
+    return llmq_host::fail_invalid("unsupported weight format %d, expected 8 or 4", wformat);
+  if (M == 0 || N == 0) return 0;
+  if (G == 0) return llmq_host::fail_invalid("a weight with no groups has no reduction axis");
+  if (!a || !sx || !qweight || !wscale || !out) return llmq_host::fail_invalid("null tensor pointer");
+  if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(qweight)) & 15u)
+    return llmq_host::fail_invalid("activation and weight pointers must be 16-byte aligned");
+  GemmArgs g{a, sx, static_cast<const uint8_t*>(qweight), wscale, bias_or_null, out, M, N, G, out_group};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case LLMQ_F32: return launch_typed<float>(g, wformat, s);
+    case LLMQ_F16: return launch_typed<f16_t>(g, wformat, s);
+    case LLMQ_BF16: return launch_typed<bf16_t>(g, wformat, s);
+  }
+  return llmq_host::fail_invalid("out must be float32, float16 or bfloat16, got dtype code %d", dtype);
+}

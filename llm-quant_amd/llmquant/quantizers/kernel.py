@@ -62,6 +62,12 @@ class KernelQuantLinear(nn.Module):
         self._packed = stored.dtype == torch.uint8
         self._needs_padding = self.in_features != self.padded_in_features
         self._weight_args = scheme.weights
+        # int8 activations: the integer GEMM (real-mode arithmetic, bit for bit) serves every M.
+        # The reference's kernel mode ignores the activation scheme (kernel.py:97-103); here it
+        # is honoured when the geometry allows (one activation group per weight group of 128).
+        act = scheme.input_activations
+        self._int8_act = (act is not None and act.num_bits == 8 and act.strategy == "group"
+                          and act.group_size == group_size == 128)
         # looked up once: a decode step runs ~113 of these modules
         self._ext = load_extension()
         self._gemv = self._ext.wq_gemv
@@ -95,6 +101,11 @@ class KernelQuantLinear(nn.Module):
         rows = x.reshape(-1, x.shape[-1])
         if self._needs_padding:
             rows = pad_activation(rows, self._weight_args)
+        if self._int8_act:
+            codes, act_scale = self._ext.quant_group_codes(rows, 8, 128, False)
+            out = self._ext.wq_gemm_a8(codes, act_scale, self.qdata, self.wscale, self.bias, self.out_group,
+                                       x.dtype)
+            return out.reshape(*x.shape[:-1], self.out_features)
         if rows.shape[0] <= KERNEL_MAX_ROWS:
             out = self._gemv(rows, self.qdata, self.wscale, self.out_group)
         else:

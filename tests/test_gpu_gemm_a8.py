@@ -1,0 +1,134 @@
+"""The integer prefill GEMM (int8 activations x int4/int8 weights) against the oracle's
+real-mode forward: activation codes and scales bit-exact, outputs bit-exact (the kernel keeps
+RealQuantLinear's rounding points and group order, llmquant/quantizers/real.py:94-99), at the
+reference's own test size, ragged sizes, and the BASELINE config-3 shapes via sampled entries."""
+
+import ctypes
+import pathlib
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import llmq_oracle as oracle
+from conftest import rel_l2, tag_of, to_np
+
+pytestmark = pytest.mark.gpu
+GROUP = 128
+
+
+@pytest.fixture(scope="module")
+def ext():
+    from llmquant.hip import load_extension
+
+    return load_extension()
+
+
+def run_case(ext, m, n, k, bits, dtype, out_group=0, bias=False, seed=0, outliers=False):
+    torch.manual_seed(seed)
+    w = (torch.randn(n, k) * 0.015).to(torch.bfloat16)
+    x = torch.randn(m, k)
+    if outliers:
+        cols = torch.randperm(k)[: k // 100]
+        x[:, cols] *= 20
+    x = x.to(dtype)
+    b = torch.randn(n) if bias else None
+    canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP, None, out_group or None)
+    q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
+    s = torch.from_numpy(scales).cuda()
+    codes, sx = ext.quant_group_codes(x.cuda(), 8, GROUP, False)
+    want_codes, want_sx = oracle.quant_group_codes(to_np(x), 8, GROUP)
+    assert np.array_equal(codes.cpu().numpy(), want_codes) and np.array_equal(to_np(sx), want_sx)
+    got = ext.wq_gemm_a8(codes, sx, q, s, b.cuda() if bias else None, out_group, dtype)
+    return got, (x, canonical, scales, b)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,n,k", [(32, 256, 512), (1, 128, 128), (37, 200, 384), (130, 129, 256), (4, 512, 2048)])
+def test_bit_exact_against_real_mode(ext, bits, dtype, m, n, k):
+    got, (x, canonical, scales, _) = run_case(ext, m, n, k, bits, dtype)
+    want = oracle.real_linear(to_np(x), canonical, scales, tag_of(dtype), None, 8)
+    assert got.shape == (m, n) and got.dtype == dtype
+    assert np.array_equal(to_np(got).view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_bias_and_head_scales(ext, bits):
+    got, (x, canonical, scales, b) = run_case(ext, 70, 192, 512, bits, torch.bfloat16, out_group=64, bias=True, seed=1)
+    want = oracle.real_linear(to_np(x), canonical, scales, "bf16", 64, 8, to_np(b))
+    assert np.array_equal(to_np(got), want)
+
+
+def test_matches_the_float64_closed_form(ext):
+    """Independent of the accumulation order: y = sum_g sx sw sum_k a q, in float64."""
+    got, (x, canonical, scales, _) = run_case(ext, 64, 256, 1024, 4, torch.float32, seed=2)
+    a, sx = oracle.quant_group_codes(to_np(x), 8, GROUP)
+    xq = (a.reshape(64, -1, GROUP).astype(np.float64) * sx[..., None].astype(np.float64)).reshape(64, -1)
+    exact = oracle.gemv_float64(xq, canonical, scales)
+    assert rel_l2(to_np(got), exact) <= 1e-6
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("m", [128, 512, 2048])
+def test_llama_8b_mlp_shapes_on_sampled_entries(ext, n, k, m):
+    """BASELINE config 3 at full size (1% outlier channels x20): 64 x 64 sampled outputs,
+    bit-exact against the oracle restricted to those rows and columns."""
+    got, (x, canonical, scales, _) = run_case(ext, m, n, k, 4, torch.bfloat16, seed=3, outliers=True)
+    rng = np.random.default_rng(0)
+    rows = np.sort(rng.choice(m, 64, replace=False))
+    cols = np.sort(rng.choice(n, 64, replace=False))
+    want = oracle.real_linear(to_np(x)[rows], canonical[cols], scales[cols], "bf16", None, 8)
+    assert np.array_equal(to_np(got)[np.ix_(rows, cols)], want)
+
+
+@pytest.mark.parametrize("name", ["W4A8", "W8A8"])
+@pytest.mark.parametrize("layout", [dict(), dict(head_dim=64), dict(out_group=64)])
+@pytest.mark.parametrize("m", [1, 4, 33])
+def test_module_equals_real_mode_on_device(name, layout, m):
+    """KernelQuantLinear with an int8 activation scheme against RealQuantLinear run by torch on
+    the same GPU (reference tests/test_kernel_linear.py's equality, for the A8 schemes)."""
+    from dataclasses import replace
+
+    from llmquant.core.scheme import QuantizationScheme, preset_name_to_scheme
+    from llmquant.quantizers import KernelQuantLinear, RealQuantLinear
+
+    base = preset_name_to_scheme(name)
+    act = replace(base.input_activations, head_dim=layout["head_dim"]) if "head_dim" in layout else base.input_activations
+    scheme = QuantizationScheme(weights=replace(base.weights, **layout), input_activations=act)
+    torch.manual_seed(0)
+    linear = nn.Linear(2048, 512, bias=True).cuda().to(torch.bfloat16)
+    x = torch.randn(m, 2048, device="cuda", dtype=torch.bfloat16)
+    got = KernelQuantLinear.from_linear(linear, scheme)(x)
+    want = RealQuantLinear.from_linear(linear, scheme)(x)
+    assert got.shape == want.shape and torch.equal(got, want)
+
+
+def test_c_oracle_agrees_at_a_larger_size(ext):
+    """The C restatement (also the timed CPU baseline) against the kernel, 256 x 1024 x 2048."""
+    root = pathlib.Path(__file__).resolve().parent.parent
+    lib = ctypes.CDLL(str(root / "oracle" / "libllmq_oracle.so"))
+    got, (x, canonical, scales, _) = run_case(ext, 256, 1024, 2048, 4, torch.float32, seed=4)
+    a, sx = oracle.quant_group_codes(to_np(x), 8, GROUP)
+    packed = oracle.pack_int4(canonical)
+    out = np.empty((256, 1024), dtype=np.float32)
+    ptr = lambda arr: arr.ctypes.data_as(ctypes.c_void_p)
+    lib.llmq_oracle_real_gemm_a8(ptr(a), ptr(np.ascontiguousarray(sx)), ptr(packed), ptr(scales), ptr(out),
+                                 256, 1024, 16, 128, 0, 1)
+    assert np.array_equal(to_np(got), out)
+
+
+def test_argument_checks(ext):
+    a = torch.zeros(4, 256, dtype=torch.int8, device="cuda")
+    sx = torch.ones(4, 2, device="cuda")
+    q = torch.zeros(8, 2, 128, dtype=torch.int8, device="cuda")
+    s = torch.ones(8, 2, device="cuda")
+    assert ext.wq_gemm_a8(a, sx, q, s).shape == (4, 8)
+    with pytest.raises(RuntimeError, match="a must be int8"):
+        ext.wq_gemm_a8(a.float(), sx, q, s)
+    with pytest.raises(RuntimeError, match="sx must be"):
+        ext.wq_gemm_a8(a, sx[:, :1], q, s)
+    with pytest.raises(RuntimeError, match="group_size 128"):
+        ext.wq_gemm_a8(a, torch.ones(4, 4, device="cuda"), torch.zeros(8, 4, 64, dtype=torch.int8, device="cuda"),
+                       torch.ones(8, 4, device="cuda"))
