@@ -51,6 +51,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the legs that report the path's other kernels and end-to-end decode")
     return ap.parse_args()
 
 
@@ -191,10 +193,141 @@ def main():
         "shapes": shapes,
     }
 
+    del cases
+    torch.cuda.empty_cache()
+    if not opts.no_extras:
+        result["other_kernels"] = other_kernels(torch)
+        result["decode"] = decode_leg(torch)
+
     if not opts.no_cpu:
+        cases = build_operands(torch)
         result["cpu_baseline"] = cpu_baseline(torch, cases, opts.cpu_seconds)
 
     print(json.dumps(result))
+
+
+def _event_time_us(torch, fn, reps=20, warm=3):
+    for _ in range(warm):
+        fn()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps * 1e3
+
+
+def other_kernels(torch):
+    """The path's other kernels, each on its BASELINE shape: fake-quant op, KV-cache decode
+    attention (config 4), W4A8 / W8A8 integer GEMM (config 3). Back-to-back launches, HIP events."""
+    from llmquant.hip import load_extension
+
+    ext = load_extension()
+    dev = "cuda:0"
+    out = {}
+    # fake quant, 2048 x 8192 bf16, g128: one read + one write (+ scales)
+    xs = [torch.randn(2048, 8192, device=dev).to(torch.bfloat16) for _ in range(12)]  # 400 MB rotation
+    i = [0]
+
+    def fq():
+        ext.fake_quant_group(xs[i[0] % len(xs)], 4, GROUP, True)
+        i[0] += 1
+
+    us = _event_time_us(torch, fq, reps=48)
+    nbytes = 2 * 2048 * 8192 * 2 + 2048 * 64 * 4
+    out["fake_quant_2048x8192_bf16_int4"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                                             "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    del xs
+    # KV decode attention, Llama-3.2-1B geometry, context 2048 (+ the token being decoded)
+    for bits in (8, 4):
+        layers, kvh, qh, d, t = 16, 8, 32, 64, 2049
+        width = d if bits == 8 else d // 2
+        dt = torch.int8 if bits == 8 else torch.uint8
+        kc = torch.randint(0, 100, (layers, kvh, t, width), device=dev).to(dt)
+        vc = torch.randint(0, 100, (layers, kvh, t, width), device=dev).to(dt)
+        ks = torch.rand(layers, kvh, t, device=dev) * 0.05
+        vs = torch.rand(layers, kvh, t, device=dev) * 0.05
+        ws = torch.zeros(layers, ext.kv_decode_workspace_floats(qh, d, t), device=dev)
+        q = torch.randn(qh, d, device=dev).to(torch.bfloat16)
+        length = torch.tensor([t], dtype=torch.int32, device=dev)
+        k1 = torch.randn(kvh, 1, d, device=dev).to(torch.bfloat16)
+        pos = torch.tensor([t - 1], dtype=torch.int32, device=dev)
+
+        def step():
+            for layer in range(layers):
+                ext.kv_append(k1, k1, kc[layer], vc[layer], ks[layer], vs[layer], pos, False)
+                ext.kv_decode_attention(q, kc[layer], vc[layer], ks[layer], vs[layer], ws[layer], length, d ** -0.5)
+
+        us = _event_time_us(torch, step, reps=10) / layers
+        nbytes = 2 * kvh * t * width + 2 * kvh * t * 4
+        out[f"kv_int{bits}_append_plus_attention_ctx2048_per_layer"] = {
+            "us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1)}
+    # integer GEMM, Llama-3-8B MLP shapes
+    gemm = []
+    for n, k in ((14336, 4096), (4096, 14336)):
+        q4 = torch.randint(0, 255, (n, k // GROUP, GROUP // 2), dtype=torch.uint8, device=dev)
+        sw = torch.rand(n, k // GROUP, device=dev) * 0.01
+        for m in (128, 512, 2048):
+            x = torch.randn(m, k, device=dev).to(torch.bfloat16)
+            a, sx = ext.quant_group_codes(x, 8, GROUP, False)
+            us = _event_time_us(torch, lambda: ext.wq_gemm_a8(a, sx, q4, sw), reps=10)
+            us_q = _event_time_us(torch, lambda: ext.quant_group_codes(x, 8, GROUP, False), reps=10)
+            gemm.append({"M": m, "N": n, "K": k, "weights": "int4", "gemm_us": round(us, 1),
+                         "act_quant_us": round(us_q, 1), "TOPS": round(2 * m * n * k / us / 1e6, 1),
+                         "frac_int8_mfma_peak": round(2 * m * n * k / us / 1e6 / 5000.0, 4)})
+    out["w4a8_gemm"] = gemm
+    return out
+
+
+def decode_leg(torch):
+    """BASELINE config 5: random-init Llama-3.2-1B architecture, attention int8 / MLP int4 /
+    lm_head int8 / int8 KV cache, 512-token prompt, 256 greedy tokens, batch 1. TTFT = median
+    time of generating 1 token; decode tok/s = (n - 1) / (median time of n tokens - TTFT), the
+    reference's definition (llmquant/eval/evaluate.py:209-218). Both sides replay a captured step."""
+    import time
+
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from llmquant import QuantConfig, oneshot
+    from llmquant.runtime import graphed_generate
+
+    torch.manual_seed(0)
+    cfg = LlamaConfig(hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, num_attention_heads=32,
+                      num_key_value_heads=8, head_dim=64, vocab_size=128256, rms_norm_eps=1e-5,
+                      rope_parameters={"rope_type": "default", "rope_theta": 500000.0},
+                      tie_word_embeddings=False, max_position_embeddings=4096)
+    model = LlamaForCausalLM(cfg)
+    for p in model.parameters():
+        if p.dim() > 1:
+            torch.nn.init.normal_(p, 0, 0.02)
+    model = model.to(torch.bfloat16).to("cuda:0").eval()
+    prompt, new = 512, 256
+    ids = torch.randint(0, cfg.vocab_size, (1, prompt), generator=torch.Generator().manual_seed(1)).to("cuda:0")
+
+    def timed(fn, n):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn(n)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    def measure(fn):
+        timed(fn, 4)
+        first = sorted(timed(fn, 1) for _ in range(3))[1]
+        full = sorted(timed(fn, new) for _ in range(3))[1]
+        return {"ttft_ms": round(first * 1e3, 2), "decode_tok_s": round((new - 1) / max(full - first, 1e-9), 1)}
+
+    res = {"prompt_tokens": prompt, "new_tokens": new, "hip_graph": True}
+    res["bf16"] = measure(lambda n: graphed_generate(model, ids, n))
+    recipe = QuantConfig(attn_weight="int8", mlp_weight="int4", head_weight="int8", kv_cache="int8")
+    oneshot(model, recipe.to_modifier("kernel"))
+    res["kernel"] = measure(lambda n: graphed_generate(model, ids, n, kv_bits=8))
+    res["config"] = recipe.describe()
+    res["speedup_vs_bf16"] = round(res["kernel"]["decode_tok_s"] / res["bf16"]["decode_tok_s"], 3)
+    del model
+    torch.cuda.empty_cache()
+    return res
 
 
 def cpu_baseline(torch, cases, budget_s: float):
