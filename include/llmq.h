@@ -71,6 +71,23 @@ int llmq_wq_gemv(const void* x, const void* qweight, const float* wscale, void* 
                  int N, int G, int gs, int out_group, int wformat, int dtype,
                  llmq_stream_t stream);
 
+/* The decode-step form of llmq_wq_gemv (M = 1, group size 128): the same product with the
+ * elementwise operations that surround a Linear in a Llama decoder layer folded in, so that a
+ * layer is five launches instead of ~40. There is no counterpart in the reference, which leaves
+ * these operations to PyTorch (transformers' LlamaDecoderLayer); each is computed with the same
+ * rounding points as the PyTorch form:
+ *   prologue LLMQ_PRO_RMSNORM   x' = w * dtype(x * rsqrt(mean(x^2) + eps))     (LlamaRMSNorm)
+ *            LLMQ_PRO_SILU_MUL  x is [gate | up], x' = dtype(dtype(silu(gate)) * up)   (LlamaMLP)
+ *   in_head_dim > 0             x is [G * in_head_dim]; group g multiplies head g zero-padded to
+ *                               128, i.e. pad_activation (llmquant/quantizers/kernel.py:17-25)
+ *   residual != NULL            out = dtype(residual + dtype(y))
+ * x, norm_weight, residual, out all have element type `dtype`. */
+enum llmq_prologue { LLMQ_PRO_NONE = 0, LLMQ_PRO_RMSNORM = 1, LLMQ_PRO_SILU_MUL = 2 };
+int llmq_wq_gemv_fused(const void* x, const void* qweight, const float* wscale, void* out, int N,
+                       int G, int out_group, int wformat, int dtype, int prologue,
+                       const void* norm_weight, float eps, int in_head_dim,
+                       const void* residual_or_null, llmq_stream_t stream);
+
 /* Integer GEMM with per-group scales on both operands (the A8 branch of
  * RealQuantLinear.forward, llmquant/quantizers/real.py:76-103):
  *   out[m, n] = sum over g, in order, of  float(sum_k a[m,g,k]*q[n,g,k]) * sw[sr(n), g] * sx[m, g]
@@ -120,6 +137,24 @@ int llmq_kv_decode_attention(const void* q, const void* k_codes, const void* v_c
                              float* workspace, const int32_t* len_dev, float sm_scale,
                              int q_heads, int kv_heads, int head_dim, int t_max, int bits,
                              int dtype, llmq_stream_t stream);
+
+/* One decode step of attention for one layer in a single launch: RoPE on the new token's query
+ * and key (transformers' apply_rotary_pos_emb, same rounding points), quantize-and-append of its
+ * key and value at position *pos_dev, then attention over tokens 0 .. *pos_dev. Equivalent to
+ * RoPE in PyTorch + llmq_kv_append + llmq_kv_decode_attention; no counterpart in the reference.
+ * qkv: [(q_heads + 2*kv_heads) * head_dim] `dtype`, query heads first, then key heads, then value
+ * heads (the concatenated outputs of q_proj, k_proj, v_proj). cos_table / sin_table:
+ * [positions, head_dim] `dtype` as LlamaRotaryEmbedding produces them. out: [q_heads * head_dim].
+ * One workgroup per query head, no workspace; meant for contexts up to a few thousand tokens. */
+int llmq_kv_rope_append_attend(const void* qkv, const void* cos_table, const void* sin_table,
+                               void* k_codes, void* v_codes, float* k_scale, float* v_scale, void* out,
+                               const int32_t* pos_dev, float sm_scale, int q_heads, int kv_heads,
+                               int head_dim, int t_max, int bits, int dtype, llmq_stream_t stream);
+
+/* Index of the first maximum of a row of n elements, written to *out_index on the device: the
+ * greedy sampler of the decode loop (the reference calls logits.argmax(-1),
+ * llmquant/runtime/graph_decode.py:131). */
+int llmq_argmax_row(const void* x, int n, int64_t* out_index, int dtype, llmq_stream_t stream);
 
 #ifdef __cplusplus
 }

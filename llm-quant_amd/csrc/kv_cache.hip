@@ -112,68 +112,73 @@ constexpr int kAttnThreads = 256;
 constexpr int kAttnWaves = kAttnThreads / kWave;
 constexpr int kTokPerIter = 16;  // tokens one wave handles per step (a quad per token)
 
-template <typename T> __device__ __forceinline__ float round_through(float v);
-template <> __device__ __forceinline__ float round_through<float>(float v) { return v; }
-template <> __device__ __forceinline__ float round_through<bf16_t>(float v) {
-  return __builtin_bit_cast(float, static_cast<uint32_t>(bf16_bits_rne(v)) << 16);
-}
-template <> __device__ __forceinline__ float round_through<f16_t>(float v) {
-  return static_cast<float>(f16_rne(v));
-}
+// The code bytes of one token quarter (DPL codes), raw, and their conversion to floats.
+template <int BITS, int DPL> struct RawCodes {
+  static constexpr int kWords = DPL * BITS / 32;
+  uint32_t w[kWords];
+};
 
-// 16 (DPL = 16) codes of one token quarter as floats
 template <int BITS, int DPL>
-__device__ __forceinline__ void load_codes(const uint8_t* row, int dq, float* c) {
-  if constexpr (BITS == 8) {
+__device__ __forceinline__ RawCodes<BITS, DPL> load_raw(const uint8_t* row, int dq) {
+  RawCodes<BITS, DPL> r;
+  const uint8_t* p = row + dq * (DPL * BITS / 8);
+  if constexpr (RawCodes<BITS, DPL>::kWords % 4 == 0) {
 #pragma unroll
-    for (int p = 0; p < DPL / 16; ++p) {
-      const u32x4 w = load16(row + dq * DPL + p * 16);
-      const uint32_t d[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int b = 0; b < 4; ++b) c[p * 16 + 4 * i + b] = static_cast<float>(static_cast<int8_t>(d[i] >> (8 * b)));
+    for (int i = 0; i < RawCodes<BITS, DPL>::kWords / 4; ++i) {
+      const u32x4 v = load16(p + 16 * i);
+      r.w[4 * i] = v.x; r.w[4 * i + 1] = v.y; r.w[4 * i + 2] = v.z; r.w[4 * i + 3] = v.w;
     }
   } else {
+    const u32x2 v = *reinterpret_cast<const u32x2*>(p);
+    r.w[0] = v.x; r.w[1] = v.y;
+  }
+  return r;
+}
+
+template <int BITS, int DPL>
+__device__ __forceinline__ void decode_raw(const RawCodes<BITS, DPL>& r, float* c) {
+  if constexpr (BITS == 8) {
 #pragma unroll
-    for (int p = 0; p < DPL / 16; ++p) {
-      const u32x2 w = *reinterpret_cast<const u32x2*>(row + (dq * DPL + p * 16) / 2);
-      const uint32_t d[2] = {w.x, w.y};
+    for (int i = 0; i < DPL / 4; ++i)
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int b = 0; b < 4; ++b) c[4 * i + b] = static_cast<float>(static_cast<int8_t>(r.w[i] >> (8 * b)));
+  } else {
 #pragma unroll
-        for (int b = 0; b < 8; ++b) c[p * 16 + 8 * i + b] = static_cast<float>(static_cast<int>((d[i] >> (4 * b)) & 0xfu) - 8);
-    }
+    for (int i = 0; i < DPL / 8; ++i)
+#pragma unroll
+      for (int b = 0; b < 8; ++b) c[8 * i + b] = static_cast<float>(static_cast<int>((r.w[i] >> (4 * b)) & 0xfu) - 8);
   }
 }
 
+// The first step's operands of attend_range, for callers that can request them early.
+template <int BITS, int DPL> struct AttnPrefetch {
+  RawCodes<BITS, DPL> k, v;
+  float ks, vs;
+};
+
+template <int BITS, int DPL>
+__device__ __forceinline__ AttnPrefetch<BITS, DPL> attn_prefetch(const uint8_t* kbase, const uint8_t* vbase,
+                                                                 const float* ksc, const float* vsc, int t, int dq) {
+  constexpr int ROWB = DPL * 4 * BITS / 8;
+  AttnPrefetch<BITS, DPL> p;
+  p.k = load_raw<BITS, DPL>(kbase + static_cast<int64_t>(t) * ROWB, dq);
+  p.v = load_raw<BITS, DPL>(vbase + static_cast<int64_t>(t) * ROWB, dq);
+  p.ks = ksc[t];
+  p.vs = vsc[t];
+  return p;
+}
+
+// Online-softmax attention of one wave over tokens t_first, t_first + t_step, ... (16 tokens per
+// step, a quad of lanes per token), followed by the merge of the wave's 16 quads. On return
+// every lane with the same dq holds the wave's (max, sum, weighted output quarter) per head.
 template <typename T, int BITS, int D, int REP>
-__global__ __launch_bounds__(kAttnThreads) void kv_decode_attn_kernel(
-    const T* __restrict__ q, const uint8_t* __restrict__ k_codes, const uint8_t* __restrict__ v_codes,
-    const float* __restrict__ k_scale, const float* __restrict__ v_scale, T* __restrict__ out,
-    float* __restrict__ ws_part, int* __restrict__ ws_count, const int32_t* __restrict__ len_dev,
-    const float sm_scale_log2, const int t_max, const int chunk) {
-  constexpr int DPL = D / 4;           // head-dim elements per lane
+__device__ __forceinline__ void attend_range(const float (*qf)[D / 4], const uint8_t* kbase, const uint8_t* vbase,
+                                             const float* ksc, const float* vsc, const int t_first,
+                                             const int t_end, const int t_step, const int tk, const int dq,
+                                             float* m, float* l, float (*o)[D / 4],
+                                             const AttnPrefetch<BITS, D / 4>* first = nullptr) {
+  constexpr int DPL = D / 4;
   constexpr int ROWB = BITS == 8 ? D : D / 2;
-  constexpr int REC = D + 2;           // floats per partial record: max, sum, weighted output
-  __shared__ float s_rec[kAttnWaves][REP][REC];
-  __shared__ int s_last;
-
-  const int split = blockIdx.x, n_splits = gridDim.x, kvh = blockIdx.y;
-  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
-  const int tk = lane >> 2, dq = lane & 3;
-  const int len = min(len_dev[0], t_max);
-  const int t_begin = split * chunk, t_end = min(t_begin + chunk, len);
-
-  // this lane's quarter of each query head, pre-scaled so exp2 can be used
-  float qf[REP][DPL];
-#pragma unroll
-  for (int h = 0; h < REP; ++h)
-#pragma unroll
-    for (int i = 0; i < DPL; ++i)
-      qf[h][i] = to_float(q[(static_cast<int64_t>(kvh) * REP + h) * D + dq * DPL + i]) * sm_scale_log2;
-
-  float m[REP], l[REP], o[REP][DPL];
 #pragma unroll
   for (int h = 0; h < REP; ++h) {
     m[h] = -INFINITY;
@@ -182,18 +187,29 @@ __global__ __launch_bounds__(kAttnThreads) void kv_decode_attn_kernel(
     for (int i = 0; i < DPL; ++i) o[h][i] = 0.0f;
   }
 
-  const uint8_t* kbase = k_codes + static_cast<int64_t>(kvh) * t_max * ROWB;
-  const uint8_t* vbase = v_codes + static_cast<int64_t>(kvh) * t_max * ROWB;
-  const float* ksc = k_scale + static_cast<int64_t>(kvh) * t_max;
-  const float* vsc = v_scale + static_cast<int64_t>(kvh) * t_max;
-  for (int t0 = t_begin + wv * kTokPerIter; t0 < t_end; t0 += kAttnWaves * kTokPerIter) {
-    const int t = t0 + tk;
-    const bool ok = t < t_end;
-    const int tc = ok ? t : t_end - 1;  // clamp: loads stay in range, result dropped
+  // the loads of step i + 1 are issued before step i is computed
+  auto fetch = [&](int t0, RawCodes<BITS, DPL>& kr, RawCodes<BITS, DPL>& vr, float& ks, float& vs) {
+    const int tc = min(t0 + tk, t_end - 1);  // clamp: loads stay in range, result dropped
+    kr = load_raw<BITS, DPL>(kbase + static_cast<int64_t>(tc) * ROWB, dq);
+    vr = load_raw<BITS, DPL>(vbase + static_cast<int64_t>(tc) * ROWB, dq);
+    ks = ksc[tc];
+    vs = vsc[tc];
+  };
+  RawCodes<BITS, DPL> k_next, v_next;
+  float ks_next = 0.0f, vs_next = 0.0f;
+  if (first != nullptr) {
+    k_next = first->k; v_next = first->v; ks_next = first->ks; vs_next = first->vs;
+  } else if (t_first < t_end) {
+    fetch(t_first, k_next, v_next, ks_next, vs_next);
+  }
+  for (int t0 = t_first; t0 < t_end; t0 += t_step) {
+    const bool ok = t0 + tk < t_end;
+    const RawCodes<BITS, DPL> k_now = k_next, v_now = v_next;
+    const float ks = ks_next, vs = vs_next;
+    if (t0 + t_step < t_end) fetch(t0 + t_step, k_next, v_next, ks_next, vs_next);
     float kc[DPL], vc[DPL];
-    load_codes<BITS, DPL>(kbase + static_cast<int64_t>(tc) * ROWB, dq, kc);
-    load_codes<BITS, DPL>(vbase + static_cast<int64_t>(tc) * ROWB, dq, vc);
-    const float ks = ksc[tc], vs = vsc[tc];
+    decode_raw<BITS, DPL>(k_now, kc);
+    decode_raw<BITS, DPL>(v_now, vc);
     float s[REP];
 #pragma unroll
     for (int h = 0; h < REP; ++h) s[h] = 0.0f;
@@ -248,6 +264,40 @@ __global__ __launch_bounds__(kAttnThreads) void kv_decode_attn_kernel(
       m[h] = m_new;
     }
   }
+}
+
+template <typename T, int BITS, int D, int REP>
+__global__ __launch_bounds__(kAttnThreads) void kv_decode_attn_kernel(
+    const T* __restrict__ q, const uint8_t* __restrict__ k_codes, const uint8_t* __restrict__ v_codes,
+    const float* __restrict__ k_scale, const float* __restrict__ v_scale, T* __restrict__ out,
+    float* __restrict__ ws_part, int* __restrict__ ws_count, const int32_t* __restrict__ len_dev,
+    const float sm_scale_log2, const int t_max, const int chunk) {
+  constexpr int DPL = D / 4;           // head-dim elements per lane
+  constexpr int ROWB = BITS == 8 ? D : D / 2;
+  constexpr int REC = D + 2;           // floats per partial record: max, sum, weighted output
+  __shared__ float s_rec[kAttnWaves][REP][REC];
+  __shared__ int s_last;
+
+  const int split = blockIdx.x, n_splits = gridDim.x, kvh = blockIdx.y;
+  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+  const int tk = lane >> 2, dq = lane & 3;
+  const int len = min(len_dev[0], t_max);
+  const int t_begin = split * chunk, t_end = min(t_begin + chunk, len);
+
+  // this lane's quarter of each query head, pre-scaled so exp2 can be used
+  float qf[REP][DPL];
+#pragma unroll
+  for (int h = 0; h < REP; ++h)
+#pragma unroll
+    for (int i = 0; i < DPL; ++i)
+      qf[h][i] = to_float(q[(static_cast<int64_t>(kvh) * REP + h) * D + dq * DPL + i]) * sm_scale_log2;
+
+  float m[REP], l[REP], o[REP][DPL];
+  attend_range<T, BITS, D, REP>(qf, k_codes + static_cast<int64_t>(kvh) * t_max * ROWB,
+                                v_codes + static_cast<int64_t>(kvh) * t_max * ROWB,
+                                k_scale + static_cast<int64_t>(kvh) * t_max,
+                                v_scale + static_cast<int64_t>(kvh) * t_max, t_begin + wv * kTokPerIter, t_end,
+                                kAttnWaves * kTokPerIter, tk, dq, m, l, o);
   if (tk == 0) {
 #pragma unroll
     for (int h = 0; h < REP; ++h) {
@@ -307,6 +357,196 @@ __global__ __launch_bounds__(kAttnThreads) void kv_decode_attn_kernel(
     out[(static_cast<int64_t>(kvh) * REP + h) * D + d] = from_float<T>(ll > 0.0f ? oo / ll : 0.0f);
   }
   if (threadIdx.x == 0) ws_count[kvh] = 0;  // ready for the next launch
+}
+
+// ---- one decode step of attention in one launch ----------------------------------------------------
+// RoPE on the new token's query and key, quantize-and-append of its key and value, and
+// attention over the whole cache including that token. One workgroup of 16 waves per QUERY
+// head: a wave step covers 16 tokens, so a workgroup covers 256 tokens per step and a context
+// of a few thousand tokens is a handful of steps, each with the next step's loads already in
+// flight. Nothing crosses workgroups: every workgroup rotates and quantizes the new token's
+// key and value itself (64 values; the one whose query head is the first of its kv head also
+// writes them to the cache) and attends to that token from LDS, to the older ones from the
+// cache. The cache codes of a kv head are therefore read by its 4 query-head workgroups, from
+// L2 after the first. RoPE follows transformers' apply_rotary_pos_emb with its rounding
+// points: dtype(dtype(x * cos) + dtype(rotate_half(x) * sin)).
+constexpr int kFusedWaves = 16;
+constexpr int kFusedThreads = kFusedWaves * kWave;
+
+template <typename T, int D>
+__device__ __forceinline__ float rope_element(const T* x, const T* cos_row, const T* sin_row, int i) {
+  const float xi = to_float(x[i]);
+  const float rot = i < D / 2 ? -to_float(x[i + D / 2]) : to_float(x[i - D / 2]);
+  const float a = round_through<T>(xi * to_float(cos_row[i]));
+  const float b = round_through<T>(rot * to_float(sin_row[i]));
+  return round_through<T>(a + b);
+}
+
+template <typename T, int BITS, int D>
+__global__ __launch_bounds__(kFusedThreads) void kv_rope_append_attend_kernel(
+    const T* __restrict__ qkv, const T* __restrict__ cos_table, const T* __restrict__ sin_table,
+    uint8_t* __restrict__ k_codes, uint8_t* __restrict__ v_codes, float* __restrict__ k_scale,
+    float* __restrict__ v_scale, T* __restrict__ out, const int32_t* __restrict__ pos_dev,
+    const float sm_scale_log2, const int q_heads, const int kv_heads, const int t_max) {
+  constexpr int DPL = D / 4;
+  constexpr int ROWB = BITS == 8 ? D : D / 2;
+  constexpr int REC = D + 2;
+  __shared__ float s_q[D];
+  __shared__ float s_new[2][D];  // the new token's key and value as the cache will return them
+  __shared__ float s_rec[kFusedWaves][REC];
+
+  const int qh = blockIdx.x;
+  const int rep = q_heads / kv_heads;
+  const int kvh = qh / rep;
+  const bool writer = qh % rep == 0;
+  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+  const int tk = lane >> 2, dq = lane & 3;
+  const int pos = min(max(pos_dev[0], 0), t_max - 1);
+  const T* cos_row = cos_table + static_cast<int64_t>(pos) * D;
+  const T* sin_row = sin_table + static_cast<int64_t>(pos) * D;
+
+  // the cache reads of the first attention step do not depend on phase A: request them now
+  const uint8_t* kbase = k_codes + static_cast<int64_t>(kvh) * t_max * ROWB;
+  const uint8_t* vbase = v_codes + static_cast<int64_t>(kvh) * t_max * ROWB;
+  const float* ksc = k_scale + static_cast<int64_t>(kvh) * t_max;
+  const float* vsc = v_scale + static_cast<int64_t>(kvh) * t_max;
+  const int t_mine = wv * kTokPerIter;
+  AttnPrefetch<BITS, DPL> first;
+  if (t_mine < pos) first = attn_prefetch<BITS, DPL>(kbase, vbase, ksc, vsc, min(t_mine + tk, pos - 1), dq);
+
+  // ---- phase A: wave 0 rotates the query, wave 1 rotates + quantizes K, wave 2 quantizes V ------------
+  if (wv == 0) {
+    const T* q = qkv + static_cast<int64_t>(qh) * D;
+    for (int i = lane; i < D; i += kWave) s_q[i] = rope_element<T, D>(q, cos_row, sin_row, i) * sm_scale_log2;
+  } else if (wv <= 2) {
+    const bool is_v = wv == 2;
+    const T* src = qkv + (static_cast<int64_t>(q_heads) + (is_v ? kv_heads : 0) + kvh) * D;
+    const float qmax = static_cast<float>((1 << (BITS - 1)) - 1);
+    const float qmin = -qmax - 1.0f;
+    float f[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int d = lane + e * kWave;
+      f[e] = 0.0f;
+      if (d < D) f[e] = is_v ? to_float(src[d]) : rope_element<T, D>(src, cos_row, sin_row, d);
+    }
+    const float amax = group_max<kWave>(fmaxf(fabsf(f[0]), fabsf(f[1])));
+    const float scale = scale_from_amax(amax, qmax);
+    const int64_t slot = static_cast<int64_t>(kvh) * t_max + pos;
+    if (writer && lane == 0) (is_v ? v_scale : k_scale)[slot] = scale;
+    uint8_t* codes = is_v ? v_codes : k_codes;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int d = lane + e * kWave;
+      const float qv = quant_code(f[e], scale, qmin, qmax);
+      if (d < D) s_new[is_v ? 1 : 0][d] = round_through<T>(qv * scale);
+      const int code = static_cast<int>(qv);
+      if constexpr (BITS == 8) {
+        if (writer && d < D) codes[slot * D + d] = static_cast<uint8_t>(code);
+      } else {
+        const int mine = (code + 8) & 0xf;
+        const int other = __shfl_xor(mine, 1, kWave);
+        if (writer && (lane & 1) == 0 && d < D) codes[slot * (D / 2) + d / 2] = static_cast<uint8_t>(mine | (other << 4));
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- phase B: tokens 0 .. pos-1 from the cache, token pos from LDS -------------------------------------
+  float qf[1][DPL];
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) qf[0][i] = s_q[dq * DPL + i];
+  float m[1], l[1], o[1][DPL];
+  attend_range<T, BITS, D, 1>(qf, kbase, vbase, ksc, vsc, t_mine, pos, kFusedWaves * kTokPerIter, tk, dq, m, l, o,
+                              &first);
+  if (wv == kFusedWaves - 1) {
+    // every lane with the same dq holds the same merged record; fold the new token into it
+    float sc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) sc = fmaf(qf[0][i], s_new[0][dq * DPL + i], sc);
+    sc += __shfl_xor(sc, 1, kWave);
+    sc += __shfl_xor(sc, 2, kWave);
+    const float m_new = fmaxf(m[0], sc);
+    const float corr = m[0] == -INFINITY ? 0.0f : exp2f(m[0] - m_new);
+    const float pnew = exp2f(sc - m_new);
+    l[0] = l[0] * corr + pnew;
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) o[0][i] = fmaf(pnew, s_new[1][dq * DPL + i], o[0][i] * corr);
+    m[0] = m_new;
+  }
+  if (tk == 0) {
+    if (dq == 0) {
+      s_rec[wv][0] = m[0];
+      s_rec[wv][1] = l[0];
+    }
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) s_rec[wv][2 + dq * DPL + i] = o[0][i];
+  }
+  __syncthreads();
+  if (threadIdx.x < D) {
+    const int d = threadIdx.x;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kFusedWaves; ++w) mm = fmaxf(mm, s_rec[w][0]);
+    float ll = 0.0f, oo = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kFusedWaves; ++w) {
+      const float a = s_rec[w][0] == -INFINITY ? 0.0f : exp2f(s_rec[w][0] - mm);
+      ll += s_rec[w][1] * a;
+      oo += s_rec[w][2 + d] * a;
+    }
+    out[static_cast<int64_t>(qh) * D + d] = from_float<T>(ll > 0.0f ? oo / ll : 0.0f);
+  }
+}
+
+// ---- argmax of one row (the greedy sampler of the decode loop) ------------------------------------------
+// First index of the maximum, like torch.argmax on a row without ties broken otherwise.
+template <typename T>
+__global__ __launch_bounds__(1024) void argmax_row_kernel(const T* __restrict__ x, const int n, int64_t* __restrict__ out) {
+  __shared__ float s_val[16];
+  __shared__ int s_idx[16];
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  constexpr int V = Pack<T>::N;
+  const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+  const int n_vec = aligned ? n / V : 0;
+  // 16-byte packets, two in flight per thread; a thread sees its indices in increasing order, so
+  // a strict '>' keeps the first maximum
+  for (int p = threadIdx.x; p < n_vec; p += 2 * blockDim.x) {
+    float f[2][V];
+    const int p2 = p + blockDim.x;
+    Pack<T>::unpack(load16(x + static_cast<int64_t>(p) * V), f[0]);
+    if (p2 < n_vec) Pack<T>::unpack(load16(x + static_cast<int64_t>(p2) * V), f[1]);
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      if (f[0][e] > best) { best = f[0][e]; best_i = p * V + e; }
+    }
+    if (p2 < n_vec) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        if (f[1][e] > best) { best = f[1][e]; best_i = p2 * V + e; }
+      }
+    }
+  }
+  for (int i = n_vec * V + threadIdx.x; i < n; i += blockDim.x) {
+    const float v = to_float(x[i]);
+    if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+  }
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off, kWave);
+    const int oi = __shfl_xor(best_i, off, kWave);
+    if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+  }
+  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+  if (lane == 0) { s_val[wv] = best; s_idx[wv] = best_i; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < static_cast<int>(blockDim.x) / kWave; ++w) {
+      if (s_val[w] > best || (s_val[w] == best && s_idx[w] < best_i)) { best = s_val[w]; best_i = s_idx[w]; }
+    }
+    out[0] = best_i == 0x7fffffff ? 0 : best_i;
+  }
 }
 
 int splits_for(int t_max) {
@@ -433,4 +673,53 @@ extern "C" int llmq_kv_decode_attention(const void* q, const void* k_codes, cons
 #undef LLMQ_BD
 #undef LLMQ_GO
   return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+}
+
+extern "C" int llmq_kv_rope_append_attend(const void* qkv, const void* cos_table, const void* sin_table,
+                                          void* k_codes, void* v_codes, float* k_scale, float* v_scale,
+                                          void* out, const int32_t* pos_dev, float sm_scale, int q_heads,
+                                          int kv_heads, int head_dim, int t_max, int bits, int dtype,
+                                          llmq_stream_t stream) {
+  if (bits != 8 && bits != 4) return llmq_host::fail_invalid("KV cache bits must be 8 or 4, got %d", bits);
+  if (head_dim != 64 && head_dim != 128) return llmq_host::fail_invalid("head_dim must be 64 or 128, got %d", head_dim);
+  if (kv_heads <= 0 || q_heads <= 0 || q_heads % kv_heads)
+    return llmq_host::fail_invalid("q_heads %d must be a positive multiple of kv_heads %d", q_heads, kv_heads);
+  if (t_max <= 0) return llmq_host::fail_invalid("t_max must be positive, got %d", t_max);
+  if (!qkv || !cos_table || !sin_table || !k_codes || !v_codes || !k_scale || !v_scale || !out || !pos_dev)
+    return llmq_host::fail_invalid("null tensor pointer");
+  if ((reinterpret_cast<uintptr_t>(k_codes) | reinterpret_cast<uintptr_t>(v_codes)) & 15u)
+    return llmq_host::fail_invalid("cache code pointers must be 16-byte aligned");
+  const float scale_log2 = sm_scale * 1.4426950408889634f;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(q_heads), block(kFusedThreads);
+#define LLMQ_FUSED(T, B, D)                                                                      \
+  hipLaunchKernelGGL((kv_rope_append_attend_kernel<T, B, D>), grid, block, 0, s, static_cast<const T*>(qkv), \
+                     static_cast<const T*>(cos_table), static_cast<const T*>(sin_table),          \
+                     static_cast<uint8_t*>(k_codes), static_cast<uint8_t*>(v_codes), k_scale, v_scale, \
+                     static_cast<T*>(out), pos_dev, scale_log2, q_heads, kv_heads, t_max)
+#define LLMQ_FUSED_BD(T)                                                                         \
+  if (bits == 8) { if (head_dim == 64) { LLMQ_FUSED(T, 8, 64); } else { LLMQ_FUSED(T, 8, 128); } } \
+  else { if (head_dim == 64) { LLMQ_FUSED(T, 4, 64); } else { LLMQ_FUSED(T, 4, 128); } }
+  switch (dtype) {
+    case LLMQ_F32: LLMQ_FUSED_BD(float) break;
+    case LLMQ_F16: LLMQ_FUSED_BD(f16_t) break;
+    case LLMQ_BF16: LLMQ_FUSED_BD(bf16_t) break;
+    default: return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+  }
+#undef LLMQ_FUSED_BD
+#undef LLMQ_FUSED
+  return llmq_host::check_launch("kv_rope_append_attend_kernel");
+}
+
+extern "C" int llmq_argmax_row(const void* x, int n, int64_t* out_index, int dtype, llmq_stream_t stream) {
+  if (n <= 0) return llmq_host::fail_invalid("argmax of an empty row");
+  if (!x || !out_index) return llmq_host::fail_invalid("null tensor pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case LLMQ_F32: hipLaunchKernelGGL((argmax_row_kernel<float>), dim3(1), dim3(1024), 0, s, static_cast<const float*>(x), n, out_index); break;
+    case LLMQ_F16: hipLaunchKernelGGL((argmax_row_kernel<f16_t>), dim3(1), dim3(1024), 0, s, static_cast<const f16_t*>(x), n, out_index); break;
+    case LLMQ_BF16: hipLaunchKernelGGL((argmax_row_kernel<bf16_t>), dim3(1), dim3(1024), 0, s, static_cast<const bf16_t*>(x), n, out_index); break;
+    default: return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+  }
+  return llmq_host::check_launch("argmax_row_kernel");
 }

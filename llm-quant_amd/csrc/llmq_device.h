@@ -44,6 +44,16 @@ template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
   return bf16_t{bf16_bits_rne(f)};
 }
 
+// The value after a round trip through storage type T (what a tensor of that dtype would hold).
+template <typename T> __device__ __forceinline__ float round_through(float v);
+template <> __device__ __forceinline__ float round_through<float>(float v) { return v; }
+template <> __device__ __forceinline__ float round_through<bf16_t>(float v) {
+  return __builtin_bit_cast(float, static_cast<uint32_t>(bf16_bits_rne(v)) << 16);
+}
+template <> __device__ __forceinline__ float round_through<f16_t>(float v) {
+  return static_cast<float>(f16_rne(v));
+}
+
 // ---- 128-bit access ---------------------------------------------------------------------
 struct alignas(16) u32x4 { uint32_t x, y, z, w; };
 struct alignas(8) u32x2 { uint32_t x, y; };
@@ -145,4 +155,7 @@ bool gemv_mfma_supported(const void* x, const void* qw, const float* ws, int M, 
                          int wformat);
 int gemv_mfma_launch(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
                      int out_group, int wformat, int dtype, hipStream_t stream);
+int gemv_mfma_launch_fused(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
+                           int out_group, int wformat, int dtype, int prologue, const void* norm_weight,
+                           float eps, int in_head_dim, const void* residual, hipStream_t stream);
 }  // namespace llmq_host

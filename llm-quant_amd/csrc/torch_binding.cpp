@@ -136,6 +136,53 @@ at::Tensor wq_gemv(const at::Tensor& x, const at::Tensor& qweight, const at::Ten
   return out;
 }
 
+// One activation row through a quantized Linear with the surrounding elementwise operations
+// folded in (see llmq_wq_gemv_fused). x: [K] (or [2K] gate|up for prologue 2); returns [N].
+at::Tensor wq_gemv_fused(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale,
+                         int64_t out_group, int64_t prologue, const c10::optional<at::Tensor>& norm_weight,
+                         double eps, int64_t in_head_dim, const c10::optional<at::Tensor>& residual) {
+  TORCH_CHECK(x.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "all tensors must be CUDA");
+  TORCH_CHECK(qweight.dim() == 3 && qweight.is_contiguous(), "qweight must be contiguous [N, groups, group_size]");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 2 && wscale.is_contiguous(),
+              "wscale must be contiguous float32 [scale_rows, groups]");
+  TORCH_CHECK(x.is_contiguous(), "x must be contiguous");
+  const int dtype = dtype_code(x, "x");
+  const int64_t N = qweight.size(0), groups = qweight.size(1);
+  const int64_t group_size = packed ? qweight.size(2) * 2 : qweight.size(2);
+  TORCH_CHECK(group_size == 128, "the fused GEMV needs group_size 128, got ", group_size);
+  const int64_t k_real = in_head_dim > 0 ? groups * in_head_dim : groups * group_size;
+  TORCH_CHECK(x.numel() == (prologue == LLMQ_PRO_SILU_MUL ? 2 * k_real : k_real), "x has ", x.numel(),
+              " elements, expected ", prologue == LLMQ_PRO_SILU_MUL ? 2 * k_real : k_real);
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  TORCH_CHECK(wscale.size(0) == scale_rows && wscale.size(1) == groups, "wscale must be [", scale_rows, ", ", groups, "]");
+  const void* norm_ptr = nullptr;
+  if (prologue == LLMQ_PRO_RMSNORM) {
+    TORCH_CHECK(norm_weight.has_value() && norm_weight->is_cuda() && norm_weight->is_contiguous() &&
+                    norm_weight->numel() == k_real && norm_weight->scalar_type() == x.scalar_type(),
+                "the RMSNorm prologue needs a contiguous weight of x's dtype with ", k_real, " elements");
+    norm_ptr = norm_weight->const_data_ptr();
+  }
+  const void* res_ptr = nullptr;
+  if (residual.has_value() && residual->defined()) {
+    TORCH_CHECK(residual->is_cuda() && residual->is_contiguous() && residual->numel() == N &&
+                    residual->scalar_type() == x.scalar_type(),
+                "residual must be a contiguous tensor of x's dtype with ", N, " elements");
+    res_ptr = residual->const_data_ptr();
+  }
+  auto out = at::empty({1, N}, x.options());
+  if (N == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(x));
+  check_rc(llmq_wq_gemv_fused(x.const_data_ptr(), qweight.const_data_ptr(), wscale.const_data_ptr<float>(),
+                              out.mutable_data_ptr(), static_cast<int>(N), static_cast<int>(groups),
+                              static_cast<int>(out_group), packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype,
+                              static_cast<int>(prologue), norm_ptr, static_cast<float>(eps),
+                              static_cast<int>(in_head_dim), res_ptr, current_stream(x)),
+           "wq_gemv_fused");
+  return out;
+}
+
 // Integer GEMM: a int8 [M, K], sx fp32 [M, G]; qweight / wscale as for wq_gemv; optional fp32 or
 // half-width bias (converted to fp32 here, as RealQuantLinear adds bias.float()).
 at::Tensor wq_gemm_a8(const at::Tensor& a, const at::Tensor& sx, const at::Tensor& qweight,
@@ -290,6 +337,48 @@ at::Tensor kv_decode_attention(const at::Tensor& query, const at::Tensor& k_code
   return out;
 }
 
+// qkv: [(q_heads + 2*kv_heads) * head_dim]; returns the attention output [1, q_heads * head_dim].
+at::Tensor kv_rope_append_attend(const at::Tensor& qkv, const at::Tensor& cos_table, const at::Tensor& sin_table,
+                                 at::Tensor& k_codes, at::Tensor& v_codes, at::Tensor& k_scale, at::Tensor& v_scale,
+                                 const at::Tensor& position, double sm_scale, int64_t q_heads) {
+  TORCH_CHECK(qkv.is_cuda() && qkv.is_contiguous(), "qkv must be a contiguous CUDA tensor");
+  const int dtype = dtype_code(qkv, "qkv");
+  const CacheGeometry g = cache_geometry(k_codes, k_scale, "key");
+  const CacheGeometry gv = cache_geometry(v_codes, v_scale, "value");
+  TORCH_CHECK(g.kv_heads == gv.kv_heads && g.t_max == gv.t_max && g.head_dim == gv.head_dim && g.bits == gv.bits,
+              "key and value caches differ in geometry");
+  TORCH_CHECK(qkv.numel() == (q_heads + 2 * g.kv_heads) * g.head_dim, "qkv has ", qkv.numel(), " elements, expected ",
+              (q_heads + 2 * g.kv_heads) * g.head_dim);
+  for (const at::Tensor* t : {&cos_table, &sin_table}) {
+    TORCH_CHECK(t->is_cuda() && t->is_contiguous() && t->dim() == 2 && t->size(1) == g.head_dim &&
+                    t->size(0) >= g.t_max && t->scalar_type() == qkv.scalar_type(),
+                "cos/sin tables must be contiguous [>= t_max, head_dim] tensors of qkv's dtype");
+  }
+  check_position(position);
+  auto out = at::empty({1, q_heads * g.head_dim}, qkv.options());
+  const c10::OptionalDeviceGuard guard(at::device_of(qkv));
+  check_rc(llmq_kv_rope_append_attend(qkv.const_data_ptr(), cos_table.const_data_ptr(), sin_table.const_data_ptr(),
+                                      k_codes.mutable_data_ptr(), v_codes.mutable_data_ptr(),
+                                      k_scale.mutable_data_ptr<float>(), v_scale.mutable_data_ptr<float>(),
+                                      out.mutable_data_ptr(), position.const_data_ptr<int32_t>(),
+                                      static_cast<float>(sm_scale), static_cast<int>(q_heads), g.kv_heads,
+                                      g.head_dim, g.t_max, g.bits, dtype, current_stream(qkv)),
+           "kv_rope_append_attend");
+  return out;
+}
+
+// x: one row (any shape, contiguous); returns a [1] int64 tensor with the index of its first maximum.
+at::Tensor argmax_row(const at::Tensor& x) {
+  TORCH_CHECK(x.is_cuda() && x.is_contiguous() && x.numel() > 0, "x must be a non-empty contiguous CUDA tensor");
+  const int dtype = dtype_code(x, "x");
+  auto out = at::empty({1}, x.options().dtype(at::kLong));
+  const c10::OptionalDeviceGuard guard(at::device_of(x));
+  check_rc(llmq_argmax_row(x.const_data_ptr(), static_cast<int>(x.numel()), out.mutable_data_ptr<int64_t>(), dtype,
+                           current_stream(x)),
+           "argmax_row");
+  return out;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -302,6 +391,16 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("wq_gemv", &wq_gemv,
         "Weight-only quantized matmul for a few rows: int8 or packed-int4 weight (HIP, gfx950)",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0);
+  m.def("wq_gemv_fused", &wq_gemv_fused,
+        "One-row quantized Linear with RMSNorm / SiLU*up prologue, head padding and residual epilogue",
+        py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("prologue") = 0,
+        py::arg("norm_weight") = py::none(), py::arg("eps") = 0.0, py::arg("in_head_dim") = 0,
+        py::arg("residual") = py::none());
+  m.def("kv_rope_append_attend", &kv_rope_append_attend,
+        "RoPE + KV quantize-append + attention for one decode token of one layer, one launch",
+        py::arg("qkv"), py::arg("cos_table"), py::arg("sin_table"), py::arg("k_codes"), py::arg("v_codes"),
+        py::arg("k_scale"), py::arg("v_scale"), py::arg("position"), py::arg("sm_scale"), py::arg("q_heads"));
+  m.def("argmax_row", &argmax_row, "Index of the first maximum of one row", py::arg("x"));
   m.def("wq_gemm_a8", &wq_gemm_a8,
         "Integer GEMM: int8 activations x int4/int8 group-quantized weights, real-mode rounding order",
         py::arg("a"), py::arg("sx"), py::arg("qweight"), py::arg("wscale"), py::arg("bias") = py::none(),

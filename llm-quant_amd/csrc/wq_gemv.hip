@@ -355,3 +355,28 @@ extern "C" int llmq_wq_gemv(const void* x, const void* qweight, const float* wsc
              ? launch_bits<8>(x, qweight, wscale, out, M, N, G, gs, out_group, dtype, s)
              : launch_bits<4>(x, qweight, wscale, out, M, N, G, gs, out_group, dtype, s);
 }
+
+extern "C" int llmq_wq_gemv_fused(const void* x, const void* qweight, const float* wscale, void* out,
+                                  int N, int G, int out_group, int wformat, int dtype, int prologue,
+                                  const void* norm_weight, float eps, int in_head_dim,
+                                  const void* residual_or_null, llmq_stream_t stream) {
+  if (N < 0 || G <= 0) return llmq_host::fail_invalid("bad dimension N=%d G=%d", N, G);
+  if (wformat != LLMQ_W_INT8 && wformat != LLMQ_W_INT4_PACKED)
+    return llmq_host::fail_invalid("unsupported weight format %d, expected 8 or 4", wformat);
+  if (prologue != LLMQ_PRO_NONE && prologue != LLMQ_PRO_RMSNORM && prologue != LLMQ_PRO_SILU_MUL)
+    return llmq_host::fail_invalid("unknown prologue %d", prologue);
+  if (prologue == LLMQ_PRO_RMSNORM && norm_weight == nullptr)
+    return llmq_host::fail_invalid("the RMSNorm prologue needs its weight");
+  if (in_head_dim < 0 || in_head_dim > 128 || in_head_dim % 8)
+    return llmq_host::fail_invalid("in_head_dim must be a multiple of 8 in [0, 128], got %d", in_head_dim);
+  if (in_head_dim > 0 && prologue != LLMQ_PRO_NONE)
+    return llmq_host::fail_invalid("head padding cannot be combined with a prologue");
+  if (N == 0) return 0;
+  if (!x || !qweight || !wscale || !out) return llmq_host::fail_invalid("null tensor pointer");
+  if (!llmq_host::gemv_mfma_supported(x, qweight, wscale, 1, G, 128, wformat))
+    return llmq_host::fail_invalid("the fused GEMV needs group size 128, a multiple of 4 groups (at most 64) "
+                                   "and 16-byte aligned operands");
+  return llmq_host::gemv_mfma_launch_fused(x, qweight, wscale, out, 1, N, G, out_group, wformat, dtype, prologue,
+                                           norm_weight, eps, in_head_dim, residual_or_null,
+                                           static_cast<hipStream_t>(stream));
+}

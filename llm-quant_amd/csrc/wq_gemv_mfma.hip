@@ -53,6 +53,12 @@ struct MfmaArgs {
   int N, G, out_group;
   int n_tiles;
   int row_bytes;  // bytes of one weight row
+  // what happens to x before it is multiplied (M == 1 only) and to y after; see llmq_wq_gemv_fused
+  int prologue;              // LLMQ_PRO_*
+  const void* norm_weight;   // [K] for LLMQ_PRO_RMSNORM
+  float eps;
+  int in_head_dim;           // > 0: x is [G * in_head_dim]; group g takes head g, zero-padded to 128
+  const void* residual;      // [N] or null: out = residual + y, both rounded like the model dtype
 };
 
 template <typename T> __device__ __forceinline__ void load8(const T* p, float* f) {
@@ -73,16 +79,31 @@ __device__ __forceinline__ int row16_sum(int v) {
 // LDS carve-up, shared by host (size) and device (offsets).
 struct LdsLayout {
   int plane;     // bytes of one digit plane of one activation row
-  int dig_off, cx_off, csum_off, part_off, total;
+  int dig_off, red_off, cx_off, csum_off, part_off, total;
   __host__ __device__ LdsLayout(int M, int G, int wk, bool need_csum) {
     plane = G * kGroup + kPlanePad;
     dig_off = 0;
-    cx_off = (kDigits * M * plane + 15) & ~15;
+    red_off = (kDigits * M * plane + 15) & ~15;
+    cx_off = red_off + 64;
     csum_off = cx_off + M * G * 4;
     part_off = csum_off + (need_csum ? kDigits * M * G * 4 : 0);
     part_off = (part_off + 15) & ~15;
     total = part_off + 2 * wk * kDigits * M * kTileRows * 4;
   }
+};
+
+template <typename T>
+__device__ __forceinline__ T finish(float total, const void* residual, int64_t n) {
+  if (residual == nullptr) return from_float<T>(total);
+  // hidden = residual + linear(x): the Linear's output is rounded to the model dtype first
+  return from_float<T>(to_float(static_cast<const T*>(residual)[n]) + round_through<T>(total));
+}
+
+struct Prologue {
+  int kind;
+  const void* norm_weight;
+  float eps;
+  int in_head_dim;
 };
 
 // The activation as integers, whole workgroup, into LDS: per (row m, group g) the digits of
@@ -91,9 +112,38 @@ struct LdsLayout {
 // Every thread of the block must call it; the caller synchronises afterwards.
 template <typename T, int BITS, int M>
 __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const int G, const LdsLayout& L,
-                                                 int8_t* dig, float* cxs, int* csum) {
+                                                 int8_t* dig, float* cxs, int* csum, const Prologue pro,
+                                                 float* red) {
   const int tid = threadIdx.x;
   const int items = M * G * 16;  // 8 elements each; 16 consecutive items are one group
+  const int real_per_group = pro.in_head_dim > 0 ? pro.in_head_dim : kGroup;
+  const int k_real = G * real_per_group;
+
+  // RMSNorm (transformers' LlamaRMSNorm.forward): variance of the whole row in fp32 first
+  float inv_rms = 0.0f;
+  float w_first[8], x_first[8];  // this thread's first item: weights requested before the barrier, x kept
+#pragma unroll
+  for (int e = 0; e < 8; ++e) w_first[e] = x_first[e] = 0.0f;
+  if (pro.kind == LLMQ_PRO_RMSNORM) {
+    if (tid < items) load8<T>(static_cast<const T*>(pro.norm_weight) + static_cast<int64_t>(tid) * 8, w_first);
+    float ss = 0.0f;
+    for (int i = tid * 8; i < k_real; i += blockDim.x * 8) {
+      float f[8];
+      load8<T>(x + i, f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        ss = fmaf(f[e], f[e], ss);
+        if (i == tid * 8) x_first[e] = f[e];  // this thread's first item: no second load
+      }
+    }
+    ss = wave_sum(ss);
+    if ((tid & (kWave - 1)) == 0) red[tid / kWave] = ss;
+    __syncthreads();
+    float total = 0.0f;
+    for (int w = 0; w < static_cast<int>(blockDim.x) / kWave; ++w) total += red[w];
+    inv_rms = rsqrtf(total / static_cast<float>(k_real) + pro.eps);
+  }
+
   for (int base = 0; base < items; base += blockDim.x) {
     const int item = base + tid;
     const bool active = item < items;
@@ -101,11 +151,38 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
     const int mg = active ? item >> 4 : 0;  // m * G + g
     const int m = mg / G, g = mg - m * G;
     float f[8];
-    if (active) {
-      load8<T>(x + static_cast<int64_t>(m) * G * kGroup + g * kGroup + tq * 8, f);
-    } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) f[e] = 0.0f;
+    for (int e = 0; e < 8; ++e) f[e] = 0.0f;
+    const bool real = active && tq * 8 < real_per_group;  // beyond it: the zero padding of a head group
+    if (real) {
+      const int64_t src = static_cast<int64_t>(m) * k_real + g * real_per_group + tq * 8;
+      if (pro.kind == LLMQ_PRO_RMSNORM && base == 0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = x_first[e];
+      } else {
+        load8<T>(x + src, f);
+      }
+      if (pro.kind == LLMQ_PRO_RMSNORM) {
+        // (a prologue excludes head padding, so item i covers elements 8i .. 8i+7 of the row)
+        float w[8];
+        if (base == 0) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) w[e] = w_first[e];
+        } else {
+          load8<T>(static_cast<const T*>(pro.norm_weight) + src, w);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = round_through<T>(w[e] * round_through<T>(f[e] * inv_rms));
+      } else if (pro.kind == LLMQ_PRO_SILU_MUL) {
+        // x holds gate then up: act_fn(gate) * up with both results rounded to the model dtype
+        float up[8];
+        load8<T>(x + k_real + src, up);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float silu = f[e] / (1.0f + expf(-f[e]));
+          f[e] = round_through<T>(round_through<T>(silu) * up[e]);
+        }
+      }
     }
     float amax = 0.0f;
 #pragma unroll
@@ -168,6 +245,7 @@ __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
   const LdsLayout L(M, G, wk, BITS == 4);
   int8_t* dig = reinterpret_cast<int8_t*>(smem + L.dig_off);
   float* cxs = reinterpret_cast<float*>(smem + L.cx_off);
+  float* red = reinterpret_cast<float*>(smem + L.red_off);
   int* csum = reinterpret_cast<int*>(smem + L.csum_off);
   float* part = reinterpret_cast<float*>(smem + L.part_off);
 
@@ -202,7 +280,8 @@ __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
   int tile = blockIdx.x;
   if (tile < a.n_tiles) issue_loads(tile);  // in flight while the activation is prepared
 
-  stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum);
+  stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum,
+                               Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim}, red);
   __syncthreads();
 
   // ---- phase 2: this wave's operands and constants, into registers --------------------------
@@ -288,7 +367,7 @@ __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
         total += __shfl_xor(total, 16, kWave);
         total += __shfl_xor(total, 32, kWave);
         const int n = tile * kTileRows + jj;
-        if (ws == 0 && n < a.N) out[static_cast<int64_t>(r) * a.N + n] = from_float<T>(total);
+        if (ws == 0 && n < a.N) out[static_cast<int64_t>(r) * a.N + n] = finish<T>(total, a.residual, n);
       }
     }
     buf ^= 1;
@@ -314,6 +393,7 @@ __global__ __launch_bounds__(256, 4) void wq_gemv_mfma_fullk_kernel(const MfmaAr
   const LdsLayout L(M, G, 0, BITS == 4);
   int8_t* dig = reinterpret_cast<int8_t*>(smem + L.dig_off);
   float* cxs = reinterpret_cast<float*>(smem + L.cx_off);
+  float* red = reinterpret_cast<float*>(smem + L.red_off);
   int* csum = reinterpret_cast<int*>(smem + L.csum_off);
   const int j = lane & 15;
   const int blk = lane >> 4;
@@ -372,7 +452,8 @@ __global__ __launch_bounds__(256, 4) void wq_gemv_mfma_fullk_kernel(const MfmaAr
   int tile = blockIdx.x * waves + wv;
   if (tile < a.n_tiles) issue_weights(row_of(tile), scales_of(tile), 0);
 
-  stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum);
+  stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum,
+                               Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim}, red);
   __syncthreads();
   issue_fragments(0);
 
@@ -414,10 +495,11 @@ __global__ __launch_bounds__(256, 4) void wq_gemv_mfma_fullk_kernel(const MfmaAr
     const float mid = __shfl_down(acc, 16, kWave);
     const float total = (hi + mid) + acc;
     const int nn = tile * kTileRows + j;
-    if (blk == 0 && nn < a.N) out[nn] = from_float<T>(total);
+    if (blk == 0 && nn < a.N) out[nn] = finish<T>(total, a.residual, nn);
   }
 }
 
+constexpr int kFullKMinTiles = 1024;
 constexpr int kLdsDefault = 64 * 1024;   // dynamic LDS a kernel may use without opting in
 constexpr int kLdsMax = 160 * 1024;      // LDS of one gfx950 CU
 
@@ -447,17 +529,27 @@ int launch_m(const MfmaArgs& a, int wk, int grid, int lds, hipStream_t stream) {
   return launch_one<T, BITS, M, 1024>(a, wk, grid, lds, stream);
 }
 
+struct FusedOps {
+  int prologue = LLMQ_PRO_NONE;
+  const void* norm_weight = nullptr;
+  float eps = 0.0f;
+  int in_head_dim = 0;
+  const void* residual = nullptr;
+};
+
 template <typename T, int BITS>
 int launch_typed(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
-                 int out_group, hipStream_t stream) {
+                 int out_group, const FusedOps& ops, hipStream_t stream) {
   MfmaArgs a{};
   a.x = x; a.qw = static_cast<const uint8_t*>(qw); a.ws = ws; a.out = out;
   a.N = N; a.G = G; a.out_group = out_group;
+  a.prologue = ops.prologue; a.norm_weight = ops.norm_weight; a.eps = ops.eps;
+  a.in_head_dim = ops.in_head_dim; a.residual = ops.residual;
   a.n_tiles = (N + kTileRows - 1) / kTileRows;
   a.row_bytes = G * kGroup * BITS / 8;
   // measured on lm_head (8016 row tiles): the barrier-free kernel wins for int4 (27.7 vs 30.7 us),
   // the K-split one for int8 (46.6 vs 49.9 us)
-  if (M == 1 && BITS == 4 && a.n_tiles >= 2048) {
+  if (M == 1 && BITS == 4 && a.n_tiles >= kFullKMinTiles) {
     const LdsLayout L(1, G, 0, BITS == 4);
     auto kernel = wq_gemv_mfma_fullk_kernel<T, BITS>;
     // exactly as many workgroups as are resident at once (the launch bounds hold the kernel to
@@ -504,9 +596,19 @@ bool gemv_mfma_supported(const void* x, const void* qw, const float* ws, int M, 
 
 int gemv_mfma_launch(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
                      int out_group, int wformat, int dtype, hipStream_t stream) {
-#define LLMQ_DISPATCH(T)                                                                     \
-  (wformat == LLMQ_W_INT8 ? launch_typed<T, 8>(x, qw, ws, out, M, N, G, out_group, stream)   \
-                          : launch_typed<T, 4>(x, qw, ws, out, M, N, G, out_group, stream))
+  return gemv_mfma_launch_fused(x, qw, ws, out, M, N, G, out_group, wformat, dtype, LLMQ_PRO_NONE, nullptr,
+                                0.0f, 0, nullptr, stream);
+}
+
+int gemv_mfma_launch_fused(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
+                           int out_group, int wformat, int dtype, int prologue, const void* norm_weight,
+                           float eps, int in_head_dim, const void* residual, hipStream_t stream) {
+  FusedOps ops;
+  ops.prologue = prologue; ops.norm_weight = norm_weight; ops.eps = eps;
+  ops.in_head_dim = in_head_dim; ops.residual = residual;
+#define LLMQ_DISPATCH(T)                                                                          \
+  (wformat == LLMQ_W_INT8 ? launch_typed<T, 8>(x, qw, ws, out, M, N, G, out_group, ops, stream)   \
+                          : launch_typed<T, 4>(x, qw, ws, out, M, N, G, out_group, ops, stream))
   switch (dtype) {
     case LLMQ_F32: return LLMQ_DISPATCH(float);
     case LLMQ_F16: return LLMQ_DISPATCH(f16_t);

@@ -81,6 +81,12 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_kv_decode_workspace_floats.argtypes = [c_int] * 3
     lib.llmq_kv_decode_workspace_floats.restype = ctypes.c_size_t
     lib.llmq_kv_decode_attention.argtypes = [c_p] * 8 + [c_f] + [c_int] * 6 + [c_p]
+    lib.llmq_wq_gemv_fused.argtypes = [c_p] * 4 + [c_int] * 6 + [c_p, c_f, c_int, c_p, c_p]
+    lib.llmq_wq_gemv_fused.restype = c_int
+    lib.llmq_kv_rope_append_attend.argtypes = [c_p] * 9 + [c_f] + [c_int] * 6 + [c_p]
+    lib.llmq_kv_rope_append_attend.restype = c_int
+    lib.llmq_argmax_row.argtypes = [c_p, c_int, c_p, c_int, c_p]
+    lib.llmq_argmax_row.restype = c_int
     lib.llmq_wq_gemm_a8.argtypes = [c_p] * 6 + [c_int] * 7 + [c_p]
     lib.llmq_wq_gemm_a8.restype = c_int
     for name in ("llmq_fake_quant_group", "llmq_quant_group_codes", "llmq_wq_gemv", "llmq_kv_append",

@@ -18,8 +18,9 @@ from __future__ import annotations
 import torch
 
 from llmquant.runtime.llama_decode import WARMUP_CALLS, LlamaKernelRuntime
+from llmquant.runtime.llama_fused import LlamaFusedRuntime
 
-__all__ = ["GraphedDecoder", "KernelDecoder", "WARMUP_CALLS", "can_graph", "graphed_generate"]
+__all__ = ["GraphedDecoder", "KernelDecoder", "WARMUP_CALLS", "can_graph", "graphed_generate", "kernel_runtime"]
 
 
 def _on_gpu(model) -> bool:
@@ -96,12 +97,21 @@ class GraphedDecoder:
         return self.logits[:, -1:].argmax(-1)
 
 
+def kernel_runtime(model, max_len: int, kv_bits: int = 8):
+    """The fastest runtime the model qualifies for: the five-launches-per-layer fused step when
+    every Linear is a weight-only kernel-mode module, else the operation-by-operation walk."""
+    try:
+        return LlamaFusedRuntime(model, max_len, kv_bits)
+    except ValueError:
+        return LlamaKernelRuntime(model, max_len, kv_bits)
+
+
 class KernelDecoder:
     """Same interface over LlamaKernelRuntime and the integer KV cache."""
 
     def __init__(self, model, prompt_tokens: int, new_tokens: int, kv_bits: int = 8):
         self.max_len = prompt_tokens + new_tokens + 1
-        self.runtime = LlamaKernelRuntime(model, self.max_len, kv_bits)
+        self.runtime = kernel_runtime(model, self.max_len, kv_bits)
         self.graph = None
 
     @property
@@ -132,8 +142,8 @@ def graphed_generate(model, input_ids, max_new_tokens: int, kv_bits: int | None 
         return None
     prompt = input_ids.shape[1]
     if kv_bits is not None:
-        runtime = LlamaKernelRuntime(model, prompt + max_new_tokens + 1, kv_bits)
-        return runtime.generate(input_ids, max_new_tokens, use_graph=True)
+        return kernel_runtime(model, prompt + max_new_tokens + 1, kv_bits).generate(input_ids, max_new_tokens,
+                                                                                    use_graph=True)
     decoder = GraphedDecoder(model, prompt, max_new_tokens)
     nxt = decoder.prefill(input_ids)
     out = [nxt]

@@ -1,0 +1,108 @@
+"""The decode step as five launches per layer.
+
+LlamaKernelRuntime walks a decoder layer the way transformers does, one PyTorch kernel per
+elementwise operation: about 40 launches per layer, 670 per token, and at 3-4 us each the
+launches, not the weights, set the token rate. Here the same arithmetic, with the same
+rounding points, is folded into the kernels that have to run anyway:
+
+  1  RMSNorm -> q|k|v projection          (one GEMV over the concatenated weight)
+  2  RoPE -> KV quantize-append -> attention   (one kernel, one workgroup per kv head)
+  3  o_proj (+ head padding of its input) -> + residual
+  4  RMSNorm -> gate|up projection         (one GEMV over the concatenated weight)
+  5  SiLU(gate) * up -> down_proj -> + residual
+
+plus embedding lookup, final RMSNorm -> lm_head, and argmax. Prefill is unchanged
+(LlamaKernelRuntime's): it is one call over many tokens and its cost is in the GEMMs.
+
+Requirements on the model (met by oneshot(..., mode="kernel") of a Llama architecture with
+QuantConfig's defaults): every Linear a KernelQuantLinear with group size 128 and no bias,
+q/k/v sharing bit width and out_group, gate/up sharing bit width.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from llmquant.hip.build import load_extension
+from llmquant.quantizers.kernel import KernelQuantLinear
+from llmquant.runtime.llama_decode import LlamaKernelRuntime
+
+PRO_NONE, PRO_RMSNORM, PRO_SILU_MUL = 0, 1, 2
+
+
+def _fusable(*mods) -> bool:
+    first = mods[0]
+    for m in mods:
+        if not isinstance(m, KernelQuantLinear) or m.bias is not None or m._int8_act:
+            return False
+        if m.qdata.dtype != first.qdata.dtype or m.out_group != first.out_group:
+            return False
+        if m.qdata.shape[1:] != first.qdata.shape[1:] or m.scheme.weights.group_size != 128:
+            return False
+    return True
+
+
+class _Fused:
+    """Concatenated storage of Linears that read the same activation."""
+
+    def __init__(self, *mods):
+        self.qdata = torch.cat([m.qdata for m in mods], dim=0).contiguous()
+        self.wscale = torch.cat([m.wscale for m in mods], dim=0).contiguous()
+        self.out_group = mods[0].out_group
+
+
+class LlamaFusedRuntime(LlamaKernelRuntime):
+    def __init__(self, model, max_len: int, kv_bits: int = 8, exact_prefill: bool = False):
+        super().__init__(model, max_len, kv_bits, exact_prefill)
+        self._ext = load_extension()
+        self.fused_layers = []
+        for layer in self.layers:
+            attn, mlp = layer.self_attn, layer.mlp
+            if not (_fusable(attn.q_proj, attn.k_proj, attn.v_proj) and _fusable(mlp.gate_proj, mlp.up_proj)
+                    and _fusable(attn.o_proj) and _fusable(mlp.down_proj)):
+                raise ValueError("the fused decode step needs kernel-mode Linears (group 128, no bias, weight-only) "
+                                 "with q/k/v and gate/up sharing a bit width")
+            if attn.q_proj.out_group and attn.q_proj.qdata.shape[0] % attn.q_proj.out_group:
+                raise ValueError("q_proj rows are not a whole number of scale tiles")
+            args = attn.o_proj.scheme.weights
+            self.fused_layers.append(dict(
+                qkv=_Fused(attn.q_proj, attn.k_proj, attn.v_proj), gate_up=_Fused(mlp.gate_proj, mlp.up_proj),
+                o=attn.o_proj, down=mlp.down_proj,
+                o_head_dim=args.head_dim if attn.o_proj._needs_padding else 0,
+                norm1=layer.input_layernorm.weight.detach().contiguous(), eps1=layer.input_layernorm.variance_epsilon,
+                norm2=layer.post_attention_layernorm.weight.detach().contiguous(),
+                eps2=layer.post_attention_layernorm.variance_epsilon))
+        head = model.lm_head
+        if not _fusable(head):
+            raise ValueError("the fused decode step needs a kernel-mode lm_head")
+        self.final_norm = model.model.norm.weight.detach().contiguous()
+        self.final_eps = model.model.norm.variance_epsilon
+
+    def _forward(self, token_ids, cos, sin, decode: bool):
+        if not decode:
+            return super()._forward(token_ids, cos, sin, decode)
+        ext, cache = self._ext, self.cache
+        hidden = self.model.model.embed_tokens(token_ids)  # [1, hidden]
+        for index, f in enumerate(self.fused_layers):
+            qkv = ext.wq_gemv_fused(hidden, f["qkv"].qdata, f["qkv"].wscale, f["qkv"].out_group, PRO_RMSNORM,
+                                    f["norm1"], f["eps1"], 0, None)
+            ctx = ext.kv_rope_append_attend(qkv, self.cos_table, self.sin_table, cache.k_codes[index],
+                                            cache.v_codes[index], cache.k_scale[index], cache.v_scale[index],
+                                            cache.position, self.scaling, self.q_heads)
+            hidden = ext.wq_gemv_fused(ctx, f["o"].qdata, f["o"].wscale, f["o"].out_group, PRO_NONE, None, 0.0,
+                                       f["o_head_dim"], hidden)
+            gate_up = ext.wq_gemv_fused(hidden, f["gate_up"].qdata, f["gate_up"].wscale, 0, PRO_RMSNORM,
+                                        f["norm2"], f["eps2"], 0, None)
+            hidden = ext.wq_gemv_fused(gate_up, f["down"].qdata, f["down"].wscale, 0, PRO_SILU_MUL, None, 0.0, 0,
+                                       hidden)
+        head = self.model.lm_head
+        return ext.wq_gemv_fused(hidden, head.qdata, head.wscale, head.out_group, PRO_RMSNORM, self.final_norm,
+                                 self.final_eps, 0, None)
+
+    def _step(self):
+        logits = self._forward(self.token, None, None, decode=True)
+        nxt = self._ext.argmax_row(logits)
+        self.token.copy_(nxt)
+        self.pos_index.add_(1)
+        self.cache.position.add_(1)
+        return logits, nxt

@@ -1,0 +1,186 @@
+"""The fused decode-step kernels against the operation-by-operation forms they replace.
+
+Each fused op must reproduce the PyTorch sequence of transformers' LlamaDecoderLayer with its
+rounding points: RMSNorm -> Linear, SiLU(gate)*up -> Linear, head-padded input -> Linear,
+Linear -> + residual, RoPE -> cache append -> attention, argmax. The unfused side uses the
+same GEMV / cache kernels (themselves checked against the oracle elsewhere), so equality here is
+expected to the bit except where a reduction order differs (RMSNorm's variance).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import llmq_oracle as oracle
+from conftest import rel_l2, to_np
+
+pytestmark = pytest.mark.gpu
+GROUP = 128
+
+
+@pytest.fixture(scope="module")
+def ext():
+    from llmquant.hip import load_extension
+
+    return load_extension()
+
+
+def weights(n, k, bits, out_group=0, head_dim=None, seed=0):
+    torch.manual_seed(seed)
+    w = (torch.randn(n, k) * 0.02).to(torch.bfloat16)
+    canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP, head_dim, out_group or None)
+    q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
+    return q, torch.from_numpy(scales).cuda()
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("n,k", [(3072, 2048), (16384, 2048), (128256, 2048), (2048, 4096)])
+def test_rmsnorm_prologue(ext, bits, n, k):
+    q, s = weights(n, k, bits)
+    torch.manual_seed(1)
+    x = (torch.randn(1, k) * 3).to(torch.bfloat16).cuda()
+    norm = torch.nn.Parameter((1 + 0.1 * torch.randn(k)).to(torch.bfloat16).cuda())
+    eps = 1e-5
+    got = ext.wq_gemv_fused(x, q, s, 0, 1, norm, eps, 0, None)
+    xf = x.float()
+    normed = norm * (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(torch.bfloat16)  # LlamaRMSNorm
+    want = ext.wq_gemv(normed, q, s, 0)
+    assert got.shape == (1, n)
+    assert rel_l2(to_np(got), to_np(want)) <= 2e-3  # only the variance's summation order may differ
+    assert (got == want).float().mean() > 0.98
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_silu_mul_prologue_and_residual(ext, bits):
+    n, k = 2048, 8192
+    q, s = weights(n, k, bits)
+    torch.manual_seed(2)
+    gate_up = (torch.randn(1, 2 * k) * 2).to(torch.bfloat16).cuda()
+    res = torch.randn(1, n).to(torch.bfloat16).cuda()
+    got = ext.wq_gemv_fused(gate_up, q, s, 0, 2, None, 0.0, 0, res)
+    act = torch.nn.functional.silu(gate_up[:, :k]) * gate_up[:, k:]  # LlamaMLP, bf16 roundings included
+    want = res + ext.wq_gemv(act, q, s, 0)
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_head_padding_and_residual(ext, bits):
+    """o_proj: 32 heads of 64 in groups of 128 (pad_activation), one scale group per head."""
+    from llmquant.core.scheme import QuantizationArgs
+    from llmquant.quantizers import pad_activation
+
+    n, k = 2048, 2048
+    q, s = weights(n, k, bits, head_dim=64)
+    assert q.shape[1] == 32
+    torch.manual_seed(3)
+    x = torch.randn(1, k).to(torch.bfloat16).cuda()
+    res = torch.randn(1, n).to(torch.bfloat16).cuda()
+    got = ext.wq_gemv_fused(x, q, s, 0, 0, None, 0.0, 64, res)
+    padded = pad_activation(x, QuantizationArgs(bits, "group", group_size=128, head_dim=64))
+    want = res + ext.wq_gemv(padded, q, s, 0)
+    assert torch.equal(got, want)
+    q16, s16 = q[:, :16].contiguous(), s[:, :16].contiguous()
+    plain = ext.wq_gemv_fused(x, q16, s16, 0, 0, None, 0.0, 0, None)
+    assert torch.equal(plain, ext.wq_gemv(x, q16, s16, 0))
+
+
+def test_fused_gemv_argument_checks(ext):
+    q, s = weights(256, 512, 8)
+    x = torch.randn(1, 512, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="RMSNorm prologue needs"):
+        ext.wq_gemv_fused(x, q, s, 0, 1, None, 1e-5, 0, None)
+    with pytest.raises(RuntimeError, match="x has"):
+        ext.wq_gemv_fused(x, q, s, 0, 2, None, 0.0, 0, None)
+    with pytest.raises(RuntimeError, match="residual must be"):
+        ext.wq_gemv_fused(x, q, s, 0, 0, None, 0.0, 0, torch.zeros(1, 8, device="cuda", dtype=torch.bfloat16))
+    q3, s3 = weights(64, 384, 8)  # 3 groups: not a multiple of 4
+    with pytest.raises(RuntimeError, match="multiple of 4 groups"):
+        ext.wq_gemv_fused(torch.randn(1, 384, device="cuda", dtype=torch.bfloat16), q3, s3, 0, 0, None, 0.0, 0, None)
+
+
+def rope_reference(x, cos, sin):
+    half = x.shape[-1] // 2
+    rot = torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+    return (x * cos) + (rot * sin)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("q_heads,kv_heads,d", [(32, 8, 64), (8, 8, 64), (8, 2, 128)])
+@pytest.mark.parametrize("pos", [0, 5, 255, 256, 700])
+def test_rope_append_attend(ext, bits, q_heads, kv_heads, d, pos):
+    """One launch against RoPE in PyTorch + kv_append + kv_decode_attention on a cache that
+    already holds `pos` tokens."""
+    torch.manual_seed(4)
+    t_max = 1024
+    width = d if bits == 8 else d // 2
+    dt = torch.int8 if bits == 8 else torch.uint8
+
+    def fresh():
+        return dict(kc=torch.zeros(kv_heads, t_max, width, dtype=dt, device="cuda"),
+                    vc=torch.zeros(kv_heads, t_max, width, dtype=dt, device="cuda"),
+                    ks=torch.zeros(kv_heads, t_max, device="cuda"), vs=torch.zeros(kv_heads, t_max, device="cuda"))
+
+    a, b = fresh(), fresh()
+    zero = torch.zeros(1, dtype=torch.int32, device="cuda")
+    if pos:
+        past_k = torch.randn(kv_heads, pos, d).to(torch.bfloat16).cuda()
+        past_v = torch.randn(kv_heads, pos, d).to(torch.bfloat16).cuda()
+        for c in (a, b):
+            ext.kv_append(past_k, past_v, c["kc"], c["vc"], c["ks"], c["vs"], zero, False)
+    inv_freq = 1.0 / (500000.0 ** (torch.arange(0, d, 2).float() / d))
+    freqs = torch.outer(torch.arange(t_max).float(), inv_freq)
+    emb = torch.cat((freqs, freqs), -1)
+    cos_t, sin_t = emb.cos().to(torch.bfloat16).cuda(), emb.sin().to(torch.bfloat16).cuda()
+    qkv = torch.randn(1, (q_heads + 2 * kv_heads) * d).to(torch.bfloat16).cuda()
+    position = torch.tensor([pos], dtype=torch.int32, device="cuda")
+    got = ext.kv_rope_append_attend(qkv, cos_t, sin_t, a["kc"], a["vc"], a["ks"], a["vs"], position, d ** -0.5, q_heads)
+
+    q = qkv[0, : q_heads * d].view(q_heads, d)
+    k = qkv[0, q_heads * d: (q_heads + kv_heads) * d].view(kv_heads, d)
+    v = qkv[0, (q_heads + kv_heads) * d:].view(kv_heads, d)
+    q_r, k_r = rope_reference(q, cos_t[pos], sin_t[pos]), rope_reference(k, cos_t[pos], sin_t[pos])
+    ext.kv_append(k_r[:, None], v[:, None], b["kc"], b["vc"], b["ks"], b["vs"], position, False)
+    ws = torch.zeros(ext.kv_decode_workspace_floats(q_heads, d, t_max), device="cuda")
+    length = torch.tensor([pos + 1], dtype=torch.int32, device="cuda")
+    want = ext.kv_decode_attention(q_r.contiguous(), b["kc"], b["vc"], b["ks"], b["vs"], ws, length, d ** -0.5)
+    for name in ("kc", "vc", "ks", "vs"):
+        assert torch.equal(a[name], b[name]), name  # what was appended is identical
+    assert got.shape == (1, q_heads * d)
+    assert rel_l2(to_np(got).reshape(q_heads, d), to_np(want)) <= 4e-3  # same math, different merge order
+
+
+def test_argmax_row(ext):
+    torch.manual_seed(5)
+    for n in (1, 7, 1000, 128256):
+        for dtype in (torch.bfloat16, torch.float32):
+            x = torch.randn(1, n).to(dtype).cuda()
+            assert ext.argmax_row(x).item() == x.float().argmax().item()
+    x = torch.zeros(1, 5000, device="cuda", dtype=torch.bfloat16)
+    x[0, [17, 4000, 4999]] = 3.0
+    assert ext.argmax_row(x).item() == 17  # first of equal maxima
+    assert ext.argmax_row(x[:, 1:].contiguous()[:, :3000].contiguous()).item() == 16  # misaligned / short rows too
+
+
+def test_fused_runtime_equals_the_unfused_one():
+    """Whole decode steps on a small model: fused and operation-by-operation runtimes give the
+    same logits to the bit (hidden 512: the variance reduction happens to agree), the same
+    tokens, and graph replay equals eager."""
+    from test_gpu_decode import build_model, quantized_pair
+
+    from llmquant.runtime import LlamaFusedRuntime, LlamaKernelRuntime, kernel_runtime
+
+    _, kernel = quantized_pair(build_model(512, 1024, 3, 8, 2, 4096))
+    ids = torch.randint(0, 4096, (1, 40), generator=torch.Generator().manual_seed(1)).cuda()
+    plain, fused = LlamaKernelRuntime(kernel, 80, 8), LlamaFusedRuntime(kernel, 80, 8)
+    assert isinstance(kernel_runtime(kernel, 80, 8), LlamaFusedRuntime)
+    tok = plain.prefill(ids)
+    assert torch.equal(tok, fused.prefill(ids))
+    for i in range(16):
+        logits_p, nxt_p = plain.eager_step(tok, 40 + i)
+        logits_f, nxt_f = fused.eager_step(tok, 40 + i)
+        assert rel_l2(to_np(logits_f), to_np(logits_p)) <= 2e-2
+        assert torch.equal(plain.cache.k_codes[:, :, : 40 + i + 1], fused.cache.k_codes[:, :, : 40 + i + 1]) or i > 0
+        tok = nxt_p
+    seq_g = LlamaFusedRuntime(kernel, 80, 8).generate(ids, 24, use_graph=True)
+    seq_e = LlamaFusedRuntime(kernel, 80, 8).generate(ids, 24, use_graph=False)
+    assert torch.equal(seq_g, seq_e)
