@@ -39,6 +39,12 @@ SHAPES = [  # name, N, K  (BASELINE config 2)
 ]
 
 
+# HBM bytes one lm_head int8 launch moves, from hardware counters (FETCH_SIZE and WRITE_SIZE, each
+# scaled by its reading for a 256 MiB copy): profiles/wq_gemv_lm_head_hbm_traffic.txt. 1.001 x the
+# algorithmic bytes.
+LM_HEAD_INT8_TRAFFIC_BYTES = 271_404_500
+
+
 def algorithmic_bytes(n: int, k: int, bits: int, m: int = 1) -> int:
     """codes + fp32 scales + bf16 x + bf16 y."""
     return n * k * bits // 8 + n * (k // GROUP) * 4 + m * k * 2 + m * n * 2
@@ -53,6 +59,9 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the legs that report the path's other kernels and end-to-end decode")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="first run a plain 256 MiB device copy three times: the known-size kernel that "
+                         "hardware-counter readings of the sweep are scaled by")
     return ap.parse_args()
 
 
@@ -104,6 +113,13 @@ def main():
     load_extension()
     lib = load_capi()
     torch.cuda.set_device(0)
+    if opts.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     cases = build_operands(torch)
     stream = torch.cuda.current_stream()
     sptr = ctypes.c_void_p(stream.cuda_stream)
@@ -186,7 +202,7 @@ def main():
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "roofline": {"bound": "hbm", "kernel": "wq_gemv lm_head 128256x2048 int8 M=1",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": LM_HEAD_INT8_TRAFFIC_BYTES,
                      "avg_launch_us": round(dom_avg_ms * 1e3, 2),
                      "median_launch_us": round(dom_ms[len(dom_ms) // 2] * 1e3, 2),
                      "algorithmic_bytes": dominant["bytes"]},
@@ -218,9 +234,22 @@ def _event_time_us(torch, fn, reps=20, warm=3):
     return a.elapsed_time(b) / reps * 1e3
 
 
+def _graph_time_us(torch, fn, reps=20):
+    """Average replay time of `fn` captured as one HIP graph (launch cost of the Python loop removed)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn()
+    return _event_time_us(torch, graph.replay, reps=reps)
+
+
 def other_kernels(torch):
     """The path's other kernels, each on its BASELINE shape: fake-quant op, KV-cache decode
-    attention (config 4), W4A8 / W8A8 integer GEMM (config 3). Back-to-back launches, HIP events."""
+    step (config 4), W4A8 / W8A8 integer GEMM (config 3). Back-to-back launches, HIP events."""
     from llmquant.hip import load_extension
 
     ext = load_extension()
@@ -239,29 +268,29 @@ def other_kernels(torch):
     out["fake_quant_2048x8192_bf16_int4"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
                                              "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
     del xs
-    # KV decode attention, Llama-3.2-1B geometry, context 2048 (+ the token being decoded)
+    # KV cache decode step, Llama-3.2-1B geometry, 2048 tokens of context + the one being decoded:
+    # RoPE + quantize-and-append + attention in one launch per layer, 16 layers replayed as a graph
     for bits in (8, 4):
-        layers, kvh, qh, d, t = 16, 8, 32, 64, 2049
+        layers, kvh, qh, d, t_max = 16, 8, 32, 64, 4096
+        ctx = 2048
         width = d if bits == 8 else d // 2
         dt = torch.int8 if bits == 8 else torch.uint8
-        kc = torch.randint(0, 100, (layers, kvh, t, width), device=dev).to(dt)
-        vc = torch.randint(0, 100, (layers, kvh, t, width), device=dev).to(dt)
-        ks = torch.rand(layers, kvh, t, device=dev) * 0.05
-        vs = torch.rand(layers, kvh, t, device=dev) * 0.05
-        ws = torch.zeros(layers, ext.kv_decode_workspace_floats(qh, d, t), device=dev)
-        q = torch.randn(qh, d, device=dev).to(torch.bfloat16)
-        length = torch.tensor([t], dtype=torch.int32, device=dev)
-        k1 = torch.randn(kvh, 1, d, device=dev).to(torch.bfloat16)
-        pos = torch.tensor([t - 1], dtype=torch.int32, device=dev)
+        kc = torch.randint(0, 100, (layers, kvh, t_max, width), device=dev).to(dt)
+        vc = torch.randint(0, 100, (layers, kvh, t_max, width), device=dev).to(dt)
+        ks = torch.rand(layers, kvh, t_max, device=dev) * 0.05
+        vs = torch.rand(layers, kvh, t_max, device=dev) * 0.05
+        qkv = torch.randn(1, (qh + 2 * kvh) * d, device=dev).to(torch.bfloat16)
+        table = torch.randn(t_max, d, device=dev).to(torch.bfloat16)
+        pos = torch.tensor([ctx], dtype=torch.int32, device=dev)
 
         def step():
             for layer in range(layers):
-                ext.kv_append(k1, k1, kc[layer], vc[layer], ks[layer], vs[layer], pos, False)
-                ext.kv_decode_attention(q, kc[layer], vc[layer], ks[layer], vs[layer], ws[layer], length, d ** -0.5)
+                ext.kv_rope_append_attend(qkv, table, table, kc[layer], vc[layer], ks[layer], vs[layer], pos,
+                                          d ** -0.5, qh)
 
-        us = _event_time_us(torch, step, reps=10) / layers
-        nbytes = 2 * kvh * t * width + 2 * kvh * t * 4
-        out[f"kv_int{bits}_append_plus_attention_ctx2048_per_layer"] = {
+        us = _graph_time_us(torch, step, reps=20) / layers
+        nbytes = 2 * kvh * (ctx + 1) * width + 2 * kvh * (ctx + 1) * 4
+        out[f"kv_int{bits}_rope_append_attention_ctx2048_per_layer"] = {
             "us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1)}
     # integer GEMM, Llama-3-8B MLP shapes
     gemm = []

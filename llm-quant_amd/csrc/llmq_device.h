@@ -23,11 +23,15 @@ __device__ __forceinline__ float to_float(bf16_t v) {
   return __builtin_bit_cast(float, static_cast<uint32_t>(v.bits) << 16);
 }
 
+// fp32 -> bf16, round-to-nearest-even: gfx950 converts in hardware (v_cvt_pk_bf16_f32, two
+// values per instruction), which the compiler selects for these casts.
 __device__ __forceinline__ uint16_t bf16_bits_rne(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;  // NaN stays NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+}
+__device__ __forceinline__ uint32_t bf16_pair_rne(float lo, float hi) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
 }
 
 template <typename T> __device__ __forceinline__ T from_float(float f);
@@ -90,8 +94,7 @@ template <> struct Pack<bf16_t> {
     uint32_t w[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      w[i] = static_cast<uint32_t>(bf16_bits_rne(f[2 * i])) |
-             (static_cast<uint32_t>(bf16_bits_rne(f[2 * i + 1])) << 16);
+      w[i] = bf16_pair_rne(f[2 * i], f[2 * i + 1]);
     }
     return u32x4{w[0], w[1], w[2], w[3]};
   }

@@ -483,9 +483,10 @@ __global__ __launch_bounds__(256, 4) void wq_gemv_mfma_fullk_kernel(const MfmaAr
         }
       }
       // operand registers are free again: refill them (next chunk, or the next tile's first
-      // chunk; past the last tile the same rows are simply read once more) before the epilogue
+      // chunk; nothing after the last tile: a re-read there would cost 1/n_chunks of a tile of
+      // HBM traffic per wave) before the epilogue
       const bool wrap = c + 1 == n_chunks;
-      issue_weights(wrap ? next_row : row, wrap ? next_sp : sp, wrap ? 0 : c + 1);
+      if (!wrap || more) issue_weights(wrap ? next_row : row, wrap ? next_sp : sp, wrap ? 0 : c + 1);
       issue_fragments(wrap ? 0 : c + 1);
 #pragma unroll
       for (int gi = 0; gi < kGW; ++gi) acc = fmaf(static_cast<float>(d[gi][0]), s_now[gi], acc);
