@@ -10,14 +10,17 @@
 // built with -ffp-contract=off so no multiply-add is fused; results equal the reference's
 // real mode bit for bit.
 //
-// Shape. A workgroup (4 waves) owns a 128 x 128 output tile and walks K one group (128) at a
-// time. Activations [M, K] int8 and weights [N, K(/2)] are staged in LDS, weights unpacked
+// Shape. A workgroup (4 waves) owns a 128 x 128 output tile (64 x 64 when the problem has too
+// few tiles to fill the chip; the text below describes the large one) and walks K one group
+// (128) at a time. Activations [M, K] int8 and weights [N, K(/2)] are staged in LDS, weights unpacked
 // there to signed int8 in natural k order (packed int4: nibble - 8 computed four at a time
 // with a borrow-free byte subtract, even/odd nibbles re-interleaved with v_perm). Each wave
 // computes a 64 x 64 quadrant as 2 x 2 MFMA tiles of 32 x 32 (A = activations, rows m;
 // B = weights, columns n), 4 k-slabs of 32 per group. The next group's global loads are in
-// flight while the current one is multiplied. After each group the int32 accumulators go
-// through the scale epilogue above and are cleared.
+// flight while the current one is multiplied. After each group the int32 sums go through the
+// scale epilogue above: four vector-ALU operations per output element per group, against 256
+// multiply-adds on the matrix core, which makes the vector ALU the unit that bounds this
+// kernel (two waves per SIMD, so that one wave's epilogue runs under the other's MFMAs).
 #include "llmq_device.h"
 
 namespace {
@@ -27,7 +30,7 @@ using namespace llmq;
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int kBM = 128, kBN = 128, kGroup = 128;
+constexpr int kGroup = 128;
 constexpr int kThreads = 256;
 constexpr int kRowStride = kGroup + 16;  // bytes; padding keeps 16-byte reads off the same banks
 
@@ -46,8 +49,12 @@ __device__ __forceinline__ uint32_t unbias4(uint32_t u) {
   return ((u | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
 }
 
-template <typename T, int BITS>
-__global__ __launch_bounds__(kThreads) void wq_gemm_a8_kernel(const GemmArgs g) {
+// W: the wave's quadrant is (32 W) x (32 W), the workgroup's tile (64 W) x (64 W). W = 2 is the
+// throughput shape; W = 1 gives four times as many workgroups when the problem is too small to
+// fill the chip with 128 x 128 tiles.
+template <typename T, int BITS, int W>
+__global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs g) {
+  constexpr int kBM = 64 * W, kBN = 64 * W;
   __shared__ __attribute__((aligned(16))) int8_t s_a[2][kBM * kRowStride];
   __shared__ __attribute__((aligned(16))) int8_t s_b[2][kBN * kRowStride];
   __shared__ __attribute__((aligned(16))) float s_sx[2][kBM];
@@ -60,11 +67,11 @@ __global__ __launch_bounds__(kThreads) void wq_gemm_a8_kernel(const GemmArgs g) 
   const int64_t w_row_bytes = BITS == 8 ? k_total : k_total / 2;
 
   // ---- staging: who loads what ------------------------------------------------------------------
-  // A tile: 128 rows x 128 B = 1024 16-byte packets, 4 per thread. Thread t: packets t + 256*i:
+  // A tile: kBM rows x 128 B = 8 kBM 16-byte packets. Thread t: packets t + 256*i:
   // row = p / 8, piece = p % 8.
-  // B tile int8: same. B tile int4: 128 rows x 64 B = 512 packets, 2 per thread: row = p / 4.
-  constexpr int kAPackets = 4;
-  constexpr int kBPackets = BITS == 8 ? 4 : 2;
+  // B tile int8: same. B tile int4: kBN rows x 64 B = 4 kBN packets: row = p / 4.
+  constexpr int kAPackets = kBM * 8 / kThreads;
+  constexpr int kBPackets = (BITS == 8 ? kBN * 8 : kBN * 4) / kThreads;
   u32x4 ra[kAPackets], rb[kBPackets];
   float r_sx = 0.0f, r_sw = 0.0f;
 
@@ -88,7 +95,7 @@ __global__ __launch_bounds__(kThreads) void wq_gemm_a8_kernel(const GemmArgs g) 
     }
     if (tid < kBM) {
       r_sx = g.sx[static_cast<int64_t>(min(m0 + tid, g.M - 1)) * g.G + grp];
-    } else {
+    } else if (tid < kBM + kBN) {
       const int n = min(n0 + tid - kBM, g.N - 1);
       r_sw = g.sw[static_cast<int64_t>(g.out_group > 0 ? n / g.out_group : n) * g.G + grp];
     }
@@ -121,14 +128,14 @@ __global__ __launch_bounds__(kThreads) void wq_gemm_a8_kernel(const GemmArgs g) 
         store16(dst + 16, u32x4{o[4], o[5], o[6], o[7]});
       }
     }
-    if (tid < kBM) s_sx[buf][tid] = r_sx; else s_sw[buf][tid - kBM] = r_sw;
+    if (tid < kBM) s_sx[buf][tid] = r_sx; else if (tid < kBM + kBN) s_sw[buf][tid - kBM] = r_sw;
   };
 
-  float acc[2][2][16];
+  float acc[W][W][16];
 #pragma unroll
-  for (int mi = 0; mi < 2; ++mi)
+  for (int mi = 0; mi < W; ++mi)
 #pragma unroll
-    for (int ni = 0; ni < 2; ++ni)
+    for (int ni = 0; ni < W; ++ni)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
 
@@ -141,54 +148,57 @@ __global__ __launch_bounds__(kThreads) void wq_gemm_a8_kernel(const GemmArgs g) 
     const int buf = grp & 1;
     if (grp + 1 < g.G) load_group(grp + 1);  // in flight during the MFMAs below
 
-    v16i d[2][2];
+    // The four 32 x 32 sub-tiles of the quadrant, one after the other: while the matrix core
+    // works on sub-tile t + 1 the vector ALU runs the scale epilogue of sub-tile t.
+    v4i fa[W][kGroup / 32], fb[kGroup / 32];
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+    for (int mi = 0; mi < W; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < 2; ++ni)
+      for (int ks = 0; ks < kGroup / 32; ++ks)
+        fa[mi][ks] = *reinterpret_cast<const v4i*>(&s_a[buf][((wm * W + mi) * 32 + frag_row) * kRowStride + ks * 32 + frag_k]);
+    auto load_b = [&](int ni) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) d[mi][ni][r] = 0;
+      for (int ks = 0; ks < kGroup / 32; ++ks)
+        fb[ks] = *reinterpret_cast<const v4i*>(&s_b[buf][((wn * W + ni) * 32 + frag_row) * kRowStride + ks * 32 + frag_k]);
+    };
+    auto multiply = [&](int mi) {
+      v16i d = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int ks = 0; ks < kGroup / 32; ++ks) {
-      v4i fa[2], fb[2];
+      for (int ks = 0; ks < kGroup / 32; ++ks) d = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[mi][ks], fb[ks], d, 0, 0, 0);
+      return d;
+    };
+    // result register r of a 32 x 32 tile is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+    auto scale_in = [&](const v16i& d, int mi, int ni) {
+      const float sw = s_sw[buf][(wn * W + ni) * 32 + (lane & 31)];
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi) {
-        fa[mi] = *reinterpret_cast<const v4i*>(&s_a[buf][(wm * 64 + mi * 32 + frag_row) * kRowStride + ks * 32 + frag_k]);
-      }
+      for (int r4 = 0; r4 < 4; ++r4) {
+        // four consecutive rows: one 128-bit LDS read of their activation scales
+        const int row = (wm * W + mi) * 32 + 8 * r4 + 4 * (lane >> 5);
+        const u32x4 s4 = *reinterpret_cast<const u32x4*>(&s_sx[buf][row]);
+        const float sx4[4] = {__builtin_bit_cast(float, s4.x), __builtin_bit_cast(float, s4.y),
+                              __builtin_bit_cast(float, s4.z), __builtin_bit_cast(float, s4.w)};
 #pragma unroll
-      for (int ni = 0; ni < 2; ++ni) {
-        fb[ni] = *reinterpret_cast<const v4i*>(&s_b[buf][(wn * 64 + ni * 32 + frag_row) * kRowStride + ks * 32 + frag_k]);
-      }
-#pragma unroll
-      for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-          d[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[mi], fb[ni], d[mi][ni], 0, 0, 0);
-    }
-
-    // scale epilogue: result register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4,
-    // column lane%32
-#pragma unroll
-    for (int ni = 0; ni < 2; ++ni) {
-      const float sw = s_sw[buf][wn * 64 + ni * 32 + (lane & 31)];
-#pragma unroll
-      for (int mi = 0; mi < 2; ++mi) {
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          // four consecutive rows: one 128-bit LDS read of their activation scales
-          const int row = wm * 64 + mi * 32 + 8 * r4 + 4 * (lane >> 5);
-          const u32x4 s4 = *reinterpret_cast<const u32x4*>(&s_sx[buf][row]);
-          const float sx4[4] = {__builtin_bit_cast(float, s4.x), __builtin_bit_cast(float, s4.y),
-                                __builtin_bit_cast(float, s4.z), __builtin_bit_cast(float, s4.w)};
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            float f = static_cast<float>(d[mi][ni][4 * r4 + i]);
-            f = f * sw;
-            f = f * sx4[i];
-            acc[mi][ni][4 * r4 + i] = acc[mi][ni][4 * r4 + i] + f;
-          }
+        for (int i = 0; i < 4; ++i) {
+          float f = static_cast<float>(d[4 * r4 + i]);
+          f = f * sw;
+          f = f * sx4[i];
+          acc[mi][ni][4 * r4 + i] = acc[mi][ni][4 * r4 + i] + f;
         }
       }
+    };
+    load_b(0);
+    if constexpr (W == 2) {
+      v16i d0 = multiply(0);
+      v16i d1 = multiply(1);
+      scale_in(d0, 0, 0);
+      load_b(1);
+      d0 = multiply(0);
+      scale_in(d1, 1, 0);
+      d1 = multiply(1);
+      scale_in(d0, 0, 1);
+      scale_in(d1, 1, 1);
+    } else {
+      scale_in(multiply(0), 0, 0);
     }
 
     if (grp + 1 < g.G) store_group(buf ^ 1);  // nobody reads that buffer any more: see barrier below
@@ -197,14 +207,14 @@ __global__ __launch_bounds__(kThreads) void wq_gemm_a8_kernel(const GemmArgs g) 
 
   T* __restrict__ out = static_cast<T*>(g.out);
 #pragma unroll
-  for (int ni = 0; ni < 2; ++ni) {
-    const int n = n0 + wn * 64 + ni * 32 + (lane & 31);
+  for (int ni = 0; ni < W; ++ni) {
+    const int n = n0 + (wn * W + ni) * 32 + (lane & 31);
     const float b = (g.bias != nullptr && n < g.N) ? g.bias[n] : 0.0f;
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
+    for (int mi = 0; mi < W; ++mi) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const int m = m0 + (wm * W + mi) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (m < g.M && n < g.N) {
           const float v = g.bias != nullptr ? acc[mi][ni][r] + b : acc[mi][ni][r];
           out[static_cast<int64_t>(m) * g.N + n] = from_float<T>(v);
@@ -214,15 +224,23 @@ __global__ __launch_bounds__(kThreads) void wq_gemm_a8_kernel(const GemmArgs g) 
   }
 }
 
-template <typename T>
-int launch_typed(const GemmArgs& g, int wformat, hipStream_t stream) {
-  const dim3 grid((g.N + kBN - 1) / kBN, (g.M + kBM - 1) / kBM), block(kThreads);
+template <typename T, int W>
+int launch_tile(const GemmArgs& g, int wformat, hipStream_t stream) {
+  constexpr int kTile = 64 * W;
+  const dim3 grid((g.N + kTile - 1) / kTile, (g.M + kTile - 1) / kTile), block(kThreads);
   if (wformat == LLMQ_W_INT8) {
-    hipLaunchKernelGGL((wq_gemm_a8_kernel<T, 8>), grid, block, 0, stream, g);
+    hipLaunchKernelGGL((wq_gemm_a8_kernel<T, 8, W>), grid, block, 0, stream, g);
   } else {
-    hipLaunchKernelGGL((wq_gemm_a8_kernel<T, 4>), grid, block, 0, stream, g);
+    hipLaunchKernelGGL((wq_gemm_a8_kernel<T, 4, W>), grid, block, 0, stream, g);
   }
   return llmq_host::check_launch("wq_gemm_a8_kernel");
+}
+
+template <typename T>
+int launch_typed(const GemmArgs& g, int wformat, hipStream_t stream) {
+  // 128 x 128 tiles when there is at least one for every CU, else 64 x 64
+  const int64_t big_tiles = static_cast<int64_t>((g.N + 127) / 128) * ((g.M + 127) / 128);
+  return big_tiles >= 256 ? launch_tile<T, 2>(g, wformat, stream) : launch_tile<T, 1>(g, wformat, stream);
 }
 
 }  // namespace

@@ -83,6 +83,19 @@ def test_llama_8b_mlp_shapes_on_sampled_entries(ext, n, k, m):
     assert np.array_equal(to_np(got)[np.ix_(rows, cols)], want)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_ragged_edges_of_the_large_tile(ext, bits):
+    """Enough 128 x 128 tiles that the large-tile kernel runs, with M and N that end inside a
+    tile: the last rows and columns (and a sample of the rest) against the oracle."""
+    m, n, k = 2050, 3970, 256
+    got, (x, canonical, scales, _) = run_case(ext, m, n, k, bits, torch.bfloat16, seed=4)
+    rng = np.random.default_rng(1)
+    rows = np.unique(np.concatenate([rng.choice(m, 48, replace=False), np.arange(m - 4, m)]))
+    cols = np.unique(np.concatenate([rng.choice(n, 48, replace=False), np.arange(n - 4, n)]))
+    want = oracle.real_linear(to_np(x)[rows], canonical[cols], scales[cols], "bf16", None, 8)
+    assert np.array_equal(to_np(got)[np.ix_(rows, cols)], want)
+
+
 @pytest.mark.parametrize("name", ["W4A8", "W8A8"])
 @pytest.mark.parametrize("layout", [dict(), dict(head_dim=64), dict(out_group=64)])
 @pytest.mark.parametrize("m", [1, 4, 33])
