@@ -234,6 +234,9 @@ def _event_time_us(torch, fn, reps=20, warm=3):
     return a.elapsed_time(b) / reps * 1e3
 
 
+_CAPI = {}
+
+
 def _graph_time_us(torch, fn, reps=20):
     """Average replay time of `fn` captured as one HIP graph (launch cost of the Python loop removed)."""
     side = torch.cuda.Stream()
@@ -252,7 +255,10 @@ def other_kernels(torch):
     step (config 4), W4A8 / W8A8 integer GEMM (config 3). Back-to-back launches, HIP events."""
     from llmquant.hip import load_extension
 
+    from llmquant.hip import load_capi
+
     ext = load_extension()
+    _CAPI["lib"] = load_capi()
     dev = "cuda:0"
     out = {}
     # fake quant, 2048 x 8192 bf16, g128: one read + one write (+ scales)
@@ -292,6 +298,38 @@ def other_kernels(torch):
         nbytes = 2 * kvh * (ctx + 1) * width + 2 * kvh * (ctx + 1) * 4
         out[f"kv_int{bits}_rope_append_attention_ctx2048_per_layer"] = {
             "us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1)}
+    # the GEMV on Llama-3-8B's linears (M = 1): random codes, buffers rotated over > 600 MB so that
+    # every launch streams from HBM; the launches of one rotation replayed as a HIP graph
+    shapes_8b = []
+    for name, n, k in (("q/o", 4096, 4096), ("k/v", 1024, 4096), ("gate/up", 14336, 4096),
+                       ("down", 4096, 14336), ("lm_head", 128256, 4096)):
+        x = torch.randn(1, k, device=dev).to(torch.bfloat16)
+        for bits in (8, 4):
+            nbytes = algorithmic_bytes(n, k, bits)
+            copies = max(2, min(24, (600 << 20) // nbytes + 1))
+            width = GROUP if bits == 8 else GROUP // 2
+            qs = [torch.randint(0, 255, (n, k // GROUP, width), dtype=torch.uint8, device=dev) for _ in range(copies)]
+            if bits == 8:
+                qs = [q.view(torch.int8) for q in qs]
+            sw = torch.rand(n, k // GROUP, device=dev) * 0.01
+            outs = torch.empty(copies, 1, n, device=dev, dtype=torch.bfloat16)
+            lib = _CAPI["lib"]
+            sptr_of = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+            def sweep():  # one launch per buffer copy, through the C ABI (no allocation: graph-safe)
+                sp = sptr_of()
+                for c in range(copies):
+                    rc = lib.llmq_wq_gemv(x.data_ptr(), qs[c].data_ptr(), sw.data_ptr(), outs[c].data_ptr(),
+                                          1, n, k // GROUP, GROUP, 0, bits, 2, sp)
+                    if rc:
+                        raise RuntimeError(lib.llmq_last_error().decode())
+
+            us = _graph_time_us(torch, sweep, reps=5) / copies
+            shapes_8b.append({"shape": name, "N": n, "K": k, "bits": bits, "bytes": nbytes, "us": round(us, 2),
+                              "GBps": round(nbytes / us / 1e3, 1),
+                              "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)})
+            del qs
+    out["gemv_llama3_8b_shapes_graph_replay"] = shapes_8b
     # integer GEMM, Llama-3-8B MLP shapes
     gemm = []
     for n, k in ((14336, 4096), (4096, 14336)):

@@ -28,7 +28,8 @@
 // m = 0..3: digits are recombined by scaling block q with 256^q in fp32.
 //
 // Work split: a workgroup owns 16 weight rows at a time and all of K; wave w owns groups
-// 4w..4w+3 (so K = 2048 -> 4 waves, 8192 -> 16 waves). Per row tile a wave issues 8 (int8)
+// 4w..4w+3 (so K = 2048 -> 4 waves, 8192 -> 16 waves; longer rows: waves that each take
+// several such chunks: 5..8 waves). Per row tile a wave issues 8 (int8)
 // or 4 (int4) 128-bit loads per lane plus one 128-bit load of its four scales, the next
 // tile's loads being issued before the current tile's epilogue. Partial sums meet in LDS.
 #include "llmq_device.h"
@@ -234,7 +235,11 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
   }
 }
 
-template <typename T, int BITS, int M, int MAXT>
+// MULTI == false: the workgroup has one wave per chunk of four groups (K <= 8192) and a wave's
+// activation fragments stay in registers for the whole kernel. MULTI == true: longer rows; wave w
+// takes chunks w, w + waves, ... of every row tile and re-reads the fragments of the chunk it is
+// about to multiply from LDS (the read is issued with the weight loads, a chunk ahead).
+template <typename T, int BITS, int M, int MAXT, bool MULTI>
 __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x;
@@ -242,6 +247,7 @@ __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
   const int wv = tid / kWave;
   const int wk = blockDim.x / kWave;
   const int G = a.G;
+  const int n_chunks = G / kGW;
   const LdsLayout L(M, G, wk, BITS == 4);
   int8_t* dig = reinterpret_cast<int8_t*>(smem + L.dig_off);
   float* cxs = reinterpret_cast<float*>(smem + L.cx_off);
@@ -251,13 +257,13 @@ __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
 
   const int j = lane & 15;    // weight row within the tile (B column / D column)
   const int blk = lane >> 4;  // k-block of the operand; digit block of the result
-  const int g0 = wv * kGW;
 
-  // ---- weight / scale loads of one row tile -------------------------------------------------
+  // ---- weight / scale loads of one chunk of one row tile ------------------------------------
   constexpr int kLoads = BITS == 8 ? 2 * kGW : kGW;
   v4i b[kLoads];
   float sc[kGW];
-  auto issue_loads = [&](int tile) {
+  auto issue_loads = [&](int tile, int chunk) {
+    const int g0 = chunk * kGW;
     const int n = min(tile * kTileRows + j, a.N - 1);  // rows past the end: loaded, not stored
     const uint8_t* row = a.qw + static_cast<int64_t>(n) * a.row_bytes;
 #pragma unroll
@@ -271,30 +277,22 @@ __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
       }
     }
     const int srow = a.out_group > 0 ? n / a.out_group : n;
-    // G and g0 are multiples of 4: the wave's four scales are one aligned 128-bit load
+    // G and g0 are multiples of 4: the chunk's four scales are one aligned 128-bit load
     const u32x4 s4 = load16(a.ws + static_cast<int64_t>(srow) * G + g0);
     sc[0] = __builtin_bit_cast(float, s4.x); sc[1] = __builtin_bit_cast(float, s4.y);
     sc[2] = __builtin_bit_cast(float, s4.z); sc[3] = __builtin_bit_cast(float, s4.w);
   };
 
-  int tile = blockIdx.x;
-  if (tile < a.n_tiles) issue_loads(tile);  // in flight while the activation is prepared
-
-  stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum,
-                               Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim}, red);
-  __syncthreads();
-
-  // ---- phase 2: this wave's operands and constants, into registers --------------------------
+  // ---- a chunk's activation operands and constants, LDS -> registers ------------------------
   v4i afrag[kGW][2];
   float fscale[kGW][M];  // 2^-sh * 256^digit of the result block this lane sits in
   v4i cinit[kGW];
-  {
+  auto load_fragments = [&](int chunk) {
     const int q = j >> 2, m = j & 3;  // A row j = 4*digit + m
     const float digit_weight = blk == 0 ? 1.0f : (blk == 1 ? 256.0f : 65536.0f);
 #pragma unroll
     for (int gi = 0; gi < kGW; ++gi) {
-      const int g = g0 + gi;
-      const bool ok = true;
+      const int g = chunk * kGW + gi;
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         afrag[gi][s] = v4i{0, 0, 0, 0};
@@ -305,47 +303,64 @@ __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
       cinit[gi] = v4i{0, 0, 0, 0};
 #pragma unroll
       for (int r = 0; r < M; ++r) {
-        fscale[gi][r] = (ok && blk < kDigits) ? cxs[r * G + g] * digit_weight : 0.0f;
+        fscale[gi][r] = blk < kDigits ? cxs[r * G + g] * digit_weight : 0.0f;
         if constexpr (BITS == 4) {
-          if (ok && blk < kDigits) cinit[gi][r] = -8 * csum[(blk * M + r) * G + g];
+          if (blk < kDigits) cinit[gi][r] = -8 * csum[(blk * M + r) * G + g];
         }
       }
     }
-  }
+  };
 
-  // ---- phase 3: stream row tiles -----------------------------------------------------------
+  int tile = blockIdx.x;
+  if (tile < a.n_tiles) issue_loads(tile, wv);  // in flight while the activation is prepared
+
+  stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum,
+                               Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim}, red);
+  __syncthreads();
+  load_fragments(wv);
+
+  // ---- stream row tiles -----------------------------------------------------------------------
   T* __restrict__ out = static_cast<T*>(a.out);
   int buf = 0;
   for (; tile < a.n_tiles; tile += gridDim.x) {
-    v4i d[kGW];
-#pragma unroll
-    for (int gi = 0; gi < kGW; ++gi) {
-      d[gi] = cinit[gi];
-      if constexpr (BITS == 8) {
-        d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][0], b[2 * gi], d[gi], 0, 0, 0);
-        d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], b[2 * gi + 1], d[gi], 0, 0, 0);
-      } else {
-        const v4i lo = b[gi] & 0x0f0f0f0f;
-        const v4i hi = (b[gi] >> 4) & 0x0f0f0f0f;
-        d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][0], lo, d[gi], 0, 0, 0);
-        d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], hi, d[gi], 0, 0, 0);
-      }
-    }
-    float s_now[kGW];
-#pragma unroll
-    for (int gi = 0; gi < kGW; ++gi) s_now[gi] = sc[gi];
-    const int next = tile + gridDim.x;
-    if (next < a.n_tiles) issue_loads(next);
-
     float acc[M];
 #pragma unroll
     for (int r = 0; r < M; ++r) acc[r] = 0.0f;
+    for (int chunk = wv; chunk < n_chunks; chunk += wk) {
+      v4i d[kGW];
 #pragma unroll
-    for (int gi = 0; gi < kGW; ++gi) {
-#pragma unroll
-      for (int r = 0; r < M; ++r) {
-        acc[r] = fmaf(static_cast<float>(d[gi][r]), s_now[gi] * fscale[gi][r], acc[r]);
+      for (int gi = 0; gi < kGW; ++gi) {
+        d[gi] = cinit[gi];
+        if constexpr (BITS == 8) {
+          d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][0], b[2 * gi], d[gi], 0, 0, 0);
+          d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], b[2 * gi + 1], d[gi], 0, 0, 0);
+        } else {
+          const v4i lo = b[gi] & 0x0f0f0f0f;
+          const v4i hi = (b[gi] >> 4) & 0x0f0f0f0f;
+          d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][0], lo, d[gi], 0, 0, 0);
+          d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], hi, d[gi], 0, 0, 0);
+        }
       }
+      float s_now[kGW][M];
+#pragma unroll
+      for (int gi = 0; gi < kGW; ++gi)
+#pragma unroll
+        for (int r = 0; r < M; ++r) s_now[gi][r] = sc[gi] * fscale[gi][r];
+      // operand registers are free: refill them with what this wave multiplies next
+      const int next_chunk = MULTI ? chunk + wk : n_chunks;
+      if (next_chunk < n_chunks) {
+        issue_loads(tile, next_chunk);
+        load_fragments(next_chunk);
+      } else if (tile + static_cast<int>(gridDim.x) < a.n_tiles) {
+        issue_loads(tile + gridDim.x, wv);
+        if constexpr (MULTI) load_fragments(wv);
+      }
+#pragma unroll
+      for (int gi = 0; gi < kGW; ++gi) {
+#pragma unroll
+        for (int r = 0; r < M; ++r) acc[r] = fmaf(static_cast<float>(d[gi][r]), s_now[gi][r], acc[r]);
+      }
+      if constexpr (!MULTI) break;
     }
     float* pbuf = part + buf * wk * kDigits * M * kTileRows;
     if (blk < kDigits) {
@@ -504,9 +519,9 @@ constexpr int kFullKMinTiles = 1024;
 constexpr int kLdsDefault = 64 * 1024;   // dynamic LDS a kernel may use without opting in
 constexpr int kLdsMax = 160 * 1024;      // LDS of one gfx950 CU
 
-template <typename T, int BITS, int M, int MAXT>
+template <typename T, int BITS, int M, int MAXT, bool MULTI>
 int launch_one(const MfmaArgs& a, int wk, int grid, int lds, hipStream_t stream) {
-  auto kernel = wq_gemv_mfma_kernel<T, BITS, M, MAXT>;
+  auto kernel = wq_gemv_mfma_kernel<T, BITS, M, MAXT, MULTI>;
   if (lds > kLdsDefault) {
     static bool raised = false;  // per instantiation; worst case two threads both set it
     if (!raised) {
@@ -525,9 +540,21 @@ int launch_one(const MfmaArgs& a, int wk, int grid, int lds, hipStream_t stream)
 
 template <typename T, int BITS, int M>
 int launch_m(const MfmaArgs& a, int wk, int grid, int lds, hipStream_t stream) {
-  if (wk <= 4) return launch_one<T, BITS, M, 256>(a, wk, grid, lds, stream);
-  if (wk <= 8) return launch_one<T, BITS, M, 512>(a, wk, grid, lds, stream);
-  return launch_one<T, BITS, M, 1024>(a, wk, grid, lds, stream);
+  if (wk * kGW < a.G) return launch_one<T, BITS, M, 512, true>(a, wk, grid, lds, stream);
+  if (wk <= 4) return launch_one<T, BITS, M, 256, false>(a, wk, grid, lds, stream);
+  if (wk <= 8) return launch_one<T, BITS, M, 512, false>(a, wk, grid, lds, stream);
+  return launch_one<T, BITS, M, 1024, false>(a, wk, grid, lds, stream);
+}
+
+// Waves per workgroup for rows of n_chunks chunks: one per chunk up to 16; beyond that (the
+// multi-chunk kernel, which needs more registers than a 16-wave workgroup leaves) the largest
+// count in 5..8 that divides the chunks evenly, else 8 (the last round is then partly idle).
+int waves_for(int n_chunks) {
+  if (n_chunks <= 16) return n_chunks;
+  for (int w = 8; w >= 5; --w) {
+    if (n_chunks % w == 0) return w;
+  }
+  return 8;
 }
 
 struct FusedOps {
@@ -562,15 +589,25 @@ int launch_typed(const void* x, const void* qw, const float* ws, void* out, int 
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), L.part_off, stream, a);
     return llmq_host::check_launch("wq_gemv_mfma_fullk_kernel");
   }
-  const int wk = (G + kGW - 1) / kGW;
+  const int wk = waves_for(G / kGW);
   const LdsLayout L(M, G, wk, BITS == 4);
-  // resident workgroups: up to 2048 threads per CU and the LDS they need
-  int per_cu = 2048 / (wk * kWave);
+  // Resident workgroups: the kernel's ~100 registers allow 16 waves per CU, and the LDS must fit.
+  // A workgroup stages the activation once and then walks row tiles, so for mid-sized N the grid
+  // is sized to be resident all at once and to give every workgroup the same number of tiles.
+  int per_cu = 16 / wk;
   const int by_lds = kLdsMax / L.total;
   if (per_cu > by_lds) per_cu = by_lds;
   if (per_cu < 1) per_cu = 1;
-  int grid = 256 * per_cu;
-  if (grid > a.n_tiles) grid = a.n_tiles;
+  const int resident = 256 * per_cu;
+  int grid;
+  if (a.n_tiles >= 4 * resident) {
+    // long streams: twice the resident count, so that a CU always has a workgroup staging its
+    // activation while the others stream (measured on lm_head: 47.5 us against 51.5 us)
+    grid = 2 * resident;
+  } else {
+    const int rounds = (a.n_tiles + resident - 1) / resident;
+    grid = (a.n_tiles + rounds - 1) / rounds;
+  }
   switch (M) {
     case 1: return launch_m<T, BITS, 1>(a, wk, grid, L.total, stream);
     case 2: return launch_m<T, BITS, 2>(a, wk, grid, L.total, stream);
@@ -586,13 +623,12 @@ namespace llmq_host {
 // Whether the matrix-core GEMV can take this problem (else the caller uses the ALU kernel).
 bool gemv_mfma_supported(const void* x, const void* qw, const float* ws, int M, int G, int gs,
                          int wformat) {
-  if (gs != kGroup || G < kGW || G > 16 * kGW || G % kGW || M < 1 || M > 4) return false;
+  if (gs != kGroup || G < kGW || G % kGW || M < 1 || M > 4) return false;
   if (wformat != LLMQ_W_INT8 && wformat != LLMQ_W_INT4_PACKED) return false;
   const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(qw) |
                          reinterpret_cast<uintptr_t>(ws);
   if (bits & 15u) return false;
-  const int wk = (G + kGW - 1) / kGW;
-  return LdsLayout(M, G, wk, wformat == LLMQ_W_INT4_PACKED).total <= kLdsMax - 1024;
+  return LdsLayout(M, G, waves_for(G / kGW), wformat == LLMQ_W_INT4_PACKED).total <= kLdsMax - 1024;
 }
 
 int gemv_mfma_launch(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,

@@ -137,6 +137,46 @@ def test_llama_1b_layer_shapes(shape, bits):
     assert rel_l2(to_np(got32), exact) <= 1e-3
 
 
+SHAPES_8B = {"q/o": (4096, 4096), "k/v": (1024, 4096), "gate/up": (14336, 4096), "down": (4096, 14336)}
+
+
+@pytest.mark.parametrize("shape", list(SHAPES_8B))
+@pytest.mark.parametrize("bits", [8, 4])
+def test_llama_8b_layer_shapes(shape, bits):
+    """Llama-3-8B linears, M=1; down_proj's rows are 112 groups long (several chunks per wave)."""
+    from llmquant.hip import load_extension
+
+    n, k = SHAPES_8B[shape]
+    gen = torch.Generator().manual_seed(1)
+    w = (torch.randn(n, k, generator=gen) * 0.02).to(torch.bfloat16)
+    x = torch.randn(1, k, generator=gen).to(torch.bfloat16)
+    canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP)
+    q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
+    got = load_extension().wq_gemv(x.cuda(), q, torch.from_numpy(scales).cuda(), 0)
+    exact = oracle.gemv_float64(to_np(x), canonical, scales)
+    assert rel_l2(to_np(got), exact) <= 1e-2
+    got32 = load_extension().wq_gemv(x.cuda().float(), q, torch.from_numpy(scales).cuda(), 0)
+    assert rel_l2(to_np(got32), exact) <= 1e-3
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("M", [1, 2, 3])
+@pytest.mark.parametrize("n,k", [(100, 8704), (70, 28672), (33, 2560 * 4)])
+def test_rows_longer_than_64_groups(bits, M, n, k):
+    """68, 224 and 80 groups: 17 chunks (uneven over 8 waves), 56 (7 rounds of 8), 20 (4 rounds of 5)."""
+    from llmquant.hip import load_extension
+
+    gen = torch.Generator().manual_seed(n)
+    w = (torch.randn(n, k, generator=gen) * 0.02).to(torch.bfloat16)
+    x = torch.randn(M, k, generator=gen)
+    canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP)
+    q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
+    got = load_extension().wq_gemv(x.cuda(), q, torch.from_numpy(scales).cuda(), 0)
+    exact = oracle.gemv_float64(to_np(x), canonical, scales)
+    assert got.shape == (M, n)
+    assert rel_l2(to_np(got), exact) <= 1e-5
+
+
 def test_lm_head_shape_by_linearity():
     """Full-size untied lm_head (128256 x 2048, int8), checked through properties that need
     no CPU GEMV: rows against float64 on a sample, and linearity in x."""
