@@ -88,6 +88,15 @@ int llmq_wq_gemv_fused(const void* x, const void* qweight, const float* wscale, 
                        const void* norm_weight, float eps, int in_head_dim,
                        const void* residual_or_null, llmq_stream_t stream);
 
+/* The dense form of a quantized weight, out[n, g*keep + k] = (dtype)(code[n,g,k] * wscale[sr(n),g])
+ * for k < keep_per_group <= gs: the matrix KernelQuantLinear builds per forward when more rows
+ * arrive than the GEMV takes (`_dequantized_weight`, llmquant/quantizers/kernel.py:68-79), in one
+ * pass. keep_per_group < gs drops the zero padding of head-aligned groups, giving the layer's real
+ * input width. out: [N, G*keep_per_group] `dtype`. gs a multiple of 16 (int8) or 32 (packed). */
+int llmq_dequant_weight(const void* qweight, const float* wscale, void* out, int N, int G, int gs,
+                        int keep_per_group, int out_group, int wformat, int dtype,
+                        llmq_stream_t stream);
+
 /* Integer GEMM with per-group scales on both operands (the A8 branch of
  * RealQuantLinear.forward, llmquant/quantizers/real.py:76-103):
  *   out[m, n] = sum over g, in order, of  float(sum_k a[m,g,k]*q[n,g,k]) * sw[sr(n), g] * sx[m, g]

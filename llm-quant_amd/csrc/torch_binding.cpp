@@ -136,6 +136,35 @@ at::Tensor wq_gemv(const at::Tensor& x, const at::Tensor& qweight, const at::Ten
   return out;
 }
 
+// qweight [N, G, gs] int8 or [N, G, gs/2] packed uint8 -> dense [N, G*keep] in out_dtype.
+at::Tensor dequant_weight(const at::Tensor& qweight, const at::Tensor& wscale, int64_t out_group,
+                          int64_t keep_per_group, at::ScalarType out_dtype) {
+  TORCH_CHECK(qweight.is_cuda() && wscale.is_cuda(), "all tensors must be CUDA");
+  TORCH_CHECK(qweight.dim() == 3 && qweight.is_contiguous(), "qweight must be contiguous [N, groups, group_size]");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar,
+              "qweight must be int8, or uint8 for nibble-packed int4");
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 2 && wscale.is_contiguous(),
+              "wscale must be contiguous float32 [scale_rows, groups]");
+  const int64_t N = qweight.size(0), groups = qweight.size(1);
+  const int64_t group_size = packed ? qweight.size(2) * 2 : qweight.size(2);
+  if (keep_per_group <= 0) keep_per_group = group_size;
+  TORCH_CHECK(out_group >= 0, "out_group must be >= 0");
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  TORCH_CHECK(wscale.size(0) == scale_rows && wscale.size(1) == groups, "wscale must be [", scale_rows,
+              ", ", groups, "], got [", wscale.size(0), ", ", wscale.size(1), "]");
+  auto out = at::empty({N, groups * keep_per_group}, qweight.options().dtype(out_dtype));
+  const int dtype = dtype_code(out, "output dtype");
+  if (out.numel() == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(qweight));
+  check_rc(llmq_dequant_weight(qweight.const_data_ptr(), wscale.const_data_ptr<float>(), out.mutable_data_ptr(),
+                               static_cast<int>(N), static_cast<int>(groups), static_cast<int>(group_size),
+                               static_cast<int>(keep_per_group), static_cast<int>(out_group),
+                               packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype, current_stream(qweight)),
+           "dequant_weight");
+  return out;
+}
+
 // One activation row through a quantized Linear with the surrounding elementwise operations
 // folded in (see llmq_wq_gemv_fused). x: [K] (or [2K] gate|up for prologue 2); returns [N].
 at::Tensor wq_gemv_fused(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale,
@@ -417,5 +446,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "Single-token GQA attention reading the quantized cache",
         py::arg("query"), py::arg("k_codes"), py::arg("v_codes"), py::arg("k_scale"), py::arg("v_scale"),
         py::arg("workspace"), py::arg("length"), py::arg("sm_scale"));
+  m.def("dequant_weight", &dequant_weight,
+        "Dense [N, groups*keep_per_group] matrix of a quantized weight (keep_per_group <= 0: whole groups)",
+        py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("keep_per_group") = 0,
+        py::arg("out_dtype") = at::kBFloat16);
   m.def("abi_version", []() { return llmq_abi_version(); });
 }

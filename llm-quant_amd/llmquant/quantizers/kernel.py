@@ -62,6 +62,10 @@ class KernelQuantLinear(nn.Module):
         self._packed = stored.dtype == torch.uint8
         self._needs_padding = self.in_features != self.padded_in_features
         self._weight_args = scheme.weights
+        # head-aligned groups (o_proj: heads of 64 in groups of 128): real elements per group
+        head_dim = scheme.weights.head_dim
+        self._head_keep = (head_dim if head_dim and head_dim < group_size
+                           and self.in_features == stored.shape[1] * head_dim else 0)
         # int8 activations: the integer GEMM (real-mode arithmetic, bit for bit) serves every M.
         # The reference's kernel mode ignores the activation scheme (kernel.py:97-103); here it
         # is honoured when the geometry allows (one activation group per weight group of 128).
@@ -93,12 +97,24 @@ class KernelQuantLinear(nn.Module):
         repeat = self.out_features // self.wscale.shape[0]
         return self.wscale.repeat_interleave(repeat, dim=0).unsqueeze(-1)
 
-    def _dequantized_weight(self, dtype):
-        """[out, padded_in] in the activation dtype, rebuilt per call and never cached."""
+    def _dequantized_weight(self, dtype, real_width: bool = False):
+        """[out, padded_in] in the activation dtype, rebuilt per call and never cached: one kernel
+        pass (the reference multiplies and casts in PyTorch, kernel.py:68-79). With `real_width`
+        and head-aligned groups the zero padding is dropped: [out, in_features]."""
+        group_size = self.padded_in_features // self.qdata.shape[1]
+        if group_size % (32 if self._packed else 16) == 0:
+            keep = self._head_keep if real_width else 0
+            return self._ext.dequant_weight(self.qdata, self.wscale, self.out_group, keep, dtype)
         return (self.qweight * self._broadcast_scale).to(dtype).reshape(self.out_features, -1)
 
     def forward(self, x):
         rows = x.reshape(-1, x.shape[-1])
+        if rows.shape[0] > KERNEL_MAX_ROWS and not self._int8_act and self._head_keep:
+            # dense branch on the real width: neither the activation nor the weight is padded
+            out = rows @ self._dequantized_weight(rows.dtype, real_width=True).T
+            if self.bias is not None:
+                out = out + self.bias.to(out.dtype)
+            return out.reshape(*x.shape[:-1], self.out_features).to(x.dtype)
         if self._needs_padding:
             rows = pad_activation(rows, self._weight_args)
         if self._int8_act:

@@ -354,3 +354,31 @@ def test_bare_c_abi_call(linear):
     assert rel_l2(to_np(out), oracle.gemv_float64(to_np(x), canonical, scales)) <= 1e-2
     assert lib.llmq_wq_gemv(x.data_ptr(), q.data_ptr(), s.data_ptr(), out.data_ptr(), 1, N, 16, GROUP,
                             0, 5, 2, stream) == 1
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_dequant_weight_is_code_times_scale_rounded_once(bits, dtype):
+    """The dense matrix of the M > 4 branch: (dtype)(code * scale) per element, bit for bit,
+    whole groups and with the head padding dropped."""
+    from llmquant.hip import load_extension
+
+    ext = load_extension()
+    gen = torch.Generator().manual_seed(9)
+    n, heads, head_dim = 96, 6, 64
+    w = (torch.randn(n, heads * head_dim, generator=gen) * 0.05).to(torch.bfloat16)
+    for hd, out_group in ((None, None), (head_dim, None), (None, 32)):
+        canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP, hd, out_group)
+        q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
+        s = torch.from_numpy(scales).cuda()
+        rows = np.repeat(scales, out_group, axis=0)[:n] if out_group else scales
+        want = torch.from_numpy(canonical.astype(np.float32) * rows[..., None]).to(dtype)
+        got = ext.dequant_weight(q, s, out_group or 0, 0, dtype)
+        assert got.shape == (n, canonical.shape[1] * GROUP) and got.dtype == dtype
+        assert torch.equal(got.cpu(), want.reshape(n, -1))
+        if hd:
+            real = ext.dequant_weight(q, s, 0, hd, dtype)
+            assert real.shape == (n, heads * head_dim)
+            assert torch.equal(real.cpu(), want[:, :, :hd].reshape(n, -1))
+    with pytest.raises(RuntimeError, match="keep_per_group"):
+        ext.dequant_weight(q, s, 32, 200, dtype)
