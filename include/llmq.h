@@ -71,6 +71,20 @@ int llmq_wq_gemv(const void* x, const void* qweight, const float* wscale, void* 
                  int N, int G, int gs, int out_group, int wformat, int dtype,
                  llmq_stream_t stream);
 
+/* Many small GEMVs in one launch: the routed experts of a Mixture-of-Experts layer. Replaces
+ * wq_gemv_batched (llmquant/cuda/csrc/wq_gemv_batched.cu:39-186). qweight is [E, N, G, gs] (or
+ * packed [E, N, G, gs/2]), wscale [E, scale_rows, G]. Plan entry b (three device int32 arrays of
+ * n_blocks entries, built by the caller on the device and never read by the host) says: rows
+ * block_row0[b] .. +block_rows[b]-1 of x [n_rows, G*gs] go through expert block_expert[b]; an entry
+ * with block_rows <= 0 is skipped, one that points outside x or the expert stack is ignored. A run
+ * holds at most llmq_wq_gemv_batched_max_rows() rows. out: [n_rows, N]; rows no entry covers are
+ * left untouched. Each row's arithmetic is llmq_wq_gemv's. */
+int llmq_wq_gemv_batched_max_rows(void);
+int llmq_wq_gemv_batched(const void* x, const void* qweight, const float* wscale, void* out,
+                         const int32_t* block_expert, const int32_t* block_row0,
+                         const int32_t* block_rows, int n_blocks, int n_rows, int n_experts, int N,
+                         int G, int gs, int out_group, int wformat, int dtype, llmq_stream_t stream);
+
 /* The decode-step form of llmq_wq_gemv (M = 1, group size 128): the same product with the
  * elementwise operations that surround a Linear in a Llama decoder layer folded in, so that a
  * layer is five launches instead of ~40. There is no counterpart in the reference, which leaves

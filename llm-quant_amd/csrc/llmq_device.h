@@ -161,4 +161,10 @@ int gemv_mfma_launch(const void* x, const void* qw, const float* ws, void* out, 
 int gemv_mfma_launch_fused(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
                            int out_group, int wformat, int dtype, int prologue, const void* norm_weight,
                            float eps, int in_head_dim, const void* residual, hipStream_t stream);
+// Batched form (a plan of expert / row runs read on the device): see llmq_wq_gemv_batched.
+bool gemv_batched_mfma_supported(const void* x, const void* qw, const float* ws, int G, int gs, int wformat);
+int gemv_batched_mfma_launch(const void* x, const void* qw, const float* ws, void* out, const int32_t* block_expert,
+                             const int32_t* block_row0, const int32_t* block_rows, int n_blocks, int n_rows,
+                             int n_experts, int N, int G, int out_group, int wformat, int dtype,
+                             hipStream_t stream);
 }  // namespace llmq_host

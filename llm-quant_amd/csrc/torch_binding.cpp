@@ -136,6 +136,49 @@ at::Tensor wq_gemv(const at::Tensor& x, const at::Tensor& qweight, const at::Ten
   return out;
 }
 
+// x [R, G*gs]; qweight [E, N, G, gs] int8 or [E, N, G, gs/2] packed; wscale [E, scale_rows, G]; the plan is
+// three int32 device tensors of equal length. Returns [R, N]; rows no plan entry covers are zero.
+at::Tensor wq_gemv_batched(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale,
+                           const at::Tensor& block_expert, const at::Tensor& block_row0,
+                           const at::Tensor& block_rows, int64_t out_group) {
+  TORCH_CHECK(x.is_cuda() && qweight.is_cuda() && wscale.is_cuda() && block_expert.is_cuda() &&
+                  block_row0.is_cuda() && block_rows.is_cuda(), "all tensors must be CUDA");
+  TORCH_CHECK(qweight.dim() == 4, "qweight must be [experts, N, groups, group_size], got ", qweight.dim(), "D");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar,
+              "qweight must be int8, or uint8 for nibble-packed int4");
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 3, "wscale must be float32 [experts, scale_rows, groups]");
+  const int dtype = dtype_code(x, "x");
+  TORCH_CHECK(x.dim() == 2, "x must be [rows, in_features]");
+  const auto xc = x.contiguous();
+  const auto wc = qweight.contiguous();
+  const auto sc = wscale.contiguous();
+  const auto be = block_expert.to(at::kInt).contiguous();
+  const auto b0 = block_row0.to(at::kInt).contiguous();
+  const auto br = block_rows.to(at::kInt).contiguous();
+  TORCH_CHECK(be.dim() == 1 && b0.sizes() == be.sizes() && br.sizes() == be.sizes(),
+              "block_expert, block_row0 and block_rows must be 1-D and of equal length");
+  const int64_t E = wc.size(0), N = wc.size(1), groups = wc.size(2);
+  const int64_t group_size = packed ? wc.size(3) * 2 : wc.size(3);
+  TORCH_CHECK(xc.size(1) == groups * group_size, "x last dim ", xc.size(1), " does not match qweight ", groups,
+              "x", group_size);
+  TORCH_CHECK(out_group >= 0, "out_group must be >= 0");
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  TORCH_CHECK(sc.size(0) == E && sc.size(1) == scale_rows && sc.size(2) == groups, "wscale must be [", E, ", ",
+              scale_rows, ", ", groups, "]");
+  auto out = at::zeros({xc.size(0), N}, xc.options());
+  if (out.numel() == 0 || be.numel() == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(xc));
+  check_rc(llmq_wq_gemv_batched(xc.const_data_ptr(), wc.const_data_ptr(), sc.const_data_ptr<float>(),
+                                out.mutable_data_ptr(), be.const_data_ptr<int32_t>(), b0.const_data_ptr<int32_t>(),
+                                br.const_data_ptr<int32_t>(), static_cast<int>(be.numel()),
+                                static_cast<int>(xc.size(0)), static_cast<int>(E), static_cast<int>(N),
+                                static_cast<int>(groups), static_cast<int>(group_size), static_cast<int>(out_group),
+                                packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype, current_stream(xc)),
+           "wq_gemv_batched");
+  return out;
+}
+
 // qweight [N, G, gs] int8 or [N, G, gs/2] packed uint8 -> dense [N, G*keep] in out_dtype.
 at::Tensor dequant_weight(const at::Tensor& qweight, const at::Tensor& wscale, int64_t out_group,
                           int64_t keep_per_group, at::ScalarType out_dtype) {
@@ -446,6 +489,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "Single-token GQA attention reading the quantized cache",
         py::arg("query"), py::arg("k_codes"), py::arg("v_codes"), py::arg("k_scale"), py::arg("v_scale"),
         py::arg("workspace"), py::arg("length"), py::arg("sm_scale"));
+  m.def("wq_gemv_batched", &wq_gemv_batched,
+        "One launch over every routed expert: rows block_row0[b].. of x through expert block_expert[b]",
+        py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("block_expert"), py::arg("block_row0"),
+        py::arg("block_rows"), py::arg("out_group") = 0);
+  m.def("wq_gemv_batched_max_rows", []() { return llmq_wq_gemv_batched_max_rows(); });
   m.def("dequant_weight", &dequant_weight,
         "Dense [N, groups*keep_per_group] matrix of a quantized weight (keep_per_group <= 0: whole groups)",
         py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("keep_per_group") = 0,

@@ -237,6 +237,58 @@ __global__ __launch_bounds__(256) void wq_gemv_scalar_kernel(
   }
 }
 
+// The batched form of the fallback: plan entry blockIdx.y names an expert and a run of rows.
+template <typename T, int BITS>
+__global__ __launch_bounds__(256) void wq_gemv_batched_scalar_kernel(
+    const T* __restrict__ x, const uint8_t* __restrict__ qw, const float* __restrict__ ws, T* __restrict__ out,
+    const int32_t* __restrict__ block_expert, const int32_t* __restrict__ block_row0,
+    const int32_t* __restrict__ block_rows, int n_rows, int n_experts, int N, int G, int gs, int out_group) {
+  const int b = blockIdx.y;
+  const int rows = block_rows[b];
+  if (rows <= 0) return;
+  const int e = block_expert[b], row0 = block_row0[b];
+  if (e < 0 || e >= n_experts || row0 < 0 || row0 + rows > n_rows) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int n = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (n >= N) return;
+  const int64_t k_total = static_cast<int64_t>(G) * gs;
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  const int srow = out_group > 0 ? n / out_group : n;
+  const float* wse = ws + (static_cast<int64_t>(e) * scale_rows + srow) * G;
+  const int64_t w0 = (static_cast<int64_t>(e) * N + n) * k_total;  // in codes
+  for (int m = row0; m < row0 + rows; ++m) {
+    float acc = 0.0f;
+    for (int g = 0; g < G; ++g) {
+      float part = 0.0f;
+      for (int k = lane; k < gs; k += kWave) {
+        const int64_t idx = w0 + static_cast<int64_t>(g) * gs + k;
+        int code;
+        if constexpr (BITS == 8) {
+          code = static_cast<int8_t>(qw[idx]);
+        } else {
+          const uint8_t byte = qw[idx >> 1];
+          code = static_cast<int>((idx & 1) ? (byte >> 4) : (byte & 0xf)) - 8;
+        }
+        part = fmaf(static_cast<float>(code), to_float(x[m * k_total + g * gs + k]), part);
+      }
+      acc = fmaf(part, wse[g], acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) out[static_cast<int64_t>(m) * N + n] = from_float<T>(acc);
+  }
+}
+
+template <typename T, int BITS>
+int launch_batched_scalar(const void* x, const void* qw, const float* ws, void* out, const int32_t* be,
+                          const int32_t* b0, const int32_t* br, int n_blocks, int n_rows, int n_experts, int N,
+                          int G, int gs, int out_group, hipStream_t stream) {
+  const dim3 g((N + 3) / 4, n_blocks), b(256);
+  hipLaunchKernelGGL((wq_gemv_batched_scalar_kernel<T, BITS>), g, b, 0, stream, static_cast<const T*>(x),
+                     static_cast<const uint8_t*>(qw), ws, static_cast<T*>(out), be, b0, br, n_rows, n_experts, N, G,
+                     gs, out_group);
+  return llmq_host::check_launch("wq_gemv_batched_scalar_kernel");
+}
+
 template <typename T, int BITS, int M>
 int launch_rows(const GemvArgs& base, int N, hipStream_t stream) {
   GemvArgs a = base;
@@ -374,9 +426,51 @@ extern "C" int llmq_wq_gemv_fused(const void* x, const void* qweight, const floa
   if (N == 0) return 0;
   if (!x || !qweight || !wscale || !out) return llmq_host::fail_invalid("null tensor pointer");
   if (!llmq_host::gemv_mfma_supported(x, qweight, wscale, 1, G, 128, wformat))
-    return llmq_host::fail_invalid("the fused GEMV needs group size 128, a multiple of 4 groups (at most 64) "
+    return llmq_host::fail_invalid("the fused GEMV needs group size 128, a multiple of 4 groups "
                                    "and 16-byte aligned operands");
   return llmq_host::gemv_mfma_launch_fused(x, qweight, wscale, out, 1, N, G, out_group, wformat, dtype, prologue,
                                            norm_weight, eps, in_head_dim, residual_or_null,
                                            static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmq_wq_gemv_batched_max_rows(void) { return 8; }
+
+extern "C" int llmq_wq_gemv_batched(const void* x, const void* qweight, const float* wscale, void* out,
+                                    const int32_t* block_expert, const int32_t* block_row0,
+                                    const int32_t* block_rows, int n_blocks, int n_rows, int n_experts, int N,
+                                    int G, int gs, int out_group, int wformat, int dtype, llmq_stream_t stream) {
+  if (n_blocks < 0 || n_rows < 0 || n_experts < 0 || N < 0 || G < 0)
+    return llmq_host::fail_invalid("negative dimension blocks=%d rows=%d experts=%d N=%d G=%d", n_blocks, n_rows,
+                                   n_experts, N, G);
+  if (gs <= 0) return llmq_host::fail_invalid("group_size must be positive, got %d", gs);
+  if (out_group < 0) return llmq_host::fail_invalid("out_group must be >= 0, got %d", out_group);
+  if (wformat != LLMQ_W_INT8 && wformat != LLMQ_W_INT4_PACKED)
+    return llmq_host::fail_invalid("unsupported weight format %d, expected 8 or 4", wformat);
+  if (wformat == LLMQ_W_INT4_PACKED && gs % 2)
+    return llmq_host::fail_invalid("group_size must be even for packed int4, got %d", gs);
+  if (n_blocks == 0 || n_rows == 0 || N == 0 || n_experts == 0) return 0;
+  if (n_blocks > 65535) return llmq_host::fail_invalid("at most 65535 plan entries per launch, got %d", n_blocks);
+  if (G == 0) return llmq_host::fail_invalid("a weight with no groups has no reduction axis");
+  if (!x || !qweight || !wscale || !out || !block_expert || !block_row0 || !block_rows)
+    return llmq_host::fail_invalid("null tensor pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // every expert's weight must be as aligned as the first one's
+  const int64_t weight_stride = static_cast<int64_t>(N) * G * gs * (wformat == LLMQ_W_INT8 ? 2 : 1) / 2;
+  if (weight_stride % 16 == 0 && llmq_host::gemv_batched_mfma_supported(x, qweight, wscale, G, gs, wformat)) {
+    return llmq_host::gemv_batched_mfma_launch(x, qweight, wscale, out, block_expert, block_row0, block_rows,
+                                               n_blocks, n_rows, n_experts, N, G, out_group, wformat, dtype, s);
+  }
+#define LLMQ_SCALAR(T)                                                                                        \
+  (wformat == LLMQ_W_INT8                                                                                     \
+       ? launch_batched_scalar<T, 8>(x, qweight, wscale, out, block_expert, block_row0, block_rows, n_blocks, \
+                                     n_rows, n_experts, N, G, gs, out_group, s)                               \
+       : launch_batched_scalar<T, 4>(x, qweight, wscale, out, block_expert, block_row0, block_rows, n_blocks, \
+                                     n_rows, n_experts, N, G, gs, out_group, s))
+  switch (dtype) {
+    case LLMQ_F32: return LLMQ_SCALAR(float);
+    case LLMQ_F16: return LLMQ_SCALAR(f16_t);
+    case LLMQ_BF16: return LLMQ_SCALAR(bf16_t);
+  }
+#undef LLMQ_SCALAR
+  return llmq_host::fail_invalid("x must be float32, float16 or bfloat16, got dtype code %d", dtype);
 }

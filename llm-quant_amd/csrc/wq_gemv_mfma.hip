@@ -111,10 +111,11 @@ struct Prologue {
 // rint(x * 2^sh) in three planes laid out so a lane's MFMA operand is 16 contiguous bytes,
 // the group's 2^-sh in cxs[m*G + g] and (int4 only) the digit sums in csum[(q*M + m)*G + g].
 // Every thread of the block must call it; the caller synchronises afterwards.
+// Rows m >= m_valid are not read and stage as zeros.
 template <typename T, int BITS, int M>
 __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const int G, const LdsLayout& L,
                                                  int8_t* dig, float* cxs, int* csum, const Prologue pro,
-                                                 float* red) {
+                                                 float* red, const int m_valid = M) {
   const int tid = threadIdx.x;
   const int items = M * G * 16;  // 8 elements each; 16 consecutive items are one group
   const int real_per_group = pro.in_head_dim > 0 ? pro.in_head_dim : kGroup;
@@ -154,7 +155,8 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
     float f[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) f[e] = 0.0f;
-    const bool real = active && tq * 8 < real_per_group;  // beyond it: the zero padding of a head group
+    // beyond real_per_group: the zero padding of a head group
+    const bool real = active && tq * 8 < real_per_group && m < m_valid;
     if (real) {
       const int64_t src = static_cast<int64_t>(m) * k_real + g * real_per_group + tq * 8;
       if (pro.kind == LLMQ_PRO_RMSNORM && base == 0) {
@@ -239,9 +241,9 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
 // activation fragments stay in registers for the whole kernel. MULTI == true: longer rows; wave w
 // takes chunks w, w + waves, ... of every row tile and re-reads the fragments of the chunk it is
 // about to multiply from LDS (the read is issued with the weight loads, a chunk ahead).
-template <typename T, int BITS, int M, int MAXT, bool MULTI>
-__global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+template <typename T, int BITS, int M, bool MULTI>
+__device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* smem, const int first_tile,
+                                            const int tile_stride, const int m_valid) {
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wv = tid / kWave;
@@ -311,18 +313,18 @@ __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
     }
   };
 
-  int tile = blockIdx.x;
+  int tile = first_tile;
   if (tile < a.n_tiles) issue_loads(tile, wv);  // in flight while the activation is prepared
 
   stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum,
-                               Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim}, red);
+                               Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim}, red, m_valid);
   __syncthreads();
   load_fragments(wv);
 
   // ---- stream row tiles -----------------------------------------------------------------------
   T* __restrict__ out = static_cast<T*>(a.out);
   int buf = 0;
-  for (; tile < a.n_tiles; tile += gridDim.x) {
+  for (; tile < a.n_tiles; tile += tile_stride) {
     float acc[M];
 #pragma unroll
     for (int r = 0; r < M; ++r) acc[r] = 0.0f;
@@ -351,8 +353,8 @@ __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
       if (next_chunk < n_chunks) {
         issue_loads(tile, next_chunk);
         load_fragments(next_chunk);
-      } else if (tile + static_cast<int>(gridDim.x) < a.n_tiles) {
-        issue_loads(tile + gridDim.x, wv);
+      } else if (tile + tile_stride < a.n_tiles) {
+        issue_loads(tile + tile_stride, wv);
         if constexpr (MULTI) load_fragments(wv);
       }
 #pragma unroll
@@ -382,10 +384,54 @@ __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
         total += __shfl_xor(total, 16, kWave);
         total += __shfl_xor(total, 32, kWave);
         const int n = tile * kTileRows + jj;
-        if (ws == 0 && n < a.N) out[static_cast<int64_t>(r) * a.N + n] = finish<T>(total, a.residual, n);
+        if (ws == 0 && n < a.N && r < m_valid) {
+          out[static_cast<int64_t>(r) * a.N + n] = finish<T>(total, a.residual, n);
+        }
       }
     }
     buf ^= 1;
+  }
+}
+
+template <typename T, int BITS, int M, int MAXT, bool MULTI>
+__global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  ksplit_body<T, BITS, M, MULTI>(a, smem, blockIdx.x, gridDim.x, M);
+}
+
+// Many small GEMVs in one launch (the routed experts of a Mixture-of-Experts layer). Plan entry
+// b = blockIdx.y names an expert's weight and a run of consecutive activation rows (a run never
+// spans two experts); an entry with no rows costs a workgroup one load and an exit. Runs of up
+// to kBatchedMaxRows rows are taken four at a time; a row's arithmetic is the single-launch
+// kernel's, so its result does not depend on what it is batched with.
+struct BatchPlan {
+  const int32_t* expert;
+  const int32_t* row0;
+  const int32_t* rows;
+  int n_experts, n_rows;
+  int64_t weight_stride;  // bytes between experts' weights
+  int64_t scale_stride;   // floats between experts' scales
+};
+constexpr int kBatchedMaxRows = 8;
+
+template <typename T, int BITS, int MAXT, bool MULTI>
+__global__ __launch_bounds__(MAXT) void wq_gemv_mfma_batched_kernel(MfmaArgs a, const BatchPlan plan) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int b = blockIdx.y;
+  const int rows = min(plan.rows[b], kBatchedMaxRows);
+  if (rows <= 0) return;
+  const int e = plan.expert[b], row0 = plan.row0[b];
+  if (e < 0 || e >= plan.n_experts || row0 < 0 || row0 + rows > plan.n_rows) return;  // not a valid run
+  a.qw += e * plan.weight_stride;
+  a.ws += e * plan.scale_stride;
+  const int64_t k_total = static_cast<int64_t>(a.G) * kGroup;
+  const T* x = static_cast<const T*>(a.x);
+  T* out = static_cast<T*>(a.out);
+  for (int done = 0; done < rows; done += 4) {
+    if (done > 0) __syncthreads();  // the previous pass is done with the LDS
+    a.x = x + (row0 + done) * k_total;
+    a.out = out + static_cast<int64_t>(row0 + done) * a.N;
+    ksplit_body<T, BITS, 4, MULTI>(a, smem, blockIdx.x, gridDim.x, min(4, rows - done));
   }
 }
 
@@ -646,6 +692,65 @@ int gemv_mfma_launch_fused(const void* x, const void* qw, const float* ws, void*
 #define LLMQ_DISPATCH(T)                                                                          \
   (wformat == LLMQ_W_INT8 ? launch_typed<T, 8>(x, qw, ws, out, M, N, G, out_group, ops, stream)   \
                           : launch_typed<T, 4>(x, qw, ws, out, M, N, G, out_group, ops, stream))
+  switch (dtype) {
+    case LLMQ_F32: return LLMQ_DISPATCH(float);
+    case LLMQ_F16: return LLMQ_DISPATCH(f16_t);
+    case LLMQ_BF16: return LLMQ_DISPATCH(bf16_t);
+  }
+#undef LLMQ_DISPATCH
+  return fail_invalid("x must be float32, float16 or bfloat16, got dtype code %d", dtype);
+}
+
+namespace {
+template <typename T, int BITS>
+int launch_batched(const MfmaArgs& a, const BatchPlan& plan, int n_blocks, hipStream_t stream) {
+  const int wk = waves_for(a.G / kGW);
+  const bool multi = wk * kGW < a.G;
+  const LdsLayout L(4, a.G, wk, BITS == 4);
+  int gx = a.n_tiles < 256 ? a.n_tiles : 256;
+  const dim3 grid(gx, n_blocks), block(wk * kWave);
+#define LLMQ_BATCHED(MAXT, MULTI)                                                                   \
+  do {                                                                                              \
+    auto kernel = wq_gemv_mfma_batched_kernel<T, BITS, MAXT, MULTI>;                                \
+    if (L.total > kLdsDefault) {                                                                    \
+      const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),             \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax); \
+      if (err != hipSuccess) {                                                                      \
+        set_error("raising the LDS limit failed: %s", hipGetErrorString(err));                      \
+        return static_cast<int>(err);                                                               \
+      }                                                                                             \
+    }                                                                                               \
+    hipLaunchKernelGGL(kernel, grid, block, L.total, stream, a, plan);                              \
+  } while (0)
+  if (multi) LLMQ_BATCHED(512, true);
+  else if (wk <= 4) LLMQ_BATCHED(256, false);
+  else if (wk <= 8) LLMQ_BATCHED(512, false);
+  else LLMQ_BATCHED(1024, false);
+#undef LLMQ_BATCHED
+  return check_launch("wq_gemv_mfma_batched_kernel");
+}
+}  // namespace
+
+// Whether the matrix-core batched GEMV can take the problem: the single-launch kernel's
+// conditions for four rows.
+bool gemv_batched_mfma_supported(const void* x, const void* qw, const float* ws, int G, int gs, int wformat) {
+  return gemv_mfma_supported(x, qw, ws, 4, G, gs, wformat);
+}
+
+int gemv_batched_mfma_launch(const void* x, const void* qw, const float* ws, void* out, const int32_t* block_expert,
+                             const int32_t* block_row0, const int32_t* block_rows, int n_blocks, int n_rows,
+                             int n_experts, int N, int G, int out_group, int wformat, int dtype,
+                             hipStream_t stream) {
+  MfmaArgs a{};
+  a.x = x; a.qw = static_cast<const uint8_t*>(qw); a.ws = ws; a.out = out;
+  a.N = N; a.G = G; a.out_group = out_group;
+  a.n_tiles = (N + kTileRows - 1) / kTileRows;
+  a.row_bytes = G * kGroup * (wformat == LLMQ_W_INT8 ? 8 : 4) / 8;
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  BatchPlan plan{block_expert, block_row0, block_rows, n_experts, n_rows,
+                 static_cast<int64_t>(N) * a.row_bytes, scale_rows * G};
+#define LLMQ_DISPATCH(T) \
+  (wformat == LLMQ_W_INT8 ? launch_batched<T, 8>(a, plan, n_blocks, stream) : launch_batched<T, 4>(a, plan, n_blocks, stream))
   switch (dtype) {
     case LLMQ_F32: return LLMQ_DISPATCH(float);
     case LLMQ_F16: return LLMQ_DISPATCH(f16_t);

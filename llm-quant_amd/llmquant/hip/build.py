@@ -89,6 +89,9 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_argmax_row.restype = c_int
     lib.llmq_wq_gemm_a8.argtypes = [c_p] * 6 + [c_int] * 7 + [c_p]
     lib.llmq_wq_gemm_a8.restype = c_int
+    lib.llmq_wq_gemv_batched.argtypes = [c_p] * 7 + [c_int] * 9 + [c_p]
+    lib.llmq_wq_gemv_batched.restype = c_int
+    lib.llmq_wq_gemv_batched_max_rows.restype = c_int
     lib.llmq_dequant_weight.argtypes = [c_p, c_p, c_p] + [c_int] * 7 + [c_p]
     lib.llmq_dequant_weight.restype = c_int
     for name in ("llmq_fake_quant_group", "llmq_quant_group_codes", "llmq_wq_gemv", "llmq_kv_append",

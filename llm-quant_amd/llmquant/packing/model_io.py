@@ -7,8 +7,10 @@ dicts filled in this sequence):
   every other state_dict tensor as bfloat16
   non-persistent buffers (e.g. rotary inv_freq) in their own dtype
 meta: model_id, layers{name: in/out features, canonical_shape, weights{...}, input_activations,
-bias}, experts{} (always empty here: the MoE path is not part of this build),
-non_persistent_buffers, kv_cache_bits, plus caller extras.
+bias}, experts{name: num_experts, hidden_dim, intermediate_dim, gate_up_shape, down_shape,
+weights, input_activations} (a Mixture-of-Experts block is written as one entry with its two
+stacked tensors "<name>.qgate_up" / "<name>.qdown" packed like a Linear's and their scales
+"<name>.sgate_up" / "<name>.sdown"), non_persistent_buffers, kv_cache_bits, plus caller extras.
 
 Loading goes straight to the HBM layout: a 4-bit layer's packed bytes are handed to
 KernelQuantLinear as they are (the reference unpacks them back to one code per byte,
@@ -23,6 +25,7 @@ import torch.nn as nn
 from llmquant.core.scheme import QuantizationArgs, QuantizationScheme
 from llmquant.packing.format import read_header, read_packed, write_packed
 from llmquant.packing.packing import pack_weight
+from llmquant.quantizers.experts import KernelQuantExperts
 from llmquant.quantizers.kernel import KernelQuantLinear
 
 _ARG_FIELDS = ("num_bits", "strategy", "group_size", "head_dim", "out_group", "symmetric", "dynamic")
@@ -63,9 +66,33 @@ def save_packed_model(model: nn.Module, path, model_id: str, kv_cache_bits=None,
         if module.bias is not None:
             tensors[f"{name}.bias"] = module.bias
 
+    experts = {}
+    for name, module in model.named_modules():
+        if not isinstance(module, KernelQuantExperts):
+            continue
+        args = module.scheme.weights
+
+        def canonical(shape, packed):
+            return [*shape[:-1], shape[-1] * 2] if packed else list(shape)
+
+        packed = module.gate_up_data.dtype == torch.uint8
+        tensors[f"{name}.qgate_up"] = module.gate_up_data  # already pack_weight(canonical, bits)
+        tensors[f"{name}.sgate_up"] = module.sgate_up
+        tensors[f"{name}.qdown"] = module.down_data
+        tensors[f"{name}.sdown"] = module.sdown
+        experts[name] = {
+            "num_experts": module.num_experts,
+            "hidden_dim": module.hidden_dim,
+            "intermediate_dim": module.intermediate_dim,
+            "gate_up_shape": canonical(module.gate_up_data.shape, packed),
+            "down_shape": canonical(module.down_data.shape, packed),
+            "weights": _args_to_dict(args),
+            "input_activations": _args_to_dict(module.scheme.input_activations),
+        }
+
     # whatever a quantized layer owns (stored or derived) is excluded by prefix, so a derived
     # buffer can never be written as bf16 and later overwrite its exactly computed value
-    owned = tuple(f"{name}." for name in layers)
+    owned = tuple(f"{name}." for name in (*layers, *experts))
     state = model.state_dict()
     for name, tensor in state.items():
         if name.startswith(owned) or name in tensors:
@@ -79,7 +106,7 @@ def save_packed_model(model: nn.Module, path, model_id: str, kv_cache_bits=None,
         tensors[name] = buffer.detach()
         non_persistent.append(name)
 
-    meta = {"model_id": model_id, "layers": layers, "experts": {}, "non_persistent_buffers": non_persistent,
+    meta = {"model_id": model_id, "layers": layers, "experts": experts, "non_persistent_buffers": non_persistent,
             "kv_cache_bits": kv_cache_bits, **(extra or {})}
     return write_packed(path, tensors, meta)
 
@@ -113,8 +140,6 @@ def load_packed_model(path, device="cuda", dtype=torch.bfloat16, config=None):
     from transformers import AutoConfig, AutoModelForCausalLM
 
     tensors, meta = read_packed(path)
-    if meta.get("experts"):
-        raise NotImplementedError("this build does not load stacked-expert (MoE) layers")
     if config is None:
         config = AutoConfig.from_pretrained(meta["model_id"])
     with torch.device("meta"):
@@ -136,9 +161,28 @@ def load_packed_model(path, device="cuda", dtype=torch.bfloat16, config=None):
             scheme, spec["in_features"])
         _set_submodule(model, name, module)
 
+    for name, spec in (meta.get("experts") or {}).items():
+        args = _args_from_dict(spec["weights"])
+        scheme = QuantizationScheme(weights=args, input_activations=_args_from_dict(spec["input_activations"]))
+
+        def stack(key, shape):
+            stored = tensors[f"{name}.{key}"]
+            shape = list(shape)
+            if stored.dtype == torch.uint8:
+                shape[-1] //= 2  # stays packed
+            else:
+                stored = stored.to(torch.int8)
+            return stored.reshape(shape).to(device)
+
+        # the activation function is architecture, not weights: taken from the block being replaced
+        module = KernelQuantExperts(stack("qgate_up", spec["gate_up_shape"]), tensors[f"{name}.sgate_up"].to(device),
+                                    stack("qdown", spec["down_shape"]), tensors[f"{name}.sdown"].to(device), scheme,
+                                    spec["hidden_dim"], spec["intermediate_dim"], model.get_submodule(name).act_fn)
+        _set_submodule(model, name, module)
+
     _give_storage_to_meta_leftovers(model, device, dtype, provided=set(tensors))
     non_persistent = set(meta.get("non_persistent_buffers", []))
-    owned = tuple(f"{name}." for name in meta["layers"])
+    owned = tuple(f"{name}." for name in (*meta["layers"], *(meta.get("experts") or {})))
     rest = {name: t.to(device=device, dtype=dtype) for name, t in tensors.items()
             if name not in non_persistent and not name.startswith(owned)}
     _, unexpected = model.load_state_dict(rest, strict=False, assign=True)

@@ -17,3 +17,16 @@ def quant_linear_for(mode: str):
 
     return {"fake": stages.FakeQuantLinear, "real": stages.RealQuantLinear,
             "kernel": stages.KernelQuantLinear}[mode]
+
+
+def quant_experts_for(mode: str):
+    """Class that replaces a stacked Mixture-of-Experts block under `mode`, or None for "fake",
+    which quantize-dequantizes the stacked parameters in place and keeps the block
+    (llmquant/quantizers/dispatch.py:37-53)."""
+    if mode not in AVAILABLE_MODES:
+        raise ValueError(f"unsupported mode {mode!r}, expected one of {sorted(AVAILABLE_MODES)}")
+    if mode == "fake":
+        return None
+    import llmquant.quantizers as stages
+
+    return {"real": stages.RealQuantExperts, "kernel": stages.KernelQuantExperts}[mode]

@@ -19,6 +19,10 @@ What pins each function (the tests that do so live in tests/test_oracle_*.py):
   pack_int4            0xD5 example, exhaustive round trip                 (reference tests/test_packing.py:31-46)
   write_packed         magic / version / alignment / round trip            (reference tests/test_packing.py:65-101)
   kv_quant             == fake_quantize at group 64; old tokens untouched  (reference tests/test_kv_cache.py)
+  route_plan           brute force over every row: coverage once, no run over two experts, run length
+                       (reference tests/test_moe.py:310-333)
+  moe_experts_real     per expert == real_linear; tracks transformers' MixtralExperts in bf16
+                       (reference tests/test_moe.py:77-117, 336-345)
   gqa_decode_attention textbook softmax attention in float64 -- parity unpinned against the
                        reference itself: the reference delegates attention to HF transformers
                        and holds no test of its arithmetic.
@@ -277,6 +281,67 @@ def gemv_float64(x, canonical, wscale2d, out_group=None):
     sw = _row_scale(np.asarray(wscale2d, dtype=np.float64), n, out_group)
     w = canonical.astype(np.float64) * sw[:, :, None]
     return np.asarray(x, dtype=np.float64) @ w.reshape(n, -1).T
+
+
+# ---------------------------------------------------------------------------------------------
+# Mixture-of-Experts -- llmquant/quantizers/real.py:117-190, llmquant/quantizers/kernel.py:176-214
+# ---------------------------------------------------------------------------------------------
+
+
+def route_plan(top_k_index, num_experts: int, limit: int):
+    """KernelQuantExperts._plan (kernel.py:176-214) with python loops: rows sorted by expert
+    (stable), every expert given ceil(rows / limit) blocks of at most `limit` rows."""
+    flat = np.asarray(top_k_index).reshape(-1)
+    order = np.argsort(flat, kind="stable")
+    per_expert = max(1, -(-flat.size // limit))
+    expert, row0, length = [], [], []
+    start = 0
+    for e in range(num_experts):
+        count = int((flat == e).sum())
+        for b in range(per_expert):
+            expert.append(e)
+            row0.append(start + b * limit)
+            length.append(min(max(count - b * limit, 0), limit))
+        start += count
+    return order, (np.array(expert), np.array(row0), np.array(length))
+
+
+def silu(x, dtype="bf16"):
+    xf = np.asarray(x, dtype=np.float32)
+    return round_to(xf / (1.0 + np.exp(-xf.astype(np.float64))).astype(np.float32), dtype)
+
+
+def moe_experts_real(hidden, top_k_index, top_k_weights, qgate_up, sgate_up, qdown, sdown, dtype="bf16"):
+    """RealQuantExperts.forward (real.py:160-190): experts in ascending order; for each, the
+    tokens routed to it go through gate_up -> silu(gate) * up -> down as dequantize-then-fp32
+    matmuls with the result rounded to `dtype` after each (here the products are summed in
+    float64 and rounded once), are scaled by the routing weight and added into the output.
+    hidden [T, H] float32 holding `dtype` values; codes [E, N, G, gs]; scales [E, rows, G]."""
+    hidden = np.asarray(hidden, dtype=np.float32)
+    index = np.asarray(top_k_index)
+    weights = np.asarray(top_k_weights, dtype=np.float32)
+    final = np.zeros_like(hidden)
+    h_dim = hidden.shape[1]
+
+    def project(x, codes, scales):
+        n = codes.shape[0]
+        w = codes.astype(np.float64) * _row_scale(scales.astype(np.float64), n, codes.shape[0] // scales.shape[0]
+                                                  if scales.shape[0] != n else None)[:, :, None]
+        w = w.reshape(n, -1)[:, : x.shape[1]]
+        return round_to((x.astype(np.float64) @ w.T).astype(np.float32), dtype)
+
+    for e in range(qgate_up.shape[0]):
+        token, slot = np.nonzero(index == e)
+        if token.size == 0:
+            continue
+        fused = project(hidden[token], qgate_up[e], sgate_up[e])
+        half = fused.shape[1] // 2
+        act = round_to(silu(fused[:, :half], dtype) * fused[:, half:], dtype)
+        out = project(act, qdown[e], sdown[e])
+        out = round_to(out * weights[token, slot, None], dtype)
+        final[token] = round_to(final[token] + out, dtype)
+    assert final.shape[1] == h_dim
+    return final
 
 
 # ---------------------------------------------------------------------------------------------
