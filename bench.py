@@ -330,6 +330,33 @@ def other_kernels(torch):
                               "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)})
             del qs
     out["gemv_llama3_8b_shapes_graph_replay"] = shapes_8b
+    # Mixture-of-Experts decode, OLMoE-1B-7B geometry (64 experts, top-8, hidden 2048, intermediate 1024,
+    # int4): the two batched launches of one layer for one token; 16 layers' stacks rotated, as a graph
+    from llmquant.quantizers import route_plan
+
+    experts, top_k, hid, inter, layers = 64, 8, 2048, 1024, 16
+    gu = [torch.randint(0, 255, (experts, 2 * inter, hid // GROUP, GROUP // 2), dtype=torch.uint8, device=dev)
+          for _ in range(layers)]
+    dn = [torch.randint(0, 255, (experts, hid, inter // GROUP, GROUP // 2), dtype=torch.uint8, device=dev)
+          for _ in range(layers)]
+    sgu = torch.rand(experts, 2 * inter, hid // GROUP, device=dev) * 0.01
+    sdn = torch.rand(experts, hid, inter // GROUP, device=dev) * 0.01
+    index = torch.randperm(experts, device=dev)[:top_k][None]
+    _, plan = route_plan(index, experts, ext.wq_gemv_batched_max_rows())
+    rows_h = torch.randn(top_k, hid, device=dev).to(torch.bfloat16)
+    rows_i = torch.randn(top_k, inter, device=dev).to(torch.bfloat16)
+
+    def moe_step():
+        for layer in range(layers):
+            ext.wq_gemv_batched(rows_h, gu[layer], sgu, *plan, 0)
+            ext.wq_gemv_batched(rows_i, dn[layer], sdn, *plan, 0)
+
+    us = _graph_time_us(torch, moe_step, reps=10) / layers
+    nbytes = top_k * (2 * inter * hid // 2 + hid * inter // 2 + (2 * inter * hid // GROUP + hid * inter // GROUP) * 4)
+    out["moe_batched_gemv_olmoe_int4_top8_per_layer"] = {
+        "us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
+        "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4), "launches": 2}
+    del gu, dn
     # integer GEMM, Llama-3-8B MLP shapes
     gemm = []
     for n, k in ((14336, 4096), (4096, 14336)):

@@ -111,13 +111,14 @@ struct Prologue {
 // rint(x * 2^sh) in three planes laid out so a lane's MFMA operand is 16 contiguous bytes,
 // the group's 2^-sh in cxs[m*G + g] and (int4 only) the digit sums in csum[(q*M + m)*G + g].
 // Every thread of the block must call it; the caller synchronises afterwards.
-// Rows m >= m_valid are not read and stage as zeros.
+// Only rows m < m_valid are staged; what LDS holds for the others is left as it was, which is
+// harmless because the caller never stores their results (integer products cannot trap).
 template <typename T, int BITS, int M>
 __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const int G, const LdsLayout& L,
                                                  int8_t* dig, float* cxs, int* csum, const Prologue pro,
                                                  float* red, const int m_valid = M) {
   const int tid = threadIdx.x;
-  const int items = M * G * 16;  // 8 elements each; 16 consecutive items are one group
+  const int items = m_valid * G * 16;  // 8 elements each; 16 consecutive items are one group
   const int real_per_group = pro.in_head_dim > 0 ? pro.in_head_dim : kGroup;
   const int k_real = G * real_per_group;
 
@@ -707,7 +708,11 @@ int launch_batched(const MfmaArgs& a, const BatchPlan& plan, int n_blocks, hipSt
   const int wk = waves_for(a.G / kGW);
   const bool multi = wk * kGW < a.G;
   const LdsLayout L(4, a.G, wk, BITS == 4);
-  int gx = a.n_tiles < 256 ? a.n_tiles : 256;
+  // about a thousand workgroups over the entries that can hold rows (at most one per row)
+  const int live = plan.n_rows < n_blocks ? plan.n_rows : n_blocks;
+  int gx = 1024 / (live > 0 ? live : 1);
+  if (gx < 16) gx = 16;
+  if (gx > a.n_tiles) gx = a.n_tiles;
   const dim3 grid(gx, n_blocks), block(wk * kWave);
 #define LLMQ_BATCHED(MAXT, MULTI)                                                                   \
   do {                                                                                              \
