@@ -59,6 +59,8 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the legs that report the path's other kernels and end-to-end decode")
+    ap.add_argument("--only", choices=("other", "decode"), default=None,
+                    help="profiling aid: run just that leg and print its JSON (not the bench line)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="first run a plain 256 MiB device copy three times: the known-size kernel that "
                          "hardware-counter readings of the sweep are scaled by")
@@ -113,6 +115,10 @@ def main():
     load_extension()
     lib = load_capi()
     torch.cuda.set_device(0)
+    if opts.only:
+        leg = other_kernels(torch) if opts.only == "other" else decode_leg(torch)
+        print(json.dumps({opts.only: leg}))
+        return
     if opts.copy_probe:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
         dst = torch.empty_like(src)
