@@ -390,7 +390,6 @@ def decode_leg(torch):
     from transformers import LlamaConfig, LlamaForCausalLM
 
     from llmquant import QuantConfig, oneshot
-    from llmquant.runtime import graphed_generate
 
     torch.manual_seed(0)
     cfg = LlamaConfig(hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, num_attention_heads=32,
@@ -403,28 +402,24 @@ def decode_leg(torch):
             torch.nn.init.normal_(p, 0, 0.02)
     model = model.to(torch.bfloat16).to("cuda:0").eval()
     prompt, new = 512, 256
-    ids = torch.randint(0, cfg.vocab_size, (1, prompt), generator=torch.Generator().manual_seed(1)).to("cuda:0")
+    from llmquant.eval import latency_row, measure_latency, reconcile
 
-    def timed(fn, n):
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        fn(n)
-        torch.cuda.synchronize()
-        return time.perf_counter() - t0
-
-    def measure(fn):
-        timed(fn, 4)
-        first = sorted(timed(fn, 1) for _ in range(3))[1]
-        full = sorted(timed(fn, new) for _ in range(3))[1]
-        return {"ttft_ms": round(first * 1e3, 2), "decode_tok_s": round((new - 1) / max(full - first, 1e-9), 1)}
+    def measure(kv_bits):
+        lat = measure_latency(model, None, prompt_tokens=prompt, new_tokens=new, iters=3, use_cuda_graph=True,
+                              kv_bits=kv_bits)
+        return lat, {"ttft_ms": round(lat["ttft_ms"], 2), "decode_tok_s": round(lat["decode_tps"], 1)}
 
     res = {"prompt_tokens": prompt, "new_tokens": new, "hip_graph": True}
-    res["bf16"] = measure(lambda n: graphed_generate(model, ids, n))
+    lat_bf16, res["bf16"] = measure(None)
     recipe = QuantConfig(attn_weight="int8", mlp_weight="int4", head_weight="int8", kv_cache="int8")
     oneshot(model, recipe.to_modifier("kernel"))
-    res["kernel"] = measure(lambda n: graphed_generate(model, ids, n, kv_bits=8))
+    lat_kernel, res["kernel"] = measure(8)
     res["config"] = recipe.describe()
     res["speedup_vs_bf16"] = round(res["kernel"]["decode_tok_s"] / res["bf16"]["decode_tok_s"], 3)
+    # the same two runs as rows of the reference's report format (eval/run.py, eval/verify.py)
+    rows = [dict(latency_row(None, "kernel", lat_bf16), verify_label="bf16 baseline"),
+            dict(latency_row(recipe, "kernel", lat_kernel), verify_label="selected")]
+    res["verify"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in reconcile(rows).items()}
     del model
     torch.cuda.empty_cache()
     return res

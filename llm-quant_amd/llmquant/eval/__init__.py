@@ -1,0 +1,7 @@
+"""Latency measurement and the measured-versus-projected check, in the reference's row format."""
+
+from llmquant.eval.latency import latency_row, measure_latency
+from llmquant.eval.verify import OUT_OF_KERNEL_AXES, PROJECTION_TOLERANCE, reconcile, verification_plan
+
+__all__ = ["OUT_OF_KERNEL_AXES", "PROJECTION_TOLERANCE", "latency_row", "measure_latency", "reconcile",
+           "verification_plan"]

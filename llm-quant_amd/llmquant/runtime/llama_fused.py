@@ -39,6 +39,8 @@ def _fusable(*mods) -> bool:
             return False
         if m.qdata.shape[1:] != first.qdata.shape[1:] or m.scheme.weights.group_size != 128:
             return False
+        if m.qdata.shape[1] % 4:  # the matrix-core GEMV walks a row four groups at a time
+            return False
     return True
 
 
@@ -60,8 +62,8 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
             attn, mlp = layer.self_attn, layer.mlp
             if not (_fusable(attn.q_proj, attn.k_proj, attn.v_proj) and _fusable(mlp.gate_proj, mlp.up_proj)
                     and _fusable(attn.o_proj) and _fusable(mlp.down_proj)):
-                raise ValueError("the fused decode step needs kernel-mode Linears (group 128, no bias, weight-only) "
-                                 "with q/k/v and gate/up sharing a bit width")
+                raise ValueError("the fused decode step needs kernel-mode Linears (group 128, a multiple of 4 groups per "
+                                 "row, no bias, weight-only) with q/k/v and gate/up sharing a bit width")
             if attn.q_proj.out_group and attn.q_proj.qdata.shape[0] % attn.q_proj.out_group:
                 raise ValueError("q_proj rows are not a whole number of scale tiles")
             args = attn.o_proj.scheme.weights

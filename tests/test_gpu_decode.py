@@ -187,3 +187,20 @@ def test_graphed_generate_api(small):
     dec.capture(16, first)
     assert dec.step().shape == (1, 1) and dec.logits.shape[-1] == 4096
     assert GraphedDecoder(base, 12, 4).max_len == 12 + 4 + 3 + 1
+
+
+def test_measure_latency_reports_the_reference_keys():
+    """llmquant/eval/evaluate.py:167-223 on a small model: graphed HF path for bf16, the fused
+    integer-KV runtime for the kernel-mode model."""
+    from llmquant.eval import measure_latency
+
+    model = build_model(256, 512, 2, 4, 2, 1024)
+    lat = measure_latency(model, None, prompt_tokens=16, new_tokens=8, iters=3, use_cuda_graph=True)
+    assert set(lat) == {"ttft_ms", "decode_tps", "cuda_graph", "peak_vram_gb", "latency_prompt_tokens",
+                        "latency_new_tokens"}
+    assert lat["cuda_graph"] is True and lat["ttft_ms"] > 0 and lat["decode_tps"] > 0
+    _, kernel = quantized_pair(model)
+    fast = measure_latency(kernel, None, prompt_tokens=16, new_tokens=8, iters=3, use_cuda_graph=True, kv_bits=8)
+    assert fast["cuda_graph"] is True and fast["decode_tps"] > 0 and fast["latency_new_tokens"] == 8
+    plain = measure_latency(model, None, prompt_tokens=16, new_tokens=4, iters=1)
+    assert plain["cuda_graph"] is False

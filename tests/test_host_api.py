@@ -313,3 +313,36 @@ def test_fake_quant_cache(bits):
     all_k, _ = cache.update(more, more.clone(), 0)
     assert all_k.shape[2] == 7 and torch.equal(all_k[:, :, :5], kept)  # old tokens are not re-quantized
     assert make_cache_factory(None) is None and isinstance(make_cache_factory(bits)(), FakeQuantCache)
+
+
+def test_verification_plan_and_reconcile_follow_the_report_format():
+    """eval/verify.py: baseline, selected, one ablation per out-of-kernel axis that is quantized;
+    measured speedup, whether the projection held, and what each ablation recovers."""
+    from llmquant import QuantConfig
+    from llmquant.eval import PROJECTION_TOLERANCE, latency_row, reconcile, verification_plan
+
+    quant = QuantConfig(attn_weight="int8", mlp_weight="int4", head_weight="int8", kv_cache="int8")
+    plan = verification_plan(quant)
+    assert [label for label, _ in plan] == ["bf16 baseline", "selected", "selected, kv_cache=bf16"]
+    assert plan[0][1] is None and plan[2][1].kv_cache == "bf16" and plan[2][1].mlp_weight == "int4"
+    both = verification_plan(QuantConfig(), {"attn_weight": "int8", "mlp_weight": "int8", "head_weight": "bf16",
+                                             "activation": "int8", "kv_cache": "int8"})
+    assert [label for label, _ in both][2:] == ["selected, kv_cache=bf16", "selected, activation=bf16"]
+    assert verification_plan(QuantConfig(mlp_weight="int4"))[-1][0] == "selected"
+
+    lat = {"ttft_ms": 8.0, "decode_tps": 250.0, "cuda_graph": True, "peak_vram_gb": 3.0,
+           "latency_prompt_tokens": 512, "latency_new_tokens": 256}
+    base = dict(latency_row(None, "kernel", lat), verify_label="bf16 baseline")
+    assert base["name"] == "bf16" and base["quantize"] is False and base["latency_mode"] == "kernel"
+    assert base["attn_weight"] == "bf16" and base["group_size"] == 128
+    sel = dict(latency_row(quant, "kernel", dict(lat, decode_tps=1000.0, ttft_ms=8.4, peak_vram_gb=1.5)),
+               verify_label="selected", decode_speedup_projected=2.8)
+    assert sel["name"] == "attn-int8_mlp-int4_head-int8_act-bf16_kv-int8_g128" and sel["kv_cache"] == "int8"
+    abl = dict(latency_row(plan[2][1], "kernel", dict(lat, decode_tps=1100.0)), verify_label="selected, kv_cache=bf16")
+    out = reconcile([base, sel, abl])
+    assert out["measured_decode_speedup"] == 4.0 and out["held_up"] is True
+    assert out["ttft_ratio"] == pytest.approx(1.05) and out["vram_ratio"] == 0.5
+    assert out["attribution"] == [{"axis": "kv_cache", "dtype": "int8", "tps_without_it": 1100.0,
+                                   "recovered": 1.1, "costs_decode_pct": pytest.approx(100 / 11)}]
+    assert reconcile([base]) == {}
+    assert reconcile([base, dict(sel, decode_speedup_projected=4.0 / PROJECTION_TOLERANCE + 0.1)])["held_up"] is False
