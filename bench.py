@@ -295,15 +295,32 @@ def other_kernels(torch):
         table = torch.randn(t_max, d, device=dev).to(torch.bfloat16)
         pos = torch.tensor([ctx], dtype=torch.int32, device=dev)
 
-        def step():
+        splits = 8
+        partials = torch.zeros(ext.kv_attend_partials_floats(qh, d, splits), device=dev)
+
+        def one_workgroup_per_head():
             for layer in range(layers):
                 ext.kv_rope_append_attend(qkv, table, table, kc[layer], vc[layer], ks[layer], vs[layer], pos,
                                           d ** -0.5, qh)
 
-        us = _graph_time_us(torch, step, reps=20) / layers
+        def split_only():  # in a decode step the records are merged by o_proj's GEMV, at no launch
+            for layer in range(layers):
+                ext.kv_rope_append_attend_split(qkv, table, table, kc[layer], vc[layer], ks[layer], vs[layer],
+                                                partials, pos, d ** -0.5, qh, splits)
+
+        def split_and_merge():
+            for layer in range(layers):
+                ext.kv_rope_append_attend_split(qkv, table, table, kc[layer], vc[layer], ks[layer], vs[layer],
+                                                partials, pos, d ** -0.5, qh, splits)
+                ext.kv_attend_merge(partials, qh, d, splits, torch.bfloat16)
+
         nbytes = 2 * kvh * (ctx + 1) * width + 2 * kvh * (ctx + 1) * 4
-        out[f"kv_int{bits}_rope_append_attention_ctx2048_per_layer"] = {
-            "us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1)}
+        entry = {"bytes": nbytes, "splits": splits}
+        for name, fn in (("one_workgroup_per_head_us", one_workgroup_per_head), ("split_us", split_only),
+                         ("split_plus_merge_kernel_us", split_and_merge)):
+            entry[name] = round(_graph_time_us(torch, fn, reps=20) / layers, 2)
+        entry["GBps"] = round(nbytes / entry["split_us"] / 1e3, 1)
+        out[f"kv_int{bits}_rope_append_attention_ctx2048_per_layer"] = entry
     # the GEMV on Llama-3-8B's linears (M = 1): random codes, buffers rotated over > 600 MB so that
     # every launch streams from HBM; the launches of one rotation replayed as a HIP graph
     shapes_8b = []

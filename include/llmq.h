@@ -96,7 +96,8 @@ int llmq_wq_gemv_batched(const void* x, const void* qweight, const float* wscale
  *                               128, i.e. pad_activation (llmquant/quantizers/kernel.py:17-25)
  *   residual != NULL            out = dtype(residual + dtype(y))
  * x, norm_weight, residual, out all have element type `dtype`. */
-enum llmq_prologue { LLMQ_PRO_NONE = 0, LLMQ_PRO_RMSNORM = 1, LLMQ_PRO_SILU_MUL = 2 };
+enum llmq_prologue { LLMQ_PRO_NONE = 0, LLMQ_PRO_RMSNORM = 1, LLMQ_PRO_SILU_MUL = 2,
+                     LLMQ_PRO_ATTN_MERGE = 3 /* only through llmq_wq_gemv_attn_merge */ };
 int llmq_wq_gemv_fused(const void* x, const void* qweight, const float* wscale, void* out, int N,
                        int G, int out_group, int wformat, int dtype, int prologue,
                        const void* norm_weight, float eps, int in_head_dim,
@@ -173,6 +174,27 @@ int llmq_kv_rope_append_attend(const void* qkv, const void* cos_table, const voi
                                void* k_codes, void* v_codes, float* k_scale, float* v_scale, void* out,
                                const int32_t* pos_dev, float sm_scale, int q_heads, int kv_heads,
                                int head_dim, int t_max, int bits, int dtype, llmq_stream_t stream);
+
+/* The same decode step with the tokens of every head spread over n_splits workgroups (256 CUs are
+ * filled by 32 heads x 8 splits; one workgroup per head leaves 7/8 of the chip idle and is bound by
+ * the dequantization arithmetic). Instead of the attention output it writes, per (head, split), a
+ * record [max, sum, 0, 0, weighted output[head_dim]] of fp32 (scores in log2 units) into
+ * `partials`, llmq_kv_attend_partials_floats(...) floats, 16-byte aligned. The records are merged
+ * by llmq_kv_attend_merge (out: [q_heads * head_dim] `dtype`), or for free by the GEMV that
+ * consumes the attention output: llmq_wq_gemv_attn_merge is llmq_wq_gemv_fused whose activation is
+ * dtype(merge(partials)) (o_proj of a decoder layer; in_head_dim / residual as there). */
+size_t llmq_kv_attend_partials_floats(int q_heads, int head_dim, int n_splits);
+int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos_table, const void* sin_table,
+                                     void* k_codes, void* v_codes, float* k_scale, float* v_scale,
+                                     float* partials, const int32_t* pos_dev, float sm_scale,
+                                     int q_heads, int kv_heads, int head_dim, int t_max, int bits,
+                                     int n_splits, int dtype, llmq_stream_t stream);
+int llmq_kv_attend_merge(const float* partials, void* out, int q_heads, int head_dim, int n_splits,
+                         int dtype, llmq_stream_t stream);
+int llmq_wq_gemv_attn_merge(const float* partials, int n_splits, int head_dim, const void* qweight,
+                            const float* wscale, void* out, int N, int G, int out_group, int wformat,
+                            int dtype, int in_head_dim, const void* residual_or_null,
+                            llmq_stream_t stream);
 
 /* Index of the first maximum of a row of n elements, written to *out_index on the device: the
  * greedy sampler of the decode loop (the reference calls logits.argmax(-1),

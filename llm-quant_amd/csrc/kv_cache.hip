@@ -499,6 +499,155 @@ __global__ __launch_bounds__(kFusedThreads) void kv_rope_append_attend_kernel(
   }
 }
 
+// ---- the same step spread over more of the chip ------------------------------------------------------
+// One workgroup per (query head, split): split s of S takes the 64-token slabs s, s + S, ... of the
+// cache (balanced at every context length, nothing to compute from the length), the last split
+// also the new token. A workgroup is 4 waves, so with S = 8 a 32-head model fills 256 CUs with one
+// workgroup each and the dequantization work of a head runs on 8 CUs instead of one. What leaves a
+// workgroup is a partial record (max, sum, weighted output relative to that max) per (head, split);
+// the records are merged by whoever consumes the attention output: llmq_kv_attend_merge, or the
+// o_proj GEMV while it stages its activation (llmq_wq_gemv_attn_merge), which costs no launch.
+constexpr int kSplitWaves = 4;
+constexpr int kSplitThreads = kSplitWaves * kWave;
+constexpr int kSplitSlab = kSplitWaves * kTokPerIter;  // 64 tokens per workgroup step
+
+template <typename T, int BITS, int D>
+__global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_kernel(
+    const T* __restrict__ qkv, const T* __restrict__ cos_table, const T* __restrict__ sin_table,
+    uint8_t* __restrict__ k_codes, uint8_t* __restrict__ v_codes, float* __restrict__ k_scale,
+    float* __restrict__ v_scale, float* __restrict__ partials, const int32_t* __restrict__ pos_dev,
+    const float sm_scale_log2, const int q_heads, const int kv_heads, const int t_max) {
+  constexpr int DPL = D / 4;
+  constexpr int ROWB = BITS == 8 ? D : D / 2;
+  constexpr int REC = D + 2;                    // per-wave record in LDS
+  constexpr int GREC = D + kAttnRecordHeader;  // per-split record in global memory
+  __shared__ float s_q[D];
+  __shared__ float s_new[2][D];
+  __shared__ float s_rec[kSplitWaves][REC];
+
+  const int qh = blockIdx.x, split = blockIdx.y, n_splits = gridDim.y;
+  const bool last_split = split == n_splits - 1;
+  const int rep = q_heads / kv_heads;
+  const int kvh = qh / rep;
+  const bool writer = last_split && qh % rep == 0;
+  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+  const int tk = lane >> 2, dq = lane & 3;
+  const int pos = min(max(pos_dev[0], 0), t_max - 1);
+  const T* cos_row = cos_table + static_cast<int64_t>(pos) * D;
+  const T* sin_row = sin_table + static_cast<int64_t>(pos) * D;
+
+  const uint8_t* kbase = k_codes + static_cast<int64_t>(kvh) * t_max * ROWB;
+  const uint8_t* vbase = v_codes + static_cast<int64_t>(kvh) * t_max * ROWB;
+  const float* ksc = k_scale + static_cast<int64_t>(kvh) * t_max;
+  const float* vsc = v_scale + static_cast<int64_t>(kvh) * t_max;
+  const int t_mine = split * kSplitSlab + wv * kTokPerIter;
+  AttnPrefetch<BITS, DPL> first;
+  if (t_mine < pos) first = attn_prefetch<BITS, DPL>(kbase, vbase, ksc, vsc, min(t_mine + tk, pos - 1), dq);
+
+  // ---- phase A: wave 0 rotates the query; in the last split wave 1 / 2 prepare the new K / V ----------
+  if (wv == 0) {
+    const T* q = qkv + static_cast<int64_t>(qh) * D;
+    for (int i = lane; i < D; i += kWave) s_q[i] = rope_element<T, D>(q, cos_row, sin_row, i) * sm_scale_log2;
+  } else if (wv <= 2 && last_split) {
+    const bool is_v = wv == 2;
+    const T* src = qkv + (static_cast<int64_t>(q_heads) + (is_v ? kv_heads : 0) + kvh) * D;
+    const float qmax = static_cast<float>((1 << (BITS - 1)) - 1);
+    const float qmin = -qmax - 1.0f;
+    float f[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int d = lane + e * kWave;
+      f[e] = 0.0f;
+      if (d < D) f[e] = is_v ? to_float(src[d]) : rope_element<T, D>(src, cos_row, sin_row, d);
+    }
+    const float amax = group_max<kWave>(fmaxf(fabsf(f[0]), fabsf(f[1])));
+    const float scale = scale_from_amax(amax, qmax);
+    const int64_t slot = static_cast<int64_t>(kvh) * t_max + pos;
+    if (writer && lane == 0) (is_v ? v_scale : k_scale)[slot] = scale;
+    uint8_t* codes = is_v ? v_codes : k_codes;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int d = lane + e * kWave;
+      const float qv = quant_code(f[e], scale, qmin, qmax);
+      if (d < D) s_new[is_v ? 1 : 0][d] = round_through<T>(qv * scale);
+      const int code = static_cast<int>(qv);
+      if constexpr (BITS == 8) {
+        if (writer && d < D) codes[slot * D + d] = static_cast<uint8_t>(code);
+      } else {
+        const int mine = (code + 8) & 0xf;
+        const int other = __shfl_xor(mine, 1, kWave);
+        if (writer && (lane & 1) == 0 && d < D) codes[slot * (D / 2) + d / 2] = static_cast<uint8_t>(mine | (other << 4));
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- phase B: this split's slabs of tokens 0 .. pos-1, and (last split) token pos from LDS ------------
+  float qf[1][DPL];
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) qf[0][i] = s_q[dq * DPL + i];
+  float m[1], l[1], o[1][DPL];
+  attend_range<T, BITS, D, 1>(qf, kbase, vbase, ksc, vsc, t_mine, pos, n_splits * kSplitSlab, tk, dq, m, l, o,
+                              t_mine < pos ? &first : nullptr);
+  if (last_split && wv == kSplitWaves - 1) {
+    float sc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) sc = fmaf(qf[0][i], s_new[0][dq * DPL + i], sc);
+    sc += __shfl_xor(sc, 1, kWave);
+    sc += __shfl_xor(sc, 2, kWave);
+    const float m_new = fmaxf(m[0], sc);
+    const float corr = m[0] == -INFINITY ? 0.0f : exp2f(m[0] - m_new);
+    const float pnew = exp2f(sc - m_new);
+    l[0] = l[0] * corr + pnew;
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) o[0][i] = fmaf(pnew, s_new[1][dq * DPL + i], o[0][i] * corr);
+    m[0] = m_new;
+  }
+  if (tk == 0) {
+    if (dq == 0) {
+      s_rec[wv][0] = m[0];
+      s_rec[wv][1] = l[0];
+    }
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) s_rec[wv][2 + dq * DPL + i] = o[0][i];
+  }
+  __syncthreads();
+  if (threadIdx.x < D) {
+    const int d = threadIdx.x;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kSplitWaves; ++w) mm = fmaxf(mm, s_rec[w][0]);
+    float ll = 0.0f, oo = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kSplitWaves; ++w) {
+      const float a = s_rec[w][0] == -INFINITY ? 0.0f : exp2f(s_rec[w][0] - mm);
+      ll += s_rec[w][1] * a;
+      oo += s_rec[w][2 + d] * a;
+    }
+    float* rec = partials + (static_cast<int64_t>(qh) * n_splits + split) * GREC;
+    if (d == 0) {
+      rec[0] = mm;
+      rec[1] = ll;
+    }
+    rec[kAttnRecordHeader + d] = oo;
+  }
+}
+
+// out[h, d0 .. d0+7] from the records of head h: one thread per eight elements.
+template <typename T>
+__global__ __launch_bounds__(256) void kv_attend_merge_kernel(const float* __restrict__ partials, T* __restrict__ out,
+                                                              const int total, const int head_dim,
+                                                              const int n_splits) {
+  const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (i >= total) return;
+  const int h = i / head_dim, d0 = i - h * head_dim;
+  float f[8];
+  merge_partials8(partials + static_cast<int64_t>(h) * n_splits * (head_dim + kAttnRecordHeader), n_splits, head_dim,
+                  d0, f);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[i + e] = from_float<T>(f[e]);
+}
+
 // ---- argmax of one row (the greedy sampler of the decode loop) ------------------------------------------
 // First index of the maximum, like torch.argmax on a row without ties broken otherwise.
 template <typename T>
@@ -722,4 +871,73 @@ extern "C" int llmq_argmax_row(const void* x, int n, int64_t* out_index, int dty
     default: return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
   }
   return llmq_host::check_launch("argmax_row_kernel");
+}
+
+extern "C" size_t llmq_kv_attend_partials_floats(int q_heads, int head_dim, int n_splits) {
+  return static_cast<size_t>(q_heads) * n_splits * (head_dim + kAttnRecordHeader);
+}
+
+extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos_table, const void* sin_table,
+                                                void* k_codes, void* v_codes, float* k_scale, float* v_scale,
+                                                float* partials, const int32_t* pos_dev, float sm_scale,
+                                                int q_heads, int kv_heads, int head_dim, int t_max, int bits,
+                                                int n_splits, int dtype, llmq_stream_t stream) {
+  if (bits != 8 && bits != 4) return llmq_host::fail_invalid("KV cache bits must be 8 or 4, got %d", bits);
+  if (head_dim != 64 && head_dim != 128) return llmq_host::fail_invalid("head_dim must be 64 or 128, got %d", head_dim);
+  if (kv_heads <= 0 || q_heads <= 0 || q_heads % kv_heads)
+    return llmq_host::fail_invalid("q_heads %d must be a positive multiple of kv_heads %d", q_heads, kv_heads);
+  if (t_max <= 0) return llmq_host::fail_invalid("t_max must be positive, got %d", t_max);
+  if (n_splits < 1 || n_splits > 256) return llmq_host::fail_invalid("n_splits must be in [1, 256], got %d", n_splits);
+  if (!qkv || !cos_table || !sin_table || !k_codes || !v_codes || !k_scale || !v_scale || !partials || !pos_dev)
+    return llmq_host::fail_invalid("null tensor pointer");
+  if ((reinterpret_cast<uintptr_t>(k_codes) | reinterpret_cast<uintptr_t>(v_codes) |
+       reinterpret_cast<uintptr_t>(partials)) & 15u)
+    return llmq_host::fail_invalid("cache code and record pointers must be 16-byte aligned");
+  const float scale_log2 = sm_scale * 1.4426950408889634f;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(q_heads, n_splits), block(kSplitThreads);
+#define LLMQ_SPLIT(T, B, D)                                                                            \
+  hipLaunchKernelGGL((kv_rope_append_attend_split_kernel<T, B, D>), grid, block, 0, s,                  \
+                     static_cast<const T*>(qkv), static_cast<const T*>(cos_table),                      \
+                     static_cast<const T*>(sin_table), static_cast<uint8_t*>(k_codes),                  \
+                     static_cast<uint8_t*>(v_codes), k_scale, v_scale, partials, pos_dev, scale_log2,   \
+                     q_heads, kv_heads, t_max)
+#define LLMQ_SPLIT_BD(T)                                                                               \
+  if (bits == 8) { if (head_dim == 64) LLMQ_SPLIT(T, 8, 64); else LLMQ_SPLIT(T, 8, 128); }             \
+  else { if (head_dim == 64) LLMQ_SPLIT(T, 4, 64); else LLMQ_SPLIT(T, 4, 128); }                       \
+  break;
+  switch (dtype) {
+    case LLMQ_F32: LLMQ_SPLIT_BD(float)
+    case LLMQ_F16: LLMQ_SPLIT_BD(f16_t)
+    case LLMQ_BF16: LLMQ_SPLIT_BD(bf16_t)
+    default: return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+  }
+#undef LLMQ_SPLIT_BD
+#undef LLMQ_SPLIT
+  return llmq_host::check_launch("kv_rope_append_attend_split_kernel");
+}
+
+extern "C" int llmq_kv_attend_merge(const float* partials, void* out, int q_heads, int head_dim, int n_splits,
+                                    int dtype, llmq_stream_t stream) {
+  if (q_heads < 0 || head_dim <= 0 || head_dim % 8 || n_splits < 1)
+    return llmq_host::fail_invalid("bad sizes q_heads=%d head_dim=%d (a multiple of 8) n_splits=%d", q_heads, head_dim,
+                                   n_splits);
+  const int total = q_heads * head_dim;
+  if (total == 0) return 0;
+  if (!partials || !out) return llmq_host::fail_invalid("null tensor pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((total / 8 + 255) / 256), block(256);
+  switch (dtype) {
+    case LLMQ_F32:
+      hipLaunchKernelGGL((kv_attend_merge_kernel<float>), grid, block, 0, s, partials, static_cast<float*>(out), total, head_dim, n_splits);
+      break;
+    case LLMQ_F16:
+      hipLaunchKernelGGL((kv_attend_merge_kernel<f16_t>), grid, block, 0, s, partials, static_cast<f16_t*>(out), total, head_dim, n_splits);
+      break;
+    case LLMQ_BF16:
+      hipLaunchKernelGGL((kv_attend_merge_kernel<bf16_t>), grid, block, 0, s, partials, static_cast<bf16_t*>(out), total, head_dim, n_splits);
+      break;
+    default: return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+  }
+  return llmq_host::check_launch("kv_attend_merge_kernel");
 }

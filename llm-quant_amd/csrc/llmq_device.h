@@ -144,6 +144,52 @@ __device__ __forceinline__ float quant_code(float v, float scale, float qmin, fl
   return fminf(fmaxf(rintf(v / scale), qmin), qmax);
 }
 
+// Split attention: the records of one query head, n_splits x [max, sum, 0, 0, weighted output[head_dim]]
+// (a four-float header keeps the output 16-byte aligned) with scores in log2 units, merged for the
+// eight output elements d0 .. d0+7: sum_s w_s o_s[d] / sum_s w_s l_s, w_s = 2^(m_s - max m). A split
+// that saw no token has m = -inf and contributes nothing. Records are read eight at a time with
+// all loads issued before any is used (a loop that waits for each record costs a memory round
+// trip per split); further batches rescale the running sums like online softmax.
+constexpr int kAttnRecordHeader = 4;
+__device__ __forceinline__ void merge_partials8(const float* rec, int n_splits, int head_dim, int d0, float* f) {
+  const int stride = head_dim + kAttnRecordHeader;
+  float mm = -INFINITY, ll = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = 0.0f;
+  for (int s0 = 0; s0 < n_splits; s0 += 8) {
+    float m_s[8], l_s[8];
+    u32x4 lo[8], hi[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float* r = rec + min(s0 + j, n_splits - 1) * stride;  // clamped: loaded, then weighted by zero
+      m_s[j] = r[0];
+      l_s[j] = r[1];
+      lo[j] = load16(r + kAttnRecordHeader + d0);
+      hi[j] = load16(r + kAttnRecordHeader + d0 + 4);
+    }
+    float m_new = mm;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (s0 + j < n_splits) m_new = fmaxf(m_new, m_s[j]);
+    }
+    const float corr = mm == -INFINITY ? 0.0f : exp2f(mm - m_new);
+    ll *= corr;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] *= corr;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float a = (s0 + j < n_splits && m_s[j] != -INFINITY) ? exp2f(m_s[j] - m_new) : 0.0f;
+      ll += l_s[j] * a;
+      const uint32_t w[8] = {lo[j].x, lo[j].y, lo[j].z, lo[j].w, hi[j].x, hi[j].y, hi[j].z, hi[j].w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] += __builtin_bit_cast(float, w[e]) * a;
+    }
+    mm = m_new;
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = ll > 0.0f ? f[e] / ll : 0.0f;
+}
+
 }  // namespace llmq
 
 // ---- host-side error plumbing -----------------------------------------------------------------
@@ -160,7 +206,8 @@ int gemv_mfma_launch(const void* x, const void* qw, const float* ws, void* out, 
                      int out_group, int wformat, int dtype, hipStream_t stream);
 int gemv_mfma_launch_fused(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
                            int out_group, int wformat, int dtype, int prologue, const void* norm_weight,
-                           float eps, int in_head_dim, const void* residual, hipStream_t stream);
+                           float eps, int in_head_dim, const void* residual, hipStream_t stream,
+                           int attn_splits = 0, int attn_head_dim = 0);
 // Batched form (a plan of expert / row runs read on the device): see llmq_wq_gemv_batched.
 bool gemv_batched_mfma_supported(const void* x, const void* qw, const float* ws, int G, int gs, int wformat);
 int gemv_batched_mfma_launch(const void* x, const void* qw, const float* ws, void* out, const int32_t* block_expert,

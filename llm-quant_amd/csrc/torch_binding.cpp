@@ -439,6 +439,103 @@ at::Tensor kv_rope_append_attend(const at::Tensor& qkv, const at::Tensor& cos_ta
   return out;
 }
 
+// The split form: fills `partials` (fp32, at least kv_attend_partials_floats(...) elements) and returns it.
+at::Tensor kv_rope_append_attend_split(const at::Tensor& qkv, const at::Tensor& cos_table,
+                                       const at::Tensor& sin_table, at::Tensor& k_codes, at::Tensor& v_codes,
+                                       at::Tensor& k_scale, at::Tensor& v_scale, at::Tensor& partials,
+                                       const at::Tensor& position, double sm_scale, int64_t q_heads,
+                                       int64_t n_splits) {
+  TORCH_CHECK(qkv.is_cuda() && qkv.is_contiguous(), "qkv must be a contiguous CUDA tensor");
+  const int dtype = dtype_code(qkv, "qkv");
+  const CacheGeometry g = cache_geometry(k_codes, k_scale, "key");
+  const CacheGeometry gv = cache_geometry(v_codes, v_scale, "value");
+  TORCH_CHECK(g.kv_heads == gv.kv_heads && g.t_max == gv.t_max && g.head_dim == gv.head_dim && g.bits == gv.bits,
+              "key and value caches differ in geometry");
+  TORCH_CHECK(qkv.numel() == (q_heads + 2 * g.kv_heads) * g.head_dim, "qkv has ", qkv.numel(), " elements, expected ",
+              (q_heads + 2 * g.kv_heads) * g.head_dim);
+  for (const at::Tensor* t : {&cos_table, &sin_table}) {
+    TORCH_CHECK(t->is_cuda() && t->is_contiguous() && t->dim() == 2 && t->size(1) == g.head_dim &&
+                    t->size(0) >= g.t_max && t->scalar_type() == qkv.scalar_type(),
+                "cos/sin tables must be contiguous [>= t_max, head_dim] tensors of qkv's dtype");
+  }
+  check_position(position);
+  TORCH_CHECK(n_splits >= 1 && n_splits <= 256, "n_splits must be in [1, 256], got ", n_splits);
+  const auto need = static_cast<int64_t>(llmq_kv_attend_partials_floats(static_cast<int>(q_heads), g.head_dim,
+                                                                        static_cast<int>(n_splits)));
+  TORCH_CHECK(partials.is_cuda() && partials.is_contiguous() && partials.scalar_type() == at::kFloat &&
+                  partials.numel() >= need,
+              "partials must be a contiguous CUDA float32 tensor of at least ", need, " elements");
+  const c10::OptionalDeviceGuard guard(at::device_of(qkv));
+  check_rc(llmq_kv_rope_append_attend_split(
+               qkv.const_data_ptr(), cos_table.const_data_ptr(), sin_table.const_data_ptr(), k_codes.mutable_data_ptr(),
+               v_codes.mutable_data_ptr(), k_scale.mutable_data_ptr<float>(), v_scale.mutable_data_ptr<float>(),
+               partials.mutable_data_ptr<float>(), position.const_data_ptr<int32_t>(), static_cast<float>(sm_scale),
+               static_cast<int>(q_heads), g.kv_heads, g.head_dim, g.t_max, g.bits, static_cast<int>(n_splits), dtype,
+               current_stream(qkv)),
+           "kv_rope_append_attend_split");
+  return partials;
+}
+
+at::Tensor kv_attend_merge(const at::Tensor& partials, int64_t q_heads, int64_t head_dim, int64_t n_splits,
+                           at::ScalarType out_dtype) {
+  TORCH_CHECK(partials.is_cuda() && partials.is_contiguous() && partials.scalar_type() == at::kFloat,
+              "partials must be a contiguous CUDA float32 tensor");
+  TORCH_CHECK(q_heads >= 0 && head_dim > 0 && n_splits >= 1, "bad sizes");
+  TORCH_CHECK(partials.numel() >= static_cast<int64_t>(llmq_kv_attend_partials_floats(
+                                      static_cast<int>(q_heads), static_cast<int>(head_dim), static_cast<int>(n_splits))),
+              "partials is too small for ", q_heads, " heads x ", n_splits, " splits");
+  auto out = at::empty({1, q_heads * head_dim}, partials.options().dtype(out_dtype));
+  const int dtype = dtype_code(out, "output dtype");
+  const c10::OptionalDeviceGuard guard(at::device_of(partials));
+  check_rc(llmq_kv_attend_merge(partials.const_data_ptr<float>(), out.mutable_data_ptr(), static_cast<int>(q_heads),
+                                static_cast<int>(head_dim), static_cast<int>(n_splits), dtype, current_stream(partials)),
+           "kv_attend_merge");
+  return out;
+}
+
+// The GEMV that consumes split attention: activation = out_dtype(merge(partials)), [q_heads * head_dim].
+at::Tensor wq_gemv_attn_merge(const at::Tensor& partials, int64_t n_splits, int64_t head_dim,
+                              const at::Tensor& qweight, const at::Tensor& wscale, int64_t out_group,
+                              int64_t in_head_dim, const c10::optional<at::Tensor>& residual,
+                              at::ScalarType out_dtype) {
+  TORCH_CHECK(partials.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "all tensors must be CUDA");
+  TORCH_CHECK(partials.is_contiguous() && partials.scalar_type() == at::kFloat, "partials must be contiguous float32");
+  TORCH_CHECK(qweight.dim() == 3 && qweight.is_contiguous(), "qweight must be contiguous [N, groups, group_size]");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 2 && wscale.is_contiguous(),
+              "wscale must be contiguous float32 [scale_rows, groups]");
+  const int64_t N = qweight.size(0), groups = qweight.size(1);
+  const int64_t group_size = packed ? qweight.size(2) * 2 : qweight.size(2);
+  TORCH_CHECK(group_size == 128, "the fused GEMV needs group_size 128, got ", group_size);
+  const int64_t k_real = in_head_dim > 0 ? groups * in_head_dim : groups * group_size;
+  TORCH_CHECK(head_dim > 0 && k_real % head_dim == 0, "input width ", k_real, " is not a whole number of heads of ", head_dim);
+  TORCH_CHECK(n_splits >= 1 && partials.numel() >= static_cast<int64_t>(llmq_kv_attend_partials_floats(
+                                   static_cast<int>(k_real / head_dim), static_cast<int>(head_dim), static_cast<int>(n_splits))),
+              "partials is too small for ", k_real / head_dim, " heads x ", n_splits, " splits");
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  TORCH_CHECK(wscale.size(0) == scale_rows && wscale.size(1) == groups, "wscale must be [", scale_rows, ", ", groups, "]");
+  auto out = at::empty({1, N}, partials.options().dtype(out_dtype));
+  const int dtype = dtype_code(out, "output dtype");
+  const void* res_ptr = nullptr;
+  if (residual.has_value() && residual->defined()) {
+    TORCH_CHECK(residual->is_cuda() && residual->is_contiguous() && residual->numel() == N &&
+                    residual->scalar_type() == out_dtype,
+                "residual must be a contiguous tensor of the output dtype with ", N, " elements");
+    res_ptr = residual->const_data_ptr();
+  }
+  if (N == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(partials));
+  check_rc(llmq_wq_gemv_attn_merge(partials.const_data_ptr<float>(), static_cast<int>(n_splits),
+                                   static_cast<int>(head_dim), qweight.const_data_ptr(),
+                                   wscale.const_data_ptr<float>(), out.mutable_data_ptr(), static_cast<int>(N),
+                                   static_cast<int>(groups), static_cast<int>(out_group),
+                                   packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype, static_cast<int>(in_head_dim),
+                                   res_ptr, current_stream(partials)),
+           "wq_gemv_attn_merge");
+  return out;
+}
+
 // x: one row (any shape, contiguous); returns a [1] int64 tensor with the index of its first maximum.
 at::Tensor argmax_row(const at::Tensor& x) {
   TORCH_CHECK(x.is_cuda() && x.is_contiguous() && x.numel() > 0, "x must be a non-empty contiguous CUDA tensor");
@@ -497,6 +594,22 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("dequant_weight", &dequant_weight,
         "Dense [N, groups*keep_per_group] matrix of a quantized weight (keep_per_group <= 0: whole groups)",
         py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("keep_per_group") = 0,
+        py::arg("out_dtype") = at::kBFloat16);
+  m.def("kv_attend_partials_floats", [](int64_t q_heads, int64_t head_dim, int64_t n_splits) {
+    return static_cast<int64_t>(llmq_kv_attend_partials_floats(static_cast<int>(q_heads), static_cast<int>(head_dim),
+                                                               static_cast<int>(n_splits)));
+  }, py::arg("q_heads"), py::arg("head_dim"), py::arg("n_splits"));
+  m.def("kv_rope_append_attend_split", &kv_rope_append_attend_split,
+        "RoPE + quantize-append + attention spread over n_splits workgroups per head; fills and returns partials",
+        py::arg("qkv"), py::arg("cos_table"), py::arg("sin_table"), py::arg("k_codes"), py::arg("v_codes"),
+        py::arg("k_scale"), py::arg("v_scale"), py::arg("partials"), py::arg("position"), py::arg("sm_scale"),
+        py::arg("q_heads"), py::arg("n_splits"));
+  m.def("kv_attend_merge", &kv_attend_merge, py::arg("partials"), py::arg("q_heads"), py::arg("head_dim"),
+        py::arg("n_splits"), py::arg("out_dtype") = at::kBFloat16);
+  m.def("wq_gemv_attn_merge", &wq_gemv_attn_merge,
+        "GEMV whose activation is the merged split-attention output",
+        py::arg("partials"), py::arg("n_splits"), py::arg("head_dim"), py::arg("qweight"), py::arg("wscale"),
+        py::arg("out_group") = 0, py::arg("in_head_dim") = 0, py::arg("residual") = py::none(),
         py::arg("out_dtype") = at::kBFloat16);
   m.def("abi_version", []() { return llmq_abi_version(); });
 }

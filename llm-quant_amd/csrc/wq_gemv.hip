@@ -433,6 +433,30 @@ extern "C" int llmq_wq_gemv_fused(const void* x, const void* qweight, const floa
                                            static_cast<hipStream_t>(stream));
 }
 
+extern "C" int llmq_wq_gemv_attn_merge(const float* partials, int n_splits, int head_dim, const void* qweight,
+                                       const float* wscale, void* out, int N, int G, int out_group, int wformat,
+                                       int dtype, int in_head_dim, const void* residual_or_null,
+                                       llmq_stream_t stream) {
+  if (N < 0 || G <= 0) return llmq_host::fail_invalid("bad dimension N=%d G=%d", N, G);
+  if (wformat != LLMQ_W_INT8 && wformat != LLMQ_W_INT4_PACKED)
+    return llmq_host::fail_invalid("unsupported weight format %d, expected 8 or 4", wformat);
+  if (n_splits < 1 || n_splits > 256) return llmq_host::fail_invalid("n_splits must be in [1, 256], got %d", n_splits);
+  if (head_dim <= 0 || head_dim % 8) return llmq_host::fail_invalid("head_dim must be a positive multiple of 8, got %d", head_dim);
+  if (in_head_dim < 0 || in_head_dim > 128 || in_head_dim % 8)
+    return llmq_host::fail_invalid("in_head_dim must be a multiple of 8 in [0, 128], got %d", in_head_dim);
+  const int k_real = G * (in_head_dim > 0 ? in_head_dim : 128);
+  if (k_real % head_dim)
+    return llmq_host::fail_invalid("the Linear's input width %d is not a whole number of heads of %d", k_real, head_dim);
+  if (N == 0) return 0;
+  if (!partials || !qweight || !wscale || !out) return llmq_host::fail_invalid("null tensor pointer");
+  if (!llmq_host::gemv_mfma_supported(partials, qweight, wscale, 1, G, 128, wformat))
+    return llmq_host::fail_invalid("the fused GEMV needs group size 128, a multiple of 4 groups "
+                                   "and 16-byte aligned operands");
+  return llmq_host::gemv_mfma_launch_fused(partials, qweight, wscale, out, 1, N, G, out_group, wformat, dtype,
+                                           LLMQ_PRO_ATTN_MERGE, nullptr, 0.0f, in_head_dim, residual_or_null,
+                                           static_cast<hipStream_t>(stream), n_splits, head_dim);
+}
+
 extern "C" int llmq_wq_gemv_batched_max_rows(void) { return 8; }
 
 extern "C" int llmq_wq_gemv_batched(const void* x, const void* qweight, const float* wscale, void* out,

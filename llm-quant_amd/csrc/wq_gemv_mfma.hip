@@ -60,6 +60,8 @@ struct MfmaArgs {
   float eps;
   int in_head_dim;           // > 0: x is [G * in_head_dim]; group g takes head g, zero-padded to 128
   const void* residual;      // [N] or null: out = residual + y, both rounded like the model dtype
+  int attn_splits;           // LLMQ_PRO_ATTN_MERGE: x is the split-attention records, this many per head
+  int attn_head_dim;         // ... of heads this wide
 };
 
 template <typename T> __device__ __forceinline__ void load8(const T* p, float* f) {
@@ -105,6 +107,8 @@ struct Prologue {
   const void* norm_weight;
   float eps;
   int in_head_dim;
+  int attn_splits = 0;
+  int attn_head_dim = 0;
 };
 
 // The activation as integers, whole workgroup, into LDS: per (row m, group g) the digits of
@@ -113,7 +117,9 @@ struct Prologue {
 // Every thread of the block must call it; the caller synchronises afterwards.
 // Only rows m < m_valid are staged; what LDS holds for the others is left as it was, which is
 // harmless because the caller never stores their results (integer products cannot trap).
-template <typename T, int BITS, int M>
+// MERGE compiles in the split-attention merge (LLMQ_PRO_ATTN_MERGE); it needs ~80 more registers
+// while staging, so only the kernels launched for that prologue carry it.
+template <typename T, int BITS, int M, bool MERGE = false>
 __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const int G, const LdsLayout& L,
                                                  int8_t* dig, float* cxs, int* csum, const Prologue pro,
                                                  float* red, const int m_valid = M) {
@@ -160,7 +166,22 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
     const bool real = active && tq * 8 < real_per_group && m < m_valid;
     if (real) {
       const int64_t src = static_cast<int64_t>(m) * k_real + g * real_per_group + tq * 8;
-      if (pro.kind == LLMQ_PRO_RMSNORM && base == 0) {
+      bool merged = false;
+      if constexpr (MERGE) {
+        if (pro.kind == LLMQ_PRO_ATTN_MERGE) {
+          // x holds the partial records of split attention; elements src .. src+7 lie in one head
+          const int hd = pro.attn_head_dim;
+          const int head = static_cast<int>(src) / hd, d0 = static_cast<int>(src) - head * hd;
+          merge_partials8(reinterpret_cast<const float*>(x) +
+                              static_cast<int64_t>(head) * pro.attn_splits * (hd + kAttnRecordHeader),
+                          pro.attn_splits, hd, d0, f);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) f[e] = round_through<T>(f[e]);
+          merged = true;
+        }
+      }
+      if (merged) {
+      } else if (pro.kind == LLMQ_PRO_RMSNORM && base == 0) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) f[e] = x_first[e];
       } else {
@@ -242,7 +263,7 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
 // activation fragments stay in registers for the whole kernel. MULTI == true: longer rows; wave w
 // takes chunks w, w + waves, ... of every row tile and re-reads the fragments of the chunk it is
 // about to multiply from LDS (the read is issued with the weight loads, a chunk ahead).
-template <typename T, int BITS, int M, bool MULTI>
+template <typename T, int BITS, int M, bool MULTI, bool MERGE = false>
 __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* smem, const int first_tile,
                                             const int tile_stride, const int m_valid) {
   const int tid = threadIdx.x;
@@ -317,8 +338,10 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
   int tile = first_tile;
   if (tile < a.n_tiles) issue_loads(tile, wv);  // in flight while the activation is prepared
 
-  stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum,
-                               Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim}, red, m_valid);
+  stage_activation<T, BITS, M, MERGE>(static_cast<const T*>(a.x), G, L, dig, cxs, csum,
+                                      Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits,
+                                               a.attn_head_dim},
+                                      red, m_valid);
   __syncthreads();
   load_fragments(wv);
 
@@ -394,10 +417,10 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
   }
 }
 
-template <typename T, int BITS, int M, int MAXT, bool MULTI>
+template <typename T, int BITS, int M, int MAXT, bool MULTI, bool MERGE = false>
 __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  ksplit_body<T, BITS, M, MULTI>(a, smem, blockIdx.x, gridDim.x, M);
+  ksplit_body<T, BITS, M, MULTI, MERGE>(a, smem, blockIdx.x, gridDim.x, M);
 }
 
 // Many small GEMVs in one launch (the routed experts of a Mixture-of-Experts layer). Plan entry
@@ -515,7 +538,9 @@ __global__ __launch_bounds__(256, 4) void wq_gemv_mfma_fullk_kernel(const MfmaAr
   if (tile < a.n_tiles) issue_weights(row_of(tile), scales_of(tile), 0);
 
   stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum,
-                               Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim}, red);
+                               Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits,
+                                        a.attn_head_dim},
+                               red);
   __syncthreads();
   issue_fragments(0);
 
@@ -566,9 +591,9 @@ constexpr int kFullKMinTiles = 1024;
 constexpr int kLdsDefault = 64 * 1024;   // dynamic LDS a kernel may use without opting in
 constexpr int kLdsMax = 160 * 1024;      // LDS of one gfx950 CU
 
-template <typename T, int BITS, int M, int MAXT, bool MULTI>
+template <typename T, int BITS, int M, int MAXT, bool MULTI, bool MERGE = false>
 int launch_one(const MfmaArgs& a, int wk, int grid, int lds, hipStream_t stream) {
-  auto kernel = wq_gemv_mfma_kernel<T, BITS, M, MAXT, MULTI>;
+  auto kernel = wq_gemv_mfma_kernel<T, BITS, M, MAXT, MULTI, MERGE>;
   if (lds > kLdsDefault) {
     static bool raised = false;  // per instantiation; worst case two threads both set it
     if (!raised) {
@@ -587,6 +612,14 @@ int launch_one(const MfmaArgs& a, int wk, int grid, int lds, hipStream_t stream)
 
 template <typename T, int BITS, int M>
 int launch_m(const MfmaArgs& a, int wk, int grid, int lds, hipStream_t stream) {
+  if constexpr (M == 1) {
+    if (a.prologue == LLMQ_PRO_ATTN_MERGE) {
+      if (wk * kGW < a.G) return launch_one<T, BITS, 1, 512, true, true>(a, wk, grid, lds, stream);
+      if (wk <= 4) return launch_one<T, BITS, 1, 256, false, true>(a, wk, grid, lds, stream);
+      if (wk <= 8) return launch_one<T, BITS, 1, 512, false, true>(a, wk, grid, lds, stream);
+      return launch_one<T, BITS, 1, 1024, false, true>(a, wk, grid, lds, stream);
+    }
+  }
   if (wk * kGW < a.G) return launch_one<T, BITS, M, 512, true>(a, wk, grid, lds, stream);
   if (wk <= 4) return launch_one<T, BITS, M, 256, false>(a, wk, grid, lds, stream);
   if (wk <= 8) return launch_one<T, BITS, M, 512, false>(a, wk, grid, lds, stream);
@@ -610,6 +643,8 @@ struct FusedOps {
   float eps = 0.0f;
   int in_head_dim = 0;
   const void* residual = nullptr;
+  int attn_splits = 0;
+  int attn_head_dim = 0;
 };
 
 template <typename T, int BITS>
@@ -620,11 +655,12 @@ int launch_typed(const void* x, const void* qw, const float* ws, void* out, int 
   a.N = N; a.G = G; a.out_group = out_group;
   a.prologue = ops.prologue; a.norm_weight = ops.norm_weight; a.eps = ops.eps;
   a.in_head_dim = ops.in_head_dim; a.residual = ops.residual;
+  a.attn_splits = ops.attn_splits; a.attn_head_dim = ops.attn_head_dim;
   a.n_tiles = (N + kTileRows - 1) / kTileRows;
   a.row_bytes = G * kGroup * BITS / 8;
   // measured on lm_head (8016 row tiles): the barrier-free kernel wins for int4 (27.7 vs 30.7 us),
   // the K-split one for int8 (46.6 vs 49.9 us)
-  if (M == 1 && BITS == 4 && a.n_tiles >= kFullKMinTiles) {
+  if (M == 1 && BITS == 4 && a.n_tiles >= kFullKMinTiles && a.prologue != LLMQ_PRO_ATTN_MERGE) {
     const LdsLayout L(1, G, 0, BITS == 4);
     auto kernel = wq_gemv_mfma_fullk_kernel<T, BITS>;
     // exactly as many workgroups as are resident at once (the launch bounds hold the kernel to
@@ -686,10 +722,12 @@ int gemv_mfma_launch(const void* x, const void* qw, const float* ws, void* out, 
 
 int gemv_mfma_launch_fused(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
                            int out_group, int wformat, int dtype, int prologue, const void* norm_weight,
-                           float eps, int in_head_dim, const void* residual, hipStream_t stream) {
+                           float eps, int in_head_dim, const void* residual, hipStream_t stream, int attn_splits,
+                           int attn_head_dim) {
   FusedOps ops;
   ops.prologue = prologue; ops.norm_weight = norm_weight; ops.eps = eps;
   ops.in_head_dim = in_head_dim; ops.residual = residual;
+  ops.attn_splits = attn_splits; ops.attn_head_dim = attn_head_dim;
 #define LLMQ_DISPATCH(T)                                                                          \
   (wformat == LLMQ_W_INT8 ? launch_typed<T, 8>(x, qw, ws, out, M, N, G, out_group, ops, stream)   \
                           : launch_typed<T, 4>(x, qw, ws, out, M, N, G, out_group, ops, stream))

@@ -85,6 +85,14 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_wq_gemv_fused.restype = c_int
     lib.llmq_kv_rope_append_attend.argtypes = [c_p] * 9 + [c_f] + [c_int] * 6 + [c_p]
     lib.llmq_kv_rope_append_attend.restype = c_int
+    lib.llmq_kv_attend_partials_floats.argtypes = [c_int] * 3
+    lib.llmq_kv_attend_partials_floats.restype = ctypes.c_size_t
+    lib.llmq_kv_rope_append_attend_split.argtypes = [c_p] * 9 + [c_f] + [c_int] * 7 + [c_p]
+    lib.llmq_kv_rope_append_attend_split.restype = c_int
+    lib.llmq_kv_attend_merge.argtypes = [c_p, c_p] + [c_int] * 4 + [c_p]
+    lib.llmq_kv_attend_merge.restype = c_int
+    lib.llmq_wq_gemv_attn_merge.argtypes = [c_p, c_int, c_int, c_p, c_p, c_p] + [c_int] * 6 + [c_p, c_p]
+    lib.llmq_wq_gemv_attn_merge.restype = c_int
     lib.llmq_argmax_row.argtypes = [c_p, c_int, c_p, c_int, c_p]
     lib.llmq_argmax_row.restype = c_int
     lib.llmq_wq_gemm_a8.argtypes = [c_p] * 6 + [c_int] * 7 + [c_p]

@@ -54,9 +54,18 @@ class _Fused:
 
 
 class LlamaFusedRuntime(LlamaKernelRuntime):
-    def __init__(self, model, max_len: int, kv_bits: int = 8, exact_prefill: bool = False):
+    def __init__(self, model, max_len: int, kv_bits: int = 8, exact_prefill: bool = False, attn_splits=None):
+        """attn_splits: workgroups per query head in the attention launch. None picks enough to put
+        a workgroup on every CU (and more for long caches); 1 keeps each head in one workgroup and
+        hands o_proj a finished attention output instead of partial records."""
         super().__init__(model, max_len, kv_bits, exact_prefill)
         self._ext = load_extension()
+        if attn_splits is None:
+            attn_splits = max(1, min(32, max(256 // max(self.q_heads, 1), (max_len + 2047) // 2048 * 4)))
+        self.attn_splits = int(attn_splits)
+        self._partials = torch.zeros(self._ext.kv_attend_partials_floats(self.q_heads, self.head_dim,
+                                                                         self.attn_splits),
+                                     dtype=torch.float32, device=self.device) if self.attn_splits > 1 else None
         self.fused_layers = []
         for layer in self.layers:
             attn, mlp = layer.self_attn, layer.mlp
@@ -88,11 +97,21 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         for index, f in enumerate(self.fused_layers):
             qkv = ext.wq_gemv_fused(hidden, f["qkv"].qdata, f["qkv"].wscale, f["qkv"].out_group, PRO_RMSNORM,
                                     f["norm1"], f["eps1"], 0, None)
-            ctx = ext.kv_rope_append_attend(qkv, self.cos_table, self.sin_table, cache.k_codes[index],
-                                            cache.v_codes[index], cache.k_scale[index], cache.v_scale[index],
-                                            cache.position, self.scaling, self.q_heads)
-            hidden = ext.wq_gemv_fused(ctx, f["o"].qdata, f["o"].wscale, f["o"].out_group, PRO_NONE, None, 0.0,
-                                       f["o_head_dim"], hidden)
+            if self.attn_splits > 1:
+                # partial records per (head, split), merged by o_proj while it stages its activation
+                ext.kv_rope_append_attend_split(qkv, self.cos_table, self.sin_table, cache.k_codes[index],
+                                                cache.v_codes[index], cache.k_scale[index], cache.v_scale[index],
+                                                self._partials, cache.position, self.scaling, self.q_heads,
+                                                self.attn_splits)
+                hidden = ext.wq_gemv_attn_merge(self._partials, self.attn_splits, self.head_dim, f["o"].qdata,
+                                                f["o"].wscale, f["o"].out_group, f["o_head_dim"], hidden,
+                                                hidden.dtype)
+            else:
+                ctx = ext.kv_rope_append_attend(qkv, self.cos_table, self.sin_table, cache.k_codes[index],
+                                                cache.v_codes[index], cache.k_scale[index], cache.v_scale[index],
+                                                cache.position, self.scaling, self.q_heads)
+                hidden = ext.wq_gemv_fused(ctx, f["o"].qdata, f["o"].wscale, f["o"].out_group, PRO_NONE, None, 0.0,
+                                           f["o_head_dim"], hidden)
             gate_up = ext.wq_gemv_fused(hidden, f["gate_up"].qdata, f["gate_up"].wscale, 0, PRO_RMSNORM,
                                         f["norm2"], f["eps2"], 0, None)
             hidden = ext.wq_gemv_fused(gate_up, f["down"].qdata, f["down"].wscale, 0, PRO_SILU_MUL, None, 0.0, 0,

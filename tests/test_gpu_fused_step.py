@@ -184,3 +184,64 @@ def test_fused_runtime_equals_the_unfused_one():
     seq_g = LlamaFusedRuntime(kernel, 80, 8).generate(ids, 24, use_graph=True)
     seq_e = LlamaFusedRuntime(kernel, 80, 8).generate(ids, 24, use_graph=False)
     assert torch.equal(seq_g, seq_e)
+    # one workgroup per head and several give the same tokens here, and each replays as it runs eagerly
+    one = LlamaFusedRuntime(kernel, 80, 8, attn_splits=1)
+    many = LlamaFusedRuntime(kernel, 80, 8, attn_splits=5)
+    assert fused.attn_splits > 1 and one.attn_splits == 1
+    assert torch.equal(one.generate(ids, 24, use_graph=True), one.generate(ids, 24, use_graph=False))
+    assert torch.equal(many.generate(ids, 24, use_graph=True), seq_g)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("q_heads,kv_heads,d", [(32, 8, 64), (8, 2, 128)])
+@pytest.mark.parametrize("pos,splits", [(0, 8), (5, 8), (63, 2), (64, 3), (700, 8), (2047, 16), (300, 1)])
+def test_split_attention_and_its_merge(ext, bits, q_heads, kv_heads, d, pos, splits):
+    """Tokens of a head spread over `splits` workgroups: the cache ends up identical to the
+    one-workgroup launch, the merged output agrees with it (another summation order), and the GEMV
+    that merges while staging equals merge-then-GEMV bit for bit."""
+    torch.manual_seed(6)
+    t_max = 2048
+    width = d if bits == 8 else d // 2
+    dt = torch.int8 if bits == 8 else torch.uint8
+
+    def fresh():
+        return dict(kc=torch.zeros(kv_heads, t_max, width, dtype=dt, device="cuda"),
+                    vc=torch.zeros(kv_heads, t_max, width, dtype=dt, device="cuda"),
+                    ks=torch.zeros(kv_heads, t_max, device="cuda"), vs=torch.zeros(kv_heads, t_max, device="cuda"))
+
+    a, b = fresh(), fresh()
+    zero = torch.zeros(1, dtype=torch.int32, device="cuda")
+    if pos:
+        past_k = torch.randn(kv_heads, pos, d).to(torch.bfloat16).cuda()
+        past_v = torch.randn(kv_heads, pos, d).to(torch.bfloat16).cuda()
+        for c in (a, b):
+            ext.kv_append(past_k, past_v, c["kc"], c["vc"], c["ks"], c["vs"], zero, False)
+    table = torch.randn(t_max, d).clamp(-1, 1).to(torch.bfloat16).cuda()
+    qkv = torch.randn(1, (q_heads + 2 * kv_heads) * d).to(torch.bfloat16).cuda()
+    position = torch.tensor([pos], dtype=torch.int32, device="cuda")
+    want = ext.kv_rope_append_attend(qkv, table, table, b["kc"], b["vc"], b["ks"], b["vs"], position, d ** -0.5, q_heads)
+    partials = torch.full((ext.kv_attend_partials_floats(q_heads, d, splits),), float("nan"), device="cuda")
+    ext.kv_rope_append_attend_split(qkv, table, table, a["kc"], a["vc"], a["ks"], a["vs"], partials, position,
+                                    d ** -0.5, q_heads, splits)
+    for name in ("kc", "vc", "ks", "vs"):
+        assert torch.equal(a[name], b[name]), name
+    merged = ext.kv_attend_merge(partials, q_heads, d, splits, torch.bfloat16)
+    assert merged.shape == want.shape and torch.isfinite(merged).all()
+    assert rel_l2(to_np(merged), to_np(want)) <= 4e-3
+
+    if q_heads * d % 512 == 0:  # a Linear over the attention output, rows of 4 groups or more
+        n, k = 256, q_heads * d
+        q, s = weights(n, k, bits, head_dim=d if d < 128 else None)
+        res = torch.randn(1, n).to(torch.bfloat16).cuda()
+        in_head_dim = d if d < 128 else 0
+        got = ext.wq_gemv_attn_merge(partials, splits, d, q, s, 0, in_head_dim, res, torch.bfloat16)
+        assert torch.equal(got, ext.wq_gemv_fused(merged, q, s, 0, 0, None, 0.0, in_head_dim, res))
+
+
+def test_split_attention_argument_checks(ext):
+    partials = torch.zeros(16, device="cuda")
+    q, s = weights(64, 512, 8)
+    with pytest.raises(RuntimeError, match="too small"):
+        ext.wq_gemv_attn_merge(partials, 8, 64, q, s, 0, 0, None, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="whole number of heads"):
+        ext.wq_gemv_attn_merge(torch.zeros(4096, device="cuda"), 2, 96, q, s, 0, 0, None, torch.bfloat16)
