@@ -187,6 +187,35 @@ def main():
                        "GBps": round(case["bytes"] / (med * 1e-3) / 1e9, 1),
                        "frac_hbm": round(case["bytes"] / (med * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
 
+    # ---- what a kernel that only reads gets out of this GPU's memory: 1 GiB per launch, rotating over 2 GiB
+    probe = [torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_(0, 255) for _ in range(2)]
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda:0")
+    probe_ms = []
+    for rep in range(12):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        rc = lib.llmq_stream_read_probe(probe[rep % 2].data_ptr(), probe[rep % 2].numel(), sink.data_ptr(), sptr)
+        b.record(stream)
+        torch.cuda.synchronize()
+        if rc:
+            raise RuntimeError(lib.llmq_last_error().decode())
+        if rep >= 2:
+            probe_ms.append(a.elapsed_time(b))
+    read_ceiling = (1 << 30) / (sum(probe_ms) / len(probe_ms) * 1e-3) / 1e9
+    del probe
+
+    # ---- the roofline kernel again, as a decode loop runs it: back-to-back launches replayed from a graph
+    def dominant_burst():
+        here = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)  # the capturing stream
+        for rep in range(12):
+            q, s = dominant["bufs"][rep % len(dominant["bufs"])]
+            rc = lib.llmq_wq_gemv(dominant["x"].data_ptr(), q.data_ptr(), s.data_ptr(), dominant["out"].data_ptr(),
+                                  1, dominant["n"], dominant["k"] // GROUP, GROUP, 0, dominant["bits"], BF16, here)
+            if rc:
+                raise RuntimeError(lib.llmq_last_error().decode())
+
+    dom_graph_us = _graph_time_us(torch, dominant_burst, reps=5) / 12
+
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     achieved = dominant["bytes"] / (dom_avg_ms * 1e-3) / 1e9
     result = {
@@ -211,7 +240,11 @@ def main():
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": LM_HEAD_INT8_TRAFFIC_BYTES,
                      "avg_launch_us": round(dom_avg_ms * 1e3, 2),
                      "median_launch_us": round(dom_ms[len(dom_ms) // 2] * 1e3, 2),
-                     "algorithmic_bytes": dominant["bytes"]},
+                     "algorithmic_bytes": dominant["bytes"],
+                     "graph_replay_launch_us": round(dom_graph_us, 2),
+                     "graph_replay_GBps": round(dominant["bytes"] / dom_graph_us / 1e3, 1),
+                     "box_streaming_read_GBps": round(read_ceiling, 1),
+                     "frac_of_box_streaming_read": round(achieved / read_ceiling, 4)},
         "shapes": shapes,
     }
 
