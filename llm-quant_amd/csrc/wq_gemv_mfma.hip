@@ -587,6 +587,138 @@ __global__ __launch_bounds__(256, 4) void wq_gemv_mfma_fullk_kernel(const MfmaAr
   }
 }
 
+// The same kernel with DEPTH chunks of weights requested ahead instead of one. When a wave has
+// only one or two row tiles (N of a few thousand rows) its time is a chain of memory round trips,
+// one per chunk; with the whole row in flight at once the chain is one round trip long. DEPTH x 16
+// (int4) or DEPTH x 32 (int8) registers hold the operands, so the kernel is built for two waves per
+// SIMD rather than four. The row must be a whole number of DEPTH-chunk rounds.
+template <typename T, int BITS, int DEPTH>
+__global__ __launch_bounds__(256, 2) void wq_gemv_mfma_fullk_deep_kernel(const MfmaArgs a) {
+  constexpr int M = 1;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wv = tid / kWave;
+  const int waves = blockDim.x / kWave;
+  const int G = a.G;
+  const LdsLayout L(M, G, 0, BITS == 4);
+  int8_t* dig = reinterpret_cast<int8_t*>(smem + L.dig_off);
+  float* cxs = reinterpret_cast<float*>(smem + L.cx_off);
+  float* red = reinterpret_cast<float*>(smem + L.red_off);
+  int* csum = reinterpret_cast<int*>(smem + L.csum_off);
+  const int j = lane & 15;
+  const int blk = lane >> 4;
+  const int n_chunks = G / kGW;
+
+  constexpr int kLoads = BITS == 8 ? 2 * kGW : kGW;
+  v4i b[DEPTH][kLoads];
+  float sc[DEPTH][kGW];
+  v4i af[kGW][2];
+  float fs[kGW];
+  int bias[kGW];
+  const int8_t* a_base = dig + min(j >> 2, kDigits - 1) * L.plane + blk * 16;
+  const float digit_weight = blk == 0 ? 1.0f : (blk == 1 ? 256.0f : (blk == 2 ? 65536.0f : 0.0f));
+  const int* csum_row = csum + (blk < kDigits ? blk : 0) * G;
+  auto issue_fragments = [&](int c) {
+#pragma unroll
+    for (int gi = 0; gi < kGW; ++gi) {
+      const int g = c * kGW + gi;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) af[gi][s] = *reinterpret_cast<const v4i*>(a_base + g * kGroup + s * 64);
+      fs[gi] = cxs[g] * digit_weight;
+      if constexpr (BITS == 4) bias[gi] = -8 * csum_row[g];
+    }
+  };
+  auto row_of = [&](int tile) {
+    return a.qw + static_cast<int64_t>(min(tile * kTileRows + j, a.N - 1)) * a.row_bytes;
+  };
+  auto scales_of = [&](int tile) {
+    const int n = min(tile * kTileRows + j, a.N - 1);
+    return a.ws + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * G;
+  };
+// slot D of the operand registers <- chunk C of the row at ROW / its scales at SP
+#define LLMQ_FILL(D, ROW, SP, C)                                                                   \
+  do {                                                                                             \
+    _Pragma("unroll") for (int gi = 0; gi < kGW; ++gi) {                                           \
+      const int g_ = (C) * kGW + gi;                                                               \
+      if constexpr (BITS == 8) {                                                                   \
+        const uint8_t* p_ = (ROW) + g_ * kGroup + blk * 16;                                        \
+        b[D][2 * gi] = *reinterpret_cast<const v4i*>(p_);                                          \
+        b[D][2 * gi + 1] = *reinterpret_cast<const v4i*>(p_ + 64);                                 \
+      } else {                                                                                     \
+        b[D][gi] = *reinterpret_cast<const v4i*>((ROW) + g_ * (kGroup / 2) + blk * 16);            \
+      }                                                                                            \
+    }                                                                                              \
+    const u32x4 s4_ = load16((SP) + (C) * kGW);                                                    \
+    sc[D][0] = __builtin_bit_cast(float, s4_.x); sc[D][1] = __builtin_bit_cast(float, s4_.y);      \
+    sc[D][2] = __builtin_bit_cast(float, s4_.z); sc[D][3] = __builtin_bit_cast(float, s4_.w);      \
+  } while (0)
+
+  const int stride = gridDim.x * waves;
+  int tile = blockIdx.x * waves + wv;
+  if (tile < a.n_tiles) {
+    const uint8_t* row0 = row_of(tile);
+    const float* sp0 = scales_of(tile);
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) LLMQ_FILL(d, row0, sp0, d);
+  }
+
+  stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum,
+                               Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits,
+                                        a.attn_head_dim},
+                               red);
+  __syncthreads();
+  issue_fragments(0);
+
+  T* __restrict__ out = static_cast<T*>(a.out);
+  for (; tile < a.n_tiles; tile += stride) {
+    const uint8_t* row = row_of(tile);
+    const float* sp = scales_of(tile);
+    const bool more = tile + stride < a.n_tiles;
+    const uint8_t* next_row = more ? row_of(tile + stride) : row;
+    const float* next_sp = more ? scales_of(tile + stride) : sp;
+    float acc = 0.0f;
+    for (int c0 = 0; c0 < n_chunks; c0 += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        const int c = c0 + d;
+        v4i r[kGW];
+        float s_now[kGW];
+#pragma unroll
+        for (int gi = 0; gi < kGW; ++gi) {
+          r[gi] = v4i{BITS == 4 ? bias[gi] : 0, 0, 0, 0};
+          s_now[gi] = sc[d][gi] * fs[gi];
+          if constexpr (BITS == 8) {
+            r[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[gi][0], b[d][2 * gi], r[gi], 0, 0, 0);
+            r[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[gi][1], b[d][2 * gi + 1], r[gi], 0, 0, 0);
+          } else {
+            const v4i lo = b[d][gi] & 0x0f0f0f0f;
+            const v4i hi = (b[d][gi] >> 4) & 0x0f0f0f0f;
+            r[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[gi][0], lo, r[gi], 0, 0, 0);
+            r[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[gi][1], hi, r[gi], 0, 0, 0);
+          }
+        }
+        // slot d is free: DEPTH chunks ahead in this row, else the start of the next tile's row
+        const int ahead = c + DEPTH;
+        if (ahead < n_chunks) {
+          LLMQ_FILL(d, row, sp, ahead);
+        } else if (more) {
+          LLMQ_FILL(d, next_row, next_sp, ahead - n_chunks);
+        }
+        issue_fragments(c + 1 == n_chunks ? 0 : c + 1);
+#pragma unroll
+        for (int gi = 0; gi < kGW; ++gi) acc = fmaf(static_cast<float>(r[gi][0]), s_now[gi], acc);
+      }
+    }
+    const float hi = __shfl_down(acc, 32, kWave);
+    const float mid = __shfl_down(acc, 16, kWave);
+    const float total = (hi + mid) + acc;
+    const int nn = tile * kTileRows + j;
+    if (blk == 0 && nn < a.N) out[nn] = finish<T>(total, a.residual, nn);
+  }
+#undef LLMQ_FILL
+}
+
 constexpr int kFullKMinTiles = 1024;
 constexpr int kLdsDefault = 64 * 1024;   // dynamic LDS a kernel may use without opting in
 constexpr int kLdsMax = 160 * 1024;      // LDS of one gfx950 CU
@@ -660,6 +792,19 @@ int launch_typed(const void* x, const void* qw, const float* ws, void* out, int 
   a.row_bytes = G * kGroup * BITS / 8;
   // measured on lm_head (8016 row tiles): the barrier-free kernel wins for int4 (27.7 vs 30.7 us),
   // the K-split one for int8 (46.6 vs 49.9 us)
+  // measured (graph replay): int4 lm_head 28.3 -> 27.2 us, 8B lm_head 55.0 -> 53.0, gate|up 9.5 -> 9.1 with four
+  // chunks ahead; for int8 (two chunks ahead fit) the K-split kernel below stays faster
+  constexpr int kDeep = 4;
+  if (M == 1 && BITS == 4 && a.n_tiles >= kFullKMinTiles && a.prologue != LLMQ_PRO_ATTN_MERGE &&
+      (G / kGW) % kDeep == 0) {
+    const LdsLayout L(1, G, 0, BITS == 4);
+    auto kernel = wq_gemv_mfma_fullk_deep_kernel<T, BITS, kDeep>;
+    constexpr int per_cu = 2;
+    int grid = 256 * per_cu;
+    if (grid * 4 > a.n_tiles) grid = (a.n_tiles + 3) / 4;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), L.part_off, stream, a);
+    return llmq_host::check_launch("wq_gemv_mfma_fullk_deep_kernel");
+  }
   if (M == 1 && BITS == 4 && a.n_tiles >= kFullKMinTiles && a.prologue != LLMQ_PRO_ATTN_MERGE) {
     const LdsLayout L(1, G, 0, BITS == 4);
     auto kernel = wq_gemv_mfma_fullk_kernel<T, BITS>;
