@@ -13,8 +13,9 @@
 // Shape. A workgroup (4 waves) owns a 128 x 128 output tile (64 x 64 when the problem has too
 // few tiles to fill the chip; the text below describes the large one) and walks K one group
 // (128) at a time. Activations [M, K] int8 and weights [N, K(/2)] are staged in LDS, weights unpacked
-// there to signed int8 in natural k order (packed int4: nibble - 8 computed four at a time
-// with a borrow-free byte subtract, even/odd nibbles re-interleaved with v_perm). Each wave
+// there to signed int8 in natural k order (packed int4: 16 x (nibble - 8) by a mask and a sign-bit
+// flip per four codes, the 16 folded into the weight scale; even/odd nibbles re-interleaved with
+// v_perm). Each wave
 // computes a 64 x 64 quadrant as 2 x 2 MFMA tiles of 32 x 32 (A = activations, rows m;
 // B = weights, columns n), 4 k-slabs of 32 per group. The next group's global loads are in
 // flight while the current one is multiplied. After each group the int32 sums go through the
@@ -43,11 +44,6 @@ struct GemmArgs {
   void* out;           // [M, N]
   int M, N, G, out_group;
 };
-
-// four codes (bytes, value + 8 in 0..15) -> four signed bytes (value), no borrow between bytes
-__device__ __forceinline__ uint32_t unbias4(uint32_t u) {
-  return ((u | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
-}
 
 // W: the wave's quadrant is (32 W) x (32 W), the workgroup's tile (64 W) x (64 W). W = 2 is the
 // throughput shape; W = 1 gives four times as many workgroups when the problem is too small to
@@ -112,13 +108,16 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
       if constexpr (BITS == 8) {
         store16(&s_b[buf][(p >> 3) * kRowStride + (p & 7) * 16], rb[i]);
       } else {
-        // 16 packed bytes = 32 codes -> 32 signed bytes in natural k order
+        // 16 packed bytes = 32 codes -> 32 signed bytes in natural k order, each 16 x its code:
+        // a nibble n = code + 8 moved to the top of its byte and its top bit flipped reads, as a
+        // signed byte, 16 (n - 8). The factor 16 leaves the integer sums exact (< 2^26) and is
+        // taken back out of the weight scale, a power of two, so no rounding changes.
         const uint32_t w[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
         uint32_t o[8];
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          const uint32_t lo = unbias4(w[d] & 0x0f0f0f0fu);         // codes k = 8d + {0,2,4,6}
-          const uint32_t hi = unbias4((w[d] >> 4) & 0x0f0f0f0fu);  // codes k = 8d + {1,3,5,7}
+          const uint32_t lo = ((w[d] << 4) & 0xf0f0f0f0u) ^ 0x80808080u;  // codes k = 8d + {0,2,4,6}
+          const uint32_t hi = (w[d] & 0xf0f0f0f0u) ^ 0x80808080u;         // codes k = 8d + {1,3,5,7}
           // bytes (lo0, hi0, lo1, hi1) and (lo2, hi2, lo3, hi3); v_perm selects from {hi:lo}
           o[2 * d] = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
           o[2 * d + 1] = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
@@ -128,7 +127,8 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
         store16(dst + 16, u32x4{o[4], o[5], o[6], o[7]});
       }
     }
-    if (tid < kBM) s_sx[buf][tid] = r_sx; else if (tid < kBM + kBN) s_sw[buf][tid - kBM] = r_sw;
+    if (tid < kBM) s_sx[buf][tid] = r_sx;
+    else if (tid < kBM + kBN) s_sw[buf][tid - kBM] = BITS == 4 ? r_sw * 0.0625f : r_sw;  // see the unpack above
   };
 
   float acc[W][W][16];
@@ -163,8 +163,10 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
     };
     auto multiply = [&](int mi) {
       v16i d = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+      __builtin_amdgcn_s_setprio(3);  // the wave that feeds the matrix core goes first; epilogues fill in
 #pragma unroll
       for (int ks = 0; ks < kGroup / 32; ++ks) d = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[mi][ks], fb[ks], d, 0, 0, 0);
+      __builtin_amdgcn_s_setprio(0);
       return d;
     };
     // result register r of a 32 x 32 tile is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
