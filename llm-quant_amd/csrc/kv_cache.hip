@@ -659,21 +659,26 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const T* __restrict__ 
   constexpr int V = Pack<T>::N;
   const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
   const int n_vec = aligned ? n / V : 0;
-  // 16-byte packets, two in flight per thread; a thread sees its indices in increasing order, so
-  // a strict '>' keeps the first maximum
-  for (int p = threadIdx.x; p < n_vec; p += 2 * blockDim.x) {
-    float f[2][V];
-    const int p2 = p + blockDim.x;
-    Pack<T>::unpack(load16(x + static_cast<int64_t>(p) * V), f[0]);
-    if (p2 < n_vec) Pack<T>::unpack(load16(x + static_cast<int64_t>(p2) * V), f[1]);
+  // 16-byte packets, eight in flight per thread (a row of logits is a few round trips, not a
+  // bandwidth problem); a thread sees its indices in increasing order, so a strict '>' keeps the
+  // first maximum
+  constexpr int kFlight = 8;
+  for (int p0 = threadIdx.x; p0 < n_vec; p0 += kFlight * blockDim.x) {
+    u32x4 raw[kFlight];
 #pragma unroll
-    for (int e = 0; e < V; ++e) {
-      if (f[0][e] > best) { best = f[0][e]; best_i = p * V + e; }
+    for (int u = 0; u < kFlight; ++u) {
+      const int p = p0 + u * blockDim.x;
+      raw[u] = p < n_vec ? load16(x + static_cast<int64_t>(p) * V) : u32x4{0, 0, 0, 0};
     }
-    if (p2 < n_vec) {
+#pragma unroll
+    for (int u = 0; u < kFlight; ++u) {
+      const int p = p0 + u * blockDim.x;
+      if (p >= n_vec) break;
+      float f[V];
+      Pack<T>::unpack(raw[u], f);
 #pragma unroll
       for (int e = 0; e < V; ++e) {
-        if (f[1][e] > best) { best = f[1][e]; best_i = p2 * V + e; }
+        if (f[e] > best) { best = f[e]; best_i = p * V + e; }
       }
     }
   }
