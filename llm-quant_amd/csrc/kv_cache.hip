@@ -66,7 +66,7 @@ __global__ __launch_bounds__(256) void kv_append_kernel(
     } else {
       // pair the even lane's code with its odd neighbour's
       const int mine = (code + 8) & 0xf;
-      const int other = __shfl_xor(mine, 1, kWave);
+      const int other = dpp<kDppXor1>(mine);
       if ((lane & 1) == 0 && d < head_dim) {
         codes[slot * (head_dim / 2) + d / 2] = static_cast<uint8_t>(mine | (other << 4));
       }
@@ -170,7 +170,8 @@ __device__ __forceinline__ AttnPrefetch<BITS, DPL> attn_prefetch(const uint8_t* 
 
 // Online-softmax attention of one wave over tokens t_first, t_first + t_step, ... (16 tokens per
 // step, a quad of lanes per token), followed by the merge of the wave's 16 quads. On return
-// every lane with the same dq holds the wave's (max, sum, weighted output quarter) per head.
+// lanes 0..3 (and every lane with the same dq, up to the order of the additions) hold the wave's
+// (max, sum, weighted output quarter) per head.
 template <typename T, int BITS, int D, int REP>
 __device__ __forceinline__ void attend_range(const float (*qf)[D / 4], const uint8_t* kbase, const uint8_t* vbase,
                                              const float* ksc, const float* vsc, const int t_first,
@@ -221,8 +222,8 @@ __device__ __forceinline__ void attend_range(const float (*qf)[D / 4], const uin
     }
 #pragma unroll
     for (int h = 0; h < REP; ++h) {
-      s[h] += __shfl_xor(s[h], 1, kWave);
-      s[h] += __shfl_xor(s[h], 2, kWave);
+      s[h] += dpp<kDppXor1>(s[h]);  // the four lanes of a token's quad
+      s[h] += dpp<kDppXor2>(s[h]);
     }
     if (ok) {
       float p[REP];
@@ -245,25 +246,30 @@ __device__ __forceinline__ void attend_range(const float (*qf)[D / 4], const uin
     }
   }
 
-  // ---- merge the 16 quads of the wave (lanes with the same dq): xor 4, 8, 16, 32 -------------------
-#pragma unroll
-  for (int off = 4; off < kWave; off <<= 1) {
+  // ---- merge the 16 quads of the wave (lanes with the same dq) ----------------------------------------
+  // Inside a row of 16 lanes: rotate by 4, then by 8 (DPP, no LDS round trip); lane i then holds
+  // quads i, i+4, i+8, i+12 of its row. Across the four rows: xor 16, xor 32.
+  auto merge_with = [&](auto exchange) {
 #pragma unroll
     for (int h = 0; h < REP; ++h) {
-      const float m_o = __shfl_xor(m[h], off, kWave);
-      const float l_o = __shfl_xor(l[h], off, kWave);
+      const float m_o = exchange(m[h]);
+      const float l_o = exchange(l[h]);
       const float m_new = fmaxf(m[h], m_o);
       const float a = m[h] == -INFINITY ? 0.0f : exp2f(m[h] - m_new);
       const float b = m_o == -INFINITY ? 0.0f : exp2f(m_o - m_new);
       l[h] = l[h] * a + l_o * b;
 #pragma unroll
       for (int i = 0; i < DPL; ++i) {
-        const float o_o = __shfl_xor(o[h][i], off, kWave);
+        const float o_o = exchange(o[h][i]);
         o[h][i] = o[h][i] * a + o_o * b;
       }
       m[h] = m_new;
     }
-  }
+  };
+  merge_with([](float v) { return dpp<0x124>(v); });  // row_ror:4
+  merge_with([](float v) { return dpp<0x128>(v); });  // row_ror:8
+  merge_with([](float v) { return __shfl_xor(v, 16, kWave); });
+  merge_with([](float v) { return __shfl_xor(v, 32, kWave); });
 }
 
 template <typename T, int BITS, int D, int REP>
@@ -445,7 +451,7 @@ __global__ __launch_bounds__(kFusedThreads) void kv_rope_append_attend_kernel(
         if (writer && d < D) codes[slot * D + d] = static_cast<uint8_t>(code);
       } else {
         const int mine = (code + 8) & 0xf;
-        const int other = __shfl_xor(mine, 1, kWave);
+        const int other = dpp<kDppXor1>(mine);
         if (writer && (lane & 1) == 0 && d < D) codes[slot * (D / 2) + d / 2] = static_cast<uint8_t>(mine | (other << 4));
       }
     }
@@ -464,8 +470,8 @@ __global__ __launch_bounds__(kFusedThreads) void kv_rope_append_attend_kernel(
     float sc = 0.0f;
 #pragma unroll
     for (int i = 0; i < DPL; ++i) sc = fmaf(qf[0][i], s_new[0][dq * DPL + i], sc);
-    sc += __shfl_xor(sc, 1, kWave);
-    sc += __shfl_xor(sc, 2, kWave);
+    sc += dpp<kDppXor1>(sc);
+    sc += dpp<kDppXor2>(sc);
     const float m_new = fmaxf(m[0], sc);
     const float corr = m[0] == -INFINITY ? 0.0f : exp2f(m[0] - m_new);
     const float pnew = exp2f(sc - m_new);
@@ -575,7 +581,7 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
         if (writer && d < D) codes[slot * D + d] = static_cast<uint8_t>(code);
       } else {
         const int mine = (code + 8) & 0xf;
-        const int other = __shfl_xor(mine, 1, kWave);
+        const int other = dpp<kDppXor1>(mine);
         if (writer && (lane & 1) == 0 && d < D) codes[slot * (D / 2) + d / 2] = static_cast<uint8_t>(mine | (other << 4));
       }
     }
@@ -593,8 +599,8 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
     float sc = 0.0f;
 #pragma unroll
     for (int i = 0; i < DPL; ++i) sc = fmaf(qf[0][i], s_new[0][dq * DPL + i], sc);
-    sc += __shfl_xor(sc, 1, kWave);
-    sc += __shfl_xor(sc, 2, kWave);
+    sc += dpp<kDppXor1>(sc);
+    sc += dpp<kDppXor2>(sc);
     const float m_new = fmaxf(m[0], sc);
     const float corr = m[0] == -INFINITY ? 0.0f : exp2f(m[0] - m_new);
     const float pnew = exp2f(sc - m_new);

@@ -122,16 +122,50 @@ template <> struct Pack<f16_t> {
 };
 
 // ---- wave64 reductions ------------------------------------------------------------------
-// Butterfly over the low `width` lanes of each aligned lane group (width a power of two).
+// Lane exchanges inside a row of 16 lanes are DPP modifiers on an ordinary ALU instruction (a
+// few cycles); __shfl_xor compiles to ds_bpermute, a round trip through the LDS unit of ~100
+// cycles, and a butterfly is a chain of them. Rows are combined through v_readlane.
+constexpr int kDppXor1 = 0xB1;         // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;         // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // lane i <-> 7 - i within each 8
+constexpr int kDppMirror = 0x140;      // lane i <-> 15 - i within each 16
+template <int CTRL> __device__ __forceinline__ float dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+template <int CTRL> __device__ __forceinline__ int dpp(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Maximum over each aligned group of WIDTH lanes (a power of two), in every lane of the group.
+// The mirror steps pair whole sub-groups that already agree, so after log2(WIDTH) steps all agree.
 template <int WIDTH> __device__ __forceinline__ float group_max(float v) {
-#pragma unroll
-  for (int off = WIDTH / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  if constexpr (WIDTH >= 2) v = fmaxf(v, dpp<kDppXor1>(v));
+  if constexpr (WIDTH >= 4) v = fmaxf(v, dpp<kDppXor2>(v));
+  if constexpr (WIDTH >= 8) v = fmaxf(v, dpp<kDppHalfMirror>(v));
+  if constexpr (WIDTH >= 16) v = fmaxf(v, dpp<kDppMirror>(v));
+  if constexpr (WIDTH == 32) {
+    const float lo = fmaxf(lane_value(v, 0), lane_value(v, 16)), hi = fmaxf(lane_value(v, 32), lane_value(v, 48));
+    v = (threadIdx.x & 32) ? hi : lo;
+  }
+  if constexpr (WIDTH == 64) {
+    v = fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
+  }
+  return v;
+}
+// Sum over each row of 16 lanes, in every lane of the row (fixed order).
+template <typename V> __device__ __forceinline__ V row16_sum(V v) {
+  v += dpp<kDppXor1>(v);
+  v += dpp<kDppXor2>(v);
+  v += dpp<kDppHalfMirror>(v);
+  v += dpp<kDppMirror>(v);
   return v;
 }
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-  return v;
+  v = row16_sum(v);
+  return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
 }
 
 // ---- the quantizer, one element ------------------------------------------------------------
@@ -186,8 +220,9 @@ __device__ __forceinline__ void merge_partials8(const float* rec, int n_splits, 
     }
     mm = m_new;
   }
+  const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) f[e] = ll > 0.0f ? f[e] / ll : 0.0f;
+  for (int e = 0; e < 8; ++e) f[e] *= inv;
 }
 
 }  // namespace llmq

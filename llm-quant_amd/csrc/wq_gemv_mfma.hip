@@ -73,12 +73,6 @@ template <typename T> __device__ __forceinline__ void load8(const T* p, float* f
   }
 }
 
-__device__ __forceinline__ int row16_sum(int v) {
-#pragma unroll
-  for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-  return v;
-}
-
 // LDS carve-up, shared by host (size) and device (offsets).
 struct LdsLayout {
   int plane;     // bytes of one digit plane of one activation row
