@@ -789,8 +789,11 @@ int launch_typed(const void* x, const void* qw, const float* ws, void* out, int 
   // measured (graph replay): int4 lm_head 28.3 -> 27.2 us, 8B lm_head 55.0 -> 53.0, gate|up 9.5 -> 9.1 with four
   // chunks ahead; for int8 (two chunks ahead fit) the K-split kernel below stays faster
   constexpr int kDeep = 4;
-  if (M == 1 && BITS == 4 && a.n_tiles >= kFullKMinTiles && a.prologue != LLMQ_PRO_ATTN_MERGE &&
-      (G / kGW) % kDeep == 0) {
+  // (rows so long that the staged activation exceeds the default LDS limit go to the K-split kernel,
+  // whose launch raises the limit)
+  const bool fullk_ok = M == 1 && BITS == 4 && a.n_tiles >= kFullKMinTiles && a.prologue != LLMQ_PRO_ATTN_MERGE &&
+                        LdsLayout(1, G, 0, true).part_off <= kLdsDefault;
+  if (fullk_ok && (G / kGW) % kDeep == 0) {
     const LdsLayout L(1, G, 0, BITS == 4);
     auto kernel = wq_gemv_mfma_fullk_deep_kernel<T, BITS, kDeep>;
     constexpr int per_cu = 2;
@@ -799,7 +802,7 @@ int launch_typed(const void* x, const void* qw, const float* ws, void* out, int 
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), L.part_off, stream, a);
     return llmq_host::check_launch("wq_gemv_mfma_fullk_deep_kernel");
   }
-  if (M == 1 && BITS == 4 && a.n_tiles >= kFullKMinTiles && a.prologue != LLMQ_PRO_ATTN_MERGE) {
+  if (fullk_ok) {
     const LdsLayout L(1, G, 0, BITS == 4);
     auto kernel = wq_gemv_mfma_fullk_kernel<T, BITS>;
     // exactly as many workgroups as are resident at once (the launch bounds hold the kernel to
@@ -894,13 +897,15 @@ int launch_batched(const MfmaArgs& a, const BatchPlan& plan, int n_blocks, hipSt
 #define LLMQ_BATCHED(MAXT, MULTI)                                                                   \
   do {                                                                                              \
     auto kernel = wq_gemv_mfma_batched_kernel<T, BITS, MAXT, MULTI>;                                \
-    if (L.total > kLdsDefault) {                                                                    \
+    static bool raised = false; /* per instantiation; worst case two threads both set it */        \
+    if (L.total > kLdsDefault && !raised) {                                                         \
       const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),             \
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax); \
       if (err != hipSuccess) {                                                                      \
         set_error("raising the LDS limit failed: %s", hipGetErrorString(err));                      \
         return static_cast<int>(err);                                                               \
       }                                                                                             \
+      raised = true;                                                                                \
     }                                                                                               \
     hipLaunchKernelGGL(kernel, grid, block, L.total, stream, a, plan);                              \
   } while (0)

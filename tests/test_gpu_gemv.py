@@ -177,6 +177,25 @@ def test_rows_longer_than_64_groups(bits, M, n, k):
     assert rel_l2(to_np(got), exact) <= 1e-5
 
 
+@pytest.mark.parametrize("bits", [8, 4])
+def test_many_long_rows(bits):
+    """N large enough for the whole-row kernel with rows of 176 groups (22528 values): the staged
+    activation no longer fits the default LDS limit, so the launch has to pick a kernel that raises it."""
+    from llmquant.hip import load_extension
+
+    n, k = 16400, 22528
+    gen = torch.Generator().manual_seed(2)
+    width = GROUP if bits == 8 else GROUP // 2
+    q = torch.randint(0, 255, (n, k // GROUP, width), generator=gen, dtype=torch.uint8)
+    scales = torch.rand(n, k // GROUP, generator=gen) * 0.01 + 1e-3
+    x = torch.randn(1, k, generator=gen)
+    codes = q.view(torch.int8).numpy() if bits == 8 else oracle.unpack_int4(q.numpy())
+    got = load_extension().wq_gemv(x.cuda(), (q.view(torch.int8) if bits == 8 else q).cuda(), scales.cuda(), 0)
+    rows = torch.randint(0, n, (256,), generator=gen)
+    exact = oracle.gemv_float64(to_np(x), codes[rows], to_np(scales[rows]))
+    assert rel_l2(to_np(got[:, rows]), exact) <= 1e-5
+
+
 def test_lm_head_shape_by_linearity():
     """Full-size untied lm_head (128256 x 2048, int8), checked through properties that need
     no CPU GEMV: rows against float64 on a sample, and linearity in x."""
