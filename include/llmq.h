@@ -107,7 +107,7 @@ int llmq_wq_gemv_fused(const void* x, const void* qweight, const float* wscale, 
  * for k < keep_per_group <= gs: the matrix KernelQuantLinear builds per forward when more rows
  * arrive than the GEMV takes (`_dequantized_weight`, llmquant/quantizers/kernel.py:68-79), in one
  * pass. keep_per_group < gs drops the zero padding of head-aligned groups, giving the layer's real
- * input width. out: [N, G*keep_per_group] `dtype`. gs a multiple of 16 (int8) or 32 (packed). */
+ * input width. out: [N, G*keep_per_group] `dtype`. gs a multiple of 8. */
 int llmq_dequant_weight(const void* qweight, const float* wscale, void* out, int N, int G, int gs,
                         int keep_per_group, int out_group, int wformat, int dtype,
                         llmq_stream_t stream);

@@ -102,7 +102,7 @@ class KernelQuantLinear(nn.Module):
         pass (the reference multiplies and casts in PyTorch, kernel.py:68-79). With `real_width`
         and head-aligned groups the zero padding is dropped: [out, in_features]."""
         group_size = self.padded_in_features // self.qdata.shape[1]
-        if group_size % (32 if self._packed else 16) == 0:
+        if group_size % 8 == 0:
             keep = self._head_keep if real_width else 0
             return self._ext.dequant_weight(self.qdata, self.wscale, self.out_group, keep, dtype)
         return (self.qweight * self._broadcast_scale).to(dtype).reshape(self.out_features, -1)

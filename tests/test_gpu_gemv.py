@@ -399,5 +399,7 @@ def test_dequant_weight_is_code_times_scale_rounded_once(bits, dtype):
             real = ext.dequant_weight(q, s, 0, hd, dtype)
             assert real.shape == (n, heads * head_dim)
             assert torch.equal(real.cpu(), want[:, :, :hd].reshape(n, -1))
+            odd = ext.dequant_weight(q, s, 0, 20, dtype)  # not a whole number of 8-value packets
+            assert torch.equal(odd.cpu(), want[:, :, :20].reshape(n, -1))
     with pytest.raises(RuntimeError, match="keep_per_group"):
         ext.dequant_weight(q, s, 32, 200, dtype)
