@@ -200,6 +200,12 @@ int llmq_wq_gemv_attn_merge(const float* partials, int n_splits, int head_dim, c
  * greedy sampler of the decode loop (the reference calls logits.argmax(-1),
  * llmquant/runtime/graph_decode.py:131). */
 int llmq_argmax_row(const void* x, int n, int64_t* out_index, int dtype, llmq_stream_t stream);
+/* The same, plus the bookkeeping the decode loop does after it in three more PyTorch kernels
+ * (llmquant/runtime/graph_decode.py:131-140): when non-NULL, *token = the index (next step's input),
+ * *step64 += 1 (the position fed to the rotary table) and *step32 += 1 (the cache's write position). */
+int llmq_argmax_advance(const void* x, int n, int64_t* out_index, int64_t* token_or_null,
+                        int64_t* step64_or_null, int32_t* step32_or_null, int dtype,
+                        llmq_stream_t stream);
 
 /* Measurement aid (no counterpart in the reference): reads `bytes` of `buffer` once with plain
  * 128-bit loads and nothing else, so that timing it gives the read rate this GPU's memory system

@@ -657,7 +657,9 @@ __global__ __launch_bounds__(256) void kv_attend_merge_kernel(const float* __res
 // ---- argmax of one row (the greedy sampler of the decode loop) ------------------------------------------
 // First index of the maximum, like torch.argmax on a row without ties broken otherwise.
 template <typename T>
-__global__ __launch_bounds__(1024) void argmax_row_kernel(const T* __restrict__ x, const int n, int64_t* __restrict__ out) {
+__global__ __launch_bounds__(1024) void argmax_row_kernel(const T* __restrict__ x, const int n, int64_t* __restrict__ out,
+                                                          int64_t* __restrict__ token, int64_t* __restrict__ step64,
+                                                          int32_t* __restrict__ step32) {
   __shared__ float s_val[16];
   __shared__ int s_idx[16];
   float best = -INFINITY;
@@ -705,7 +707,12 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const T* __restrict__ 
     for (int w = 1; w < static_cast<int>(blockDim.x) / kWave; ++w) {
       if (s_val[w] > best || (s_val[w] == best && s_idx[w] < best_i)) { best = s_val[w]; best_i = s_idx[w]; }
     }
-    out[0] = best_i == 0x7fffffff ? 0 : best_i;
+    const int64_t winner = best_i == 0x7fffffff ? 0 : best_i;
+    out[0] = winner;
+    // the bookkeeping of a greedy decode loop, when asked for: next input token, position counters
+    if (token != nullptr) token[0] = winner;
+    if (step64 != nullptr) step64[0] += 1;
+    if (step32 != nullptr) step32[0] += 1;
   }
 }
 
@@ -871,17 +878,27 @@ extern "C" int llmq_kv_rope_append_attend(const void* qkv, const void* cos_table
   return llmq_host::check_launch("kv_rope_append_attend_kernel");
 }
 
-extern "C" int llmq_argmax_row(const void* x, int n, int64_t* out_index, int dtype, llmq_stream_t stream) {
+extern "C" int llmq_argmax_advance(const void* x, int n, int64_t* out_index, int64_t* token_or_null,
+                                   int64_t* step64_or_null, int32_t* step32_or_null, int dtype,
+                                   llmq_stream_t stream) {
   if (n <= 0) return llmq_host::fail_invalid("argmax of an empty row");
   if (!x || !out_index) return llmq_host::fail_invalid("null tensor pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
+#define LLMQ_ARGMAX(T)                                                                                     \
+  hipLaunchKernelGGL((argmax_row_kernel<T>), dim3(1), dim3(1024), 0, s, static_cast<const T*>(x), n, out_index, \
+                     token_or_null, step64_or_null, step32_or_null)
   switch (dtype) {
-    case LLMQ_F32: hipLaunchKernelGGL((argmax_row_kernel<float>), dim3(1), dim3(1024), 0, s, static_cast<const float*>(x), n, out_index); break;
-    case LLMQ_F16: hipLaunchKernelGGL((argmax_row_kernel<f16_t>), dim3(1), dim3(1024), 0, s, static_cast<const f16_t*>(x), n, out_index); break;
-    case LLMQ_BF16: hipLaunchKernelGGL((argmax_row_kernel<bf16_t>), dim3(1), dim3(1024), 0, s, static_cast<const bf16_t*>(x), n, out_index); break;
+    case LLMQ_F32: LLMQ_ARGMAX(float); break;
+    case LLMQ_F16: LLMQ_ARGMAX(f16_t); break;
+    case LLMQ_BF16: LLMQ_ARGMAX(bf16_t); break;
     default: return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
   }
+#undef LLMQ_ARGMAX
   return llmq_host::check_launch("argmax_row_kernel");
+}
+
+extern "C" int llmq_argmax_row(const void* x, int n, int64_t* out_index, int dtype, llmq_stream_t stream) {
+  return llmq_argmax_advance(x, n, out_index, nullptr, nullptr, nullptr, dtype, stream);
 }
 
 extern "C" size_t llmq_kv_attend_partials_floats(int q_heads, int head_dim, int n_splits) {

@@ -548,6 +548,22 @@ at::Tensor argmax_row(const at::Tensor& x) {
   return out;
 }
 
+// argmax_row plus: token <- index, step64 += 1, step32 += 1 (one-element int64 / int64 / int32 device tensors).
+at::Tensor argmax_advance(const at::Tensor& x, at::Tensor& token, at::Tensor& step64, at::Tensor& step32) {
+  TORCH_CHECK(x.is_cuda() && x.is_contiguous() && x.numel() > 0, "x must be a non-empty contiguous CUDA tensor");
+  TORCH_CHECK(token.is_cuda() && token.scalar_type() == at::kLong && token.numel() == 1, "token must be one int64");
+  TORCH_CHECK(step64.is_cuda() && step64.scalar_type() == at::kLong && step64.numel() == 1, "step64 must be one int64");
+  TORCH_CHECK(step32.is_cuda() && step32.scalar_type() == at::kInt && step32.numel() == 1, "step32 must be one int32");
+  const int dtype = dtype_code(x, "x");
+  auto out = at::empty({1}, x.options().dtype(at::kLong));
+  const c10::OptionalDeviceGuard guard(at::device_of(x));
+  check_rc(llmq_argmax_advance(x.const_data_ptr(), static_cast<int>(x.numel()), out.mutable_data_ptr<int64_t>(),
+                               token.mutable_data_ptr<int64_t>(), step64.mutable_data_ptr<int64_t>(),
+                               step32.mutable_data_ptr<int32_t>(), dtype, current_stream(x)),
+           "argmax_advance");
+  return out;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -611,5 +627,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("partials"), py::arg("n_splits"), py::arg("head_dim"), py::arg("qweight"), py::arg("wscale"),
         py::arg("out_group") = 0, py::arg("in_head_dim") = 0, py::arg("residual") = py::none(),
         py::arg("out_dtype") = at::kBFloat16);
+  m.def("argmax_advance", &argmax_advance, "argmax_row, then token <- index, step64 += 1, step32 += 1",
+        py::arg("x"), py::arg("token"), py::arg("step64"), py::arg("step32"));
   m.def("abi_version", []() { return llmq_abi_version(); });
 }

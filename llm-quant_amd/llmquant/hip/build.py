@@ -97,6 +97,8 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_stream_read_probe.restype = c_int
     lib.llmq_argmax_row.argtypes = [c_p, c_int, c_p, c_int, c_p]
     lib.llmq_argmax_row.restype = c_int
+    lib.llmq_argmax_advance.argtypes = [c_p, c_int, c_p, c_p, c_p, c_p, c_int, c_p]
+    lib.llmq_argmax_advance.restype = c_int
     lib.llmq_wq_gemm_a8.argtypes = [c_p] * 6 + [c_int] * 7 + [c_p]
     lib.llmq_wq_gemm_a8.restype = c_int
     lib.llmq_wq_gemv_batched.argtypes = [c_p] * 7 + [c_int] * 9 + [c_p]

@@ -122,8 +122,6 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
 
     def _step(self):
         logits = self._forward(self.token, None, None, decode=True)
-        nxt = self._ext.argmax_row(logits)
-        self.token.copy_(nxt)
-        self.pos_index.add_(1)
-        self.cache.position.add_(1)
+        # greedy pick, next input token and both position counters in one launch
+        nxt = self._ext.argmax_advance(logits, self.token, self.pos_index, self.cache.position)
         return logits, nxt

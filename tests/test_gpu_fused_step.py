@@ -161,6 +161,17 @@ def test_argmax_row(ext):
     assert ext.argmax_row(x[:, 1:].contiguous()[:, :3000].contiguous()).item() == 16  # misaligned / short rows too
 
 
+def test_argmax_advance_does_the_loop_bookkeeping(ext):
+    x = torch.randn(1, 5000, device="cuda").to(torch.bfloat16)
+    token = torch.zeros(1, dtype=torch.long, device="cuda")
+    step64 = torch.tensor([41], dtype=torch.long, device="cuda")
+    step32 = torch.tensor([41], dtype=torch.int32, device="cuda")
+    for _ in range(2):
+        got = ext.argmax_advance(x, token, step64, step32)
+    want = x.float().argmax().item()
+    assert got.item() == want and token.item() == want and step64.item() == 43 and step32.item() == 43
+
+
 def test_fused_runtime_equals_the_unfused_one():
     """Whole decode steps on a small model: fused and operation-by-operation runtimes give the
     same logits to the bit (hidden 512: the variance reduction happens to agree), the same
