@@ -68,10 +68,24 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
   // B tile int8: same. B tile int4: kBN rows x 64 B = 4 kBN packets: row = p / 4.
   constexpr int kAPackets = kBM * 8 / kThreads;
   constexpr int kBPackets = (BITS == 8 ? kBN * 8 : kBN * 4) / kThreads;
-  u32x4 ra[kAPackets], rb[kBPackets];
-  float r_sx = 0.0f, r_sw = 0.0f;
+  // what a thread holds of one group between its global loads and its LDS stores
+  struct Staged {
+    u32x4 ra[kAPackets], rb[kBPackets];
+    float r_sx, r_sw;
+  };
+  // The small tile has little work per group, so with one group in flight its loop runs at one
+  // memory round trip per iteration: it keeps two register sets and requests a group three
+  // iterations before it is multiplied. The large tile has no registers for that: it requests the
+  // next group at the top of an iteration and moves it to LDS at the bottom.
+  constexpr int kAhead = W == 1 ? 2 : 0;
+  constexpr int kSets = kAhead > 0 ? kAhead : 1;
+  Staged st[kSets];
 
-  auto load_group = [&](int grp) {
+  auto load_group = [&](int grp, Staged& t) {
+    u32x4* ra = t.ra;
+    u32x4* rb = t.rb;
+    float& r_sx = t.r_sx;
+    float& r_sw = t.r_sw;
 #pragma unroll
     for (int i = 0; i < kAPackets; ++i) {
       const int p = tid + kThreads * i;
@@ -96,7 +110,10 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
       r_sw = g.sw[static_cast<int64_t>(g.out_group > 0 ? n / g.out_group : n) * g.G + grp];
     }
   };
-  auto store_group = [&](int buf) {
+  auto store_group = [&](int buf, const Staged& t) {
+    const u32x4* ra = t.ra;
+    const u32x4* rb = t.rb;
+    const float r_sx = t.r_sx, r_sw = t.r_sw;
 #pragma unroll
     for (int i = 0; i < kAPackets; ++i) {
       const int p = tid + kThreads * i;
@@ -139,14 +156,20 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
 
-  load_group(0);
-  store_group(0);
+  load_group(0, st[0]);
+  store_group(0, st[0]);
   __syncthreads();
+#pragma unroll
+  for (int a = 0; a < kAhead; ++a) {
+    if (1 + a < g.G) load_group(1 + a, st[a]);  // st[a] will hold groups 1 + a, 1 + a + kAhead, ...
+  }
 
   const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
-  for (int grp = 0; grp < g.G; ++grp) {
+  // one group: multiply it from LDS buffer grp & 1, move group grp + 1 (in `next`) into the other
+  // buffer, and with kAhead > 0 request group grp + 1 + kAhead into the registers that frees
+  auto iterate = [&](int grp, Staged& next) {
     const int buf = grp & 1;
-    if (grp + 1 < g.G) load_group(grp + 1);  // in flight during the MFMAs below
+    if (kAhead == 0 && grp + 1 < g.G) load_group(grp + 1, next);  // in flight during the MFMAs below
 
     // The four 32 x 32 sub-tiles of the quadrant, one after the other: while the matrix core
     // works on sub-tile t + 1 the vector ALU runs the scale epilogue of sub-tile t.
@@ -203,8 +226,15 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
       scale_in(multiply(0), 0, 0);
     }
 
-    if (grp + 1 < g.G) store_group(buf ^ 1);  // nobody reads that buffer any more: see barrier below
+    if (grp + 1 < g.G) store_group(buf ^ 1, next);  // nobody reads that buffer any more: see barrier below
+    if (kAhead > 0 && grp + 1 + kAhead < g.G) load_group(grp + 1 + kAhead, next);
     __syncthreads();
+  };
+  for (int grp = 0; grp < g.G; grp += kSets) {
+#pragma unroll
+    for (int a = 0; a < kSets; ++a) {
+      if (grp + a < g.G) iterate(grp + a, st[a]);
+    }
   }
 
   T* __restrict__ out = static_cast<T*>(g.out);
