@@ -118,8 +118,12 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
                                                  int8_t* dig, float* cxs, int* csum, const Prologue pro,
                                                  float* red, const int m_valid = M) {
   const int tid = threadIdx.x;
-  const int items = m_valid * G * 16;  // 8 elements each; 16 consecutive items are one group
   const int real_per_group = pro.in_head_dim > 0 ? pro.in_head_dim : kGroup;
+  // Items of 8 elements, 16 consecutive ones to a group. Heads of at most 64 values under int8
+  // weights: the group's upper half is padding that the multiply skips, so 8 items cover a group.
+  const bool compact = BITS == 8 && pro.in_head_dim > 0 && pro.in_head_dim <= kGroup / 2;
+  const int lg = compact ? 3 : 4;
+  const int items = (m_valid * G) << lg;
   const int k_real = G * real_per_group;
 
   // RMSNorm (transformers' LlamaRMSNorm.forward): variance of the whole row in fp32 first
@@ -150,8 +154,8 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
   for (int base = 0; base < items; base += blockDim.x) {
     const int item = base + tid;
     const bool active = item < items;
-    const int tq = item & 15;
-    const int mg = active ? item >> 4 : 0;  // m * G + g
+    const int tq = item & ((1 << lg) - 1);
+    const int mg = active ? item >> lg : 0;  // m * G + g
     const int m = mg / G, g = mg - m * G;
     float f[8];
 #pragma unroll
@@ -206,7 +210,8 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
     float amax = 0.0f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(f[e]));
-    amax = group_max<16>(amax);
+    amax = group_max<8>(amax);
+    if (!compact) amax = fmaxf(amax, dpp<kDppMirror>(amax));
     const int ebits = static_cast<int>((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xffu);
     const int sh = 148 - ebits;  // amax * 2^sh in [2^21, 2^22)
     uint32_t packed[kDigits][2] = {};
@@ -276,9 +281,14 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
   const int j = lane & 15;    // weight row within the tile (B column / D column)
   const int blk = lane >> 4;  // k-block of the operand; digit block of the result
 
+  // Heads of at most 64 values, each padded to a group of its own: the activation's upper half of
+  // every group is zero whatever the weights there hold, so an int8 row's second 64 bytes of a
+  // group are neither read nor multiplied.
+  const bool half_groups = BITS == 8 && a.in_head_dim > 0 && a.in_head_dim <= kGroup / 2;
+
   // ---- weight / scale loads of one chunk of one row tile ------------------------------------
   constexpr int kLoads = BITS == 8 ? 2 * kGW : kGW;
-  v4i b[kLoads];
+  v4i b[kLoads] = {};
   float sc[kGW];
   auto issue_loads = [&](int tile, int chunk) {
     const int g0 = chunk * kGW;
@@ -289,7 +299,7 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
       if constexpr (BITS == 8) {
         const uint8_t* p = row + (g0 + gi) * kGroup + blk * 16;
         b[2 * gi] = *reinterpret_cast<const v4i*>(p);
-        b[2 * gi + 1] = *reinterpret_cast<const v4i*>(p + 64);
+        if (!half_groups) b[2 * gi + 1] = *reinterpret_cast<const v4i*>(p + 64);
       } else {
         b[gi] = *reinterpret_cast<const v4i*>(row + (g0 + gi) * (kGroup / 2) + blk * 16);
       }
@@ -314,7 +324,7 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         afrag[gi][s] = v4i{0, 0, 0, 0};
-        if (q < kDigits && m < M) {
+        if (q < kDigits && m < M && !(s == 1 && half_groups)) {
           afrag[gi][s] = *reinterpret_cast<const v4i*>(dig + (q * M + m) * L.plane + g * kGroup + s * 64 + blk * 16);
         }
       }
@@ -353,7 +363,7 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
         d[gi] = cinit[gi];
         if constexpr (BITS == 8) {
           d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][0], b[2 * gi], d[gi], 0, 0, 0);
-          d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], b[2 * gi + 1], d[gi], 0, 0, 0);
+          if (!half_groups) d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], b[2 * gi + 1], d[gi], 0, 0, 0);
         } else {
           const v4i lo = b[gi] & 0x0f0f0f0f;
           const v4i hi = (b[gi] >> 4) & 0x0f0f0f0f;
