@@ -103,6 +103,18 @@ int llmq_wq_gemv_fused(const void* x, const void* qweight, const float* wscale, 
                        const void* norm_weight, float eps, int in_head_dim,
                        const void* residual_or_null, llmq_stream_t stream);
 
+/* llmq_wq_gemv_fused for the gate|up weight of a gated MLP with the activation folded into the
+ * store: qweight is [2 * intermediate, G, gs] (gate rows, then up rows: transformers' fused
+ * gate_up_proj, or gate_proj over up_proj), out is [intermediate] with
+ *   out[i] = dtype(dtype(silu(dtype(y[i]))) * dtype(y[intermediate + i]))
+ * which is LLMQ_PRO_SILU_MUL applied to the [gate | up] output of the plain GEMV (LlamaMLP), so the
+ * GEMV that follows (down_proj) takes it with no prologue. A row tile multiplies eight gate rows
+ * and their eight up rows; `intermediate` must be a multiple of 8. prologue: LLMQ_PRO_NONE or
+ * LLMQ_PRO_RMSNORM. One scale row per weight row. No counterpart in the reference. */
+int llmq_wq_gemv_gate_up_silu(const void* x, const void* qweight, const float* wscale, void* out,
+                              int intermediate, int G, int wformat, int dtype, int prologue,
+                              const void* norm_weight, float eps, llmq_stream_t stream);
+
 /* The dense form of a quantized weight, out[n, g*keep + k] = (dtype)(code[n,g,k] * wscale[sr(n),g])
  * for k < keep_per_group <= gs: the matrix KernelQuantLinear builds per forward when more rows
  * arrive than the GEMV takes (`_dequantized_weight`, llmquant/quantizers/kernel.py:68-79), in one

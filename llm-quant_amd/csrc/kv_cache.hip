@@ -266,8 +266,8 @@ __device__ __forceinline__ void attend_range(const float (*qf)[D / 4], const uin
       m[h] = m_new;
     }
   };
-  merge_with([](float v) { return dpp<0x124>(v); });  // row_ror:4
-  merge_with([](float v) { return dpp<0x128>(v); });  // row_ror:8
+  merge_with([](float v) { return dpp<kDppRor4>(v); });
+  merge_with([](float v) { return dpp<kDppRor8>(v); });
   merge_with([](float v) { return __shfl_xor(v, 16, kWave); });
   merge_with([](float v) { return __shfl_xor(v, 32, kWave); });
 }

@@ -129,6 +129,8 @@ constexpr int kDppXor1 = 0xB1;         // quad_perm [1,0,3,2]
 constexpr int kDppXor2 = 0x4E;         // quad_perm [2,3,0,1]
 constexpr int kDppHalfMirror = 0x141;  // lane i <-> 7 - i within each 8
 constexpr int kDppMirror = 0x140;      // lane i <-> 15 - i within each 16
+constexpr int kDppRor4 = 0x124;        // lane i <- lane (i + 4) % 16 of its row of 16
+constexpr int kDppRor8 = 0x128;        // lane i <- lane (i + 8) % 16 of its row of 16
 template <int CTRL> __device__ __forceinline__ float dpp(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
@@ -242,7 +244,7 @@ int gemv_mfma_launch(const void* x, const void* qw, const float* ws, void* out, 
 int gemv_mfma_launch_fused(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
                            int out_group, int wformat, int dtype, int prologue, const void* norm_weight,
                            float eps, int in_head_dim, const void* residual, hipStream_t stream,
-                           int attn_splits = 0, int attn_head_dim = 0);
+                           int attn_splits = 0, int attn_head_dim = 0, int pair_half = 0);
 // Batched form (a plan of expert / row runs read on the device): see llmq_wq_gemv_batched.
 bool gemv_batched_mfma_supported(const void* x, const void* qw, const float* ws, int G, int gs, int wformat);
 int gemv_batched_mfma_launch(const void* x, const void* qw, const float* ws, void* out, const int32_t* block_expert,

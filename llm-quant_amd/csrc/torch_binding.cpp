@@ -255,6 +255,42 @@ at::Tensor wq_gemv_fused(const at::Tensor& x, const at::Tensor& qweight, const a
   return out;
 }
 
+// One-row gate|up Linear of a gated MLP with act(gate) * up folded into the store (see
+// llmq_wq_gemv_gate_up_silu). qweight: [2I, groups, group_size], gate rows first; returns [1, I].
+at::Tensor wq_gemv_gate_up_silu(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale,
+                                int64_t prologue, const c10::optional<at::Tensor>& norm_weight, double eps) {
+  TORCH_CHECK(x.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "all tensors must be CUDA");
+  TORCH_CHECK(qweight.dim() == 3 && qweight.is_contiguous(), "qweight must be contiguous [2I, groups, group_size]");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 2 && wscale.is_contiguous(),
+              "wscale must be contiguous float32 [2I, groups]");
+  TORCH_CHECK(x.is_contiguous(), "x must be contiguous");
+  const int dtype = dtype_code(x, "x");
+  const int64_t N = qweight.size(0), groups = qweight.size(1);
+  const int64_t group_size = packed ? qweight.size(2) * 2 : qweight.size(2);
+  TORCH_CHECK(group_size == 128, "the fused GEMV needs group_size 128, got ", group_size);
+  TORCH_CHECK(N % 16 == 0, "gate|up needs an even number of rows with halves that are multiples of 8, got ", N);
+  TORCH_CHECK(x.numel() == groups * group_size, "x has ", x.numel(), " elements, expected ", groups * group_size);
+  TORCH_CHECK(wscale.size(0) == N && wscale.size(1) == groups, "wscale must be [", N, ", ", groups, "]");
+  const void* norm_ptr = nullptr;
+  if (prologue == LLMQ_PRO_RMSNORM) {
+    TORCH_CHECK(norm_weight.has_value() && norm_weight->is_cuda() && norm_weight->is_contiguous() &&
+                    norm_weight->numel() == x.numel() && norm_weight->scalar_type() == x.scalar_type(),
+                "the RMSNorm prologue needs a contiguous weight of x's dtype with ", x.numel(), " elements");
+    norm_ptr = norm_weight->const_data_ptr();
+  }
+  auto out = at::empty({1, N / 2}, x.options());
+  if (N == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(x));
+  check_rc(llmq_wq_gemv_gate_up_silu(x.const_data_ptr(), qweight.const_data_ptr(), wscale.const_data_ptr<float>(),
+                                     out.mutable_data_ptr(), static_cast<int>(N / 2), static_cast<int>(groups),
+                                     packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype, static_cast<int>(prologue),
+                                     norm_ptr, static_cast<float>(eps), current_stream(x)),
+           "wq_gemv_gate_up_silu");
+  return out;
+}
+
 // Integer GEMM: a int8 [M, K], sx fp32 [M, G]; qweight / wscale as for wq_gemv; optional fp32 or
 // half-width bias (converted to fp32 here, as RealQuantLinear adds bias.float()).
 at::Tensor wq_gemm_a8(const at::Tensor& a, const at::Tensor& sx, const at::Tensor& qweight,
@@ -581,6 +617,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("prologue") = 0,
         py::arg("norm_weight") = py::none(), py::arg("eps") = 0.0, py::arg("in_head_dim") = 0,
         py::arg("residual") = py::none());
+  m.def("wq_gemv_gate_up_silu", &wq_gemv_gate_up_silu,
+        "One-row gate|up Linear that stores act(gate) * up, optional RMSNorm prologue",
+        py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("prologue") = 0,
+        py::arg("norm_weight") = py::none(), py::arg("eps") = 0.0);
   m.def("kv_rope_append_attend", &kv_rope_append_attend,
         "RoPE + KV quantize-append + attention for one decode token of one layer, one launch",
         py::arg("qkv"), py::arg("cos_table"), py::arg("sin_table"), py::arg("k_codes"), py::arg("v_codes"),

@@ -457,6 +457,28 @@ extern "C" int llmq_wq_gemv_attn_merge(const float* partials, int n_splits, int 
                                            static_cast<hipStream_t>(stream), n_splits, head_dim);
 }
 
+extern "C" int llmq_wq_gemv_gate_up_silu(const void* x, const void* qweight, const float* wscale, void* out,
+                                        int intermediate, int G, int wformat, int dtype, int prologue,
+                                        const void* norm_weight, float eps, llmq_stream_t stream) {
+  if (intermediate < 0 || G <= 0) return llmq_host::fail_invalid("bad dimension intermediate=%d G=%d", intermediate, G);
+  if (intermediate % 8) return llmq_host::fail_invalid("the intermediate width must be a multiple of 8, got %d", intermediate);
+  if (intermediate > (1 << 29)) return llmq_host::fail_invalid("intermediate width %d is too large", intermediate);
+  if (wformat != LLMQ_W_INT8 && wformat != LLMQ_W_INT4_PACKED)
+    return llmq_host::fail_invalid("unsupported weight format %d, expected 8 or 4", wformat);
+  if (prologue != LLMQ_PRO_NONE && prologue != LLMQ_PRO_RMSNORM)
+    return llmq_host::fail_invalid("the gate|up GEMV takes no prologue or RMSNorm, got %d", prologue);
+  if (prologue == LLMQ_PRO_RMSNORM && norm_weight == nullptr)
+    return llmq_host::fail_invalid("the RMSNorm prologue needs its weight");
+  if (intermediate == 0) return 0;
+  if (!x || !qweight || !wscale || !out) return llmq_host::fail_invalid("null tensor pointer");
+  if (!llmq_host::gemv_mfma_supported(x, qweight, wscale, 1, G, 128, wformat))
+    return llmq_host::fail_invalid("the fused GEMV needs group size 128, a multiple of 4 groups "
+                                   "and 16-byte aligned operands");
+  return llmq_host::gemv_mfma_launch_fused(x, qweight, wscale, out, 1, 2 * intermediate, G, 0, wformat, dtype,
+                                           prologue, norm_weight, eps, 0, nullptr,
+                                           static_cast<hipStream_t>(stream), 0, 0, intermediate);
+}
+
 extern "C" int llmq_wq_gemv_batched_max_rows(void) { return 8; }
 
 extern "C" int llmq_wq_gemv_batched(const void* x, const void* qweight, const float* wscale, void* out,

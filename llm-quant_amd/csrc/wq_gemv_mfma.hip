@@ -60,6 +60,10 @@ struct MfmaArgs {
   float eps;
   int in_head_dim;           // > 0: x is [G * in_head_dim]; group g takes head g, zero-padded to 128
   const void* residual;      // [N] or null: out = residual + y, both rounded like the model dtype
+  // > 0: the weight is gate rows [0, pair_half) over up rows [pair_half, 2 * pair_half); a row tile
+  // is eight gate rows and the eight up rows that go with them, n_tiles = pair_half / 8, and out is
+  // [pair_half]: act(gate) * up as the SiLU prologue would compute it from the two outputs
+  int pair_half;
   int attn_splits;           // LLMQ_PRO_ATTN_MERGE: x is the split-attention records, this many per head
   int attn_head_dim;         // ... of heads this wide
 };
@@ -94,6 +98,32 @@ __device__ __forceinline__ T finish(float total, const void* residual, int64_t n
   if (residual == nullptr) return from_float<T>(total);
   // hidden = residual + linear(x): the Linear's output is rounded to the model dtype first
   return from_float<T>(to_float(static_cast<const T*>(residual)[n]) + round_through<T>(total));
+}
+
+// Weight row that lane j (0..15) of a row tile multiplies; rows past the end are clamped (loaded,
+// never stored).
+__device__ __forceinline__ int tile_row(const MfmaArgs& a, int tile, int j) {
+  if (a.pair_half > 0) return tile * 8 + (j & 7) + (j >= 8 ? a.pair_half : 0);
+  return min(tile * kTileRows + j, a.N - 1);
+}
+
+// Stores row j's result of a tile. Every lane of a 16-lane row must call it (the paired form moves
+// data between lanes); `owner` marks the lanes whose `total` is the finished sum.
+template <typename T>
+__device__ __forceinline__ void store_row(const MfmaArgs& a, T* __restrict__ out, int tile, int j, float total,
+                                          bool owner) {
+  if (a.pair_half > 0) {
+    const float up = dpp<kDppRor8>(total);  // lane j < 8 <- lane j + 8: the up row of gate row j
+    if (owner && j < 8) {
+      // exactly the SiLU prologue on the two rounded outputs
+      const float g = round_through<T>(total), u = round_through<T>(up);
+      const float silu = g / (1.0f + expf(-g));
+      out[tile * 8 + j] = from_float<T>(round_through<T>(silu) * u);
+    }
+    return;
+  }
+  const int n = tile * kTileRows + j;
+  if (owner && n < a.N) out[n] = finish<T>(total, a.residual, n);
 }
 
 struct Prologue {
@@ -292,7 +322,7 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
   float sc[kGW];
   auto issue_loads = [&](int tile, int chunk) {
     const int g0 = chunk * kGW;
-    const int n = min(tile * kTileRows + j, a.N - 1);  // rows past the end: loaded, not stored
+    const int n = tile_row(a, tile, j);
     const uint8_t* row = a.qw + static_cast<int64_t>(n) * a.row_bytes;
 #pragma unroll
     for (int gi = 0; gi < kGW; ++gi) {
@@ -411,9 +441,13 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
         }
         total += __shfl_xor(total, 16, kWave);
         total += __shfl_xor(total, 32, kWave);
-        const int n = tile * kTileRows + jj;
-        if (ws == 0 && n < a.N && r < m_valid) {
-          out[static_cast<int64_t>(r) * a.N + n] = finish<T>(total, a.residual, n);
+        if constexpr (M == 1) {
+          store_row<T>(a, out, tile, jj, total, ws == 0);
+        } else {
+          const int n = tile * kTileRows + jj;
+          if (ws == 0 && n < a.N && r < m_valid) {
+            out[static_cast<int64_t>(r) * a.N + n] = finish<T>(total, a.residual, n);
+          }
         }
       }
     }
@@ -530,10 +564,10 @@ __global__ __launch_bounds__(256, 4) void wq_gemv_mfma_fullk_kernel(const MfmaAr
     }
   };
   auto row_of = [&](int tile) {
-    return a.qw + static_cast<int64_t>(min(tile * kTileRows + j, a.N - 1)) * a.row_bytes;
+    return a.qw + static_cast<int64_t>(tile_row(a, tile, j)) * a.row_bytes;
   };
   auto scales_of = [&](int tile) {
-    const int n = min(tile * kTileRows + j, a.N - 1);
+    const int n = tile_row(a, tile, j);
     return a.ws + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * G;
   };
 
@@ -586,8 +620,7 @@ __global__ __launch_bounds__(256, 4) void wq_gemv_mfma_fullk_kernel(const MfmaAr
     const float hi = __shfl_down(acc, 32, kWave);
     const float mid = __shfl_down(acc, 16, kWave);
     const float total = (hi + mid) + acc;
-    const int nn = tile * kTileRows + j;
-    if (blk == 0 && nn < a.N) out[nn] = finish<T>(total, a.residual, nn);
+    store_row<T>(a, out, tile, j, total, blk == 0);
   }
 }
 
@@ -634,10 +667,10 @@ __global__ __launch_bounds__(256, 2) void wq_gemv_mfma_fullk_deep_kernel(const M
     }
   };
   auto row_of = [&](int tile) {
-    return a.qw + static_cast<int64_t>(min(tile * kTileRows + j, a.N - 1)) * a.row_bytes;
+    return a.qw + static_cast<int64_t>(tile_row(a, tile, j)) * a.row_bytes;
   };
   auto scales_of = [&](int tile) {
-    const int n = min(tile * kTileRows + j, a.N - 1);
+    const int n = tile_row(a, tile, j);
     return a.ws + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * G;
   };
 // slot D of the operand registers <- chunk C of the row at ROW / its scales at SP
@@ -717,8 +750,7 @@ __global__ __launch_bounds__(256, 2) void wq_gemv_mfma_fullk_deep_kernel(const M
     const float hi = __shfl_down(acc, 32, kWave);
     const float mid = __shfl_down(acc, 16, kWave);
     const float total = (hi + mid) + acc;
-    const int nn = tile * kTileRows + j;
-    if (blk == 0 && nn < a.N) out[nn] = finish<T>(total, a.residual, nn);
+    store_row<T>(a, out, tile, j, total, blk == 0);
   }
 #undef LLMQ_FILL
 }
@@ -781,6 +813,7 @@ struct FusedOps {
   const void* residual = nullptr;
   int attn_splits = 0;
   int attn_head_dim = 0;
+  int pair_half = 0;
 };
 
 template <typename T, int BITS>
@@ -792,6 +825,8 @@ int launch_typed(const void* x, const void* qw, const float* ws, void* out, int 
   a.prologue = ops.prologue; a.norm_weight = ops.norm_weight; a.eps = ops.eps;
   a.in_head_dim = ops.in_head_dim; a.residual = ops.residual;
   a.attn_splits = ops.attn_splits; a.attn_head_dim = ops.attn_head_dim;
+  a.pair_half = ops.pair_half;
+  // (paired: N = 2 * pair_half weight rows, eight gate + eight up rows to a tile, the same count)
   a.n_tiles = (N + kTileRows - 1) / kTileRows;
   a.row_bytes = G * kGroup * BITS / 8;
   // measured on lm_head (8016 row tiles): the barrier-free kernel wins for int4 (27.7 vs 30.7 us),
@@ -875,8 +910,9 @@ int gemv_mfma_launch(const void* x, const void* qw, const float* ws, void* out, 
 int gemv_mfma_launch_fused(const void* x, const void* qw, const float* ws, void* out, int M, int N, int G,
                            int out_group, int wformat, int dtype, int prologue, const void* norm_weight,
                            float eps, int in_head_dim, const void* residual, hipStream_t stream, int attn_splits,
-                           int attn_head_dim) {
+                           int attn_head_dim, int pair_half) {
   FusedOps ops;
+  ops.pair_half = pair_half;
   ops.prologue = prologue; ops.norm_weight = norm_weight; ops.eps = eps;
   ops.in_head_dim = in_head_dim; ops.residual = residual;
   ops.attn_splits = attn_splits; ops.attn_head_dim = attn_head_dim;

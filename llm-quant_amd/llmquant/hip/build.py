@@ -83,6 +83,8 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_kv_decode_attention.argtypes = [c_p] * 8 + [c_f] + [c_int] * 6 + [c_p]
     lib.llmq_wq_gemv_fused.argtypes = [c_p] * 4 + [c_int] * 6 + [c_p, c_f, c_int, c_p, c_p]
     lib.llmq_wq_gemv_fused.restype = c_int
+    lib.llmq_wq_gemv_gate_up_silu.argtypes = [c_p] * 4 + [c_int] * 5 + [c_p, c_f, c_p]
+    lib.llmq_wq_gemv_gate_up_silu.restype = c_int
     lib.llmq_kv_rope_append_attend.argtypes = [c_p] * 9 + [c_f] + [c_int] * 6 + [c_p]
     lib.llmq_kv_rope_append_attend.restype = c_int
     lib.llmq_kv_attend_partials_floats.argtypes = [c_int] * 3

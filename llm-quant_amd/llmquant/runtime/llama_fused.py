@@ -80,6 +80,8 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
                 qkv=_Fused(attn.q_proj, attn.k_proj, attn.v_proj), gate_up=_Fused(mlp.gate_proj, mlp.up_proj),
                 o=attn.o_proj, down=mlp.down_proj,
                 o_head_dim=args.head_dim if attn.o_proj._needs_padding else 0,
+                # act(gate) * up inside the gate|up launch: a row tile there is eight gate rows and their up rows
+                act_in_gate_up=mlp.gate_proj.qdata.shape[0] % 8 == 0,
                 norm1=layer.input_layernorm.weight.detach().contiguous(), eps1=layer.input_layernorm.variance_epsilon,
                 norm2=layer.post_attention_layernorm.weight.detach().contiguous(),
                 eps2=layer.post_attention_layernorm.variance_epsilon))
@@ -112,10 +114,15 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
                                                 cache.position, self.scaling, self.q_heads)
                 hidden = ext.wq_gemv_fused(ctx, f["o"].qdata, f["o"].wscale, f["o"].out_group, PRO_NONE, None, 0.0,
                                            f["o_head_dim"], hidden)
-            gate_up = ext.wq_gemv_fused(hidden, f["gate_up"].qdata, f["gate_up"].wscale, 0, PRO_RMSNORM,
-                                        f["norm2"], f["eps2"], 0, None)
-            hidden = ext.wq_gemv_fused(gate_up, f["down"].qdata, f["down"].wscale, 0, PRO_SILU_MUL, None, 0.0, 0,
-                                       hidden)
+            if f["act_in_gate_up"]:
+                act = ext.wq_gemv_gate_up_silu(hidden, f["gate_up"].qdata, f["gate_up"].wscale, PRO_RMSNORM,
+                                               f["norm2"], f["eps2"])
+                hidden = ext.wq_gemv_fused(act, f["down"].qdata, f["down"].wscale, 0, PRO_NONE, None, 0.0, 0, hidden)
+            else:
+                gate_up = ext.wq_gemv_fused(hidden, f["gate_up"].qdata, f["gate_up"].wscale, 0, PRO_RMSNORM,
+                                            f["norm2"], f["eps2"], 0, None)
+                hidden = ext.wq_gemv_fused(gate_up, f["down"].qdata, f["down"].wscale, 0, PRO_SILU_MUL, None, 0.0,
+                                           0, hidden)
         head = self.model.lm_head
         return ext.wq_gemv_fused(hidden, head.qdata, head.wscale, head.out_group, PRO_RMSNORM, self.final_norm,
                                  self.final_eps, 0, None)

@@ -64,6 +64,36 @@ def test_silu_mul_prologue_and_residual(ext, bits):
 
 
 @pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("inter,k", [(8192, 2048), (14336, 4096), (264, 512), (2056, 9216)])
+@pytest.mark.parametrize("prologue", [0, 1])
+def test_gate_up_silu_epilogue(ext, bits, inter, k, prologue):
+    """gate|up GEMV that stores act(gate) * up == the plain GEMV followed by LlamaMLP's elementwise step.
+    (8192, 2048) / (14336, 4096): the whole-row int4 kernels; 264: two tiles past a multiple of 16 rows;
+    (2056, 9216): rows of 72 groups, the multi-chunk K-split kernel."""
+    q, s = weights(2 * inter, k, bits, seed=5)
+    torch.manual_seed(6)
+    x = (torch.randn(1, k) * 2).to(torch.bfloat16).cuda()
+    norm = (1 + 0.1 * torch.randn(k)).to(torch.bfloat16).cuda() if prologue else None
+    got = ext.wq_gemv_gate_up_silu(x, q, s, prologue, norm, 1e-5)
+    plain = ext.wq_gemv_fused(x, q, s, 0, prologue, norm, 1e-5, 0, None)
+    want = torch.nn.functional.silu(plain[:, :inter]) * plain[:, inter:]
+    assert got.shape == (1, inter)
+    assert torch.equal(got, want)
+
+
+def test_gate_up_silu_argument_checks(ext):
+    q, s = weights(48, 512, 8)
+    x = torch.randn(1, 512).to(torch.bfloat16).cuda()
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        ext.wq_gemv_gate_up_silu(x, q[:40].contiguous(), s[:40].contiguous(), 0, None, 0.0)
+    with pytest.raises(RuntimeError, match="no prologue or RMSNorm"):
+        ext.wq_gemv_gate_up_silu(x, q, s, 2, None, 0.0)
+    with pytest.raises(RuntimeError, match="RMSNorm prologue needs"):
+        ext.wq_gemv_gate_up_silu(x, q, s, 1, None, 0.0)
+    assert ext.wq_gemv_gate_up_silu(x, q, s, 0, None, 0.0).shape == (1, 24)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
 def test_head_padding_and_residual(ext, bits):
     """o_proj: 32 heads of 64 in groups of 128 (pad_activation), one scale group per head."""
     from llmquant.core.scheme import QuantizationArgs
