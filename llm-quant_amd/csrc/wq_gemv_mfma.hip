@@ -143,35 +143,83 @@ struct Prologue {
 // harmless because the caller never stores their results (integer products cannot trap).
 // MERGE compiles in the split-attention merge (LLMQ_PRO_ATTN_MERGE); it needs ~80 more registers
 // while staging, so only the kernels launched for that prologue carry it.
+// How the activation is cut into items of 8 elements, 16 consecutive ones to a group. Heads of at
+// most 64 values under int8 weights: the group's upper half is padding that the multiply skips, so
+// 8 items cover a group.
+template <int BITS> struct StageGeometry {
+  int real_per_group, lg, items, k_real;
+  __device__ __forceinline__ StageGeometry(int G, const Prologue& pro, int m_valid) {
+    real_per_group = pro.in_head_dim > 0 ? pro.in_head_dim : kGroup;
+    const bool compact = BITS == 8 && pro.in_head_dim > 0 && pro.in_head_dim <= kGroup / 2;
+    lg = compact ? 3 : 4;
+    items = (m_valid * G) << lg;
+    k_real = G * real_per_group;
+  }
+};
+template <int M> struct StageItem {
+  bool active, real;
+  int tq, mg, m, g;
+  int64_t src;  // first of the item's 8 elements in x
+  template <int BITS>
+  __device__ __forceinline__ StageItem(const StageGeometry<BITS>& geo, int item, int G, int m_valid) {
+    active = item < geo.items;
+    tq = item & ((1 << geo.lg) - 1);
+    mg = active ? item >> geo.lg : 0;  // m * G + g
+    m = M == 1 ? 0 : mg / G;
+    g = mg - m * G;
+    // beyond real_per_group: the zero padding of a head group
+    real = active && tq * 8 < geo.real_per_group && m < m_valid;
+    src = static_cast<int64_t>(m) * geo.k_real + g * geo.real_per_group + tq * 8;
+  }
+};
+
+// What a thread's first item reads from memory, requested at the very top of a kernel: the
+// activation heads the kernel's longest dependency chain (load -> digits -> LDS -> barrier ->
+// operand fragments -> multiply), while the weight loads that are issued next have slack.
+struct StageFirst {
+  float x[8];  // the item's elements (the gate half under LLMQ_PRO_SILU_MUL)
+  float w[8];  // RMSNorm weights, or the up half
+};
+template <typename T, int BITS, int M>
+__device__ __forceinline__ StageFirst stage_first(const T* __restrict__ x, const int G, const Prologue& pro,
+                                                  const int m_valid = M) {
+  StageFirst r;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) r.x[e] = r.w[e] = 0.0f;
+  if (pro.kind == LLMQ_PRO_ATTN_MERGE) return r;  // its records are read where they are merged
+  const StageGeometry<BITS> geo(G, pro, m_valid);
+  const StageItem<M> it(geo, threadIdx.x, G, m_valid);
+  if (it.real) {
+    load8<T>(x + it.src, r.x);
+    if (pro.kind == LLMQ_PRO_RMSNORM) load8<T>(static_cast<const T*>(pro.norm_weight) + it.src, r.w);
+    if (pro.kind == LLMQ_PRO_SILU_MUL) load8<T>(x + geo.k_real + it.src, r.w);
+  }
+  return r;
+}
+
 template <typename T, int BITS, int M, bool MERGE = false>
 __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const int G, const LdsLayout& L,
                                                  int8_t* dig, float* cxs, int* csum, const Prologue pro,
-                                                 float* red, const int m_valid = M) {
+                                                 float* red, const StageFirst& first, const int m_valid = M) {
   const int tid = threadIdx.x;
-  const int real_per_group = pro.in_head_dim > 0 ? pro.in_head_dim : kGroup;
-  // Items of 8 elements, 16 consecutive ones to a group. Heads of at most 64 values under int8
-  // weights: the group's upper half is padding that the multiply skips, so 8 items cover a group.
-  const bool compact = BITS == 8 && pro.in_head_dim > 0 && pro.in_head_dim <= kGroup / 2;
-  const int lg = compact ? 3 : 4;
-  const int items = (m_valid * G) << lg;
-  const int k_real = G * real_per_group;
+  const StageGeometry<BITS> geo(G, pro, m_valid);
+  const int items = geo.items, k_real = geo.k_real;
+  const bool compact = geo.lg == 3;
 
   // RMSNorm (transformers' LlamaRMSNorm.forward): variance of the whole row in fp32 first
+  // (a prologue excludes head padding and M > 1, so item i covers elements 8i .. 8i+7 of the row)
   float inv_rms = 0.0f;
-  float w_first[8], x_first[8];  // this thread's first item: weights requested before the barrier, x kept
-#pragma unroll
-  for (int e = 0; e < 8; ++e) w_first[e] = x_first[e] = 0.0f;
   if (pro.kind == LLMQ_PRO_RMSNORM) {
-    if (tid < items) load8<T>(static_cast<const T*>(pro.norm_weight) + static_cast<int64_t>(tid) * 8, w_first);
     float ss = 0.0f;
-    for (int i = tid * 8; i < k_real; i += blockDim.x * 8) {
+    if (tid * 8 < k_real) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss = fmaf(first.x[e], first.x[e], ss);
+    }
+    for (int i = (tid + blockDim.x) * 8; i < k_real; i += blockDim.x * 8) {
       float f[8];
       load8<T>(x + i, f);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        ss = fmaf(f[e], f[e], ss);
-        if (i == tid * 8) x_first[e] = f[e];  // this thread's first item: no second load
-      }
+      for (int e = 0; e < 8; ++e) ss = fmaf(f[e], f[e], ss);
     }
     ss = wave_sum(ss);
     if ((tid & (kWave - 1)) == 0) red[tid / kWave] = ss;
@@ -182,18 +230,14 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
   }
 
   for (int base = 0; base < items; base += blockDim.x) {
-    const int item = base + tid;
-    const bool active = item < items;
-    const int tq = item & ((1 << lg) - 1);
-    const int mg = active ? item >> lg : 0;  // m * G + g
-    const int m = mg / G, g = mg - m * G;
+    const StageItem<M> it(geo, base + tid, G, m_valid);
+    const bool active = it.active;
+    const int tq = it.tq, mg = it.mg, m = it.m, g = it.g;
     float f[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) f[e] = 0.0f;
-    // beyond real_per_group: the zero padding of a head group
-    const bool real = active && tq * 8 < real_per_group && m < m_valid;
-    if (real) {
-      const int64_t src = static_cast<int64_t>(m) * k_real + g * real_per_group + tq * 8;
+    if (it.real) {
+      const int64_t src = it.src;
       bool merged = false;
       if constexpr (MERGE) {
         if (pro.kind == LLMQ_PRO_ATTN_MERGE) {
@@ -209,18 +253,17 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
         }
       }
       if (merged) {
-      } else if (pro.kind == LLMQ_PRO_RMSNORM && base == 0) {
+      } else if (base == 0) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) f[e] = x_first[e];
+        for (int e = 0; e < 8; ++e) f[e] = first.x[e];
       } else {
         load8<T>(x + src, f);
       }
       if (pro.kind == LLMQ_PRO_RMSNORM) {
-        // (a prologue excludes head padding, so item i covers elements 8i .. 8i+7 of the row)
         float w[8];
         if (base == 0) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) w[e] = w_first[e];
+          for (int e = 0; e < 8; ++e) w[e] = first.w[e];
         } else {
           load8<T>(static_cast<const T*>(pro.norm_weight) + src, w);
         }
@@ -229,7 +272,12 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
       } else if (pro.kind == LLMQ_PRO_SILU_MUL) {
         // x holds gate then up: act_fn(gate) * up with both results rounded to the model dtype
         float up[8];
-        load8<T>(x + k_real + src, up);
+        if (base == 0) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) up[e] = first.w[e];
+        } else {
+          load8<T>(x + k_real + src, up);
+        }
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float silu = f[e] / (1.0f + expf(-f[e]));
@@ -244,23 +292,33 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
     if (!compact) amax = fmaxf(amax, dpp<kDppMirror>(amax));
     const int ebits = static_cast<int>((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xffu);
     const int sh = 148 - ebits;  // amax * 2^sh in [2^21, 2^22)
-    uint32_t packed[kDigits][2] = {};
-    int dsum[kDigits] = {};
+    // xi = x * 2^sh as an integer of three signed base-256 digits d0 + 256 d1 + 65536 d2. With
+    // t1 = (xi + 128) >> 8 and t2 = (t1 + 128) >> 8 the digits are the low bytes of xi, t1, t2, and
+    // t2 = (xi + 128 + 32768) >> 16: d0 is byte 0 of xi, d1 byte 1 of xi + 0x80, d2 byte 2 of
+    // xi + 0x8080. (A group of zeros gives xi = 0 without a special case.)
+    uint32_t y[kDigits][8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int xi = amax > 0.0f ? static_cast<int>(rintf(ldexpf(f[e], sh))) : 0;
-      const int d0 = static_cast<int8_t>(xi);
-      const int t1 = (xi - d0) >> 8;
-      const int d1 = static_cast<int8_t>(t1);
-      const int d2 = (t1 - d1) >> 8;
-      const int d[kDigits] = {d0, d1, d2};
+      const uint32_t xi = static_cast<uint32_t>(static_cast<int>(rintf(ldexpf(f[e], sh))));
+      y[0][e] = xi;
+      y[1][e] = xi + 0x80u;
+      y[2][e] = xi + 0x8080u;
+    }
+    // int8: bytes in element order. int4: even elements first (they meet the low nibbles), odd
+    // elements second.
+    uint32_t packed[kDigits][2];
+    int dsum[kDigits] = {};
 #pragma unroll
-      for (int q = 0; q < kDigits; ++q) {
-        dsum[q] += d[q];
-        // int8: bytes in element order. int4: even elements first (they meet the low
-        // nibbles), odd elements second.
-        const int slot = BITS == 8 ? e : (e >> 1) + 4 * (e & 1);
-        packed[q][slot >> 2] |= (static_cast<uint32_t>(d[q]) & 0xffu) << (8 * (slot & 3));
+    for (int q = 0; q < kDigits; ++q) {
+      // byte q of each of a, b: -> (a.q, b.q, 0, 0)
+      const uint32_t pick = 0x0c0c0000u | (static_cast<uint32_t>(4 + q) << 8) | static_cast<uint32_t>(q);
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int e0 = BITS == 8 ? 4 * h : h, step = BITS == 8 ? 1 : 2;
+        const uint32_t lo = __builtin_amdgcn_perm(y[q][e0 + step], y[q][e0], pick);
+        const uint32_t hi = __builtin_amdgcn_perm(y[q][e0 + 3 * step], y[q][e0 + 2 * step], pick);
+        packed[q][h] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        if constexpr (BITS == 4) dsum[q] = __builtin_amdgcn_sdot4(static_cast<int>(packed[q][h]), 0x01010101, dsum[q], false);
       }
     }
     if (active) {
@@ -324,13 +382,17 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
     const int g0 = chunk * kGW;
     const int n = tile_row(a, tile, j);
     const uint8_t* row = a.qw + static_cast<int64_t>(n) * a.row_bytes;
+    if constexpr (BITS == 8) {
+      const uint8_t* p = row + g0 * kGroup + blk * 16;
 #pragma unroll
-    for (int gi = 0; gi < kGW; ++gi) {
-      if constexpr (BITS == 8) {
-        const uint8_t* p = row + (g0 + gi) * kGroup + blk * 16;
-        b[2 * gi] = *reinterpret_cast<const v4i*>(p);
-        if (!half_groups) b[2 * gi + 1] = *reinterpret_cast<const v4i*>(p + 64);
-      } else {
+      for (int gi = 0; gi < kGW; ++gi) b[2 * gi] = *reinterpret_cast<const v4i*>(p + gi * kGroup);
+      if (!half_groups) {  // one branch for the chunk, not one per load
+#pragma unroll
+        for (int gi = 0; gi < kGW; ++gi) b[2 * gi + 1] = *reinterpret_cast<const v4i*>(p + gi * kGroup + 64);
+      }
+    } else {
+#pragma unroll
+      for (int gi = 0; gi < kGW; ++gi) {
         b[gi] = *reinterpret_cast<const v4i*>(row + (g0 + gi) * (kGroup / 2) + blk * 16);
       }
     }
@@ -369,13 +431,12 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
     }
   };
 
+  const Prologue pro{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits, a.attn_head_dim};
+  const StageFirst first = stage_first<T, BITS, M>(static_cast<const T*>(a.x), G, pro, m_valid);
   int tile = first_tile;
   if (tile < a.n_tiles) issue_loads(tile, wv);  // in flight while the activation is prepared
 
-  stage_activation<T, BITS, M, MERGE>(static_cast<const T*>(a.x), G, L, dig, cxs, csum,
-                                      Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits,
-                                               a.attn_head_dim},
-                                      red, m_valid);
+  stage_activation<T, BITS, M, MERGE>(static_cast<const T*>(a.x), G, L, dig, cxs, csum, pro, red, first, m_valid);
   __syncthreads();
   load_fragments(wv);
 
@@ -393,12 +454,19 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
         d[gi] = cinit[gi];
         if constexpr (BITS == 8) {
           d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][0], b[2 * gi], d[gi], 0, 0, 0);
-          if (!half_groups) d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], b[2 * gi + 1], d[gi], 0, 0, 0);
         } else {
           const v4i lo = b[gi] & 0x0f0f0f0f;
           const v4i hi = (b[gi] >> 4) & 0x0f0f0f0f;
           d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][0], lo, d[gi], 0, 0, 0);
           d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], hi, d[gi], 0, 0, 0);
+        }
+      }
+      if constexpr (BITS == 8) {
+        if (!half_groups) {
+#pragma unroll
+          for (int gi = 0; gi < kGW; ++gi) {
+            d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], b[2 * gi + 1], d[gi], 0, 0, 0);
+          }
         }
       }
       float s_now[kGW][M];
@@ -571,14 +639,13 @@ __global__ __launch_bounds__(256, 4) void wq_gemv_mfma_fullk_kernel(const MfmaAr
     return a.ws + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * G;
   };
 
+  const Prologue pro{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits, a.attn_head_dim};
+  const StageFirst first = stage_first<T, BITS, M>(static_cast<const T*>(a.x), G, pro);
   const int stride = gridDim.x * waves;
   int tile = blockIdx.x * waves + wv;
   if (tile < a.n_tiles) issue_weights(row_of(tile), scales_of(tile), 0);
 
-  stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum,
-                               Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits,
-                                        a.attn_head_dim},
-                               red);
+  stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum, pro, red, first);
   __syncthreads();
   issue_fragments(0);
 
@@ -691,6 +758,8 @@ __global__ __launch_bounds__(256, 2) void wq_gemv_mfma_fullk_deep_kernel(const M
     sc[D][2] = __builtin_bit_cast(float, s4_.z); sc[D][3] = __builtin_bit_cast(float, s4_.w);      \
   } while (0)
 
+  const Prologue pro{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits, a.attn_head_dim};
+  const StageFirst first = stage_first<T, BITS, M>(static_cast<const T*>(a.x), G, pro);
   const int stride = gridDim.x * waves;
   int tile = blockIdx.x * waves + wv;
   if (tile < a.n_tiles) {
@@ -700,10 +769,7 @@ __global__ __launch_bounds__(256, 2) void wq_gemv_mfma_fullk_deep_kernel(const M
     for (int d = 0; d < DEPTH; ++d) LLMQ_FILL(d, row0, sp0, d);
   }
 
-  stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum,
-                               Prologue{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits,
-                                        a.attn_head_dim},
-                               red);
+  stage_activation<T, BITS, M>(static_cast<const T*>(a.x), G, L, dig, cxs, csum, pro, red, first);
   __syncthreads();
   issue_fragments(0);
 
