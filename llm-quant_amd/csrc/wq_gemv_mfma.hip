@@ -146,12 +146,11 @@ struct Prologue {
 // How the activation is cut into items of 8 elements, 16 consecutive ones to a group. Heads of at
 // most 64 values under int8 weights: the group's upper half is padding that the multiply skips, so
 // 8 items cover a group.
-template <int BITS> struct StageGeometry {
+template <bool HALF> struct StageGeometry {
   int real_per_group, lg, items, k_real;
   __device__ __forceinline__ StageGeometry(int G, const Prologue& pro, int m_valid) {
     real_per_group = pro.in_head_dim > 0 ? pro.in_head_dim : kGroup;
-    const bool compact = BITS == 8 && pro.in_head_dim > 0 && pro.in_head_dim <= kGroup / 2;
-    lg = compact ? 3 : 4;
+    lg = HALF ? 3 : 4;
     items = (m_valid * G) << lg;
     k_real = G * real_per_group;
   }
@@ -160,8 +159,8 @@ template <int M> struct StageItem {
   bool active, real;
   int tq, mg, m, g;
   int64_t src;  // first of the item's 8 elements in x
-  template <int BITS>
-  __device__ __forceinline__ StageItem(const StageGeometry<BITS>& geo, int item, int G, int m_valid) {
+  template <bool HALF>
+  __device__ __forceinline__ StageItem(const StageGeometry<HALF>& geo, int item, int G, int m_valid) {
     active = item < geo.items;
     tq = item & ((1 << geo.lg) - 1);
     mg = active ? item >> geo.lg : 0;  // m * G + g
@@ -180,14 +179,14 @@ struct StageFirst {
   float x[8];  // the item's elements (the gate half under LLMQ_PRO_SILU_MUL)
   float w[8];  // RMSNorm weights, or the up half
 };
-template <typename T, int BITS, int M>
+template <typename T, int M, bool HALF = false>
 __device__ __forceinline__ StageFirst stage_first(const T* __restrict__ x, const int G, const Prologue& pro,
                                                   const int m_valid = M) {
   StageFirst r;
 #pragma unroll
   for (int e = 0; e < 8; ++e) r.x[e] = r.w[e] = 0.0f;
   if (pro.kind == LLMQ_PRO_ATTN_MERGE) return r;  // its records are read where they are merged
-  const StageGeometry<BITS> geo(G, pro, m_valid);
+  const StageGeometry<HALF> geo(G, pro, m_valid);
   const StageItem<M> it(geo, threadIdx.x, G, m_valid);
   if (it.real) {
     load8<T>(x + it.src, r.x);
@@ -197,14 +196,14 @@ __device__ __forceinline__ StageFirst stage_first(const T* __restrict__ x, const
   return r;
 }
 
-template <typename T, int BITS, int M, bool MERGE = false>
+template <typename T, int BITS, int M, bool MERGE = false, bool HALF = false>
 __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const int G, const LdsLayout& L,
                                                  int8_t* dig, float* cxs, int* csum, const Prologue pro,
                                                  float* red, const StageFirst& first, const int m_valid = M) {
   const int tid = threadIdx.x;
-  const StageGeometry<BITS> geo(G, pro, m_valid);
+  static_assert(!HALF || BITS == 8, "only int8 rows have a whole multiply step of padding per group");
+  const StageGeometry<HALF> geo(G, pro, m_valid);
   const int items = geo.items, k_real = geo.k_real;
-  const bool compact = geo.lg == 3;
 
   // RMSNorm (transformers' LlamaRMSNorm.forward): variance of the whole row in fp32 first
   // (a prologue excludes head padding and M > 1, so item i covers elements 8i .. 8i+7 of the row)
@@ -289,7 +288,7 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
 #pragma unroll
     for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(f[e]));
     amax = group_max<8>(amax);
-    if (!compact) amax = fmaxf(amax, dpp<kDppMirror>(amax));
+    if constexpr (!HALF) amax = fmaxf(amax, dpp<kDppMirror>(amax));
     const int ebits = static_cast<int>((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xffu);
     const int sh = 148 - ebits;  // amax * 2^sh in [2^21, 2^22)
     // xi = x * 2^sh as an integer of three signed base-256 digits d0 + 256 d1 + 65536 d2. With
@@ -350,7 +349,7 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
 // activation fragments stay in registers for the whole kernel. MULTI == true: longer rows; wave w
 // takes chunks w, w + waves, ... of every row tile and re-reads the fragments of the chunk it is
 // about to multiply from LDS (the read is issued with the weight loads, a chunk ahead).
-template <typename T, int BITS, int M, bool MULTI, bool MERGE = false>
+template <typename T, int BITS, int M, bool MULTI, bool MERGE = false, bool HALF = false>
 __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* smem, const int first_tile,
                                             const int tile_stride, const int m_valid) {
   const int tid = threadIdx.x;
@@ -369,30 +368,28 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
   const int j = lane & 15;    // weight row within the tile (B column / D column)
   const int blk = lane >> 4;  // k-block of the operand; digit block of the result
 
-  // Heads of at most 64 values, each padded to a group of its own: the activation's upper half of
-  // every group is zero whatever the weights there hold, so an int8 row's second 64 bytes of a
-  // group are neither read nor multiplied.
-  const bool half_groups = BITS == 8 && a.in_head_dim > 0 && a.in_head_dim <= kGroup / 2;
+  // HALF: heads of at most 64 values, each padded to a group of its own. The activation's upper
+  // half of every group is zero whatever the weights there hold, so an int8 row's second 64 bytes
+  // of a group are neither read nor multiplied. (A template parameter: a run-time test here, in
+  // the middle of the load sequence, costs the ordinary case a quarter of its bandwidth.)
+  static_assert(!HALF || (BITS == 8 && M == 1), "the half-group form is for int8 rows, one activation row");
 
   // ---- weight / scale loads of one chunk of one row tile ------------------------------------
-  constexpr int kLoads = BITS == 8 ? 2 * kGW : kGW;
-  v4i b[kLoads] = {};
+  constexpr int kLoads = BITS == 8 ? (HALF ? kGW : 2 * kGW) : kGW;
+  constexpr int kB = BITS == 8 && !HALF ? 2 : 1;  // operand registers per group
+  v4i b[kLoads];
   float sc[kGW];
   auto issue_loads = [&](int tile, int chunk) {
     const int g0 = chunk * kGW;
     const int n = tile_row(a, tile, j);
     const uint8_t* row = a.qw + static_cast<int64_t>(n) * a.row_bytes;
-    if constexpr (BITS == 8) {
-      const uint8_t* p = row + g0 * kGroup + blk * 16;
 #pragma unroll
-      for (int gi = 0; gi < kGW; ++gi) b[2 * gi] = *reinterpret_cast<const v4i*>(p + gi * kGroup);
-      if (!half_groups) {  // one branch for the chunk, not one per load
-#pragma unroll
-        for (int gi = 0; gi < kGW; ++gi) b[2 * gi + 1] = *reinterpret_cast<const v4i*>(p + gi * kGroup + 64);
-      }
-    } else {
-#pragma unroll
-      for (int gi = 0; gi < kGW; ++gi) {
+    for (int gi = 0; gi < kGW; ++gi) {
+      if constexpr (BITS == 8) {
+        const uint8_t* p = row + (g0 + gi) * kGroup + blk * 16;
+        b[kB * gi] = *reinterpret_cast<const v4i*>(p);
+        if constexpr (!HALF) b[kB * gi + 1] = *reinterpret_cast<const v4i*>(p + 64);
+      } else {
         b[gi] = *reinterpret_cast<const v4i*>(row + (g0 + gi) * (kGroup / 2) + blk * 16);
       }
     }
@@ -416,7 +413,7 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         afrag[gi][s] = v4i{0, 0, 0, 0};
-        if (q < kDigits && m < M && !(s == 1 && half_groups)) {
+        if (q < kDigits && m < M && !(s == 1 && HALF)) {
           afrag[gi][s] = *reinterpret_cast<const v4i*>(dig + (q * M + m) * L.plane + g * kGroup + s * 64 + blk * 16);
         }
       }
@@ -432,11 +429,12 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
   };
 
   const Prologue pro{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits, a.attn_head_dim};
-  const StageFirst first = stage_first<T, BITS, M>(static_cast<const T*>(a.x), G, pro, m_valid);
+  const StageFirst first = stage_first<T, M, HALF>(static_cast<const T*>(a.x), G, pro, m_valid);
   int tile = first_tile;
   if (tile < a.n_tiles) issue_loads(tile, wv);  // in flight while the activation is prepared
 
-  stage_activation<T, BITS, M, MERGE>(static_cast<const T*>(a.x), G, L, dig, cxs, csum, pro, red, first, m_valid);
+  stage_activation<T, BITS, M, MERGE, HALF>(static_cast<const T*>(a.x), G, L, dig, cxs, csum, pro, red, first,
+                                            m_valid);
   __syncthreads();
   load_fragments(wv);
 
@@ -453,20 +451,15 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
       for (int gi = 0; gi < kGW; ++gi) {
         d[gi] = cinit[gi];
         if constexpr (BITS == 8) {
-          d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][0], b[2 * gi], d[gi], 0, 0, 0);
+          d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][0], b[kB * gi], d[gi], 0, 0, 0);
+          if constexpr (!HALF) {
+            d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], b[kB * gi + 1], d[gi], 0, 0, 0);
+          }
         } else {
           const v4i lo = b[gi] & 0x0f0f0f0f;
           const v4i hi = (b[gi] >> 4) & 0x0f0f0f0f;
           d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][0], lo, d[gi], 0, 0, 0);
           d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], hi, d[gi], 0, 0, 0);
-        }
-      }
-      if constexpr (BITS == 8) {
-        if (!half_groups) {
-#pragma unroll
-          for (int gi = 0; gi < kGW; ++gi) {
-            d[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[gi][1], b[2 * gi + 1], d[gi], 0, 0, 0);
-          }
         }
       }
       float s_now[kGW][M];
@@ -523,10 +516,10 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
   }
 }
 
-template <typename T, int BITS, int M, int MAXT, bool MULTI, bool MERGE = false>
+template <typename T, int BITS, int M, int MAXT, bool MULTI, bool MERGE = false, bool HALF = false>
 __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_kernel(const MfmaArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  ksplit_body<T, BITS, M, MULTI, MERGE>(a, smem, blockIdx.x, gridDim.x, M);
+  ksplit_body<T, BITS, M, MULTI, MERGE, HALF>(a, smem, blockIdx.x, gridDim.x, M);
 }
 
 // Many small GEMVs in one launch (the routed experts of a Mixture-of-Experts layer). Plan entry
@@ -640,7 +633,7 @@ __global__ __launch_bounds__(256, 4) void wq_gemv_mfma_fullk_kernel(const MfmaAr
   };
 
   const Prologue pro{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits, a.attn_head_dim};
-  const StageFirst first = stage_first<T, BITS, M>(static_cast<const T*>(a.x), G, pro);
+  const StageFirst first = stage_first<T, M>(static_cast<const T*>(a.x), G, pro);
   const int stride = gridDim.x * waves;
   int tile = blockIdx.x * waves + wv;
   if (tile < a.n_tiles) issue_weights(row_of(tile), scales_of(tile), 0);
@@ -759,7 +752,7 @@ __global__ __launch_bounds__(256, 2) void wq_gemv_mfma_fullk_deep_kernel(const M
   } while (0)
 
   const Prologue pro{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits, a.attn_head_dim};
-  const StageFirst first = stage_first<T, BITS, M>(static_cast<const T*>(a.x), G, pro);
+  const StageFirst first = stage_first<T, M>(static_cast<const T*>(a.x), G, pro);
   const int stride = gridDim.x * waves;
   int tile = blockIdx.x * waves + wv;
   if (tile < a.n_tiles) {
@@ -825,9 +818,9 @@ constexpr int kFullKMinTiles = 1024;
 constexpr int kLdsDefault = 64 * 1024;   // dynamic LDS a kernel may use without opting in
 constexpr int kLdsMax = 160 * 1024;      // LDS of one gfx950 CU
 
-template <typename T, int BITS, int M, int MAXT, bool MULTI, bool MERGE = false>
+template <typename T, int BITS, int M, int MAXT, bool MULTI, bool MERGE = false, bool HALF = false>
 int launch_one(const MfmaArgs& a, int wk, int grid, int lds, hipStream_t stream) {
-  auto kernel = wq_gemv_mfma_kernel<T, BITS, M, MAXT, MULTI, MERGE>;
+  auto kernel = wq_gemv_mfma_kernel<T, BITS, M, MAXT, MULTI, MERGE, HALF>;
   if (lds > kLdsDefault) {
     static bool raised = false;  // per instantiation; worst case two threads both set it
     if (!raised) {
@@ -846,6 +839,20 @@ int launch_one(const MfmaArgs& a, int wk, int grid, int lds, hipStream_t stream)
 
 template <typename T, int BITS, int M>
 int launch_m(const MfmaArgs& a, int wk, int grid, int lds, hipStream_t stream) {
+  if constexpr (M == 1 && BITS == 8) {
+    // heads of at most half a group, each padded to a group of its own (o_proj of a model with
+    // 64-wide heads): the variants that skip the padding
+    if (a.in_head_dim > 0 && a.in_head_dim <= kGroup / 2 && wk * kGW == a.G) {
+      if (a.prologue == LLMQ_PRO_ATTN_MERGE) {
+        if (wk <= 4) return launch_one<T, 8, 1, 256, false, true, true>(a, wk, grid, lds, stream);
+        if (wk <= 8) return launch_one<T, 8, 1, 512, false, true, true>(a, wk, grid, lds, stream);
+        return launch_one<T, 8, 1, 1024, false, true, true>(a, wk, grid, lds, stream);
+      }
+      if (wk <= 4) return launch_one<T, 8, 1, 256, false, false, true>(a, wk, grid, lds, stream);
+      if (wk <= 8) return launch_one<T, 8, 1, 512, false, false, true>(a, wk, grid, lds, stream);
+      return launch_one<T, 8, 1, 1024, false, false, true>(a, wk, grid, lds, stream);
+    }
+  }
   if constexpr (M == 1) {
     if (a.prologue == LLMQ_PRO_ATTN_MERGE) {
       if (wk * kGW < a.G) return launch_one<T, BITS, 1, 512, true, true>(a, wk, grid, lds, stream);
