@@ -187,7 +187,14 @@ __device__ __forceinline__ float quant_code(float v, float scale, float qmin, fl
 // all loads issued before any is used (a loop that waits for each record costs a memory round
 // trip per split); further batches rescale the running sums like online softmax.
 constexpr int kAttnRecordHeader = 4;
-__device__ __forceinline__ void merge_partials8(const float* rec, int n_splits, int head_dim, int d0, float* f) {
+struct NoHook {
+  __device__ __forceinline__ void operator()() const {}
+};
+// `after_first_loads` runs once, between the first batch's loads and their first use: the place for
+// a caller's own loads that have more slack than these.
+template <typename Hook = NoHook>
+__device__ __forceinline__ void merge_partials8(const float* rec, int n_splits, int head_dim, int d0, float* f,
+                                                Hook after_first_loads = Hook()) {
   const int stride = head_dim + kAttnRecordHeader;
   float mm = -INFINITY, ll = 0.0f;
 #pragma unroll
@@ -203,6 +210,7 @@ __device__ __forceinline__ void merge_partials8(const float* rec, int n_splits, 
       lo[j] = load16(r + kAttnRecordHeader + d0);
       hi[j] = load16(r + kAttnRecordHeader + d0 + 4);
     }
+    if (s0 == 0) after_first_loads();
     float m_new = mm;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {

@@ -196,15 +196,23 @@ __device__ __forceinline__ StageFirst stage_first(const T* __restrict__ x, const
   return r;
 }
 
-template <typename T, int BITS, int M, bool MERGE = false, bool HALF = false>
+// `after_first_loads`: called by every thread once, as soon as its first item's loads from memory
+// are requested when those are requested here (the merge prologue), else at the top.
+template <typename T, int BITS, int M, bool MERGE = false, bool HALF = false, typename Hook = NoHook>
 __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const int G, const LdsLayout& L,
                                                  int8_t* dig, float* cxs, int* csum, const Prologue pro,
-                                                 float* red, const StageFirst& first, const int m_valid = M) {
+                                                 float* red, const StageFirst& first, const int m_valid = M,
+                                                 Hook after_first_loads = Hook()) {
   const int tid = threadIdx.x;
   static_assert(!HALF || BITS == 8, "only int8 rows have a whole multiply step of padding per group");
   const StageGeometry<HALF> geo(G, pro, m_valid);
   const int items = geo.items, k_real = geo.k_real;
 
+  bool hook_pending = true;
+  if (!(MERGE && pro.kind == LLMQ_PRO_ATTN_MERGE)) {
+    after_first_loads();
+    hook_pending = false;
+  }
   // RMSNorm (transformers' LlamaRMSNorm.forward): variance of the whole row in fp32 first
   // (a prologue excludes head padding and M > 1, so item i covers elements 8i .. 8i+7 of the row)
   float inv_rms = 0.0f;
@@ -243,9 +251,13 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
           // x holds the partial records of split attention; elements src .. src+7 lie in one head
           const int hd = pro.attn_head_dim;
           const int head = static_cast<int>(src) / hd, d0 = static_cast<int>(src) - head * hd;
+          const bool fire = hook_pending;
+          hook_pending = false;
           merge_partials8(reinterpret_cast<const float*>(x) +
                               static_cast<int64_t>(head) * pro.attn_splits * (hd + kAttnRecordHeader),
-                          pro.attn_splits, hd, d0, f);
+                          pro.attn_splits, hd, d0, f, [&] {
+                            if (fire) after_first_loads();
+                          });
 #pragma unroll
           for (int e = 0; e < 8; ++e) f[e] = round_through<T>(f[e]);
           merged = true;
@@ -342,7 +354,12 @@ __device__ __forceinline__ void stage_activation(const T* __restrict__ x, const 
       }
     }
     if (active && tq == 0) cxs[mg] = amax > 0.0f ? ldexpf(1.0f, -sh) : 0.0f;
+    if (hook_pending) {  // this thread's first item read nothing
+      after_first_loads();
+      hook_pending = false;
+    }
   }
+  if (hook_pending) after_first_loads();
 }
 
 // MULTI == false: the workgroup has one wave per chunk of four groups (K <= 8192) and a wave's
@@ -430,11 +447,13 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
 
   const Prologue pro{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits, a.attn_head_dim};
   const StageFirst first = stage_first<T, M, HALF>(static_cast<const T*>(a.x), G, pro, m_valid);
+  // the first tile's weights: in flight while the activation is prepared, requested right after the
+  // activation's own first loads
   int tile = first_tile;
-  if (tile < a.n_tiles) issue_loads(tile, wv);  // in flight while the activation is prepared
-
   stage_activation<T, BITS, M, MERGE, HALF>(static_cast<const T*>(a.x), G, L, dig, cxs, csum, pro, red, first,
-                                            m_valid);
+                                            m_valid, [&] {
+                                              if (tile < a.n_tiles) issue_loads(tile, wv);
+                                            });
   __syncthreads();
   load_fragments(wv);
 
