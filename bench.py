@@ -42,7 +42,7 @@ SHAPES = [  # name, N, K  (BASELINE config 2)
 # HBM bytes one lm_head int8 launch moves, from hardware counters (FETCH_SIZE and WRITE_SIZE, each
 # scaled by its reading for a 256 MiB copy): profiles/wq_gemv_lm_head_hbm_traffic.txt. 1.001 x the
 # algorithmic bytes.
-LM_HEAD_INT8_TRAFFIC_BYTES = 271_404_500
+LM_HEAD_INT8_TRAFFIC_BYTES = 271_451_500
 
 
 def algorithmic_bytes(n: int, k: int, bits: int, m: int = 1) -> int:
