@@ -150,7 +150,7 @@ __device__ __forceinline__ void decode_raw(const RawCodes<BITS, DPL>& r, float* 
   }
 }
 
-// The first step's operands of attend_range, for callers that can request them early.
+// One step's operands of attend_range, for callers that can request the first steps early.
 template <int BITS, int DPL> struct AttnPrefetch {
   RawCodes<BITS, DPL> k, v;
   float ks, vs;
@@ -172,12 +172,21 @@ __device__ __forceinline__ AttnPrefetch<BITS, DPL> attn_prefetch(const uint8_t* 
 // step, a quad of lanes per token), followed by the merge of the wave's 16 quads. On return
 // lanes 0..3 (and every lane with the same dq, up to the order of the additions) hold the wave's
 // (max, sum, weighted output quarter) per head.
-template <typename T, int BITS, int D, int REP>
+// The loads of step i + NPRE are issued before step i is computed. `first`, when given, holds the
+// operands of steps 0 .. NPRE-1 (token rows min(t_first + i t_step + tk, t_clamp)), requested by the
+// caller before it knew t_end; every row up to t_clamp must be readable, what lies at or beyond
+// t_end is loaded and dropped.
+// ROW_PARTIALS (REP == 1): instead of the merged wave result, every lane returns the wave's maximum
+// in m and, in l / o, the sums over the four quads of its own row of 16 lanes that share its dq,
+// already scaled to that maximum: the caller adds the four rows (lanes 0..3, 16..19, 32..35, 48..51).
+// One exponential and two DPP additions per value, against a rescaling exchange per step and two
+// trips through the LDS permute path for the full merge.
+template <typename T, int BITS, int D, int REP, int NPRE = 1, bool ROW_PARTIALS = false>
 __device__ __forceinline__ void attend_range(const float (*qf)[D / 4], const uint8_t* kbase, const uint8_t* vbase,
                                              const float* ksc, const float* vsc, const int t_first,
                                              const int t_end, const int t_step, const int tk, const int dq,
                                              float* m, float* l, float (*o)[D / 4],
-                                             const AttnPrefetch<BITS, D / 4>* first = nullptr) {
+                                             const AttnPrefetch<BITS, D / 4>* first = nullptr, int t_clamp = -1) {
   constexpr int DPL = D / 4;
   constexpr int ROWB = BITS == 8 ? D : D / 2;
 #pragma unroll
@@ -188,26 +197,27 @@ __device__ __forceinline__ void attend_range(const float (*qf)[D / 4], const uin
     for (int i = 0; i < DPL; ++i) o[h][i] = 0.0f;
   }
 
-  // the loads of step i + 1 are issued before step i is computed
-  auto fetch = [&](int t0, RawCodes<BITS, DPL>& kr, RawCodes<BITS, DPL>& vr, float& ks, float& vs) {
-    const int tc = min(t0 + tk, t_end - 1);  // clamp: loads stay in range, result dropped
-    kr = load_raw<BITS, DPL>(kbase + static_cast<int64_t>(tc) * ROWB, dq);
-    vr = load_raw<BITS, DPL>(vbase + static_cast<int64_t>(tc) * ROWB, dq);
-    ks = ksc[tc];
-    vs = vsc[tc];
-  };
-  RawCodes<BITS, DPL> k_next, v_next;
-  float ks_next = 0.0f, vs_next = 0.0f;
-  if (first != nullptr) {
-    k_next = first->k; v_next = first->v; ks_next = first->ks; vs_next = first->vs;
-  } else if (t_first < t_end) {
-    fetch(t_first, k_next, v_next, ks_next, vs_next);
+  if (t_clamp < 0) t_clamp = t_end - 1;  // clamp: loads stay in range, result dropped
+  AttnPrefetch<BITS, DPL> ring[NPRE];
+#pragma unroll
+  for (int r = 0; r < NPRE; ++r) {
+    if (first != nullptr) {
+      ring[r] = first[r];
+    } else if (t_first + r * t_step < t_end) {
+      ring[r] = attn_prefetch<BITS, DPL>(kbase, vbase, ksc, vsc, min(t_first + r * t_step + tk, t_clamp), dq);
+    }
   }
-  for (int t0 = t_first; t0 < t_end; t0 += t_step) {
+  for (int t_round = t_first; t_round < t_end; t_round += NPRE * t_step) {
+#pragma unroll
+  for (int r = 0; r < NPRE; ++r) {
+    const int t0 = t_round + r * t_step;
+    if (t0 >= t_end) break;
     const bool ok = t0 + tk < t_end;
-    const RawCodes<BITS, DPL> k_now = k_next, v_now = v_next;
-    const float ks = ks_next, vs = vs_next;
-    if (t0 + t_step < t_end) fetch(t0 + t_step, k_next, v_next, ks_next, vs_next);
+    const RawCodes<BITS, DPL> k_now = ring[r].k, v_now = ring[r].v;
+    const float ks = ring[r].ks, vs = ring[r].vs;
+    if (t0 + NPRE * t_step < t_end) {
+      ring[r] = attn_prefetch<BITS, DPL>(kbase, vbase, ksc, vsc, min(t0 + NPRE * t_step + tk, t_clamp), dq);
+    }
     float kc[DPL], vc[DPL];
     decode_raw<BITS, DPL>(k_now, kc);
     decode_raw<BITS, DPL>(v_now, vc);
@@ -245,7 +255,25 @@ __device__ __forceinline__ void attend_range(const float (*qf)[D / 4], const uin
       }
     }
   }
+  }
 
+  if constexpr (ROW_PARTIALS) {
+    static_assert(REP == 1, "row partials are kept for one head per wave");
+    const float m_wave = group_max<kWave>(m[0]);
+    const float a = m[0] == -INFINITY ? 0.0f : exp2f(m[0] - m_wave);
+    l[0] *= a;
+    l[0] += dpp<kDppRor4>(l[0]);
+    l[0] += dpp<kDppRor8>(l[0]);
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+      float v = o[0][i] * a;
+      v += dpp<kDppRor4>(v);
+      v += dpp<kDppRor8>(v);
+      o[0][i] = v;
+    }
+    m[0] = m_wave;
+    return;
+  }
   // ---- merge the 16 quads of the wave (lanes with the same dq) ----------------------------------------
   // Inside a row of 16 lanes: rotate by 4, then by 8 (DPP, no LDS round trip); lane i then holds
   // quads i, i+4, i+8, i+12 of its row. Across the four rows: xor 16, xor 32.
@@ -516,6 +544,7 @@ __global__ __launch_bounds__(kFusedThreads) void kv_rope_append_attend_kernel(
 constexpr int kSplitWaves = 4;
 constexpr int kSplitThreads = kSplitWaves * kWave;
 constexpr int kSplitSlab = kSplitWaves * kTokPerIter;  // 64 tokens per workgroup step
+constexpr int kSplitPrefetch = 2;  // steps of cache rows a wave requests before it knows the position
 
 template <typename T, int BITS, int D>
 __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_kernel(
@@ -529,7 +558,8 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
   constexpr int GREC = D + kAttnRecordHeader;  // per-split record in global memory
   __shared__ float s_q[D];
   __shared__ float s_new[2][D];
-  __shared__ float s_rec[kSplitWaves][REC];
+  __shared__ float s_rec[kSplitWaves][4][REC];  // per wave and row of 16 lanes: (wave max, sum, output)
+  __shared__ float s_new_score;                 // the new token's score (last split), else -inf
 
   const int qh = blockIdx.x, split = blockIdx.y, n_splits = gridDim.y;
   const bool last_split = split == n_splits - 1;
@@ -538,17 +568,25 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
   const bool writer = last_split && qh % rep == 0;
   const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
   const int tk = lane >> 2, dq = lane & 3;
-  const int pos = min(max(pos_dev[0], 0), t_max - 1);
-  const T* cos_row = cos_table + static_cast<int64_t>(pos) * D;
-  const T* sin_row = sin_table + static_cast<int64_t>(pos) * D;
 
+  // The wave's first steps of cache rows do not depend on the position (rows up to t_max - 1 exist;
+  // what lies at or beyond the position is dropped later): requested first, so that the position's
+  // own round trip and phase A run under them.
   const uint8_t* kbase = k_codes + static_cast<int64_t>(kvh) * t_max * ROWB;
   const uint8_t* vbase = v_codes + static_cast<int64_t>(kvh) * t_max * ROWB;
   const float* ksc = k_scale + static_cast<int64_t>(kvh) * t_max;
   const float* vsc = v_scale + static_cast<int64_t>(kvh) * t_max;
   const int t_mine = split * kSplitSlab + wv * kTokPerIter;
-  AttnPrefetch<BITS, DPL> first;
-  if (t_mine < pos) first = attn_prefetch<BITS, DPL>(kbase, vbase, ksc, vsc, min(t_mine + tk, pos - 1), dq);
+  const int t_step = n_splits * kSplitSlab;
+  AttnPrefetch<BITS, DPL> first[kSplitPrefetch];
+#pragma unroll
+  for (int r = 0; r < kSplitPrefetch; ++r) {
+    first[r] = attn_prefetch<BITS, DPL>(kbase, vbase, ksc, vsc, min(t_mine + r * t_step + tk, t_max - 1), dq);
+  }
+
+  const int pos = min(max(pos_dev[0], 0), t_max - 1);
+  const T* cos_row = cos_table + static_cast<int64_t>(pos) * D;
+  const T* sin_row = sin_table + static_cast<int64_t>(pos) * D;
 
   // ---- phase A: wave 0 rotates the query; in the last split wave 1 / 2 prepare the new K / V ----------
   if (wv == 0) {
@@ -593,42 +631,44 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
 #pragma unroll
   for (int i = 0; i < DPL; ++i) qf[0][i] = s_q[dq * DPL + i];
   float m[1], l[1], o[1][DPL];
-  attend_range<T, BITS, D, 1>(qf, kbase, vbase, ksc, vsc, t_mine, pos, n_splits * kSplitSlab, tk, dq, m, l, o,
-                              t_mine < pos ? &first : nullptr);
-  if (last_split && wv == kSplitWaves - 1) {
+  attend_range<T, BITS, D, 1, kSplitPrefetch, true>(qf, kbase, vbase, ksc, vsc, t_mine, pos, t_step, tk, dq, m, l, o,
+                                                    first, t_max - 1);
+  if (wv == kSplitWaves - 1) {
+    // the new token is a record of its own: score here, its value is s_new[1]
     float sc = 0.0f;
 #pragma unroll
     for (int i = 0; i < DPL; ++i) sc = fmaf(qf[0][i], s_new[0][dq * DPL + i], sc);
     sc += dpp<kDppXor1>(sc);
     sc += dpp<kDppXor2>(sc);
-    const float m_new = fmaxf(m[0], sc);
-    const float corr = m[0] == -INFINITY ? 0.0f : exp2f(m[0] - m_new);
-    const float pnew = exp2f(sc - m_new);
-    l[0] = l[0] * corr + pnew;
-#pragma unroll
-    for (int i = 0; i < DPL; ++i) o[0][i] = fmaf(pnew, s_new[1][dq * DPL + i], o[0][i] * corr);
-    m[0] = m_new;
+    if (lane == 0) s_new_score = last_split ? sc : -INFINITY;
   }
-  if (tk == 0) {
+  if ((tk & 3) == 0) {
+    const int row = lane >> 4;
     if (dq == 0) {
-      s_rec[wv][0] = m[0];
-      s_rec[wv][1] = l[0];
+      s_rec[wv][row][0] = m[0];
+      s_rec[wv][row][1] = l[0];
     }
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) s_rec[wv][2 + dq * DPL + i] = o[0][i];
+    for (int i = 0; i < DPL; ++i) s_rec[wv][row][2 + dq * DPL + i] = o[0][i];
   }
   __syncthreads();
   if (threadIdx.x < D) {
     const int d = threadIdx.x;
-    float mm = -INFINITY;
+    const float new_score = s_new_score;
+    float mm = new_score;
 #pragma unroll
-    for (int w = 0; w < kSplitWaves; ++w) mm = fmaxf(mm, s_rec[w][0]);
+    for (int w = 0; w < kSplitWaves; ++w) mm = fmaxf(mm, s_rec[w][0][0]);
     float ll = 0.0f, oo = 0.0f;
 #pragma unroll
     for (int w = 0; w < kSplitWaves; ++w) {
-      const float a = s_rec[w][0] == -INFINITY ? 0.0f : exp2f(s_rec[w][0] - mm);
-      ll += s_rec[w][1] * a;
-      oo += s_rec[w][2 + d] * a;
+      const float a = s_rec[w][0][0] == -INFINITY ? 0.0f : exp2f(s_rec[w][0][0] - mm);
+      ll += ((s_rec[w][0][1] + s_rec[w][1][1]) + (s_rec[w][2][1] + s_rec[w][3][1])) * a;
+      oo += ((s_rec[w][0][2 + d] + s_rec[w][1][2 + d]) + (s_rec[w][2][2 + d] + s_rec[w][3][2 + d])) * a;
+    }
+    if (new_score != -INFINITY) {
+      const float b = exp2f(new_score - mm);
+      ll += b;
+      oo = fmaf(b, s_new[1][d], oo);
     }
     float* rec = partials + (static_cast<int64_t>(qh) * n_splits + split) * GREC;
     if (d == 0) {
