@@ -114,6 +114,33 @@ def test_head_padding_and_residual(ext, bits):
     assert torch.equal(plain, ext.wq_gemv(x, q16, s16, 0))
 
 
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("heads,head_dim", [(8, 64), (16, 64), (64, 64), (80, 64), (32, 32), (16, 96), (40, 8)])
+def test_head_padding_widths(ext, bits, heads, head_dim):
+    """Heads narrower than a group, each padded to a group of its own: every workgroup size of the int8
+    form that skips the padded half (8 / 16 / 64 heads of 64 or less), rows too long for it (80 heads:
+    the multi-chunk kernel), heads wider than half a group (96: nothing can be skipped), tiny heads."""
+    from llmquant.core.scheme import QuantizationArgs
+    from llmquant.quantizers import pad_activation
+
+    n, k = 272, heads * head_dim
+    q, s = weights(n, k, bits, head_dim=head_dim, seed=11)
+    assert q.shape[1] == heads
+    torch.manual_seed(12)
+    x = torch.randn(1, k).to(torch.bfloat16).cuda()
+    res = torch.randn(1, n).to(torch.bfloat16).cuda()
+    got = ext.wq_gemv_fused(x, q, s, 0, 0, None, 0.0, head_dim, res)
+    padded = pad_activation(x, QuantizationArgs(bits, "group", group_size=128, head_dim=head_dim))
+    assert torch.equal(got, res + ext.wq_gemv(padded, q, s, 0))
+    # what the padded half of the weight holds must not matter: the activation there is zero
+    noisy = q.clone()
+    if bits == 8:
+        noisy[:, :, head_dim:] = 77
+    else:
+        noisy[:, :, (head_dim + 1) // 2:] = 0x5A
+    assert torch.equal(ext.wq_gemv_fused(x, noisy, s, 0, 0, None, 0.0, head_dim, res), got)
+
+
 def test_fused_gemv_argument_checks(ext):
     q, s = weights(256, 512, 8)
     x = torch.randn(1, 512, device="cuda", dtype=torch.bfloat16)
