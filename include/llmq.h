@@ -77,7 +77,8 @@ int llmq_wq_gemv(const void* x, const void* qweight, const float* wscale, void* 
  * n_blocks entries, built by the caller on the device and never read by the host) says: rows
  * block_row0[b] .. +block_rows[b]-1 of x [n_rows, G*gs] go through expert block_expert[b]; an entry
  * with block_rows <= 0 is skipped, one that points outside x or the expert stack is ignored. A run
- * holds at most llmq_wq_gemv_batched_max_rows() rows. out: [n_rows, N]; rows no entry covers are
+ * holds at most llmq_wq_gemv_batched_max_rows() rows, and runs do not overlap (so at most n_rows
+ * entries hold rows: the launch is sized for that many). out: [n_rows, N]; rows no entry covers are
  * left untouched. Each row's arithmetic is llmq_wq_gemv's. */
 int llmq_wq_gemv_batched_max_rows(void);
 int llmq_wq_gemv_batched(const void* x, const void* qweight, const float* wscale, void* out,

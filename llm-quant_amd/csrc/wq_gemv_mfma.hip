@@ -550,7 +550,7 @@ struct BatchPlan {
   const int32_t* expert;
   const int32_t* row0;
   const int32_t* rows;
-  int n_experts, n_rows;
+  int n_experts, n_rows, n_blocks;
   int64_t weight_stride;  // bytes between experts' weights
   int64_t scale_stride;   // floats between experts' scales
 };
@@ -559,7 +559,27 @@ constexpr int kBatchedMaxRows = 8;
 template <typename T, int BITS, int MAXT, bool MULTI>
 __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_batched_kernel(MfmaArgs a, const BatchPlan plan) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int b = blockIdx.y;
+  // blockIdx.y counts the entries that hold rows, not the entries: with 8 of 64 experts routed, a
+  // grid over all entries is seven eighths workgroups that start only to exit. Each wave finds the
+  // entry for itself: 64 entries per step, one load, a ballot and a count.
+  int b = -1;
+  {
+    const int lane = threadIdx.x & (kWave - 1);
+    int seen = 0;
+    for (int base = 0; base < plan.n_blocks; base += kWave) {
+      const int idx = base + lane;
+      const int r = idx < plan.n_blocks ? plan.rows[idx] : 0;
+      unsigned long long mask = __ballot(r > 0);
+      const int cnt = __popcll(mask);
+      if (static_cast<int>(blockIdx.y) < seen + cnt) {
+        for (int skip = static_cast<int>(blockIdx.y) - seen; skip > 0; --skip) mask &= mask - 1;
+        b = base + __ffsll(static_cast<long long>(mask)) - 1;
+        break;
+      }
+      seen += cnt;
+    }
+  }
+  if (b < 0) return;  // fewer entries hold rows than the grid allows for
   const int rows = min(plan.rows[b], kBatchedMaxRows);
   if (rows <= 0) return;
   const int e = plan.expert[b], row0 = plan.row0[b];
@@ -569,6 +589,14 @@ __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_batched_kernel(MfmaArgs a, 
   const int64_t k_total = static_cast<int64_t>(a.G) * kGroup;
   const T* x = static_cast<const T*>(a.x);
   T* out = static_cast<T*>(a.out);
+  if (rows == 1) {
+    // the decode case (one token: every routed expert has one row): the single-row body, which
+    // stages a quarter of the fragments and accumulators of the four-row one
+    a.x = x + row0 * k_total;
+    a.out = out + static_cast<int64_t>(row0) * a.N;
+    ksplit_body<T, BITS, 1, MULTI>(a, smem, blockIdx.x, gridDim.x, 1);
+    return;
+  }
   for (int done = 0; done < rows; done += 4) {
     if (done > 0) __syncthreads();  // the previous pass is done with the LDS
     a.x = x + (row0 + done) * k_total;
@@ -1026,12 +1054,13 @@ int launch_batched(const MfmaArgs& a, const BatchPlan& plan, int n_blocks, hipSt
   const int wk = waves_for(a.G / kGW);
   const bool multi = wk * kGW < a.G;
   const LdsLayout L(4, a.G, wk, BITS == 4);
-  // about a thousand workgroups over the entries that can hold rows (at most one per row)
+  // about five hundred workgroups (all resident at once at this kernel's register count) over the
+  // entries that can hold rows: at most one per row
   const int live = plan.n_rows < n_blocks ? plan.n_rows : n_blocks;
-  int gx = 1024 / (live > 0 ? live : 1);
+  int gx = 512 / (live > 0 ? live : 1);
   if (gx < 16) gx = 16;
   if (gx > a.n_tiles) gx = a.n_tiles;
-  const dim3 grid(gx, n_blocks), block(wk * kWave);
+  const dim3 grid(gx, live), block(wk * kWave);
 #define LLMQ_BATCHED(MAXT, MULTI)                                                                   \
   do {                                                                                              \
     auto kernel = wq_gemv_mfma_batched_kernel<T, BITS, MAXT, MULTI>;                                \
@@ -1072,7 +1101,7 @@ int gemv_batched_mfma_launch(const void* x, const void* qw, const float* ws, voi
   a.n_tiles = (N + kTileRows - 1) / kTileRows;
   a.row_bytes = G * kGroup * (wformat == LLMQ_W_INT8 ? 8 : 4) / 8;
   const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
-  BatchPlan plan{block_expert, block_row0, block_rows, n_experts, n_rows,
+  BatchPlan plan{block_expert, block_row0, block_rows, n_experts, n_rows, n_blocks,
                  static_cast<int64_t>(N) * a.row_bytes, scale_rows * G};
 #define LLMQ_DISPATCH(T) \
   (wformat == LLMQ_W_INT8 ? launch_batched<T, 8>(a, plan, n_blocks, stream) : launch_batched<T, 4>(a, plan, n_blocks, stream))
