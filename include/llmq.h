@@ -86,6 +86,20 @@ int llmq_wq_gemv_batched(const void* x, const void* qweight, const float* wscale
                          const int32_t* block_rows, int n_blocks, int n_rows, int n_experts, int N,
                          int G, int gs, int out_group, int wformat, int dtype, llmq_stream_t stream);
 
+/* The routing plan llmq_wq_gemv_batched takes, in one launch: what KernelQuantExperts._plan
+ * (llmquant/quantizers/kernel.py:176-214) computes with a stable argsort, scatter_add, cumsum and
+ * arange arithmetic in PyTorch, same integers. expert_of_row: [n_rows] expert of every (token, slot)
+ * row (top_k_index flattened; an id outside [0, n_experts) is counted with the nearest valid one).
+ * order: [n_rows], order[i] = index of the i-th row when the rows are sorted by expert, equal experts
+ * in their original order. Every expert gets B = llmq_route_plan_blocks_per_expert(n_rows, limit) =
+ * max(1, ceil(n_rows / limit)) entries: block_expert / block_row0 / block_rows are [n_experts * B],
+ * entry e * B + b = (e, first[e] + b * limit, clamp(count[e] - b * limit, 0, limit)). One workgroup;
+ * llmq_route_plan_supported says whether the sizes fit it (up to 8192 rows, 1024 experts). */
+int llmq_route_plan_blocks_per_expert(int n_rows, int limit);
+int llmq_route_plan_supported(int n_rows, int n_experts);
+int llmq_route_plan(const int64_t* expert_of_row, int n_rows, int n_experts, int limit, int64_t* order,
+                    int32_t* block_expert, int32_t* block_row0, int32_t* block_rows, llmq_stream_t stream);
+
 /* The decode-step form of llmq_wq_gemv (M = 1, group size 128): the same product with the
  * elementwise operations that surround a Linear in a Llama decoder layer folded in, so that a
  * layer is five launches instead of ~40. There is no counterpart in the reference, which leaves

@@ -255,6 +255,33 @@ at::Tensor wq_gemv_fused(const at::Tensor& x, const at::Tensor& qweight, const a
   return out;
 }
 
+// The batched GEMV's routing plan in one launch (see llmq_route_plan). top_k_index: integer tensor of
+// any shape; returns (order int64 [rows], block_expert, block_row0, block_rows int32 [experts * B]).
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> route_plan(const at::Tensor& top_k_index,
+                                                                      int64_t num_experts, int64_t limit) {
+  TORCH_CHECK(top_k_index.is_cuda(), "top_k_index must be a CUDA tensor");
+  TORCH_CHECK(at::isIntegralType(top_k_index.scalar_type(), false), "top_k_index must hold integers");
+  const at::Tensor flat = top_k_index.reshape({-1}).to(at::kLong).contiguous();
+  const int64_t rows = flat.numel();
+  TORCH_CHECK(limit > 0, "limit must be positive, got ", limit);
+  TORCH_CHECK(llmq_route_plan_supported(static_cast<int>(std::min<int64_t>(rows, INT32_MAX)),
+                                        static_cast<int>(std::min<int64_t>(num_experts, INT32_MAX))),
+              "the routing-plan kernel does not take ", rows, " rows and ", num_experts, " experts");
+  const int64_t per_expert = llmq_route_plan_blocks_per_expert(static_cast<int>(rows), static_cast<int>(limit));
+  auto order = at::empty({rows}, flat.options());
+  auto i32 = flat.options().dtype(at::kInt);
+  auto block_expert = at::empty({num_experts * per_expert}, i32);
+  auto block_row0 = at::empty({num_experts * per_expert}, i32);
+  auto block_rows = at::empty({num_experts * per_expert}, i32);
+  const c10::OptionalDeviceGuard guard(at::device_of(flat));
+  check_rc(llmq_route_plan(flat.const_data_ptr<int64_t>(), static_cast<int>(rows), static_cast<int>(num_experts),
+                           static_cast<int>(limit), order.mutable_data_ptr<int64_t>(),
+                           block_expert.mutable_data_ptr<int32_t>(), block_row0.mutable_data_ptr<int32_t>(),
+                           block_rows.mutable_data_ptr<int32_t>(), current_stream(flat)),
+           "route_plan");
+  return {order, block_expert, block_row0, block_rows};
+}
+
 // One-row gate|up Linear of a gated MLP with act(gate) * up folded into the store (see
 // llmq_wq_gemv_gate_up_silu). qweight: [2I, groups, group_size], gate rows first; returns [1, I].
 at::Tensor wq_gemv_gate_up_silu(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale,
@@ -617,6 +644,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("prologue") = 0,
         py::arg("norm_weight") = py::none(), py::arg("eps") = 0.0, py::arg("in_head_dim") = 0,
         py::arg("residual") = py::none());
+  m.def("route_plan", &route_plan, "Routing plan of the batched GEMV in one launch",
+        py::arg("top_k_index"), py::arg("num_experts"), py::arg("limit"));
+  m.def("route_plan_supported", [](int64_t rows, int64_t experts) {
+    return rows <= INT32_MAX && experts <= INT32_MAX &&
+           llmq_route_plan_supported(static_cast<int>(rows), static_cast<int>(experts)) != 0;
+  }, py::arg("rows"), py::arg("num_experts"));
   m.def("wq_gemv_gate_up_silu", &wq_gemv_gate_up_silu,
         "One-row gate|up Linear that stores act(gate) * up, optional RMSNorm prologue",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("prologue") = 0,

@@ -192,6 +192,11 @@ class KernelQuantExperts(_QuantExperts):
         return self._matmul(x, data[expert], scales[expert], real_in, padded_in)
 
     def _plan(self, top_k_index):
+        """`route_plan` in one launch when the sizes fit the kernel's single workgroup (they do wherever the
+        batched path runs: a few tokens), else the PyTorch form: the same integers either way."""
+        if self._ext.route_plan_supported(top_k_index.numel(), self.num_experts):
+            order, *plan = self._ext.route_plan(top_k_index, self.num_experts, self._batched_max_rows)
+            return order, tuple(plan)
         return route_plan(top_k_index, self.num_experts, self._batched_max_rows)
 
     def _batched(self, x, qweight, wscale, plan, real_in, padded_in):

@@ -191,3 +191,44 @@ def test_a_small_mixtral_in_kernel_mode_and_through_a_packed_file(tmp_path):
     assert torch.equal(again.gate_up_data, block.gate_up_data) and torch.equal(again.sdown, block.sdown)
     with torch.no_grad():
         assert torch.equal(loaded(ids).logits, kernel(ids).logits)
+
+
+@pytest.mark.parametrize("tokens,top_k,experts,limit", [(1, 8, 64, 8), (8, 8, 64, 8), (3, 2, 8, 8), (5, 4, 60, 3),
+                                                         (64, 8, 64, 8), (1, 1, 1, 8), (700, 8, 128, 8), (9, 2, 1000, 4)])
+def test_route_plan_kernel_matches_the_pytorch_form(tokens, top_k, experts, limit):
+    """One launch against the argsort / scatter_add / cumsum form (itself pinned to the oracle on the CPU):
+    the same order and the same blocks, for one token, many tokens, experts nobody picked, runs longer than
+    the limit and a limit that does not divide them."""
+    from llmquant.hip import load_extension
+    from llmquant.quantizers import route_plan
+
+    ext = load_extension()
+    gen = torch.Generator().manual_seed(tokens * 131 + experts)
+    index = torch.stack([torch.randperm(experts, generator=gen)[:top_k] for _ in range(tokens)]).cuda()
+    assert ext.route_plan_supported(index.numel(), experts)
+    for idx in (index, index.to(torch.int32)):
+        order, be, r0, rows = ext.route_plan(idx, experts, limit)
+        want_order, (want_be, want_r0, want_rows) = route_plan(index, experts, limit)
+        assert order.dtype == torch.int64 and be.dtype == torch.int32
+        assert torch.equal(order, want_order)
+        assert torch.equal(be, want_be) and torch.equal(r0, want_r0) and torch.equal(rows, want_rows)
+    # a skewed routing: every token picks the same experts, so their runs exceed the limit
+    same = torch.arange(top_k).repeat(tokens, 1).cuda() % experts
+    order, be, r0, rows = ext.route_plan(same, experts, limit)
+    want_order, want = route_plan(same, experts, limit)
+    assert torch.equal(order, want_order)
+    assert all(torch.equal(a, b) for a, b in zip((be, r0, rows), want))
+
+
+def test_route_plan_kernel_limits():
+    from llmquant.hip import load_extension
+
+    ext = load_extension()
+    assert not ext.route_plan_supported(8193, 64)
+    assert not ext.route_plan_supported(8, 1025)
+    with pytest.raises(RuntimeError, match="does not take"):
+        ext.route_plan(torch.zeros(8193, dtype=torch.int64, device="cuda"), 64, 8)
+    with pytest.raises(RuntimeError, match="limit must be positive"):
+        ext.route_plan(torch.zeros(8, dtype=torch.int64, device="cuda"), 64, 0)
+    order, be, r0, rows = ext.route_plan(torch.zeros(0, dtype=torch.int64, device="cuda"), 4, 8)
+    assert order.numel() == 0 and be.tolist() == [0, 1, 2, 3] and rows.tolist() == [0, 0, 0, 0]
