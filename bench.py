@@ -412,7 +412,21 @@ def other_kernels(torch):
     out["moe_batched_gemv_olmoe_int4_top8_per_layer"] = {
         "us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
         "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4), "launches": 2}
-    del gu, dn
+    # the whole experts block for one token (routing plan, both projections, weighted sum): the module's
+    # four-launch forward against the operation-by-operation form of the reference's KernelQuantExperts
+    from llmquant.core.scheme import QuantizationArgs, QuantizationScheme
+    from llmquant.quantizers import KernelQuantExperts
+
+    scheme = QuantizationScheme(weights=QuantizationArgs(4, "group", group_size=GROUP), input_activations=None)
+    block = KernelQuantExperts(gu[0], sgu, dn[0], sdn, scheme, hid, inter, torch.nn.SiLU()).to(dev)
+    hidden = torch.randn(1, hid, device=dev).to(torch.bfloat16)
+    gates = torch.rand(1, top_k, device=dev).to(torch.bfloat16)
+    fused_us = _graph_time_us(torch, lambda: [block(hidden, index, gates) for _ in range(layers)], reps=10) / layers
+    plain_us = _graph_time_us(torch, lambda: [block._forward_unfused(hidden, index, gates) for _ in range(layers)],
+                              reps=10) / layers
+    out["moe_experts_block_one_token_olmoe_int4"] = {"us": round(fused_us, 2), "launches": 4,
+                                                     "operation_by_operation_us": round(plain_us, 2)}
+    del gu, dn, block
     # integer GEMM, Llama-3-8B MLP shapes
     gemm = []
     for n, k in ((14336, 4096), (4096, 14336)):

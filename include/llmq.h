@@ -100,6 +100,30 @@ int llmq_route_plan_supported(int n_rows, int n_experts);
 int llmq_route_plan(const int64_t* expert_of_row, int n_rows, int n_experts, int limit, int64_t* order,
                     int32_t* block_expert, int32_t* block_row0, int32_t* block_rows, llmq_stream_t stream);
 
+/* llmq_wq_gemv_batched for the two projections of a gated Mixture-of-Experts block with the
+ * PyTorch steps around them folded in (KernelQuantExperts.forward, llmquant/quantizers/kernel.py:
+ * 221-253, runs them as separate kernels). Group size 128, one scale row per weight row.
+ *   x_row_stride  elements between the rows of x; 0: every row is x[0] (one token routed to several
+ *                 experts: `hidden_states[tokens_per_row]` without the gather)
+ *   act_pair != 0 qweight is [experts, 2I, G, gs] (gate rows, then up rows) and out is [n_rows, I]
+ *                 = dtype(dtype(silu(dtype(gate))) * dtype(up)): `act_fn(gate) * up` for SiLU
+ * Every row must be covered by the plan (out is written, not accumulated). */
+int llmq_wq_gemv_batched_fused(const void* x, int64_t x_row_stride, const void* qweight,
+                               const float* wscale, void* out, const int32_t* block_expert,
+                               const int32_t* block_row0, const int32_t* block_rows, int n_blocks,
+                               int n_rows, int n_experts, int N, int G, int wformat, int dtype,
+                               int act_pair, llmq_stream_t stream);
+
+/* The end of KernelQuantExperts.forward (kernel.py:247-252) in one launch:
+ *   final[t, :] = sum over the rows i routed from token t of dtype(rows_out[i, :] * weights[order[i]])
+ * accumulated in `dtype` (every addition rounded, as index_add_ on a `dtype` tensor does) in the
+ * order of the sorted rows, i.e. by ascending expert: one of the orders the reference's atomic
+ * index_add_ may take, and the same one on every run. rows_out: [n_rows, width]; order: [n_rows]
+ * from llmq_route_plan (order[i] = token * top_k + slot); weights: [n_tokens * top_k] `dtype`;
+ * final: [n_tokens, width], written in full (tokens nobody routed get zeros). */
+int llmq_moe_combine(const void* rows_out, const int64_t* order, const void* weights, void* final_out,
+                     int n_rows, int top_k, int n_tokens, int width, int dtype, llmq_stream_t stream);
+
 /* The decode-step form of llmq_wq_gemv (M = 1, group size 128): the same product with the
  * elementwise operations that surround a Linear in a Llama decoder layer folded in, so that a
  * layer is five launches instead of ~40. There is no counterpart in the reference, which leaves

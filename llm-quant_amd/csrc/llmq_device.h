@@ -258,5 +258,5 @@ bool gemv_batched_mfma_supported(const void* x, const void* qw, const float* ws,
 int gemv_batched_mfma_launch(const void* x, const void* qw, const float* ws, void* out, const int32_t* block_expert,
                              const int32_t* block_row0, const int32_t* block_rows, int n_blocks, int n_rows,
                              int n_experts, int N, int G, int out_group, int wformat, int dtype,
-                             hipStream_t stream);
+                             hipStream_t stream, int64_t x_row_stride = -1, int pair_half = 0);
 }  // namespace llmq_host

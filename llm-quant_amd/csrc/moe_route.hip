@@ -1,4 +1,5 @@
-// Routing plan of a Mixture-of-Experts layer in one launch.
+// Routing plan of a Mixture-of-Experts layer in one launch, and the weighted sum of the experts'
+// outputs per token in another.
 //
 // KernelQuantExperts._plan (llmquant/quantizers/kernel.py:176-214) builds the plan of the batched
 // GEMV from about ten PyTorch kernels (stable argsort, scatter_add, cumsum, arange arithmetic):
@@ -70,7 +71,50 @@ __global__ __launch_bounds__(kRouteThreads) void route_plan_kernel(
   }
 }
 
+// final[t, c] = the rows routed from token t, each times its routing weight, added up in sorted
+// order with every product and sum rounded to T. One thread per (token, column).
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const T* __restrict__ rows_out,
+                                                          const int64_t* __restrict__ order,
+                                                          const T* __restrict__ weights, T* __restrict__ final_out,
+                                                          const int n_rows, const int top_k, const int width) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int t = blockIdx.y;
+  if (c >= width) return;
+  float acc = 0.0f;
+  for (int i = 0; i < n_rows; ++i) {
+    const int64_t flat = order[i];  // the same address for the whole workgroup
+    if (flat / top_k != t) continue;
+    const float prod = llmq::round_through<T>(llmq::to_float(rows_out[static_cast<int64_t>(i) * width + c]) *
+                                              llmq::to_float(weights[flat]));
+    acc = llmq::round_through<T>(acc + prod);
+  }
+  final_out[static_cast<int64_t>(t) * width + c] = llmq::from_float<T>(acc);
+}
+
 }  // namespace
+
+extern "C" int llmq_moe_combine(const void* rows_out, const int64_t* order, const void* weights, void* final_out,
+                                int n_rows, int top_k, int n_tokens, int width, int dtype, llmq_stream_t stream) {
+  if (n_rows < 0 || top_k <= 0 || n_tokens < 0 || width < 0)
+    return llmq_host::fail_invalid("bad dimension rows=%d top_k=%d tokens=%d width=%d", n_rows, top_k, n_tokens, width);
+  if (n_tokens == 0 || width == 0) return 0;
+  if (n_tokens > 65535) return llmq_host::fail_invalid("at most 65535 tokens per launch, got %d", n_tokens);
+  if (!final_out || !weights || (n_rows > 0 && (!rows_out || !order))) return llmq_host::fail_invalid("null tensor pointer");
+  const dim3 grid((width + 255) / 256, n_tokens), block(256);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define LLMQ_COMBINE(T)                                                                                       \
+  hipLaunchKernelGGL(moe_combine_kernel<T>, grid, block, 0, s, static_cast<const T*>(rows_out), order,        \
+                     static_cast<const T*>(weights), static_cast<T*>(final_out), n_rows, top_k, width)
+  switch (dtype) {
+    case LLMQ_F32: LLMQ_COMBINE(float); break;
+    case LLMQ_F16: LLMQ_COMBINE(llmq::f16_t); break;
+    case LLMQ_BF16: LLMQ_COMBINE(llmq::bf16_t); break;
+    default: return llmq_host::fail_invalid("dtype code %d is not float32, float16 or bfloat16", dtype);
+  }
+#undef LLMQ_COMBINE
+  return llmq_host::check_launch("moe_combine_kernel");
+}
 
 extern "C" int llmq_route_plan_blocks_per_expert(int n_rows, int limit) {
   if (limit <= 0) return 0;

@@ -282,6 +282,69 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> route_plan(const at::
   return {order, block_expert, block_row0, block_rows};
 }
 
+// A projection of a gated MoE block over every routed expert (see llmq_wq_gemv_batched_fused).
+// x: [n_rows, K] rows in sorted order, or [1, K] with broadcast_x (every row is that one token).
+// Returns [n_rows, N], or [n_rows, N / 2] = silu(gate) * up with act_pair.
+at::Tensor wq_gemv_batched_fused(const at::Tensor& x, bool broadcast_x, int64_t n_rows, const at::Tensor& qweight,
+                                 const at::Tensor& wscale, const at::Tensor& block_expert,
+                                 const at::Tensor& block_row0, const at::Tensor& block_rows, bool act_pair) {
+  TORCH_CHECK(x.is_cuda() && qweight.is_cuda() && wscale.is_cuda() && block_expert.is_cuda() &&
+                  block_row0.is_cuda() && block_rows.is_cuda(), "all tensors must be CUDA");
+  TORCH_CHECK(qweight.dim() == 4 && qweight.is_contiguous(), "qweight must be contiguous [experts, N, groups, group_size]");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
+  const int64_t E = qweight.size(0), N = qweight.size(1), groups = qweight.size(2);
+  const int64_t group_size = packed ? qweight.size(3) * 2 : qweight.size(3);
+  TORCH_CHECK(group_size == 128, "the fused batched GEMV needs group_size 128, got ", group_size);
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.is_contiguous() && wscale.dim() == 3 &&
+                  wscale.size(0) == E && wscale.size(1) == N && wscale.size(2) == groups,
+              "wscale must be contiguous float32 [", E, ", ", N, ", ", groups, "]");
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous() && x.size(1) == groups * group_size, "x must be contiguous [rows, ",
+              groups * group_size, "]");
+  TORCH_CHECK(broadcast_x ? x.size(0) == 1 : x.size(0) == n_rows, "x has ", x.size(0), " rows, expected ",
+              broadcast_x ? 1 : n_rows);
+  for (const at::Tensor* t : {&block_expert, &block_row0, &block_rows}) {
+    TORCH_CHECK(t->scalar_type() == at::kInt && t->is_contiguous() && t->dim() == 1 &&
+                    t->numel() == block_expert.numel(), "the plan must be three contiguous int32 vectors of one length");
+  }
+  TORCH_CHECK(!act_pair || N % 16 == 0, "gate|up needs halves that are multiples of 8 rows, got ", N);
+  const int dtype = dtype_code(x, "x");
+  auto out = at::empty({n_rows, act_pair ? N / 2 : N}, x.options());
+  if (out.numel() == 0 || block_expert.numel() == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(x));
+  check_rc(llmq_wq_gemv_batched_fused(x.const_data_ptr(), broadcast_x ? 0 : x.size(1), qweight.const_data_ptr(),
+                                      wscale.const_data_ptr<float>(), out.mutable_data_ptr(),
+                                      block_expert.const_data_ptr<int32_t>(), block_row0.const_data_ptr<int32_t>(),
+                                      block_rows.const_data_ptr<int32_t>(), static_cast<int>(block_expert.numel()),
+                                      static_cast<int>(n_rows), static_cast<int>(E), static_cast<int>(N),
+                                      static_cast<int>(groups), packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype,
+                                      act_pair ? 1 : 0, current_stream(x)),
+           "wq_gemv_batched_fused");
+  return out;
+}
+
+// final[t] = sum of the rows routed from token t times their routing weights (see llmq_moe_combine).
+at::Tensor moe_combine(const at::Tensor& rows_out, const at::Tensor& order, const at::Tensor& weights,
+                       int64_t n_tokens) {
+  TORCH_CHECK(rows_out.is_cuda() && order.is_cuda() && weights.is_cuda(), "all tensors must be CUDA");
+  TORCH_CHECK(rows_out.dim() == 2 && rows_out.is_contiguous(), "rows_out must be contiguous [rows, width]");
+  TORCH_CHECK(order.scalar_type() == at::kLong && order.is_contiguous() && order.numel() == rows_out.size(0),
+              "order must be a contiguous int64 vector with one entry per row");
+  TORCH_CHECK(weights.dim() == 2 && weights.is_contiguous() && weights.size(0) == n_tokens &&
+                  weights.scalar_type() == rows_out.scalar_type() && weights.numel() == order.numel(),
+              "weights must be contiguous [tokens, top_k] of the rows' dtype, one per row");
+  const int dtype = dtype_code(rows_out, "rows_out");
+  auto out = at::empty({n_tokens, rows_out.size(1)}, rows_out.options());
+  if (out.numel() == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(rows_out));
+  check_rc(llmq_moe_combine(rows_out.const_data_ptr(), order.const_data_ptr<int64_t>(), weights.const_data_ptr(),
+                            out.mutable_data_ptr(), static_cast<int>(rows_out.size(0)),
+                            static_cast<int>(weights.size(1)), static_cast<int>(n_tokens),
+                            static_cast<int>(rows_out.size(1)), dtype, current_stream(rows_out)),
+           "moe_combine");
+  return out;
+}
+
 // One-row gate|up Linear of a gated MLP with act(gate) * up folded into the store (see
 // llmq_wq_gemv_gate_up_silu). qweight: [2I, groups, group_size], gate rows first; returns [1, I].
 at::Tensor wq_gemv_gate_up_silu(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale,
@@ -644,6 +707,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("prologue") = 0,
         py::arg("norm_weight") = py::none(), py::arg("eps") = 0.0, py::arg("in_head_dim") = 0,
         py::arg("residual") = py::none());
+  m.def("wq_gemv_batched_fused", &wq_gemv_batched_fused,
+        "Batched expert GEMV with the row gather (one token) and silu(gate) * up folded in",
+        py::arg("x"), py::arg("broadcast_x"), py::arg("n_rows"), py::arg("qweight"), py::arg("wscale"),
+        py::arg("block_expert"), py::arg("block_row0"), py::arg("block_rows"), py::arg("act_pair"));
+  m.def("moe_combine", &moe_combine, "Routing-weighted sum of the experts' rows per token",
+        py::arg("rows_out"), py::arg("order"), py::arg("weights"), py::arg("n_tokens"));
   m.def("route_plan", &route_plan, "Routing plan of the batched GEMV in one launch",
         py::arg("top_k_index"), py::arg("num_experts"), py::arg("limit"));
   m.def("route_plan_supported", [](int64_t rows, int64_t experts) {

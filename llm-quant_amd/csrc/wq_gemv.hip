@@ -520,3 +520,29 @@ extern "C" int llmq_wq_gemv_batched(const void* x, const void* qweight, const fl
 #undef LLMQ_SCALAR
   return llmq_host::fail_invalid("x must be float32, float16 or bfloat16, got dtype code %d", dtype);
 }
+
+extern "C" int llmq_wq_gemv_batched_fused(const void* x, int64_t x_row_stride, const void* qweight,
+                                         const float* wscale, void* out, const int32_t* block_expert,
+                                         const int32_t* block_row0, const int32_t* block_rows, int n_blocks,
+                                         int n_rows, int n_experts, int N, int G, int wformat, int dtype,
+                                         int act_pair, llmq_stream_t stream) {
+  if (n_blocks < 0 || n_rows < 0 || n_experts < 0 || N < 0 || G <= 0)
+    return llmq_host::fail_invalid("bad dimension blocks=%d rows=%d experts=%d N=%d G=%d", n_blocks, n_rows,
+                                   n_experts, N, G);
+  if (x_row_stride < 0) return llmq_host::fail_invalid("x_row_stride must be >= 0");
+  if (wformat != LLMQ_W_INT8 && wformat != LLMQ_W_INT4_PACKED)
+    return llmq_host::fail_invalid("unsupported weight format %d, expected 8 or 4", wformat);
+  if (act_pair && N % 16) return llmq_host::fail_invalid("gate|up needs halves that are multiples of 8 rows, got N=%d", N);
+  if (n_blocks == 0 || n_rows == 0 || N == 0 || n_experts == 0) return 0;
+  if (n_blocks > 65535) return llmq_host::fail_invalid("at most 65535 plan entries per launch, got %d", n_blocks);
+  if (!x || !qweight || !wscale || !out || !block_expert || !block_row0 || !block_rows)
+    return llmq_host::fail_invalid("null tensor pointer");
+  const int64_t weight_stride = static_cast<int64_t>(N) * G * 128 * (wformat == LLMQ_W_INT8 ? 2 : 1) / 2;
+  if (weight_stride % 16 || (x_row_stride * (dtype == LLMQ_F32 ? 4 : 2)) % 16 ||
+      !llmq_host::gemv_batched_mfma_supported(x, qweight, wscale, G, 128, wformat))
+    return llmq_host::fail_invalid("the fused batched GEMV needs group size 128, a multiple of 4 groups and "
+                                   "16-byte aligned operands and rows");
+  return llmq_host::gemv_batched_mfma_launch(x, qweight, wscale, out, block_expert, block_row0, block_rows, n_blocks,
+                                             n_rows, n_experts, N, G, 0, wformat, dtype,
+                                             static_cast<hipStream_t>(stream), x_row_stride, act_pair ? N / 2 : 0);
+}

@@ -64,6 +64,7 @@ struct MfmaArgs {
   // is eight gate rows and the eight up rows that go with them, n_tiles = pair_half / 8, and out is
   // [pair_half]: act(gate) * up as the SiLU prologue would compute it from the two outputs
   int pair_half;
+  int64_t x_row_stride;      // elements between activation rows; < 0: the rows are packed (the row's width)
   int attn_splits;           // LLMQ_PRO_ATTN_MERGE: x is the split-attention records, this many per head
   int attn_head_dim;         // ... of heads this wide
 };
@@ -133,6 +134,7 @@ struct Prologue {
   int in_head_dim;
   int attn_splits = 0;
   int attn_head_dim = 0;
+  int64_t x_row_stride = -1;  // elements between rows of x; < 0: packed
 };
 
 // The activation as integers, whole workgroup, into LDS: per (row m, group g) the digits of
@@ -148,11 +150,13 @@ struct Prologue {
 // 8 items cover a group.
 template <bool HALF> struct StageGeometry {
   int real_per_group, lg, items, k_real;
+  int64_t row_stride;
   __device__ __forceinline__ StageGeometry(int G, const Prologue& pro, int m_valid) {
     real_per_group = pro.in_head_dim > 0 ? pro.in_head_dim : kGroup;
     lg = HALF ? 3 : 4;
     items = (m_valid * G) << lg;
     k_real = G * real_per_group;
+    row_stride = pro.x_row_stride >= 0 ? pro.x_row_stride : k_real;
   }
 };
 template <int M> struct StageItem {
@@ -168,7 +172,7 @@ template <int M> struct StageItem {
     g = mg - m * G;
     // beyond real_per_group: the zero padding of a head group
     real = active && tq * 8 < geo.real_per_group && m < m_valid;
-    src = static_cast<int64_t>(m) * geo.k_real + g * geo.real_per_group + tq * 8;
+    src = m * geo.row_stride + g * geo.real_per_group + tq * 8;
   }
 };
 
@@ -445,7 +449,8 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
     }
   };
 
-  const Prologue pro{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits, a.attn_head_dim};
+  const Prologue pro{a.prologue, a.norm_weight, a.eps, a.in_head_dim, a.attn_splits, a.attn_head_dim,
+                     a.x_row_stride};
   const StageFirst first = stage_first<T, M, HALF>(static_cast<const T*>(a.x), G, pro, m_valid);
   // the first tile's weights: in flight while the activation is prepared, requested right after the
   // activation's own first loads
@@ -523,6 +528,14 @@ __device__ __forceinline__ void ksplit_body(const MfmaArgs& a, unsigned char* sm
         total += __shfl_xor(total, 32, kWave);
         if constexpr (M == 1) {
           store_row<T>(a, out, tile, jj, total, ws == 0);
+        } else if (a.pair_half > 0) {
+          // row r of several, gate|up pairs: see store_row
+          const float up = dpp<kDppRor8>(total);
+          if (ws == 0 && jj < 8 && r < m_valid) {
+            const float gv = round_through<T>(total), uv = round_through<T>(up);
+            const float silu = gv / (1.0f + expf(-gv));
+            out[static_cast<int64_t>(r) * a.pair_half + tile * 8 + jj] = from_float<T>(round_through<T>(silu) * uv);
+          }
         } else {
           const int n = tile * kTileRows + jj;
           if (ws == 0 && n < a.N && r < m_valid) {
@@ -586,21 +599,22 @@ __global__ __launch_bounds__(MAXT) void wq_gemv_mfma_batched_kernel(MfmaArgs a, 
   if (e < 0 || e >= plan.n_experts || row0 < 0 || row0 + rows > plan.n_rows) return;  // not a valid run
   a.qw += e * plan.weight_stride;
   a.ws += e * plan.scale_stride;
-  const int64_t k_total = static_cast<int64_t>(a.G) * kGroup;
+  const int64_t x_stride = a.x_row_stride >= 0 ? a.x_row_stride : static_cast<int64_t>(a.G) * kGroup;
+  const int64_t out_stride = a.pair_half > 0 ? a.pair_half : a.N;
   const T* x = static_cast<const T*>(a.x);
   T* out = static_cast<T*>(a.out);
   if (rows == 1) {
     // the decode case (one token: every routed expert has one row): the single-row body, which
     // stages a quarter of the fragments and accumulators of the four-row one
-    a.x = x + row0 * k_total;
-    a.out = out + static_cast<int64_t>(row0) * a.N;
+    a.x = x + row0 * x_stride;
+    a.out = out + row0 * out_stride;
     ksplit_body<T, BITS, 1, MULTI>(a, smem, blockIdx.x, gridDim.x, 1);
     return;
   }
   for (int done = 0; done < rows; done += 4) {
     if (done > 0) __syncthreads();  // the previous pass is done with the LDS
-    a.x = x + (row0 + done) * k_total;
-    a.out = out + static_cast<int64_t>(row0 + done) * a.N;
+    a.x = x + (row0 + done) * x_stride;
+    a.out = out + (row0 + done) * out_stride;
     ksplit_body<T, BITS, 4, MULTI>(a, smem, blockIdx.x, gridDim.x, min(4, rows - done));
   }
 }
@@ -946,6 +960,7 @@ int launch_typed(const void* x, const void* qw, const float* ws, void* out, int 
   a.in_head_dim = ops.in_head_dim; a.residual = ops.residual;
   a.attn_splits = ops.attn_splits; a.attn_head_dim = ops.attn_head_dim;
   a.pair_half = ops.pair_half;
+  a.x_row_stride = -1;
   // (paired: N = 2 * pair_half weight rows, eight gate + eight up rows to a tile, the same count)
   a.n_tiles = (N + kTileRows - 1) / kTileRows;
   a.row_bytes = G * kGroup * BITS / 8;
@@ -1094,10 +1109,11 @@ bool gemv_batched_mfma_supported(const void* x, const void* qw, const float* ws,
 int gemv_batched_mfma_launch(const void* x, const void* qw, const float* ws, void* out, const int32_t* block_expert,
                              const int32_t* block_row0, const int32_t* block_rows, int n_blocks, int n_rows,
                              int n_experts, int N, int G, int out_group, int wformat, int dtype,
-                             hipStream_t stream) {
+                             hipStream_t stream, int64_t x_row_stride, int pair_half) {
   MfmaArgs a{};
   a.x = x; a.qw = static_cast<const uint8_t*>(qw); a.ws = ws; a.out = out;
   a.N = N; a.G = G; a.out_group = out_group;
+  a.x_row_stride = x_row_stride; a.pair_half = pair_half;
   a.n_tiles = (N + kTileRows - 1) / kTileRows;
   a.row_bytes = G * kGroup * (wformat == LLMQ_W_INT8 ? 8 : 4) / 8;
   const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;

@@ -83,6 +83,10 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_kv_decode_attention.argtypes = [c_p] * 8 + [c_f] + [c_int] * 6 + [c_p]
     lib.llmq_wq_gemv_fused.argtypes = [c_p] * 4 + [c_int] * 6 + [c_p, c_f, c_int, c_p, c_p]
     lib.llmq_wq_gemv_fused.restype = c_int
+    lib.llmq_wq_gemv_batched_fused.argtypes = [c_p, c_i64, c_p, c_p, c_p, c_p, c_p, c_p] + [c_int] * 8 + [c_p]
+    lib.llmq_wq_gemv_batched_fused.restype = c_int
+    lib.llmq_moe_combine.argtypes = [c_p] * 4 + [c_int] * 5 + [c_p]
+    lib.llmq_moe_combine.restype = c_int
     lib.llmq_route_plan_blocks_per_expert.argtypes = [c_int, c_int]
     lib.llmq_route_plan_blocks_per_expert.restype = c_int
     lib.llmq_route_plan_supported.argtypes = [c_int, c_int]

@@ -153,9 +153,19 @@ class KernelQuantExperts(_QuantExperts):
         self._down_padded = self.down_data.shape[2] * self.down_data.shape[3] * per_byte
         self._weight_args = self.scheme.weights
         self._ext = load_extension()
+        # The fused forward folds act_fn(gate) * up into the gate|up launch, which is written for SiLU
+        # (MixtralExperts / OlmoeExperts); anything else keeps the operation-by-operation form.
+        self._act_is_silu = self._probe_silu()
         self._gemv = self._ext.wq_gemv
         self._gemv_batched = self._ext.wq_gemv_batched
         self._batched_max_rows = self._ext.wq_gemv_batched_max_rows()
+
+    def _probe_silu(self) -> bool:
+        probe = torch.linspace(-6.0, 6.0, 25)
+        try:
+            return bool(torch.equal(self.act_fn(probe), nn.functional.silu(probe)))
+        except Exception:
+            return False
 
     @property
     def qgate_up(self) -> torch.Tensor:
@@ -204,11 +214,43 @@ class KernelQuantExperts(_QuantExperts):
             qweight = pack_int4(qweight)
         return self._gemv_batched(self._pad(x, real_in, padded_in), qweight, wscale, *plan, 0)
 
+    def _fusable(self, hidden_states, top_k_index, top_k_weights) -> bool:
+        """Whether the four-launch forward applies: SiLU experts, group size 128 with rows of a multiple of
+        four groups and no input padding (the matrix-core kernels), a routing problem the plan kernel takes,
+        routing weights in the activations' dtype."""
+        groups_ok = self.gate_up_data.shape[2] % 4 == 0 and self.down_data.shape[2] % 4 == 0
+        return (self._act_is_silu and self._weight_args.group_size == 128 and groups_ok
+                and self._gate_up_padded == self.hidden_dim and self._down_padded == self.intermediate_dim
+                and self.intermediate_dim % 8 == 0
+                and hidden_states.dim() == 2 and hidden_states.is_contiguous()
+                and top_k_weights.dtype == hidden_states.dtype and top_k_weights.shape == top_k_index.shape
+                and self._ext.route_plan_supported(top_k_index.numel(), self.num_experts))
+
+    def _forward_fused(self, hidden_states, top_k_index, top_k_weights):
+        """Plan, gate|up (storing act(gate) * up), down, weighted sum per token: four launches. With one
+        token every row reads that token's activation, so `hidden_states[tokens_per_row]` is not formed."""
+        ext = self._ext
+        tokens, top_k = hidden_states.shape[0], top_k_index.shape[-1]
+        rows = top_k_index.numel()
+        with torch.no_grad():
+            order, *plan = ext.route_plan(top_k_index, self.num_experts, self._batched_max_rows)
+        one = tokens == 1
+        x = hidden_states if one else hidden_states[order // top_k]
+        act = ext.wq_gemv_batched_fused(x, one, rows, self.gate_up_data, self.sgate_up, *plan, True)
+        out = ext.wq_gemv_batched_fused(act, False, rows, self.down_data, self.sdown, *plan, False)
+        return ext.moe_combine(out, order, top_k_weights.contiguous(), tokens)
+
     def forward(self, hidden_states, top_k_index, top_k_weights):
         # An expert cannot be picked twice by one token, so no expert sees more rows than there
         # are tokens: the shape alone says whether the batched kernel's run length suffices.
         if hidden_states.shape[0] > self._batched_max_rows:
             return self._each_hit_expert(hidden_states, top_k_index, top_k_weights)
+        if self._fusable(hidden_states, top_k_index, top_k_weights):
+            return self._forward_fused(hidden_states, top_k_index, top_k_weights)
+        return self._forward_unfused(hidden_states, top_k_index, top_k_weights)
+
+    def _forward_unfused(self, hidden_states, top_k_index, top_k_weights):
+        """KernelQuantExperts.forward of the reference, operation by operation."""
         top_k = top_k_index.shape[-1]
         with torch.no_grad():
             order, plan = self._plan(top_k_index)

@@ -232,3 +232,54 @@ def test_route_plan_kernel_limits():
         ext.route_plan(torch.zeros(8, dtype=torch.int64, device="cuda"), 64, 0)
     order, be, r0, rows = ext.route_plan(torch.zeros(0, dtype=torch.int64, device="cuda"), 4, 8)
     assert order.numel() == 0 and be.tolist() == [0, 1, 2, 3] and rows.tolist() == [0, 0, 0, 0]
+
+
+@pytest.mark.parametrize("bits", ["int8", "int4"])
+@pytest.mark.parametrize("tokens", [1, 3, 8])
+def test_fused_forward_pieces_equal_the_operation_by_operation_form(ext, bits, tokens):
+    """gate|up with act(gate) * up in its store, the one-token form that skips the row gather, and the
+    weighted sum per token, each against the PyTorch steps of KernelQuantExperts.forward."""
+    _, quant, _, cfg = kernel_block(bits)
+    top_k = cfg.num_experts_per_tok
+    torch.manual_seed(10 + tokens)
+    hidden = torch.randn(tokens, cfg.hidden_size, device="cuda", dtype=torch.bfloat16)
+    index, weights = routing(tokens, cfg.num_local_experts, top_k, seed=tokens)
+    index, weights = index.cuda(), weights.to(torch.bfloat16).cuda()
+    assert quant._fusable(hidden, index, weights)
+    with torch.no_grad():
+        order, plan = quant._plan(index)
+        rows = hidden[order // top_k]
+        plain = quant._batched(rows, quant.gate_up_data, quant.sgate_up, plan, quant.hidden_dim, quant._gate_up_padded)
+        gate, up = plain.chunk(2, dim=-1)
+        want_act = torch.nn.functional.silu(gate) * up
+        act = ext.wq_gemv_batched_fused(rows, False, rows.shape[0], quant.gate_up_data, quant.sgate_up, *plan, True)
+        assert torch.equal(act, want_act)
+        if tokens == 1:
+            again = ext.wq_gemv_batched_fused(hidden, True, rows.shape[0], quant.gate_up_data, quant.sgate_up, *plan, True)
+            assert torch.equal(again, want_act)
+        out = ext.wq_gemv_batched_fused(act, False, rows.shape[0], quant.down_data, quant.sdown, *plan, False)
+        assert torch.equal(out, quant._batched(act, quant.down_data, quant.sdown, plan, quant.intermediate_dim,
+                                               quant._down_padded))
+        # index_add_ on a bf16 tensor rounds after every addition, in no fixed order; the kernel takes the
+        # order of the sorted rows
+        final = torch.zeros_like(hidden)
+        flat_w = weights.reshape(-1)
+        for i, src in enumerate(order.tolist()):
+            final[src // top_k] = final[src // top_k] + out[i] * flat_w[src]
+        got = ext.moe_combine(out, order, weights, tokens)
+        assert torch.equal(got, final)
+        assert torch.equal(quant._forward_fused(hidden, index, weights), final)
+        loose = quant._forward_unfused(hidden, index, weights)
+        assert rel_l2(to_np(got), to_np(loose)) <= 1e-2
+
+
+def test_experts_that_are_not_silu_keep_the_unfused_forward(ext):
+    _, quant, _, cfg = kernel_block("int8")
+    assert quant._probe_silu()
+    quant.act_fn = torch.nn.GELU()
+    quant._act_is_silu = quant._probe_silu()
+    hidden = torch.randn(2, cfg.hidden_size, device="cuda", dtype=torch.bfloat16)
+    index, weights = routing(2, cfg.num_local_experts, cfg.num_experts_per_tok, seed=3)
+    index, weights = index.cuda(), weights.to(torch.bfloat16).cuda()
+    assert not quant._fusable(hidden, index, weights)
+    assert torch.isfinite(quant(hidden, index, weights)).all()
