@@ -84,7 +84,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const T* __restrict__ 
   float acc = 0.0f;
   for (int i = 0; i < n_rows; ++i) {
     const int64_t flat = order[i];  // the same address for the whole workgroup
-    if (flat / top_k != t) continue;
+    // (an entry that is not a row index of this problem names no token here: skipped)
+    if (flat < 0 || flat / top_k != t) continue;
     const float prod = llmq::round_through<T>(llmq::to_float(rows_out[static_cast<int64_t>(i) * width + c]) *
                                               llmq::to_float(weights[flat]));
     acc = llmq::round_through<T>(acc + prod);
