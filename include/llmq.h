@@ -233,7 +233,10 @@ int llmq_kv_rope_append_attend(const void* qkv, const void* cos_table, const voi
  * `partials`, llmq_kv_attend_partials_floats(...) floats, 16-byte aligned. The records are merged
  * by llmq_kv_attend_merge (out: [q_heads * head_dim] `dtype`), or for free by the GEMV that
  * consumes the attention output: llmq_wq_gemv_attn_merge is llmq_wq_gemv_fused whose activation is
- * dtype(merge(partials)) (o_proj of a decoder layer; in_head_dim / residual as there). */
+ * dtype(merge(partials)) (o_proj of a decoder layer; in_head_dim / residual as there).
+ * With n_splits >= 32 and q_heads / kv_heads a multiple of 4 a workgroup takes four query heads of
+ * a kv head together, so every cache row is read and dequantized once for the four (long caches:
+ * the step is bound by that arithmetic); the records and their layout are the same. */
 size_t llmq_kv_attend_partials_floats(int q_heads, int head_dim, int n_splits);
 int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos_table, const void* sin_table,
                                      void* k_codes, void* v_codes, float* k_scale, float* v_scale,

@@ -176,7 +176,7 @@ __device__ __forceinline__ AttnPrefetch<BITS, DPL> attn_prefetch(const uint8_t* 
 // operands of steps 0 .. NPRE-1 (token rows min(t_first + i t_step + tk, t_clamp)), requested by the
 // caller before it knew t_end; every row up to t_clamp must be readable, what lies at or beyond
 // t_end is loaded and dropped.
-// ROW_PARTIALS (REP == 1): instead of the merged wave result, every lane returns the wave's maximum
+// ROW_PARTIALS: instead of the merged wave result, every lane returns the wave's maximum
 // in m and, in l / o, the sums over the four quads of its own row of 16 lanes that share its dq,
 // already scaled to that maximum: the caller adds the four rows (lanes 0..3, 16..19, 32..35, 48..51).
 // One exponential and two DPP additions per value, against a rescaling exchange per step and two
@@ -242,10 +242,15 @@ __device__ __forceinline__ void attend_range(const float (*qf)[D / 4], const uin
         const float m_new = fmaxf(m[h], s[h]);
         const float corr = exp2f(m[h] - m_new);  // exp2f(-inf) == 0 on the first token
         p[h] = exp2f(s[h] - m_new);
-        l[h] = l[h] * corr + p[h];
-        m[h] = m_new;
+        // Once the running maxima have settled no lane of the wave raises its own any more and the
+        // correction is exactly 1 everywhere: the rescaling is skipped (same bits, fewer multiplies).
+        if (__builtin_amdgcn_ballot_w64(m_new != m[h]) != 0) {
+          l[h] = l[h] * corr;
 #pragma unroll
-        for (int i = 0; i < DPL; ++i) o[h][i] *= corr;
+          for (int i = 0; i < DPL; ++i) o[h][i] *= corr;
+        }
+        l[h] = l[h] + p[h];
+        m[h] = m_new;
       }
 #pragma unroll
       for (int i = 0; i < DPL; ++i) {
@@ -258,20 +263,22 @@ __device__ __forceinline__ void attend_range(const float (*qf)[D / 4], const uin
   }
 
   if constexpr (ROW_PARTIALS) {
-    static_assert(REP == 1, "row partials are kept for one head per wave");
-    const float m_wave = group_max<kWave>(m[0]);
-    const float a = m[0] == -INFINITY ? 0.0f : exp2f(m[0] - m_wave);
-    l[0] *= a;
-    l[0] += dpp<kDppRor4>(l[0]);
-    l[0] += dpp<kDppRor8>(l[0]);
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) {
-      float v = o[0][i] * a;
-      v += dpp<kDppRor4>(v);
-      v += dpp<kDppRor8>(v);
-      o[0][i] = v;
+    for (int h = 0; h < REP; ++h) {
+      const float m_wave = group_max<kWave>(m[h]);
+      const float a = m[h] == -INFINITY ? 0.0f : exp2f(m[h] - m_wave);
+      l[h] *= a;
+      l[h] += dpp<kDppRor4>(l[h]);
+      l[h] += dpp<kDppRor8>(l[h]);
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        float v = o[h][i] * a;
+        v += dpp<kDppRor4>(v);
+        v += dpp<kDppRor8>(v);
+        o[h][i] = v;
+      }
+      m[h] = m_wave;
     }
-    m[0] = m_wave;
     return;
   }
   // ---- merge the 16 quads of the wave (lanes with the same dq) ----------------------------------------
@@ -546,7 +553,11 @@ constexpr int kSplitThreads = kSplitWaves * kWave;
 constexpr int kSplitSlab = kSplitWaves * kTokPerIter;  // 64 tokens per workgroup step
 constexpr int kSplitPrefetch = 2;  // steps of cache rows a wave requests before it knows the position
 
-template <typename T, int BITS, int D>
+// HEADS: query heads of one kv head that a workgroup takes together (1, or 4 under grouped-query
+// attention with long caches). Every cache row is then read and dequantized once for the four of
+// them: beyond a few thousand tokens the step is bound by exactly that arithmetic, which one
+// workgroup per query head repeats q_heads / kv_heads times.
+template <typename T, int BITS, int D, int HEADS>
 __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_kernel(
     const T* __restrict__ qkv, const T* __restrict__ cos_table, const T* __restrict__ sin_table,
     uint8_t* __restrict__ k_codes, uint8_t* __restrict__ v_codes, float* __restrict__ k_scale,
@@ -556,16 +567,16 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
   constexpr int ROWB = BITS == 8 ? D : D / 2;
   constexpr int REC = D + 2;                    // per-wave record in LDS
   constexpr int GREC = D + kAttnRecordHeader;  // per-split record in global memory
-  __shared__ float s_q[D];
+  __shared__ float s_q[HEADS][D];
   __shared__ float s_new[2][D];
-  __shared__ float s_rec[kSplitWaves][4][REC];  // per wave and row of 16 lanes: (wave max, sum, output)
-  __shared__ float s_new_score;                 // the new token's score (last split), else -inf
+  __shared__ float s_rec[kSplitWaves][4][HEADS][REC];  // per wave and row of 16 lanes: (wave max, sum, output)
+  __shared__ float s_new_score[HEADS];                 // the new token's scores (last split), else -inf
 
-  const int qh = blockIdx.x, split = blockIdx.y, n_splits = gridDim.y;
+  const int qh0 = blockIdx.x * HEADS, split = blockIdx.y, n_splits = gridDim.y;  // heads qh0 .. qh0 + HEADS - 1
   const bool last_split = split == n_splits - 1;
-  const int rep = q_heads / kv_heads;
-  const int kvh = qh / rep;
-  const bool writer = last_split && qh % rep == 0;
+  const int rep = q_heads / kv_heads;  // a multiple of HEADS
+  const int kvh = qh0 / rep;
+  const bool writer = last_split && qh0 % rep == 0;
   const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
   const int tk = lane >> 2, dq = lane & 3;
 
@@ -588,11 +599,13 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
   const T* cos_row = cos_table + static_cast<int64_t>(pos) * D;
   const T* sin_row = sin_table + static_cast<int64_t>(pos) * D;
 
-  // ---- phase A: wave 0 rotates the query; in the last split wave 1 / 2 prepare the new K / V ----------
-  if (wv == 0) {
-    const T* q = qkv + static_cast<int64_t>(qh) * D;
-    for (int i = lane; i < D; i += kWave) s_q[i] = rope_element<T, D>(q, cos_row, sin_row, i) * sm_scale_log2;
-  } else if (wv <= 2 && last_split) {
+  // ---- phase A: the waves rotate the query heads (one head: wave 0); in the last split wave 1 / 2 also
+  // prepare the new K / V ----------------------------------------------------------------------------
+  for (int h = wv; h < HEADS; h += kSplitWaves) {
+    const T* q = qkv + static_cast<int64_t>(qh0 + h) * D;
+    for (int i = lane; i < D; i += kWave) s_q[h][i] = rope_element<T, D>(q, cos_row, sin_row, i) * sm_scale_log2;
+  }
+  if (wv >= 1 && wv <= 2 && last_split) {
     const bool is_v = wv == 2;
     const T* src = qkv + (static_cast<int64_t>(q_heads) + (is_v ? kv_heads : 0) + kvh) * D;
     const float qmax = static_cast<float>((1 << (BITS - 1)) - 1);
@@ -627,50 +640,58 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
   __syncthreads();
 
   // ---- phase B: this split's slabs of tokens 0 .. pos-1, and (last split) token pos from LDS ------------
-  float qf[1][DPL];
+  float qf[HEADS][DPL];
 #pragma unroll
-  for (int i = 0; i < DPL; ++i) qf[0][i] = s_q[dq * DPL + i];
-  float m[1], l[1], o[1][DPL];
-  attend_range<T, BITS, D, 1, kSplitPrefetch, true>(qf, kbase, vbase, ksc, vsc, t_mine, pos, t_step, tk, dq, m, l, o,
-                                                    first, t_max - 1);
+  for (int h = 0; h < HEADS; ++h)
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) qf[h][i] = s_q[h][dq * DPL + i];
+  float m[HEADS], l[HEADS], o[HEADS][DPL];
+  attend_range<T, BITS, D, HEADS, kSplitPrefetch, true>(qf, kbase, vbase, ksc, vsc, t_mine, pos, t_step, tk, dq, m, l,
+                                                        o, first, t_max - 1);
   if (wv == kSplitWaves - 1) {
-    // the new token is a record of its own: score here, its value is s_new[1]
-    float sc = 0.0f;
+    // the new token is a record of its own: scores here, its value is s_new[1]
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) sc = fmaf(qf[0][i], s_new[0][dq * DPL + i], sc);
-    sc += dpp<kDppXor1>(sc);
-    sc += dpp<kDppXor2>(sc);
-    if (lane == 0) s_new_score = last_split ? sc : -INFINITY;
+    for (int h = 0; h < HEADS; ++h) {
+      float sc = 0.0f;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) sc = fmaf(qf[h][i], s_new[0][dq * DPL + i], sc);
+      sc += dpp<kDppXor1>(sc);
+      sc += dpp<kDppXor2>(sc);
+      if (lane == 0) s_new_score[h] = last_split ? sc : -INFINITY;
+    }
   }
   if ((tk & 3) == 0) {
     const int row = lane >> 4;
-    if (dq == 0) {
-      s_rec[wv][row][0] = m[0];
-      s_rec[wv][row][1] = l[0];
-    }
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) s_rec[wv][row][2 + dq * DPL + i] = o[0][i];
+    for (int h = 0; h < HEADS; ++h) {
+      if (dq == 0) {
+        s_rec[wv][row][h][0] = m[h];
+        s_rec[wv][row][h][1] = l[h];
+      }
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) s_rec[wv][row][h][2 + dq * DPL + i] = o[h][i];
+    }
   }
   __syncthreads();
-  if (threadIdx.x < D) {
-    const int d = threadIdx.x;
-    const float new_score = s_new_score;
+  for (int item = threadIdx.x; item < HEADS * D; item += kSplitThreads) {
+    const int h = item / D, d = item - h * D;
+    const float new_score = s_new_score[h];
     float mm = new_score;
 #pragma unroll
-    for (int w = 0; w < kSplitWaves; ++w) mm = fmaxf(mm, s_rec[w][0][0]);
+    for (int w = 0; w < kSplitWaves; ++w) mm = fmaxf(mm, s_rec[w][0][h][0]);
     float ll = 0.0f, oo = 0.0f;
 #pragma unroll
     for (int w = 0; w < kSplitWaves; ++w) {
-      const float a = s_rec[w][0][0] == -INFINITY ? 0.0f : exp2f(s_rec[w][0][0] - mm);
-      ll += ((s_rec[w][0][1] + s_rec[w][1][1]) + (s_rec[w][2][1] + s_rec[w][3][1])) * a;
-      oo += ((s_rec[w][0][2 + d] + s_rec[w][1][2 + d]) + (s_rec[w][2][2 + d] + s_rec[w][3][2 + d])) * a;
+      const float a = s_rec[w][0][h][0] == -INFINITY ? 0.0f : exp2f(s_rec[w][0][h][0] - mm);
+      ll += ((s_rec[w][0][h][1] + s_rec[w][1][h][1]) + (s_rec[w][2][h][1] + s_rec[w][3][h][1])) * a;
+      oo += ((s_rec[w][0][h][2 + d] + s_rec[w][1][h][2 + d]) + (s_rec[w][2][h][2 + d] + s_rec[w][3][h][2 + d])) * a;
     }
     if (new_score != -INFINITY) {
       const float b = exp2f(new_score - mm);
       ll += b;
       oo = fmaf(b, s_new[1][d], oo);
     }
-    float* rec = partials + (static_cast<int64_t>(qh) * n_splits + split) * GREC;
+    float* rec = partials + (static_cast<int64_t>(qh0 + h) * n_splits + split) * GREC;
     if (d == 0) {
       rec[0] = mm;
       rec[1] = ll;
@@ -963,13 +984,29 @@ extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos
     return llmq_host::fail_invalid("cache code and record pointers must be 16-byte aligned");
   const float scale_log2 = sm_scale * 1.4426950408889634f;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(q_heads, n_splits), block(kSplitThreads);
+  // Four query heads of a kv head per workgroup once the caller asks for 32 splits or more (it does
+  // for caches beyond ~12 K tokens): measured at 32 splits, ctx 8 K / 16 K / 32 K: 9.7 / 13.6 / 20.9 us
+  // per layer against 13.0 / 19.7 / 32.0 us for one head per workgroup at its best split count; below
+  // that the one-head form, which puts more workgroups on the chip, is as fast or faster.
+  const int rep_heads = q_heads / kv_heads;
+  const bool grouped = rep_heads % 4 == 0 && n_splits >= 32;
+  const dim3 grid(grouped ? q_heads / 4 : q_heads, n_splits), block(kSplitThreads);
 #define LLMQ_SPLIT(T, B, D)                                                                            \
-  hipLaunchKernelGGL((kv_rope_append_attend_split_kernel<T, B, D>), grid, block, 0, s,                  \
-                     static_cast<const T*>(qkv), static_cast<const T*>(cos_table),                      \
-                     static_cast<const T*>(sin_table), static_cast<uint8_t*>(k_codes),                  \
-                     static_cast<uint8_t*>(v_codes), k_scale, v_scale, partials, pos_dev, scale_log2,   \
-                     q_heads, kv_heads, t_max)
+  do {                                                                                                 \
+    if (grouped) {                                                                                     \
+      hipLaunchKernelGGL((kv_rope_append_attend_split_kernel<T, B, D, 4>), grid, block, 0, s,          \
+                         static_cast<const T*>(qkv), static_cast<const T*>(cos_table),                 \
+                         static_cast<const T*>(sin_table), static_cast<uint8_t*>(k_codes),             \
+                         static_cast<uint8_t*>(v_codes), k_scale, v_scale, partials, pos_dev,          \
+                         scale_log2, q_heads, kv_heads, t_max);                                        \
+    } else {                                                                                           \
+      hipLaunchKernelGGL((kv_rope_append_attend_split_kernel<T, B, D, 1>), grid, block, 0, s,          \
+                         static_cast<const T*>(qkv), static_cast<const T*>(cos_table),                 \
+                         static_cast<const T*>(sin_table), static_cast<uint8_t*>(k_codes),             \
+                         static_cast<uint8_t*>(v_codes), k_scale, v_scale, partials, pos_dev,          \
+                         scale_log2, q_heads, kv_heads, t_max);                                        \
+    }                                                                                                  \
+  } while (0)
 #define LLMQ_SPLIT_BD(T)                                                                               \
   if (bits == 8) { if (head_dim == 64) LLMQ_SPLIT(T, 8, 64); else LLMQ_SPLIT(T, 8, 128); }             \
   else { if (head_dim == 64) LLMQ_SPLIT(T, 4, 64); else LLMQ_SPLIT(T, 4, 128); }                       \

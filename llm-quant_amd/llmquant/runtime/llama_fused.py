@@ -61,7 +61,14 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         super().__init__(model, max_len, kv_bits, exact_prefill)
         self._ext = load_extension()
         if attn_splits is None:
-            attn_splits = max(1, min(32, max(256 // max(self.q_heads, 1), (max_len + 2047) // 2048 * 4)))
+            # one workgroup per CU at least, four more splits per 2048 tokens of cache up to 16; from
+            # ~12 K tokens on 32 splits, where the kernel takes the four query heads of a kv head
+            # together (grouped-query models) and dequantizes every cache row once for all of them
+            grouped = self.kv_heads > 0 and (self.q_heads // self.kv_heads) % 4 == 0
+            if max_len >= 12288 and grouped:
+                attn_splits = 32
+            else:
+                attn_splits = max(1, 256 // max(self.q_heads, 1), min(16, (max_len + 2047) // 2048 * 4))
         self.attn_splits = int(attn_splits)
         self._partials = torch.zeros(self._ext.kv_attend_partials_floats(self.q_heads, self.head_dim,
                                                                          self.attn_splits),
