@@ -262,7 +262,9 @@ def test_fused_runtime_equals_the_unfused_one():
 
 @pytest.mark.parametrize("bits", [8, 4])
 @pytest.mark.parametrize("q_heads,kv_heads,d", [(32, 8, 64), (8, 2, 128)])
-@pytest.mark.parametrize("pos,splits", [(0, 8), (5, 8), (63, 2), (64, 3), (700, 8), (2047, 16), (300, 1), (1500, 2)])
+# (32 splits and more: four query heads of a kv head share a workgroup)
+@pytest.mark.parametrize("pos,splits", [(0, 8), (5, 8), (63, 2), (64, 3), (700, 8), (2047, 16), (300, 1), (1500, 2),
+                                        (0, 32), (77, 32), (2047, 32), (1900, 40)])
 def test_split_attention_and_its_merge(ext, bits, q_heads, kv_heads, d, pos, splits):
     """Tokens of a head spread over `splits` workgroups: the cache ends up identical to the
     one-workgroup launch, the merged output agrees with it (another summation order), and the GEMV
