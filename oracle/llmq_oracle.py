@@ -23,9 +23,10 @@ What pins each function (the tests that do so live in tests/test_oracle_*.py):
                        (reference tests/test_moe.py:310-333)
   moe_experts_real     per expert == real_linear; tracks transformers' MixtralExperts in bf16
                        (reference tests/test_moe.py:77-117, 336-345)
-  gqa_decode_attention textbook softmax attention in float64 -- parity unpinned against the
-                       reference itself: the reference delegates attention to HF transformers
-                       and holds no test of its arithmetic.
+  gqa_decode_attention the reference delegates attention to HF transformers and holds no test of its
+                       arithmetic; pinned against the routines it delegates to (transformers'
+                       eager_attention_forward and torch's scaled_dot_product_attention, grouped-query,
+                       on the CPU) and by closed forms (uniform scores -> mean of V, one dominant key).
 """
 
 from __future__ import annotations

@@ -344,6 +344,37 @@ def test_attention_reduces_to_a_uniform_average():
     assert np.allclose(out[1], v[0, 2]) and np.allclose(out[2], v[1, 2])
 
 
+def test_attention_matches_the_library_routines_the_reference_delegates_to():
+    """The reference hands attention to transformers (LlamaAttention -> eager_attention_forward, or
+    torch's scaled_dot_product_attention): the oracle must agree with both on grouped-query inputs
+    where every kv head differs, at a scale other than 1 and with unequal head counts, so a wrong
+    head-to-kv-head map (h % kv_heads instead of h // rep), a dropped scale or a transposed operand
+    shows. fp32 library arithmetic against the float64 oracle: 1e-5."""
+    import types
+
+    import torch
+    from transformers.models.llama.modeling_llama import eager_attention_forward
+
+    rng = np.random.default_rng(3)
+    hq, hkv, t, d = 12, 3, 37, 16
+    q = rng.standard_normal((hq, d)).astype(np.float32)
+    k = rng.standard_normal((hkv, t, d)).astype(np.float32) * 2.0
+    v = rng.standard_normal((hkv, t, d)).astype(np.float32)
+    scale = 0.31
+    mine = oracle.gqa_decode_attention(q, k, v, scale, "f32")
+
+    tq, tk, tv = torch.from_numpy(q)[None, :, None, :], torch.from_numpy(k)[None], torch.from_numpy(v)[None]
+    module = types.SimpleNamespace(num_key_value_groups=hq // hkv, training=False)
+    eager, _ = eager_attention_forward(module, tq, tk, tv, None, scale)  # [1, 1, Hq, D]
+    assert np.allclose(mine, eager[0, 0].numpy(), rtol=1e-5, atol=1e-5)
+    sdpa = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, scale=scale, enable_gqa=True)
+    assert np.allclose(mine, sdpa[0, :, 0].numpy(), rtol=1e-5, atol=1e-5)
+    # the wrong grouping is far outside that tolerance on these inputs
+    wrong = oracle.gqa_decode_attention(q, k[[0, 1, 2] * 4][:hq].reshape(hq, t, d), v[[0, 1, 2] * 4][:hq].reshape(hq, t, d),
+                                        scale, "f32")
+    assert not np.allclose(wrong, eager[0, 0].numpy(), rtol=1e-2, atol=1e-2)
+
+
 # ---- the C oracle says the same ----------------------------------------------------------------------------
 
 @pytest.fixture(scope="module")
