@@ -173,6 +173,17 @@ int llmq_wq_gemm_a8(const int8_t* a, const float* sx, const void* qweight, const
                     const float* bias_or_null, void* out, int M, int N, int G, int gs,
                     int out_group, int wformat, int dtype, llmq_stream_t stream);
 
+/* Weight-only GEMM for more rows than the GEMV takes, without the dense copy of the weight that
+ * KernelQuantLinear builds per forward for M > KERNEL_MAX_ROWS (`_dequantized_weight` + matmul,
+ * llmquant/quantizers/kernel.py:68-79, 88-91):
+ *   out[m, n] = sum over g of  wscale[sr(n), g] * sum_k x[m, g*128 + k] * code[n, g, k]
+ * in the form of RealQuantLinear's weight-only branch (llmquant/quantizers/real.py:84-91), fp32
+ * accumulation on the matrix cores, cast to `dtype`. x, out: LLMQ_F16 or LLMQ_BF16, [M, G*128] and
+ * [M, N]; qweight/wscale as for llmq_wq_gemv; gs must be 128. Any M: rows are taken 64 at a time and
+ * every slab streams the weight once, so this pays up to a few dozen rows. */
+int llmq_wq_gemm_a16(const void* x, const void* qweight, const float* wscale, void* out, int M, int N,
+                     int G, int gs, int out_group, int wformat, int dtype, llmq_stream_t stream);
+
 /* KV cache, one layer. Codes are [kv_heads, t_max, head_dim] int8 (bits == 8) or
  * [kv_heads, t_max, head_dim/2] nibble-packed uint8 (bits == 4); scales are fp32
  * [kv_heads, t_max]: one scale per token per head, which is what FakeQuantCache's

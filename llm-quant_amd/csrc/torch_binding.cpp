@@ -423,6 +423,38 @@ at::Tensor wq_gemm_a8(const at::Tensor& a, const at::Tensor& sx, const at::Tenso
   return out;
 }
 
+// Weight-only GEMM for a few dozen rows: x fp16/bf16 [M, K]; qweight / wscale as for wq_gemv.
+at::Tensor wq_gemm_a16(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale, int64_t out_group) {
+  TORCH_CHECK(x.is_cuda(), "x must be a CUDA tensor");
+  TORCH_CHECK(qweight.is_cuda() && wscale.is_cuda(), "qweight and wscale must be CUDA tensors");
+  TORCH_CHECK(x.scalar_type() == at::kHalf || x.scalar_type() == at::kBFloat16,
+              "the fused GEMM takes float16 or bfloat16 activations");
+  TORCH_CHECK(x.dim() == 2, "x must be [M, K]");
+  TORCH_CHECK(qweight.dim() == 3, "qweight must be [N, groups, group_size], got ", qweight.dim(), "D");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 2, "wscale must be float32 [scale_rows, groups]");
+  const auto xc = x.contiguous();
+  const auto wc = qweight.contiguous();
+  const auto sc = wscale.contiguous();
+  const int64_t M = xc.size(0), N = wc.size(0), groups = wc.size(1);
+  const int64_t group_size = packed ? wc.size(2) * 2 : wc.size(2);
+  TORCH_CHECK(group_size == 128, "the fused GEMM needs group_size 128, got ", group_size);
+  TORCH_CHECK(xc.size(1) == groups * group_size, "x last dim ", xc.size(1), " does not match qweight ", groups, "x",
+              group_size);
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  TORCH_CHECK(sc.size(0) == scale_rows && sc.size(1) == groups, "wscale must be [", scale_rows, ", ", groups, "]");
+  auto out = at::empty({M, N}, xc.options());
+  if (M == 0 || N == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(xc));
+  check_rc(llmq_wq_gemm_a16(xc.const_data_ptr(), wc.const_data_ptr(), sc.const_data_ptr<float>(),
+                            out.mutable_data_ptr(), static_cast<int>(M), static_cast<int>(N),
+                            static_cast<int>(groups), static_cast<int>(group_size), static_cast<int>(out_group),
+                            packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype_code(xc, "x"), current_stream(xc)),
+           "wq_gemm_a16");
+  return out;
+}
+
 // ---- quantized KV cache -------------------------------------------------------------------------------
 // Cache tensors of one layer: codes [kv_heads, t_max, head_dim] int8 or [kv_heads, t_max,
 // head_dim / 2] uint8, scales [kv_heads, t_max] fp32. `position` is a device int32 tensor.
@@ -732,6 +764,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "Integer GEMM: int8 activations x int4/int8 group-quantized weights, real-mode rounding order",
         py::arg("a"), py::arg("sx"), py::arg("qweight"), py::arg("wscale"), py::arg("bias") = py::none(),
         py::arg("out_group") = 0, py::arg("out_dtype") = at::kBFloat16);
+  m.def("wq_gemm_a16", &wq_gemm_a16,
+        "Weight-only GEMM for a few dozen rows: fp16/bf16 activations x int4/int8 group-quantized weights, no dense copy",
+        py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0);
   m.def("kv_append", &kv_append,
         "Quantize new K/V tokens into one layer's cache at the device-side position",
         py::arg("key"), py::arg("value"), py::arg("k_codes"), py::arg("v_codes"), py::arg("k_scale"),

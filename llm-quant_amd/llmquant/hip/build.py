@@ -113,6 +113,8 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_argmax_advance.restype = c_int
     lib.llmq_wq_gemm_a8.argtypes = [c_p] * 6 + [c_int] * 7 + [c_p]
     lib.llmq_wq_gemm_a8.restype = c_int
+    lib.llmq_wq_gemm_a16.argtypes = [c_p] * 4 + [c_int] * 7 + [c_p]
+    lib.llmq_wq_gemm_a16.restype = c_int
     lib.llmq_wq_gemv_batched.argtypes = [c_p] * 7 + [c_int] * 9 + [c_p]
     lib.llmq_wq_gemv_batched.restype = c_int
     lib.llmq_wq_gemv_batched_max_rows.restype = c_int

@@ -21,6 +21,9 @@ from llmquant.quantizers.real import quantize_weight
 #: up to this many activation rows the GEMV kernel runs; above it the weight is dequantized
 #: once and a dense matmul takes over
 KERNEL_MAX_ROWS = 4
+#: ... except that up to this many rows of a 16-bit activation go to the fused GEMM, which reads
+#: the codes once and builds no dense weight (measured crossover with dequantize + matmul)
+FUSED_GEMM_MAX_ROWS = 32
 
 
 def pad_activation(flat: torch.Tensor, args) -> torch.Tensor:
@@ -109,7 +112,9 @@ class KernelQuantLinear(nn.Module):
 
     def forward(self, x):
         rows = x.reshape(-1, x.shape[-1])
-        if rows.shape[0] > KERNEL_MAX_ROWS and not self._int8_act and self._head_keep:
+        fused = (KERNEL_MAX_ROWS < rows.shape[0] <= FUSED_GEMM_MAX_ROWS and rows.dtype in (torch.bfloat16, torch.float16)
+                 and self.padded_in_features == self.qdata.shape[1] * 128)
+        if rows.shape[0] > KERNEL_MAX_ROWS and not self._int8_act and self._head_keep and not fused:
             # dense branch on the real width: neither the activation nor the weight is padded
             out = rows @ self._dequantized_weight(rows.dtype, real_width=True).T
             if self.bias is not None:
@@ -124,6 +129,8 @@ class KernelQuantLinear(nn.Module):
             return out.reshape(*x.shape[:-1], self.out_features)
         if rows.shape[0] <= KERNEL_MAX_ROWS:
             out = self._gemv(rows, self.qdata, self.wscale, self.out_group)
+        elif fused:
+            out = self._ext.wq_gemm_a16(rows, self.qdata, self.wscale, self.out_group)
         else:
             out = rows @ self._dequantized_weight(rows.dtype).T
         if self.bias is not None:

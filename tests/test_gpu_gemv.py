@@ -278,18 +278,42 @@ def test_shape_and_dtype_checks(linear):
 
 
 def test_dense_branch_lands_where_fake_quant_does(linear):
-    from llmquant.quantizers import KERNEL_MAX_ROWS, FakeQuantLinear, KernelQuantLinear, RealQuantLinear
+    from llmquant.quantizers import FUSED_GEMM_MAX_ROWS, FakeQuantLinear, KernelQuantLinear, RealQuantLinear
 
     lin = linear.cuda()
     for name, spec in LAYOUTS.items():
         spec = dict(spec)
         scheme = weight_only(spec.pop("bits"), **spec)
         torch.manual_seed(0)
-        x = torch.randn(KERNEL_MAX_ROWS * 4, K, device="cuda", dtype=torch.bfloat16)
+        x = torch.randn(FUSED_GEMM_MAX_ROWS + 8, K, device="cuda", dtype=torch.bfloat16)
         kernel = KernelQuantLinear.from_linear(lin, scheme)(x).float()
         fake = FakeQuantLinear.from_linear(lin, scheme)(x).float()
         real = RealQuantLinear.from_linear(lin, scheme)(x).float()
         assert torch.isclose((kernel - real).abs().max(), (fake - real).abs().max(), rtol=1e-3), name
+
+
+@pytest.mark.parametrize("name", list(LAYOUTS))
+@pytest.mark.parametrize("M", [5, 16, 32])
+def test_a_few_dozen_rows_take_the_fused_gemm(name, M, linear):
+    """Between the GEMV's rows and the dense branch: no dense weight is built, and the result is
+    the real-mode sum (as for the GEMV), in every layout incl. padded heads and head scales."""
+    from llmquant.quantizers import FUSED_GEMM_MAX_ROWS, KERNEL_MAX_ROWS, KernelQuantLinear
+
+    assert KERNEL_MAX_ROWS < M <= FUSED_GEMM_MAX_ROWS
+    spec = dict(LAYOUTS[name])
+    bits = spec.pop("bits")
+    module = KernelQuantLinear.from_linear(linear.cuda(), weight_only(bits, **spec))
+    module._dequantized_weight = None  # the dense branch would fail loudly
+    torch.manual_seed(M)
+    x = torch.randn(M, K).to(torch.bfloat16)
+    got = module(x.cuda())
+    assert got.shape == (M, N) and got.dtype == torch.bfloat16
+    _, _, real, exact = oracle_forward(linear.weight, x, bits, torch.bfloat16, **spec)
+    assert rel_l2(to_np(got), exact) <= 2e-3
+    assert rel_l2(to_np(got), real) <= 2e-3
+    # rows do not depend on what they are batched with beyond the last place: the GEMV's answer
+    single = module(x[:1].cuda())
+    assert rel_l2(to_np(got[:1]), to_np(single)) <= 2e-3
 
 
 def test_real_width_and_padded_width(linear):
