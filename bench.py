@@ -465,6 +465,46 @@ def other_kernels(torch):
                          "act_quant_us": round(us_q, 1), "TOPS": round(2 * m * n * k / us / 1e6, 1),
                          "frac_int8_mfma_peak": round(2 * m * n * k / us / 1e6 / 5000.0, 4)})
     out["w4a8_gemm"] = gemm
+    # a few dozen rows of a 16-bit activation: the fused GEMM (codes straight from HBM to the matrix cores)
+    # against the dense branch it replaces (dequantize the weight, then a dense matmul), Llama-3-8B MLP
+    # shapes, int4, weights rotated over > 600 MB, one rotation replayed as a graph
+    lib = _CAPI["lib"]
+    fused = []
+    for n, k in ((14336, 4096), (4096, 14336)):
+        nbytes_w = n * k // 2 + n * (k // GROUP) * 4
+        copies = (600 << 20) // nbytes_w + 1
+        qs = [torch.randint(0, 255, (n, k // GROUP, GROUP // 2), dtype=torch.uint8, device=dev) for _ in range(copies)]
+        sw = torch.rand(n, k // GROUP, device=dev) * 0.01
+        for m in (8, 16, 32, 64):
+            x = torch.randn(m, k, device=dev).to(torch.bfloat16)
+            y = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
+            dense = torch.empty(n, k, device=dev, dtype=torch.bfloat16)
+
+            def fused_sweep():
+                sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                for c in range(copies):
+                    rc = lib.llmq_wq_gemm_a16(x.data_ptr(), qs[c].data_ptr(), sw.data_ptr(), y.data_ptr(), m, n,
+                                              k // GROUP, GROUP, 0, 4, 2, sp)
+                    if rc:
+                        raise RuntimeError(lib.llmq_last_error().decode())
+
+            def dense_sweep():
+                sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                for c in range(copies):
+                    rc = lib.llmq_dequant_weight(qs[c].data_ptr(), sw.data_ptr(), dense.data_ptr(), n, k // GROUP,
+                                                 GROUP, GROUP, 0, 4, 2, sp)
+                    if rc:
+                        raise RuntimeError(lib.llmq_last_error().decode())
+                    torch.matmul(x, dense.T, out=y)
+
+            us = _graph_time_us(torch, fused_sweep, reps=5) / copies
+            us_dense = _graph_time_us(torch, dense_sweep, reps=5) / copies
+            nbytes = nbytes_w + m * k * 2 + m * n * 2
+            fused.append({"M": m, "N": n, "K": k, "weights": "int4", "us": round(us, 2),
+                          "dequant_plus_matmul_us": round(us_dense, 2), "bytes": nbytes,
+                          "GBps": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)})
+        del qs
+    out["w4a16_fused_gemm_small_m"] = fused
     return out
 
 

@@ -186,15 +186,19 @@ class KernelQuantExperts(_QuantExperts):
         return pad_activation(x, self._weight_args) if real_in != padded_in else x
 
     def _matmul(self, x, qweight, wscale, real_in, padded_in):
-        """One expert's projection: the GEMV up to KERNEL_MAX_ROWS rows, else dequantize + matmul.
-        `qweight` is that expert's slice, stored (packed) or canonical."""
-        from llmquant.quantizers.kernel import KERNEL_MAX_ROWS
+        """One expert's projection: the GEMV up to KERNEL_MAX_ROWS rows, the fused GEMM up to
+        FUSED_GEMM_MAX_ROWS rows of a 16-bit activation, else dequantize + matmul. `qweight` is that
+        expert's slice, stored (packed) or canonical."""
+        from llmquant.quantizers.kernel import FUSED_GEMM_MAX_ROWS, KERNEL_MAX_ROWS
 
         x = self._pad(x, real_in, padded_in)
         if qweight.dtype == torch.int8 and self._packed:
             qweight = pack_int4(qweight)
         if x.shape[0] <= KERNEL_MAX_ROWS:
             return self._gemv(x, qweight, wscale, 0)
+        if (x.shape[0] <= FUSED_GEMM_MAX_ROWS and x.dtype in (torch.bfloat16, torch.float16)
+                and self._weight_args.group_size == 128):
+            return self._ext.wq_gemm_a16(x, qweight.contiguous(), wscale, 0)
         return x @ self._ext.dequant_weight(qweight.contiguous(), wscale, 0, 0, x.dtype).T
 
     def _project(self, x, which, expert):

@@ -22,8 +22,12 @@ from llmquant.quantizers.real import quantize_weight
 #: once and a dense matmul takes over
 KERNEL_MAX_ROWS = 4
 #: ... except that up to this many rows of a 16-bit activation go to the fused GEMM, which reads
-#: the codes once and builds no dense weight (measured crossover with dequantize + matmul)
+#: the codes once and builds no dense weight (the measured crossover with dequantize + matmul:
+#: 32 rows, 64 for layers at least FUSED_GEMM_WIDE_FEATURES wide, whose row tiles share the
+#: activation two by two)
 FUSED_GEMM_MAX_ROWS = 32
+FUSED_GEMM_MAX_ROWS_WIDE = 64
+FUSED_GEMM_WIDE_FEATURES = 8192
 
 
 def pad_activation(flat: torch.Tensor, args) -> torch.Tensor:
@@ -75,6 +79,11 @@ class KernelQuantLinear(nn.Module):
         act = scheme.input_activations
         self._int8_act = (act is not None and act.num_bits == 8 and act.strategy == "group"
                           and act.group_size == group_size == 128)
+        # the fused GEMM's reach (it needs groups of 128)
+        self._fused_max_rows = 0
+        if group_size == 128:
+            wide = self.out_features >= FUSED_GEMM_WIDE_FEATURES
+            self._fused_max_rows = FUSED_GEMM_MAX_ROWS_WIDE if wide else FUSED_GEMM_MAX_ROWS
         # looked up once: a decode step runs ~113 of these modules
         self._ext = load_extension()
         self._gemv = self._ext.wq_gemv
@@ -112,8 +121,8 @@ class KernelQuantLinear(nn.Module):
 
     def forward(self, x):
         rows = x.reshape(-1, x.shape[-1])
-        fused = (KERNEL_MAX_ROWS < rows.shape[0] <= FUSED_GEMM_MAX_ROWS and rows.dtype in (torch.bfloat16, torch.float16)
-                 and self.padded_in_features == self.qdata.shape[1] * 128)
+        fused = (KERNEL_MAX_ROWS < rows.shape[0] <= self._fused_max_rows
+                 and rows.dtype in (torch.bfloat16, torch.float16) and not self._int8_act)
         if rows.shape[0] > KERNEL_MAX_ROWS and not self._int8_act and self._head_keep and not fused:
             # dense branch on the real width: neither the activation nor the weight is padded
             out = rows @ self._dequantized_weight(rows.dtype, real_width=True).T
