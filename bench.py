@@ -497,10 +497,24 @@ def other_kernels(torch):
                         raise RuntimeError(lib.llmq_last_error().decode())
                     torch.matmul(x, dense.T, out=y)
 
-            us = _graph_time_us(torch, fused_sweep, reps=5) / copies
+            need = lib.llmq_wq_gemm_a16_workspace_bytes(m, n, k // GROUP)
+            scratch = torch.empty(max(need // 4, 4), device=dev)
+
+            def split_sweep():  # the reduction axis split across workgroups: two launches, flat in M
+                sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                for c in range(copies):
+                    rc = lib.llmq_wq_gemm_a16_split(x.data_ptr(), qs[c].data_ptr(), sw.data_ptr(), y.data_ptr(),
+                                                    scratch.data_ptr(), need, m, n, k // GROUP, GROUP, 0, 4, 2, sp)
+                    if rc:
+                        raise RuntimeError(lib.llmq_last_error().decode())
+
+            us_whole = _graph_time_us(torch, fused_sweep, reps=5) / copies
+            us_split = _graph_time_us(torch, split_sweep, reps=5) / copies
             us_dense = _graph_time_us(torch, dense_sweep, reps=5) / copies
+            us = us_whole if m <= 16 else us_split  # what KernelQuantLinear picks (FUSED_GEMM_WHOLE_ROWS)
             nbytes = nbytes_w + m * k * 2 + m * n * 2
             fused.append({"M": m, "N": n, "K": k, "weights": "int4", "us": round(us, 2),
+                          "whole_rows_form_us": round(us_whole, 2), "split_form_us": round(us_split, 2),
                           "dequant_plus_matmul_us": round(us_dense, 2), "bytes": nbytes,
                           "GBps": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)})
         del qs

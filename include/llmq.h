@@ -184,6 +184,19 @@ int llmq_wq_gemm_a8(const int8_t* a, const float* sx, const void* qweight, const
 int llmq_wq_gemm_a16(const void* x, const void* qweight, const float* wscale, void* out, int M, int N,
                      int G, int gs, int out_group, int wformat, int dtype, llmq_stream_t stream);
 
+/* The same GEMM with the reduction axis split across workgroups (128 weight rows x 4 groups each):
+ * every workgroup copies only its slice of x into LDS, so the bytes the CUs pull in stay close to
+ * the codes' own whatever M, and the launch has N/128 * ceil(G/4) workgroups whatever the shape. The
+ * slices' fp32 sums go through `workspace` (llmq_wq_gemm_a16_workspace_bytes(M, N, G) bytes, 16-byte
+ * aligned, contents irrelevant before and after) and a second launch adds them in a fixed order; with
+ * G <= 4 there is one slice, no workspace and no second launch. Same arguments and result form as
+ * llmq_wq_gemm_a16 otherwise. Calls that share a workspace must not overlap. No counterpart in the
+ * reference. */
+size_t llmq_wq_gemm_a16_workspace_bytes(int M, int N, int G);
+int llmq_wq_gemm_a16_split(const void* x, const void* qweight, const float* wscale, void* out,
+                           void* workspace, size_t workspace_bytes, int M, int N, int G, int gs,
+                           int out_group, int wformat, int dtype, llmq_stream_t stream);
+
 /* KV cache, one layer. Codes are [kv_heads, t_max, head_dim] int8 (bits == 8) or
  * [kv_heads, t_max, head_dim/2] nibble-packed uint8 (bits == 4); scales are fp32
  * [kv_heads, t_max]: one scale per token per head, which is what FakeQuantCache's

@@ -424,7 +424,8 @@ at::Tensor wq_gemm_a8(const at::Tensor& a, const at::Tensor& sx, const at::Tenso
 }
 
 // Weight-only GEMM for a few dozen rows: x fp16/bf16 [M, K]; qweight / wscale as for wq_gemv.
-at::Tensor wq_gemm_a16(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale, int64_t out_group) {
+at::Tensor wq_gemm_a16(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale, int64_t out_group,
+                       bool split) {
   TORCH_CHECK(x.is_cuda(), "x must be a CUDA tensor");
   TORCH_CHECK(qweight.is_cuda() && wscale.is_cuda(), "qweight and wscale must be CUDA tensors");
   TORCH_CHECK(x.scalar_type() == at::kHalf || x.scalar_type() == at::kBFloat16,
@@ -447,6 +448,17 @@ at::Tensor wq_gemm_a16(const at::Tensor& x, const at::Tensor& qweight, const at:
   auto out = at::empty({M, N}, xc.options());
   if (M == 0 || N == 0) return out;
   const c10::OptionalDeviceGuard guard(at::device_of(xc));
+  if (split) {
+    const size_t need = llmq_wq_gemm_a16_workspace_bytes(static_cast<int>(M), static_cast<int>(N), static_cast<int>(groups));
+    auto workspace = at::empty({static_cast<int64_t>((need + 3) / 4)}, xc.options().dtype(at::kFloat));
+    check_rc(llmq_wq_gemm_a16_split(xc.const_data_ptr(), wc.const_data_ptr(), sc.const_data_ptr<float>(),
+                                    out.mutable_data_ptr(), need ? workspace.mutable_data_ptr() : nullptr, need,
+                                    static_cast<int>(M), static_cast<int>(N), static_cast<int>(groups),
+                                    static_cast<int>(group_size), static_cast<int>(out_group),
+                                    packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype_code(xc, "x"), current_stream(xc)),
+             "wq_gemm_a16_split");
+    return out;
+  }
   check_rc(llmq_wq_gemm_a16(xc.const_data_ptr(), wc.const_data_ptr(), sc.const_data_ptr<float>(),
                             out.mutable_data_ptr(), static_cast<int>(M), static_cast<int>(N),
                             static_cast<int>(groups), static_cast<int>(group_size), static_cast<int>(out_group),
@@ -766,7 +778,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("out_group") = 0, py::arg("out_dtype") = at::kBFloat16);
   m.def("wq_gemm_a16", &wq_gemm_a16,
         "Weight-only GEMM for a few dozen rows: fp16/bf16 activations x int4/int8 group-quantized weights, no dense copy",
-        py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0);
+        py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("split") = false);
   m.def("kv_append", &kv_append,
         "Quantize new K/V tokens into one layer's cache at the device-side position",
         py::arg("key"), py::arg("value"), py::arg("k_codes"), py::arg("v_codes"), py::arg("k_scale"),

@@ -115,6 +115,10 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_wq_gemm_a8.restype = c_int
     lib.llmq_wq_gemm_a16.argtypes = [c_p] * 4 + [c_int] * 7 + [c_p]
     lib.llmq_wq_gemm_a16.restype = c_int
+    lib.llmq_wq_gemm_a16_split.argtypes = [c_p] * 5 + [ctypes.c_size_t] + [c_int] * 7 + [c_p]
+    lib.llmq_wq_gemm_a16_split.restype = c_int
+    lib.llmq_wq_gemm_a16_workspace_bytes.argtypes = [c_int] * 3
+    lib.llmq_wq_gemm_a16_workspace_bytes.restype = ctypes.c_size_t
     lib.llmq_wq_gemv_batched.argtypes = [c_p] * 7 + [c_int] * 9 + [c_p]
     lib.llmq_wq_gemv_batched.restype = c_int
     lib.llmq_wq_gemv_batched_max_rows.restype = c_int

@@ -22,12 +22,12 @@ from llmquant.quantizers.real import quantize_weight
 #: once and a dense matmul takes over
 KERNEL_MAX_ROWS = 4
 #: ... except that up to this many rows of a 16-bit activation go to the fused GEMM, which reads
-#: the codes once and builds no dense weight (the measured crossover with dequantize + matmul:
-#: 32 rows, 64 for layers at least FUSED_GEMM_WIDE_FEATURES wide, whose row tiles share the
-#: activation two by two)
-FUSED_GEMM_MAX_ROWS = 32
-FUSED_GEMM_MAX_ROWS_WIDE = 64
-FUSED_GEMM_WIDE_FEATURES = 8192
+#: the codes once and builds no dense weight (the measured crossover with dequantize + matmul).
+#: Up to FUSED_GEMM_WHOLE_ROWS rows in its one-launch form (a workgroup owns whole weight rows),
+#: above that in the form that splits the reduction axis across workgroups (two launches, flat in
+#: the row count).
+FUSED_GEMM_MAX_ROWS = 64
+FUSED_GEMM_WHOLE_ROWS = 16
 
 
 def pad_activation(flat: torch.Tensor, args) -> torch.Tensor:
@@ -80,10 +80,7 @@ class KernelQuantLinear(nn.Module):
         self._int8_act = (act is not None and act.num_bits == 8 and act.strategy == "group"
                           and act.group_size == group_size == 128)
         # the fused GEMM's reach (it needs groups of 128)
-        self._fused_max_rows = 0
-        if group_size == 128:
-            wide = self.out_features >= FUSED_GEMM_WIDE_FEATURES
-            self._fused_max_rows = FUSED_GEMM_MAX_ROWS_WIDE if wide else FUSED_GEMM_MAX_ROWS
+        self._fused_max_rows = FUSED_GEMM_MAX_ROWS if group_size == 128 else 0
         # looked up once: a decode step runs ~113 of these modules
         self._ext = load_extension()
         self._gemv = self._ext.wq_gemv
@@ -139,7 +136,8 @@ class KernelQuantLinear(nn.Module):
         if rows.shape[0] <= KERNEL_MAX_ROWS:
             out = self._gemv(rows, self.qdata, self.wscale, self.out_group)
         elif fused:
-            out = self._ext.wq_gemm_a16(rows, self.qdata, self.wscale, self.out_group)
+            out = self._ext.wq_gemm_a16(rows, self.qdata, self.wscale, self.out_group,
+                                        rows.shape[0] > FUSED_GEMM_WHOLE_ROWS)
         else:
             out = rows @ self._dequantized_weight(rows.dtype).T
         if self.bias is not None:

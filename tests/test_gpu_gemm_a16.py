@@ -50,13 +50,17 @@ def ulp_distance(a, b, dtype):
     return int(np.abs(ia - ib)[big].max())
 
 
+SPLIT = pytest.mark.parametrize("split", [False, True], ids=["whole rows", "split reduction axis"])
+
+
+@SPLIT
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("m,n,k", [(5, 256, 512), (16, 128, 128), (17, 200, 384), (33, 129, 256), (64, 512, 2048),
-                                   (70, 96, 640), (1, 16, 128), (48, 64, 1152)])
-def test_against_closed_form_and_real_mode(ext, bits, dtype, m, n, k):
+                                   (70, 96, 640), (1, 16, 128), (48, 64, 1152), (130, 300, 768)])
+def test_against_closed_form_and_real_mode(ext, bits, dtype, m, n, k, split):
     x, q, s, canonical, scales = make_case(m, n, k, bits, dtype)
-    got = ext.wq_gemm_a16(x.cuda(), q, s, 0)
+    got = ext.wq_gemm_a16(x.cuda(), q, s, 0, split)
     assert got.shape == (m, n) and got.dtype == dtype
     exact = oracle.gemv_float64(to_np(x), canonical, scales)
     assert rel_l2(to_np(got), exact) <= 2e-3
@@ -67,29 +71,32 @@ def test_against_closed_form_and_real_mode(ext, bits, dtype, m, n, k):
     assert rel_l2(to_np(got), want) <= 2e-3
 
 
+@SPLIT
 @pytest.mark.parametrize("bits", [4, 8])
-def test_head_scales(ext, bits):
+def test_head_scales(ext, bits, split):
     x, q, s, canonical, scales = make_case(24, 192, 512, bits, torch.bfloat16, out_group=64, seed=1)
-    got = ext.wq_gemm_a16(x.cuda(), q, s, 64)
+    got = ext.wq_gemm_a16(x.cuda(), q, s, 64, split)
     exact = oracle.gemv_float64(to_np(x), canonical, scales, 64)
     assert rel_l2(to_np(got), exact) <= 2e-3
 
 
+@SPLIT
 @pytest.mark.parametrize("bits", [4, 8])
-def test_rows_agree_with_the_gemv(ext, bits):
+def test_rows_agree_with_the_gemv(ext, bits, split):
     """Each row against the GEMV kernel on that row: two routes to the same sum, one ulp."""
     x, q, s, _, _ = make_case(12, 320, 1024, bits, torch.bfloat16, seed=2)
-    got = to_np(ext.wq_gemm_a16(x.cuda(), q, s, 0))
+    got = to_np(ext.wq_gemm_a16(x.cuda(), q, s, 0, split))
     for r0 in range(0, 12, 4):
         rows = to_np(ext.wq_gemv(x[r0:r0 + 4].cuda(), q, s, 0))
         assert ulp_distance(got[r0:r0 + 4], rows, torch.bfloat16) <= 1
 
 
+@SPLIT
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336), (8192, 2048), (2048, 8192)])
 @pytest.mark.parametrize("m", [8, 64])
-def test_llama_shapes_on_sampled_entries(ext, n, k, m):
+def test_llama_shapes_on_sampled_entries(ext, n, k, m, split):
     x, q, s, canonical, scales = make_case(m, n, k, 4, torch.bfloat16, seed=3)
-    got = to_np(ext.wq_gemm_a16(x.cuda(), q, s, 0))
+    got = to_np(ext.wq_gemm_a16(x.cuda(), q, s, 0, split))
     rng = np.random.default_rng(0)
     cols = np.sort(rng.choice(n, 64, replace=False))
     exact = oracle.gemv_float64(to_np(x), canonical[cols], scales[cols])
@@ -106,3 +113,26 @@ def test_argument_checks(ext):
         ext.wq_gemm_a16(x, q, s, 0)
     empty = ext.wq_gemm_a16(x[:0].cuda(), q, s, 0)
     assert empty.shape == (0, 64)
+
+
+def test_split_form_repeats_itself_and_checks_its_workspace(ext):
+    """The slices are added in a fixed order: two runs agree to the bit. The C entry refuses a
+    workspace that is too small."""
+    import ctypes
+
+    from llmquant.hip import load_capi
+
+    x, q, s, _, _ = make_case(16, 384, 2048, 4, torch.bfloat16, seed=5)
+    xd = x.cuda()
+    first = ext.wq_gemm_a16(xd, q, s, 0, True)
+    for _ in range(3):
+        assert torch.equal(ext.wq_gemm_a16(xd, q, s, 0, True), first)
+    lib = load_capi()
+    need = lib.llmq_wq_gemm_a16_workspace_bytes(16, 384, 16)
+    assert need == 4 * 16 * 384 * 4
+    assert lib.llmq_wq_gemm_a16_workspace_bytes(16, 384, 4) == 0
+    out = torch.empty(16, 384, device="cuda", dtype=torch.bfloat16)
+    small = torch.empty(need // 4 - 4, device="cuda", dtype=torch.float32)
+    rc = lib.llmq_wq_gemm_a16_split(xd.data_ptr(), q.data_ptr(), s.data_ptr(), out.data_ptr(), small.data_ptr(),
+                                    small.numel() * 4, 16, 384, 16, 128, 0, 4, 2, None)
+    assert rc != 0 and b"workspace" in lib.llmq_last_error()

@@ -293,7 +293,7 @@ def test_dense_branch_lands_where_fake_quant_does(linear):
 
 
 @pytest.mark.parametrize("name", list(LAYOUTS))
-@pytest.mark.parametrize("M", [5, 16, 32])
+@pytest.mark.parametrize("M", [5, 16, 17, 64])
 def test_a_few_dozen_rows_take_the_fused_gemm(name, M, linear):
     """Between the GEMV's rows and the dense branch: no dense weight is built, and the result is
     the real-mode sum (as for the GEMV), in every layout incl. padded heads and head scales."""
