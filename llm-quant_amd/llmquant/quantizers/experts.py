@@ -189,7 +189,7 @@ class KernelQuantExperts(_QuantExperts):
         """One expert's projection: the GEMV up to KERNEL_MAX_ROWS rows, the fused GEMM up to
         FUSED_GEMM_MAX_ROWS rows of a 16-bit activation, else dequantize + matmul. `qweight` is that
         expert's slice, stored (packed) or canonical."""
-        from llmquant.quantizers.kernel import FUSED_GEMM_MAX_ROWS, FUSED_GEMM_WHOLE_ROWS, KERNEL_MAX_ROWS
+        from llmquant.quantizers.kernel import FUSED_GEMM_MAX_ROWS, KERNEL_MAX_ROWS, fused_gemm_splits
 
         x = self._pad(x, real_in, padded_in)
         if qweight.dtype == torch.int8 and self._packed:
@@ -198,7 +198,7 @@ class KernelQuantExperts(_QuantExperts):
             return self._gemv(x, qweight, wscale, 0)
         if (x.shape[0] <= FUSED_GEMM_MAX_ROWS and x.dtype in (torch.bfloat16, torch.float16)
                 and self._weight_args.group_size == 128):
-            return self._ext.wq_gemm_a16(x, qweight.contiguous(), wscale, 0, x.shape[0] > FUSED_GEMM_WHOLE_ROWS)
+            return self._ext.wq_gemm_a16(x, qweight.contiguous(), wscale, 0, fused_gemm_splits(x.shape[0], qweight.shape[1]))
         return x @ self._ext.dequant_weight(qweight.contiguous(), wscale, 0, 0, x.dtype).T
 
     def _project(self, x, which, expert):

@@ -24,10 +24,16 @@ KERNEL_MAX_ROWS = 4
 #: ... except that up to this many rows of a 16-bit activation go to the fused GEMM, which reads
 #: the codes once and builds no dense weight (the measured crossover with dequantize + matmul).
 #: Up to FUSED_GEMM_WHOLE_ROWS rows in its one-launch form (a workgroup owns whole weight rows),
-#: above that in the form that splits the reduction axis across workgroups (two launches, flat in
-#: the row count).
+#: above that, and for rows of FUSED_GEMM_SPLIT_GROUPS groups or more (down_proj), in the form
+#: that splits the reduction axis across workgroups (two launches, flat in the row count).
 FUSED_GEMM_MAX_ROWS = 64
 FUSED_GEMM_WHOLE_ROWS = 16
+FUSED_GEMM_SPLIT_GROUPS = 64
+
+
+def fused_gemm_splits(rows: int, groups: int) -> bool:
+    """Which form of the fused GEMM is faster for this many activation rows and groups per weight row."""
+    return rows > FUSED_GEMM_WHOLE_ROWS or groups >= FUSED_GEMM_SPLIT_GROUPS
 
 
 def pad_activation(flat: torch.Tensor, args) -> torch.Tensor:
@@ -137,7 +143,7 @@ class KernelQuantLinear(nn.Module):
             out = self._gemv(rows, self.qdata, self.wscale, self.out_group)
         elif fused:
             out = self._ext.wq_gemm_a16(rows, self.qdata, self.wscale, self.out_group,
-                                        rows.shape[0] > FUSED_GEMM_WHOLE_ROWS)
+                                        fused_gemm_splits(rows.shape[0], self.qdata.shape[1]))
         else:
             out = rows @ self._dequantized_weight(rows.dtype).T
         if self.bias is not None:
