@@ -186,19 +186,20 @@ class KernelQuantExperts(_QuantExperts):
         return pad_activation(x, self._weight_args) if real_in != padded_in else x
 
     def _matmul(self, x, qweight, wscale, real_in, padded_in):
-        """One expert's projection: the GEMV up to KERNEL_MAX_ROWS rows, the fused GEMM up to
-        FUSED_GEMM_MAX_ROWS rows of a 16-bit activation, else dequantize + matmul. `qweight` is that
+        """One expert's projection: the GEMV for one or two rows (up to KERNEL_MAX_ROWS for fp32), the fused
+        GEMM for FUSED_GEMM_MIN_ROWS .. FUSED_GEMM_MAX_ROWS rows of a 16-bit activation, else dequantize + matmul. `qweight` is that
         expert's slice, stored (packed) or canonical."""
-        from llmquant.quantizers.kernel import FUSED_GEMM_MAX_ROWS, KERNEL_MAX_ROWS, fused_gemm_splits
+        from llmquant.quantizers.kernel import (FUSED_GEMM_MAX_ROWS, FUSED_GEMM_MIN_ROWS, KERNEL_MAX_ROWS,
+                                               fused_gemm_splits)
 
         x = self._pad(x, real_in, padded_in)
         if qweight.dtype == torch.int8 and self._packed:
             qweight = pack_int4(qweight)
-        if x.shape[0] <= KERNEL_MAX_ROWS:
-            return self._gemv(x, qweight, wscale, 0)
-        if (x.shape[0] <= FUSED_GEMM_MAX_ROWS and x.dtype in (torch.bfloat16, torch.float16)
+        if (FUSED_GEMM_MIN_ROWS <= x.shape[0] <= FUSED_GEMM_MAX_ROWS and x.dtype in (torch.bfloat16, torch.float16)
                 and self._weight_args.group_size == 128):
             return self._ext.wq_gemm_a16(x, qweight.contiguous(), wscale, 0, fused_gemm_splits(x.shape[0], qweight.shape[1]))
+        if x.shape[0] <= KERNEL_MAX_ROWS:
+            return self._gemv(x, qweight, wscale, 0)
         return x @ self._ext.dequant_weight(qweight.contiguous(), wscale, 0, 0, x.dtype).T
 
     def _project(self, x, which, expert):

@@ -28,6 +28,10 @@ KERNEL_MAX_ROWS = 4
 #: that splits the reduction axis across workgroups (two launches, flat in the row count).
 FUSED_GEMM_MAX_ROWS = 64
 FUSED_GEMM_WHOLE_ROWS = 16
+#: ... and from this many rows on it is also faster than the GEMV kernel, which multiplies its rows
+#: as int8 digit planes and slows down with each row (14336 x 4096 int4, graph replay: GEMV 9.6 /
+#: 13.0 / 14.8 / 21.0 us for 1-4 rows, the fused GEMM 13.4-14.3 us for any of them)
+FUSED_GEMM_MIN_ROWS = 3
 FUSED_GEMM_SPLIT_GROUPS = 64
 
 
@@ -124,7 +128,7 @@ class KernelQuantLinear(nn.Module):
 
     def forward(self, x):
         rows = x.reshape(-1, x.shape[-1])
-        fused = (KERNEL_MAX_ROWS < rows.shape[0] <= self._fused_max_rows
+        fused = (FUSED_GEMM_MIN_ROWS <= rows.shape[0] <= self._fused_max_rows
                  and rows.dtype in (torch.bfloat16, torch.float16) and not self._int8_act)
         if rows.shape[0] > KERNEL_MAX_ROWS and not self._int8_act and self._head_keep and not fused:
             # dense branch on the real width: neither the activation nor the weight is padded
@@ -139,11 +143,11 @@ class KernelQuantLinear(nn.Module):
             out = self._ext.wq_gemm_a8(codes, act_scale, self.qdata, self.wscale, self.bias, self.out_group,
                                        x.dtype)
             return out.reshape(*x.shape[:-1], self.out_features)
-        if rows.shape[0] <= KERNEL_MAX_ROWS:
-            out = self._gemv(rows, self.qdata, self.wscale, self.out_group)
-        elif fused:
+        if fused:
             out = self._ext.wq_gemm_a16(rows, self.qdata, self.wscale, self.out_group,
                                         fused_gemm_splits(rows.shape[0], self.qdata.shape[1]))
+        elif rows.shape[0] <= KERNEL_MAX_ROWS:
+            out = self._gemv(rows, self.qdata, self.wscale, self.out_group)
         else:
             out = rows @ self._dequantized_weight(rows.dtype).T
         if self.bias is not None:

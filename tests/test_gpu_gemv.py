@@ -293,13 +293,14 @@ def test_dense_branch_lands_where_fake_quant_does(linear):
 
 
 @pytest.mark.parametrize("name", list(LAYOUTS))
-@pytest.mark.parametrize("M", [5, 16, 17, 64])
+@pytest.mark.parametrize("M", [3, 4, 5, 16, 17, 64])
 def test_a_few_dozen_rows_take_the_fused_gemm(name, M, linear):
     """Between the GEMV's rows and the dense branch: no dense weight is built, and the result is
     the real-mode sum (as for the GEMV), in every layout incl. padded heads and head scales."""
-    from llmquant.quantizers import FUSED_GEMM_MAX_ROWS, KERNEL_MAX_ROWS, KernelQuantLinear
+    from llmquant.quantizers import FUSED_GEMM_MAX_ROWS, KernelQuantLinear
+    from llmquant.quantizers.kernel import FUSED_GEMM_MIN_ROWS
 
-    assert KERNEL_MAX_ROWS < M <= FUSED_GEMM_MAX_ROWS
+    assert FUSED_GEMM_MIN_ROWS <= M <= FUSED_GEMM_MAX_ROWS
     spec = dict(LAYOUTS[name])
     bits = spec.pop("bits")
     module = KernelQuantLinear.from_linear(linear.cuda(), weight_only(bits, **spec))
