@@ -101,8 +101,8 @@ def build_operands(torch, copies_bytes=600 << 20):
 def main():
     opts = parse()
     if opts.gpus != 1:
-        print("bench.py measures one GPU: this path has no multi-GPU form (see DESIGN.md, "
-              "'How the path would shard'). Run with --gpus 1.", file=sys.stderr)
+        print("bench.py measures one GPU: this path has no multi-GPU form (it would shard by output rows, "
+              "kv heads and experts, with no exchange inside a kernel). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import torch
