@@ -197,6 +197,24 @@ int llmq_wq_gemm_a16_split(const void* x, const void* qweight, const float* wsca
                            void* workspace, size_t workspace_bytes, int M, int N, int G, int gs,
                            int out_group, int wformat, int dtype, llmq_stream_t stream);
 
+/* The elementwise pieces of a prompt pass, one launch each, with the rounding points of the PyTorch
+ * sequences they replace (the same ones the decode kernels use). dtype: LLMQ_F32 / F16 / BF16; all
+ * tensors 16-byte aligned. No counterpart in the reference, which leaves these to transformers
+ * (LlamaRMSNorm.forward, apply_rotary_pos_emb, LlamaMLP.forward: ~20 PyTorch kernels per layer).
+ *   llmq_rmsnorm   out[r, :] = weight * (dtype)(x[r, :] * rsqrt(mean(x[r, :]^2) + eps)), fp32 inside;
+ *                  hidden a multiple of 8 (4 for fp32)
+ *   llmq_rope_qk   q [tokens, q_heads * head_dim] and k [tokens, kv_heads * head_dim] (row strides in
+ *                  elements) rotated by cos / sin [tokens, head_dim] into contiguous q_out / k_out:
+ *                  (dtype)((dtype)(x * cos) + (dtype)(rotate_half(x) * sin)); head_dim a multiple of 16
+ *                  (8 for fp32)
+ *   llmq_silu_mul  out = (dtype)((dtype)silu(gate) * up) over `count` elements */
+int llmq_rmsnorm(const void* x, const void* weight, void* out, int rows, int hidden, float eps, int dtype,
+                 llmq_stream_t stream);
+int llmq_rope_qk(const void* q, const void* k, const void* cos_rows, const void* sin_rows, void* q_out,
+                 void* k_out, int tokens, int q_heads, int kv_heads, int head_dim, int64_t q_row_stride,
+                 int64_t k_row_stride, int dtype, llmq_stream_t stream);
+int llmq_silu_mul(const void* gate, const void* up, void* out, int64_t count, int dtype, llmq_stream_t stream);
+
 /* KV cache, one layer. Codes are [kv_heads, t_max, head_dim] int8 (bits == 8) or
  * [kv_heads, t_max, head_dim/2] nibble-packed uint8 (bits == 4); scales are fp32
  * [kv_heads, t_max]: one scale per token per head, which is what FakeQuantCache's

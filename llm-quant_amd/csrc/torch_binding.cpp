@@ -467,6 +467,65 @@ at::Tensor wq_gemm_a16(const at::Tensor& x, const at::Tensor& qweight, const at:
   return out;
 }
 
+// ---- elementwise pieces of a prompt pass ----------------------------------------------------------------
+at::Tensor rmsnorm(const at::Tensor& x, const at::Tensor& weight, double eps) {
+  TORCH_CHECK(x.is_cuda() && weight.is_cuda(), "x and weight must be CUDA tensors");
+  TORCH_CHECK(x.dim() >= 1 && weight.dim() == 1 && weight.size(0) == x.size(-1), "weight must be [hidden]");
+  TORCH_CHECK(weight.scalar_type() == x.scalar_type(), "weight must have x's dtype");
+  const auto xc = x.contiguous();
+  const auto wc = weight.contiguous();
+  auto out = at::empty_like(xc);
+  const int64_t hidden = xc.size(-1);
+  const int64_t rows = hidden ? xc.numel() / hidden : 0;
+  if (rows == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(xc));
+  check_rc(llmq_rmsnorm(xc.const_data_ptr(), wc.const_data_ptr(), out.mutable_data_ptr(), static_cast<int>(rows),
+                        static_cast<int>(hidden), static_cast<float>(eps), dtype_code(xc, "x"), current_stream(xc)),
+           "rmsnorm");
+  return out;
+}
+
+// q [tokens, q_heads * D], k [tokens, kv_heads * D] (rows may be strided), cos / sin [tokens, D].
+std::tuple<at::Tensor, at::Tensor> rope_qk(const at::Tensor& q, const at::Tensor& k, const at::Tensor& cos,
+                                           const at::Tensor& sin, int64_t q_heads, int64_t kv_heads) {
+  TORCH_CHECK(q.is_cuda() && k.is_cuda() && cos.is_cuda() && sin.is_cuda(), "all tensors must be CUDA");
+  TORCH_CHECK(q.dim() == 2 && k.dim() == 2 && cos.dim() == 2 && sin.dim() == 2, "q, k, cos, sin must be 2-D");
+  TORCH_CHECK(q.stride(1) == 1 && k.stride(1) == 1, "q and k need a contiguous last axis");
+  TORCH_CHECK(q_heads > 0 && kv_heads > 0, "head counts must be positive");
+  const int64_t tokens = q.size(0), head_dim = cos.size(1);
+  TORCH_CHECK(k.size(0) == tokens && cos.size(0) == tokens && sin.size(0) == tokens && sin.size(1) == head_dim,
+              "q, k, cos and sin must cover the same tokens");
+  TORCH_CHECK(q.size(1) == q_heads * head_dim && k.size(1) == kv_heads * head_dim, "q / k widths do not match the heads");
+  TORCH_CHECK(k.scalar_type() == q.scalar_type() && cos.scalar_type() == q.scalar_type() &&
+                  sin.scalar_type() == q.scalar_type(), "k, cos and sin must have q's dtype");
+  const auto cc = cos.contiguous();
+  const auto sc = sin.contiguous();
+  auto q_out = at::empty({tokens, q_heads, head_dim}, q.options());
+  auto k_out = at::empty({tokens, kv_heads, head_dim}, k.options());
+  if (tokens == 0) return {q_out, k_out};
+  const c10::OptionalDeviceGuard guard(at::device_of(q));
+  check_rc(llmq_rope_qk(q.const_data_ptr(), k.const_data_ptr(), cc.const_data_ptr(), sc.const_data_ptr(),
+                        q_out.mutable_data_ptr(), k_out.mutable_data_ptr(), static_cast<int>(tokens),
+                        static_cast<int>(q_heads), static_cast<int>(kv_heads), static_cast<int>(head_dim), q.stride(0),
+                        k.stride(0), dtype_code(q, "q"), current_stream(q)),
+           "rope_qk");
+  return {q_out, k_out};
+}
+
+at::Tensor silu_mul(const at::Tensor& gate, const at::Tensor& up) {
+  TORCH_CHECK(gate.is_cuda() && up.is_cuda(), "gate and up must be CUDA tensors");
+  TORCH_CHECK(gate.sizes() == up.sizes() && gate.scalar_type() == up.scalar_type(), "gate and up must match");
+  const auto gc = gate.contiguous();
+  const auto uc = up.contiguous();
+  auto out = at::empty_like(gc);
+  if (gc.numel() == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(gc));
+  check_rc(llmq_silu_mul(gc.const_data_ptr(), uc.const_data_ptr(), out.mutable_data_ptr(), gc.numel(),
+                         dtype_code(gc, "gate"), current_stream(gc)),
+           "silu_mul");
+  return out;
+}
+
 // ---- quantized KV cache -------------------------------------------------------------------------------
 // Cache tensors of one layer: codes [kv_heads, t_max, head_dim] int8 or [kv_heads, t_max,
 // head_dim / 2] uint8, scales [kv_heads, t_max] fp32. `position` is a device int32 tensor.
@@ -779,6 +838,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("wq_gemm_a16", &wq_gemm_a16,
         "Weight-only GEMM for a few dozen rows: fp16/bf16 activations x int4/int8 group-quantized weights, no dense copy",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("split") = false);
+  m.def("rmsnorm", &rmsnorm, "LlamaRMSNorm over the last axis, one launch", py::arg("x"), py::arg("weight"), py::arg("eps"));
+  m.def("rope_qk", &rope_qk, "apply_rotary_pos_emb on the q and k projections of a prompt, one launch",
+        py::arg("q"), py::arg("k"), py::arg("cos"), py::arg("sin"), py::arg("q_heads"), py::arg("kv_heads"));
+  m.def("silu_mul", &silu_mul, "silu(gate) * up with both roundings, one launch", py::arg("gate"), py::arg("up"));
   m.def("kv_append", &kv_append,
         "Quantize new K/V tokens into one layer's cache at the device-side position",
         py::arg("key"), py::arg("value"), py::arg("k_codes"), py::arg("v_codes"), py::arg("k_scale"),

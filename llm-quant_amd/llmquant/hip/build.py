@@ -119,6 +119,12 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_wq_gemm_a16_split.restype = c_int
     lib.llmq_wq_gemm_a16_workspace_bytes.argtypes = [c_int] * 3
     lib.llmq_wq_gemm_a16_workspace_bytes.restype = ctypes.c_size_t
+    lib.llmq_rmsnorm.argtypes = [c_p, c_p, c_p, c_int, c_int, ctypes.c_float, c_int, c_p]
+    lib.llmq_rmsnorm.restype = c_int
+    lib.llmq_rope_qk.argtypes = [c_p] * 6 + [c_int] * 4 + [ctypes.c_int64] * 2 + [c_int, c_p]
+    lib.llmq_rope_qk.restype = c_int
+    lib.llmq_silu_mul.argtypes = [c_p, c_p, c_p, ctypes.c_int64, c_int, c_p]
+    lib.llmq_silu_mul.restype = c_int
     lib.llmq_wq_gemv_batched.argtypes = [c_p] * 7 + [c_int] * 9 + [c_p]
     lib.llmq_wq_gemv_batched.restype = c_int
     lib.llmq_wq_gemv_batched_max_rows.restype = c_int

@@ -19,6 +19,7 @@ from __future__ import annotations
 import torch
 import torch.nn.functional as F
 
+from llmquant.hip.build import load_extension
 from llmquant.runtime.kv_cache import KernelQuantCache
 
 WARMUP_CALLS = 3
@@ -44,6 +45,9 @@ class LlamaKernelRuntime:
         self.head_dim = getattr(cfg, "head_dim", None) or cfg.hidden_size // cfg.num_attention_heads
         self.scaling = self.head_dim ** -0.5
         self.max_len = max_len
+        self._ext = load_extension()
+        # RMSNorm, RoPE and SiLU * up as one launch each (16-bit models); False walks the PyTorch modules
+        self._one_launch_ops = self.dtype in (torch.bfloat16, torch.float16)
         self.cache = KernelQuantCache(len(self.layers), self.kv_heads, self.head_dim, max_len, kv_bits,
                                       q_heads=self.q_heads, device=self.device)
         # cos / sin for every position, computed the way LlamaRotaryEmbedding.forward does
@@ -79,14 +83,34 @@ class LlamaKernelRuntime:
         ctx = torch.matmul(probs, v.float()[:, None])  # [Hkv, rep, T, D]
         return ctx.reshape(self.q_heads, tokens, self.head_dim).transpose(0, 1).reshape(tokens, -1).to(q.dtype)
 
+    # ---- the elementwise pieces, one launch each where the module is the stock Llama one -----------
+    def _norm(self, module, x):
+        """LlamaRMSNorm in one launch (seven PyTorch kernels otherwise)."""
+        if (self._one_launch_ops and type(module).__name__.endswith("RMSNorm") and hasattr(module, "variance_epsilon")
+                and x.shape[-1] % 8 == 0 and module.weight.dtype == x.dtype):
+            return self._ext.rmsnorm(x, module.weight, module.variance_epsilon)
+        return module(x)
+
+    def _rotated(self, q, k, cos, sin):
+        """q [T, Hq*D], k [T, Hkv*D] -> rotated [T, Hq, D], [T, Hkv, D]."""
+        tokens = q.shape[0]
+        if self._one_launch_ops and self.head_dim % 16 == 0 and q.dtype == cos.dtype:
+            return self._ext.rope_qk(q, k, cos, sin, self.q_heads, self.kv_heads)
+        return self._rope(q.view(tokens, self.q_heads, self.head_dim), k.view(tokens, self.kv_heads, self.head_dim),
+                          cos, sin)
+
+    def _gated(self, mlp, x):
+        gate, up = mlp.gate_proj(x), mlp.up_proj(x)
+        if self._one_launch_ops and "SiLU" in type(mlp.act_fn).__name__ and gate.shape[-1] % 8 == 0:
+            return self._ext.silu_mul(gate, up)
+        return mlp.act_fn(gate) * up
+
     def _layer(self, index, layer, hidden, cos, sin, decode: bool):
         attn = layer.self_attn
         tokens = hidden.shape[0]
-        x = layer.input_layernorm(hidden)
-        q = attn.q_proj(x).view(tokens, self.q_heads, self.head_dim)
-        k = attn.k_proj(x).view(tokens, self.kv_heads, self.head_dim)
+        x = self._norm(layer.input_layernorm, hidden)
         v = attn.v_proj(x).view(tokens, self.kv_heads, self.head_dim)
-        q, k = self._rope(q, k, cos, sin)
+        q, k = self._rotated(attn.q_proj(x), attn.k_proj(x), cos, sin)
         if decode:
             self.cache.append(index, k.transpose(0, 1), v.transpose(0, 1))
             ctx = self.cache.attend(index, q[0].contiguous(), self.scaling).reshape(1, -1)
@@ -101,15 +125,14 @@ class LlamaKernelRuntime:
                                                      is_causal=True, scale=self.scaling, enable_gqa=True)
                 ctx = ctx[0].transpose(0, 1).reshape(tokens, -1)
         hidden = hidden + attn.o_proj(ctx)
-        x = layer.post_attention_layernorm(hidden)
-        mlp = layer.mlp
-        return hidden + mlp.down_proj(mlp.act_fn(mlp.gate_proj(x)) * mlp.up_proj(x))
+        x = self._norm(layer.post_attention_layernorm, hidden)
+        return hidden + layer.mlp.down_proj(self._gated(layer.mlp, x))
 
     def _forward(self, token_ids, cos, sin, decode: bool):
         hidden = self.model.model.embed_tokens(token_ids)
         for index, layer in enumerate(self.layers):
             hidden = self._layer(index, layer, hidden, cos, sin, decode)
-        hidden = self.model.model.norm(hidden[-1:])
+        hidden = self._norm(self.model.model.norm, hidden[-1:].contiguous())
         return self.model.lm_head(hidden)
 
     # ---- prefill ------------------------------------------------------------------------------------

@@ -1,0 +1,115 @@
+"""The one-launch RMSNorm, RoPE and SiLU * up of a prompt pass against the transformers modules and
+functions they replace (LlamaRMSNorm.forward, apply_rotary_pos_emb, act_fn(gate) * up): the same
+rounding points, so equal to the bit except where the fp32 mean of squares is summed in another order
+(RMSNorm: at most one unit in the last place of a few elements)."""
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ext():
+    from llmquant.hip import load_extension
+
+    return load_extension()
+
+
+def ulps(a, b):
+    """Elementwise distance in units of the last place of a 16-bit tensor."""
+    ia = a.view(torch.int16).to(torch.int32)
+    ib = b.view(torch.int16).to(torch.int32)
+    ia = torch.where(ia < 0, -(ia & 0x7fff), ia)
+    ib = torch.where(ib < 0, -(ib & 0x7fff), ib)
+    return (ia - ib).abs()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("rows,hidden", [(1, 2048), (512, 2048), (7, 4096), (3, 136), (64, 8)])
+def test_rmsnorm_matches_llama_rmsnorm(ext, dtype, rows, hidden):
+    from transformers.models.llama.modeling_llama import LlamaRMSNorm
+
+    torch.manual_seed(rows + hidden)
+    norm = LlamaRMSNorm(hidden, eps=1e-5).to("cuda", dtype)
+    with torch.no_grad():
+        norm.weight.copy_(torch.randn(hidden) * 0.5 + 1.0)
+    x = (torch.randn(rows, hidden, device="cuda") * 3.0).to(dtype)
+    with torch.no_grad():
+        want = norm(x)
+    got = ext.rmsnorm(x, norm.weight, 1e-5)
+    assert got.shape == want.shape and got.dtype == dtype
+    if dtype == torch.float32:
+        assert torch.allclose(got, want, rtol=2e-6, atol=0)
+    else:
+        d = ulps(got, want)
+        assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 0.02
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("tokens,q_heads,kv_heads,head_dim", [(512, 32, 8, 64), (1, 32, 8, 64), (5, 8, 8, 128), (3, 4, 1, 16)])
+def test_rope_matches_apply_rotary_pos_emb(ext, dtype, tokens, q_heads, kv_heads, head_dim):
+    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+
+    torch.manual_seed(tokens)
+    q = torch.randn(tokens, q_heads * head_dim, device="cuda").to(dtype)
+    k = torch.randn(tokens, kv_heads * head_dim, device="cuda").to(dtype)
+    freqs = torch.rand(tokens, head_dim // 2, device="cuda") * 6.28
+    emb = torch.cat((freqs, freqs), dim=-1)
+    cos, sin = emb.cos().to(dtype), emb.sin().to(dtype)
+    # transformers' layout: [batch, heads, tokens, D] with cos / sin [batch, tokens, D]
+    q4 = q.view(1, tokens, q_heads, head_dim).transpose(1, 2)
+    k4 = k.view(1, tokens, kv_heads, head_dim).transpose(1, 2)
+    want_q, want_k = apply_rotary_pos_emb(q4, k4, cos[None], sin[None])
+    got_q, got_k = ext.rope_qk(q, k, cos, sin, q_heads, kv_heads)
+    assert got_q.shape == (tokens, q_heads, head_dim) and got_k.shape == (tokens, kv_heads, head_dim)
+    assert torch.equal(got_q, want_q[0].transpose(0, 1)) and torch.equal(got_k, want_k[0].transpose(0, 1))
+
+
+def test_rope_takes_strided_rows(ext):
+    """q and k as column slices of one fused projection output."""
+    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+
+    torch.manual_seed(0)
+    tokens, hq, hkv, d = 9, 4, 2, 64
+    qkv = torch.randn(tokens, (hq + 2 * hkv) * d, device="cuda").to(torch.bfloat16)
+    q, k = qkv[:, : hq * d], qkv[:, hq * d: (hq + hkv) * d]
+    freqs = torch.rand(tokens, d // 2, device="cuda")
+    emb = torch.cat((freqs, freqs), dim=-1)
+    cos, sin = emb.cos().to(torch.bfloat16), emb.sin().to(torch.bfloat16)
+    want_q, want_k = apply_rotary_pos_emb(q.reshape(1, tokens, hq, d).transpose(1, 2),
+                                          k.reshape(1, tokens, hkv, d).transpose(1, 2), cos[None], sin[None])
+    got_q, got_k = ext.rope_qk(q, k, cos, sin, hq, hkv)
+    assert torch.equal(got_q, want_q[0].transpose(0, 1)) and torch.equal(got_k, want_k[0].transpose(0, 1))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(512, 8192), (1, 8), (3, 5, 64)])
+def test_silu_mul_matches_the_mlp(ext, dtype, shape):
+    from transformers.activations import ACT2FN
+
+    torch.manual_seed(1)
+    gate = (torch.randn(*shape, device="cuda") * 4.0).to(dtype)
+    up = torch.randn(*shape, device="cuda").to(dtype)
+    want = ACT2FN["silu"](gate) * up
+    got = ext.silu_mul(gate, up)
+    if dtype == torch.float32:
+        assert torch.allclose(got, want, rtol=1e-6, atol=1e-7)
+    else:
+        d = ulps(got, want)  # (the exponential is evaluated by different routines)
+        assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 0.01
+
+
+def test_argument_checks(ext):
+    x = torch.randn(4, 64, device="cuda").to(torch.bfloat16)
+    w = torch.ones(64, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        ext.rmsnorm(x[:, :60].contiguous(), w[:60].contiguous(), 1e-5)
+    with pytest.raises(RuntimeError, match="weight must be"):
+        ext.rmsnorm(x, w[:32].contiguous(), 1e-5)
+    with pytest.raises(RuntimeError, match="must match"):
+        ext.silu_mul(x, x[:2])
+    with pytest.raises(RuntimeError, match="widths do not match"):
+        ext.rope_qk(x, x, x[:, :16].contiguous(), x[:, :16].contiguous(), 2, 4)
+    assert ext.rmsnorm(x[:0], w, 1e-5).shape == (0, 64)
