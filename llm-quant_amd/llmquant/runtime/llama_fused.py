@@ -51,6 +51,24 @@ class _Fused:
         self.qdata = torch.cat([m.qdata for m in mods], dim=0).contiguous()
         self.wscale = torch.cat([m.wscale for m in mods], dim=0).contiguous()
         self.out_group = mods[0].out_group
+        self.sources = _sources(mods)
+
+
+def _sources(mods):
+    """What a concatenation was built from: the buffers' addresses and versions (a buffer that was
+    replaced or written in place since makes the copy stale)."""
+    return tuple((t.data_ptr(), t._version, tuple(t.shape)) for m in mods for t in (m.qdata, m.wscale))
+
+
+def _fused(owner, name, *mods):
+    """The concatenation of `mods`, kept on `owner` (the attention / MLP module) between runtimes: a
+    generate call builds a new runtime, and copying 0.4 GB of weights again each time is a
+    millisecond of its time to first token."""
+    kept = owner.__dict__.get(name)
+    if kept is None or kept.sources != _sources(mods):
+        kept = _Fused(*mods)
+        owner.__dict__[name] = kept
+    return kept
 
 
 class LlamaFusedRuntime(LlamaKernelRuntime):
@@ -84,7 +102,8 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
                 raise ValueError("q_proj rows are not a whole number of scale tiles")
             args = attn.o_proj.scheme.weights
             self.fused_layers.append(dict(
-                qkv=_Fused(attn.q_proj, attn.k_proj, attn.v_proj), gate_up=_Fused(mlp.gate_proj, mlp.up_proj),
+                qkv=_fused(attn, "_llmq_fused_qkv", attn.q_proj, attn.k_proj, attn.v_proj),
+                gate_up=_fused(mlp, "_llmq_fused_gate_up", mlp.gate_proj, mlp.up_proj),
                 o=attn.o_proj, down=mlp.down_proj,
                 o_head_dim=args.head_dim if attn.o_proj._needs_padding else 0,
                 # act(gate) * up inside the gate|up launch: a row tile there is eight gate rows and their up rows
