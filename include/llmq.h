@@ -207,13 +207,17 @@ int llmq_wq_gemm_a16_split(const void* x, const void* qweight, const float* wsca
  *                  elements) rotated by cos / sin [tokens, head_dim] into contiguous q_out / k_out:
  *                  (dtype)((dtype)(x * cos) + (dtype)(rotate_half(x) * sin)); head_dim a multiple of 16
  *                  (8 for fp32)
- *   llmq_silu_mul  out = (dtype)((dtype)silu(gate) * up) over `count` elements */
+ *   llmq_silu_mul  out = (dtype)((dtype)silu(gate) * up) over `count` elements; _rows: gate and up as
+ *                  [rows, width] with row strides in elements (two column blocks of one projection's output),
+ *                  out contiguous [rows, width] */
 int llmq_rmsnorm(const void* x, const void* weight, void* out, int rows, int hidden, float eps, int dtype,
                  llmq_stream_t stream);
 int llmq_rope_qk(const void* q, const void* k, const void* cos_rows, const void* sin_rows, void* q_out,
                  void* k_out, int tokens, int q_heads, int kv_heads, int head_dim, int64_t q_row_stride,
                  int64_t k_row_stride, int dtype, llmq_stream_t stream);
 int llmq_silu_mul(const void* gate, const void* up, void* out, int64_t count, int dtype, llmq_stream_t stream);
+int llmq_silu_mul_rows(const void* gate, const void* up, void* out, int64_t rows, int width,
+                       int64_t gate_row_stride, int64_t up_row_stride, int dtype, llmq_stream_t stream);
 
 /* KV cache, one layer. Codes are [kv_heads, t_max, head_dim] int8 (bits == 8) or
  * [kv_heads, t_max, head_dim/2] nibble-packed uint8 (bits == 4); scales are fp32

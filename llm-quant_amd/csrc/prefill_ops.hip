@@ -90,15 +90,19 @@ __global__ __launch_bounds__(256) void rope_kernel(const T* __restrict__ q, cons
   store16(dst + i + D / 2, Pack<T>::pack(o_hi));
 }
 
+// gate, up: [rows, width] with row strides (two column blocks of one projection output, or two tensors).
 template <typename T>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict__ up,
-                                                       T* __restrict__ out, const int64_t packets) {
+                                                       T* __restrict__ out, const int64_t packets, const int per_row,
+                                                       const int64_t gate_stride, const int64_t up_stride) {
   constexpr int V = Pack<T>::N;
   const int64_t p = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (p >= packets) return;
+  const int64_t row = p / per_row;
+  const int col = static_cast<int>(p - row * per_row) * V;
   float g[V], u[V];
-  Pack<T>::unpack(load16(gate + p * V), g);
-  Pack<T>::unpack(load16(up + p * V), u);
+  Pack<T>::unpack(load16(gate + row * gate_stride + col), g);
+  Pack<T>::unpack(load16(up + row * up_stride + col), u);
 #pragma unroll
   for (int e = 0; e < V; ++e) g[e] = round_through<T>(g[e] / (1.0f + expf(-g[e]))) * u[e];
   store16(out + p * V, Pack<T>::pack(g));
@@ -160,19 +164,30 @@ extern "C" int llmq_rope_qk(const void* q, const void* k, const void* cos_rows, 
   return llmq_host::check_launch("rope_kernel");
 }
 
-extern "C" int llmq_silu_mul(const void* gate, const void* up, void* out, int64_t count, int dtype, llmq_stream_t stream) {
-  if (count < 0) return llmq_host::fail_invalid("negative element count");
+extern "C" int llmq_silu_mul_rows(const void* gate, const void* up, void* out, int64_t rows, int width,
+                                  int64_t gate_row_stride, int64_t up_row_stride, int dtype, llmq_stream_t stream) {
+  if (rows < 0 || width < 0) return llmq_host::fail_invalid("negative dimension");
   if (dtype != LLMQ_F32 && dtype != LLMQ_F16 && dtype != LLMQ_BF16)
     return llmq_host::fail_invalid("dtype code %d is not float32, float16 or bfloat16", dtype);
   const int v = packet_of(dtype);
-  if (count % v) return llmq_host::fail_invalid("the element count must be a multiple of %d", v);
-  if (count == 0) return 0;
+  if (width % v || gate_row_stride % v || up_row_stride % v)
+    return llmq_host::fail_invalid("the width and the row strides must be multiples of %d elements", v);
+  if (rows == 0 || width == 0) return 0;
   if (!gate || !up || !out) return llmq_host::fail_invalid("null tensor pointer");
   if (!aligned16(gate, up, out)) return llmq_host::fail_invalid("gate, up and out must be 16-byte aligned");
-  const int64_t packets = count / v;
+  const int per_row = width / v;
+  const int64_t packets = rows * per_row;
   const dim3 grid(static_cast<unsigned>((packets + 255) / 256)), block(256);
   hipStream_t s = static_cast<hipStream_t>(stream);
   LLMQ_BY_DTYPE(hipLaunchKernelGGL(silu_mul_kernel<T>, grid, block, 0, s, static_cast<const T*>(gate),
-                                   static_cast<const T*>(up), static_cast<T*>(out), packets));
+                                   static_cast<const T*>(up), static_cast<T*>(out), packets, per_row, gate_row_stride,
+                                   up_row_stride));
   return llmq_host::check_launch("silu_mul_kernel");
+}
+
+extern "C" int llmq_silu_mul(const void* gate, const void* up, void* out, int64_t count, int dtype, llmq_stream_t stream) {
+  if (count < 0) return llmq_host::fail_invalid("negative element count");
+  const int v = dtype == LLMQ_F32 ? 4 : 8;
+  if (count % v) return llmq_host::fail_invalid("the element count must be a multiple of %d", v);
+  return llmq_silu_mul_rows(gate, up, out, count / v, v, v, v, dtype, stream);  // rows of one packet each
 }

@@ -512,17 +512,26 @@ std::tuple<at::Tensor, at::Tensor> rope_qk(const at::Tensor& q, const at::Tensor
   return {q_out, k_out};
 }
 
+// gate, up: same shape; 2-D inputs may be column blocks of a wider tensor (row strides, contiguous last axis).
 at::Tensor silu_mul(const at::Tensor& gate, const at::Tensor& up) {
   TORCH_CHECK(gate.is_cuda() && up.is_cuda(), "gate and up must be CUDA tensors");
   TORCH_CHECK(gate.sizes() == up.sizes() && gate.scalar_type() == up.scalar_type(), "gate and up must match");
-  const auto gc = gate.contiguous();
-  const auto uc = up.contiguous();
-  auto out = at::empty_like(gc);
-  if (gc.numel() == 0) return out;
+  const bool strided = gate.dim() == 2 && gate.stride(1) == 1 && up.stride(1) == 1;
+  const auto gc = strided ? gate : gate.contiguous();
+  const auto uc = strided ? up : up.contiguous();
+  auto out = at::empty(gate.sizes(), gate.options());
+  if (gate.numel() == 0) return out;
   const c10::OptionalDeviceGuard guard(at::device_of(gc));
-  check_rc(llmq_silu_mul(gc.const_data_ptr(), uc.const_data_ptr(), out.mutable_data_ptr(), gc.numel(),
-                         dtype_code(gc, "gate"), current_stream(gc)),
-           "silu_mul");
+  if (strided) {
+    check_rc(llmq_silu_mul_rows(gc.const_data_ptr(), uc.const_data_ptr(), out.mutable_data_ptr(), gc.size(0),
+                                static_cast<int>(gc.size(1)), gc.stride(0), uc.stride(0), dtype_code(gc, "gate"),
+                                current_stream(gc)),
+             "silu_mul");
+  } else {
+    check_rc(llmq_silu_mul(gc.const_data_ptr(), uc.const_data_ptr(), out.mutable_data_ptr(), gc.numel(),
+                           dtype_code(gc, "gate"), current_stream(gc)),
+             "silu_mul");
+  }
   return out;
 }
 

@@ -125,6 +125,8 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_rope_qk.restype = c_int
     lib.llmq_silu_mul.argtypes = [c_p, c_p, c_p, ctypes.c_int64, c_int, c_p]
     lib.llmq_silu_mul.restype = c_int
+    lib.llmq_silu_mul_rows.argtypes = [c_p, c_p, c_p, ctypes.c_int64, c_int, ctypes.c_int64, ctypes.c_int64, c_int, c_p]
+    lib.llmq_silu_mul_rows.restype = c_int
     lib.llmq_wq_gemv_batched.argtypes = [c_p] * 7 + [c_int] * 9 + [c_p]
     lib.llmq_wq_gemv_batched.restype = c_int
     lib.llmq_wq_gemv_batched_max_rows.restype = c_int

@@ -99,9 +99,21 @@ class LlamaKernelRuntime:
         return self._rope(q.view(tokens, self.q_heads, self.head_dim), k.view(tokens, self.kv_heads, self.head_dim),
                           cos, sin)
 
-    def _gated(self, mlp, x):
-        gate, up = mlp.gate_proj(x), mlp.up_proj(x)
-        if self._one_launch_ops and "SiLU" in type(mlp.act_fn).__name__ and gate.shape[-1] % 8 == 0:
+    def _qkv(self, index, layer, x):
+        """The three projections of a layer, each [tokens, heads * head_dim]."""
+        attn = layer.self_attn
+        return attn.q_proj(x), attn.k_proj(x), attn.v_proj(x)
+
+    def _gate_up(self, index, layer, x):
+        return layer.mlp.gate_proj(x), layer.mlp.up_proj(x)
+
+    def _gated(self, index, layer, x):
+        mlp = layer.mlp
+        gate, up = self._gate_up(index, layer, x)
+        packets = (gate.shape[-1] % 8 == 0 and gate.stride(-1) == 1 and up.stride(-1) == 1
+                   and gate.data_ptr() % 16 == 0 and up.data_ptr() % 16 == 0
+                   and (gate.dim() != 2 or (gate.stride(0) % 8 == 0 and up.stride(0) % 8 == 0)))
+        if self._one_launch_ops and "SiLU" in type(mlp.act_fn).__name__ and packets:
             return self._ext.silu_mul(gate, up)
         return mlp.act_fn(gate) * up
 
@@ -109,8 +121,9 @@ class LlamaKernelRuntime:
         attn = layer.self_attn
         tokens = hidden.shape[0]
         x = self._norm(layer.input_layernorm, hidden)
-        v = attn.v_proj(x).view(tokens, self.kv_heads, self.head_dim)
-        q, k = self._rotated(attn.q_proj(x), attn.k_proj(x), cos, sin)
+        q, k, v = self._qkv(index, layer, x)
+        v = v.view(tokens, self.kv_heads, self.head_dim)
+        q, k = self._rotated(q, k, cos, sin)
         if decode:
             self.cache.append(index, k.transpose(0, 1), v.transpose(0, 1))
             ctx = self.cache.attend(index, q[0].contiguous(), self.scaling).reshape(1, -1)
@@ -126,7 +139,7 @@ class LlamaKernelRuntime:
                 ctx = ctx[0].transpose(0, 1).reshape(tokens, -1)
         hidden = hidden + attn.o_proj(ctx)
         x = self._norm(layer.post_attention_layernorm, hidden)
-        return hidden + layer.mlp.down_proj(self._gated(layer.mlp, x))
+        return hidden + layer.mlp.down_proj(self._gated(index, layer, x))
 
     def _forward(self, token_ids, cos, sin, decode: bool):
         hidden = self.model.model.embed_tokens(token_ids)

@@ -117,6 +117,33 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         self.final_norm = model.model.norm.weight.detach().contiguous()
         self.final_eps = model.model.norm.variance_epsilon
 
+    # ---- the prompt pass: q|k|v and gate|up as one projection each ----------------------------------
+    def _project(self, x, fused):
+        """x [tokens, K] times a concatenated weight: what KernelQuantLinear.forward would pick for this
+        many rows, once for the whole concatenation (three or two matmuls and dequantize passes fewer
+        per layer, and the host's matmul dispatch is the longest part of a prompt pass)."""
+        from llmquant.quantizers.kernel import (FUSED_GEMM_MAX_ROWS, FUSED_GEMM_MIN_ROWS, KERNEL_MAX_ROWS,
+                                                fused_gemm_splits)
+
+        rows = x.shape[0]
+        if FUSED_GEMM_MIN_ROWS <= rows <= FUSED_GEMM_MAX_ROWS and x.dtype in (torch.bfloat16, torch.float16):
+            return self._ext.wq_gemm_a16(x, fused.qdata, fused.wscale, fused.out_group,
+                                         fused_gemm_splits(rows, fused.qdata.shape[1]))
+        if rows <= KERNEL_MAX_ROWS:
+            return self._ext.wq_gemv(x, fused.qdata, fused.wscale, fused.out_group)
+        return x @ self._ext.dequant_weight(fused.qdata, fused.wscale, fused.out_group, 0, x.dtype).T
+
+    def _qkv(self, index, layer, x):
+        out = self._project(x, self.fused_layers[index]["qkv"])
+        q_width, kv_width = self.q_heads * self.head_dim, self.kv_heads * self.head_dim
+        # (the cache append wants k and v with the same strides: k comes out of the rotation contiguous)
+        return out[:, :q_width], out[:, q_width:q_width + kv_width], out[:, q_width + kv_width:].contiguous()
+
+    def _gate_up(self, index, layer, x):
+        out = self._project(x, self.fused_layers[index]["gate_up"])
+        half = out.shape[1] // 2
+        return out[:, :half], out[:, half:]
+
     def _forward(self, token_ids, cos, sin, decode: bool):
         if not decode:
             return super()._forward(token_ids, cos, sin, decode)

@@ -101,6 +101,46 @@ def test_silu_mul_matches_the_mlp(ext, dtype, shape):
         assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 0.01
 
 
+def test_silu_mul_takes_the_two_halves_of_one_projection(ext):
+    from transformers.activations import ACT2FN
+
+    torch.manual_seed(2)
+    both = (torch.randn(37, 2 * 1024, device="cuda") * 3.0).to(torch.bfloat16)
+    gate, up = both[:, :1024], both[:, 1024:]
+    got = ext.silu_mul(gate, up)
+    assert got.is_contiguous() and torch.equal(got, ext.silu_mul(gate.contiguous(), up.contiguous()))
+    d = ulps(got, ACT2FN["silu"](gate) * up)
+    assert int(d.max()) <= 1
+
+
+def test_prompt_pass_with_one_projection_per_group_matches_the_module_walk():
+    """LlamaFusedRuntime projects q|k|v and gate|up through the concatenated weights in a prompt pass;
+    LlamaKernelRuntime calls the five modules: the same first token, and logits that agree to the
+    rounding of two bf16 matmuls with different tilings."""
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from llmquant import QuantConfig, oneshot
+    from llmquant.runtime.llama_decode import LlamaKernelRuntime
+    from llmquant.runtime.llama_fused import LlamaFusedRuntime
+
+    torch.manual_seed(0)
+    cfg = LlamaConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=8,
+                      num_key_value_heads=2, head_dim=64, vocab_size=512, tie_word_embeddings=False,
+                      max_position_embeddings=256)
+    model = LlamaForCausalLM(cfg).to(torch.bfloat16).cuda().eval()
+    oneshot(model, QuantConfig(attn_weight="int8", mlp_weight="int4", head_weight="int8", kv_cache="int8").to_modifier("kernel"))
+    for tokens in (3, 40, 100):  # the GEMV's, the fused GEMM's and the dense branch's row counts
+        ids = torch.randint(0, 512, (1, tokens), device="cuda")
+        plain, fused = LlamaKernelRuntime(model, 128), LlamaFusedRuntime(model, 128)
+        with torch.no_grad():
+            plain.cache.set_position(0); plain.cache.length.fill_(tokens)
+            a = plain._forward(ids[0], plain.cos_table[:tokens], plain.sin_table[:tokens], decode=False).float()
+            fused.cache.set_position(0); fused.cache.length.fill_(tokens)
+            b = fused._forward(ids[0], fused.cos_table[:tokens], fused.sin_table[:tokens], decode=False).float()
+        assert float((a - b).norm() / a.norm()) < 3e-2
+        assert torch.equal(plain.cache.k_codes[0, :, :tokens], fused.cache.k_codes[0, :, :tokens])
+
+
 def test_argument_checks(ext):
     x = torch.randn(4, 64, device="cuda").to(torch.bfloat16)
     w = torch.ones(64, device="cuda", dtype=torch.bfloat16)
