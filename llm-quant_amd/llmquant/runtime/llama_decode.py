@@ -160,7 +160,8 @@ class LlamaKernelRuntime:
         self.cache.length.fill_(tokens)
         logits = self._forward(ids, self.cos_table[:tokens], self.sin_table[:tokens], decode=False)
         self.cache.set_position(tokens)
-        return logits.argmax(-1)
+        # (one row of logits: the kernel that the decode step uses, first maximum like torch.argmax)
+        return self._ext.argmax_row(logits) if logits.shape[0] == 1 and logits.is_contiguous() else logits.argmax(-1)
 
     # ---- decode ---------------------------------------------------------------------------------------
     def _step(self):
