@@ -20,7 +20,8 @@ import torch
 from llmquant.runtime.llama_decode import WARMUP_CALLS, LlamaKernelRuntime
 from llmquant.runtime.llama_fused import LlamaFusedRuntime
 
-__all__ = ["GraphedDecoder", "KernelDecoder", "WARMUP_CALLS", "can_graph", "graphed_generate", "kernel_runtime"]
+__all__ = ["GraphedDecoder", "KernelDecoder", "WARMUP_CALLS", "can_graph", "graphed_generate", "kept_kernel_runtime",
+           "kernel_runtime"]
 
 
 def _on_gpu(model) -> bool:
@@ -106,6 +107,42 @@ def kernel_runtime(model, max_len: int, kv_bits: int = 8):
         return LlamaKernelRuntime(model, max_len, kv_bits)
 
 
+_KEPT_RUNTIMES = 4
+
+
+def _weights_key(model):
+    """Identity of everything a captured step has baked in: the quantized buffers' addresses and
+    versions (a re-quantized or moved model gets new ones)."""
+    from llmquant.quantizers.kernel import KernelQuantLinear
+
+    key = []
+    for module in model.modules():
+        if isinstance(module, KernelQuantLinear):
+            key.append((module.qdata.data_ptr(), module.qdata._version, module.wscale.data_ptr(), module.wscale._version))
+    return tuple(key)
+
+
+def kept_kernel_runtime(model, max_len: int, kv_bits: int = 8):
+    """kernel_runtime, kept on the model between generate calls together with its captured step (which
+    reads token and position from the device, so it serves any prompt that fits max_len): a serving
+    loop does not rebuild and re-capture per request. Up to _KEPT_RUNTIMES cache lengths are kept; a
+    change of the model's quantized buffers drops them all."""
+    weights = _weights_key(model)
+    kept = model.__dict__.get("_llmq_kept_runtimes")
+    if kept is None or kept["weights"] != weights:
+        kept = {"weights": weights, "runtimes": {}}
+        model.__dict__["_llmq_kept_runtimes"] = kept
+    runtimes = kept["runtimes"]
+    key = (max_len, kv_bits)
+    runtime = runtimes.pop(key, None)
+    if runtime is None:
+        runtime = kernel_runtime(model, max_len, kv_bits)
+        while len(runtimes) >= _KEPT_RUNTIMES:
+            runtimes.pop(next(iter(runtimes)))  # the least recently used
+    runtimes[key] = runtime  # most recently used last
+    return runtime
+
+
 class KernelDecoder:
     """Same interface over LlamaKernelRuntime and the integer KV cache."""
 
@@ -142,8 +179,8 @@ def graphed_generate(model, input_ids, max_new_tokens: int, kv_bits: int | None 
         return None
     prompt = input_ids.shape[1]
     if kv_bits is not None:
-        return kernel_runtime(model, prompt + max_new_tokens + 1, kv_bits).generate(input_ids, max_new_tokens,
-                                                                                    use_graph=True)
+        return kept_kernel_runtime(model, prompt + max_new_tokens + 1, kv_bits).generate(input_ids, max_new_tokens,
+                                                                                         use_graph=True)
     decoder = GraphedDecoder(model, prompt, max_new_tokens)
     nxt = decoder.prefill(input_ids)
     out = [nxt]

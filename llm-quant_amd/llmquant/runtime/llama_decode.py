@@ -226,7 +226,10 @@ class LlamaKernelRuntime:
         out = [nxt.reshape(1, 1)]
         if max_new_tokens > 1:
             if use_graph:
-                self.capture(nxt, prompt)
+                if self.graph is None:
+                    self.capture(nxt, prompt)
+                else:  # a kept runtime: the captured step reads token and position from the device
+                    self._set_step_inputs(nxt, prompt)
                 for _ in range(max_new_tokens - 1):
                     out.append(self.step().clone().reshape(1, 1))
             else:

@@ -189,6 +189,39 @@ def test_graphed_generate_api(small):
     assert GraphedDecoder(base, 12, 4).max_len == 12 + 4 + 3 + 1
 
 
+def test_generate_calls_share_a_kept_runtime_and_its_captured_step(small):
+    """graphed_generate keeps the runtime and the captured step on the model: a second call with another
+    prompt (other length, same cache size) replays the same graph and gives what a fresh runtime gives;
+    re-quantizing the model drops what was kept."""
+    from llmquant.runtime import graphed_generate, kernel_runtime
+    from llmquant.runtime.graph_decode import kept_kernel_runtime
+
+    _, kernel = small
+    gen = torch.Generator().manual_seed(7)
+    first = torch.randint(0, 4096, (1, 20), generator=gen).cuda()
+    second = torch.randint(0, 4096, (1, 12), generator=gen).cuda()
+    kernel.__dict__.pop("_llmq_kept_runtimes", None)
+    a = graphed_generate(kernel, first, 12, kv_bits=8)           # cache of 33
+    kept = kept_kernel_runtime(kernel, 33, 8)
+    graph = kept.graph
+    assert graph is not None
+    b = graphed_generate(kernel, second, 20, kv_bits=8)          # cache of 33 again: same runtime, same graph
+    assert kept_kernel_runtime(kernel, 33, 8) is kept and kept.graph is graph
+    with torch.no_grad():
+        fresh_a = kernel_runtime(kernel, 33, 8).generate(first, 12, use_graph=True)
+        fresh_b = kernel_runtime(kernel, 33, 8).generate(second, 20, use_graph=True)
+    assert torch.equal(a, fresh_a) and torch.equal(b, fresh_b)
+    # and once more the first prompt, after the second one used the cache
+    assert torch.equal(graphed_generate(kernel, first, 12, kv_bits=8), fresh_a)
+    # another cache size: another runtime beside it
+    graphed_generate(kernel, first, 4, kv_bits=8)
+    assert len(kernel.__dict__["_llmq_kept_runtimes"]["runtimes"]) == 2
+    # a buffer written in place: everything kept is dropped
+    next(m for m in kernel.modules() if hasattr(m, "qdata")).wscale.mul_(1.0)
+    assert kept_kernel_runtime(kernel, 33, 8) is not kept
+    kernel.__dict__.pop("_llmq_kept_runtimes", None)
+
+
 def test_measure_latency_reports_the_reference_keys():
     """llmquant/eval/evaluate.py:167-223 on a small model: graphed HF path for bf16, the fused
     integer-KV runtime for the kernel-mode model."""
