@@ -202,7 +202,9 @@ int llmq_wq_gemm_a16_split(const void* x, const void* qweight, const float* wsca
  * tensors 16-byte aligned. No counterpart in the reference, which leaves these to transformers
  * (LlamaRMSNorm.forward, apply_rotary_pos_emb, LlamaMLP.forward: ~20 PyTorch kernels per layer).
  *   llmq_rmsnorm   out[r, :] = weight * (dtype)(x[r, :] * rsqrt(mean(x[r, :]^2) + eps)), fp32 inside;
- *                  hidden a multiple of 8 (4 for fp32)
+ *                  hidden a multiple of 8 (4 for fp32). llmq_add_rmsnorm: the same on (dtype)(x + delta),
+ *                  which is also written to sum_out (the residual add in front of a norm); delta and
+ *                  sum_out both NULL make it llmq_rmsnorm
  *   llmq_rope_qk   q [tokens, q_heads * head_dim] and k [tokens, kv_heads * head_dim] (row strides in
  *                  elements) rotated by cos / sin [tokens, head_dim] into contiguous q_out / k_out:
  *                  (dtype)((dtype)(x * cos) + (dtype)(rotate_half(x) * sin)); head_dim a multiple of 16
@@ -212,6 +214,8 @@ int llmq_wq_gemm_a16_split(const void* x, const void* qweight, const float* wsca
  *                  out contiguous [rows, width] */
 int llmq_rmsnorm(const void* x, const void* weight, void* out, int rows, int hidden, float eps, int dtype,
                  llmq_stream_t stream);
+int llmq_add_rmsnorm(const void* x, const void* delta_or_null, const void* weight, void* sum_out_or_null,
+                     void* out, int rows, int hidden, float eps, int dtype, llmq_stream_t stream);
 int llmq_rope_qk(const void* q, const void* k, const void* cos_rows, const void* sin_rows, void* q_out,
                  void* k_out, int tokens, int q_heads, int kv_heads, int head_dim, int64_t q_row_stride,
                  int64_t k_row_stride, int dtype, llmq_stream_t stream);

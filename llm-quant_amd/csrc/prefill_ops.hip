@@ -6,7 +6,8 @@
 // than the matmuls. Each of the three below is one pass over its tensor with the rounding points of
 // the PyTorch sequence it replaces, the same ones the decode kernels use.
 //
-//   rmsnorm    out = w * T(x_f32 * rsqrt(mean(x_f32^2) + eps))        (LlamaRMSNorm.forward)
+//   rmsnorm    out = w * T(x_f32 * rsqrt(mean(x_f32^2) + eps))        (LlamaRMSNorm.forward), optionally
+//              on x = T(x + delta), the residual add in front of it, which is stored as well
 //   rope_qk    out = T(T(x * cos) + T(rotate_half(x) * sin))           (apply_rotary_pos_emb), q and k
 //   silu_mul   out = T(T(silu(gate)) * up)                             (LlamaMLP: act_fn(gate) * up)
 #include "llmq_device.h"
@@ -17,19 +18,30 @@ using namespace llmq;
 
 constexpr int kNormThreads = 256;
 
-// One workgroup per row. The row is read twice (the second time from cache).
-template <typename T>
-__global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ w,
+// One workgroup per row. The row is read twice (the second time from cache). With `delta` the row is
+// first replaced by T(x + delta), which is also stored to `sum_out`: the residual add in front of a
+// norm (hidden = hidden + branch; normed = norm(hidden)) in the same launch.
+template <typename T, bool ADD>
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ delta,
+                                                              const T* __restrict__ w, T* __restrict__ sum_out,
                                                               T* __restrict__ out, const int hidden, const float eps) {
   constexpr int V = Pack<T>::N;
   __shared__ float red[kNormThreads / kWave];
-  const T* row = x + static_cast<int64_t>(blockIdx.x) * hidden;
-  T* orow = out + static_cast<int64_t>(blockIdx.x) * hidden;
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * hidden;
+  const T* row = x + base;
+  T* orow = out + base;
   const int tid = threadIdx.x;
   float ss = 0.0f;
   for (int i = tid * V; i < hidden; i += kNormThreads * V) {
     float f[V];
     Pack<T>::unpack(load16(row + i), f);
+    if constexpr (ADD) {
+      float d[V];
+      Pack<T>::unpack(load16(delta + base + i), d);
+#pragma unroll
+      for (int e = 0; e < V; ++e) f[e] = round_through<T>(f[e] + d[e]);
+      store16(sum_out + base + i, Pack<T>::pack(f));
+    }
 #pragma unroll
     for (int e = 0; e < V; ++e) ss = fmaf(f[e], f[e], ss);
   }
@@ -40,9 +52,11 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(const T* __restri
 #pragma unroll
   for (int k = 0; k < kNormThreads / kWave; ++k) total += red[k];
   const float inv_rms = rsqrtf(total / static_cast<float>(hidden) + eps);
+  // (with ADD a thread reads back exactly the packets it stored above)
+  const T* src = ADD ? sum_out + base : row;
   for (int i = tid * V; i < hidden; i += kNormThreads * V) {
     float f[V], g[V];
-    Pack<T>::unpack(load16(row + i), f);
+    Pack<T>::unpack(load16(src + i), f);
     Pack<T>::unpack(load16(w + i), g);
 #pragma unroll
     for (int e = 0; e < V; ++e) f[e] = g[e] * round_through<T>(f[e] * inv_rms);
@@ -124,19 +138,36 @@ int packet_of(int dtype) { return dtype == LLMQ_F32 ? 4 : 8; }
     default: return llmq_host::fail_invalid("dtype code %d is not float32, float16 or bfloat16", dtype);      \
   }
 
-extern "C" int llmq_rmsnorm(const void* x, const void* weight, void* out, int rows, int hidden, float eps, int dtype,
-                            llmq_stream_t stream) {
+extern "C" int llmq_add_rmsnorm(const void* x, const void* delta_or_null, const void* weight, void* sum_out_or_null,
+                                void* out, int rows, int hidden, float eps, int dtype, llmq_stream_t stream) {
   if (rows < 0 || hidden <= 0) return llmq_host::fail_invalid("bad dimension rows=%d hidden=%d", rows, hidden);
   if (dtype != LLMQ_F32 && dtype != LLMQ_F16 && dtype != LLMQ_BF16)
     return llmq_host::fail_invalid("dtype code %d is not float32, float16 or bfloat16", dtype);
   if (hidden % packet_of(dtype)) return llmq_host::fail_invalid("hidden must be a multiple of %d, got %d", packet_of(dtype), hidden);
   if (rows == 0) return 0;
   if (!x || !weight || !out) return llmq_host::fail_invalid("null tensor pointer");
-  if (!aligned16(x, weight, out)) return llmq_host::fail_invalid("x, weight and out must be 16-byte aligned");
+  if ((delta_or_null == nullptr) != (sum_out_or_null == nullptr))
+    return llmq_host::fail_invalid("delta and sum_out go together");
+  if (!aligned16(x, weight, out) || !aligned16(delta_or_null, sum_out_or_null))
+    return llmq_host::fail_invalid("tensors must be 16-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  LLMQ_BY_DTYPE(hipLaunchKernelGGL(rmsnorm_kernel<T>, dim3(rows), dim3(kNormThreads), 0, s, static_cast<const T*>(x),
-                                   static_cast<const T*>(weight), static_cast<T*>(out), hidden, eps));
+  if (delta_or_null) {
+    LLMQ_BY_DTYPE(hipLaunchKernelGGL((rmsnorm_kernel<T, true>), dim3(rows), dim3(kNormThreads), 0, s,
+                                     static_cast<const T*>(x), static_cast<const T*>(delta_or_null),
+                                     static_cast<const T*>(weight), static_cast<T*>(sum_out_or_null),
+                                     static_cast<T*>(out), hidden, eps));
+  } else {
+    LLMQ_BY_DTYPE(hipLaunchKernelGGL((rmsnorm_kernel<T, false>), dim3(rows), dim3(kNormThreads), 0, s,
+                                     static_cast<const T*>(x), static_cast<const T*>(nullptr),
+                                     static_cast<const T*>(weight), static_cast<T*>(nullptr), static_cast<T*>(out),
+                                     hidden, eps));
+  }
   return llmq_host::check_launch("rmsnorm_kernel");
+}
+
+extern "C" int llmq_rmsnorm(const void* x, const void* weight, void* out, int rows, int hidden, float eps, int dtype,
+                            llmq_stream_t stream) {
+  return llmq_add_rmsnorm(x, nullptr, weight, nullptr, out, rows, hidden, eps, dtype, stream);
 }
 
 extern "C" int llmq_rope_qk(const void* q, const void* k, const void* cos_rows, const void* sin_rows, void* q_out,

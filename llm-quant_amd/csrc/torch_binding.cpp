@@ -485,6 +485,29 @@ at::Tensor rmsnorm(const at::Tensor& x, const at::Tensor& weight, double eps) {
   return out;
 }
 
+// (x + delta, LlamaRMSNorm(x + delta)): the residual add in front of a norm, one launch.
+std::tuple<at::Tensor, at::Tensor> add_rmsnorm(const at::Tensor& x, const at::Tensor& delta, const at::Tensor& weight,
+                                               double eps) {
+  TORCH_CHECK(x.is_cuda() && delta.is_cuda() && weight.is_cuda(), "x, delta and weight must be CUDA tensors");
+  TORCH_CHECK(x.sizes() == delta.sizes() && x.scalar_type() == delta.scalar_type(), "x and delta must match");
+  TORCH_CHECK(x.dim() >= 1 && weight.dim() == 1 && weight.size(0) == x.size(-1), "weight must be [hidden]");
+  TORCH_CHECK(weight.scalar_type() == x.scalar_type(), "weight must have x's dtype");
+  const auto xc = x.contiguous();
+  const auto dc = delta.contiguous();
+  const auto wc = weight.contiguous();
+  auto sum = at::empty_like(xc);
+  auto out = at::empty_like(xc);
+  const int64_t hidden = xc.size(-1);
+  const int64_t rows = hidden ? xc.numel() / hidden : 0;
+  if (rows == 0) return {sum, out};
+  const c10::OptionalDeviceGuard guard(at::device_of(xc));
+  check_rc(llmq_add_rmsnorm(xc.const_data_ptr(), dc.const_data_ptr(), wc.const_data_ptr(), sum.mutable_data_ptr(),
+                            out.mutable_data_ptr(), static_cast<int>(rows), static_cast<int>(hidden),
+                            static_cast<float>(eps), dtype_code(xc, "x"), current_stream(xc)),
+           "add_rmsnorm");
+  return {sum, out};
+}
+
 // q [tokens, q_heads * D], k [tokens, kv_heads * D] (rows may be strided), cos / sin [tokens, D].
 std::tuple<at::Tensor, at::Tensor> rope_qk(const at::Tensor& q, const at::Tensor& k, const at::Tensor& cos,
                                            const at::Tensor& sin, int64_t q_heads, int64_t kv_heads) {
@@ -848,6 +871,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "Weight-only GEMM for a few dozen rows: fp16/bf16 activations x int4/int8 group-quantized weights, no dense copy",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("split") = false);
   m.def("rmsnorm", &rmsnorm, "LlamaRMSNorm over the last axis, one launch", py::arg("x"), py::arg("weight"), py::arg("eps"));
+  m.def("add_rmsnorm", &add_rmsnorm, "(x + delta, LlamaRMSNorm(x + delta)), one launch", py::arg("x"), py::arg("delta"),
+        py::arg("weight"), py::arg("eps"));
   m.def("rope_qk", &rope_qk, "apply_rotary_pos_emb on the q and k projections of a prompt, one launch",
         py::arg("q"), py::arg("k"), py::arg("cos"), py::arg("sin"), py::arg("q_heads"), py::arg("kv_heads"));
   m.def("silu_mul", &silu_mul, "silu(gate) * up with both roundings, one launch", py::arg("gate"), py::arg("up"));

@@ -121,6 +121,8 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_wq_gemm_a16_workspace_bytes.restype = ctypes.c_size_t
     lib.llmq_rmsnorm.argtypes = [c_p, c_p, c_p, c_int, c_int, ctypes.c_float, c_int, c_p]
     lib.llmq_rmsnorm.restype = c_int
+    lib.llmq_add_rmsnorm.argtypes = [c_p] * 5 + [c_int, c_int, ctypes.c_float, c_int, c_p]
+    lib.llmq_add_rmsnorm.restype = c_int
     lib.llmq_rope_qk.argtypes = [c_p] * 6 + [c_int] * 4 + [ctypes.c_int64] * 2 + [c_int, c_p]
     lib.llmq_rope_qk.restype = c_int
     lib.llmq_silu_mul.argtypes = [c_p, c_p, c_p, ctypes.c_int64, c_int, c_p]

@@ -91,6 +91,17 @@ class LlamaKernelRuntime:
             return self._ext.rmsnorm(x, module.weight, module.variance_epsilon)
         return module(x)
 
+    def _add_norm(self, module, hidden, branch):
+        """(hidden + branch, norm(hidden + branch)): the residual add in the launch of the norm after it.
+        branch None: (hidden, norm(hidden))."""
+        if branch is None:
+            return hidden, self._norm(module, hidden)
+        if (self._one_launch_ops and type(module).__name__.endswith("RMSNorm") and hasattr(module, "variance_epsilon")
+                and hidden.shape[-1] % 8 == 0 and module.weight.dtype == hidden.dtype and branch.dtype == hidden.dtype):
+            return self._ext.add_rmsnorm(hidden, branch, module.weight, module.variance_epsilon)
+        hidden = hidden + branch
+        return hidden, module(hidden)
+
     def _rotated(self, q, k, cos, sin):
         """q [T, Hq*D], k [T, Hkv*D] -> rotated [T, Hq, D], [T, Hkv, D]."""
         tokens = q.shape[0]
@@ -117,10 +128,13 @@ class LlamaKernelRuntime:
             return self._ext.silu_mul(gate, up)
         return mlp.act_fn(gate) * up
 
-    def _layer(self, index, layer, hidden, cos, sin, decode: bool):
+    def _layer(self, index, layer, hidden, cos, sin, decode: bool, branch=None, defer: bool = False):
+        """One decoder layer. `branch`: the previous layer's MLP output, still to be added to `hidden`
+        (done in the launch of this layer's first norm). `defer`: hand back (hidden, MLP output) and
+        leave the last add to the caller's next norm; otherwise the layer's output."""
         attn = layer.self_attn
         tokens = hidden.shape[0]
-        x = self._norm(layer.input_layernorm, hidden)
+        hidden, x = self._add_norm(layer.input_layernorm, hidden, branch)
         q, k, v = self._qkv(index, layer, x)
         v = v.view(tokens, self.kv_heads, self.head_dim)
         q, k = self._rotated(q, k, cos, sin)
@@ -137,16 +151,18 @@ class LlamaKernelRuntime:
                 ctx = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k_dq[None], v_dq[None],
                                                      is_causal=True, scale=self.scaling, enable_gqa=True)
                 ctx = ctx[0].transpose(0, 1).reshape(tokens, -1)
-        hidden = hidden + attn.o_proj(ctx)
-        x = self._norm(layer.post_attention_layernorm, hidden)
-        return hidden + layer.mlp.down_proj(self._gated(index, layer, x))
+        hidden, x = self._add_norm(layer.post_attention_layernorm, hidden, attn.o_proj(ctx))
+        out = layer.mlp.down_proj(self._gated(index, layer, x))
+        return (hidden, out) if defer else hidden + out
 
     def _forward(self, token_ids, cos, sin, decode: bool):
-        hidden = self.model.model.embed_tokens(token_ids)
+        hidden, branch = self.model.model.embed_tokens(token_ids), None
         for index, layer in enumerate(self.layers):
-            hidden = self._layer(index, layer, hidden, cos, sin, decode)
-        hidden = self._norm(self.model.model.norm, hidden[-1:].contiguous())
-        return self.model.lm_head(hidden)
+            hidden, branch = self._layer(index, layer, hidden, cos, sin, decode, branch, defer=True)
+        # only the last position goes on: its residual add and the final norm in one launch
+        _, last = self._add_norm(self.model.model.norm, hidden[-1:].contiguous(),
+                                 None if branch is None else branch[-1:].contiguous())
+        return self.model.lm_head(last)
 
     # ---- prefill ------------------------------------------------------------------------------------
     @torch.no_grad()

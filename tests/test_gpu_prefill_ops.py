@@ -48,6 +48,17 @@ def test_rmsnorm_matches_llama_rmsnorm(ext, dtype, rows, hidden):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_add_rmsnorm_is_the_add_then_the_norm(ext, dtype):
+    torch.manual_seed(4)
+    x = (torch.randn(33, 1024, device="cuda") * 2.0).to(dtype)
+    delta = torch.randn(33, 1024, device="cuda").to(dtype)
+    w = (torch.randn(1024, device="cuda") * 0.3 + 1.0).to(dtype)
+    total, normed = ext.add_rmsnorm(x, delta, w, 1e-5)
+    assert torch.equal(total, x + delta)
+    assert torch.equal(normed, ext.rmsnorm(x + delta, w, 1e-5))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("tokens,q_heads,kv_heads,head_dim", [(512, 32, 8, 64), (1, 32, 8, 64), (5, 8, 8, 128), (3, 4, 1, 16)])
 def test_rope_matches_apply_rotary_pos_emb(ext, dtype, tokens, q_heads, kv_heads, head_dim):
     from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
