@@ -59,7 +59,7 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the legs that report the path's other kernels and end-to-end decode")
-    ap.add_argument("--only", choices=("other", "decode"), default=None,
+    ap.add_argument("--only", choices=("other", "decode", "prefill"), default=None,
                     help="profiling aid: run just that leg and print its JSON (not the bench line)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="first run a plain 256 MiB device copy three times: the known-size kernel that "
@@ -116,7 +116,7 @@ def main():
     lib = load_capi()
     torch.cuda.set_device(0)
     if opts.only:
-        leg = other_kernels(torch) if opts.only == "other" else decode_leg(torch)
+        leg = {"other": other_kernels, "decode": decode_leg, "prefill": prefill_leg}[opts.only](torch)
         print(json.dumps({opts.only: leg}))
         return
     if opts.copy_probe:
@@ -565,6 +565,46 @@ def decode_leg(torch):
     del model
     torch.cuda.empty_cache()
     return res
+
+
+def prefill_leg(torch):
+    """The prompt pass of config 5 by itself: twelve 512-token prefills through the kernel runtime on the
+    random-init Llama-3.2-1B architecture (attention int8 / MLP int4 / lm_head int8 / int8 KV), wall time
+    and HIP events per call. The run to profile for what a time-to-first-token is made of."""
+    import time
+
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from llmquant import QuantConfig, oneshot
+    from llmquant.runtime import kernel_runtime
+
+    torch.manual_seed(0)
+    cfg = LlamaConfig(hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, num_attention_heads=32,
+                      num_key_value_heads=8, head_dim=64, vocab_size=128256, rms_norm_eps=1e-5,
+                      rope_parameters={"rope_type": "default", "rope_theta": 500000.0},
+                      tie_word_embeddings=False, max_position_embeddings=4096)
+    model = LlamaForCausalLM(cfg).to(torch.bfloat16).to("cuda:0").eval()
+    oneshot(model, QuantConfig(attn_weight="int8", mlp_weight="int4", head_weight="int8",
+                               kv_cache="int8").to_modifier("kernel"))
+    prompt = 512
+    ids = torch.randint(0, 128256, (1, prompt), generator=torch.Generator().manual_seed(1)).to("cuda:0")
+    wall, gpu = [], []
+    with torch.no_grad():
+        runtime = kernel_runtime(model, prompt + 2, 8)
+        for rep in range(15):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            a.record()
+            runtime.prefill(ids)
+            b.record()
+            torch.cuda.synchronize()
+            if rep >= 3:
+                wall.append((time.perf_counter() - t0) * 1e3)
+                gpu.append(a.elapsed_time(b))
+    wall.sort(), gpu.sort()
+    return {"prompt_tokens": prompt, "calls": len(wall), "runtime": type(runtime).__name__,
+            "median_wall_ms": round(wall[len(wall) // 2], 3), "median_events_ms": round(gpu[len(gpu) // 2], 3)}
 
 
 def cpu_baseline(torch, cases, budget_s: float):
