@@ -142,6 +142,22 @@ def test_kernel_mode_fails_loudly_without_a_gpu():
         KernelQuantLinear.from_linear(nn.Linear(128, 8), QuantizationScheme(weights=None, input_activations=None))
 
 
+def test_row_count_routing_of_the_kernel_mode_linear():
+    from llmquant.quantizers import FUSED_GEMM_MAX_ROWS, KERNEL_MAX_ROWS
+    from llmquant.quantizers.kernel import FUSED_GEMM_MIN_ROWS, FUSED_GEMM_WHOLE_ROWS, fused_gemm_splits
+
+    # the GEMV keeps the one- and two-row cases, the fused GEMM starts inside the GEMV's range
+    # (so there is no gap) and ends where the dense branch takes over
+    assert 1 < FUSED_GEMM_MIN_ROWS <= KERNEL_MAX_ROWS + 1
+    assert FUSED_GEMM_WHOLE_ROWS < FUSED_GEMM_MAX_ROWS == 64
+    # gate/up of Llama-3-8B (32 groups per row): whole rows up to 16 activation rows, split above
+    assert not fused_gemm_splits(3, 32) and not fused_gemm_splits(16, 32)
+    assert fused_gemm_splits(17, 32) and fused_gemm_splits(64, 32)
+    # down_proj (112 groups per row) has enough reduction axis to split at any row count
+    assert fused_gemm_splits(3, 112) and fused_gemm_splits(64, 112)
+    assert not fused_gemm_splits(8, 63) and fused_gemm_splits(8, 64)
+
+
 # ---- layout ---------------------------------------------------------------------------------------------
 
 def test_layout_geometry():
