@@ -30,7 +30,7 @@ sys.path[:0] = [str(ROOT / "llm-quant_amd")]
 
 GROUP = 128
 HBM_PEAK_GBPS = 8000.0  # MI355X, published
-SHAPES = [  # name, N, K  (BASELINE config 2)
+SHAPES = [  # name, N, K  (the linear layers of Llama-3.2-1B and its lm_head)
     ("q/o", 2048, 2048),
     ("k/v", 512, 2048),
     ("gate/up", 8192, 2048),
@@ -290,7 +290,7 @@ def _graph_time_us(torch, fn, reps=20):
 
 
 def other_kernels(torch):
-    """The path's other kernels, each on its BASELINE shape: fake-quant op, KV-cache decode
+    """The path's other kernels, each on the shape the reference quotes it on: fake-quant op, KV-cache decode
     step (config 4), W4A8 / W8A8 integer GEMM (config 3). Back-to-back launches, HIP events."""
     from llmquant.hip import load_extension
 
@@ -523,7 +523,7 @@ def other_kernels(torch):
 
 
 def decode_leg(torch):
-    """BASELINE config 5: random-init Llama-3.2-1B architecture, attention int8 / MLP int4 /
+    """The end-to-end decode case: random-init Llama-3.2-1B architecture, attention int8 / MLP int4 /
     lm_head int8 / int8 KV cache, 512-token prompt, 256 greedy tokens, batch 1. TTFT = median
     time of generating 1 token; decode tok/s = (n - 1) / (median time of n tokens - TTFT), the
     reference's definition (llmquant/eval/evaluate.py:209-218). Both sides replay a captured step."""

@@ -1,5 +1,5 @@
 """End-to-end decode on the kernel path: random-init Llama-architecture models, attention
-weights int8, MLP int4, lm_head int8, int8 KV cache (BASELINE config 5, at reduced and at
+weights int8, MLP int4, lm_head int8, int8 KV cache (the end-to-end decode case, at reduced and at
 full size).
 
 What is asserted, and why it is not plain token equality with the oracle model: the oracle
@@ -128,7 +128,7 @@ def test_teacher_forced_margin_small(small):
 
 
 def test_teacher_forced_margin_llama_1b_config():
-    """BASELINE config 5 at full size: 16 layers, hidden 2048, FFN 8192, 32/8 heads, vocab
+    """The end-to-end decode case at full size: 16 layers, hidden 2048, FFN 8192, 32/8 heads, vocab
     128256, prompt 512, 64 decoded tokens."""
     model = build_model(2048, 8192, 16, 32, 8, 128256)
     real, kernel = quantized_pair(model)

@@ -1,7 +1,7 @@
 """The integer prefill GEMM (int8 activations x int4/int8 weights) against the oracle's
 real-mode forward: activation codes and scales bit-exact, outputs bit-exact (the kernel keeps
 RealQuantLinear's rounding points and group order, llmquant/quantizers/real.py:94-99), at the
-reference's own test size, ragged sizes, and the BASELINE config-3 shapes via sampled entries."""
+reference's own test size, ragged sizes, and the Llama-3.2-1B prefill shapes via sampled entries."""
 
 import ctypes
 import pathlib
@@ -73,7 +73,7 @@ def test_matches_the_float64_closed_form(ext):
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
 @pytest.mark.parametrize("m", [128, 512, 2048])
 def test_llama_8b_mlp_shapes_on_sampled_entries(ext, n, k, m):
-    """BASELINE config 3 at full size (1% outlier channels x20): 64 x 64 sampled outputs,
+    """The 512-token prefill case at full size (1% outlier channels x20): 64 x 64 sampled outputs,
     bit-exact against the oracle restricted to those rows and columns."""
     got, (x, canonical, scales, _) = run_case(ext, m, n, k, 4, torch.bfloat16, seed=3, outliers=True)
     rng = np.random.default_rng(0)

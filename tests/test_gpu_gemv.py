@@ -1,5 +1,5 @@
 """The HIP GEMV against the CPU oracle (RealQuantLinear's arithmetic), on the reference's
-case list (reference tests/test_kernel_linear.py) and on the BASELINE layer shapes.
+case list (reference tests/test_kernel_linear.py) and on the Llama-3.2-1B layer shapes.
 
 Tolerances (stated by the task, not chosen to fit): rel-L2 <= 1e-3 against the float64
 closed form for fp32 outputs, <= 1e-2 for bf16/fp16 outputs. Codes, scales and packed bytes
@@ -121,7 +121,7 @@ SHAPES_1B = {"q/o": (2048, 2048), "k/v": (512, 2048), "gate/up": (8192, 2048), "
 @pytest.mark.parametrize("shape", list(SHAPES_1B))
 @pytest.mark.parametrize("bits", [8, 4])
 def test_llama_1b_layer_shapes(shape, bits):
-    """BASELINE configs 1-2: bf16 N(0, 0.02) weights, bf16 N(0, 1) activation, M=1."""
+    """The Llama-3.2-1B layer shapes: bf16 N(0, 0.02) weights, bf16 N(0, 1) activation, M=1."""
     from llmquant.hip import load_extension
 
     n, k = SHAPES_1B[shape]

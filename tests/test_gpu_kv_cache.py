@@ -126,7 +126,7 @@ def attention_case(ext, bits, dtype, q_heads, kv_heads, d, t_max, length, seed=0
 @pytest.mark.parametrize("bits", [8, 4])
 @pytest.mark.parametrize("length", [1, 15, 64, 777, 2049])
 def test_decode_attention_llama_1b_geometry(ext, bits, length):
-    """BASELINE config 4: 32 query heads, 8 kv heads, head_dim 64, context up to 2048 + 1."""
+    """The Llama-3.2-1B attention geometry: 32 query heads, 8 kv heads, head_dim 64, context up to 2048 + 1."""
     out, want, _ = attention_case(ext, bits, torch.bfloat16, 32, 8, 64, 2049, length)
     assert out.shape == (32, 64) and out.dtype == torch.bfloat16
     assert rel_l2(to_np(out), want) <= 1e-2
