@@ -11,7 +11,10 @@
 
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
+#include <hipblaslt/hipblaslt.h>
 
+#include <map>
+#include <mutex>
 #include <tuple>
 
 #include "llmq.h"
@@ -206,6 +209,103 @@ at::Tensor dequant_weight(const at::Tensor& qweight, const at::Tensor& wscale, i
                                packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype, current_stream(qweight)),
            "dequant_weight");
   return out;
+}
+
+// ---- the dense branch in one call: dequantize, then the BLAS library's matmul ----------------------
+// at::mm spends ~19 us of host time per call on this stack, most of it on building descriptors and
+// asking the library's heuristic again; a prompt pass makes four such calls per layer and the host
+// is what bounds it. Here the descriptors and the heuristic's first choice are kept per
+// (dtype, M, N, K) and a call costs ~10 us. The algorithm is the one at::mm gets from the same
+// heuristic, so the results are the same bits.
+struct DensePlan {
+  hipblasLtMatmulDesc_t desc = nullptr;
+  hipblasLtMatrixLayout_t w = nullptr, x = nullptr, out = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+};
+struct DenseState {
+  hipblasLtHandle_t handle = nullptr;
+  std::map<std::tuple<int, int64_t, int64_t, int64_t>, DensePlan> plans;
+  std::map<void*, at::Tensor> workspaces;  // one per stream: calls on two streams may overlap
+};
+constexpr int64_t kDenseWorkspaceBytes = 32 << 20;
+std::mutex g_dense_lock;
+
+DenseState& dense_state(int device) {
+  // never destroyed: at process exit the HIP runtime may already be gone when statics are torn down
+  static auto* states = new std::map<int, DenseState>;
+  return (*states)[device];
+}
+
+void check_lt(hipblasStatus_t status, const char* what) {
+  TORCH_CHECK(status == HIPBLAS_STATUS_SUCCESS, "hipBLASLt ", what, " failed with status ", static_cast<int>(status));
+}
+
+const DensePlan& dense_plan(DenseState& st, bool bf16, int64_t M, int64_t N, int64_t K) {
+  const auto key = std::make_tuple(static_cast<int>(bf16), M, N, K);
+  auto found = st.plans.find(key);
+  if (found != st.plans.end()) return found->second;
+  DensePlan p;
+  const hipDataType t = bf16 ? HIP_R_16BF : HIP_R_16F;
+  check_lt(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F), "MatmulDescCreate");
+  const hipblasOperation_t transposed = HIPBLAS_OP_T, plain = HIPBLAS_OP_N;
+  check_lt(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &transposed, sizeof(transposed)), "TRANSA");
+  check_lt(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &plain, sizeof(plain)), "TRANSB");
+  // in the library's column-major terms: out^T [N, M] = (w as [K, N])^T * (x as [K, M])
+  check_lt(hipblasLtMatrixLayoutCreate(&p.w, t, K, N, K), "MatrixLayoutCreate");
+  check_lt(hipblasLtMatrixLayoutCreate(&p.x, t, K, M, K), "MatrixLayoutCreate");
+  check_lt(hipblasLtMatrixLayoutCreate(&p.out, t, N, M, N), "MatrixLayoutCreate");
+  hipblasLtMatmulPreference_t pref = nullptr;
+  check_lt(hipblasLtMatmulPreferenceCreate(&pref), "MatmulPreferenceCreate");
+  const size_t cap = static_cast<size_t>(kDenseWorkspaceBytes);
+  check_lt(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &cap, sizeof(cap)),
+           "MAX_WORKSPACE_BYTES");
+  hipblasLtMatmulHeuristicResult_t results[4];
+  int n_results = 0;
+  const hipblasStatus_t status =
+      hipblasLtMatmulAlgoGetHeuristic(st.handle, p.desc, p.w, p.x, p.out, p.out, pref, 4, results, &n_results);
+  hipblasLtMatmulPreferenceDestroy(pref);
+  check_lt(status, "MatmulAlgoGetHeuristic");
+  int pick = -1;
+  for (int i = 0; i < n_results && pick < 0; ++i) {
+    if (results[i].state == HIPBLAS_STATUS_SUCCESS && results[i].workspaceSize <= cap) pick = i;
+  }
+  TORCH_CHECK(pick >= 0, "hipBLASLt offers no algorithm for a ", M, " x ", N, " x ", K, " matmul");
+  p.algo = results[pick].algo;
+  return st.plans.emplace(key, p).first->second;
+}
+
+at::Tensor dense_linear(const at::Tensor& x, const at::Tensor& w) {
+  TORCH_CHECK(x.is_cuda() && w.is_cuda(), "all tensors must be CUDA");
+  TORCH_CHECK(x.dim() == 2 && w.dim() == 2 && x.is_contiguous() && w.is_contiguous(),
+              "x [M, K] and w [N, K] must be contiguous matrices");
+  TORCH_CHECK(x.scalar_type() == at::kBFloat16 || x.scalar_type() == at::kHalf, "x must be float16 or bfloat16, got ",
+              x.scalar_type());
+  TORCH_CHECK(w.scalar_type() == x.scalar_type(), "w must have x's dtype");
+  TORCH_CHECK(x.size(1) == w.size(1), "x has ", x.size(1), " columns, w ", w.size(1));
+  const int64_t M = x.size(0), K = x.size(1), N = w.size(0);
+  auto out = at::empty({M, N}, x.options());
+  if (out.numel() == 0) return out;
+  if (K == 0) return out.zero_();
+  const c10::OptionalDeviceGuard guard(at::device_of(x));
+  const auto stream = c10::hip::getCurrentHIPStream(x.device().index());
+  const std::lock_guard<std::mutex> lock(g_dense_lock);
+  DenseState& st = dense_state(x.device().index());
+  if (st.handle == nullptr) check_lt(hipblasLtCreate(&st.handle), "Create");
+  at::Tensor& workspace = st.workspaces[static_cast<void*>(stream.stream())];
+  if (!workspace.defined()) workspace = at::empty({kDenseWorkspaceBytes}, x.options().dtype(at::kByte));
+  const DensePlan& plan = dense_plan(st, x.scalar_type() == at::kBFloat16, M, N, K);
+  const float one = 1.0f, zero = 0.0f;
+  check_lt(hipblasLtMatmul(st.handle, plan.desc, &one, w.const_data_ptr(), plan.w, x.const_data_ptr(), plan.x, &zero,
+                           out.const_data_ptr(), plan.out, out.mutable_data_ptr(), plan.out, &plan.algo,
+                           workspace.mutable_data_ptr(), static_cast<size_t>(kDenseWorkspaceBytes), stream.stream()),
+           "Matmul");
+  return out;
+}
+
+at::Tensor wq_dense_linear(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale, int64_t out_group,
+                           int64_t keep_per_group) {
+  TORCH_CHECK(x.is_cuda(), "x must be a CUDA tensor");
+  return dense_linear(x, dequant_weight(qweight, wscale, out_group, keep_per_group, x.scalar_type()));
 }
 
 // One activation row through a quantized Linear with the surrounding elementwise operations
@@ -897,6 +997,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "Dense [N, groups*keep_per_group] matrix of a quantized weight (keep_per_group <= 0: whole groups)",
         py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("keep_per_group") = 0,
         py::arg("out_dtype") = at::kBFloat16);
+  m.def("dense_linear", &dense_linear,
+        "x [M, K] @ w [N, K].T for float16 / bfloat16 through hipBLASLt with the descriptors and the heuristic's "
+        "choice kept per shape (the same algorithm, and bits, as torch's matmul at half the host time)",
+        py::arg("x"), py::arg("w"));
+  m.def("wq_dense_linear", &wq_dense_linear,
+        "The dense branch in one call: dequant_weight into x's dtype, then dense_linear",
+        py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("keep_per_group") = 0);
   m.def("kv_attend_partials_floats", [](int64_t q_heads, int64_t head_dim, int64_t n_splits) {
     return static_cast<int64_t>(llmq_kv_attend_partials_floats(static_cast<int>(q_heads), static_cast<int>(head_dim),
                                                                static_cast<int>(n_splits)));

@@ -126,13 +126,22 @@ class KernelQuantLinear(nn.Module):
             return self._ext.dequant_weight(self.qdata, self.wscale, self.out_group, keep, dtype)
         return (self.qweight * self._broadcast_scale).to(dtype).reshape(self.out_features, -1)
 
+    def _dense(self, rows, real_width: bool = False):
+        """rows @ W.T on the dense branch. bf16 / fp16: one extension call (dequantize pass, then the BLAS
+        library's matmul with its plan kept per shape: same bits as `@`, half the host time)."""
+        group_size = self.padded_in_features // self.qdata.shape[1]
+        if rows.dtype in (torch.bfloat16, torch.float16) and group_size % 8 == 0:
+            keep = self._head_keep if real_width else 0
+            return self._ext.wq_dense_linear(rows.contiguous(), self.qdata, self.wscale, self.out_group, keep)
+        return rows @ self._dequantized_weight(rows.dtype, real_width).T
+
     def forward(self, x):
         rows = x.reshape(-1, x.shape[-1])
         fused = (FUSED_GEMM_MIN_ROWS <= rows.shape[0] <= self._fused_max_rows
                  and rows.dtype in (torch.bfloat16, torch.float16) and not self._int8_act)
         if rows.shape[0] > KERNEL_MAX_ROWS and not self._int8_act and self._head_keep and not fused:
             # dense branch on the real width: neither the activation nor the weight is padded
-            out = rows @ self._dequantized_weight(rows.dtype, real_width=True).T
+            out = self._dense(rows, real_width=True)
             if self.bias is not None:
                 out = out + self.bias.to(out.dtype)
             return out.reshape(*x.shape[:-1], self.out_features).to(x.dtype)
@@ -149,7 +158,7 @@ class KernelQuantLinear(nn.Module):
         elif rows.shape[0] <= KERNEL_MAX_ROWS:
             out = self._gemv(rows, self.qdata, self.wscale, self.out_group)
         else:
-            out = rows @ self._dequantized_weight(rows.dtype).T
+            out = self._dense(rows)
         if self.bias is not None:
             out = out + self.bias.to(out.dtype)
         return out.reshape(*x.shape[:-1], self.out_features).to(x.dtype)

@@ -131,6 +131,8 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
                                          fused_gemm_splits(rows, fused.qdata.shape[1]))
         if rows <= KERNEL_MAX_ROWS:
             return self._ext.wq_gemv(x, fused.qdata, fused.wscale, fused.out_group)
+        if x.dtype in (torch.bfloat16, torch.float16):
+            return self._ext.wq_dense_linear(x.contiguous(), fused.qdata, fused.wscale, fused.out_group, 0)
         return x @ self._ext.dequant_weight(fused.qdata, fused.wscale, fused.out_group, 0, x.dtype).T
 
     def _qkv(self, index, layer, x):

@@ -304,7 +304,7 @@ def test_a_few_dozen_rows_take_the_fused_gemm(name, M, linear):
     spec = dict(LAYOUTS[name])
     bits = spec.pop("bits")
     module = KernelQuantLinear.from_linear(linear.cuda(), weight_only(bits, **spec))
-    module._dequantized_weight = None  # the dense branch would fail loudly
+    module._dequantized_weight = module._dense = None  # the dense branch would fail loudly
     torch.manual_seed(M)
     x = torch.randn(M, K).to(torch.bfloat16)
     got = module(x.cuda())
@@ -428,3 +428,57 @@ def test_dequant_weight_is_code_times_scale_rounded_once(bits, dtype):
             assert torch.equal(odd.cpu(), want[:, :, :20].reshape(n, -1))
     with pytest.raises(RuntimeError, match="keep_per_group"):
         ext.dequant_weight(q, s, 32, 200, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_dense_linear_is_the_library_matmul_with_a_kept_plan(dtype):
+    """The dense branch's matmul: hipBLASLt through a plan kept per shape. Checked against the
+    fp64 product (the tolerance of a bf16 / fp16 GEMM with fp32 accumulation), against torch's
+    own matmul, and for repeat calls and several shapes sharing the one workspace."""
+    from llmquant.hip import load_extension
+
+    ext = load_extension()
+    gen = torch.Generator().manual_seed(21)
+    for (m, n, k) in [(72, 256, 384), (512, 3072, 2048), (100, 2048, 2048), (65, 96, 128), (300, 200, 136)]:
+        x = torch.randn(m, k, generator=gen).to(dtype).cuda()
+        w = (torch.randn(n, k, generator=gen) * 0.05).to(dtype).cuda()
+        want = (x.double() @ w.double().T).cpu().numpy()
+        first = ext.dense_linear(x, w)
+        again = ext.dense_linear(x, w)
+        assert first.shape == (m, n) and first.dtype == dtype
+        assert torch.equal(first, again), (m, n, k)
+        assert rel_l2(to_np(first), want) <= (1e-2 if dtype == torch.bfloat16 else 2e-3), (m, n, k)
+        assert rel_l2(to_np(first), to_np(x @ w.T)) <= 1e-3, (m, n, k)   # in practice the same bits
+    assert ext.dense_linear(x[:0], w).shape == (0, n)
+    with pytest.raises(RuntimeError, match="float16 or bfloat16"):
+        ext.dense_linear(x.float(), w.float())
+    with pytest.raises(RuntimeError, match="columns"):
+        ext.dense_linear(x, w[:, :-8].contiguous())
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ext.dense_linear(x, w.T)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        ext.dense_linear(x.cpu(), w)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_wq_dense_linear_is_dequantize_then_matmul(bits):
+    """One call for the dense branch: the dequantized matrix (bit-exact, tested above) times x, whole
+    groups and with the head padding dropped, against the fp64 product with that same matrix."""
+    from llmquant.hip import load_extension
+
+    ext = load_extension()
+    gen = torch.Generator().manual_seed(5)
+    n, heads, head_dim, m = 96, 6, 64, 80
+    w = (torch.randn(n, heads * head_dim, generator=gen) * 0.05).to(torch.bfloat16)
+    for hd, out_group in ((None, None), (head_dim, None), (None, 32)):
+        canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP, hd, out_group)
+        q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
+        s = torch.from_numpy(scales).cuda()
+        for keep in ((0, hd) if hd else (0,)):
+            dense = ext.dequant_weight(q, s, out_group or 0, keep, torch.bfloat16)
+            x = torch.randn(m, dense.shape[1], generator=gen).to(torch.bfloat16).cuda()
+            got = ext.wq_dense_linear(x, q, s, out_group or 0, keep)
+            want = (x.double() @ dense.double().T).cpu().numpy()
+            assert got.shape == (m, n) and got.dtype == torch.bfloat16
+            assert rel_l2(to_np(got), want) <= 1e-2, (hd, out_group, keep)
+            assert torch.equal(got, ext.dense_linear(x, dense))
