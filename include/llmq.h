@@ -240,6 +240,21 @@ int llmq_kv_append(const void* k_new, const void* v_new, int64_t head_stride,
                    const int32_t* pos_dev, int n_new, int kv_heads, int head_dim, int t_max,
                    int bits, int dtype, llmq_stream_t stream);
 
+/* The prompt pass's RoPE and append in one launch: equivalent to llmq_rope_qk on q and k followed
+ * by llmq_kv_append of the rotated k and of v, bit for bit (the rotated key is rounded to `dtype`
+ * before it is quantized, as the tensor between the two launches would be). q / k / v: [tokens,
+ * heads, head_dim] with the given element strides between tokens (column blocks of one q|k|v
+ * projection output work); cos_rows / sin_rows: [tokens, head_dim]; q_out: [tokens, q_heads,
+ * head_dim]; dq_k / dq_v: [kv_heads, tokens, head_dim] or both NULL. head_dim 64 or 128. No
+ * counterpart in the reference, which runs apply_rotary_pos_emb and FakeQuantCache.update as
+ * PyTorch chains (llmquant/quantizers/fake.py:39-55). */
+int llmq_rope_kv_append(const void* q, const void* k, const void* v, int64_t q_row_stride,
+                        int64_t k_row_stride, int64_t v_row_stride, const void* cos_rows,
+                        const void* sin_rows, void* q_out, void* k_codes, void* v_codes, float* k_scale,
+                        float* v_scale, void* dq_k_or_null, void* dq_v_or_null, const int32_t* pos_dev,
+                        int tokens, int q_heads, int kv_heads, int head_dim, int t_max, int bits,
+                        int dtype, llmq_stream_t stream);
+
 /* Dequantize positions 0 .. n_tokens-1 of one layer's cache to [kv_heads, n_tokens, head_dim]
  * `dtype`: (dtype)(code * scale), the tensor FakeQuantCache.update returns
  * (llmquant/quantizers/fake.py:52-55) when attention is not run by the fused decode kernel. */

@@ -74,6 +74,90 @@ __global__ __launch_bounds__(256) void kv_append_kernel(
   }
 }
 
+// ---- prompt pass: RoPE on q and k, then the append, in one launch -----------------------------------
+// One wave per (token, head) over the query, key and value heads of a token, heads of a token side
+// by side so that a row of the q|k|v projection is read in order. Lane l holds elements l and
+// l + 64 of the head vector, as in kv_append_kernel; the RoPE partner of element i is i +- D/2, the
+// same lane for D = 128 and lane l ^ 32 for D = 64. Query waves rotate and store; key waves rotate,
+// round to T (the tensor the two-launch path hands to the append) and quantize; value waves quantize.
+template <typename T, int BITS, int D>
+__global__ __launch_bounds__(256) void rope_kv_append_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const int64_t q_stride,
+    const int64_t k_stride, const int64_t v_stride, const T* __restrict__ cos_rows,
+    const T* __restrict__ sin_rows, T* __restrict__ q_out, uint8_t* __restrict__ k_codes,
+    uint8_t* __restrict__ v_codes, float* __restrict__ k_scale, float* __restrict__ v_scale,
+    T* __restrict__ dq_k, T* __restrict__ dq_v, const int32_t* __restrict__ pos_dev, const int tokens,
+    const int q_heads, const int kv_heads, const int t_max) {
+  static_assert(D == 64 || D == 128, "lane layout below");
+  constexpr int E = D / kWave;  // elements per lane
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
+  const int heads = q_heads + 2 * kv_heads;
+  if (wave >= static_cast<int64_t>(tokens) * heads) return;  // whole waves leave together
+  const int tok = static_cast<int>(wave / heads);
+  const int h = static_cast<int>(wave - static_cast<int64_t>(tok) * heads);
+  const bool is_q = h < q_heads;
+  const bool is_v = h >= q_heads + kv_heads;
+  const int head = is_q ? h : (is_v ? h - q_heads - kv_heads : h - q_heads);
+  const T* src = is_q   ? q + tok * q_stride + static_cast<int64_t>(head) * D
+                 : is_v ? v + tok * v_stride + static_cast<int64_t>(head) * D
+                        : k + tok * k_stride + static_cast<int64_t>(head) * D;
+  float f[2] = {0.0f, 0.0f};
+#pragma unroll
+  for (int e = 0; e < E; ++e) f[e] = to_float(src[lane + e * kWave]);
+
+  if (!is_v) {
+    float rot[2] = {0.0f, 0.0f};
+    if constexpr (D == 128) {
+      rot[0] = -f[1];
+      rot[1] = f[0];
+    } else {
+      const float other = __shfl_xor(f[0], 32, kWave);
+      rot[0] = lane < 32 ? -other : other;
+    }
+    const T* cos_row = cos_rows + static_cast<int64_t>(tok) * D;
+    const T* sin_row = sin_rows + static_cast<int64_t>(tok) * D;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const float a = round_through<T>(f[e] * to_float(cos_row[lane + e * kWave]));
+      const float b = round_through<T>(rot[e] * to_float(sin_row[lane + e * kWave]));
+      f[e] = round_through<T>(a + b);
+    }
+  }
+  if (is_q) {
+    T* dst = q_out + (static_cast<int64_t>(tok) * q_heads + head) * D;
+#pragma unroll
+    for (int e = 0; e < E; ++e) dst[lane + e * kWave] = from_float<T>(f[e]);
+    return;
+  }
+
+  const int pos = pos_dev[0] + tok;
+  if (pos < 0 || pos >= t_max) return;
+  const float qmax = static_cast<float>((1 << (BITS - 1)) - 1);
+  const float qmin = -qmax - 1.0f;
+  float amax = fmaxf(fabsf(f[0]), fabsf(f[1]));
+  amax = group_max<kWave>(amax);
+  const float scale = scale_from_amax(amax, qmax);
+  const int64_t slot = static_cast<int64_t>(head) * t_max + pos;
+  if (lane == 0) (is_v ? v_scale : k_scale)[slot] = scale;
+  uint8_t* codes = is_v ? v_codes : k_codes;
+  T* dq = is_v ? dq_v : dq_k;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int d = lane + e * kWave;
+    const float qv = quant_code(f[e], scale, qmin, qmax);
+    if (dq != nullptr) dq[(static_cast<int64_t>(head) * tokens + tok) * D + d] = from_float<T>(qv * scale);
+    const int code = static_cast<int>(qv);
+    if constexpr (BITS == 8) {
+      codes[slot * D + d] = static_cast<uint8_t>(code);
+    } else {
+      const int mine = (code + 8) & 0xf;
+      const int other = dpp<kDppXor1>(mine);
+      if ((lane & 1) == 0) codes[slot * (D / 2) + d / 2] = static_cast<uint8_t>(mine | (other << 4));
+    }
+  }
+}
+
 // ---- dequantize a range of the cache (what update() hands back outside of decode) ---------------
 template <typename T, int BITS>
 __global__ __launch_bounds__(256) void kv_dequant_kernel(
@@ -837,6 +921,50 @@ extern "C" int llmq_kv_append(const void* k_new, const void* v_new, int64_t head
   }
 #undef LLMQ_APPEND
   return llmq_host::check_launch("kv_append_kernel");
+}
+
+extern "C" int llmq_rope_kv_append(const void* q, const void* k, const void* v, int64_t q_row_stride,
+                                   int64_t k_row_stride, int64_t v_row_stride, const void* cos_rows,
+                                   const void* sin_rows, void* q_out, void* k_codes, void* v_codes, float* k_scale,
+                                   float* v_scale, void* dq_k_or_null, void* dq_v_or_null, const int32_t* pos_dev,
+                                   int tokens, int q_heads, int kv_heads, int head_dim, int t_max, int bits,
+                                   int dtype, llmq_stream_t stream) {
+  if (bits != 8 && bits != 4) return llmq_host::fail_invalid("KV cache bits must be 8 or 4, got %d", bits);
+  if (head_dim != 64 && head_dim != 128) return llmq_host::fail_invalid("head_dim must be 64 or 128, got %d", head_dim);
+  if (tokens < 0 || q_heads < 0 || kv_heads < 0 || t_max < 0) return llmq_host::fail_invalid("negative size");
+  if (dtype != LLMQ_F32 && dtype != LLMQ_F16 && dtype != LLMQ_BF16)
+    return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+  if (tokens == 0 || q_heads + kv_heads == 0) return 0;
+  if (!cos_rows || !sin_rows || !pos_dev || (q_heads && (!q || !q_out)) ||
+      (kv_heads && (!k || !v || !k_codes || !v_codes || !k_scale || !v_scale)))
+    return llmq_host::fail_invalid("null tensor pointer");
+  if ((dq_k_or_null == nullptr) != (dq_v_or_null == nullptr))
+    return llmq_host::fail_invalid("dq_k and dq_v go together");
+  const int64_t waves = static_cast<int64_t>(tokens) * (q_heads + 2 * kv_heads);
+  const dim3 grid(static_cast<unsigned>((waves + 3) / 4)), block(256);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define LLMQ_ROPE_APPEND(T, B, D)                                                                          \
+  hipLaunchKernelGGL((rope_kv_append_kernel<T, B, D>), grid, block, 0, s, static_cast<const T*>(q),         \
+                     static_cast<const T*>(k), static_cast<const T*>(v), q_row_stride, k_row_stride,        \
+                     v_row_stride, static_cast<const T*>(cos_rows), static_cast<const T*>(sin_rows),        \
+                     static_cast<T*>(q_out), static_cast<uint8_t*>(k_codes), static_cast<uint8_t*>(v_codes), \
+                     k_scale, v_scale, static_cast<T*>(dq_k_or_null), static_cast<T*>(dq_v_or_null), pos_dev, \
+                     tokens, q_heads, kv_heads, t_max)
+#define LLMQ_ROPE_APPEND_T(T)                                             \
+  do {                                                                    \
+    if (bits == 8 && head_dim == 64) LLMQ_ROPE_APPEND(T, 8, 64);          \
+    else if (bits == 8) LLMQ_ROPE_APPEND(T, 8, 128);                      \
+    else if (head_dim == 64) LLMQ_ROPE_APPEND(T, 4, 64);                  \
+    else LLMQ_ROPE_APPEND(T, 4, 128);                                     \
+  } while (0)
+  switch (dtype) {
+    case LLMQ_F32: LLMQ_ROPE_APPEND_T(float); break;
+    case LLMQ_F16: LLMQ_ROPE_APPEND_T(f16_t); break;
+    default: LLMQ_ROPE_APPEND_T(bf16_t); break;
+  }
+#undef LLMQ_ROPE_APPEND_T
+#undef LLMQ_ROPE_APPEND
+  return llmq_host::check_launch("rope_kv_append_kernel");
 }
 
 extern "C" int llmq_kv_dequant(const void* codes, const float* scale, void* out, int kv_heads,

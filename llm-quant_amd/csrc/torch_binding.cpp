@@ -228,6 +228,7 @@ struct DenseState {
   std::map<void*, at::Tensor> workspaces;  // one per stream: calls on two streams may overlap
 };
 constexpr int64_t kDenseWorkspaceBytes = 32 << 20;
+constexpr size_t kDenseMaxPlans = 4096;
 std::mutex g_dense_lock;
 
 DenseState& dense_state(int device) {
@@ -244,6 +245,15 @@ const DensePlan& dense_plan(DenseState& st, bool bf16, int64_t M, int64_t N, int
   const auto key = std::make_tuple(static_cast<int>(bf16), M, N, K);
   auto found = st.plans.find(key);
   if (found != st.plans.end()) return found->second;
+  if (st.plans.size() >= kDenseMaxPlans) {  // a caller with ever-changing row counts: start over
+    for (auto& kept : st.plans) {
+      hipblasLtMatmulDescDestroy(kept.second.desc);
+      hipblasLtMatrixLayoutDestroy(kept.second.w);
+      hipblasLtMatrixLayoutDestroy(kept.second.x);
+      hipblasLtMatrixLayoutDestroy(kept.second.out);
+    }
+    st.plans.clear();
+  }
   DensePlan p;
   const hipDataType t = bf16 ? HIP_R_16BF : HIP_R_16F;
   check_lt(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F), "MatmulDescCreate");
@@ -721,6 +731,55 @@ std::tuple<at::Tensor, at::Tensor> kv_append(const at::Tensor& key, const at::Te
   return std::make_tuple(dq_k, dq_v);
 }
 
+// q [tokens, q_heads*head_dim], k / v [tokens, kv_heads*head_dim]: rows of the projections (column
+// slices of one q|k|v output are fine). Returns (q rotated [tokens, q_heads, head_dim], dq_k, dq_v
+// [kv_heads, tokens, head_dim]; the last two empty without return_dequantized).
+std::tuple<at::Tensor, at::Tensor, at::Tensor> rope_kv_append(
+    const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& cos, const at::Tensor& sin,
+    at::Tensor& k_codes, at::Tensor& v_codes, at::Tensor& k_scale, at::Tensor& v_scale, const at::Tensor& position,
+    int64_t q_heads, bool return_dequantized) {
+  TORCH_CHECK(q.is_cuda() && k.is_cuda() && v.is_cuda() && cos.is_cuda() && sin.is_cuda(), "all tensors must be CUDA");
+  TORCH_CHECK(q.dim() == 2 && k.dim() == 2 && v.dim() == 2 && q.stride(1) == 1 && k.stride(1) == 1 && v.stride(1) == 1,
+              "q, k and v must be [tokens, heads * head_dim] with a contiguous last axis");
+  const int dtype = dtype_code(q, "q");
+  TORCH_CHECK(k.scalar_type() == q.scalar_type() && v.scalar_type() == q.scalar_type() &&
+                  cos.scalar_type() == q.scalar_type() && sin.scalar_type() == q.scalar_type(),
+              "q, k, v, cos and sin must share a dtype");
+  const CacheGeometry g = cache_geometry(k_codes, k_scale, "key");
+  const CacheGeometry gv = cache_geometry(v_codes, v_scale, "value");
+  TORCH_CHECK(g.kv_heads == gv.kv_heads && g.t_max == gv.t_max && g.head_dim == gv.head_dim && g.bits == gv.bits,
+              "key and value caches differ in geometry");
+  const int64_t tokens = q.size(0);
+  TORCH_CHECK(q_heads > 0 && q.size(1) == q_heads * g.head_dim, "q has ", q.size(1), " columns, expected ",
+              q_heads * g.head_dim);
+  TORCH_CHECK(k.size(0) == tokens && v.size(0) == tokens && k.size(1) == g.kv_heads * g.head_dim &&
+                  v.size(1) == k.size(1),
+              "k and v must be [", tokens, ", ", g.kv_heads * g.head_dim, "]");
+  TORCH_CHECK(cos.dim() == 2 && cos.is_contiguous() && sin.is_contiguous() && cos.sizes() == sin.sizes() &&
+                  cos.size(0) == tokens && cos.size(1) == g.head_dim,
+              "cos and sin must be contiguous [tokens, head_dim]");
+  check_position(position);
+  auto q_out = at::empty({tokens, q_heads, g.head_dim}, q.options());
+  at::Tensor dq_k = at::empty({0}, q.options()), dq_v = at::empty({0}, q.options());
+  if (return_dequantized) {
+    dq_k = at::empty({g.kv_heads, tokens, g.head_dim}, q.options());
+    dq_v = at::empty({g.kv_heads, tokens, g.head_dim}, q.options());
+  }
+  if (tokens == 0) return std::make_tuple(q_out, dq_k, dq_v);
+  const c10::OptionalDeviceGuard guard(at::device_of(q));
+  check_rc(llmq_rope_kv_append(q.const_data_ptr(), k.const_data_ptr(), v.const_data_ptr(), q.stride(0), k.stride(0),
+                               v.stride(0), cos.const_data_ptr(), sin.const_data_ptr(), q_out.mutable_data_ptr(),
+                               k_codes.mutable_data_ptr(), v_codes.mutable_data_ptr(),
+                               k_scale.mutable_data_ptr<float>(), v_scale.mutable_data_ptr<float>(),
+                               return_dequantized ? dq_k.mutable_data_ptr() : nullptr,
+                               return_dequantized ? dq_v.mutable_data_ptr() : nullptr,
+                               position.const_data_ptr<int32_t>(), static_cast<int>(tokens),
+                               static_cast<int>(q_heads), g.kv_heads, g.head_dim, g.t_max, g.bits, dtype,
+                               current_stream(q)),
+           "rope_kv_append");
+  return std::make_tuple(q_out, dq_k, dq_v);
+}
+
 at::Tensor kv_dequant(const at::Tensor& codes, const at::Tensor& scale, int64_t n_tokens,
                       at::ScalarType out_dtype) {
   const CacheGeometry g = cache_geometry(codes, scale, "cache");
@@ -980,6 +1039,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "Quantize new K/V tokens into one layer's cache at the device-side position",
         py::arg("key"), py::arg("value"), py::arg("k_codes"), py::arg("v_codes"), py::arg("k_scale"),
         py::arg("v_scale"), py::arg("position"), py::arg("return_dequantized") = false);
+  m.def("rope_kv_append", &rope_kv_append,
+        "Prompt pass: RoPE on q and k, then quantize-and-append of k and v, in one launch (rope_qk + kv_append, same bits)",
+        py::arg("q"), py::arg("k"), py::arg("v"), py::arg("cos"), py::arg("sin"), py::arg("k_codes"),
+        py::arg("v_codes"), py::arg("k_scale"), py::arg("v_scale"), py::arg("position"), py::arg("q_heads"),
+        py::arg("return_dequantized") = false);
   m.def("kv_dequant", &kv_dequant, "Dequantize the first n_tokens of one layer's cache",
         py::arg("codes"), py::arg("scale"), py::arg("n_tokens"), py::arg("out_dtype"));
   m.def("kv_decode_workspace_floats", &kv_decode_workspace_floats, py::arg("q_heads"),

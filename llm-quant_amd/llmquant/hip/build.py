@@ -125,6 +125,8 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_add_rmsnorm.restype = c_int
     lib.llmq_rope_qk.argtypes = [c_p] * 6 + [c_int] * 4 + [ctypes.c_int64] * 2 + [c_int, c_p]
     lib.llmq_rope_qk.restype = c_int
+    lib.llmq_rope_kv_append.argtypes = ([c_p] * 3 + [ctypes.c_int64] * 3 + [c_p] * 10 + [c_int] * 7 + [c_p])
+    lib.llmq_rope_kv_append.restype = c_int
     lib.llmq_silu_mul.argtypes = [c_p, c_p, c_p, ctypes.c_int64, c_int, c_p]
     lib.llmq_silu_mul.restype = c_int
     lib.llmq_silu_mul_rows.argtypes = [c_p, c_p, c_p, ctypes.c_int64, c_int, ctypes.c_int64, ctypes.c_int64, c_int, c_p]

@@ -110,6 +110,12 @@ class LlamaKernelRuntime:
         return self._rope(q.view(tokens, self.q_heads, self.head_dim), k.view(tokens, self.kv_heads, self.head_dim),
                           cos, sin)
 
+    def _rope_append_in_one_launch(self, q, k, v, cos):
+        """RoPE and the cache append of a prompt as one launch (llmq_rope_kv_append): stock rotation,
+        heads of 64 or 128, rows of the projections with a contiguous last axis."""
+        return (self._one_launch_ops and self.head_dim in (64, 128) and q.dtype == cos.dtype and cos.is_contiguous()
+                and all(t.dim() == 2 and t.stride(1) == 1 for t in (q, k, v)))
+
     def _qkv(self, index, layer, x):
         """The three projections of a layer, each [tokens, heads * head_dim]."""
         attn = layer.self_attn
@@ -136,21 +142,30 @@ class LlamaKernelRuntime:
         tokens = hidden.shape[0]
         hidden, x = self._add_norm(layer.input_layernorm, hidden, branch)
         q, k, v = self._qkv(index, layer, x)
-        v = v.view(tokens, self.kv_heads, self.head_dim)
-        q, k = self._rotated(q, k, cos, sin)
-        if decode:
-            self.cache.append(index, k.transpose(0, 1), v.transpose(0, 1))
-            ctx = self.cache.attend(index, q[0].contiguous(), self.scaling).reshape(1, -1)
+        k_dq = v_dq = None
+        if not decode and self._rope_append_in_one_launch(q, k, v, cos):
+            cache = self.cache
+            q, k_dq, v_dq = self._ext.rope_kv_append(q, k, v, cos, sin, cache.k_codes[index], cache.v_codes[index],
+                                                     cache.k_scale[index], cache.v_scale[index], cache.position,
+                                                     self.q_heads, True)
         else:
+            if v.stride(0) != self.kv_heads * self.head_dim:
+                v = v.contiguous()  # the append wants k's strides, and k comes out of the rotation contiguous
+            v = v.view(tokens, self.kv_heads, self.head_dim)
+            q, k = self._rotated(q, k, cos, sin)
+            appended = self.cache.append(index, k.transpose(0, 1), v.transpose(0, 1), return_dequantized=not decode)
+            if not decode:
+                k_dq, v_dq = appended
+        if decode:
+            ctx = self.cache.attend(index, q[0].contiguous(), self.scaling).reshape(1, -1)
+        elif self.exact_prefill:
             # prompt: attention sees the fake-quantized K/V of the prompt itself, which is what
             # FakeQuantCache.update returns on an empty cache
-            k_dq, v_dq = self.cache.append(index, k.transpose(0, 1), v.transpose(0, 1), return_dequantized=True)
-            if self.exact_prefill:
-                ctx = self._fp32_causal_attention(q, k_dq, v_dq)
-            else:
-                ctx = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k_dq[None], v_dq[None],
-                                                     is_causal=True, scale=self.scaling, enable_gqa=True)
-                ctx = ctx[0].transpose(0, 1).reshape(tokens, -1)
+            ctx = self._fp32_causal_attention(q, k_dq, v_dq)
+        else:
+            ctx = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k_dq[None], v_dq[None],
+                                                 is_causal=True, scale=self.scaling, enable_gqa=True)
+            ctx = ctx[0].transpose(0, 1).reshape(tokens, -1)
         hidden, x = self._add_norm(layer.post_attention_layernorm, hidden, attn.o_proj(ctx))
         out = layer.mlp.down_proj(self._gated(index, layer, x))
         return (hidden, out) if defer else hidden + out

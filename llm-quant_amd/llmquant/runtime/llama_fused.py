@@ -138,8 +138,7 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
     def _qkv(self, index, layer, x):
         out = self._project(x, self.fused_layers[index]["qkv"])
         q_width, kv_width = self.q_heads * self.head_dim, self.kv_heads * self.head_dim
-        # (the cache append wants k and v with the same strides: k comes out of the rotation contiguous)
-        return out[:, :q_width], out[:, q_width:q_width + kv_width], out[:, q_width + kv_width:].contiguous()
+        return out[:, :q_width], out[:, q_width:q_width + kv_width], out[:, q_width + kv_width:]
 
     def _gate_up(self, index, layer, x):
         out = self._project(x, self.fused_layers[index]["gate_up"])

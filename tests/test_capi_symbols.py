@@ -123,3 +123,18 @@ def test_prompt_pass_argument_checks_need_no_device(lib):
     assert b"row strides" in lib.llmq_last_error()
     assert lib.llmq_silu_mul_rows(None, None, None, 4, 8192, 16384, 16384, 2, None) == 1
     assert b"null tensor pointer" in lib.llmq_last_error()
+
+
+def test_rope_and_append_argument_checks_need_no_device(lib):
+    # (q, k, v, q_row_stride, k_row_stride, v_row_stride, cos, sin, q_out, k_codes, v_codes, k_scale, v_scale,
+    #  dq_k, dq_v, pos, tokens, q_heads, kv_heads, head_dim, t_max, bits, dtype, stream)
+    nulls = [None] * 3 + [3072] * 3 + [None] * 10
+    assert lib.llmq_rope_kv_append(*nulls, 4, 32, 8, 64, 16, 6, 2, None) == 1
+    assert b"bits must be 8 or 4" in lib.llmq_last_error()
+    assert lib.llmq_rope_kv_append(*nulls, 4, 32, 8, 96, 16, 8, 2, None) == 1
+    assert b"head_dim must be 64 or 128" in lib.llmq_last_error()
+    assert lib.llmq_rope_kv_append(*nulls, 4, 32, 8, 64, 16, 8, 9, None) == 1
+    assert b"dtype" in lib.llmq_last_error()
+    assert lib.llmq_rope_kv_append(*nulls, 4, 32, 8, 64, 16, 8, 2, None) == 1
+    assert b"null tensor pointer" in lib.llmq_last_error()
+    assert lib.llmq_rope_kv_append(*nulls, 0, 32, 8, 64, 16, 8, 2, None) == 0   # no tokens: nothing to do

@@ -152,6 +152,74 @@ def test_prompt_pass_with_one_projection_per_group_matches_the_module_walk():
         assert torch.equal(plain.cache.k_codes[0, :, :tokens], fused.cache.k_codes[0, :, :tokens])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("tokens,q_heads,kv_heads,head_dim,start",
+                         [(512, 32, 8, 64, 0), (5, 8, 8, 128, 3), (1, 4, 1, 64, 9), (37, 6, 2, 128, 0)])
+def test_rope_and_append_in_one_launch_equal_the_two_launches(ext, dtype, bits, tokens, q_heads, kv_heads, head_dim, start):
+    """llmq_rope_kv_append against llmq_rope_qk followed by llmq_kv_append (each tested on its own
+    against transformers and the oracle): the same rotated query, codes, scales and dequantized K/V,
+    to the bit, with q | k | v as column blocks of one projection output and a non-zero start position."""
+    from llmquant.runtime.kv_cache import KernelQuantCache
+
+    torch.manual_seed(tokens * 7 + head_dim + bits)
+    qkv = (torch.randn(tokens, (q_heads + 2 * kv_heads) * head_dim, device="cuda") * 2.0).to(dtype)
+    q_width, kv_width = q_heads * head_dim, kv_heads * head_dim
+    q, k, v = qkv[:, :q_width], qkv[:, q_width:q_width + kv_width], qkv[:, q_width + kv_width:]
+    freqs = torch.rand(tokens, head_dim // 2, device="cuda") * 6.28
+    emb = torch.cat((freqs, freqs), dim=-1)
+    cos, sin = emb.cos().to(dtype), emb.sin().to(dtype)
+    max_len = start + tokens + 2
+    two, one = (KernelQuantCache(1, kv_heads, head_dim, max_len, bits, q_heads=q_heads) for _ in range(2))
+    two.set_position(start)
+    one.set_position(start)
+
+    want_q, rotated_k = ext.rope_qk(q, k, cos, sin, q_heads, kv_heads)
+    want_k_dq, want_v_dq = two.append(0, rotated_k.transpose(0, 1),
+                                      v.contiguous().view(tokens, kv_heads, head_dim).transpose(0, 1),
+                                      return_dequantized=True)
+    got_q, got_k_dq, got_v_dq = ext.rope_kv_append(q, k, v, cos, sin, one.k_codes[0], one.v_codes[0], one.k_scale[0],
+                                                   one.v_scale[0], one.position, q_heads, True)
+    assert got_q.shape == (tokens, q_heads, head_dim) and got_k_dq.shape == (kv_heads, tokens, head_dim)
+    assert torch.equal(got_q, want_q)
+    assert torch.equal(got_k_dq, want_k_dq) and torch.equal(got_v_dq, want_v_dq)
+    assert torch.equal(one.k_codes, two.k_codes) and torch.equal(one.v_codes, two.v_codes)
+    assert torch.equal(one.k_scale, two.k_scale) and torch.equal(one.v_scale, two.v_scale)
+    assert float(one.k_scale[0, :, start:start + tokens].min()) > 0.0   # ... and something was written
+    # without the dequantized copies: the same cache contents
+    bare = KernelQuantCache(1, kv_heads, head_dim, max_len, bits, q_heads=q_heads)
+    bare.set_position(start)
+    _, none_k, none_v = ext.rope_kv_append(q, k, v, cos, sin, bare.k_codes[0], bare.v_codes[0], bare.k_scale[0],
+                                           bare.v_scale[0], bare.position, q_heads, False)
+    assert none_k.numel() == 0 and none_v.numel() == 0
+    assert torch.equal(bare.k_codes, two.k_codes) and torch.equal(bare.v_scale, two.v_scale)
+
+
+def test_rope_and_append_argument_checks(ext):
+    from llmquant.runtime.kv_cache import KernelQuantCache
+
+    cache = KernelQuantCache(1, 2, 64, 16, 8, q_heads=4)
+    q = torch.randn(3, 4 * 64, device="cuda").to(torch.bfloat16)
+    k = torch.randn(3, 2 * 64, device="cuda").to(torch.bfloat16)
+    cos = torch.ones(3, 64, device="cuda", dtype=torch.bfloat16)
+    args = (cache.k_codes[0], cache.v_codes[0], cache.k_scale[0], cache.v_scale[0], cache.position)
+    with pytest.raises(RuntimeError, match="columns"):
+        ext.rope_kv_append(q, k, k, cos, cos, *args, 3, True)
+    with pytest.raises(RuntimeError, match="k and v must be"):
+        ext.rope_kv_append(q, k[:2], k, cos, cos, *args, 4, True)
+    with pytest.raises(RuntimeError, match="cos and sin"):
+        ext.rope_kv_append(q, k, k, cos[:, :32].contiguous(), cos[:, :32].contiguous(), *args, 4, True)
+    with pytest.raises(RuntimeError, match="share a dtype"):
+        ext.rope_kv_append(q, k, k.float(), cos, cos, *args, 4, True)
+    small = KernelQuantCache(1, 2, 32, 16, 8, q_heads=4)   # head_dim 32: the two-launch path's case
+    with pytest.raises(RuntimeError, match="head_dim must be 64 or 128"):
+        ext.rope_kv_append(q[:, :128].contiguous(), k[:, :64].contiguous(), k[:, :64].contiguous(),
+                           cos[:, :32].contiguous(), cos[:, :32].contiguous(), small.k_codes[0], small.v_codes[0],
+                           small.k_scale[0], small.v_scale[0], small.position, 4, True)
+    out = ext.rope_kv_append(q[:0], k[:0], k[:0], cos[:0], cos[:0], *args, 4, True)
+    assert out[0].shape == (0, 4, 64)
+
+
 def test_argument_checks(ext):
     x = torch.randn(4, 64, device="cuda").to(torch.bfloat16)
     w = torch.ones(64, device="cuda", dtype=torch.bfloat16)
