@@ -482,3 +482,31 @@ def test_wq_dense_linear_is_dequantize_then_matmul(bits):
             assert got.shape == (m, n) and got.dtype == torch.bfloat16
             assert rel_l2(to_np(got), want) <= 1e-2, (hd, out_group, keep)
             assert torch.equal(got, ext.dense_linear(x, dense))
+
+
+def test_the_dense_branch_replays_from_a_graph():
+    """A caller may capture the dense branch (a batch of more rows than the fused GEMM takes): every
+    replay, with fresh inputs and eager work between the replays, equals the eager call."""
+    from llmquant.hip import load_extension
+
+    ext = load_extension()
+    gen = torch.Generator().manual_seed(33)
+    n, k, m = 512, 1024, 80
+    w = (torch.randn(n, k, generator=gen) * 0.05).to(torch.bfloat16)
+    canonical, scales = oracle.canonical_weight(to_np(w), 4, GROUP)
+    q = torch.from_numpy(oracle.pack_int4(canonical)).cuda()
+    s = torch.from_numpy(scales).cuda()
+    static_x = torch.randn(m, k, generator=gen).to(torch.bfloat16).cuda()
+    ext.wq_dense_linear(static_x, q, s, 0, 0)  # plan and workspace exist before the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = ext.wq_dense_linear(static_x, q, s, 0, 0)
+    for replay in range(4):
+        x = torch.randn(m, k, generator=gen).to(torch.bfloat16).cuda()
+        want = ext.wq_dense_linear(x, q, s, 0, 0)   # eager work between the replays
+        torch.cuda.synchronize()
+        static_x.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_out, want), replay
