@@ -110,15 +110,35 @@ def kernel_runtime(model, max_len: int, kv_bits: int = 8):
 _KEPT_RUNTIMES = 4
 
 
-def _weights_key(model):
-    """Identity of everything a captured step has baked in: the quantized buffers' addresses and
-    versions (a re-quantized or moved model gets new ones)."""
+def _module_tree(model):
+    """Every (parent, name, child) edge of the module tree and the kernel-mode Linears in it."""
     from llmquant.quantizers.kernel import KernelQuantLinear
 
+    edges, quantized = [], []
+    for parent in model.modules():
+        if isinstance(parent, KernelQuantLinear):
+            quantized.append(parent)
+        for name, child in parent._modules.items():
+            if child is not None:
+                edges.append((parent, name, child))
+    return {"edges": edges, "quantized": quantized}
+
+
+def _weights_key(model):
+    """Identity of everything a captured step has baked in: the quantized buffers' addresses and
+    versions (a re-quantized or moved model gets new ones). The walk over the module tree is done
+    once and kept; a call checks that every edge of the tree still holds the module it held (a
+    replaced module, e.g. by another oneshot, walks again) and reads the buffers through their
+    modules (a call costs ~0.1 ms of the time to first token instead of 0.25)."""
+    tree = model.__dict__.get("_llmq_module_tree")
+    if tree is None or not all(parent._modules.get(name) is child for parent, name, child in tree["edges"]):
+        tree = _module_tree(model)
+        model.__dict__["_llmq_module_tree"] = tree
     key = []
-    for module in model.modules():
-        if isinstance(module, KernelQuantLinear):
-            key.append((module.qdata.data_ptr(), module.qdata._version, module.wscale.data_ptr(), module.wscale._version))
+    for module in tree["quantized"]:
+        buffers = module._buffers
+        qdata, wscale = buffers["qdata"], buffers["wscale"]
+        key.append((qdata.data_ptr(), qdata._version, wscale.data_ptr(), wscale._version))
     return tuple(key)
 
 

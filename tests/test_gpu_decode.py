@@ -218,7 +218,22 @@ def test_generate_calls_share_a_kept_runtime_and_its_captured_step(small):
     assert len(kernel.__dict__["_llmq_kept_runtimes"]["runtimes"]) == 2
     # a buffer written in place: everything kept is dropped
     next(m for m in kernel.modules() if hasattr(m, "qdata")).wscale.mul_(1.0)
-    assert kept_kernel_runtime(kernel, 33, 8) is not kept
+    again = kept_kernel_runtime(kernel, 33, 8)
+    assert again is not kept and kept_kernel_runtime(kernel, 33, 8) is again
+    # a module swapped for another object over the same buffers: nothing baked in has changed, so the runtime
+    # stays, but the tree is walked again and it is the new module that is watched from here on
+    import copy
+
+    mlp = kernel.model.layers[0].mlp
+    twin = copy.copy(mlp.down_proj)
+    twin._buffers, twin._parameters, twin._modules = dict(twin._buffers), dict(twin._parameters), dict(twin._modules)
+    mlp.down_proj = twin
+    swapped = kept_kernel_runtime(kernel, 33, 8)
+    assert swapped is again
+    # a buffer replaced by a tensor at another address
+    mlp.down_proj.wscale = mlp.down_proj.wscale.clone()
+    assert kept_kernel_runtime(kernel, 33, 8) is not swapped
+    assert torch.equal(graphed_generate(kernel, first, 12, kv_bits=8), fresh_a)
     kernel.__dict__.pop("_llmq_kept_runtimes", None)
 
 
