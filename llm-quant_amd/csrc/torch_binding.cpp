@@ -296,6 +296,11 @@ at::Tensor dense_linear(const at::Tensor& x, const at::Tensor& w) {
   auto out = at::empty({M, N}, x.options());
   if (out.numel() == 0) return out;
   if (K == 0) return out.zero_();
+  // the kept plan is chosen once per shape, for operands as the allocator hands them out; rows that are
+  // not whole 16-byte packets, or a view at an odd offset, go the general way
+  const bool packets = K % 8 == 0 &&
+                       ((reinterpret_cast<uintptr_t>(x.const_data_ptr()) | reinterpret_cast<uintptr_t>(w.const_data_ptr())) & 15u) == 0;
+  if (!packets) return at::mm(x, w.t());
   const c10::OptionalDeviceGuard guard(at::device_of(x));
   const auto stream = c10::hip::getCurrentHIPStream(x.device().index());
   const std::lock_guard<std::mutex> lock(g_dense_lock);

@@ -439,7 +439,7 @@ def test_dense_linear_is_the_library_matmul_with_a_kept_plan(dtype):
 
     ext = load_extension()
     gen = torch.Generator().manual_seed(21)
-    for (m, n, k) in [(72, 256, 384), (512, 3072, 2048), (100, 2048, 2048), (65, 96, 128), (300, 200, 136)]:
+    for (m, n, k) in [(72, 256, 384), (512, 3072, 2048), (100, 2048, 2048), (65, 96, 128), (70, 48, 100), (300, 200, 136)]:
         x = torch.randn(m, k, generator=gen).to(dtype).cuda()
         w = (torch.randn(n, k, generator=gen) * 0.05).to(dtype).cuda()
         want = (x.double() @ w.double().T).cpu().numpy()
@@ -449,6 +449,10 @@ def test_dense_linear_is_the_library_matmul_with_a_kept_plan(dtype):
         assert torch.equal(first, again), (m, n, k)
         assert rel_l2(to_np(first), want) <= (1e-2 if dtype == torch.bfloat16 else 2e-3), (m, n, k)
         assert rel_l2(to_np(first), to_np(x @ w.T)) <= 1e-3, (m, n, k)   # in practice the same bits
+    # rows that are not whole 16-byte packets (k = 100 above) and a view two bytes off a packet boundary
+    view = torch.randn(m * k + 1, generator=gen).to(dtype).cuda()[1:].view(m, k)
+    assert view.data_ptr() % 16 != 0
+    assert rel_l2(to_np(ext.dense_linear(view, w)), (view.double() @ w.double().T).cpu().numpy()) <= 1e-2
     assert ext.dense_linear(x[:0], w).shape == (0, n)
     with pytest.raises(RuntimeError, match="float16 or bfloat16"):
         ext.dense_linear(x.float(), w.float())
