@@ -86,18 +86,24 @@ def test_graph_replay_equals_eager_bit_for_bit(small):
     assert seq_a.shape == (1, 64) and torch.equal(seq_a, seq_b)
 
 
-def teacher_forced(real, kernel, prompt, new_tokens, vocab):
+def teacher_forced(real, kernel, prompt, new_tokens, vocab, runtime="walk"):
+    """Both models fed the oracle's own greedy stream. Rows: (same argmax, oracle top-2 gap, max logit
+    error, relative logit error); also the oracle's stream (its free-running greedy tokens) and the prompt.
+    runtime: "walk" = the operation-by-operation LlamaKernelRuntime, "fused" = LlamaFusedRuntime, the
+    five-launches-per-layer step that graphed_generate and the benchmark run."""
     from llmquant.quantizers import make_cache_factory
-    from llmquant.runtime import LlamaKernelRuntime
+    from llmquant.runtime import LlamaFusedRuntime, LlamaKernelRuntime
 
     ids = torch.randint(0, vocab, (1, prompt), generator=torch.Generator().manual_seed(1)).cuda()
     cache = make_cache_factory(8)()
     with torch.no_grad():
         want = real(ids, past_key_values=cache, use_cache=True).logits[0, -1]
-    rt = LlamaKernelRuntime(kernel, prompt + new_tokens + 2, 8)
+    cls = LlamaFusedRuntime if runtime == "fused" else LlamaKernelRuntime
+    rt = cls(kernel, prompt + new_tokens + 2, 8)
     first = rt.prefill(ids)
     rows = [(first.item() == want.argmax().item(), 0.0, 0.0, 0.0)]
     tok = want.argmax().reshape(1)
+    stream = [tok.item()]
     for i in range(new_tokens):
         with torch.no_grad():
             want = real(tok.reshape(1, 1), past_key_values=cache, use_cache=True).logits[0, -1].float()
@@ -107,7 +113,8 @@ def teacher_forced(real, kernel, prompt, new_tokens, vocab):
         rows.append((nxt.item() == want.argmax().item(), (top2[0] - top2[1]).item(),
                      (got - want).abs().max().item(), ((got - want).norm() / want.norm()).item()))
         tok = want.argmax().reshape(1)
-    return rows
+        stream.append(tok.item())
+    return rows, stream, ids
 
 
 def check_margin(rows, rel_bound):
@@ -121,23 +128,97 @@ def check_margin(rows, rel_bound):
 
 def test_teacher_forced_margin_small(small):
     real, kernel = small
-    rows = teacher_forced(real, kernel, 48, 64, 4096)
+    rows, _, _ = teacher_forced(real, kernel, 48, 64, 4096)
     agree = check_margin(rows, 0.05)
     print(f"teacher-forced agreement {agree}/{len(rows)}")
     assert agree >= 0.8 * len(rows)
 
 
-def test_teacher_forced_margin_llama_1b_config():
+def identical_prefix(a, b) -> int:
+    n = 0
+    for x, y in zip(a, b):
+        if x != y:
+            break
+        n += 1
+    return n
+
+
+@pytest.mark.parametrize("runtime", ["fused", "walk"])
+def test_teacher_forced_margin_small_both_runtimes(small, runtime):
+    real, kernel = small
+    rows, _, _ = teacher_forced(real, kernel, 48, 32, 4096, runtime)
+    assert check_margin(rows, 0.05) >= 0.8 * len(rows)
+
+
+@pytest.fixture(scope="module")
+def llama_1b():
     """The end-to-end decode case at full size: 16 layers, hidden 2048, FFN 8192, 32/8 heads, vocab
-    128256, prompt 512, 64 decoded tokens."""
+    128256; attention int8, MLP int4, lm_head int8, int8 KV cache."""
     model = build_model(2048, 8192, 16, 32, 8, 128256)
-    real, kernel = quantized_pair(model)
+    pair = quantized_pair(model)
     del model
-    rows = teacher_forced(real, kernel, 512, 64, 128256)
-    agree = check_margin(rows, 0.08)
-    print(f"teacher-forced agreement {agree}/{len(rows)}; median gap "
-          f"{sorted(r[1] for r in rows[1:])[32]:.3f}, max logit error {max(r[2] for r in rows):.3f}")
+    torch.cuda.empty_cache()
+    return pair
+
+
+#: teacher-forced relative logit error allowed at full size. A random-init 16-layer network turns
+#: one-ulp bf16 differences between two correct implementations (summation order of the projections, the
+#: attention's rounding points) into a few per cent of logit noise: measured 0.02-0.05 on this model.
+FULL_SIZE_REL_BOUND = 0.08
+
+
+_FULL_SIZE_ROWS = {}
+
+
+def full_size_rows(pair, runtime):
+    """teacher_forced at full size, run once per runtime and shared between the tests below."""
+    if runtime not in _FULL_SIZE_ROWS:
+        _FULL_SIZE_ROWS[runtime] = teacher_forced(*pair, 512, 64, 128256, runtime)
+    return _FULL_SIZE_ROWS[runtime]
+
+
+@pytest.mark.parametrize("runtime", ["fused", "walk"])
+def test_teacher_forced_margin_llama_1b_config(llama_1b, runtime):
+    """Prompt 512, 64 decoded tokens, through the fused five-launch step (what graphed_generate and the
+    benchmark run) and through the operation-by-operation walk, each against the real-mode model under
+    HF transformers with FakeQuantCache(8)."""
+    rows, _, _ = full_size_rows(llama_1b, runtime)
+    agree = check_margin(rows, FULL_SIZE_REL_BOUND)
+    print(f"[{runtime}] teacher-forced agreement {agree}/{len(rows)}; median gap "
+          f"{sorted(r[1] for r in rows[1:])[32]:.3f}, max logit error {max(r[2] for r in rows):.3f}, "
+          f"max relative error {max(r[3] for r in rows):.4f}")
     assert agree >= 0.85 * len(rows)
+
+
+#: identical-prefix length of the free-running streams measured on this model and prompt (64 = the whole
+#: window). The assertion below allows it to move only where the oracle itself is at a near-tie.
+MEASURED_FREE_RUNNING_PREFIX = 2
+
+
+def test_free_running_prefix_llama_1b_config(llama_1b):
+    """The first 64 greedy tokens, free-running on both sides: the real-mode model's own stream against
+    graphed_generate's (fused step, HIP graph replay). Reports the identical-prefix length and asserts
+    (a) it is at least the length recorded above, and (b) where the streams part, they part at a token
+    whose top-2 logit gap in the oracle is within twice the logit error measured at that very step under
+    teacher forcing, i.e. at a near-tie that arithmetic noise decides, never at a clear margin. Up to the
+    parting point both sides have seen the same tokens, so the teacher-forced row describes that step."""
+    from llmquant.runtime import LlamaFusedRuntime, graphed_generate
+
+    real, kernel = llama_1b
+    rows, oracle_stream, ids = full_size_rows(llama_1b, "fused")
+    kernel.__dict__.pop("_llmq_kept_runtimes", None)
+    free = graphed_generate(kernel, ids, 65, kv_bits=8)[0, 512:].tolist()
+    eager = LlamaFusedRuntime(kernel, 512 + 65 + 1, 8).generate(ids, 65, use_graph=False)[0, 512:].tolist()
+    kernel.__dict__.pop("_llmq_kept_runtimes", None)
+    assert free == eager  # replay == eager at full size, bit for bit in the tokens
+    prefix = identical_prefix(free[:64], oracle_stream[:64])
+    agree = sum(a == b for a, b in zip(free[:64], oracle_stream[:64]))
+    print(f"free-running: identical prefix {prefix}/64 tokens, {agree}/64 positions equal")
+    if prefix < 64:
+        ok, gap, err, rel = rows[prefix]
+        print(f"streams part at token {prefix}: oracle top-2 gap {gap:.4f}, logit error there {err:.4f}")
+        assert not ok and gap <= 2 * err
+    assert prefix >= MEASURED_FREE_RUNNING_PREFIX
 
 
 def test_runtime_layer_equals_the_hf_layer(small):

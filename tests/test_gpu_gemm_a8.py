@@ -145,3 +145,41 @@ def test_argument_checks(ext):
     with pytest.raises(RuntimeError, match="group_size 128"):
         ext.wq_gemm_a8(a, torch.ones(4, 4, device="cuda"), torch.zeros(8, 4, 64, dtype=torch.int8, device="cuda"),
                        torch.ones(8, 4, device="cuda"))
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("m", [128, 512, 2048])
+def test_one_activation_scale_per_token(ext, n, k, m):
+    """The prefill case with the activation quantized per token (one int8 scale per row, the literal
+    "per-token symmetric int8"): the quantizer run with group = K, its scale broadcast to the [M, G] the
+    kernel takes. The reference has no arithmetic of its own for this form (its activation scheme is per
+    token x group-128, llmquant/core/scheme.py:41-44), so the anchor is the closed form
+    y[m, n] = s_x[m] * sum_g s_w[n, g] * sum_k a[m, g, k] q[n, g, k] in float64 on sampled entries; codes and
+    scales of the activation are bit-exact against the oracle's quantizer."""
+    torch.manual_seed(7)
+    w = (torch.randn(n, k) * 0.015).to(torch.bfloat16)
+    x = torch.randn(m, k)
+    x[:, torch.randperm(k)[: k // 100]] *= 20
+    x = x.to(torch.bfloat16)
+    canonical, scales = oracle.canonical_weight(to_np(w), 4, GROUP)
+    q = torch.from_numpy(oracle.pack_int4(canonical)).cuda()
+    s = torch.from_numpy(scales).cuda()
+    codes, sx = ext.quant_group_codes(x.cuda(), 8, k, False)
+    want_codes, want_sx = oracle.quant_group_codes(to_np(x), 8, k)
+    assert sx.shape == (m, 1)
+    assert np.array_equal(codes.cpu().numpy(), want_codes) and np.array_equal(to_np(sx), want_sx)
+    sx_groups = sx.expand(m, k // GROUP).contiguous()
+    rng = np.random.default_rng(2)
+    rows = np.sort(rng.choice(m, 64, replace=False))
+    cols = np.sort(rng.choice(n, 96, replace=False))
+    a = want_codes[rows].astype(np.float64)
+    wq = (canonical[cols].astype(np.float64) * scales[cols].astype(np.float64)[:, :, None]).reshape(len(cols), -1)
+    exact = (a @ wq.T) * want_sx[rows].astype(np.float64)
+    for dtype, tol in ((torch.float32, 1e-6), (torch.bfloat16, 1e-2)):
+        got = ext.wq_gemm_a8(codes, sx_groups, q, s, None, 0, dtype)
+        assert got.shape == (m, n) and got.dtype == dtype
+        assert rel_l2(to_np(got)[np.ix_(rows, cols)], exact) <= tol
+    # against the unquantized product: what per-token int8 activations + int4 weights cost in accuracy
+    dense = to_np(x)[rows].astype(np.float64) @ to_np(w)[cols].astype(np.float64).T
+    print(f"per-token A8 x W4 vs bf16 product, M={m} N={n} K={k}: rel-L2 "
+          f"{rel_l2(to_np(got)[np.ix_(rows, cols)], dense):.4f}")

@@ -211,3 +211,94 @@ def test_argument_checks(ext):
     ws = torch.zeros(ext.kv_decode_workspace_floats(6, 64, 16), device="cuda")
     with pytest.raises(RuntimeError, match="multiple of kv_heads|must be 1, 2, 4 or 8"):
         ext.kv_decode_attention(q[:6], cache["k_codes"], cache["v_codes"], cache["k_scale"], cache["v_scale"], ws, pos, 0.125)
+
+
+# ---- the kernels the decode step runs, straight against the oracle -------------------------------------
+
+
+def rope_oracle(x, cos, sin):
+    """transformers' apply_rotary_pos_emb on bf16 values, every product and the sum rounded to bf16
+    (x [H, D]; cos, sin [D]): x * cos + rotate_half(x) * sin."""
+    half = x.shape[-1] // 2
+    rot = np.concatenate((-x[..., half:], x[..., :half]), axis=-1)
+    a = oracle.round_to(x * cos, "bf16")
+    b = oracle.round_to(rot * sin, "bf16")
+    return oracle.round_to(a + b, "bf16")
+
+
+def decode_step_case(ext, bits, ctx, q_heads=32, kv_heads=8, d=64, seed=0):
+    """KV-cache quantization in decode attention, Llama-3.2-1B geometry: a cache of `ctx` tokens with
+    per-channel scale variance, one new token through RoPE -> quantize-append -> attention. Returns the
+    device-side cache, the q|k|v row and tables, and the oracle's attention output [Hq, D] (bf16 values)."""
+    gen = torch.Generator().manual_seed(seed)
+    channel = torch.exp(0.5 * torch.randn(d, generator=gen))
+    k = (torch.randn(kv_heads, ctx, d, generator=gen) * channel).to(torch.bfloat16)
+    v = (torch.randn(kv_heads, ctx, d, generator=gen) * channel).to(torch.bfloat16)
+    qkv = torch.randn(1, (q_heads + 2 * kv_heads) * d, generator=gen).to(torch.bfloat16)
+    qkv[:, q_heads * d:] *= channel.repeat(2 * kv_heads).to(torch.bfloat16)
+    t_max = ctx + 1
+    inv_freq = 1.0 / (500000.0 ** (torch.arange(0, d, 2).float() / d))
+    emb = torch.outer(torch.arange(t_max).float(), inv_freq)
+    emb = torch.cat((emb, emb), -1)
+    cos_t, sin_t = emb.cos().to(torch.bfloat16), emb.sin().to(torch.bfloat16)
+
+    cache = new_cache(kv_heads, t_max, d, bits)
+    if ctx:
+        append(ext, cache, k.cuda(), v.cuda(), 0)
+
+    row = to_np(qkv)[0]
+    q_new = row[: q_heads * d].reshape(q_heads, d)
+    k_new = row[q_heads * d: (q_heads + kv_heads) * d].reshape(kv_heads, d)
+    v_new = row[(q_heads + kv_heads) * d:].reshape(kv_heads, d)
+    cos, sin = to_np(cos_t)[ctx], to_np(sin_t)[ctx]
+    q_rot, k_rot = rope_oracle(q_new, cos, sin), rope_oracle(k_new, cos, sin)
+    k_all = np.concatenate((to_np(k), k_rot[:, None]), axis=1)
+    v_all = np.concatenate((to_np(v), v_new[:, None]), axis=1)
+    kq, ks = oracle.kv_quant(k_all, bits)
+    vq, vs = oracle.kv_quant(v_all, bits)
+    want = oracle.gqa_decode_attention(q_rot, oracle.kv_dequant(kq, ks, "bf16"), oracle.kv_dequant(vq, vs, "bf16"),
+                                       d ** -0.5, "bf16")
+    return cache, qkv.cuda(), cos_t.cuda(), sin_t.cuda(), want, (kq, ks, vq, vs)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("ctx,splits", [(2048, 8), (2048, 16), (2048, 32), (2048, 1), (640, 8), (0, 8), (63, 8)])
+def test_decode_step_attention_against_the_oracle(ext, bits, ctx, splits):
+    """RoPE -> quantize-append -> split attention -> merge, the launches of the decode step, compared
+    directly with the oracle (RoPE with transformers' rounding points, FakeQuantCache's codes and scales,
+    float64 softmax attention over the bf16(code * scale) values): the appended codes and scales bit for
+    bit, the attention output within rel-L2 1e-2, and o_proj taken as the GEMV that merges the split
+    records while it stages its activation against the float64 closed form on the oracle's attention
+    output. splits = 1 is the one-workgroup-per-head launch, 32 the form that shares a kv head's rows
+    between its four query heads."""
+    q_heads, kv_heads, d = 32, 8, 64
+    cache, qkv, cos_t, sin_t, want, (kq, ks, vq, vs) = decode_step_case(ext, bits, ctx)
+    position = torch.tensor([ctx], dtype=torch.int32, device="cuda")
+    args = (cache["k_codes"], cache["v_codes"], cache["k_scale"], cache["v_scale"])
+    if splits == 1:
+        merged = ext.kv_rope_append_attend(qkv, cos_t, sin_t, *args, position, d ** -0.5, q_heads)
+    else:
+        partials = torch.full((ext.kv_attend_partials_floats(q_heads, d, splits),), float("nan"), device="cuda")
+        ext.kv_rope_append_attend_split(qkv, cos_t, sin_t, *args, partials, position, d ** -0.5, q_heads, splits)
+        merged = ext.kv_attend_merge(partials, q_heads, d, splits, torch.bfloat16)
+    # what the step appended, and everything before it, is what FakeQuantCache's rule gives
+    assert np.array_equal(codes_np(cache["k_codes"], bits), kq)
+    assert np.array_equal(codes_np(cache["v_codes"], bits), vq)
+    assert np.array_equal(to_np(cache["k_scale"]), ks) and np.array_equal(to_np(cache["v_scale"]), vs)
+    got = to_np(merged).reshape(q_heads, d)
+    assert rel_l2(got, want) <= 1e-2
+    per_head = np.linalg.norm(got - want, axis=1) / np.linalg.norm(want, axis=1)
+    assert per_head.max() <= 2e-2, per_head.argmax()  # no single head hides in the norm of the others
+
+    if splits > 1:
+        # o_proj over the oracle's attention output: heads of 64 padded to groups of 128, int8
+        torch.manual_seed(3)
+        n = 2048
+        w = (torch.randn(n, q_heads * d) * 0.02).to(torch.bfloat16)
+        canonical, scales = oracle.canonical_weight(to_np(w), 8, 128, d, None)
+        res = torch.randn(1, n).to(torch.bfloat16)
+        out = ext.wq_gemv_attn_merge(partials, splits, d, torch.from_numpy(canonical).cuda(),
+                                     torch.from_numpy(scales).cuda(), 0, d, res.cuda(), torch.bfloat16)
+        padded = oracle.pad_activation(want.reshape(1, -1), 128, d)
+        exact = oracle.gemv_float64(padded, canonical, scales) + to_np(res).astype(np.float64)
+        assert rel_l2(to_np(out), exact) <= 1e-2
