@@ -278,6 +278,20 @@ int llmq_kv_decode_attention(const void* q, const void* k_codes, const void* v_c
                              int q_heads, int kv_heads, int head_dim, int t_max, int bits,
                              int dtype, llmq_stream_t stream);
 
+/* llmq_kv_decode_attention for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): same arguments without the workspace,
+ * same kernel, same result bit for bit. It has no counterpart in the reference. The partial records and
+ * arrival counters live in a device array inside the library, 4.3 MB on every GPU the library runs on,
+ * held until the process ends. Limits: q_heads <= 128 (more is an error that names the limit; head_dim and
+ * t_max as for llmq_kv_decode_attention). Calls no hipMalloc / hipFree and no allocating routine. Every
+ * call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams) race; calls on one
+ * stream, and calls on different GPUs, are fine. Each call clears the counters first with a one-workgroup
+ * fill kernel (not a memset node, so the call can be captured). */
+int llmq_kv_decode_attention_static(const void* q, const void* k_codes, const void* v_codes,
+                                    const float* k_scale, const float* v_scale, void* out,
+                                    const int32_t* len_dev, float sm_scale, int q_heads, int kv_heads,
+                                    int head_dim, int t_max, int bits, int dtype, llmq_stream_t stream);
+
 /* One decode step of attention for one layer in a single launch: RoPE on the new token's query
  * and key (transformers' apply_rotary_pos_emb, same rounding points), quantize-and-append of its
  * key and value at position *pos_dev, then attention over tokens 0 .. *pos_dev. Equivalent to

@@ -11,6 +11,8 @@
 // [kv_heads, t_max, head_dim/2] nibble-packed uint8 (4 bit, +8 bias, even index low), scales
 // [kv_heads, t_max] fp32. The write position and the valid length live on the device, so a
 // decode step is the same sequence of launches every token and can be replayed from a graph.
+#include <mutex>
+
 #include "llmq_device.h"
 
 namespace {
@@ -1029,6 +1031,100 @@ extern "C" int llmq_kv_decode_attention(const void* q, const void* k_codes, cons
 #undef LLMQ_BD
 #undef LLMQ_GO
   return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+}
+
+// ---- the same attention for callers that cannot allocate ----------------------------------------------
+// The partial records and arrival counters live in a file-scope device array instead of a caller's
+// workspace. Every GPU the library runs on holds its own copy of the array (at its own address, found once
+// per device with hipGetSymbolAddress) until the process ends. Layout: kStaticCounters int32 arrival
+// counters first, at a fixed place whatever the geometry of a call, then the partial records.
+constexpr int kStaticMaxQHeads = 128;
+constexpr int kStaticCounters = 256;  // >= kStaticMaxQHeads, and a whole number of 256-byte lines
+constexpr size_t kStaticPartFloats = static_cast<size_t>(kStaticMaxQHeads) * 64 * (128 + 2);
+static __device__ __align__(256) float g_attn_scratch[kStaticCounters + kStaticPartFloats];
+
+__global__ void clear_counters_kernel(int* __restrict__ count) { count[threadIdx.x] = 0; }
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+// The array's address on the current device; looked up on the first call per device. Returns nullptr
+// with the error text set when the runtime refuses.
+float* static_scratch() {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess || device < 0 || device >= kMaxDevices) {
+    llmq_host::set_error("static scratch: hipGetDevice gave device %d (%s)", device, hipGetErrorString(err));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    void* ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_attn_scratch));
+    if (err != hipSuccess || ptr == nullptr) {
+      llmq_host::set_error("static scratch: hipGetSymbolAddress failed on device %d (%s)", device,
+                           hipGetErrorString(err));
+      return nullptr;
+    }
+    g_scratch_ptr[device] = static_cast<float*>(ptr);
+  }
+  return g_scratch_ptr[device];
+}
+}  // namespace
+
+extern "C" int llmq_kv_decode_attention_static(const void* q, const void* k_codes, const void* v_codes,
+                                               const float* k_scale, const float* v_scale, void* out,
+                                               const int32_t* len_dev, float sm_scale, int q_heads,
+                                               int kv_heads, int head_dim, int t_max, int bits, int dtype,
+                                               llmq_stream_t stream) {
+  if (bits != 8 && bits != 4) return llmq_host::fail_invalid("KV cache bits must be 8 or 4, got %d", bits);
+  if (head_dim != 64 && head_dim != 128) return llmq_host::fail_invalid("head_dim must be 64 or 128, got %d", head_dim);
+  if (kv_heads <= 0 || q_heads <= 0 || q_heads % kv_heads) return llmq_host::fail_invalid("q_heads %d must be a positive multiple of kv_heads %d", q_heads, kv_heads);
+  if (q_heads > kStaticMaxQHeads)
+    return llmq_host::fail_invalid("the static scratch holds up to %d query heads, got %d (use llmq_kv_decode_attention "
+                                   "with a workspace of your own)", kStaticMaxQHeads, q_heads);
+  if (t_max <= 0) return llmq_host::fail_invalid("t_max must be positive, got %d", t_max);
+  if (!q || !k_codes || !v_codes || !k_scale || !v_scale || !out || !len_dev)
+    return llmq_host::fail_invalid("null tensor pointer");
+  if ((reinterpret_cast<uintptr_t>(k_codes) | reinterpret_cast<uintptr_t>(v_codes)) & 15u)
+    return llmq_host::fail_invalid("cache code pointers must be 16-byte aligned");
+  if (dtype != LLMQ_F32 && dtype != LLMQ_F16 && dtype != LLMQ_BF16)
+    return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+  const int rep = q_heads / kv_heads;
+  if (rep != 1 && rep != 2 && rep != 4 && rep != 8)
+    return llmq_host::fail_invalid("q_heads / kv_heads must be 1, 2, 4 or 8, got %d", rep);
+  const int splits = splits_for(t_max);
+  if (static_cast<size_t>(q_heads) * splits * (head_dim + 2) > kStaticPartFloats)
+    return llmq_host::fail_invalid("partial records exceed the static scratch");
+  float* scratch = static_scratch();
+  if (scratch == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
+  int* count = reinterpret_cast<int*>(scratch);
+  float* part = scratch + kStaticCounters;
+  const int chunk = (t_max + splits - 1) / splits;
+  const dim3 grid(splits, kv_heads);
+  const float scale_log2 = sm_scale * 1.4426950408889634f;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // the counters must start at zero whatever the last call on this GPU left behind (a fill kernel, not
+  // a memset: a caller may be capturing a graph)
+  hipLaunchKernelGGL(clear_counters_kernel, dim3(1), dim3(kStaticCounters), 0, s, count);
+  if (int rc = llmq_host::check_launch("clear_counters_kernel")) return rc;
+  const uint8_t* kc = static_cast<const uint8_t*>(k_codes);
+  const uint8_t* vc = static_cast<const uint8_t*>(v_codes);
+#define LLMQ_GO(T, B, D)                                                                        \
+  return launch_attn_rep<T, B, D>(rep, grid, s, static_cast<const T*>(q), kc, vc, k_scale, v_scale, \
+                                  static_cast<T*>(out), part, count, len_dev, scale_log2, t_max, chunk)
+#define LLMQ_BD(T)                                                                              \
+  if (bits == 8) { if (head_dim == 64) LLMQ_GO(T, 8, 64); else LLMQ_GO(T, 8, 128); }            \
+  else { if (head_dim == 64) LLMQ_GO(T, 4, 64); else LLMQ_GO(T, 4, 128); }
+  switch (dtype) {
+    case LLMQ_F32: LLMQ_BD(float)
+    case LLMQ_F16: LLMQ_BD(f16_t)
+    default: LLMQ_BD(bf16_t)
+  }
+#undef LLMQ_BD
+#undef LLMQ_GO
 }
 
 extern "C" int llmq_kv_rope_append_attend(const void* qkv, const void* cos_table, const void* sin_table,

@@ -81,6 +81,8 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_kv_decode_workspace_floats.argtypes = [c_int] * 3
     lib.llmq_kv_decode_workspace_floats.restype = ctypes.c_size_t
     lib.llmq_kv_decode_attention.argtypes = [c_p] * 8 + [c_f] + [c_int] * 6 + [c_p]
+    lib.llmq_kv_decode_attention_static.argtypes = [c_p] * 7 + [c_f] + [c_int] * 6 + [c_p]
+    lib.llmq_kv_decode_attention_static.restype = c_int
     lib.llmq_wq_gemv_fused.argtypes = [c_p] * 4 + [c_int] * 6 + [c_p, c_f, c_int, c_p, c_p]
     lib.llmq_wq_gemv_fused.restype = c_int
     lib.llmq_wq_gemv_batched_fused.argtypes = [c_p, c_i64, c_p, c_p, c_p, c_p, c_p, c_p] + [c_int] * 8 + [c_p]
