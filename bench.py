@@ -191,14 +191,18 @@ def main():
     probe = [torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_(0, 255) for _ in range(2)]
     sink = torch.zeros(1, dtype=torch.int32, device="cuda:0")
     probe_ms = []
+    # (the probe kernel is a measurement aid in a small library of its own, beside the product library)
+    probe_lib = ctypes.CDLL(str(ROOT / "llm-quant_amd" / "llmquant" / "hip" / "libllmq_bench_probe.so"))
+    probe_lib.bench_stream_read_probe.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p]
+    probe_lib.bench_stream_read_probe.restype = ctypes.c_int
     for rep in range(12):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record(stream)
-        rc = lib.llmq_stream_read_probe(probe[rep % 2].data_ptr(), probe[rep % 2].numel(), sink.data_ptr(), sptr)
+        rc = probe_lib.bench_stream_read_probe(probe[rep % 2].data_ptr(), probe[rep % 2].numel(), sink.data_ptr(), sptr)
         b.record(stream)
         torch.cuda.synchronize()
         if rc:
-            raise RuntimeError(lib.llmq_last_error().decode())
+            raise RuntimeError(f"bench_stream_read_probe: hipError {rc}")
         if rep >= 2:
             probe_ms.append(a.elapsed_time(b))
     read_ceiling = (1 << 30) / (sum(probe_ms) / len(probe_ms) * 1e-3) / 1e9

@@ -340,12 +340,6 @@ int llmq_argmax_advance(const void* x, int n, int64_t* out_index, int64_t* token
                         int64_t* step64_or_null, int32_t* step32_or_null, int dtype,
                         llmq_stream_t stream);
 
-/* Measurement aid (no counterpart in the reference): reads `bytes` of `buffer` once with plain
- * 128-bit loads and nothing else, so that timing it gives the read rate this GPU's memory system
- * actually delivers to a kernel; bench.py reports the GEMV against it beside the published peak.
- * `sink` is one device word that is (practically never) written. */
-int llmq_stream_read_probe(const void* buffer, size_t bytes, uint32_t* sink, llmq_stream_t stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -1,10 +1,11 @@
-// Measurement aid, not part of the quantized path: a plain streaming read of a buffer with
+// Measurement aid for bench.py, built into its own small library (libllmq_bench_probe.so) and not part
+// of the product library or its header: a plain streaming read of a buffer with
 // non-temporal 128-bit loads, eight in flight per lane, one workgroup per CU (of the grid sizes
 // and load flavours tried, 256 x 256 threads with eight loads in flight read fastest on MI355X:
 // 6.2 TB/s, against 4.7-5.9 TB/s for 1024-8192 workgroups). Its rate is what this GPU's
 // memory system delivers to a kernel that does nothing but read, i.e. the ceiling the GEMV's
 // bytes-per-second figure is to be compared with beside the published peak.
-#include "llmq_device.h"
+#include "../llmq_device.h"
 
 namespace {
 
@@ -41,11 +42,11 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const u32x4* __restric
 
 }  // namespace
 
-extern "C" int llmq_stream_read_probe(const void* buffer, size_t bytes, uint32_t* sink, llmq_stream_t stream) {
+// Returns 0 or a hipError_t.
+extern "C" int bench_stream_read_probe(const void* buffer, size_t bytes, uint32_t* sink, void* stream) {
   if (bytes == 0) return 0;
-  if (!buffer || !sink) return llmq_host::fail_invalid("null pointer");
-  if (reinterpret_cast<uintptr_t>(buffer) & 15u) return llmq_host::fail_invalid("buffer must be 16-byte aligned");
+  if (!buffer || !sink || (reinterpret_cast<uintptr_t>(buffer) & 15u)) return static_cast<int>(hipErrorInvalidValue);
   hipLaunchKernelGGL(stream_read_kernel, dim3(256), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const u32x4*>(buffer), bytes / 16, sink);
-  return llmq_host::check_launch("stream_read_kernel");
+  return static_cast<int>(hipGetLastError());
 }

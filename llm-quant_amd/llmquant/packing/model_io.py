@@ -93,7 +93,12 @@ def save_packed_model(model: nn.Module, path, model_id: str, kv_cache_bits=None,
     # whatever a quantized layer owns (stored or derived) is excluded by prefix, so a derived
     # buffer can never be written as bf16 and later overwrite its exactly computed value
     owned = tuple(f"{name}." for name in (*layers, *experts))
-    state = model.state_dict()
+    # (the quantized modules' own state_dict form unpacks 4-bit codes: walk the other modules only)
+    state = {}
+    for prefix, module in model.named_modules():
+        full = f"{prefix}." if prefix else ""
+        if not full.startswith(owned):
+            module._save_to_state_dict(state, full, keep_vars=False)
     for name, tensor in state.items():
         if name.startswith(owned) or name in tensors:
             continue

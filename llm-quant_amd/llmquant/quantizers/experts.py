@@ -175,6 +175,26 @@ class KernelQuantExperts(_QuantExperts):
     def qdown(self) -> torch.Tensor:
         return unpack_int4(self.down_data) if self._packed else self.down_data
 
+    # state_dict in the reference's terms: `qgate_up` / `qdown` as int8 [E, N, groups, gs]
+    # (llmquant/quantizers/kernel.py:134-137); load_state_dict takes that form or the stored one.
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        super()._save_to_state_dict(destination, prefix, keep_vars)
+        kept = {name: destination.pop(prefix + name) for name in ("gate_up_data", "sgate_up", "down_data", "sdown")}
+        unpack = unpack_int4 if self._packed else (lambda t: t)
+        destination[prefix + "qgate_up"] = unpack(kept["gate_up_data"])
+        destination[prefix + "sgate_up"] = kept["sgate_up"]
+        destination[prefix + "qdown"] = unpack(kept["down_data"])
+        destination[prefix + "sdown"] = kept["sdown"]
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                              error_msgs):
+        for theirs, mine in (("qgate_up", "gate_up_data"), ("qdown", "down_data")):
+            codes = state_dict.pop(prefix + theirs, None)
+            if codes is not None and prefix + mine not in state_dict:
+                state_dict[prefix + mine] = pack_int4(codes) if self._packed and codes.dtype == torch.int8 else codes
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                                      error_msgs)
+
     def _stored(self, which):
         if which == "gate_up":
             return self.gate_up_data, self.sgate_up, self.hidden_dim, self._gate_up_padded

@@ -116,6 +116,32 @@ class KernelQuantLinear(nn.Module):
         repeat = self.out_features // self.wscale.shape[0]
         return self.wscale.repeat_interleave(repeat, dim=0).unsqueeze(-1)
 
+    # ---- state_dict in the reference's terms -----------------------------------------------------------
+    # The reference registers `qweight` ([N, groups, gs] int8), `wscale` and `_broadcast_scale` ([N, groups, 1])
+    # as persistent buffers (llmquant/quantizers/kernel.py:36-54). state_dict() here writes those three keys
+    # with those shapes and dtypes (4-bit codes unpacked to one per int8 byte), and load_state_dict() takes
+    # either that form or this module's own stored form (`qdata`, nibble-packed for 4 bits), so a kernel-mode
+    # state_dict moves between the two implementations in both directions.
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        super()._save_to_state_dict(destination, prefix, keep_vars)
+        stored = destination.pop(prefix + "qdata")
+        wscale = destination.pop(prefix + "wscale")
+        destination[prefix + "qweight"] = unpack_int4(stored) if self._packed else stored
+        destination[prefix + "wscale"] = wscale
+        broadcast = self._broadcast_scale
+        destination[prefix + "_broadcast_scale"] = broadcast if keep_vars else broadcast.detach()
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                              error_msgs):
+        theirs = state_dict.pop(prefix + "qweight", None)
+        if theirs is not None and prefix + "qdata" not in state_dict:
+            if self._packed and theirs.dtype == torch.int8:
+                theirs = pack_int4(theirs)
+            state_dict[prefix + "qdata"] = theirs
+        state_dict.pop(prefix + "_broadcast_scale", None)  # derived from wscale on demand
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                                      error_msgs)
+
     def _dequantized_weight(self, dtype, real_width: bool = False):
         """[out, padded_in] in the activation dtype, rebuilt per call and never cached: one kernel
         pass (the reference multiplies and casts in PyTorch, kernel.py:68-79). With `real_width`

@@ -20,8 +20,8 @@ import torch
 from llmquant.runtime.llama_decode import WARMUP_CALLS, LlamaKernelRuntime
 from llmquant.runtime.llama_fused import LlamaFusedRuntime
 
-__all__ = ["GraphedDecoder", "KernelDecoder", "WARMUP_CALLS", "can_graph", "graphed_generate", "kept_kernel_runtime",
-           "kernel_runtime"]
+__all__ = ["GraphedDecoder", "KernelDecoder", "WARMUP_CALLS", "can_graph", "graphed_generate", "kept_graphed_decoder",
+           "kept_kernel_runtime", "kernel_runtime"]
 
 
 def _on_gpu(model) -> bool:
@@ -111,34 +111,40 @@ _KEPT_RUNTIMES = 4
 
 
 def _module_tree(model):
-    """Every (parent, name, child) edge of the module tree and the kernel-mode Linears in it."""
-    from llmquant.quantizers.kernel import KernelQuantLinear
-
-    edges, quantized = [], []
+    """Every (parent, name, child) edge of the module tree and every place a tensor hangs in it (the
+    `_parameters` / `_buffers` dict of a module and the name in it)."""
+    edges, slots = [], []
     for parent in model.modules():
-        if isinstance(parent, KernelQuantLinear):
-            quantized.append(parent)
         for name, child in parent._modules.items():
             if child is not None:
                 edges.append((parent, name, child))
-    return {"edges": edges, "quantized": quantized}
+        for holder in (parent._parameters, parent._buffers):
+            for name, tensor in holder.items():
+                if tensor is not None:
+                    slots.append((holder, name))
+    return {"edges": edges, "slots": slots}
 
 
 def _weights_key(model):
-    """Identity of everything a captured step has baked in: the quantized buffers' addresses and
-    versions (a re-quantized or moved model gets new ones). The walk over the module tree is done
-    once and kept; a call checks that every edge of the tree still holds the module it held (a
-    replaced module, e.g. by another oneshot, walks again) and reads the buffers through their
-    modules (a call costs ~0.1 ms of the time to first token instead of 0.25)."""
+    """Identity of everything a captured step has baked in: address, version and dtype of every parameter
+    and buffer of the model: the quantized codes and scales, and also the embedding table, the norm weights
+    and the rotary frequencies, whose addresses (or the tables computed from them) a captured step reads. A
+    re-quantized or moved model, resize_token_embeddings, a norm weight replaced by a new Parameter, a
+    load_state_dict(assign=True) or an in-place write all change it. The walk over the module tree is done
+    once and kept; a call checks that every edge of the tree still holds the module it held (a replaced
+    module, e.g. by another oneshot, walks again) and reads the tensors through their holders (a call costs
+    ~0.1 ms of the time to first token)."""
     tree = model.__dict__.get("_llmq_module_tree")
     if tree is None or not all(parent._modules.get(name) is child for parent, name, child in tree["edges"]):
         tree = _module_tree(model)
         model.__dict__["_llmq_module_tree"] = tree
     key = []
-    for module in tree["quantized"]:
-        buffers = module._buffers
-        qdata, wscale = buffers["qdata"], buffers["wscale"]
-        key.append((qdata.data_ptr(), qdata._version, wscale.data_ptr(), wscale._version))
+    for holder, name in tree["slots"]:
+        tensor = holder.get(name)
+        if tensor is None:
+            key.append(None)
+        else:
+            key.append((tensor.data_ptr(), tensor._version, tensor.dtype))
     return tuple(key)
 
 
@@ -146,7 +152,7 @@ def kept_kernel_runtime(model, max_len: int, kv_bits: int = 8):
     """kernel_runtime, kept on the model between generate calls together with its captured step (which
     reads token and position from the device, so it serves any prompt that fits max_len): a serving
     loop does not rebuild and re-capture per request. Up to _KEPT_RUNTIMES cache lengths are kept; a
-    change of the model's quantized buffers drops them all."""
+    change of any parameter or buffer of the model drops them all."""
     weights = _weights_key(model)
     kept = model.__dict__.get("_llmq_kept_runtimes")
     if kept is None or kept["weights"] != weights:
@@ -161,6 +167,28 @@ def kept_kernel_runtime(model, max_len: int, kv_bits: int = 8):
             runtimes.pop(next(iter(runtimes)))  # the least recently used
     runtimes[key] = runtime  # most recently used last
     return runtime
+
+
+def kept_graphed_decoder(model, prompt_tokens: int, new_tokens: int):
+    """A GraphedDecoder (HF module walk over a StaticCache) kept on the model between generate calls with
+    its captured step, exactly as kept_kernel_runtime keeps the kernel runtime: the captured step reads the
+    token, the position and the cache length from the device, so after the first call a generate is cache
+    reset + eager prompt pass + replays, on this side as on the kernel side. Keyed by the run's lengths;
+    dropped when any parameter or buffer of the model changes."""
+    weights = _weights_key(model)
+    kept = model.__dict__.get("_llmq_kept_decoders")
+    if kept is None or kept["weights"] != weights:
+        kept = {"weights": weights, "decoders": {}}
+        model.__dict__["_llmq_kept_decoders"] = kept
+    decoders = kept["decoders"]
+    key = (prompt_tokens, new_tokens)
+    decoder = decoders.pop(key, None)
+    if decoder is None:
+        decoder = GraphedDecoder(model, prompt_tokens, new_tokens)
+        while len(decoders) >= _KEPT_RUNTIMES:
+            decoders.pop(next(iter(decoders)))
+    decoders[key] = decoder
+    return decoder
 
 
 class KernelDecoder:
@@ -201,12 +229,14 @@ def graphed_generate(model, input_ids, max_new_tokens: int, kv_bits: int | None 
     if kv_bits is not None:
         return kept_kernel_runtime(model, prompt + max_new_tokens + 1, kv_bits).generate(input_ids, max_new_tokens,
                                                                                          use_graph=True)
-    decoder = GraphedDecoder(model, prompt, max_new_tokens)
+    decoder = kept_graphed_decoder(model, prompt, max_new_tokens)
+    decoder.cache.reset()
     nxt = decoder.prefill(input_ids)
     out = [nxt]
     if max_new_tokens > 1:
         decoder.token.copy_(nxt.reshape(1, 1))
-        decoder.capture(prompt)
+        if decoder.graph is None:
+            decoder.capture(prompt)
         for i in range(1, max_new_tokens):
             nxt = decoder.step(nxt, prompt + i - 1)
             out.append(nxt)

@@ -98,8 +98,14 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
                     and _fusable(attn.o_proj) and _fusable(mlp.down_proj)):
                 raise ValueError("the fused decode step needs kernel-mode Linears (group 128, a multiple of 4 groups per "
                                  "row, no bias, weight-only) with q/k/v and gate/up sharing a bit width")
-            if attn.q_proj.out_group and attn.q_proj.qdata.shape[0] % attn.q_proj.out_group:
-                raise ValueError("q_proj rows are not a whole number of scale tiles")
+            for name in ("q_proj", "k_proj", "v_proj"):
+                proj = getattr(attn, name)
+                if proj.out_group and proj.qdata.shape[0] % proj.out_group:
+                    raise ValueError(f"{name} rows are not a whole number of scale tiles: the concatenated "
+                                     "q|k|v weight would misalign the scale rows of what follows it")
+            if any(m.out_group for m in (mlp.gate_proj, mlp.up_proj, mlp.down_proj)):
+                raise ValueError("the fused decode step takes MLP weights with one scale row per output row "
+                                 "(out_group 0)")
             args = attn.o_proj.scheme.weights
             self.fused_layers.append(dict(
                 qkv=_fused(attn, "_llmq_fused_qkv", attn.q_proj, attn.k_proj, attn.v_proj),

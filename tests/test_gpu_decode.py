@@ -315,7 +315,77 @@ def test_generate_calls_share_a_kept_runtime_and_its_captured_step(small):
     mlp.down_proj.wscale = mlp.down_proj.wscale.clone()
     assert kept_kernel_runtime(kernel, 33, 8) is not swapped
     assert torch.equal(graphed_generate(kernel, first, 12, kv_bits=8), fresh_a)
+    # tensors the step reads that are not quantized buffers: a norm weight replaced by a new Parameter, the
+    # embedding table swapped for another, a norm weight written in place. Each must drop what was kept
+    # (the captured step has the old addresses baked in) and the output must follow the new values.
+    before = kept_kernel_runtime(kernel, 33, 8)
+    norm = kernel.model.layers[1].input_layernorm
+    old_norm = norm.weight
+    norm.weight = torch.nn.Parameter(old_norm.detach() * 1.5, requires_grad=False)
+    after = kept_kernel_runtime(kernel, 33, 8)
+    assert after is not before
+    changed = graphed_generate(kernel, first, 12, kv_bits=8)
+    with torch.no_grad():
+        assert torch.equal(changed, kernel_runtime(kernel, 33, 8).generate(first, 12, use_graph=True))
+    assert not torch.equal(changed, fresh_a)
+    norm.weight = old_norm
+    assert torch.equal(graphed_generate(kernel, first, 12, kv_bits=8), fresh_a)
+    before = kept_kernel_runtime(kernel, 33, 8)
+    embed = kernel.model.embed_tokens
+    old_table = embed.weight
+    embed.weight = torch.nn.Parameter(old_table.detach().flip(0).contiguous(), requires_grad=False)
+    assert kept_kernel_runtime(kernel, 33, 8) is not before
+    flipped = graphed_generate(kernel, first, 12, kv_bits=8)
+    with torch.no_grad():
+        assert torch.equal(flipped, kernel_runtime(kernel, 33, 8).generate(first, 12, use_graph=True))
+    embed.weight = old_table
+    before = kept_kernel_runtime(kernel, 33, 8)
+    kernel.model.norm.weight.data.mul_(1.0)
+    assert kept_kernel_runtime(kernel, 33, 8) is not before
+    assert torch.equal(graphed_generate(kernel, first, 12, kv_bits=8), fresh_a)
     kernel.__dict__.pop("_llmq_kept_runtimes", None)
+
+
+def test_fused_runtime_refuses_layouts_it_does_not_take(small):
+    """MLP weights with tiled scales, or k_proj rows that are not whole scale tiles: the fused runtime's
+    constructor says so (ValueError) and kernel_runtime falls back to the operation-by-operation walk,
+    instead of a failure at capture time."""
+    from llmquant.runtime import LlamaFusedRuntime, LlamaKernelRuntime, kernel_runtime
+
+    _, kernel = small
+    mlp = kernel.model.layers[0].mlp
+    try:
+        mlp.gate_proj.out_group = mlp.up_proj.out_group = 64
+        with pytest.raises(ValueError, match="out_group 0"):
+            LlamaFusedRuntime(kernel, 64, 8)
+        assert type(kernel_runtime(kernel, 64, 8)) is LlamaKernelRuntime
+    finally:
+        mlp.gate_proj.out_group = mlp.up_proj.out_group = 0
+    assert isinstance(kernel_runtime(kernel, 64, 8), LlamaFusedRuntime)
+
+
+def test_the_bf16_baseline_keeps_its_captured_step_too():
+    """graphed_generate without kv_bits (the HF module walk over a StaticCache, the bf16 baseline): the
+    decoder and its captured graph are kept between calls as on the kernel side, and a second call with
+    another prompt gives what a fresh decoder gives."""
+    from llmquant.runtime import graphed_generate
+    from llmquant.runtime.graph_decode import kept_graphed_decoder
+
+    base = build_model(256, 512, 2, 4, 2, 1024, seed=3)
+    gen = torch.Generator().manual_seed(9)
+    a = torch.randint(0, 1024, (1, 12), generator=gen).cuda()
+    b = torch.randint(0, 1024, (1, 12), generator=gen).cuda()
+    out_a = graphed_generate(base, a, 10)
+    kept = kept_graphed_decoder(base, 12, 10)
+    graph = kept.graph
+    assert graph is not None
+    out_b = graphed_generate(base, b, 10)
+    assert kept_graphed_decoder(base, 12, 10) is kept and kept.graph is graph
+    base.__dict__.pop("_llmq_kept_decoders", None)
+    assert torch.equal(graphed_generate(base, b, 10), out_b)   # a fresh decoder and capture: same tokens
+    assert torch.equal(graphed_generate(base, a, 10), out_a)   # the kept one after another prompt used its cache
+    base.model.norm.weight.data.mul_(1.0)
+    assert kept_graphed_decoder(base, 12, 10) is not kept
 
 
 def test_measure_latency_reports_the_reference_keys():

@@ -405,6 +405,42 @@ def test_int4_view_is_int8_in_range(linear):
     assert module.qdata.dtype == torch.uint8 and module.qdata.shape[-1] == GROUP // 2
 
 
+@pytest.mark.parametrize("name", list(LAYOUTS))
+def test_state_dict_speaks_the_reference_buffer_names(name, linear):
+    """state_dict() of a kernel-mode Linear holds what the reference's module registers
+    (llmquant/quantizers/kernel.py:36-54): `qweight` int8 [N, groups, 128], `wscale` fp32 [scale_rows, groups],
+    `_broadcast_scale` fp32 [N, groups, 1]; load_state_dict takes that form (strict) as well as the stored
+    one (`qdata`, nibble-packed for 4 bits), and the loaded module computes what the source does."""
+    from llmquant.quantizers import KernelQuantLinear
+
+    spec = dict(LAYOUTS[name])
+    bits = spec.pop("bits")
+    scheme = weight_only(bits, **spec)
+    source = KernelQuantLinear.from_linear(linear.cuda(), scheme)
+    state = source.state_dict()
+    assert list(state) == ["qweight", "wscale", "_broadcast_scale"]
+    groups = source.padded_in_features // GROUP
+    assert state["qweight"].dtype == torch.int8 and state["qweight"].shape == (N, groups, GROUP)
+    assert torch.equal(state["qweight"], source.qweight)
+    assert state["_broadcast_scale"].shape == (N, groups, 1) and state["_broadcast_scale"].dtype == torch.float32
+    rows = N // state["wscale"].shape[0]
+    assert torch.equal(state["_broadcast_scale"][:, :, 0], state["wscale"].repeat_interleave(rows, dim=0))
+
+    torch.manual_seed(9)
+    other = nn.Linear(K, N, bias=False).to(torch.bfloat16).cuda()
+    x = torch.randn(2, K, device="cuda", dtype=torch.bfloat16)
+    for form in (state, {"qdata": source.qdata, "wscale": source.wscale}):
+        target = KernelQuantLinear.from_linear(other, scheme)
+        assert not torch.equal(target.qdata, source.qdata)
+        result = target.load_state_dict(form, strict=True)
+        assert not result.missing_keys and not result.unexpected_keys
+        assert target.qdata.dtype == source.qdata.dtype and torch.equal(target.qdata, source.qdata)
+        assert torch.equal(target.wscale, source.wscale)
+        assert torch.equal(target(x), source(x))
+    wrapped = nn.Sequential(source)
+    assert list(wrapped.state_dict()) == ["0.qweight", "0.wscale", "0._broadcast_scale"]
+
+
 def test_bias_is_applied():
     from llmquant.core.scheme import preset_name_to_scheme
     from llmquant.quantizers import KernelQuantLinear
