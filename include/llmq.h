@@ -197,6 +197,20 @@ int llmq_wq_gemm_a16_split(const void* x, const void* qweight, const float* wsca
                            void* workspace, size_t workspace_bytes, int M, int N, int G, int gs,
                            int out_group, int wformat, int dtype, llmq_stream_t stream);
 
+/* The same GEMM for prompt-sized activations (M in the hundreds and thousands), the reference's M > 4 branch
+ * (dequantize the whole weight to the activation dtype, then the BLAS library: llmquant/quantizers/kernel.py:
+ * 68-79, 88-91) without the dense weight: 128 x 256 output tiles, bf16 matrix cores, codes turned into bf16
+ * operands in registers, the reduction axis split across workgroups (fp32 partial tiles, added in a fixed
+ * order by a second launch) when the output has too few tiles to occupy the chip. Same sum as
+ * llmq_wq_gemm_a16: products exact, fp32 accumulation, one scale per group.
+ * x, out: LLMQ_BF16 only, 16-byte aligned; gs must be 128. `workspace`: llmq_wq_gemm_a16_tile_workspace_bytes
+ * (M, N, G) bytes, 16-byte aligned, contents irrelevant before and after (it holds the activation in operand
+ * order, its per-group sums, and the partial tiles). Calls that share a workspace must not overlap. */
+size_t llmq_wq_gemm_a16_tile_workspace_bytes(int M, int N, int G);
+int llmq_wq_gemm_a16_tile(const void* x, const void* qweight, const float* wscale, void* out, void* workspace,
+                          size_t workspace_bytes, int M, int N, int G, int gs, int out_group, int wformat,
+                          int dtype, llmq_stream_t stream);
+
 /* The elementwise pieces of a prompt pass, one launch each, with the rounding points of the PyTorch
  * sequences they replace (the same ones the decode kernels use). dtype: LLMQ_F32 / F16 / BF16; all
  * tensors 16-byte aligned. No counterpart in the reference, which leaves these to transformers

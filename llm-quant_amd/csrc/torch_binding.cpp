@@ -582,6 +582,40 @@ at::Tensor wq_gemm_a16(const at::Tensor& x, const at::Tensor& qweight, const at:
   return out;
 }
 
+// The fused GEMM for prompt-sized M (bf16): 128 x 256 tiles, no dense weight.
+at::Tensor wq_gemm_a16_tile(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale, int64_t out_group) {
+  TORCH_CHECK(x.is_cuda(), "x must be a CUDA tensor");
+  TORCH_CHECK(qweight.is_cuda() && wscale.is_cuda(), "qweight and wscale must be CUDA tensors");
+  TORCH_CHECK(x.scalar_type() == at::kBFloat16, "the tiled fused GEMM takes bfloat16 activations");
+  TORCH_CHECK(x.dim() == 2, "x must be [M, K]");
+  TORCH_CHECK(qweight.dim() == 3, "qweight must be [N, groups, group_size], got ", qweight.dim(), "D");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 2, "wscale must be float32 [scale_rows, groups]");
+  const auto xc = x.contiguous();
+  const auto wc = qweight.contiguous();
+  const auto sc = wscale.contiguous();
+  const int64_t M = xc.size(0), N = wc.size(0), groups = wc.size(1);
+  const int64_t group_size = packed ? wc.size(2) * 2 : wc.size(2);
+  TORCH_CHECK(group_size == 128, "the tiled fused GEMM needs group_size 128, got ", group_size);
+  TORCH_CHECK(xc.size(1) == groups * group_size, "x last dim ", xc.size(1), " does not match qweight ", groups, "x",
+              group_size);
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  TORCH_CHECK(sc.size(0) == scale_rows && sc.size(1) == groups, "wscale must be [", scale_rows, ", ", groups, "]");
+  auto out = at::empty({M, N}, xc.options());
+  if (M == 0 || N == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(xc));
+  const size_t need = llmq_wq_gemm_a16_tile_workspace_bytes(static_cast<int>(M), static_cast<int>(N), static_cast<int>(groups));
+  auto workspace = at::empty({static_cast<int64_t>((need + 3) / 4)}, xc.options().dtype(at::kFloat));
+  check_rc(llmq_wq_gemm_a16_tile(xc.const_data_ptr(), wc.const_data_ptr(), sc.const_data_ptr<float>(),
+                                 out.mutable_data_ptr(), workspace.mutable_data_ptr(), need, static_cast<int>(M),
+                                 static_cast<int>(N), static_cast<int>(groups), static_cast<int>(group_size),
+                                 static_cast<int>(out_group), packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8,
+                                 dtype_code(xc, "x"), current_stream(xc)),
+           "wq_gemm_a16_tile");
+  return out;
+}
+
 // ---- elementwise pieces of a prompt pass ----------------------------------------------------------------
 at::Tensor rmsnorm(const at::Tensor& x, const at::Tensor& weight, double eps) {
   TORCH_CHECK(x.is_cuda() && weight.is_cuda(), "x and weight must be CUDA tensors");
@@ -1034,6 +1068,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("wq_gemm_a16", &wq_gemm_a16,
         "Weight-only GEMM for a few dozen rows: fp16/bf16 activations x int4/int8 group-quantized weights, no dense copy",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("split") = false);
+  m.def("wq_gemm_a16_tile", &wq_gemm_a16_tile,
+        "Fused weight-only GEMM for prompt-sized bf16 activations: 128 x 256 tiles on the bf16 matrix cores, no dense weight",
+        py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0);
   m.def("rmsnorm", &rmsnorm, "LlamaRMSNorm over the last axis, one launch", py::arg("x"), py::arg("weight"), py::arg("eps"));
   m.def("add_rmsnorm", &add_rmsnorm, "(x + delta, LlamaRMSNorm(x + delta)), one launch", py::arg("x"), py::arg("delta"),
         py::arg("weight"), py::arg("eps"));

@@ -1,0 +1,472 @@
+// Weight-only quantized GEMM for prompt-sized activations (M in the hundreds and thousands), gfx950:
+// bf16 activations times int4 / int8 group-quantized weights on the bf16 matrix core, with no dense
+// copy of the weight anywhere.
+//
+//   out[m, n] = sum over g of  wscale[sr(n), g] * sum_k x[m, g*128 + k] * code[n, g, k]
+//
+// the weight-only branch of RealQuantLinear.forward (llmquant/quantizers/real.py:84-91): products of a
+// bf16 value and a small integer are exact in fp32, the matrix core adds them in fp32, and the scale is
+// applied once per group. (The reference's kernel mode dequantizes the whole weight to the activation
+// dtype and calls the BLAS library for M > 4, llmquant/quantizers/kernel.py:68-79,88-91: nine times the
+// int4 codes' bytes through HBM per call, and a second rounding per weight.)
+//
+// Shape. A workgroup of four waves owns a 128 (m) x 256 (n) tile of the output; every wave owns 64 of
+// the 256 columns and all 128 rows: 4 x 2 MFMA tiles of 32 x 32 (v_mfma_f32_32x32x16_bf16), eight
+// k-steps of 16 per group. What bounds a tiled GEMM on this chip is LDS bandwidth (one 16-byte operand
+// read per lane per MFMA is all the LDS delivers), so only the activation goes through LDS, shared by
+// the four waves, and each operand read feeds two MFMAs; the weights never touch LDS: a lane reads the
+// codes of its own column straight from HBM in operand layout (32 bytes of int4 or 64 of int8 per group)
+// and converts them in registers.
+//
+// Codes become bf16 without a conversion instruction: a nibble n = code + 8 placed in the mantissa of
+// 16.0 (bits 0x4180 | n << 3) IS the bf16 value 16 + n, two nibbles per AND-OR (int8: code + 128 through
+// v_cvt_f32_ubyte, whose upper half is the bf16 value). The matrix core therefore sums x * (code + B),
+// B = 24 or 128, and B * sum_k x is taken out again per group. That correction is a rank-one term,
+// -B * wscale[n, g] * xsum[m, g], and it too runs on the matrix core: both factors are cut into three
+// bf16 pieces and the six significant cross products fill one more k-step, accumulated straight into
+// the running total.
+//
+// The activation is prepared once per call by act_prep_kernel: within every 16-byte chunk the eight
+// values are reordered to (0, 4, 1, 5, 2, 6, 3, 7), the order in which the AND-OR above leaves the
+// codes (a sum does not care about the order of its terms, as long as both operands agree), and the
+// per-group sums are cut into their bf16 pieces. The GEMM then moves activation tiles from global
+// memory to LDS without passing through registers (global_load_lds_dwordx4), XOR-swizzled by row so the
+// operand reads are conflict-free.
+//
+// Small N: a split of the reduction axis across workgroups, fp32 partial tiles in a workspace, added in a
+// fixed order by a second launch (the result does not depend on which workgroup finished first).
+#include "llmq_device.h"
+
+namespace {
+
+using namespace llmq;
+
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kGroup = 128;
+constexpr int kBM = 128;            // activation rows per workgroup
+constexpr int kWaveN = 64;          // weight rows (output columns) per wave
+constexpr int kWaves = 4;
+constexpr int kBN = kWaveN * kWaves;
+constexpr int kThreads = kWaves * kWave;
+constexpr int kRowBytes = kGroup * 2;          // one activation row of one group
+constexpr int kTileBytes = kBM * kRowBytes;    // 32 KB
+constexpr int kMT = kBM / 32, kNT = kWaveN / 32;
+
+template <int BITS> constexpr float kCodeBias = BITS == 4 ? 24.0f : 128.0f;
+
+// ---- activation preparation -----------------------------------------------------------------------
+// One lane per 16-byte chunk, 16 lanes per (row, group).
+__global__ __launch_bounds__(256) void act_prep_kernel(const u32x4* __restrict__ x, u32x4* __restrict__ xp,
+                                                       u32x4* __restrict__ rec, const int64_t n_chunks) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const bool active = i < n_chunks;  // n_chunks is a multiple of 16: a row of 16 lanes is active or idle as one
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (active) v = x[i];
+  float f[8];
+  Pack<bf16_t>::unpack(v, f);
+  float s = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
+  s = row16_sum(s);
+  if (!active) return;
+  // (x0 x1)(x2 x3)(x4 x5)(x6 x7) -> (x0 x4)(x1 x5)(x2 x6)(x3 x7)
+  u32x4 o;
+  o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+  o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+  o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+  o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+  xp[i] = o;
+  if ((threadIdx.x & 15) == 0) {
+    // s = hi + mid + lo, each a bf16: 24 bits of the sum
+    const uint32_t hi = bf16_bits_rne(s);
+    const float r1 = s - __builtin_bit_cast(float, hi << 16);
+    const uint32_t mid = bf16_bits_rne(r1);
+    const float r2 = r1 - __builtin_bit_cast(float, mid << 16);
+    const uint32_t lo = bf16_bits_rne(r2);
+    rec[i >> 4] = u32x4{hi | (mid << 16), lo, 0u, 0u};  // k' slots 0..2 of the correction step
+  }
+}
+
+struct TileArgs {
+  const uint8_t* xp;   // [M, G*128] bf16, chunks reordered
+  const uint8_t* rec;  // [M, G] records of 16 bytes
+  const uint8_t* qw;   // [N, G, 128] int8 or [N, G, 64] packed int4
+  const float* sw;     // [scale_rows, G]
+  void* out;           // [M, N] bf16 (one split)
+  float* partial;      // [splits][M][N] fp32 (more)
+  int M, N, G, out_group;
+  int m_tiles, n_tiles, splits, groups_per_split;
+};
+
+// LDS, per buffer (two buffers): the activation tile [128 rows][16 slots of 16 bytes], the raw codes of
+// the workgroup's 256 weight rows for one group ([256][64] bytes of int4 or [256][128] of int8, slots
+// XOR-swizzled by row like the activation), and the 128 activation-sum records.
+template <int BITS> constexpr int kCodeRowBytes = BITS == 4 ? kGroup / 2 : kGroup;
+template <int BITS> constexpr int kCodeTileBytes = kBN * kCodeRowBytes<BITS>;
+constexpr int kRecTileBytes = kBM * 16;
+template <int BITS> constexpr int kStageBytes = kTileBytes + kCodeTileBytes<BITS> + kRecTileBytes;
+template <int BITS> constexpr int kLdsBytes = 2 * kStageBytes<BITS>;
+
+// slot of chunk c in weight row `row`: 16 consecutive rows read the same chunk at once and must land in
+// 16 different bank quads
+template <int BITS> __device__ __forceinline__ int code_slot(int row, int c) {
+  return BITS == 4 ? c ^ ((row >> 2) & 3) : c ^ ((row >> 1) & 7);
+}
+
+// (value & mask) | bits in one instruction; the compiler leaves it as two. One operand of a VOP3 may
+// come from a scalar register on this chip, so the mask is scalar and the bits sit in a vector register.
+constexpr uint32_t kNibbleMask = 0x00780078u;
+__device__ __forceinline__ uint32_t and_or(uint32_t value, uint32_t mask_scalar, uint32_t bits) {
+  uint32_t d;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(value), "s"(mask_scalar), "v"(bits));
+  return d;
+}
+
+template <int BITS>
+__device__ __forceinline__ v8bf code_operand(const u32x4* raw, int step, uint32_t sixteen) {
+  uint32_t b[4];
+  if constexpr (BITS == 4) {
+    const u32x4 q = raw[step >> 2];
+    const uint32_t w = (step & 3) == 0 ? q.x : (step & 3) == 1 ? q.y : (step & 3) == 2 ? q.z : q.w;
+    b[0] = and_or(w << 3, kNibbleMask, sixteen);  // nibbles 0 and 4
+    b[1] = and_or(w >> 1, kNibbleMask, sixteen);  // 1 and 5
+    b[2] = and_or(w >> 5, kNibbleMask, sixteen);  // 2 and 6
+    b[3] = and_or(w >> 9, kNibbleMask, sixteen);  // 3 and 7
+  } else {
+    const u32x4 q = raw[step >> 1];
+    const uint32_t w0 = ((step & 1) ? q.z : q.x) ^ 0x80808080u;  // codes 0..3 of the step, + 128
+    const uint32_t w1 = ((step & 1) ? q.w : q.y) ^ 0x80808080u;  // codes 4..7
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float lo = static_cast<float>((w0 >> (8 * i)) & 0xffu);
+      const float hi = static_cast<float>((w1 >> (8 * i)) & 0xffu);
+      // integers below 256: the upper half of the float is the bf16 value, exactly
+      b[i] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, hi), __builtin_bit_cast(uint32_t, lo), 0x07060302u);
+    }
+  }
+  return __builtin_bit_cast(v8bf, u32x4{b[0], b[1], b[2], b[3]});
+}
+
+template <int BITS>
+__global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const TileArgs a) {
+  extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
+
+  // Workgroups are dealt to the 8 XCDs round-robin by their index; a run of consecutive logical tiles
+  // (the m-tiles of one n-tile first: they read the same weights) is put on one XCD, so the codes come
+  // out of that XCD's L2 after the first reader.
+  const int n_work = a.m_tiles * a.n_tiles * a.splits;
+  const int per_xcd = (n_work + 7) / 8;
+  const int logical = static_cast<int>(blockIdx.x % 8) * per_xcd + static_cast<int>(blockIdx.x / 8);
+  if (logical >= n_work) return;
+  const int mt = logical % a.m_tiles;
+  const int nt = (logical / a.m_tiles) % a.n_tiles;
+  const int sp = logical / (a.m_tiles * a.n_tiles);
+
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int lm = lane & 31, lh = lane >> 5;
+  const int m0 = mt * kBM, n0 = nt * kBN;
+  const int g_begin = sp * a.groups_per_split;
+  const int g_end = min(g_begin + a.groups_per_split, a.G);
+
+  // ---- global -> LDS: what this lane fetches for each of its wave's transfer instructions -------------
+  // One instruction moves 64 x 16 bytes into 1 KB of consecutive LDS; which global chunk a lane fetches
+  // for its place there carries the swizzle.
+  // activation: instruction i of a wave = rows wv*32 + 4 i .. + 3, lane = (row, slot)
+  const uint32_t x_row_bytes = static_cast<uint32_t>(a.G) * kRowBytes;
+  uint32_t x_off[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = wv * 32 + i * 4 + (lane >> 4);
+    const int chunk = (lane & 15) ^ (row & 15);
+    x_off[i] = static_cast<uint32_t>(min(m0 + row, a.M - 1)) * x_row_bytes + chunk * 16;
+  }
+  // codes: 4 (int4) or 8 (int8) instructions per wave; 16 or 8 weight rows each
+  constexpr int kCodeInstr = kCodeTileBytes<BITS> / 1024 / kWaves;
+  constexpr int kRowsPerInstr = 1024 / kCodeRowBytes<BITS>;
+  constexpr int kSlots = kCodeRowBytes<BITS> / 16;
+  const uint32_t w_row_bytes = static_cast<uint32_t>(a.G) * kCodeRowBytes<BITS>;
+  uint32_t w_off[kCodeInstr];
+#pragma unroll
+  for (int i = 0; i < kCodeInstr; ++i) {
+    const int row = (wv * kCodeInstr + i) * kRowsPerInstr + lane / kSlots;
+    const int chunk = code_slot<BITS>(row, lane % kSlots);  // the swizzle is its own inverse
+    w_off[i] = static_cast<uint32_t>(min(n0 + row, a.N - 1)) * w_row_bytes + chunk * 16;
+  }
+  // records: waves 0 and 1, 64 rows each
+  const uint32_t r_off = static_cast<uint32_t>(min(m0 + (wv & 1) * 64 + lane, a.M - 1)) * a.G * 16;
+
+  auto request = [&](int g, int buf) {
+    uint8_t* stage = smem + buf * kStageBytes<BITS>;
+    const uint8_t* xg = a.xp + static_cast<uint32_t>(g) * kRowBytes;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(xg + x_off[i]),
+                                       reinterpret_cast<u32x4*>(stage + (wv * 32 + i * 4) * kRowBytes), 16, 0, 0);
+    }
+    const uint8_t* wg = a.qw + static_cast<uint32_t>(g) * kCodeRowBytes<BITS>;
+#pragma unroll
+    for (int i = 0; i < kCodeInstr; ++i) {
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(wg + w_off[i]),
+                                       reinterpret_cast<u32x4*>(stage + kTileBytes + (wv * kCodeInstr + i) * 1024), 16,
+                                       0, 0);
+    }
+    if (wv < 2) {
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(a.rec + r_off + static_cast<uint32_t>(g) * 16),
+                                       reinterpret_cast<u32x4*>(stage + kTileBytes + kCodeTileBytes<BITS> + wv * 1024),
+                                       16, 0, 0);
+    }
+  };
+
+  // ---- LDS -> operands ----------------------------------------------------------------------------------
+  // activation operand of k-step j: row mi*32 + lm, chunk 8 lh + j
+  uint32_t a_off[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) a_off[j] = lm * kRowBytes + (((8 * lh + j) ^ (lm & 15)) << 4);
+  // this lane's codes of a group: weight row wv*64 + ni*32 + lm, k in [64 lh, 64 lh + 64)
+  constexpr int kRawLoads = BITS == 4 ? 2 : 4;
+  uint32_t c_off[kNT][kRawLoads];
+  const float* s_ptr[kNT];
+#pragma unroll
+  for (int ni = 0; ni < kNT; ++ni) {
+    const int row = wv * kWaveN + ni * 32 + lm;
+#pragma unroll
+    for (int q = 0; q < kRawLoads; ++q)
+      c_off[ni][q] = kTileBytes + row * kCodeRowBytes<BITS> + code_slot<BITS>(row, lh * kRawLoads + q) * 16;
+    const int n = min(n0 + row, a.N - 1);
+    s_ptr[ni] = a.sw + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * a.G;
+  }
+
+  float total[kMT][kNT][16];
+#pragma unroll
+  for (int mi = 0; mi < kMT; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < kNT; ++ni)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) total[mi][ni][r] = 0.0f;
+  uint32_t sixteen = 0x41804180u;  // bf16 16.0 twice; kept in a vector register (see and_or)
+  asm volatile("" : "+v"(sixteen));
+
+  request(g_begin, 0);
+  float scale_next[kNT];
+#pragma unroll
+  for (int ni = 0; ni < kNT; ++ni) scale_next[ni] = s_ptr[ni][g_begin];
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  for (int g = g_begin; g < g_end; ++g) {
+    const int buf = (g - g_begin) & 1;
+    float scale[kNT];
+#pragma unroll
+    for (int ni = 0; ni < kNT; ++ni) scale[ni] = scale_next[ni];
+    if (g + 1 < g_end) {
+      request(g + 1, buf ^ 1);
+#pragma unroll
+      for (int ni = 0; ni < kNT; ++ni) scale_next[ni] = s_ptr[ni][g + 1];
+    }
+    const uint8_t* stage = smem + buf * kStageBytes<BITS>;
+
+    u32x4 raw[kNT][kRawLoads];
+#pragma unroll
+    for (int ni = 0; ni < kNT; ++ni)
+#pragma unroll
+      for (int q = 0; q < kRawLoads; ++q) raw[ni][q] = *reinterpret_cast<const u32x4*>(stage + c_off[ni][q]);
+
+    // The group's sums start at -B * xsum[m] (one k-step: the three bf16 pieces of the activation sum
+    // against the constant -B; the upper half of the wave, k' 8..15, multiplies zeros), then take the
+    // eight k-steps of x * (code + B).
+    v16f acc[kMT][kNT];
+    {
+      const uint32_t nb = bf16_bits_rne(-kCodeBias<BITS>);  // exact
+      const uint32_t nb2 = lh ? 0u : (nb | (nb << 16));
+      const v8bf bv = __builtin_bit_cast(v8bf, u32x4{nb2, nb2, 0u, 0u});
+      const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int mi = 0; mi < kMT; ++mi) {
+        const v8bf rec = __builtin_bit_cast(
+            v8bf, *reinterpret_cast<const u32x4*>(stage + kTileBytes + kCodeTileBytes<BITS> + (mi * 32 + lm) * 16));
+#pragma unroll
+        for (int ni = 0; ni < kNT; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rec, bv, zero, 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      v8bf fa[kMT], fb[kNT];
+#pragma unroll
+      for (int mi = 0; mi < kMT; ++mi)
+        fa[mi] = __builtin_bit_cast(v8bf, *reinterpret_cast<const u32x4*>(stage + mi * 32 * kRowBytes + a_off[j]));
+#pragma unroll
+      for (int ni = 0; ni < kNT; ++ni) fb[ni] = code_operand<BITS>(raw[ni], j, sixteen);
+#pragma unroll
+      for (int mi = 0; mi < kMT; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < kNT; ++ni)
+          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi], fb[ni], acc[mi][ni], 0, 0, 0);
+    }
+#pragma unroll
+    for (int mi = 0; mi < kMT; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < kNT; ++ni)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) total[mi][ni][r] = fmaf(scale[ni], acc[mi][ni][r], total[mi][ni][r]);
+
+    // the next group has landed in the other buffer, and nobody reads this one any more
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+
+  // ---- store: register r of a 32 x 32 tile is row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
+  if (a.splits == 1) {
+    bf16_t* __restrict__ out = static_cast<bf16_t*>(a.out);
+#pragma unroll
+    for (int ni = 0; ni < kNT; ++ni) {
+      const int n = n0 + wv * kWaveN + ni * 32 + lm;
+#pragma unroll
+      for (int mi = 0; mi < kMT; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          if (m < a.M && n < a.N) out[static_cast<int64_t>(m) * a.N + n] = from_float<bf16_t>(total[mi][ni][r]);
+        }
+    }
+  } else {
+    float* __restrict__ part = a.partial + static_cast<int64_t>(sp) * a.M * a.N;
+#pragma unroll
+    for (int ni = 0; ni < kNT; ++ni) {
+      const int n = n0 + wv * kWaveN + ni * 32 + lm;
+#pragma unroll
+      for (int mi = 0; mi < kMT; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          if (m < a.M && n < a.N) part[static_cast<int64_t>(m) * a.N + n] = total[mi][ni][r];
+        }
+    }
+  }
+}
+
+// out[i] = bf16(partial[0][i] + partial[1][i] + ...), slices added in order; four values per lane.
+__global__ __launch_bounds__(256) void add_splits_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
+                                                         const int64_t count, const int splits) {
+  const int64_t i4 = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  if (i4 >= count) return;
+  if (i4 + 4 <= count && (count & 3) == 0) {
+    u32x4 v = load16(partial + i4);
+    float s[4];
+    Pack<float>::unpack(v, s);
+    for (int k = 1; k < splits; ++k) {
+      float t[4];
+      Pack<float>::unpack(load16(partial + k * count + i4), t);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] = s[e] + t[e];
+    }
+    *reinterpret_cast<u32x2*>(out + i4) = u32x2{bf16_pair_rne(s[0], s[1]), bf16_pair_rne(s[2], s[3])};
+  } else {
+    for (int64_t i = i4; i < count; ++i) {
+      float s = partial[i];
+      for (int k = 1; k < splits; ++k) s = s + partial[k * count + i];
+      out[i] = from_float<bf16_t>(s);
+    }
+  }
+}
+
+template <int BITS>
+int launch_tiles(const TileArgs& a, dim3 grid, hipStream_t stream) {
+  auto kernel = wq_gemm_a16_tile_kernel<BITS>;
+  static bool raised = false;  // per instantiation; worst case two threads both set it
+  if (!raised) {
+    const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes<BITS>);
+    if (err != hipSuccess) {
+      llmq_host::set_error("raising the LDS limit failed: %s", hipGetErrorString(err));
+      return static_cast<int>(err);
+    }
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(kThreads), kLdsBytes<BITS>, stream, a);
+  return llmq_host::check_launch("wq_gemm_a16_tile_kernel");
+}
+
+constexpr size_t kAlign = 256;
+size_t aligned(size_t bytes) { return (bytes + kAlign - 1) / kAlign * kAlign; }
+
+struct Plan {
+  int m_tiles, n_tiles, splits, groups_per_split;
+  size_t xp_bytes, rec_bytes, partial_bytes;
+};
+
+Plan plan_for(int M, int N, int G) {
+  Plan p{};
+  p.m_tiles = (M + kBM - 1) / kBM;
+  p.n_tiles = (N + kBN - 1) / kBN;
+  const int tiles = p.m_tiles * p.n_tiles;
+  // fewer tiles than would occupy most CUs: cut the reduction axis, at least four groups per slice
+  int splits = 1;
+  if (tiles < 160) {
+    splits = (256 + tiles - 1) / tiles;
+    if (splits > G / 4) splits = G / 4;
+    if (splits < 1) splits = 1;
+  }
+  p.groups_per_split = (G + splits - 1) / splits;
+  p.splits = (G + p.groups_per_split - 1) / p.groups_per_split;  // every slice holds at least one group
+  p.xp_bytes = aligned(static_cast<size_t>(M) * G * kRowBytes);
+  p.rec_bytes = aligned(static_cast<size_t>(M) * G * 16);
+  p.partial_bytes = p.splits > 1 ? aligned(static_cast<size_t>(p.splits) * M * N * sizeof(float)) : 0;
+  return p;
+}
+
+}  // namespace
+
+extern "C" size_t llmq_wq_gemm_a16_tile_workspace_bytes(int M, int N, int G) {
+  if (M <= 0 || N <= 0 || G <= 0) return 0;
+  const Plan p = plan_for(M, N, G);
+  return p.xp_bytes + p.rec_bytes + p.partial_bytes;
+}
+
+extern "C" int llmq_wq_gemm_a16_tile(const void* x, const void* qweight, const float* wscale, void* out,
+                                     void* workspace, size_t workspace_bytes, int M, int N, int G, int gs,
+                                     int out_group, int wformat, int dtype, llmq_stream_t stream) {
+  if (M < 0 || N < 0 || G < 0) return llmq_host::fail_invalid("negative dimension M=%d N=%d G=%d", M, N, G);
+  if (gs != kGroup) return llmq_host::fail_invalid("the tiled fused GEMM needs group_size 128, got %d", gs);
+  if (dtype != LLMQ_BF16) return llmq_host::fail_invalid("the tiled fused GEMM takes bfloat16 activations, got dtype code %d", dtype);
+  if (wformat != LLMQ_W_INT8 && wformat != LLMQ_W_INT4_PACKED)
+    return llmq_host::fail_invalid("unsupported weight format %d, expected 8 or 4", wformat);
+  if (out_group < 0) return llmq_host::fail_invalid("out_group must be >= 0, got %d", out_group);
+  if (M == 0 || N == 0) return 0;
+  if (G == 0) return llmq_host::fail_invalid("a weight with no groups has no reduction axis");
+  if (!x || !qweight || !wscale || !out || !workspace) return llmq_host::fail_invalid("null tensor pointer");
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(qweight) | reinterpret_cast<uintptr_t>(workspace) |
+       reinterpret_cast<uintptr_t>(out)) & 15u)
+    return llmq_host::fail_invalid("activation, weight, output and workspace pointers must be 16-byte aligned");
+  if (static_cast<uint64_t>(M) * G * kRowBytes >= (1ull << 32))
+    return llmq_host::fail_invalid("activation of %d x %d values is beyond the kernel's 32-bit offsets", M, G * kGroup);
+  const Plan p = plan_for(M, N, G);
+  if (workspace_bytes < p.xp_bytes + p.rec_bytes + p.partial_bytes)
+    return llmq_host::fail_invalid("workspace of %zu bytes is too small, need %zu", workspace_bytes,
+                                   p.xp_bytes + p.rec_bytes + p.partial_bytes);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint8_t* ws = static_cast<uint8_t*>(workspace);
+  uint8_t* xp = ws;
+  uint8_t* rec = ws + p.xp_bytes;
+  float* partial = reinterpret_cast<float*>(ws + p.xp_bytes + p.rec_bytes);
+
+  const int64_t n_chunks = static_cast<int64_t>(M) * G * 16;
+  hipLaunchKernelGGL(act_prep_kernel, dim3(static_cast<unsigned>((n_chunks + 255) / 256)), dim3(256), 0, s,
+                     static_cast<const u32x4*>(x), reinterpret_cast<u32x4*>(xp), reinterpret_cast<u32x4*>(rec),
+                     n_chunks);
+  if (int rc = llmq_host::check_launch("act_prep_kernel")) return rc;
+
+  TileArgs a{xp, rec, static_cast<const uint8_t*>(qweight), wscale, out, partial, M, N, G, out_group,
+             p.m_tiles, p.n_tiles, p.splits, p.groups_per_split};
+  const int total = p.m_tiles * p.n_tiles * p.splits;
+  const dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8));
+  if (static_cast<uint64_t>(N) * G * kGroup >= (1ull << 32))
+    return llmq_host::fail_invalid("weight of %d x %d codes is beyond the kernel's 32-bit offsets", N, G * kGroup);
+  if (int rc = wformat == LLMQ_W_INT4_PACKED ? launch_tiles<4>(a, grid, s) : launch_tiles<8>(a, grid, s)) return rc;
+  if (p.splits > 1) {
+    const int64_t count = static_cast<int64_t>(M) * N;
+    hipLaunchKernelGGL(add_splits_kernel, dim3(static_cast<unsigned>((count / 4 + 256) / 256)), dim3(256), 0, s,
+                       partial, static_cast<bf16_t*>(out), count, p.splits);
+    return llmq_host::check_launch("add_splits_kernel");
+  }
+  return 0;
+}

@@ -117,6 +117,10 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_wq_gemm_a16.restype = c_int
     lib.llmq_wq_gemm_a16_split.argtypes = [c_p] * 5 + [ctypes.c_size_t] + [c_int] * 7 + [c_p]
     lib.llmq_wq_gemm_a16_split.restype = c_int
+    lib.llmq_wq_gemm_a16_tile.argtypes = [c_p] * 5 + [ctypes.c_size_t] + [c_int] * 7 + [c_p]
+    lib.llmq_wq_gemm_a16_tile.restype = c_int
+    lib.llmq_wq_gemm_a16_tile_workspace_bytes.argtypes = [c_int] * 3
+    lib.llmq_wq_gemm_a16_tile_workspace_bytes.restype = ctypes.c_size_t
     lib.llmq_wq_gemm_a16_workspace_bytes.argtypes = [c_int] * 3
     lib.llmq_wq_gemm_a16_workspace_bytes.restype = ctypes.c_size_t
     lib.llmq_rmsnorm.argtypes = [c_p, c_p, c_p, c_int, c_int, ctypes.c_float, c_int, c_p]

@@ -136,3 +136,102 @@ def test_split_form_repeats_itself_and_checks_its_workspace(ext):
     rc = lib.llmq_wq_gemm_a16_split(xd.data_ptr(), q.data_ptr(), s.data_ptr(), out.data_ptr(), small.data_ptr(),
                                     small.numel() * 4, 16, 384, 16, 128, 0, 4, 2, None)
     assert rc != 0 and b"workspace" in lib.llmq_last_error()
+
+
+# ---- the tiled form for prompt-sized M ---------------------------------------------------------------------
+
+
+def tile_case(ext, m, n, k, bits, out_group=0, head_dim=None, seed=0, scale=1.0, offset=0.0):
+    """x [m, k] bf16 against a quantized [n, k] weight through wq_gemm_a16_tile; returns the result and the
+    oracle's operands (activation padded the way the weight was)."""
+    torch.manual_seed(seed)
+    w = (torch.randn(n, k) * 0.02).to(torch.bfloat16)
+    x = (torch.randn(m, k) * scale + offset).to(torch.bfloat16)
+    canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP, head_dim, out_group or None)
+    q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
+    s = torch.from_numpy(scales).cuda()
+    padded = oracle.pad_activation(to_np(x), GROUP, head_dim)
+    got = ext.wq_gemm_a16_tile(torch.from_numpy(padded).to(torch.bfloat16).cuda(), q, s, out_group)
+    return got, padded, canonical, scales
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,n,k", [(128, 256, 128), (65, 256, 256), (130, 300, 768), (512, 512, 2048), (300, 70, 384),
+                                   (129, 257, 1152), (1, 16, 128), (256, 1024, 8192)])
+def test_tiled_gemm_against_the_oracle(ext, bits, m, n, k):
+    """Whole outputs against the float64 closed form and the real-mode forward: full tiles, ragged M and N
+    (rows and columns past the end are clamped for the loads and dropped at the store), one group, rows long
+    enough that the reduction axis is split across workgroups."""
+    got, x, canonical, scales = tile_case(ext, m, n, k, bits, seed=m + n)
+    assert got.shape == (m, n) and got.dtype == torch.bfloat16
+    exact = oracle.gemv_float64(x, canonical, scales)
+    assert rel_l2(to_np(got), exact) <= 2e-3
+    real = oracle.real_linear(x, canonical, scales, "bf16")
+    assert ulp_distance(to_np(got), real, torch.bfloat16) <= 1
+    assert (to_np(got) == real).mean() > 0.99
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_tiled_gemm_with_one_signed_activation(ext, bits):
+    """Activations that do not cancel (all positive, mean 3): the codes enter the matrix core with an offset
+    (code + 24 or + 128) that is taken out per group through the activation's sum, and this is the input on
+    which that term is largest beside the result."""
+    got, x, canonical, scales = tile_case(ext, 256, 512, 1024, bits, seed=5, scale=0.5, offset=3.0)
+    exact = oracle.gemv_float64(x, canonical, scales)
+    assert rel_l2(to_np(got), exact) <= 2e-3
+    wide = ext.wq_gemm_a16_tile((torch.from_numpy(x) * 0 + 1).to(torch.bfloat16).cuda(),
+                                torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda(),
+                                torch.from_numpy(scales).cuda(), 0)
+    ones = oracle.gemv_float64(np.ones_like(x), canonical, scales)   # x = 1: the plain row sums of the weight
+    assert rel_l2(to_np(wide), ones) <= 4e-3
+
+
+PREFILL_SHAPES = {
+    "q|k|v 3072x2048 int8, one scale row per head": dict(n=3072, k=2048, bits=8, out_group=64),
+    "o_proj 2048x2048 int8, heads of 64 padded to groups": dict(n=2048, k=2048, bits=8, head_dim=64),
+    "gate|up 16384x2048 int4": dict(n=16384, k=2048, bits=4),
+    "down 2048x8192 int4": dict(n=2048, k=8192, bits=4),
+}
+
+
+@pytest.mark.parametrize("name", list(PREFILL_SHAPES))
+def test_tiled_gemm_at_the_prompt_pass_shapes(ext, name):
+    """The four projections of a 512-token prompt pass of the Llama-3.2-1B configuration, on 96 x 128 sampled
+    outputs (and the last rows and columns) against the float64 closed form, rel-L2 <= 2e-3, and against the
+    real-mode forward restricted to the sample."""
+    spec = dict(PREFILL_SHAPES[name])
+    m, n, k, bits = 512, spec.pop("n"), spec.pop("k"), spec.pop("bits")
+    got, x, canonical, scales = tile_case(ext, m, n, k, bits, seed=11, **spec)
+    out_group = spec.get("out_group")
+    rng = np.random.default_rng(3)
+    rows = np.unique(np.concatenate([rng.choice(m, 96, replace=False), [m - 1]]))
+    cols = np.unique(np.concatenate([rng.choice(n, 128, replace=False), [n - 1]]))
+    full_scales = np.repeat(scales, out_group, axis=0)[:n] if out_group else scales
+    exact = oracle.gemv_float64(x[rows], canonical[cols], full_scales[cols])
+    sample = to_np(got)[np.ix_(rows, cols)]
+    assert rel_l2(sample, exact) <= 2e-3
+    real = oracle.real_linear(x[rows], canonical[cols], full_scales[cols], "bf16")
+    assert (sample == real).mean() > 0.99 and ulp_distance(sample, real, torch.bfloat16) <= 1
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("m", [128, 2048])
+def test_tiled_gemm_at_llama_8b_mlp_shapes(ext, n, k, m):
+    got, x, canonical, scales = tile_case(ext, m, n, k, 4, seed=13)
+    rng = np.random.default_rng(4)
+    rows = np.sort(rng.choice(m, 64, replace=False))
+    cols = np.sort(rng.choice(n, 96, replace=False))
+    exact = oracle.gemv_float64(x[rows], canonical[cols], scales[cols])
+    assert rel_l2(to_np(got)[np.ix_(rows, cols)], exact) <= 2e-3
+
+
+def test_tiled_gemm_argument_checks(ext):
+    x, q, s, _, _ = make_case(128, 256, 256, 4, torch.bfloat16)
+    assert ext.wq_gemm_a16_tile(x.cuda(), q, s, 0).shape == (128, 256)
+    with pytest.raises(RuntimeError, match="bfloat16"):
+        ext.wq_gemm_a16_tile(x.cuda().half(), q, s, 0)
+    with pytest.raises(RuntimeError, match="does not match qweight"):
+        ext.wq_gemm_a16_tile(x.cuda()[:, :128].contiguous(), q, s, 0)
+    with pytest.raises(RuntimeError, match="wscale must be"):
+        ext.wq_gemm_a16_tile(x.cuda(), q, s[:-1], 0)
+    assert ext.wq_gemm_a16_tile(x.cuda()[:0], q, s, 0).shape == (0, 256)
