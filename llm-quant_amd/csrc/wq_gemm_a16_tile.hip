@@ -10,31 +10,35 @@
 // dtype and calls the BLAS library for M > 4, llmquant/quantizers/kernel.py:68-79,88-91: nine times the
 // int4 codes' bytes through HBM per call, and a second rounding per weight.)
 //
-// Shape. A workgroup of four waves owns a 128 (m) x 256 (n) tile of the output; every wave owns 64 of
-// the 256 columns and all 128 rows: 4 x 2 MFMA tiles of 32 x 32 (v_mfma_f32_32x32x16_bf16), eight
-// k-steps of 16 per group. What bounds a tiled GEMM on this chip is LDS bandwidth (one 16-byte operand
-// read per lane per MFMA is all the LDS delivers), so only the activation goes through LDS, shared by
-// the four waves, and each operand read feeds two MFMAs; the weights never touch LDS: a lane reads the
-// codes of its own column straight from HBM in operand layout (32 bytes of int4 or 64 of int8 per group)
-// and converts them in registers.
+// Shape. A workgroup of eight waves owns a 128 (m) x 256 (n) tile of the output, two waves per SIMD; a
+// wave owns 64 rows x 64 columns: 2 x 2 MFMA tiles of 32 x 32 (v_mfma_f32_32x32x16_bf16), eight k-steps
+// of 16 per group, accumulators and running totals in vector registers (128 of them, which is what lets
+// two waves share a SIMD: one converts codes or folds its group sums into the totals while the other
+// keeps the matrix core busy). Every operand reaches LDS straight from global memory, without passing
+// through registers (global_load_lds_dwordx4, 1 KB per wave instruction): the activation tile
+// [128 rows][256 bytes] of a group, the raw codes of the 256 weight rows (64 or 128 bytes each) and the
+// activation-sum records (below), double-buffered, one barrier per group. 16-byte slots are XOR-swizzled
+// by row on the way in (the lane that fills a slot chooses which global chunk goes there), so the
+// 16-byte operand reads of 16 consecutive rows hit 16 different bank groups. A lane takes the activation
+// operand of a k-step from LDS (one read feeds two MFMAs), and its own column's codes once per group (32
+// or 64 bytes), which it converts in registers.
 //
 // Codes become bf16 without a conversion instruction: a nibble n = code + 8 placed in the mantissa of
 // 16.0 (bits 0x4180 | n << 3) IS the bf16 value 16 + n, two nibbles per AND-OR (int8: code + 128 through
 // v_cvt_f32_ubyte, whose upper half is the bf16 value). The matrix core therefore sums x * (code + B),
-// B = 24 or 128, and B * sum_k x is taken out again per group. That correction is a rank-one term,
-// -B * wscale[n, g] * xsum[m, g], and it too runs on the matrix core: both factors are cut into three
-// bf16 pieces and the six significant cross products fill one more k-step, accumulated straight into
-// the running total.
+// B = 24 or 128, and B * sum_k x is taken out again per group, also on the matrix core: the group's
+// accumulators start from one more k-step whose activation operand is the group's activation sum cut
+// into three bf16 pieces (24 bits) and whose weight operand is the constant -B.
 //
 // The activation is prepared once per call by act_prep_kernel: within every 16-byte chunk the eight
 // values are reordered to (0, 4, 1, 5, 2, 6, 3, 7), the order in which the AND-OR above leaves the
 // codes (a sum does not care about the order of its terms, as long as both operands agree), and the
-// per-group sums are cut into their bf16 pieces. The GEMM then moves activation tiles from global
-// memory to LDS without passing through registers (global_load_lds_dwordx4), XOR-swizzled by row so the
-// operand reads are conflict-free.
+// per-group sums are cut into their pieces (the records).
 //
 // Small N: a split of the reduction axis across workgroups, fp32 partial tiles in a workspace, added in a
 // fixed order by a second launch (the result does not depend on which workgroup finished first).
+#include <type_traits>
+
 #include "llmq_device.h"
 
 namespace {
@@ -46,13 +50,14 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kGroup = 128;
 constexpr int kBM = 128;            // activation rows per workgroup
+constexpr int kWaveM = 64;          // activation rows per wave
 constexpr int kWaveN = 64;          // weight rows (output columns) per wave
-constexpr int kWaves = 4;
-constexpr int kBN = kWaveN * kWaves;
+constexpr int kWaves = 8;           // 2 (rows) x 4 (columns)
+constexpr int kBN = kWaveN * 4;
 constexpr int kThreads = kWaves * kWave;
 constexpr int kRowBytes = kGroup * 2;          // one activation row of one group
 constexpr int kTileBytes = kBM * kRowBytes;    // 32 KB
-constexpr int kMT = kBM / 32, kNT = kWaveN / 32;
+constexpr int kMT = kWaveM / 32, kNT = kWaveN / 32;
 
 template <int BITS> constexpr float kCodeBias = BITS == 4 ? 24.0f : 128.0f;
 
@@ -122,29 +127,37 @@ __device__ __forceinline__ uint32_t and_or(uint32_t value, uint32_t mask_scalar,
   return d;
 }
 
+// Two of the four operand words of a k-step: a k-step's eight codes are one 32-bit word of int4 or two of
+// int8; operand word i pairs codes i and i + 4. `half` selects words (0, 1) or (2, 3).
 template <int BITS>
-__device__ __forceinline__ v8bf code_operand(const u32x4* raw, int step, uint32_t sixteen) {
-  uint32_t b[4];
+__device__ __forceinline__ void code_words(const u32x4* raw, int step, int half, uint32_t sixteen, uint32_t* out) {
   if constexpr (BITS == 4) {
     const u32x4 q = raw[step >> 2];
     const uint32_t w = (step & 3) == 0 ? q.x : (step & 3) == 1 ? q.y : (step & 3) == 2 ? q.z : q.w;
-    b[0] = and_or(w << 3, kNibbleMask, sixteen);  // nibbles 0 and 4
-    b[1] = and_or(w >> 1, kNibbleMask, sixteen);  // 1 and 5
-    b[2] = and_or(w >> 5, kNibbleMask, sixteen);  // 2 and 6
-    b[3] = and_or(w >> 9, kNibbleMask, sixteen);  // 3 and 7
+    if (half == 0) {
+      out[0] = and_or(w << 3, kNibbleMask, sixteen);  // nibbles 0 and 4
+      out[1] = and_or(w >> 1, kNibbleMask, sixteen);  // 1 and 5
+    } else {
+      out[0] = and_or(w >> 5, kNibbleMask, sixteen);  // 2 and 6
+      out[1] = and_or(w >> 9, kNibbleMask, sixteen);  // 3 and 7
+    }
   } else {
     const u32x4 q = raw[step >> 1];
     const uint32_t w0 = ((step & 1) ? q.z : q.x) ^ 0x80808080u;  // codes 0..3 of the step, + 128
     const uint32_t w1 = ((step & 1) ? q.w : q.y) ^ 0x80808080u;  // codes 4..7
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float lo = static_cast<float>((w0 >> (8 * i)) & 0xffu);
-      const float hi = static_cast<float>((w1 >> (8 * i)) & 0xffu);
+    for (int i = 0; i < 2; ++i) {
+      const int e = 2 * half + i;
+      const float lo = static_cast<float>((w0 >> (8 * e)) & 0xffu);
+      const float hi = static_cast<float>((w1 >> (8 * e)) & 0xffu);
       // integers below 256: the upper half of the float is the bf16 value, exactly
-      b[i] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, hi), __builtin_bit_cast(uint32_t, lo), 0x07060302u);
+      out[i] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, hi), __builtin_bit_cast(uint32_t, lo), 0x07060302u);
     }
   }
-  return __builtin_bit_cast(v8bf, u32x4{b[0], b[1], b[2], b[3]});
+}
+
+__device__ __forceinline__ v16f mfma(const u32x4& a, const u32x4& b, const v16f& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
 }
 
 template <int BITS>
@@ -163,6 +176,7 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   const int sp = logical / (a.m_tiles * a.n_tiles);
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int wm = wv & 1, wn = wv >> 1;  // the wave's half of the rows, quarter of the columns
   const int lm = lane & 31, lh = lane >> 5;
   const int m0 = mt * kBM, n0 = nt * kBN;
   const int g_begin = sp * a.groups_per_split;
@@ -170,17 +184,19 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
 
   // ---- global -> LDS: what this lane fetches for each of its wave's transfer instructions -------------
   // One instruction moves 64 x 16 bytes into 1 KB of consecutive LDS; which global chunk a lane fetches
-  // for its place there carries the swizzle.
-  // activation: instruction i of a wave = rows wv*32 + 4 i .. + 3, lane = (row, slot)
+  // for its place there carries the swizzle. The activation and its records are the kernel's own
+  // buffers, padded to whole tiles of rows, so their rows need no clamping.
+  // activation: instruction i of a wave = rows wv*16 + 4 i .. + 3, lane = (row, slot); slot p of row r
+  // holds chunk p ^ (r & 15), and r & 15 = 4 i + lane / 16
+  constexpr int kXInstr = kBM / 4 / kWaves;  // 4
   const uint32_t x_row_bytes = static_cast<uint32_t>(a.G) * kRowBytes;
-  uint32_t x_off[8];
+  uint32_t x_off[kXInstr];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = wv * 32 + i * 4 + (lane >> 4);
-    const int chunk = (lane & 15) ^ (row & 15);
-    x_off[i] = static_cast<uint32_t>(min(m0 + row, a.M - 1)) * x_row_bytes + chunk * 16;
+  for (int i = 0; i < kXInstr; ++i) {
+    const int row = wv * (kBM / kWaves) + i * 4 + (lane >> 4);
+    x_off[i] = static_cast<uint32_t>(m0 + row) * x_row_bytes + (((lane & 15) ^ (row & 15)) << 4);
   }
-  // codes: 4 (int4) or 8 (int8) instructions per wave; 16 or 8 weight rows each
+  // codes: 2 (int4) or 4 (int8) instructions per wave; 16 or 8 weight rows each
   constexpr int kCodeInstr = kCodeTileBytes<BITS> / 1024 / kWaves;
   constexpr int kRowsPerInstr = 1024 / kCodeRowBytes<BITS>;
   constexpr int kSlots = kCodeRowBytes<BITS> / 16;
@@ -193,15 +209,16 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
     w_off[i] = static_cast<uint32_t>(min(n0 + row, a.N - 1)) * w_row_bytes + chunk * 16;
   }
   // records: waves 0 and 1, 64 rows each
-  const uint32_t r_off = static_cast<uint32_t>(min(m0 + (wv & 1) * 64 + lane, a.M - 1)) * a.G * 16;
+  const uint32_t r_off = static_cast<uint32_t>(m0 + (wv & 1) * 64 + lane) * a.G * 16;
 
   auto request = [&](int g, int buf) {
     uint8_t* stage = smem + buf * kStageBytes<BITS>;
     const uint8_t* xg = a.xp + static_cast<uint32_t>(g) * kRowBytes;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kXInstr; ++i) {
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(xg + x_off[i]),
-                                       reinterpret_cast<u32x4*>(stage + (wv * 32 + i * 4) * kRowBytes), 16, 0, 0);
+                                       reinterpret_cast<u32x4*>(stage + (wv * (kBM / kWaves) + i * 4) * kRowBytes), 16,
+                                       0, 0);
     }
     const uint8_t* wg = a.qw + static_cast<uint32_t>(g) * kCodeRowBytes<BITS>;
 #pragma unroll
@@ -218,23 +235,21 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   };
 
   // ---- LDS -> operands ----------------------------------------------------------------------------------
-  // activation operand of k-step j: row mi*32 + lm, chunk 8 lh + j
-  uint32_t a_off[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) a_off[j] = lm * kRowBytes + (((8 * lh + j) ^ (lm & 15)) << 4);
-  // this lane's codes of a group: weight row wv*64 + ni*32 + lm, k in [64 lh, 64 lh + 64)
+  // activation operand of k-step j, row tile mi: row wm*64 + mi*32 + lm, chunk (8 lh + j) ^ (lm & 15)
+  const uint32_t a_base = (wm * 64 + lm) * kRowBytes + (((8 * lh) ^ (lm & 15)) << 4);  // k-step j: a_base ^ (j << 4)
+  // this lane's codes of a group: weight row wn*64 + ni*32 + lm, k in [64 lh, 64 lh + 64): 16-byte chunks
+  // lh * kRawLoads + q, at c_base ^ (q << 4)
   constexpr int kRawLoads = BITS == 4 ? 2 : 4;
-  uint32_t c_off[kNT][kRawLoads];
+  uint32_t c_base[kNT];
   const float* s_ptr[kNT];
 #pragma unroll
   for (int ni = 0; ni < kNT; ++ni) {
-    const int row = wv * kWaveN + ni * 32 + lm;
-#pragma unroll
-    for (int q = 0; q < kRawLoads; ++q)
-      c_off[ni][q] = kTileBytes + row * kCodeRowBytes<BITS> + code_slot<BITS>(row, lh * kRawLoads + q) * 16;
+    const int row = wn * kWaveN + ni * 32 + lm;
+    c_base[ni] = kTileBytes + row * kCodeRowBytes<BITS> + code_slot<BITS>(row, lh * kRawLoads) * 16;
     const int n = min(n0 + row, a.N - 1);
     s_ptr[ni] = a.sw + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * a.G;
   }
+  auto read16 = [&](const uint8_t* stage, uint32_t offset) { return *reinterpret_cast<const u32x4*>(stage + offset); };
 
   float total[kMT][kNT][16];
 #pragma unroll
@@ -245,6 +260,9 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
       for (int r = 0; r < 16; ++r) total[mi][ni][r] = 0.0f;
   uint32_t sixteen = 0x41804180u;  // bf16 16.0 twice; kept in a vector register (see and_or)
   asm volatile("" : "+v"(sixteen));
+  const uint32_t nb = bf16_bits_rne(-kCodeBias<BITS>);  // exact
+  const uint32_t nb2 = lh ? 0u : (nb | (nb << 16));
+  const u32x4 bias_operand = {nb2, nb2, 0u, 0u};
 
   request(g_begin, 0);
   float scale_next[kNT];
@@ -253,6 +271,9 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
+  // Two waves share a SIMD: while one converts codes or adds its group sums into the totals, the other
+  // keeps the matrix core busy. Within a wave the next k-step's activation operands are requested before
+  // the current step's multiplications.
   for (int g = g_begin; g < g_end; ++g) {
     const int buf = (g - g_begin) & 1;
     float scale[kNT];
@@ -265,42 +286,46 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
     }
     const uint8_t* stage = smem + buf * kStageBytes<BITS>;
 
-    u32x4 raw[kNT][kRawLoads];
+    u32x4 raw[kNT][kRawLoads], rec[kMT], fa[2][kMT];
+#pragma unroll
+    for (int mi = 0; mi < kMT; ++mi)
+      rec[mi] = read16(stage, kTileBytes + kCodeTileBytes<BITS> + (wm * 64 + mi * 32 + lm) * 16);
 #pragma unroll
     for (int ni = 0; ni < kNT; ++ni)
 #pragma unroll
-      for (int q = 0; q < kRawLoads; ++q) raw[ni][q] = *reinterpret_cast<const u32x4*>(stage + c_off[ni][q]);
+      for (int q = 0; q < kRawLoads; ++q) raw[ni][q] = read16(stage, c_base[ni] ^ (q << 4));
+#pragma unroll
+    for (int mi = 0; mi < kMT; ++mi) fa[0][mi] = read16(stage, mi * 32 * kRowBytes + a_base);
 
     // The group's sums start at -B * xsum[m] (one k-step: the three bf16 pieces of the activation sum
     // against the constant -B; the upper half of the wave, k' 8..15, multiplies zeros), then take the
     // eight k-steps of x * (code + B).
     v16f acc[kMT][kNT];
     {
-      const uint32_t nb = bf16_bits_rne(-kCodeBias<BITS>);  // exact
-      const uint32_t nb2 = lh ? 0u : (nb | (nb << 16));
-      const v8bf bv = __builtin_bit_cast(v8bf, u32x4{nb2, nb2, 0u, 0u});
       const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-      for (int mi = 0; mi < kMT; ++mi) {
-        const v8bf rec = __builtin_bit_cast(
-            v8bf, *reinterpret_cast<const u32x4*>(stage + kTileBytes + kCodeTileBytes<BITS> + (mi * 32 + lm) * 16));
+      for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < kNT; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rec, bv, zero, 0, 0, 0);
-      }
+        for (int ni = 0; ni < kNT; ++ni) acc[mi][ni] = mfma(rec[mi], bias_operand, zero);
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      v8bf fa[kMT], fb[kNT];
+      if (j < 7) {
+#pragma unroll
+        for (int mi = 0; mi < kMT; ++mi) fa[(j + 1) & 1][mi] = read16(stage, mi * 32 * kRowBytes + (a_base ^ ((j + 1) << 4)));
+      }
+      u32x4 fb[kNT];
+#pragma unroll
+      for (int ni = 0; ni < kNT; ++ni) {
+        uint32_t lo[2], hi[2];
+        code_words<BITS>(raw[ni], j, 0, sixteen, lo);
+        code_words<BITS>(raw[ni], j, 1, sixteen, hi);
+        fb[ni] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      }
 #pragma unroll
       for (int mi = 0; mi < kMT; ++mi)
-        fa[mi] = __builtin_bit_cast(v8bf, *reinterpret_cast<const u32x4*>(stage + mi * 32 * kRowBytes + a_off[j]));
 #pragma unroll
-      for (int ni = 0; ni < kNT; ++ni) fb[ni] = code_operand<BITS>(raw[ni], j, sixteen);
-#pragma unroll
-      for (int mi = 0; mi < kMT; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < kNT; ++ni)
-          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi], fb[ni], acc[mi][ni], 0, 0, 0);
+        for (int ni = 0; ni < kNT; ++ni) acc[mi][ni] = mfma(fa[j & 1][mi], fb[ni], acc[mi][ni]);
     }
 #pragma unroll
     for (int mi = 0; mi < kMT; ++mi)
@@ -319,12 +344,12 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
     bf16_t* __restrict__ out = static_cast<bf16_t*>(a.out);
 #pragma unroll
     for (int ni = 0; ni < kNT; ++ni) {
-      const int n = n0 + wv * kWaveN + ni * 32 + lm;
+      const int n = n0 + wn * kWaveN + ni * 32 + lm;
 #pragma unroll
       for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int m = m0 + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          const int m = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
           if (m < a.M && n < a.N) out[static_cast<int64_t>(m) * a.N + n] = from_float<bf16_t>(total[mi][ni][r]);
         }
     }
@@ -332,12 +357,12 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
     float* __restrict__ part = a.partial + static_cast<int64_t>(sp) * a.M * a.N;
 #pragma unroll
     for (int ni = 0; ni < kNT; ++ni) {
-      const int n = n0 + wv * kWaveN + ni * 32 + lm;
+      const int n = n0 + wn * kWaveN + ni * 32 + lm;
 #pragma unroll
       for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int m = m0 + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          const int m = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
           if (m < a.M && n < a.N) part[static_cast<int64_t>(m) * a.N + n] = total[mi][ni][r];
         }
     }
@@ -408,8 +433,9 @@ Plan plan_for(int M, int N, int G) {
   }
   p.groups_per_split = (G + splits - 1) / splits;
   p.splits = (G + p.groups_per_split - 1) / p.groups_per_split;  // every slice holds at least one group
-  p.xp_bytes = aligned(static_cast<size_t>(M) * G * kRowBytes);
-  p.rec_bytes = aligned(static_cast<size_t>(M) * G * 16);
+  // (rows padded to whole tiles: the kernel reads them without clamping; what the pad rows hold is never stored)
+  p.xp_bytes = aligned(static_cast<size_t>(p.m_tiles) * kBM * G * kRowBytes);
+  p.rec_bytes = aligned(static_cast<size_t>(p.m_tiles) * kBM * G * 16);
   p.partial_bytes = p.splits > 1 ? aligned(static_cast<size_t>(p.splits) * M * N * sizeof(float)) : 0;
   return p;
 }
@@ -437,7 +463,7 @@ extern "C" int llmq_wq_gemm_a16_tile(const void* x, const void* qweight, const f
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(qweight) | reinterpret_cast<uintptr_t>(workspace) |
        reinterpret_cast<uintptr_t>(out)) & 15u)
     return llmq_host::fail_invalid("activation, weight, output and workspace pointers must be 16-byte aligned");
-  if (static_cast<uint64_t>(M) * G * kRowBytes >= (1ull << 32))
+  if ((static_cast<uint64_t>(M) + kBM) * G * kRowBytes >= (1ull << 32))
     return llmq_host::fail_invalid("activation of %d x %d values is beyond the kernel's 32-bit offsets", M, G * kGroup);
   const Plan p = plan_for(M, N, G);
   if (workspace_bytes < p.xp_bytes + p.rec_bytes + p.partial_bytes)
