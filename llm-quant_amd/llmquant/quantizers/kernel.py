@@ -35,6 +35,19 @@ FUSED_GEMM_MIN_ROWS = 3
 FUSED_GEMM_SPLIT_GROUPS = 64
 
 
+#: Prompt-sized bf16 activations: the tiled fused GEMM (128 x 256 output tiles, no dense weight) up to this
+#: many rows, where it runs level with or ahead of dequantize + the BLAS library's matmul (measured at 128
+#: and 512 rows; at 2048 rows the library's 1.1-1.2 PFLOP/s kernels win by more than the dequantize pass costs)
+TILED_GEMM_MAX_ROWS = 1024
+
+
+def tiled_gemm_pays(rows: int, out_features: int, groups: int) -> bool:
+    """Whether the tiled fused GEMM beats dequantize + matmul for this many activation rows: wide outputs
+    (enough 128 x 256 tiles to fill the chip) or long rows (the reduction axis is split instead). Narrow,
+    short weights (q|k|v, o_proj of a 1B model) have too few tiles either way and stay with the library."""
+    return FUSED_GEMM_MAX_ROWS < rows <= TILED_GEMM_MAX_ROWS and (out_features >= 8192 or groups >= 64)
+
+
 def fused_gemm_splits(rows: int, groups: int) -> bool:
     """Which form of the fused GEMM is faster for this many activation rows and groups per weight row."""
     return rows > FUSED_GEMM_WHOLE_ROWS or groups >= FUSED_GEMM_SPLIT_GROUPS
@@ -165,7 +178,9 @@ class KernelQuantLinear(nn.Module):
         rows = x.reshape(-1, x.shape[-1])
         fused = (FUSED_GEMM_MIN_ROWS <= rows.shape[0] <= self._fused_max_rows
                  and rows.dtype in (torch.bfloat16, torch.float16) and not self._int8_act)
-        if rows.shape[0] > KERNEL_MAX_ROWS and not self._int8_act and self._head_keep and not fused:
+        tiled = (self._fused_max_rows > 0 and rows.dtype == torch.bfloat16 and not self._int8_act
+                 and tiled_gemm_pays(rows.shape[0], self.out_features, self.qdata.shape[1]))
+        if rows.shape[0] > KERNEL_MAX_ROWS and not self._int8_act and self._head_keep and not fused and not tiled:
             # dense branch on the real width: neither the activation nor the weight is padded
             out = self._dense(rows, real_width=True)
             if self.bias is not None:
@@ -183,6 +198,8 @@ class KernelQuantLinear(nn.Module):
                                         fused_gemm_splits(rows.shape[0], self.qdata.shape[1]))
         elif rows.shape[0] <= KERNEL_MAX_ROWS:
             out = self._gemv(rows, self.qdata, self.wscale, self.out_group)
+        elif tiled:
+            out = self._ext.wq_gemm_a16_tile(rows, self.qdata, self.wscale, self.out_group)
         else:
             out = self._dense(rows)
         if self.bias is not None:

@@ -129,7 +129,7 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         many rows, once for the whole concatenation (three or two matmuls and dequantize passes fewer
         per layer, and the host's matmul dispatch is the longest part of a prompt pass)."""
         from llmquant.quantizers.kernel import (FUSED_GEMM_MAX_ROWS, FUSED_GEMM_MIN_ROWS, KERNEL_MAX_ROWS,
-                                                fused_gemm_splits)
+                                                fused_gemm_splits, tiled_gemm_pays)
 
         rows = x.shape[0]
         if FUSED_GEMM_MIN_ROWS <= rows <= FUSED_GEMM_MAX_ROWS and x.dtype in (torch.bfloat16, torch.float16):
@@ -137,6 +137,8 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
                                          fused_gemm_splits(rows, fused.qdata.shape[1]))
         if rows <= KERNEL_MAX_ROWS:
             return self._ext.wq_gemv(x, fused.qdata, fused.wscale, fused.out_group)
+        if x.dtype == torch.bfloat16 and tiled_gemm_pays(rows, fused.qdata.shape[0], fused.qdata.shape[1]):
+            return self._ext.wq_gemm_a16_tile(x.contiguous(), fused.qdata, fused.wscale, fused.out_group)
         if x.dtype in (torch.bfloat16, torch.float16):
             return self._ext.wq_dense_linear(x.contiguous(), fused.qdata, fused.wscale, fused.out_group, 0)
         return x @ self._ext.dequant_weight(fused.qdata, fused.wscale, fused.out_group, 0, x.dtype).T

@@ -235,3 +235,36 @@ def test_tiled_gemm_argument_checks(ext):
     with pytest.raises(RuntimeError, match="wscale must be"):
         ext.wq_gemm_a16_tile(x.cuda(), q, s[:-1], 0)
     assert ext.wq_gemm_a16_tile(x.cuda()[:0], q, s, 0).shape == (0, 256)
+
+
+@pytest.mark.parametrize("bits,layout", [(4, {}), (8, {"out_group": 64}), (4, {"head_dim": 64})])
+def test_module_takes_the_tiled_gemm_for_a_prompt(ext, bits, layout):
+    """KernelQuantLinear on a prompt-sized bf16 batch against a wide weight: the tiled fused GEMM runs (the
+    dense branch is made to fail loudly), padded heads and head scales included, and the result is the
+    real-mode sum."""
+    import torch.nn as nn
+
+    from llmquant.core.scheme import QuantizationArgs, QuantizationScheme
+    from llmquant.quantizers import KernelQuantLinear
+    from llmquant.quantizers.kernel import tiled_gemm_pays
+
+    torch.manual_seed(21)
+    linear = nn.Linear(1024, 8192, bias=False).to(torch.bfloat16).cuda()
+    scheme = QuantizationScheme(weights=QuantizationArgs(num_bits=bits, strategy="group", group_size=GROUP, **layout),
+                                input_activations=None)
+    module = KernelQuantLinear.from_linear(linear, scheme)
+    module._dequantized_weight = module._dense = None
+    m = 200
+    assert tiled_gemm_pays(m, 8192, module.qdata.shape[1]) and not tiled_gemm_pays(2048, 8192, 8)
+    x = torch.randn(2, m // 2, 1024).to(torch.bfloat16)
+    got = module(x.cuda())
+    assert got.shape == (2, m // 2, 8192) and got.dtype == torch.bfloat16
+    canonical, scales = oracle.canonical_weight(to_np(linear.weight), bits, GROUP, layout.get("head_dim"),
+                                                layout.get("out_group"))
+    padded = oracle.pad_activation(to_np(x).reshape(m, -1), GROUP, layout.get("head_dim"))
+    rng = np.random.default_rng(5)
+    cols = np.sort(rng.choice(8192, 256, replace=False))
+    og = layout.get("out_group")
+    full_scales = np.repeat(scales, og, axis=0)[:8192] if og else scales
+    exact = oracle.gemv_float64(padded, canonical[cols], full_scales[cols])
+    assert rel_l2(to_np(got).reshape(m, -1)[:, cols], exact) <= 2e-3
