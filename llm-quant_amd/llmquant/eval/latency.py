@@ -60,8 +60,10 @@ def measure_latency(model, tokenizer=None, prompt_tokens: int = 512, new_tokens:
     }
 
 
-def latency_row(quant: QuantConfig | None, mode: str, latency: dict, eval_sec: float | None = None) -> dict:
-    """The row run_one() writes for one configuration, latency part: the recipe's axes, the
+def latency_row(quant: QuantConfig | None, mode: str, latency: dict, eval_sec: float | None = None,
+                cost: dict | None = None) -> dict:
+    """The row run_one() writes for one configuration (llmquant/eval/run.py:108-159) without the accuracy
+    columns: the recipe's axes, the cost columns when `cost` (llmquant.eval.deployed_cost) is given, the
     timings, and which path produced them (`latency_mode`). quant None = the bf16 baseline."""
     quantize = quant is not None
     q = quant or QuantConfig()
@@ -75,6 +77,10 @@ def latency_row(quant: QuantConfig | None, mode: str, latency: dict, eval_sec: f
         "kv_cache": normalize_dtype(q.kv_cache),
         "group_size": q.group_size,
     }
+    if cost is not None:
+        from llmquant.eval.cost import cost_columns
+
+        row.update(cost_columns(cost))
     row.update(latency)
     row["latency_mode"] = mode
     if eval_sec is not None:

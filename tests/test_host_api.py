@@ -362,3 +362,42 @@ def test_verification_plan_and_reconcile_follow_the_report_format():
                                    "recovered": 1.1, "costs_decode_pct": pytest.approx(100 / 11)}]
     assert reconcile([base]) == {}
     assert reconcile([base, dict(sel, decode_speedup_projected=4.0 / PROJECTION_TOLERANCE + 0.1)])["held_up"] is False
+
+
+def test_deployed_cost_of_a_bf16_model_and_the_row_columns():
+    """llmquant.eval.deployed_cost on an unquantized model: every Linear and the untied lm_head at two bytes
+    per weight, the embedding on disk but not in the per-token traffic, the KV cache per token of context
+    (llmquant/core/metrics.py:183-200: 32 KB per token at the Llama-3.2-1B geometry in bf16, 17 KB as int8
+    with one fp32 scale per token per head, 9 KB as int4); and the four columns a result row carries."""
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from llmquant.eval import cost_columns, deployed_cost, kv_cache_bytes_per_token, latency_row
+
+    cfg = LlamaConfig(hidden_size=64, intermediate_size=128, num_hidden_layers=2, num_attention_heads=4,
+                      num_key_value_heads=2, head_dim=16, vocab_size=100, tie_word_embeddings=False)
+    model = LlamaForCausalLM(cfg)
+    linears = 2 * (64 * 64 * 2 + 2 * 32 * 64 + 3 * 64 * 128) + 100 * 64   # q, o, k, v, gate, up, down; lm_head
+    norms = (2 * 2 + 1) * 64
+    cost = deployed_cost(model, None)
+    assert cost["decode_bytes_per_token"] == 2 * (linears + norms)
+    assert cost["deployed_bytes"] == 2 * (linears + norms + 100 * 64)
+    assert cost["bits_per_element"] == 16.0
+    assert cost["kv_bytes_per_token"] == 2 * 2 * 2 * 16 * 2
+
+    class Geometry:
+        config = LlamaConfig(hidden_size=2048, num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8,
+                             head_dim=64)
+
+    assert kv_cache_bytes_per_token(Geometry, None) == 32 * 1024
+    assert kv_cache_bytes_per_token(Geometry, 8) == 17 * 1024
+    assert kv_cache_bytes_per_token(Geometry, 4) == 9 * 1024
+    row = latency_row(None, "hf_static_cache_graph", {"ttft_ms": 1.0, "decode_tps": 2.0}, cost=cost)
+    assert set(cost_columns(cost)) <= set(row) and row["latency_mode"] == "hf_static_cache_graph"
+    assert list(row)[:8] == ["name", "quantize", "attn_weight", "mlp_weight", "head_weight", "activation", "kv_cache",
+                             "group_size"]
+    tied = LlamaForCausalLM(LlamaConfig(hidden_size=64, intermediate_size=128, num_hidden_layers=1,
+                                        num_attention_heads=4, num_key_value_heads=2, head_dim=16, vocab_size=100,
+                                        tie_word_embeddings=True))
+    shared = deployed_cost(tied, None)
+    per_layer = 64 * 64 * 2 + 2 * 32 * 64 + 3 * 64 * 128
+    assert shared["deployed_bytes"] == 2 * (per_layer + 3 * 64 + 100 * 64)   # the shared table once
