@@ -10,30 +10,28 @@
 // dtype and calls the BLAS library for M > 4, llmquant/quantizers/kernel.py:68-79,88-91: nine times the
 // int4 codes' bytes through HBM per call, and a second rounding per weight.)
 //
-// Shape. A workgroup of eight waves owns a 128 (m) x 256 (n) tile of the output, two waves per SIMD; a
-// wave owns 64 rows x 64 columns: 2 x 2 MFMA tiles of 32 x 32 (v_mfma_f32_32x32x16_bf16), eight k-steps
-// of 16 per group, accumulators and running totals in vector registers (128 of them, which is what lets
-// two waves share a SIMD: one converts codes or folds its group sums into the totals while the other
-// keeps the matrix core busy). Every operand reaches LDS straight from global memory, without passing
-// through registers (global_load_lds_dwordx4, 1 KB per wave instruction): the activation tile
-// [128 rows][256 bytes] of a group, the raw codes of the 256 weight rows (64 or 128 bytes each) and the
-// activation-sum records (below), double-buffered, one barrier per group. 16-byte slots are XOR-swizzled
-// by row on the way in (the lane that fills a slot chooses which global chunk goes there), so the
-// 16-byte operand reads of 16 consecutive rows hit 16 different bank groups. A lane takes the activation
-// operand of a k-step from LDS (one read feeds two MFMAs), and its own column's codes once per group (32
-// or 64 bytes), which it converts in registers.
+// Shape. A workgroup of four waves owns a 128 (m) x 256 (n) tile of the output; every wave owns 64 of
+// the 256 columns and all 128 rows: 4 x 2 MFMA tiles of 32 x 32 (v_mfma_f32_32x32x16_bf16), eight
+// k-steps of 16 per group. What bounds a tiled GEMM on this chip is LDS bandwidth (one 16-byte operand
+// read per lane per MFMA is all the LDS delivers), so only the activation goes through LDS, shared by
+// the four waves, and each operand read feeds two MFMAs; the weights never touch LDS: a lane reads the
+// codes of its own column straight from HBM in operand layout (32 bytes of int4 or 64 of int8 per group)
+// and converts them in registers.
 //
 // Codes become bf16 without a conversion instruction: a nibble n = code + 8 placed in the mantissa of
 // 16.0 (bits 0x4180 | n << 3) IS the bf16 value 16 + n, two nibbles per AND-OR (int8: code + 128 through
 // v_cvt_f32_ubyte, whose upper half is the bf16 value). The matrix core therefore sums x * (code + B),
-// B = 24 or 128, and B * sum_k x is taken out again per group, also on the matrix core: the group's
-// accumulators start from one more k-step whose activation operand is the group's activation sum cut
-// into three bf16 pieces (24 bits) and whose weight operand is the constant -B.
+// B = 24 or 128, and B * sum_k x is taken out again per group. That correction is a rank-one term,
+// -B * wscale[n, g] * xsum[m, g], and it too runs on the matrix core: both factors are cut into three
+// bf16 pieces and the six significant cross products fill one more k-step, accumulated straight into
+// the running total.
 //
 // The activation is prepared once per call by act_prep_kernel: within every 16-byte chunk the eight
 // values are reordered to (0, 4, 1, 5, 2, 6, 3, 7), the order in which the AND-OR above leaves the
 // codes (a sum does not care about the order of its terms, as long as both operands agree), and the
-// per-group sums are cut into their pieces (the records).
+// per-group sums are cut into their bf16 pieces. The GEMM then moves activation tiles from global
+// memory to LDS without passing through registers (global_load_lds_dwordx4), XOR-swizzled by row so the
+// operand reads are conflict-free.
 //
 // Small N: a split of the reduction axis across workgroups, fp32 partial tiles in a workspace, added in a
 // fixed order by a second launch (the result does not depend on which workgroup finished first).
@@ -109,8 +107,12 @@ struct TileArgs {
 template <int BITS> constexpr int kCodeRowBytes = BITS == 4 ? kGroup / 2 : kGroup;
 template <int BITS> constexpr int kCodeTileBytes = kBN * kCodeRowBytes<BITS>;
 constexpr int kRecTileBytes = kBM * 16;
-template <int BITS> constexpr int kStageBytes = kTileBytes + kCodeTileBytes<BITS> + kRecTileBytes;
-template <int BITS> constexpr int kLdsBytes = 2 * kStageBytes<BITS>;
+constexpr int kScaleTileBytes = kBN * 4;
+template <int BITS> constexpr int kStageBytes = kTileBytes + kCodeTileBytes<BITS> + kRecTileBytes + kScaleTileBytes;
+// three stages where they fit the 160 KB of LDS (int4: 153 KB): a group's transfers are requested two
+// groups before it is multiplied; int8 codes leave room for two
+template <int BITS> constexpr int kStages = BITS == 4 ? 3 : 2;
+template <int BITS> constexpr int kLdsBytes = kStages<BITS> * kStageBytes<BITS>;
 
 // slot of chunk c in weight row `row`: 16 consecutive rows read the same chunk at once and must land in
 // 16 different bank quads
@@ -208,8 +210,13 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
     const int chunk = code_slot<BITS>(row, lane % kSlots);  // the swizzle is its own inverse
     w_off[i] = static_cast<uint32_t>(min(n0 + row, a.N - 1)) * w_row_bytes + chunk * 16;
   }
-  // records: waves 0 and 1, 64 rows each
+  // records: waves 0 and 1, 64 rows each; scales: waves 2..5, 64 columns each
   const uint32_t r_off = static_cast<uint32_t>(m0 + (wv & 1) * 64 + lane) * a.G * 16;
+  const float* sw_lane;
+  {
+    const int n = min(n0 + ((wv - 2) & 3) * 64 + lane, a.N - 1);
+    sw_lane = a.sw + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * a.G;
+  }
 
   auto request = [&](int g, int buf) {
     uint8_t* stage = smem + buf * kStageBytes<BITS>;
@@ -231,8 +238,16 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(a.rec + r_off + static_cast<uint32_t>(g) * 16),
                                        reinterpret_cast<u32x4*>(stage + kTileBytes + kCodeTileBytes<BITS> + wv * 1024),
                                        16, 0, 0);
+    } else if (wv < 6) {
+      // the scales of 64 columns, one float per lane
+      __builtin_amdgcn_global_load_lds(
+          sw_lane + g, reinterpret_cast<float*>(stage + kTileBytes + kCodeTileBytes<BITS> + kRecTileBytes + (wv - 2) * 256),
+          4, 0, 0);
     }
   };
+  // transfer instructions per wave and group (a compile-time count per branch: the waits below name how many
+  // of the youngest may still be in flight)
+  constexpr int kDmaPerWave = kXInstr + kCodeInstr + 1;   // waves 0..5; waves 6, 7: one fewer
 
   // ---- LDS -> operands ----------------------------------------------------------------------------------
   // activation operand of k-step j, row tile mi: row wm*64 + mi*32 + lm, chunk (8 lh + j) ^ (lm & 15)
@@ -241,13 +256,10 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   // lh * kRawLoads + q, at c_base ^ (q << 4)
   constexpr int kRawLoads = BITS == 4 ? 2 : 4;
   uint32_t c_base[kNT];
-  const float* s_ptr[kNT];
 #pragma unroll
   for (int ni = 0; ni < kNT; ++ni) {
     const int row = wn * kWaveN + ni * 32 + lm;
     c_base[ni] = kTileBytes + row * kCodeRowBytes<BITS> + code_slot<BITS>(row, lh * kRawLoads) * 16;
-    const int n = min(n0 + row, a.N - 1);
-    s_ptr[ni] = a.sw + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * a.G;
   }
   auto read16 = [&](const uint8_t* stage, uint32_t offset) { return *reinterpret_cast<const u32x4*>(stage + offset); };
 
@@ -264,29 +276,20 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   const uint32_t nb2 = lh ? 0u : (nb | (nb << 16));
   const u32x4 bias_operand = {nb2, nb2, 0u, 0u};
 
-  request(g_begin, 0);
-  float scale_next[kNT];
+  // ---- prologue: the first groups on their way, the first one's operands in registers ---------------------
 #pragma unroll
-  for (int ni = 0; ni < kNT; ++ni) scale_next[ni] = s_ptr[ni][g_begin];
+  for (int st = 0; st < kStages<BITS>; ++st) {
+    if (g_begin + st < g_end) request(g_begin + st, st);
+  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
+  __builtin_amdgcn_s_barrier();
 
-  // Two waves share a SIMD: while one converts codes or adds its group sums into the totals, the other
-  // keeps the matrix core busy. Within a wave the next k-step's activation operands are requested before
-  // the current step's multiplications.
-  for (int g = g_begin; g < g_end; ++g) {
-    const int buf = (g - g_begin) & 1;
-    float scale[kNT];
-#pragma unroll
-    for (int ni = 0; ni < kNT; ++ni) scale[ni] = scale_next[ni];
-    if (g + 1 < g_end) {
-      request(g + 1, buf ^ 1);
-#pragma unroll
-      for (int ni = 0; ni < kNT; ++ni) scale_next[ni] = s_ptr[ni][g + 1];
-    }
-    const uint8_t* stage = smem + buf * kStageBytes<BITS>;
-
-    u32x4 raw[kNT][kRawLoads], rec[kMT], fa[2][kMT];
+  // What a lane holds of the group it is about to multiply: the records (operand of the correction
+  // step), its raw codes, its columns' scales and the activation operands of k-step 0.
+  u32x4 raw[kNT][kRawLoads], rec[kMT], fa[2][kMT];
+  float scale[kNT];
+  auto fetch_group_operands = [&](int st) {
+    const uint8_t* stage = smem + st * kStageBytes<BITS>;
 #pragma unroll
     for (int mi = 0; mi < kMT; ++mi)
       rec[mi] = read16(stage, kTileBytes + kCodeTileBytes<BITS> + (wm * 64 + mi * 32 + lm) * 16);
@@ -295,7 +298,28 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
 #pragma unroll
       for (int q = 0; q < kRawLoads; ++q) raw[ni][q] = read16(stage, c_base[ni] ^ (q << 4));
 #pragma unroll
+    for (int ni = 0; ni < kNT; ++ni)
+      scale[ni] = *reinterpret_cast<const float*>(stage + kTileBytes + kCodeTileBytes<BITS> + kRecTileBytes +
+                                                  (wn * kWaveN + ni * 32 + lm) * 4);
+#pragma unroll
     for (int mi = 0; mi < kMT; ++mi) fa[0][mi] = read16(stage, mi * 32 * kRowBytes + a_base);
+  };
+  fetch_group_operands(0);
+
+  // Two waves share a SIMD: while one converts codes or adds its group sums into the totals, the other
+  // keeps the matrix core busy. Within a wave the next k-step's activation operands are requested before
+  // the current step's multiplications. The workgroup meets once per group, before the last k-step: by
+  // then every read of the group's LDS stage has been issued and has returned (the last step's operands are
+  // in registers), so behind the barrier that stage takes the transfers of the group kStages ahead; and each
+  // wave has waited, in front of the barrier, for its own transfers of the next group (requested kStages - 1
+  // groups ago), so behind the barrier the next group's stage is complete: the last k-step runs while the
+  // next group's operands come out of it, and no wave starts a group waiting for memory or LDS.
+  int st = 0;  // the stage of group g
+  for (int g = g_begin; g < g_end; ++g) {
+    const uint8_t* stage = smem + st * kStageBytes<BITS>;
+    const int st_next = st + 1 == kStages<BITS> ? 0 : st + 1;
+    const float scale_now[kNT] = {scale[0], scale[1]};
+    static_assert(kNT == 2, "scale_now");
 
     // The group's sums start at -B * xsum[m] (one k-step: the three bf16 pieces of the activation sum
     // against the constant -B; the upper half of the wave, k' 8..15, multiplies zeros), then take the
@@ -310,10 +334,6 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      if (j < 7) {
-#pragma unroll
-        for (int mi = 0; mi < kMT; ++mi) fa[(j + 1) & 1][mi] = read16(stage, mi * 32 * kRowBytes + (a_base ^ ((j + 1) << 4)));
-      }
       u32x4 fb[kNT];
 #pragma unroll
       for (int ni = 0; ni < kNT; ++ni) {
@@ -321,6 +341,22 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
         code_words<BITS>(raw[ni], j, 0, sixteen, lo);
         code_words<BITS>(raw[ni], j, 1, sixteen, hi);
         fb[ni] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      }
+      if (j < 7) {
+#pragma unroll
+        for (int mi = 0; mi < kMT; ++mi) fa[(j + 1) & 1][mi] = read16(stage, mi * 32 * kRowBytes + (a_base ^ ((j + 1) << 4)));
+      } else {
+        // own transfers of the next group have landed (the youngest kStages - 2 batches may stay in flight)
+        if (kStages<BITS> == 3 && g + 2 < g_end) {  // (the batch of group g + 2 exists and is younger)
+          if (wv < 6) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDmaPerWave) : "memory");
+          else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDmaPerWave - 1) : "memory");
+        } else {
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        if (g + kStages<BITS> < g_end) request(g + kStages<BITS>, st);
+        if (g + 1 < g_end) fetch_group_operands(st_next);  // (fa[0]: step 7 multiplies out of fa[1])
       }
 #pragma unroll
       for (int mi = 0; mi < kMT; ++mi)
@@ -332,11 +368,8 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
 #pragma unroll
       for (int ni = 0; ni < kNT; ++ni)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) total[mi][ni][r] = fmaf(scale[ni], acc[mi][ni][r], total[mi][ni][r]);
-
-    // the next group has landed in the other buffer, and nobody reads this one any more
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+        for (int r = 0; r < 16; ++r) total[mi][ni][r] = fmaf(scale_now[ni], acc[mi][ni][r], total[mi][ni][r]);
+    st = st_next;
   }
 
   // ---- store: register r of a 32 x 32 tile is row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
