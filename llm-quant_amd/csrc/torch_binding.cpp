@@ -498,9 +498,14 @@ at::Tensor wq_gemv_gate_up_silu(const at::Tensor& x, const at::Tensor& qweight, 
 
 // Integer GEMM: a int8 [M, K], sx fp32 [M, G]; qweight / wscale as for wq_gemv; optional fp32 or
 // half-width bias (converted to fp32 here, as RealQuantLinear adds bias.float()).
+// exact = true: RealQuantLinear's fp32 roundings and group order, bit for bit. exact = false: the same integer
+// group sums folded in with one multiply-add fewer per output and group, the reduction axis split across
+// workgroups where the output has few tiles: agrees to fp32 rounding. sx is [M, groups], or [M, 1] for one scale
+// per token (the exact form multiplies by the broadcast scale group by group; the fast form takes the scale
+// out of the sum over groups).
 at::Tensor wq_gemm_a8(const at::Tensor& a, const at::Tensor& sx, const at::Tensor& qweight,
                       const at::Tensor& wscale, const c10::optional<at::Tensor>& bias, int64_t out_group,
-                      at::ScalarType out_dtype) {
+                      at::ScalarType out_dtype, bool exact) {
   TORCH_CHECK(a.is_cuda() && sx.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "all tensors must be CUDA");
   TORCH_CHECK(a.scalar_type() == at::kChar && a.dim() == 2, "a must be int8 [M, K]");
   TORCH_CHECK(sx.scalar_type() == at::kFloat && sx.dim() == 2, "sx must be float32 [M, groups]");
@@ -509,7 +514,7 @@ at::Tensor wq_gemm_a8(const at::Tensor& a, const at::Tensor& sx, const at::Tenso
   TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
   TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 2, "wscale must be float32 [scale_rows, groups]");
   const auto ac = a.contiguous();
-  const auto sxc = sx.contiguous();
+  auto sxc = sx.contiguous();
   const auto wc = qweight.contiguous();
   const auto sc = wscale.contiguous();
   const int64_t M = ac.size(0), N = wc.size(0), groups = wc.size(1);
@@ -517,7 +522,10 @@ at::Tensor wq_gemm_a8(const at::Tensor& a, const at::Tensor& sx, const at::Tenso
   TORCH_CHECK(group_size == 128, "the integer GEMM needs group_size 128, got ", group_size);
   TORCH_CHECK(ac.size(1) == groups * group_size, "a last dim ", ac.size(1), " does not match qweight ",
               groups, "x", group_size);
-  TORCH_CHECK(sxc.size(0) == M && sxc.size(1) == groups, "sx must be [", M, ", ", groups, "]");
+  TORCH_CHECK(sxc.size(0) == M && (sxc.size(1) == groups || sxc.size(1) == 1), "sx must be [", M, ", ", groups,
+              "] or [", M, ", 1]");
+  const int64_t sx_groups = sxc.size(1);
+  if (exact && sx_groups != groups) sxc = sxc.expand({M, groups}).contiguous();
   const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
   TORCH_CHECK(sc.size(0) == scale_rows && sc.size(1) == groups, "wscale must be [", scale_rows, ", ", groups, "]");
   at::Tensor bias_f;
@@ -529,6 +537,18 @@ at::Tensor wq_gemm_a8(const at::Tensor& a, const at::Tensor& sx, const at::Tenso
   const int dtype = dtype_code(out, "output dtype");
   if (M == 0 || N == 0) return out;
   const c10::OptionalDeviceGuard guard(at::device_of(ac));
+  if (!exact) {
+    const size_t need = llmq_wq_gemm_a8_fast_workspace_bytes(static_cast<int>(M), static_cast<int>(N), static_cast<int>(groups));
+    auto workspace = at::empty({static_cast<int64_t>((need + 3) / 4)}, ac.options().dtype(at::kFloat));
+    check_rc(llmq_wq_gemm_a8_fast(ac.const_data_ptr<int8_t>(), sxc.const_data_ptr<float>(), wc.const_data_ptr(),
+                                  sc.const_data_ptr<float>(), bias_f.defined() ? bias_f.const_data_ptr<float>() : nullptr,
+                                  out.mutable_data_ptr(), workspace.mutable_data_ptr(), need, static_cast<int>(M),
+                                  static_cast<int>(N), static_cast<int>(groups), static_cast<int>(sx_groups),
+                                  static_cast<int>(group_size), static_cast<int>(out_group),
+                                  packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype, current_stream(ac)),
+             "wq_gemm_a8 (fast form)");
+    return out;
+  }
   check_rc(llmq_wq_gemm_a8(ac.const_data_ptr<int8_t>(), sxc.const_data_ptr<float>(), wc.const_data_ptr(),
                            sc.const_data_ptr<float>(), bias_f.defined() ? bias_f.const_data_ptr<float>() : nullptr,
                            out.mutable_data_ptr(), static_cast<int>(M), static_cast<int>(N),
@@ -1064,7 +1084,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("wq_gemm_a8", &wq_gemm_a8,
         "Integer GEMM: int8 activations x int4/int8 group-quantized weights, real-mode rounding order",
         py::arg("a"), py::arg("sx"), py::arg("qweight"), py::arg("wscale"), py::arg("bias") = py::none(),
-        py::arg("out_group") = 0, py::arg("out_dtype") = at::kBFloat16);
+        py::arg("out_group") = 0, py::arg("out_dtype") = at::kBFloat16, py::arg("exact") = true);
   m.def("wq_gemm_a16", &wq_gemm_a16,
         "Weight-only GEMM for a few dozen rows: fp16/bf16 activations x int4/int8 group-quantized weights, no dense copy",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("split") = false);

@@ -113,6 +113,10 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_argmax_advance.restype = c_int
     lib.llmq_wq_gemm_a8.argtypes = [c_p] * 6 + [c_int] * 7 + [c_p]
     lib.llmq_wq_gemm_a8.restype = c_int
+    lib.llmq_wq_gemm_a8_fast.argtypes = [c_p] * 7 + [ctypes.c_size_t] + [c_int] * 8 + [c_p]
+    lib.llmq_wq_gemm_a8_fast.restype = c_int
+    lib.llmq_wq_gemm_a8_fast_workspace_bytes.argtypes = [c_int] * 3
+    lib.llmq_wq_gemm_a8_fast_workspace_bytes.restype = ctypes.c_size_t
     lib.llmq_wq_gemm_a16.argtypes = [c_p] * 4 + [c_int] * 7 + [c_p]
     lib.llmq_wq_gemm_a16.restype = c_int
     lib.llmq_wq_gemm_a16_split.argtypes = [c_p] * 5 + [ctypes.c_size_t] + [c_int] * 7 + [c_p]

@@ -179,7 +179,97 @@ def test_one_activation_scale_per_token(ext, n, k, m):
         got = ext.wq_gemm_a8(codes, sx_groups, q, s, None, 0, dtype)
         assert got.shape == (m, n) and got.dtype == dtype
         assert rel_l2(to_np(got)[np.ix_(rows, cols)], exact) <= tol
+        # the fast form with the scale as [M, 1]: out of the sum over groups, applied once at the store
+        fast = ext.wq_gemm_a8(codes, sx, q, s, None, 0, dtype, False)
+        assert rel_l2(to_np(fast)[np.ix_(rows, cols)], exact) <= tol
+        assert rel_l2(to_np(fast), to_np(got)) <= (1e-6 if dtype == torch.float32 else 4e-3)
+        # (and the exact form takes [M, 1] too, broadcasting it itself)
+        assert torch.equal(ext.wq_gemm_a8(codes, sx, q, s, None, 0, dtype), got)
     # against the unquantized product: what per-token int8 activations + int4 weights cost in accuracy
     dense = to_np(x)[rows].astype(np.float64) @ to_np(w)[cols].astype(np.float64).T
     print(f"per-token A8 x W4 vs bf16 product, M={m} N={n} K={k}: rel-L2 "
           f"{rel_l2(to_np(got)[np.ix_(rows, cols)], dense):.4f}")
+
+
+# ---- the fast form: same integer sums, one rounding fewer per group, split reduction axis -------------------
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(128, 256, 128), (130, 300, 768), (1, 16, 128), (65, 257, 1152), (512, 512, 2048),
+                                   (256, 1024, 8192)])
+def test_fast_form_agrees_with_real_mode_to_fp32_rounding(ext, bits, dtype, m, n, k):
+    """wq_gemm_a8(exact=False) against the oracle's real-mode forward and the float64 closed form: full and
+    ragged tiles, one group, rows long enough that the reduction axis is split across workgroups."""
+    torch.manual_seed(m + n)
+    w = (torch.randn(n, k) * 0.015).to(torch.bfloat16)
+    x = torch.randn(m, k)
+    x[:, torch.randperm(k)[: max(k // 100, 1)]] *= 20
+    x = x.to(torch.bfloat16)
+    canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP)
+    q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
+    s = torch.from_numpy(scales).cuda()
+    codes, sx = ext.quant_group_codes(x.cuda(), 8, GROUP, False)
+    got = ext.wq_gemm_a8(codes, sx, q, s, None, 0, dtype, False)
+    assert got.shape == (m, n) and got.dtype == dtype
+    a, sxo = oracle.quant_group_codes(to_np(x), 8, GROUP)
+    xq = (a.reshape(m, -1, GROUP).astype(np.float64) * sxo[..., None].astype(np.float64)).reshape(m, -1)
+    exact = oracle.gemv_float64(xq, canonical, scales)
+    assert rel_l2(to_np(got), exact) <= (1e-6 if dtype == torch.float32 else 4e-3)
+    real = oracle.real_linear(to_np(x), canonical, scales, tag_of(dtype), None, 8)
+    if dtype == torch.float32:
+        assert rel_l2(to_np(got), real) <= 1e-6
+    else:
+        assert (to_np(got) == real).mean() > 0.99
+    # and against the bit-exact kernel on the same operands
+    slow = ext.wq_gemm_a8(codes, sx, q, s, None, 0, dtype, True)
+    assert rel_l2(to_np(got), to_np(slow)) <= (1e-6 if dtype == torch.float32 else 4e-3)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_fast_form_bias_head_scales_and_split(ext, bits):
+    torch.manual_seed(3)
+    m, n, k = 70, 192, 2048   # one tile: the reduction axis is split, the bias is added by the second launch
+    w = (torch.randn(n, k) * 0.015).to(torch.bfloat16)
+    x = torch.randn(m, k).to(torch.bfloat16)
+    b = torch.randn(n)
+    canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP, None, 64)
+    q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
+    codes, sx = ext.quant_group_codes(x.cuda(), 8, GROUP, False)
+    got = ext.wq_gemm_a8(codes, sx, q, torch.from_numpy(scales).cuda(), b.cuda(), 64, torch.float32, False)
+    want = oracle.real_linear(to_np(x), canonical, scales, "f32", 64, 8, to_np(b))
+    assert rel_l2(to_np(got), want) <= 1e-6
+    one = ext.wq_gemm_a8(codes[:, :512].contiguous(), sx[:, :4].contiguous(), q[:, :4].contiguous(),
+                         torch.from_numpy(scales[:, :4].copy()).cuda(), b.cuda(), 64, torch.float32, False)
+    want_one = oracle.real_linear(to_np(x)[:, :512], canonical[:, :4], scales[:, :4], "f32", 64, 8, to_np(b))
+    assert rel_l2(to_np(one), want_one) <= 1e-6   # four groups: one slice, the bias added in the kernel
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("m", [128, 2048])
+def test_fast_form_at_llama_8b_mlp_shapes(ext, n, k, m):
+    got, (x, canonical, scales, _) = run_case(ext, m, n, k, 4, torch.bfloat16, seed=3, outliers=True)
+    codes, sx = ext.quant_group_codes(x.cuda(), 8, GROUP, False)
+    q = torch.from_numpy(oracle.pack_int4(canonical)).cuda()
+    fast = ext.wq_gemm_a8(codes, sx, q, torch.from_numpy(scales).cuda(), None, 0, torch.bfloat16, False)
+    same = (fast == got).float().mean().item()
+    assert same > 0.99 and rel_l2(to_np(fast), to_np(got)) <= 2e-3   # got: the bit-exact kernel
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_fast_form_one_scale_per_token_small_and_split(ext, bits):
+    """One activation scale per token through the fast form on ragged tiles, with a bias, and on a shape whose
+    reduction axis is split (the token's scale is applied to each partial tile)."""
+    for m, n, k in ((70, 192, 2048), (130, 300, 768), (3, 40, 128)):
+        torch.manual_seed(k)
+        w = (torch.randn(n, k) * 0.015).to(torch.bfloat16)
+        x = torch.randn(m, k).to(torch.bfloat16)
+        b = torch.randn(n)
+        canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP)
+        q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
+        codes, sx = ext.quant_group_codes(x.cuda(), 8, k, False)
+        want_codes, want_sx = oracle.quant_group_codes(to_np(x), 8, k)
+        got = ext.wq_gemm_a8(codes, sx, q, torch.from_numpy(scales).cuda(), b.cuda(), 0, torch.float32, False)
+        wq = (canonical.astype(np.float64) * scales.astype(np.float64)[:, :, None]).reshape(n, -1)
+        exact = (want_codes.astype(np.float64) @ wq.T) * want_sx.astype(np.float64) + to_np(b).astype(np.float64)
+        assert rel_l2(to_np(got), exact) <= 1e-6
