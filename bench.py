@@ -480,14 +480,23 @@ def other_kernels(torch):
                 turn[0] += 1
                 return ext.wq_gemm_a8(a, sx, q4s[turn[0] % copies], sw, None, 0, torch.bfloat16, False)
 
+            sx_token = sx[:, :1].contiguous()   # (timing only: what one scale per token costs to apply)
+
+            def fast_token():
+                turn[0] += 1
+                return ext.wq_gemm_a8(a, sx_token, q4s[turn[0] % copies], sw, None, 0, torch.bfloat16, False)
+
             us = _event_time_us(torch, one, reps=2 * copies)
             us_f = _event_time_us(torch, fast, reps=2 * copies)
+            us_t = _event_time_us(torch, fast_token, reps=2 * copies)
             us_q = _event_time_us(torch, lambda: ext.quant_group_codes(x, 8, GROUP, False), reps=10)
             gemm.append({"M": m, "N": n, "K": k, "weights": "int4", "gemm_us": round(us, 1),
                          "act_quant_us": round(us_q, 1), "TOPS": round(2 * m * n * k / us / 1e6, 1),
                          "frac_int8_mfma_peak": round(2 * m * n * k / us / 1e6 / 5000.0, 4),
                          "fast_form_us": round(us_f, 1), "fast_form_TOPS": round(2 * m * n * k / us_f / 1e6, 1),
                          "fast_form_frac_int8_mfma_peak": round(2 * m * n * k / us_f / 1e6 / 5000.0, 4),
+                         "fast_form_one_scale_per_token_us": round(us_t, 1),
+                         "fast_form_one_scale_per_token_TOPS": round(2 * m * n * k / us_t / 1e6, 1),
                          "weights_rotated_over_bytes": copies * (n * k // 2)})
         del q4s
     out["w4a8_gemm"] = gemm

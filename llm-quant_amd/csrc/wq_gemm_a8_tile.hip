@@ -12,21 +12,29 @@
 //
 // Shape: that of the tiled bf16 GEMM (wq_gemm_a16_tile.hip). A workgroup of eight waves, two per SIMD, owns a
 // 128 (m) x 256 (n) output tile; a wave owns 64 x 64: 2 x 2 tiles of v_mfma_i32_32x32x32_i8, four k-steps of
-// 32 per group, int32 group sums and fp32 totals in vector registers. All operands reach LDS straight from
-// global memory (global_load_lds, 1 KB per wave instruction; 16-byte slots XOR-swizzled by row so that the
-// operand reads of 16 consecutive rows are conflict-free), three or four stages deep: the activation tile
-// [128 rows][128 bytes], the raw codes of the 256 weight rows, the 128 activation scales and the 256 weight
-// scales of the group. A lane reads the activation operand of a k-step from LDS (one read feeds two MFMAs)
-// and its own column's codes once per group. int4 is unpacked in registers as the stored nibbles n = code + 8
-// (one AND for the even codes of a word, a shift and an AND for the odd ones), and the 8 is taken back out by
-// starting each group's sum at -8 * (sum of the group's activations) instead of zero: the preparation pass
-// writes that number per token and group, and it reaches the matrix core as the C operand of the first
-// k-step. Unpacking leaves the even codes of a 32-bit word in one operand register and the odd ones in the
-// next, so the activation is prepared once per call (act_prep_i8_kernel) with the bytes of every 8 in the same
-// order: a sum does not care about the order of its terms as long as both operands agree.
+// 32 per group, int32 group sums and fp32 totals in vector registers. (For a single tile of rows and a wide
+// weight a workgroup owns 128 x 64 instead, a wave 32 x 32: four times the workgroups, no split.) All operands
+// reach LDS straight from global memory (global_load_lds, 1 KB per wave instruction; 16-byte slots
+// XOR-swizzled by row so that the operand reads of 16 consecutive rows are conflict-free), three or four
+// stages deep: the activation tile [128 rows][128 bytes], the raw codes of the weight rows, the 128 activation
+// scales and the weight scales of the group. A lane reads the activation operand of a k-step from LDS (one
+// read feeds two MFMAs) and its own column's codes once per group. int4 is unpacked in registers as the
+// stored nibbles n = code + 8 (one AND for the even codes of a word, a shift and an AND for the odd ones), and
+// the 8 is taken back out by starting each group's sum at -8 * (sum of the group's activations) instead of
+// zero: the preparation pass writes that number per token and group, and it reaches the matrix core as the C
+// operand of the first k-step. Unpacking leaves the even codes of a 32-bit word in one operand register and
+// the odd ones in the next, so the activation is prepared once per call (act_prep_i8_kernel) with the bytes
+// of every 8 in the same order: a sum does not care about the order of its terms as long as both operands
+// agree.
 //
-// The kernel is bound by vector-ALU issue, not by the matrix core: folding a group's 64 x 64 sums into the
-// totals is 3 instructions per output (convert, two scales) = 12 per MFMA, against the MFMA's 8 issue slots.
+// What bounds the kernel is the vector ALU's issue port, which the matrix core shares: measured on this GPU,
+// a SIMD that issues one 32x32x32 int8 MFMA and v other vector instructions per wave takes about
+// 16 + 4 v cycles per MFMA (the MFMA holds the port for half of its 32 cycles; only the other half is free for
+// other waves' instructions). Folding a group's 64 x 64 sums into the totals is 3 instructions per output
+// (convert, two scales) = 12 per MFMA, 8 with one activation scale per token, and unpacking int4 is 3 more:
+// 60-70 issue cycles per MFMA against the MFMA's own 32, so the matrix core cannot be more than about half
+// busy whatever the schedule (interleaving the fold under the MFMAs by hand, a fifth k-step for the -8
+// instead of the C operand, DPP-broadcast scales and deeper LDS prefetch all measured the same or slower).
 //
 // Small N: the reduction axis is split across workgroups, fp32 partial tiles in a workspace, added in a fixed
 // order (and the bias after them) by a second launch.
@@ -40,19 +48,36 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kGroup = 128;
-constexpr int kBM = 128, kBN = 256;
+constexpr int kBM = 128;
 constexpr int kWaves = 8, kThreads = kWaves * kWave;
-constexpr int kWaveM = 64, kWaveN = 64;
-constexpr int kMT = kWaveM / 32, kNT = kWaveN / 32;
 constexpr int kARowBytes = kGroup;                // int8 activation row of one group
 constexpr int kATileBytes = kBM * kARowBytes;     // 16 KB
 template <int BITS> constexpr int kCodeRowBytes = BITS == 4 ? kGroup / 2 : kGroup;
-template <int BITS> constexpr int kCodeTileBytes = kBN * kCodeRowBytes<BITS>;
-constexpr int kSxTileBytes = kBM * 4, kSwTileBytes = kBN * 4, kStartTileBytes = kBM * 4;
-template <int BITS>
-constexpr int kStageBytes = kATileBytes + kCodeTileBytes<BITS> + kSxTileBytes + kSwTileBytes + kStartTileBytes;
-template <int BITS> constexpr int kStages = BITS == 4 ? 4 : 3;   // 136 KB / 150 KB of the 160 KB
-template <int BITS> constexpr int kLdsBytes = kStages<BITS> * kStageBytes<BITS>;
+constexpr int kSxTileBytes = kBM * 4, kStartTileBytes = kBM * 4;
+
+// The shape of a workgroup's tile: 128 rows by BN columns, eight waves as WM x WN, a wave owning MT x NT MFMA
+// tiles of 32 x 32. Wide (MT = NT = 2: 2 x 4 waves of 64 x 64, BN = 256) is the throughput shape: every operand
+// read from LDS feeds two MFMAs. Narrow (MT = NT = 1: 4 x 2 waves of 32 x 32, BN = 64) gives four times as many
+// workgroups, for activations of a tile or two of rows, where the wide shape would leave most of the chip idle
+// or split the reduction axis many ways.
+template <int BITS, int MT, int NT>
+struct Shape {
+  static constexpr int kWM = kBM / (32 * MT), kWN = kWaves / kWM;
+  static constexpr int kWaveM = 32 * MT, kWaveN = 32 * NT;
+  static constexpr int kBN = kWN * kWaveN;
+  static constexpr int kCodeTileBytes = kBN * kCodeRowBytes<BITS>;
+  static constexpr int kSwTileBytes = kBN * 4;
+  static constexpr int kScalesAt = kATileBytes + kCodeTileBytes;
+  static constexpr int kStageBytes = kScalesAt + kSxTileBytes + kSwTileBytes + kStartTileBytes;
+  static constexpr int kStages = kStageBytes * 4 <= 160 * 1024 ? 4 : 3;
+  static constexpr int kLdsBytes = kStages * kStageBytes;
+  // transfers of 64 lanes each that fill one stage: 1 KB of activations or codes, or 64 four-byte values
+  static constexpr int kAUnits = kATileBytes / 1024, kCodeUnits = kCodeTileBytes / 1024;
+  static constexpr int kSxUnits = kBM / 64, kSwUnits = kBN / 64, kStartUnits = BITS == 4 ? kBM / 64 : 0;
+  static constexpr int kUnits = kAUnits + kCodeUnits + kSxUnits + kSwUnits + kStartUnits;
+  static constexpr int kDmaPerWave = (kUnits + kWaves - 1) / kWaves;
+  static_assert(kBM % kWaveM == 0 && kWM * kWN == kWaves && kBN % 64 == 0 && kCodeTileBytes % 1024 == 0, "tile shape");
+};
 
 // ---- activation preparation: rows padded to whole tiles, bytes in operand order -------------------------
 // One lane per 16-byte chunk, eight lanes per group. For int4 weights the bytes of each 8 become
@@ -117,8 +142,12 @@ __device__ __forceinline__ v4i code_operand(const u32x4* raw, int step) {
 // TOKEN: one activation scale per token (sx[M]) instead of one per token and group (sx[M, G]): the scale leaves
 // the sum over groups, a group's sums are folded in with two instructions per output instead of three, and
 // the token's scale is applied once, at the store.
-template <typename T, int BITS, bool TOKEN>
+template <typename T, int BITS, bool TOKEN, int MT, int NT>
 __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Args a) {
+  using S = Shape<BITS, MT, NT>;
+  constexpr int kMT = MT, kNT = NT, kBN = S::kBN, kWaveM = S::kWaveM, kWaveN = S::kWaveN;
+  constexpr int kScalesAt = S::kScalesAt, kSwTileBytes = S::kSwTileBytes, kStageBytes = S::kStageBytes;
+  constexpr int kStages = S::kStages, kDmaPerWave = S::kDmaPerWave;
   extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
 
   // consecutive logical tiles (the m-tiles of one n-tile first) on one XCD: the codes come out of its L2
@@ -130,73 +159,92 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
   const int nt = (logical / a.m_tiles) % a.n_tiles;
   const int sp = logical / (a.m_tiles * a.n_tiles);
 
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  const int wm = wv & 1, wn = wv >> 1;
+  const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wv % S::kWM, wn = wv / S::kWM;
   const int lm = lane & 31, lh = lane >> 5;
   const int m0 = mt * kBM, n0 = nt * kBN;
   const int g_begin = sp * a.groups_per_split;
   const int g_end = min(g_begin + a.groups_per_split, a.G);
 
   // ---- global -> LDS ----------------------------------------------------------------------------------------
-  // activation: 2 instructions per wave, 8 rows each; lane = (row, slot), slot p of row r holds chunk
-  // p ^ ((r >> 1) & 7)
-  constexpr int kAInstr = kATileBytes / 1024 / kWaves;  // 2
-  const uint32_t a_row_bytes = static_cast<uint32_t>(a.G) * kARowBytes;
-  uint32_t a_off[kAInstr];
-#pragma unroll
-  for (int i = 0; i < kAInstr; ++i) {
-    const int row = (wv * kAInstr + i) * 8 + (lane >> 3);
-    a_off[i] = static_cast<uint32_t>(m0 + row) * a_row_bytes + (((lane & 7) ^ ((row >> 1) & 7)) << 4);
-  }
-  constexpr int kCodeInstr = kCodeTileBytes<BITS> / 1024 / kWaves;  // 2 or 4
-  constexpr int kRowsPerInstr = 1024 / kCodeRowBytes<BITS>;
+  // A stage is filled by S::kUnits transfers of 64 lanes: 16 of activations (8 rows each; lane = (row, slot),
+  // slot p of row r holds chunk p ^ ((r >> 1) & 7)), the codes (1 KB each, slots swizzled by code_slot), the
+  // activation scales of 64 rows, the weight scales of 64 columns and (int4) the group starts of 64 rows, four
+  // bytes a lane. Every wave issues kDmaPerWave of them per group, wave w the units w * kDmaPerWave + 0, 1, ...
+  // (modulo the count: a few units are transferred twice, with the same bytes, so that every wave has the same
+  // number in flight and one vmcnt serves all).
+  constexpr int kRowsPerUnit = 1024 / kCodeRowBytes<BITS>;
   constexpr int kSlots = kCodeRowBytes<BITS> / 16;
-  const uint32_t w_row_bytes = static_cast<uint32_t>(a.G) * kCodeRowBytes<BITS>;
-  uint32_t w_off[kCodeInstr];
-#pragma unroll
-  for (int i = 0; i < kCodeInstr; ++i) {
-    const int row = (wv * kCodeInstr + i) * kRowsPerInstr + lane / kSlots;
-    w_off[i] = static_cast<uint32_t>(min(n0 + row, a.N - 1)) * w_row_bytes + (code_slot<BITS>(row, lane % kSlots) << 4);
-  }
-  // scales, one 4-byte value per lane: waves 0, 1 the activation's (64 rows each), waves 2..5 the weight's
-  // (64 columns each), waves 6, 7 the rows' group starts (int4; for int8 they repeat the activation scales)
-  const float* s_lane;
-  int s_at, s_step = 1;
-  constexpr int kScalesAt = kATileBytes + kCodeTileBytes<BITS>;
-  if (wv < 2 || wv >= 6) {
-    const int row = min(m0 + (wv & 1) * 64 + lane, a.M - 1);
-    const bool starts = BITS == 4 && wv >= 6;
-    if (starts) {
-      s_lane = reinterpret_cast<const float*>(a.start) + static_cast<int64_t>(row) * a.G;
-    } else if (TOKEN) {
-      s_lane = a.sx + row, s_step = 0;   // (the tile is not read: the transfer keeps every wave's count the same)
+  const uint8_t* dma_base[kDmaPerWave];
+  uint32_t dma_off[kDmaPerWave], dma_step[kDmaPerWave], dma_dst[kDmaPerWave];
+  bool dma_wide[kDmaPerWave];
+  // unit u of the activation tile / the code tile / the 64-value vectors, as this lane's part of a transfer
+  auto a_unit = [&](int i, int u) {
+    const int row = u * 8 + (lane >> 3);
+    dma_base[i] = a.ap, dma_step[i] = kARowBytes, dma_dst[i] = u * 1024, dma_wide[i] = true;
+    dma_off[i] = static_cast<uint32_t>(m0 + row) * (static_cast<uint32_t>(a.G) * kARowBytes) +
+                 (((lane & 7) ^ ((row >> 1) & 7)) << 4);
+  };
+  auto code_unit = [&](int i, int u) {
+    const int row = u * kRowsPerUnit + lane / kSlots;
+    dma_base[i] = a.qw, dma_step[i] = kCodeRowBytes<BITS>, dma_dst[i] = kATileBytes + u * 1024, dma_wide[i] = true;
+    dma_off[i] = static_cast<uint32_t>(min(n0 + row, a.N - 1)) * (static_cast<uint32_t>(a.G) * kCodeRowBytes<BITS>) +
+                 (code_slot<BITS>(row, lane % kSlots) << 4);
+  };
+  auto vector_unit = [&](int i, int u) {   // u counts through the activation scales, the weight scales, the starts
+    dma_wide[i] = false, dma_step[i] = 4;
+    if (u < S::kSxUnits) {
+      const uint32_t row = static_cast<uint32_t>(min(m0 + u * 64 + lane, a.M - 1));
+      dma_base[i] = reinterpret_cast<const uint8_t*>(a.sx), dma_dst[i] = kScalesAt + u * 256;
+      // (TOKEN: the tile is not read; the transfer keeps every wave's count of requests in flight the same)
+      dma_off[i] = TOKEN ? row * 4 : row * static_cast<uint32_t>(a.G) * 4;
+      if (TOKEN) dma_step[i] = 0;
+    } else if (u < S::kSxUnits + S::kSwUnits) {
+      u -= S::kSxUnits;
+      const int n = min(n0 + u * 64 + lane, a.N - 1);
+      dma_base[i] = reinterpret_cast<const uint8_t*>(a.sw), dma_dst[i] = kScalesAt + kSxTileBytes + u * 256;
+      dma_off[i] = static_cast<uint32_t>(a.out_group > 0 ? n / a.out_group : n) * static_cast<uint32_t>(a.G) * 4;
     } else {
-      s_lane = a.sx + static_cast<int64_t>(row) * a.G;
+      u -= S::kSxUnits + S::kSwUnits;
+      const uint32_t row = static_cast<uint32_t>(min(m0 + u * 64 + lane, a.M - 1));
+      dma_base[i] = reinterpret_cast<const uint8_t*>(a.start);
+      dma_dst[i] = kScalesAt + kSxTileBytes + kSwTileBytes + u * 256;
+      dma_off[i] = row * static_cast<uint32_t>(a.G) * 4;
     }
-    s_at = kScalesAt + (starts ? kSxTileBytes + kSwTileBytes : 0) + (wv & 1) * 256;
+  };
+  constexpr int kVectorUnits = S::kSxUnits + S::kSwUnits + S::kStartUnits;
+  if constexpr (S::kAUnits % kWaves == 0 && S::kCodeUnits % kWaves == 0 && kVectorUnits <= kWaves) {
+    // every wave the same kinds in the same slots: the transfer widths are compile-time facts
+    constexpr int kA = S::kAUnits / kWaves, kC = S::kCodeUnits / kWaves;
+    static_assert(kDmaPerWave == kA + kC + 1, "slots");
+#pragma unroll
+    for (int i = 0; i < kA; ++i) a_unit(i, wv * kA + i);
+#pragma unroll
+    for (int i = 0; i < kC; ++i) code_unit(kA + i, wv * kC + i);
+    vector_unit(kA + kC, wv % kVectorUnits);
   } else {
-    const int n = min(n0 + (wv - 2) * 64 + lane, a.N - 1);
-    s_lane = a.sw + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * a.G;
-    s_at = kScalesAt + kSxTileBytes + (wv - 2) * 256;
+#pragma unroll
+    for (int i = 0; i < kDmaPerWave; ++i) {
+      const int u = (wv * kDmaPerWave + i) % S::kUnits;
+      if (u < S::kAUnits) a_unit(i, u);
+      else if (u < S::kAUnits + S::kCodeUnits) code_unit(i, u - S::kAUnits);
+      else vector_unit(i, u - S::kAUnits - S::kCodeUnits);
+    }
   }
-  constexpr int kDmaPerWave = kAInstr + kCodeInstr + 1;
 
   auto request = [&](int g, int st) {
-    uint8_t* stage = smem + st * kStageBytes<BITS>;
-    const uint8_t* ag = a.ap + static_cast<uint32_t>(g) * kARowBytes;
+    uint8_t* stage = smem + st * kStageBytes;
 #pragma unroll
-    for (int i = 0; i < kAInstr; ++i) {
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(ag + a_off[i]),
-                                       reinterpret_cast<u32x4*>(stage + (wv * kAInstr + i) * 1024), 16, 0, 0);
+    for (int i = 0; i < kDmaPerWave; ++i) {
+      const uint8_t* from = dma_base[i] + dma_off[i] + static_cast<uint32_t>(g) * dma_step[i];
+      if (dma_wide[i]) {
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(from), reinterpret_cast<u32x4*>(stage + dma_dst[i]),
+                                         16, 0, 0);
+      } else {
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const float*>(from), reinterpret_cast<float*>(stage + dma_dst[i]),
+                                         4, 0, 0);
+      }
     }
-    const uint8_t* wg = a.qw + static_cast<uint32_t>(g) * kCodeRowBytes<BITS>;
-#pragma unroll
-    for (int i = 0; i < kCodeInstr; ++i) {
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(wg + w_off[i]),
-                                       reinterpret_cast<u32x4*>(stage + kATileBytes + (wv * kCodeInstr + i) * 1024), 16, 0,
-                                       0);
-    }
-    __builtin_amdgcn_global_load_lds(s_lane + g * s_step, reinterpret_cast<float*>(stage + s_at), 4, 0, 0);
   };
   // Wait until at most `younger` of this wave's request batches are still in flight.
   auto wait_requests = [&](int younger) {
@@ -204,14 +252,14 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
     else if (younger == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDmaPerWave) : "memory");
     else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDmaPerWave) : "memory");
   };
-  static_assert(kStages<BITS> <= 4 && 2 * kDmaPerWave < 64, "wait_requests");
+  static_assert(kStages <= 4 && 2 * kDmaPerWave < 64, "wait_requests");
 
   // ---- LDS -> operands ------------------------------------------------------------------------------------
   // activation operand of k-step j, row tile mi: row wm*64 + mi*32 + lm, chunk 4 lh + j
   uint32_t a_rd[kMT][4];
 #pragma unroll
   for (int mi = 0; mi < kMT; ++mi) {
-    const int row = wm * 64 + mi * 32 + lm;
+    const int row = wm * kWaveM + mi * 32 + lm;
 #pragma unroll
     for (int j = 0; j < 4; ++j) a_rd[mi][j] = row * kARowBytes + (((4 * lh + j) ^ ((row >> 1) & 7)) << 4);
   }
@@ -226,7 +274,7 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
       c_rd[ni][q] = kATileBytes + row * kCodeRowBytes<BITS> + (code_slot<BITS>(row, lh * kRawLoads + q) << 4);
   }
   // per-row values of this lane's outputs (rows 8 q + 4 lh + 0..3 of row tile mi): scales, group starts
-  const uint32_t row_rd = kScalesAt + (wm * 64 + 4 * lh) * 4;
+  const uint32_t row_rd = kScalesAt + (wm * kWaveM + 4 * lh) * 4;
   const uint32_t sw_rd = kScalesAt + kSxTileBytes + (wn * kWaveN + lm) * 4;
   auto read16 = [&](const uint8_t* stage, uint32_t offset) { return *reinterpret_cast<const u32x4*>(stage + offset); };
 
@@ -240,10 +288,10 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
 
   const int n_groups = g_end - g_begin;
 #pragma unroll
-  for (int st = 0; st < kStages<BITS>; ++st) {
+  for (int st = 0; st < kStages; ++st) {
     if (st < n_groups) request(g_begin + st, st);
   }
-  wait_requests(min(kStages<BITS>, n_groups) - 1);
+  wait_requests(min(kStages, n_groups) - 1);
   __builtin_amdgcn_s_barrier();
 
   // The two waves of a SIMD work half a group apart. Between two barriers waves 0..3 multiply the group and
@@ -285,17 +333,22 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
 
   int st = 0;
   for (int g = g_begin; g < g_end; ++g) {
-    const uint8_t* stage = smem + st * kStageBytes<BITS>;
+    const uint8_t* stage = smem + st * kStageBytes;
     if (late && g > g_begin) fold();
 
     // what a lane holds of the group: its own columns' codes and weight scales, the first activation operand
-    u32x4 raw[kNT][kRawLoads], fa[2][kMT];
+    // (the narrow shape has registers to spare and little work to hide an LDS round trip under: it requests
+    // the activation operands of all four k-steps at once, the wide one those of the next k-step)
+    constexpr bool kAllAtOnce = MT * NT == 1;
+    u32x4 raw[kNT][kRawLoads], fa[kAllAtOnce ? 4 : 2][kMT];
 #pragma unroll
     for (int ni = 0; ni < kNT; ++ni)
 #pragma unroll
       for (int q = 0; q < kRawLoads; ++q) raw[ni][q] = read16(stage, c_rd[ni][q]);
 #pragma unroll
-    for (int mi = 0; mi < kMT; ++mi) fa[0][mi] = read16(stage, a_rd[mi][0]);
+    for (int j = 0; j < (kAllAtOnce ? 4 : 1); ++j)
+#pragma unroll
+      for (int mi = 0; mi < kMT; ++mi) fa[j][mi] = read16(stage, a_rd[mi][j]);
     v16i begin[kMT];
     if constexpr (BITS == 4) {
 #pragma unroll
@@ -315,27 +368,34 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
 #pragma unroll
     for (int ni = 0; ni < kNT; ++ni) sw_now[ni] = *reinterpret_cast<const float*>(stage + sw_rd + ni * 128);
 
+    // activation scales of this lane's output rows (rows 8 q + 4 lh + 0..3 of each row tile)
+    auto read_row_scales = [&]() {
+#pragma unroll
+      for (int mi = 0; mi < kMT; ++mi)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) sx_now[mi][q] = read16(stage, row_rd + (mi * 32 + 8 * q) * 4);
+    };
+    if constexpr (!TOKEN && kAllAtOnce) read_row_scales();
+    if constexpr (kAllAtOnce) __builtin_amdgcn_sched_barrier(0);   // (or the compiler sinks each read to its use)
+
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       v4i fb[kNT];
 #pragma unroll
       for (int ni = 0; ni < kNT; ++ni) fb[ni] = code_operand<BITS>(raw[ni], j);
       if (j < 3) {
+        if constexpr (!kAllAtOnce) {
 #pragma unroll
-        for (int mi = 0; mi < kMT; ++mi) fa[(j + 1) & 1][mi] = read16(stage, a_rd[mi][j + 1]);
-      } else if constexpr (!TOKEN) {
-        // activation scales of this lane's output rows (rows 8 q + 4 lh + 0..3 of each row tile)
-#pragma unroll
-        for (int mi = 0; mi < kMT; ++mi)
-#pragma unroll
-          for (int q = 0; q < 4; ++q)
-            sx_now[mi][q] = read16(stage, row_rd + (mi * 32 + 8 * q) * 4);
+          for (int mi = 0; mi < kMT; ++mi) fa[(j + 1) & 1][mi] = read16(stage, a_rd[mi][j + 1]);
+        }
+      } else if constexpr (!TOKEN && !kAllAtOnce) {
+        read_row_scales();
       }
 #pragma unroll
       for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
         for (int ni = 0; ni < kNT; ++ni) {
-          const v4i av = __builtin_bit_cast(v4i, fa[j & 1][mi]);
+          const v4i av = __builtin_bit_cast(v4i, fa[kAllAtOnce ? j : (j & 1)][mi]);
           acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, fb[ni], j == 0 ? begin[mi] : acc[mi][ni], 0, 0, 0);
         }
     }
@@ -345,12 +405,12 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
     // group kStages ahead; and each wave's own transfers of the next group have landed (younger batches may
     // stay in flight), so behind the barrier the next group's stage is complete.
     if (g + 1 < g_end) {
-      wait_requests(min(kStages<BITS> - 2, g_end - 2 - g));
+      wait_requests(min(kStages - 2, g_end - 2 - g));
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_s_barrier();
-      if (g + kStages<BITS> < g_end) request(g + kStages<BITS>, st);
+      if (g + kStages < g_end) request(g + kStages, st);
     }
-    st = st + 1 == kStages<BITS> ? 0 : st + 1;
+    st = st + 1 == kStages ? 0 : st + 1;
   }
   if (late) fold();
 
@@ -360,7 +420,7 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
     for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float sx = a.sx[min(m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3), a.M - 1)];
+        const float sx = a.sx[min(m0 + wm * kWaveM + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3), a.M - 1)];
 #pragma unroll
         for (int ni = 0; ni < kNT; ++ni) total[mi][ni][r] *= sx;
       }
@@ -375,7 +435,7 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
       for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          const int m = m0 + wm * kWaveM + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
           if (m < a.M && n < a.N) out[static_cast<int64_t>(m) * a.N + n] = from_float<T>(total[mi][ni][r] + b);
         }
     }
@@ -388,7 +448,7 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
       for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          const int m = m0 + wm * kWaveM + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
           if (m < a.M && n < a.N) part[static_cast<int64_t>(m) * a.N + n] = total[mi][ni][r];
         }
     }
@@ -412,17 +472,28 @@ constexpr size_t kAlign = 256;
 size_t aligned(size_t bytes) { return (bytes + kAlign - 1) / kAlign * kAlign; }
 
 struct Plan {
+  bool narrow;
   int m_tiles, n_tiles, splits, groups_per_split;
   size_t ap_bytes, start_bytes, partial_bytes;
 };
 
+constexpr int kWideBN = 256, kNarrowBN = 64;
+constexpr int kFillTiles = 160;   // fewer workgroups than this leave too much of the 256-CU chip idle
+
 Plan plan_for(int M, int N, int G) {
   Plan p{};
   p.m_tiles = (M + kBM - 1) / kBM;
-  p.n_tiles = (N + kBN - 1) / kBN;
+  // the narrow tile for one tile of rows where it fills the chip by itself; elsewhere the wide one, the
+  // reduction axis split if need be (measured: 128 x 14336 x 4096 narrow 38 us, wide and split 52 us;
+  // 128 x 4096 x 14336, where both must split, 37 and 33 us; 512 x 4096 x 14336 105 and 68 us)
+  const int wide_tiles = p.m_tiles * ((N + kWideBN - 1) / kWideBN);
+  const int narrow_tiles = p.m_tiles * ((N + kNarrowBN - 1) / kNarrowBN);
+  p.narrow = p.m_tiles == 1 && wide_tiles < kFillTiles && narrow_tiles >= kFillTiles;
+  const int bn = p.narrow ? kNarrowBN : kWideBN;
+  p.n_tiles = (N + bn - 1) / bn;
   const int tiles = p.m_tiles * p.n_tiles;
   int splits = 1;
-  if (tiles < 160) {  // too few tiles to occupy the chip: cut the reduction axis, at least four groups a slice
+  if (tiles < kFillTiles) {  // cut the reduction axis, at least four groups a slice
     splits = (256 + tiles - 1) / tiles;
     if (splits > G / 4) splits = G / 4;
     if (splits < 1) splits = 1;
@@ -435,21 +506,27 @@ Plan plan_for(int M, int N, int G) {
   return p;
 }
 
-template <typename T, int BITS, bool TOKEN>
+template <typename T, int BITS, bool TOKEN, int MT, int NT>
 int launch_tiles(const A8Args& a, dim3 grid, hipStream_t stream) {
-  auto kernel = wq_gemm_a8_tile_kernel<T, BITS, TOKEN>;
+  auto kernel = wq_gemm_a8_tile_kernel<T, BITS, TOKEN, MT, NT>;
+  constexpr int kLds = Shape<BITS, MT, NT>::kLdsBytes;
   static bool raised = false;  // per instantiation; worst case two threads both set it
   if (!raised) {
     const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes<BITS>);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (err != hipSuccess) {
       llmq_host::set_error("raising the LDS limit failed: %s", hipGetErrorString(err));
       return static_cast<int>(err);
     }
     raised = true;
   }
-  hipLaunchKernelGGL(kernel, grid, dim3(kThreads), kLdsBytes<BITS>, stream, a);
+  hipLaunchKernelGGL(kernel, grid, dim3(kThreads), kLds, stream, a);
   return llmq_host::check_launch("wq_gemm_a8_tile_kernel");
+}
+
+template <typename T, int BITS, bool TOKEN>
+int launch_shape(const A8Args& a, const Plan& p, dim3 grid, hipStream_t s) {
+  return p.narrow ? launch_tiles<T, BITS, TOKEN, 1, 1>(a, grid, s) : launch_tiles<T, BITS, TOKEN, 2, 2>(a, grid, s);
 }
 
 template <typename T>
@@ -457,8 +534,8 @@ int run_typed(A8Args& a, const Plan& p, int wformat, bool token, hipStream_t s) 
   const int total = p.m_tiles * p.n_tiles * p.splits;
   const dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8));
   int rc;
-  if (wformat == LLMQ_W_INT4_PACKED) rc = token ? launch_tiles<T, 4, true>(a, grid, s) : launch_tiles<T, 4, false>(a, grid, s);
-  else rc = token ? launch_tiles<T, 8, true>(a, grid, s) : launch_tiles<T, 8, false>(a, grid, s);
+  if (wformat == LLMQ_W_INT4_PACKED) rc = token ? launch_shape<T, 4, true>(a, p, grid, s) : launch_shape<T, 4, false>(a, p, grid, s);
+  else rc = token ? launch_shape<T, 8, true>(a, p, grid, s) : launch_shape<T, 8, false>(a, p, grid, s);
   if (rc) return rc;
   if (p.splits > 1) {
     const int64_t count = static_cast<int64_t>(a.M) * a.N;

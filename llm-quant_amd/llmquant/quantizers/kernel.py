@@ -102,6 +102,10 @@ class KernelQuantLinear(nn.Module):
         act = scheme.input_activations
         self._int8_act = (act is not None and act.num_bits == 8 and act.strategy == "group"
                           and act.group_size == group_size == 128)
+        #: int8 activations: True keeps RealQuantLinear's fp32 roundings bit for bit; False takes the tiled
+        #: integer GEMM that folds a group in with one rounding fewer (same integer sums, agrees to ~1e-7
+        #: relative) and runs up to twice as fast on prompt-sized activations
+        self.a8_exact = True
         # the fused GEMM's reach (it needs groups of 128)
         self._fused_max_rows = FUSED_GEMM_MAX_ROWS if group_size == 128 else 0
         # looked up once: a decode step runs ~113 of these modules
@@ -191,7 +195,7 @@ class KernelQuantLinear(nn.Module):
         if self._int8_act:
             codes, act_scale = self._ext.quant_group_codes(rows, 8, 128, False)
             out = self._ext.wq_gemm_a8(codes, act_scale, self.qdata, self.wscale, self.bias, self.out_group,
-                                       x.dtype)
+                                       x.dtype, self.a8_exact)
             return out.reshape(*x.shape[:-1], self.out_features)
         if fused:
             out = self._ext.wq_gemm_a16(rows, self.qdata, self.wscale, self.out_group,

@@ -113,9 +113,16 @@ def test_module_equals_real_mode_on_device(name, layout, m):
     torch.manual_seed(0)
     linear = nn.Linear(2048, 512, bias=True).cuda().to(torch.bfloat16)
     x = torch.randn(m, 2048, device="cuda", dtype=torch.bfloat16)
-    got = KernelQuantLinear.from_linear(linear, scheme)(x)
+    module = KernelQuantLinear.from_linear(linear, scheme)
+    got = module(x)
     want = RealQuantLinear.from_linear(linear, scheme)(x)
     assert got.shape == want.shape and torch.equal(got, want)
+    # the module's switch to the fast form: same integer sums, one rounding fewer per group
+    module.a8_exact = False
+    fast = module(x)
+    assert fast.shape == want.shape
+    assert (fast == want).float().mean().item() > 0.98
+    assert rel_l2(fast.detach().float().cpu().numpy(), want.detach().float().cpu().numpy()) <= 4e-3
 
 
 def test_c_oracle_agrees_at_a_larger_size(ext):
@@ -140,8 +147,11 @@ def test_argument_checks(ext):
     assert ext.wq_gemm_a8(a, sx, q, s).shape == (4, 8)
     with pytest.raises(RuntimeError, match="a must be int8"):
         ext.wq_gemm_a8(a.float(), sx, q, s)
+    assert ext.wq_gemm_a8(a, sx[:, :1], q, s).shape == (4, 8)   # one scale per token
     with pytest.raises(RuntimeError, match="sx must be"):
-        ext.wq_gemm_a8(a, sx[:, :1], q, s)
+        ext.wq_gemm_a8(a, torch.ones(4, 3, device="cuda"), q, s)
+    with pytest.raises(RuntimeError, match="sx must be"):
+        ext.wq_gemm_a8(a, torch.ones(4, 3, device="cuda"), q, s, None, 0, torch.float32, False)
     with pytest.raises(RuntimeError, match="group_size 128"):
         ext.wq_gemm_a8(a, torch.ones(4, 4, device="cuda"), torch.zeros(8, 4, 64, dtype=torch.int8, device="cuda"),
                        torch.ones(8, 4, device="cuda"))
