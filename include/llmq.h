@@ -175,13 +175,14 @@ int llmq_wq_gemm_a8(const int8_t* a, const float* sx, const void* qweight, const
 
 /* The same GEMM in its fast form: the same exact integer group sums, folded into the total as
  * fma((float)isum * sw, sx, total) (one instruction and one rounding fewer than RealQuantLinear's
- * ((float)isum * sw) * sx followed by an add, llmquant/quantizers/real.py:94-99), with the reduction axis split
- * across workgroups where the output has few 128 x 256 tiles (fp32 partial tiles added in a fixed order by a
- * second launch). Agrees with llmq_wq_gemm_a8 to fp32 rounding (rel-L2 ~1e-7), not bit for bit. Arguments as
- * for llmq_wq_gemm_a8 plus `sx_groups`: G for sx [M, G], or 1 for one activation scale per token, sx [M] (the
- * scale then leaves the sum over groups: two instructions per output and group instead of three); and `workspace`: llmq_wq_gemm_a8_fast_workspace_bytes(M, N, G) bytes, 16-byte aligned,
- * contents irrelevant before and after (the activation in operand order and the partial tiles); calls that
- * share a workspace must not overlap. */
+ * ((float)isum * sw) * sx followed by an add, llmquant/quantizers/real.py:94-99). Where the output has too few
+ * tiles to fill the chip the reduction axis is split across workgroups (fp32 partial tiles added in a fixed
+ * order by a second launch). Agrees with llmq_wq_gemm_a8 to fp32 rounding (rel-L2 ~1e-7), not bit for bit.
+ * Arguments as for llmq_wq_gemm_a8 plus `sx_groups`: G for sx [M, G], or 1 for one activation scale per token,
+ * sx [M] (the scale then leaves the sum over groups: two instructions per output and group instead of
+ * three); and `workspace`: llmq_wq_gemm_a8_fast_workspace_bytes(M, N, G) bytes (0 where nothing is split: then
+ * it may be null), 16-byte aligned, contents irrelevant before and after (the activation in operand order and
+ * the partial tiles); calls that share a workspace must not overlap. */
 size_t llmq_wq_gemm_a8_fast_workspace_bytes(int M, int N, int G);
 int llmq_wq_gemm_a8_fast(const int8_t* a, const float* sx, const void* qweight, const float* wscale,
                          const float* bias_or_null, void* out, void* workspace, size_t workspace_bytes, int M,

@@ -244,6 +244,11 @@ int fail_invalid(const char* fmt, ...);   // records the text, returns hipErrorI
 int check_launch(const char* what);       // hipGetLastError() -> 0 or the error, text recorded
 
 bool gemv_force_alu();
+// The integer GEMM's kernel with its scale epilogue in three (or, one activation scale per token, two)
+// vector instructions per output and group instead of real mode's four (wq_gemm_a8.hip).
+int gemm_a8_relaxed(const int8_t* a, const float* sx, const void* qweight, const float* wscale,
+                    const float* bias_or_null, void* out, int M, int N, int G, bool token_scale, int out_group,
+                    int wformat, int dtype, hipStream_t stream);
 // Matrix-core GEMV (wq_gemv_mfma.hip): whether it can take a problem, and its launch.
 bool gemv_mfma_supported(const void* x, const void* qw, const float* ws, int M, int G, int gs,
                          int wformat);

@@ -542,7 +542,7 @@ at::Tensor wq_gemm_a8(const at::Tensor& a, const at::Tensor& sx, const at::Tenso
     auto workspace = at::empty({static_cast<int64_t>((need + 3) / 4)}, ac.options().dtype(at::kFloat));
     check_rc(llmq_wq_gemm_a8_fast(ac.const_data_ptr<int8_t>(), sxc.const_data_ptr<float>(), wc.const_data_ptr(),
                                   sc.const_data_ptr<float>(), bias_f.defined() ? bias_f.const_data_ptr<float>() : nullptr,
-                                  out.mutable_data_ptr(), workspace.mutable_data_ptr(), need, static_cast<int>(M),
+                                  out.mutable_data_ptr(), need ? workspace.mutable_data_ptr() : nullptr, need, static_cast<int>(M),
                                   static_cast<int>(N), static_cast<int>(groups), static_cast<int>(sx_groups),
                                   static_cast<int>(group_size), static_cast<int>(out_group),
                                   packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype, current_stream(ac)),

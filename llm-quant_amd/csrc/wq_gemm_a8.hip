@@ -22,6 +22,11 @@
 // scale epilogue above: four vector-ALU operations per output element per group, against 256
 // multiply-adds on the matrix core, which makes the vector ALU the unit that bounds this
 // kernel (two waves per SIMD, so that one wave's epilogue runs under the other's MFMAs).
+//
+// MODE. 0 is the arithmetic above, bit for bit. 1 and 2 are the tolerance forms behind llmq_wq_gemm_a8_fast:
+// the same exact integer group sums, folded in with fewer vector instructions: 1: fma((float)isum * sw, sx,
+// total), three per output and group instead of four; 2: one activation scale per token (sx[M]), which
+// leaves the sum over groups: fma((float)isum, sw, total), two, and the token's scale once at the store.
 #include <type_traits>
 
 #include "llmq_device.h"
@@ -39,7 +44,7 @@ constexpr int kRowStride = kGroup + 16;  // bytes; padding keeps 16-byte reads o
 
 struct GemmArgs {
   const int8_t* a;     // [M, G*128]
-  const float* sx;     // [M, G]
+  const float* sx;     // [M, G]; MODE 2: [M]
   const uint8_t* qw;   // [N, G, 128] int8 or [N, G, 64] packed
   const float* sw;     // [scale_rows, G]
   const float* bias;   // [N] or null
@@ -50,7 +55,7 @@ struct GemmArgs {
 // W: the wave's quadrant is (32 W) x (32 W), the workgroup's tile (64 W) x (64 W). W = 2 is the
 // throughput shape; W = 1 gives four times as many workgroups when the problem is too small to
 // fill the chip with 128 x 128 tiles.
-template <typename T, int BITS, int W>
+template <typename T, int BITS, int W, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs g) {
   constexpr int kBM = 64 * W, kBN = 64 * W;
   __shared__ __attribute__((aligned(16))) int8_t s_a[2][kBM * kRowStride];
@@ -117,7 +122,7 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
     // loads that may stay in flight instead of draining them all
     if constexpr (!kBranchFreeLoop) {
       if (tid < kBM) {
-        r_sx = g.sx[static_cast<int64_t>(min(m0 + tid, g.M - 1)) * g.G + grp];
+        if constexpr (MODE != 2) r_sx = g.sx[static_cast<int64_t>(min(m0 + tid, g.M - 1)) * g.G + grp];
       } else if (tid < kBM + kBN) {
         const int n = min(n0 + tid - kBM, g.N - 1);
         r_sw = g.sw[static_cast<int64_t>(g.out_group > 0 ? n / g.out_group : n) * g.G + grp];
@@ -125,8 +130,9 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
     } else {
       const int idx = tid < kBM ? tid : (tid - kBM) & (kBN - 1);
       const int n = min(n0 + idx, g.N - 1);
-      const float* sp = tid < kBM ? g.sx + static_cast<int64_t>(min(m0 + idx, g.M - 1)) * g.G
-                                  : g.sw + static_cast<int64_t>(g.out_group > 0 ? n / g.out_group : n) * g.G;
+      // (MODE 2 has no activation scale per group: those threads repeat a weight scale's load)
+      const float* sp = (tid < kBM && MODE != 2) ? g.sx + static_cast<int64_t>(min(m0 + idx, g.M - 1)) * g.G
+                                                 : g.sw + static_cast<int64_t>(g.out_group > 0 ? n / g.out_group : n) * g.G;
       const float v = sp[grp];
       r_sx = v;
       r_sw = v;
@@ -224,15 +230,21 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
       for (int r4 = 0; r4 < 4; ++r4) {
         // four consecutive rows: one 128-bit LDS read of their activation scales
         const int row = (wm * W + mi) * 32 + 8 * r4 + 4 * (lane >> 5);
-        const u32x4 s4 = *reinterpret_cast<const u32x4*>(&s_sx[buf][row]);
+        const u32x4 s4 = MODE == 2 ? u32x4{0, 0, 0, 0} : *reinterpret_cast<const u32x4*>(&s_sx[buf][row]);
         const float sx4[4] = {__builtin_bit_cast(float, s4.x), __builtin_bit_cast(float, s4.y),
                               __builtin_bit_cast(float, s4.z), __builtin_bit_cast(float, s4.w)};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           float f = static_cast<float>(d[4 * r4 + i]);
-          f = f * sw;
-          f = f * sx4[i];
-          acc[mi][ni][4 * r4 + i] = acc[mi][ni][4 * r4 + i] + f;
+          if constexpr (MODE == 0) {
+            f = f * sw;
+            f = f * sx4[i];
+            acc[mi][ni][4 * r4 + i] = acc[mi][ni][4 * r4 + i] + f;
+          } else if constexpr (MODE == 1) {
+            acc[mi][ni][4 * r4 + i] = fmaf(f * sw, sx4[i], acc[mi][ni][4 * r4 + i]);
+          } else {
+            acc[mi][ni][4 * r4 + i] = fmaf(f, sw, acc[mi][ni][4 * r4 + i]);
+          }
         }
       }
     };
@@ -281,6 +293,7 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + (wm * W + mi) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (m < g.M && n < g.N) {
+          if constexpr (MODE == 2) acc[mi][ni][r] *= g.sx[m];
           const float v = g.bias != nullptr ? acc[mi][ni][r] + b : acc[mi][ni][r];
           out[static_cast<int64_t>(m) * g.N + n] = from_float<T>(v);
         }
@@ -289,23 +302,33 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
   }
 }
 
-template <typename T, int W>
+template <typename T, int W, int MODE>
 int launch_tile(const GemmArgs& g, int wformat, hipStream_t stream) {
   constexpr int kTile = 64 * W;
   const dim3 grid((g.N + kTile - 1) / kTile, (g.M + kTile - 1) / kTile), block(kThreads);
   if (wformat == LLMQ_W_INT8) {
-    hipLaunchKernelGGL((wq_gemm_a8_kernel<T, 8, W>), grid, block, 0, stream, g);
+    hipLaunchKernelGGL((wq_gemm_a8_kernel<T, 8, W, MODE>), grid, block, 0, stream, g);
   } else {
-    hipLaunchKernelGGL((wq_gemm_a8_kernel<T, 4, W>), grid, block, 0, stream, g);
+    hipLaunchKernelGGL((wq_gemm_a8_kernel<T, 4, W, MODE>), grid, block, 0, stream, g);
   }
   return llmq_host::check_launch("wq_gemm_a8_kernel");
 }
 
-template <typename T>
+template <typename T, int MODE>
 int launch_typed(const GemmArgs& g, int wformat, hipStream_t stream) {
   // 128 x 128 tiles when there is at least one for every CU, else 64 x 64
   const int64_t big_tiles = static_cast<int64_t>((g.N + 127) / 128) * ((g.M + 127) / 128);
-  return big_tiles >= 256 ? launch_tile<T, 2>(g, wformat, stream) : launch_tile<T, 1>(g, wformat, stream);
+  return big_tiles >= 256 ? launch_tile<T, 2, MODE>(g, wformat, stream) : launch_tile<T, 1, MODE>(g, wformat, stream);
+}
+
+template <int MODE>
+int launch_mode(const GemmArgs& g, int wformat, int dtype, hipStream_t s) {
+  switch (dtype) {
+    case LLMQ_F32: return launch_typed<float, MODE>(g, wformat, s);
+    case LLMQ_F16: return launch_typed<f16_t, MODE>(g, wformat, s);
+    case LLMQ_BF16: return launch_typed<bf16_t, MODE>(g, wformat, s);
+  }
+  return llmq_host::fail_invalid("out must be float32, float16 or bfloat16, got dtype code %d", dtype);
 }
 
 }  // namespace
@@ -325,11 +348,13 @@ extern "C" int llmq_wq_gemm_a8(const int8_t* a, const float* sx, const void* qwe
   if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(qweight)) & 15u)
     return llmq_host::fail_invalid("activation and weight pointers must be 16-byte aligned");
   GemmArgs g{a, sx, static_cast<const uint8_t*>(qweight), wscale, bias_or_null, out, M, N, G, out_group};
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  switch (dtype) {
-    case LLMQ_F32: return launch_typed<float>(g, wformat, s);
-    case LLMQ_F16: return launch_typed<f16_t>(g, wformat, s);
-    case LLMQ_BF16: return launch_typed<bf16_t>(g, wformat, s);
-  }
-  return llmq_host::fail_invalid("out must be float32, float16 or bfloat16, got dtype code %d", dtype);
+  return launch_mode<0>(g, wformat, dtype, static_cast<hipStream_t>(stream));
+}
+
+// The tolerance forms of the same kernel (arguments already checked by llmq_wq_gemm_a8_fast).
+int llmq_host::gemm_a8_relaxed(const int8_t* a, const float* sx, const void* qweight, const float* wscale,
+                               const float* bias_or_null, void* out, int M, int N, int G, bool token_scale,
+                               int out_group, int wformat, int dtype, hipStream_t stream) {
+  GemmArgs g{a, sx, static_cast<const uint8_t*>(qweight), wscale, bias_or_null, out, M, N, G, out_group};
+  return token_scale ? launch_mode<2>(g, wformat, dtype, stream) : launch_mode<1>(g, wformat, dtype, stream);
 }

@@ -1,5 +1,5 @@
-// Integer prefill GEMM, the fast form: int8 activations (one scale per token and group) times int4 / int8
-// group-quantized weights on the int8 matrix core,
+// Integer prefill GEMM, the fast form: int8 activations (one scale per token and group, or one per token) times
+// int4 / int8 group-quantized weights on the int8 matrix core,
 //
 //   out[m, n] = sum over g of  sx[m, g] * sw[sr(n), g] * (float)(sum_k a[m, g, k] * q[n, g, k])
 //
@@ -7,13 +7,21 @@
 // group sums but not the same fp32 roundings: there each group contributes ((float)isum * sw) * sx, added to
 // the total, four separately rounded operations in group order (llmq_wq_gemm_a8 reproduces exactly that,
 // and is bound by those four vector-ALU instructions per output and group); here a group contributes
-// fma((float)isum * sw, sx, total), three instructions and one rounding fewer, and the reduction axis may be
-// split across workgroups, so results agree with real mode to fp32 rounding (~1e-7), not bit for bit.
+// fma((float)isum * sw, sx, total), three instructions and one rounding fewer (two with one scale per token,
+// which leaves the sum), and the reduction axis may be split across workgroups, so results agree with real
+// mode to fp32 rounding (~1e-7), not bit for bit.
+//
+// llmq_wq_gemm_a8_fast has two kernels behind it. Where the output alone has tiles enough to fill the chip it
+// is the kernel of llmq_wq_gemm_a8 with the relaxed epilogue (wq_gemm_a8.hip, MODE 1 / 2). Where it has not
+// (a weight of a few thousand rows under a prompt of a few hundred tokens: N = 4096, K = 14336, M = 128 leaves
+// that kernel at 4 % of the matrix core's peak), the reduction axis is split across workgroups by the kernel
+// of this file: fp32 partial tiles in a workspace, added in a fixed order (and the bias after them) by a second
+// launch.
 //
 // Shape: that of the tiled bf16 GEMM (wq_gemm_a16_tile.hip). A workgroup of eight waves, two per SIMD, owns a
-// 128 (m) x 256 (n) output tile; a wave owns 64 x 64: 2 x 2 tiles of v_mfma_i32_32x32x32_i8, four k-steps of
-// 32 per group, int32 group sums and fp32 totals in vector registers. (For a single tile of rows and a wide
-// weight a workgroup owns 128 x 64 instead, a wave 32 x 32: four times the workgroups, no split.) All operands
+// 128 (m) x 256 (n) output tile over its slice of the groups; a wave owns 64 x 64: 2 x 2 tiles of
+// v_mfma_i32_32x32x32_i8, four k-steps of 32 per group, int32 group sums and fp32 totals in vector registers.
+// All operands
 // reach LDS straight from global memory (global_load_lds, 1 KB per wave instruction; 16-byte slots
 // XOR-swizzled by row so that the operand reads of 16 consecutive rows are conflict-free), three or four
 // stages deep: the activation tile [128 rows][128 bytes], the raw codes of the weight rows, the 128 activation
@@ -35,9 +43,6 @@
 // 60-70 issue cycles per MFMA against the MFMA's own 32, so the matrix core cannot be more than about half
 // busy whatever the schedule (interleaving the fold under the MFMAs by hand, a fifth k-step for the -8
 // instead of the C operand, DPP-broadcast scales and deeper LDS prefetch all measured the same or slower).
-//
-// Small N: the reduction axis is split across workgroups, fp32 partial tiles in a workspace, added in a fixed
-// order (and the bias after them) by a second launch.
 #include "llmq_device.h"
 
 namespace {
@@ -56,10 +61,7 @@ template <int BITS> constexpr int kCodeRowBytes = BITS == 4 ? kGroup / 2 : kGrou
 constexpr int kSxTileBytes = kBM * 4, kStartTileBytes = kBM * 4;
 
 // The shape of a workgroup's tile: 128 rows by BN columns, eight waves as WM x WN, a wave owning MT x NT MFMA
-// tiles of 32 x 32. Wide (MT = NT = 2: 2 x 4 waves of 64 x 64, BN = 256) is the throughput shape: every operand
-// read from LDS feeds two MFMAs. Narrow (MT = NT = 1: 4 x 2 waves of 32 x 32, BN = 64) gives four times as many
-// workgroups, for activations of a tile or two of rows, where the wide shape would leave most of the chip idle
-// or split the reduction axis many ways.
+// tiles of 32 x 32. MT = NT = 2 (2 x 4 waves of 64 x 64, BN = 256): every operand read from LDS feeds two MFMAs.
 template <int BITS, int MT, int NT>
 struct Shape {
   static constexpr int kWM = kBM / (32 * MT), kWN = kWaves / kWM;
@@ -77,6 +79,8 @@ struct Shape {
   static constexpr int kUnits = kAUnits + kCodeUnits + kSxUnits + kSwUnits + kStartUnits;
   static constexpr int kDmaPerWave = (kUnits + kWaves - 1) / kWaves;
   static_assert(kBM % kWaveM == 0 && kWM * kWN == kWaves && kBN % 64 == 0 && kCodeTileBytes % 1024 == 0, "tile shape");
+  // every wave the same kinds of transfer in the same slots: the widths are compile-time facts
+  static_assert(kAUnits % kWaves == 0 && kCodeUnits % kWaves == 0 && kSxUnits + kSwUnits + kStartUnits <= kWaves, "slots");
 };
 
 // ---- activation preparation: rows padded to whole tiles, bytes in operand order -------------------------
@@ -114,8 +118,8 @@ struct A8Args {
   const float* sx;     // [M, G], or [M] (one scale per token)
   const uint8_t* qw;   // [N, G, 128] int8 or [N, G, 64] packed int4
   const float* sw;     // [scale_rows, G]
-  const float* bias;   // [N] or null (applied here with one split, else by the second launch)
-  void* out;           // [M, N]
+  const float* bias;   // [N] or null (added by the second launch)
+  void* out;           // [M, N] (written by the second launch)
   float* partial;      // [splits][M][N]
   int M, N, G, out_group;
   int m_tiles, n_tiles, splits, groups_per_split;
@@ -142,7 +146,7 @@ __device__ __forceinline__ v4i code_operand(const u32x4* raw, int step) {
 // TOKEN: one activation scale per token (sx[M]) instead of one per token and group (sx[M, G]): the scale leaves
 // the sum over groups, a group's sums are folded in with two instructions per output instead of three, and
 // the token's scale is applied once, at the store.
-template <typename T, int BITS, bool TOKEN, int MT, int NT>
+template <int BITS, bool TOKEN, int MT, int NT>
 __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Args a) {
   using S = Shape<BITS, MT, NT>;
   constexpr int kMT = MT, kNT = NT, kBN = S::kBN, kWaveM = S::kWaveM, kWaveN = S::kWaveN;
@@ -167,12 +171,12 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
   const int g_end = min(g_begin + a.groups_per_split, a.G);
 
   // ---- global -> LDS ----------------------------------------------------------------------------------------
-  // A stage is filled by S::kUnits transfers of 64 lanes: 16 of activations (8 rows each; lane = (row, slot),
-  // slot p of row r holds chunk p ^ ((r >> 1) & 7)), the codes (1 KB each, slots swizzled by code_slot), the
-  // activation scales of 64 rows, the weight scales of 64 columns and (int4) the group starts of 64 rows, four
-  // bytes a lane. Every wave issues kDmaPerWave of them per group, wave w the units w * kDmaPerWave + 0, 1, ...
-  // (modulo the count: a few units are transferred twice, with the same bytes, so that every wave has the same
-  // number in flight and one vmcnt serves all).
+  // A stage is filled by transfers of 64 lanes: 16 of activations (8 rows each; lane = (row, slot), slot p of
+  // row r holds chunk p ^ ((r >> 1) & 7)), the codes (1 KB each, slots swizzled by code_slot), and four bytes
+  // a lane for the activation scales of 64 rows, the weight scales of 64 columns and (int4) the group starts
+  // of 64 rows. Every wave issues kDmaPerWave of them per group: its share of the activation and code units
+  // and one of the 64-value vectors (a wave beyond their count repeats one, with the same bytes, so that every
+  // wave has the same number in flight and one vmcnt serves all).
   constexpr int kRowsPerUnit = 1024 / kCodeRowBytes<BITS>;
   constexpr int kSlots = kCodeRowBytes<BITS> / 16;
   const uint8_t* dma_base[kDmaPerWave];
@@ -213,24 +217,13 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
     }
   };
   constexpr int kVectorUnits = S::kSxUnits + S::kSwUnits + S::kStartUnits;
-  if constexpr (S::kAUnits % kWaves == 0 && S::kCodeUnits % kWaves == 0 && kVectorUnits <= kWaves) {
-    // every wave the same kinds in the same slots: the transfer widths are compile-time facts
-    constexpr int kA = S::kAUnits / kWaves, kC = S::kCodeUnits / kWaves;
-    static_assert(kDmaPerWave == kA + kC + 1, "slots");
+  constexpr int kA = S::kAUnits / kWaves, kC = S::kCodeUnits / kWaves;
+  static_assert(kDmaPerWave == kA + kC + 1, "slots");
 #pragma unroll
-    for (int i = 0; i < kA; ++i) a_unit(i, wv * kA + i);
+  for (int i = 0; i < kA; ++i) a_unit(i, wv * kA + i);
 #pragma unroll
-    for (int i = 0; i < kC; ++i) code_unit(kA + i, wv * kC + i);
-    vector_unit(kA + kC, wv % kVectorUnits);
-  } else {
-#pragma unroll
-    for (int i = 0; i < kDmaPerWave; ++i) {
-      const int u = (wv * kDmaPerWave + i) % S::kUnits;
-      if (u < S::kAUnits) a_unit(i, u);
-      else if (u < S::kAUnits + S::kCodeUnits) code_unit(i, u - S::kAUnits);
-      else vector_unit(i, u - S::kAUnits - S::kCodeUnits);
-    }
-  }
+  for (int i = 0; i < kC; ++i) code_unit(kA + i, wv * kC + i);
+  vector_unit(kA + kC, wv % kVectorUnits);
 
   auto request = [&](int g, int st) {
     uint8_t* stage = smem + st * kStageBytes;
@@ -337,18 +330,13 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
     if (late && g > g_begin) fold();
 
     // what a lane holds of the group: its own columns' codes and weight scales, the first activation operand
-    // (the narrow shape has registers to spare and little work to hide an LDS round trip under: it requests
-    // the activation operands of all four k-steps at once, the wide one those of the next k-step)
-    constexpr bool kAllAtOnce = MT * NT == 1;
-    u32x4 raw[kNT][kRawLoads], fa[kAllAtOnce ? 4 : 2][kMT];
+    u32x4 raw[kNT][kRawLoads], fa[2][kMT];
 #pragma unroll
     for (int ni = 0; ni < kNT; ++ni)
 #pragma unroll
       for (int q = 0; q < kRawLoads; ++q) raw[ni][q] = read16(stage, c_rd[ni][q]);
 #pragma unroll
-    for (int j = 0; j < (kAllAtOnce ? 4 : 1); ++j)
-#pragma unroll
-      for (int mi = 0; mi < kMT; ++mi) fa[j][mi] = read16(stage, a_rd[mi][j]);
+    for (int mi = 0; mi < kMT; ++mi) fa[0][mi] = read16(stage, a_rd[mi][0]);
     v16i begin[kMT];
     if constexpr (BITS == 4) {
 #pragma unroll
@@ -375,8 +363,6 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
 #pragma unroll
         for (int q = 0; q < 4; ++q) sx_now[mi][q] = read16(stage, row_rd + (mi * 32 + 8 * q) * 4);
     };
-    if constexpr (!TOKEN && kAllAtOnce) read_row_scales();
-    if constexpr (kAllAtOnce) __builtin_amdgcn_sched_barrier(0);   // (or the compiler sinks each read to its use)
 
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -384,18 +370,16 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
 #pragma unroll
       for (int ni = 0; ni < kNT; ++ni) fb[ni] = code_operand<BITS>(raw[ni], j);
       if (j < 3) {
-        if constexpr (!kAllAtOnce) {
 #pragma unroll
-          for (int mi = 0; mi < kMT; ++mi) fa[(j + 1) & 1][mi] = read16(stage, a_rd[mi][j + 1]);
-        }
-      } else if constexpr (!TOKEN && !kAllAtOnce) {
-        read_row_scales();
+        for (int mi = 0; mi < kMT; ++mi) fa[(j + 1) & 1][mi] = read16(stage, a_rd[mi][j + 1]);
+      } else if constexpr (!TOKEN) {
+        read_row_scales();   // (while the stage still holds them)
       }
 #pragma unroll
       for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
         for (int ni = 0; ni < kNT; ++ni) {
-          const v4i av = __builtin_bit_cast(v4i, fa[kAllAtOnce ? j : (j & 1)][mi]);
+          const v4i av = __builtin_bit_cast(v4i, fa[j & 1][mi]);
           acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, fb[ni], j == 0 ? begin[mi] : acc[mi][ni], 0, 0, 0);
         }
     }
@@ -425,33 +409,18 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a8_tile_kernel(const A8Ar
         for (int ni = 0; ni < kNT; ++ni) total[mi][ni][r] *= sx;
       }
   }
-  if (a.splits == 1) {
-    T* __restrict__ out = static_cast<T*>(a.out);
+  // this slice's partial tile; the second launch adds the slices in order, then the bias
+  float* __restrict__ part = a.partial + static_cast<int64_t>(sp) * a.M * a.N;
 #pragma unroll
-    for (int ni = 0; ni < kNT; ++ni) {
-      const int n = n0 + wn * kWaveN + ni * 32 + lm;
-      const float b = (a.bias != nullptr && n < a.N) ? a.bias[n] : 0.0f;
+  for (int ni = 0; ni < kNT; ++ni) {
+    const int n = n0 + wn * kWaveN + ni * 32 + lm;
 #pragma unroll
-      for (int mi = 0; mi < kMT; ++mi)
+    for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm * kWaveM + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-          if (m < a.M && n < a.N) out[static_cast<int64_t>(m) * a.N + n] = from_float<T>(total[mi][ni][r] + b);
-        }
-    }
-  } else {
-    float* __restrict__ part = a.partial + static_cast<int64_t>(sp) * a.M * a.N;
-#pragma unroll
-    for (int ni = 0; ni < kNT; ++ni) {
-      const int n = n0 + wn * kWaveN + ni * 32 + lm;
-#pragma unroll
-      for (int mi = 0; mi < kMT; ++mi)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm * kWaveM + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-          if (m < a.M && n < a.N) part[static_cast<int64_t>(m) * a.N + n] = total[mi][ni][r];
-        }
-    }
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * kWaveM + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+        if (m < a.M && n < a.N) part[static_cast<int64_t>(m) * a.N + n] = total[mi][ni][r];
+      }
   }
 }
 
@@ -472,43 +441,43 @@ constexpr size_t kAlign = 256;
 size_t aligned(size_t bytes) { return (bytes + kAlign - 1) / kAlign * kAlign; }
 
 struct Plan {
-  bool narrow;
   int m_tiles, n_tiles, splits, groups_per_split;
   size_t ap_bytes, start_bytes, partial_bytes;
 };
 
-constexpr int kWideBN = 256, kNarrowBN = 64;
+constexpr int kTileBN = Shape<4, 2, 2>::kBN;
 constexpr int kFillTiles = 160;   // fewer workgroups than this leave too much of the 256-CU chip idle
 
+// splits == 1: the kernel of llmq_wq_gemm_a8 with the relaxed epilogue takes the call (no preparation pass,
+// several independent workgroups per CU, 64 x 64 tiles where 128 x 128 are too few). This file's kernel takes
+// it where the output has too few tiles and the rows are long, the reduction axis cut into slices of at
+// least four groups. Measured, int4, us (that kernel / this one): 128 x 4096 x 14336 64.5 / 32.8;
+// 512 x 4096 x 14336 85.5 / 67.4; but 128 x 14336 x 4096 (32 groups a row) 29.2 / 51.6; and where neither
+// splits, 2048 x 14336 x 4096 252 / 261, 2048 x 4096 x 14336 209 / 214.
+constexpr int kSplitMinGroups = 64;
 Plan plan_for(int M, int N, int G) {
   Plan p{};
   p.m_tiles = (M + kBM - 1) / kBM;
-  // the narrow tile for one tile of rows where it fills the chip by itself; elsewhere the wide one, the
-  // reduction axis split if need be (measured: 128 x 14336 x 4096 narrow 38 us, wide and split 52 us;
-  // 128 x 4096 x 14336, where both must split, 37 and 33 us; 512 x 4096 x 14336 105 and 68 us)
-  const int wide_tiles = p.m_tiles * ((N + kWideBN - 1) / kWideBN);
-  const int narrow_tiles = p.m_tiles * ((N + kNarrowBN - 1) / kNarrowBN);
-  p.narrow = p.m_tiles == 1 && wide_tiles < kFillTiles && narrow_tiles >= kFillTiles;
-  const int bn = p.narrow ? kNarrowBN : kWideBN;
-  p.n_tiles = (N + bn - 1) / bn;
+  p.n_tiles = (N + kTileBN - 1) / kTileBN;
   const int tiles = p.m_tiles * p.n_tiles;
   int splits = 1;
-  if (tiles < kFillTiles) {  // cut the reduction axis, at least four groups a slice
+  if (tiles < kFillTiles && G >= kSplitMinGroups) {
     splits = (256 + tiles - 1) / tiles;
     if (splits > G / 4) splits = G / 4;
     if (splits < 1) splits = 1;
   }
   p.groups_per_split = (G + splits - 1) / splits;
   p.splits = (G + p.groups_per_split - 1) / p.groups_per_split;
+  if (p.splits == 1) return p;   // (no workspace)
   p.ap_bytes = aligned(static_cast<size_t>(p.m_tiles) * kBM * G * kARowBytes);
   p.start_bytes = aligned(static_cast<size_t>(M) * G * sizeof(int));
-  p.partial_bytes = p.splits > 1 ? aligned(static_cast<size_t>(p.splits) * M * N * sizeof(float)) : 0;
+  p.partial_bytes = aligned(static_cast<size_t>(p.splits) * M * N * sizeof(float));
   return p;
 }
 
-template <typename T, int BITS, bool TOKEN, int MT, int NT>
+template <int BITS, bool TOKEN, int MT, int NT>
 int launch_tiles(const A8Args& a, dim3 grid, hipStream_t stream) {
-  auto kernel = wq_gemm_a8_tile_kernel<T, BITS, TOKEN, MT, NT>;
+  auto kernel = wq_gemm_a8_tile_kernel<BITS, TOKEN, MT, NT>;
   constexpr int kLds = Shape<BITS, MT, NT>::kLdsBytes;
   static bool raised = false;  // per instantiation; worst case two threads both set it
   if (!raised) {
@@ -524,26 +493,18 @@ int launch_tiles(const A8Args& a, dim3 grid, hipStream_t stream) {
   return llmq_host::check_launch("wq_gemm_a8_tile_kernel");
 }
 
-template <typename T, int BITS, bool TOKEN>
-int launch_shape(const A8Args& a, const Plan& p, dim3 grid, hipStream_t s) {
-  return p.narrow ? launch_tiles<T, BITS, TOKEN, 1, 1>(a, grid, s) : launch_tiles<T, BITS, TOKEN, 2, 2>(a, grid, s);
-}
-
 template <typename T>
 int run_typed(A8Args& a, const Plan& p, int wformat, bool token, hipStream_t s) {
   const int total = p.m_tiles * p.n_tiles * p.splits;
   const dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8));
   int rc;
-  if (wformat == LLMQ_W_INT4_PACKED) rc = token ? launch_shape<T, 4, true>(a, p, grid, s) : launch_shape<T, 4, false>(a, p, grid, s);
-  else rc = token ? launch_shape<T, 8, true>(a, p, grid, s) : launch_shape<T, 8, false>(a, p, grid, s);
+  if (wformat == LLMQ_W_INT4_PACKED) rc = token ? launch_tiles<4, true, 2, 2>(a, grid, s) : launch_tiles<4, false, 2, 2>(a, grid, s);
+  else rc = token ? launch_tiles<8, true, 2, 2>(a, grid, s) : launch_tiles<8, false, 2, 2>(a, grid, s);
   if (rc) return rc;
-  if (p.splits > 1) {
-    const int64_t count = static_cast<int64_t>(a.M) * a.N;
-    hipLaunchKernelGGL((add_splits_bias_kernel<T>), dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, s,
-                       a.partial, a.bias, static_cast<T*>(a.out), count, a.N, p.splits);
-    return llmq_host::check_launch("add_splits_bias_kernel");
-  }
-  return 0;
+  const int64_t count = static_cast<int64_t>(a.M) * a.N;
+  hipLaunchKernelGGL((add_splits_bias_kernel<T>), dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, s,
+                     a.partial, a.bias, static_cast<T*>(a.out), count, a.N, p.splits);
+  return llmq_host::check_launch("add_splits_bias_kernel");
 }
 
 }  // namespace
@@ -569,18 +530,22 @@ extern "C" int llmq_wq_gemm_a8_fast(const int8_t* a, const float* sx, const void
     return llmq_host::fail_invalid("out must be float32, float16 or bfloat16, got dtype code %d", dtype);
   if (M == 0 || N == 0) return 0;
   if (G == 0) return llmq_host::fail_invalid("a weight with no groups has no reduction axis");
-  if (!a || !sx || !qweight || !wscale || !out || !workspace) return llmq_host::fail_invalid("null tensor pointer");
+  const Plan p = plan_for(M, N, G);
+  const size_t need = p.ap_bytes + p.start_bytes + p.partial_bytes;
+  if (!a || !sx || !qweight || !wscale || !out || (need > 0 && !workspace)) return llmq_host::fail_invalid("null tensor pointer");
   if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(qweight) | reinterpret_cast<uintptr_t>(workspace)) & 15u)
     return llmq_host::fail_invalid("activation, weight and workspace pointers must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool token = sx_groups == 1 && G > 1;
+  if (p.splits == 1) {
+    return llmq_host::gemm_a8_relaxed(a, sx, qweight, wscale, bias_or_null, out, M, N, G, token, out_group, wformat, dtype, s);
+  }
   if ((static_cast<uint64_t>(M) + kBM) * G * kARowBytes >= (1ull << 32) ||
       static_cast<uint64_t>(N) * G * kGroup >= (1ull << 32))
     return llmq_host::fail_invalid("operands of %d x %d and %d x %d are beyond the kernel's 32-bit offsets", M,
                                    G * kGroup, N, G * kGroup);
-  const Plan p = plan_for(M, N, G);
-  const size_t need = p.ap_bytes + p.start_bytes + p.partial_bytes;
   if (workspace_bytes < need)
     return llmq_host::fail_invalid("workspace of %zu bytes is too small, need %zu", workspace_bytes, need);
-  hipStream_t s = static_cast<hipStream_t>(stream);
   uint8_t* ws = static_cast<uint8_t*>(workspace);
   const int64_t n_chunks = static_cast<int64_t>(M) * G * (kARowBytes / 16);
   hipLaunchKernelGGL(act_prep_i8_kernel, dim3(static_cast<unsigned>((n_chunks + 255) / 256)), dim3(256), 0, s,
@@ -590,7 +555,6 @@ extern "C" int llmq_wq_gemm_a8_fast(const int8_t* a, const float* sx, const void
   A8Args args{ws, reinterpret_cast<const int*>(ws + p.ap_bytes), sx, static_cast<const uint8_t*>(qweight), wscale,
               bias_or_null, out, reinterpret_cast<float*>(ws + p.ap_bytes + p.start_bytes), M, N, G, out_group,
               p.m_tiles, p.n_tiles, p.splits, p.groups_per_split};
-  const bool token = sx_groups == 1 && G > 1;
   switch (dtype) {
     case LLMQ_F32: return run_typed<float>(args, p, wformat, token, s);
     case LLMQ_F16: return run_typed<f16_t>(args, p, wformat, token, s);

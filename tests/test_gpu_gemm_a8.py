@@ -239,7 +239,7 @@ def test_fast_form_agrees_with_real_mode_to_fp32_rounding(ext, bits, dtype, m, n
 @pytest.mark.parametrize("bits", [4, 8])
 def test_fast_form_bias_head_scales_and_split(ext, bits):
     torch.manual_seed(3)
-    m, n, k = 70, 192, 2048   # one tile: the reduction axis is split, the bias is added by the second launch
+    m, n, k = 70, 192, 8192   # one tile of long rows: the reduction axis is split, the bias is added by the second launch
     w = (torch.randn(n, k) * 0.015).to(torch.bfloat16)
     x = torch.randn(m, k).to(torch.bfloat16)
     b = torch.randn(n)
@@ -252,7 +252,7 @@ def test_fast_form_bias_head_scales_and_split(ext, bits):
     one = ext.wq_gemm_a8(codes[:, :512].contiguous(), sx[:, :4].contiguous(), q[:, :4].contiguous(),
                          torch.from_numpy(scales[:, :4].copy()).cuda(), b.cuda(), 64, torch.float32, False)
     want_one = oracle.real_linear(to_np(x)[:, :512], canonical[:, :4], scales[:, :4], "f32", 64, 8, to_np(b))
-    assert rel_l2(to_np(one), want_one) <= 1e-6   # four groups: one slice, the bias added in the kernel
+    assert rel_l2(to_np(one), want_one) <= 1e-6   # four groups: nothing is split, the bias added in the kernel
 
 
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
@@ -270,7 +270,7 @@ def test_fast_form_at_llama_8b_mlp_shapes(ext, n, k, m):
 def test_fast_form_one_scale_per_token_small_and_split(ext, bits):
     """One activation scale per token through the fast form on ragged tiles, with a bias, and on a shape whose
     reduction axis is split (the token's scale is applied to each partial tile)."""
-    for m, n, k in ((70, 192, 2048), (130, 300, 768), (3, 40, 128)):
+    for m, n, k in ((70, 192, 8192), (130, 300, 768), (3, 40, 128)):
         torch.manual_seed(k)
         w = (torch.randn(n, k) * 0.015).to(torch.bfloat16)
         x = torch.randn(m, k).to(torch.bfloat16)
