@@ -160,6 +160,19 @@ class KernelQuantExperts(_QuantExperts):
         self._gemv_batched = self._ext.wq_gemv_batched
         self._batched_max_rows = self._ext.wq_gemv_batched_max_rows()
 
+    # (the loaded extension is a module object, which copy and pickle refuse: a copy looks it up again)
+    def __getstate__(self):
+        state = dict(self.__dict__)
+        for name in ("_ext", "_gemv", "_gemv_batched"):
+            state.pop(name, None)
+        return state
+
+    def __setstate__(self, state):
+        super().__setstate__(state)
+        self._ext = load_extension()
+        self._gemv = self._ext.wq_gemv
+        self._gemv_batched = self._ext.wq_gemv_batched
+
     def _probe_silu(self) -> bool:
         probe = torch.linspace(-6.0, 6.0, 25)
         try:

@@ -112,6 +112,19 @@ class KernelQuantLinear(nn.Module):
         self._ext = load_extension()
         self._gemv = self._ext.wq_gemv
 
+    # the loaded extension is a module object, which copy and pickle refuse: a copy (copy.deepcopy(model),
+    # torch.save of the module) carries everything else and looks the extension up again
+    def __getstate__(self):
+        state = dict(self.__dict__)
+        state.pop("_ext", None)
+        state.pop("_gemv", None)
+        return state
+
+    def __setstate__(self, state):
+        super().__setstate__(state)
+        self._ext = load_extension()
+        self._gemv = self._ext.wq_gemv
+
     @classmethod
     def from_linear(cls, linear: nn.Linear, scheme: QuantizationScheme):
         if scheme.weights is None:

@@ -110,6 +110,18 @@ def kernel_runtime(model, max_len: int, kv_bits: int = 8):
 _KEPT_RUNTIMES = 4
 
 
+class _Kept(dict):
+    """What is kept on a model between generate calls (runtimes, captured graphs, the walked module tree). It
+    belongs to that model object only: a deep copy or a pickle of the model carries an empty one (a captured
+    graph can be neither copied nor pickled, and a copy's parameters live elsewhere anyway)."""
+
+    def __deepcopy__(self, memo):
+        return _Kept()
+
+    def __reduce__(self):
+        return (_Kept, ())
+
+
 def _module_tree(model):
     """Every (parent, name, child) edge of the module tree and every place a tensor hangs in it (the
     `_parameters` / `_buffers` dict of a module and the name in it)."""
@@ -122,7 +134,7 @@ def _module_tree(model):
             for name, tensor in holder.items():
                 if tensor is not None:
                     slots.append((holder, name))
-    return {"edges": edges, "slots": slots}
+    return _Kept(edges=edges, slots=slots)
 
 
 def _weights_key(model):
@@ -135,7 +147,7 @@ def _weights_key(model):
     module, e.g. by another oneshot, walks again) and reads the tensors through their holders (a call costs
     ~0.1 ms of the time to first token)."""
     tree = model.__dict__.get("_llmq_module_tree")
-    if tree is None or not all(parent._modules.get(name) is child for parent, name, child in tree["edges"]):
+    if not tree or not all(parent._modules.get(name) is child for parent, name, child in tree["edges"]):
         tree = _module_tree(model)
         model.__dict__["_llmq_module_tree"] = tree
     key = []
@@ -155,8 +167,8 @@ def kept_kernel_runtime(model, max_len: int, kv_bits: int = 8):
     change of any parameter or buffer of the model drops them all."""
     weights = _weights_key(model)
     kept = model.__dict__.get("_llmq_kept_runtimes")
-    if kept is None or kept["weights"] != weights:
-        kept = {"weights": weights, "runtimes": {}}
+    if not kept or kept["weights"] != weights:
+        kept = _Kept(weights=weights, runtimes={})
         model.__dict__["_llmq_kept_runtimes"] = kept
     runtimes = kept["runtimes"]
     key = (max_len, kv_bits)
@@ -177,8 +189,8 @@ def kept_graphed_decoder(model, prompt_tokens: int, new_tokens: int):
     dropped when any parameter or buffer of the model changes."""
     weights = _weights_key(model)
     kept = model.__dict__.get("_llmq_kept_decoders")
-    if kept is None or kept["weights"] != weights:
-        kept = {"weights": weights, "decoders": {}}
+    if not kept or kept["weights"] != weights:
+        kept = _Kept(weights=weights, decoders={})
         model.__dict__["_llmq_kept_decoders"] = kept
     decoders = kept["decoders"]
     key = (prompt_tokens, new_tokens)

@@ -390,6 +390,29 @@ def test_the_bf16_baseline_keeps_its_captured_step_too():
     assert kept_graphed_decoder(base, 12, 10) is not kept
 
 
+def test_a_model_with_kept_steps_can_still_be_copied():
+    """What graphed_generate keeps on a model (runtimes, captured graphs) stays with that object: a deep copy
+    of the model (oneshot callers copy before quantizing) works, starts with nothing kept and generates the
+    same tokens."""
+    import copy
+
+    from llmquant.runtime import graphed_generate
+
+    base = build_model(256, 512, 2, 4, 2, 1024, seed=5)
+    ids = torch.randint(0, 1024, (1, 12), generator=torch.Generator().manual_seed(2)).cuda()
+    out = graphed_generate(base, ids, 8)
+    assert base.__dict__["_llmq_kept_decoders"]["decoders"]
+    twin = copy.deepcopy(base)
+    assert not twin.__dict__.get("_llmq_kept_decoders") and not twin.__dict__.get("_llmq_module_tree")
+    assert torch.equal(graphed_generate(twin, ids, 8), out)
+    _, kernel = quantized_pair(base)
+    fast = graphed_generate(kernel, ids, 8, kv_bits=8)
+    assert kernel.__dict__["_llmq_kept_runtimes"]["runtimes"]
+    twin = copy.deepcopy(kernel)
+    assert not twin.__dict__.get("_llmq_kept_runtimes")
+    assert torch.equal(graphed_generate(twin, ids, 8, kv_bits=8), fast)
+
+
 def test_measure_latency_reports_the_reference_keys():
     """llmquant/eval/evaluate.py:167-223 on a small model: graphed HF path for bf16, the fused
     integer-KV runtime for the kernel-mode model."""
