@@ -369,6 +369,17 @@ int llmq_argmax_row(const void* x, int n, int64_t* out_index, int dtype, llmq_st
 int llmq_argmax_advance(const void* x, int n, int64_t* out_index, int64_t* token_or_null,
                         int64_t* step64_or_null, int32_t* step32_or_null, int dtype,
                         llmq_stream_t stream);
+/* llmq_argmax_advance over 32 workgroups instead of one (the workgroup that finishes last picks among the
+ * slices' first maxima: the same index), and, when embed_or_null is given, the next step's embedding lookup
+ * as well: hidden_out[0 .. hidden_dim) = embed[index * hidden_dim ..], what the reference's loop does with
+ * model.embed_tokens on the token it feeds back (llmquant/runtime/graph_decode.py:131-140). `workspace`:
+ * llmq_argmax_workspace_bytes() bytes, 16-byte aligned, zero before the first call; every call leaves it
+ * ready for the next; calls that share it must not overlap. x must be 16-byte aligned. */
+size_t llmq_argmax_workspace_bytes(void);
+int llmq_argmax_advance_embed(const void* x, int n, int64_t* out_index, int64_t* token_or_null,
+                              int64_t* step64_or_null, int32_t* step32_or_null, const void* embed_or_null,
+                              void* hidden_out_or_null, int hidden_dim, void* workspace, int dtype,
+                              llmq_stream_t stream);
 
 #ifdef __cplusplus
 }

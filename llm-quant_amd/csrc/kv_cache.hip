@@ -863,6 +863,97 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const T* __restrict__ 
   }
 }
 
+// The same over kArgmaxBlocks workgroups, each taking a contiguous slice of the row; the workgroup that
+// finishes last (a ticket from one atomic counter; nobody waits) picks the winner among the slices' first
+// maxima, does the loop's bookkeeping and, when asked, copies the winner's row of the embedding table to
+// `hidden_out`: the next decode step then starts at its first GEMV instead of at an embedding launch.
+// part_val / part_idx / counter: kArgmaxBlocks floats, as many ints and one arrival counter that is zero before
+// the first call and set back to zero by every call.
+constexpr int kArgmaxBlocks = 32;
+template <typename T>
+__global__ __launch_bounds__(256) void argmax_split_kernel(const T* __restrict__ x, const int n, int64_t* __restrict__ out,
+                                                           int64_t* __restrict__ token, int64_t* __restrict__ step64,
+                                                           int32_t* __restrict__ step32, const T* __restrict__ embed,
+                                                           T* __restrict__ hidden_out, const int hidden,
+                                                           float* part_val, int* part_idx, unsigned* counter) {
+  __shared__ float s_val[4];
+  __shared__ int s_idx[4];
+  __shared__ int s_winner;   // -1: this workgroup is not the last one
+  constexpr int V = Pack<T>::N;
+  // slices of whole 16-byte packets (the row's base is 16-byte aligned: checked by the caller)
+  const int per = ((n + kArgmaxBlocks - 1) / kArgmaxBlocks + V - 1) / V * V;
+  const int begin = min(static_cast<int>(blockIdx.x) * per, n), end = min(begin + per, n);
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  const int n_vec = (end - begin) / V;
+  constexpr int kFlight = 2;
+  for (int p0 = threadIdx.x; p0 < n_vec; p0 += kFlight * blockDim.x) {
+    u32x4 raw[kFlight];
+#pragma unroll
+    for (int u = 0; u < kFlight; ++u) {
+      const int p = p0 + u * blockDim.x;
+      raw[u] = p < n_vec ? load16(x + begin + static_cast<int64_t>(p) * V) : u32x4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int u = 0; u < kFlight; ++u) {
+      const int p = p0 + u * blockDim.x;
+      if (p >= n_vec) break;
+      float f[V];
+      Pack<T>::unpack(raw[u], f);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        if (f[e] > best) { best = f[e]; best_i = begin + p * V + e; }
+      }
+    }
+  }
+  for (int i = begin + n_vec * V + threadIdx.x; i < end; i += blockDim.x) {
+    const float v = to_float(x[i]);
+    if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+  }
+  auto take = [&](float ov, int oi) {
+    if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+  };
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) take(__shfl_xor(best, off, kWave), __shfl_xor(best_i, off, kWave));
+  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+  if (lane == 0) { s_val[wv] = best; s_idx[wv] = best_i; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < static_cast<int>(blockDim.x) / kWave; ++w) take(s_val[w], s_idx[w]);
+    __hip_atomic_store(part_val + blockIdx.x, best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(part_idx + blockIdx.x, best_i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __threadfence();   // the slice's result is visible to the other XCDs before the ticket is
+    const unsigned ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    s_winner = ticket == gridDim.x - 1 ? 0 : -1;
+  }
+  __syncthreads();
+  if (s_winner < 0) return;
+  // the last workgroup: every slice's result is in memory
+  if (wv == 0) {
+    best = -INFINITY, best_i = 0x7fffffff;
+    if (lane < static_cast<int>(gridDim.x)) {
+      best = __hip_atomic_load(part_val + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      best_i = __hip_atomic_load(part_idx + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) take(__shfl_xor(best, off, kWave), __shfl_xor(best_i, off, kWave));
+    if (lane == 0) {
+      const int64_t winner = best_i == 0x7fffffff ? 0 : best_i;
+      out[0] = winner;
+      if (token != nullptr) token[0] = winner;
+      if (step64 != nullptr) step64[0] += 1;
+      if (step32 != nullptr) step32[0] += 1;
+      __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
+      s_winner = static_cast<int>(winner);
+    }
+  }
+  __syncthreads();
+  if (embed != nullptr) {
+    const T* row = embed + static_cast<int64_t>(s_winner) * hidden;
+    for (int i = threadIdx.x * V; i < hidden; i += blockDim.x * V) store16(hidden_out + i, load16(row + i));
+  }
+}
+
 int splits_for(int t_max) {
   int s = (t_max + 63) / 64;
   if (s > 64) s = 64;
@@ -1180,6 +1271,42 @@ extern "C" int llmq_argmax_advance(const void* x, int n, int64_t* out_index, int
   }
 #undef LLMQ_ARGMAX
   return llmq_host::check_launch("argmax_row_kernel");
+}
+
+extern "C" size_t llmq_argmax_workspace_bytes(void) { return kArgmaxBlocks * 8 + 256; }
+
+extern "C" int llmq_argmax_advance_embed(const void* x, int n, int64_t* out_index, int64_t* token_or_null,
+                                         int64_t* step64_or_null, int32_t* step32_or_null,
+                                         const void* embed_or_null, void* hidden_out_or_null, int hidden_dim,
+                                         void* workspace, int dtype, llmq_stream_t stream) {
+  if (n <= 0) return llmq_host::fail_invalid("argmax of an empty row");
+  if (!x || !out_index || !workspace) return llmq_host::fail_invalid("null tensor pointer");
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(workspace)) & 15u)
+    return llmq_host::fail_invalid("the row and the workspace must be 16-byte aligned");
+  const int packet = dtype == LLMQ_F32 ? 4 : 8;
+  if (embed_or_null != nullptr) {
+    if (!hidden_out_or_null || hidden_dim <= 0 || hidden_dim % packet != 0)
+      return llmq_host::fail_invalid("the embedding hand-off needs an output row and a width that is a multiple of %d, got %d",
+                                     packet, hidden_dim);
+    if ((reinterpret_cast<uintptr_t>(embed_or_null) | reinterpret_cast<uintptr_t>(hidden_out_or_null)) & 15u)
+      return llmq_host::fail_invalid("embedding table and output row must be 16-byte aligned");
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* part_val = static_cast<float*>(workspace);
+  int* part_idx = reinterpret_cast<int*>(part_val + kArgmaxBlocks);
+  unsigned* counter = reinterpret_cast<unsigned*>(part_idx + kArgmaxBlocks);
+#define LLMQ_ARGMAX(T)                                                                                              \
+  hipLaunchKernelGGL((argmax_split_kernel<T>), dim3(kArgmaxBlocks), dim3(256), 0, s, static_cast<const T*>(x), n,   \
+                     out_index, token_or_null, step64_or_null, step32_or_null, static_cast<const T*>(embed_or_null), \
+                     static_cast<T*>(hidden_out_or_null), hidden_dim, part_val, part_idx, counter)
+  switch (dtype) {
+    case LLMQ_F32: LLMQ_ARGMAX(float); break;
+    case LLMQ_F16: LLMQ_ARGMAX(f16_t); break;
+    case LLMQ_BF16: LLMQ_ARGMAX(bf16_t); break;
+    default: return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+  }
+#undef LLMQ_ARGMAX
+  return llmq_host::check_launch("argmax_split_kernel");
 }
 
 extern "C" int llmq_argmax_row(const void* x, int n, int64_t* out_index, int dtype, llmq_stream_t stream) {

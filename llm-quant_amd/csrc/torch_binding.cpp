@@ -1027,6 +1027,42 @@ at::Tensor argmax_row(const at::Tensor& x) {
   return out;
 }
 
+// argmax_advance over 32 workgroups, and the winner's row of the embedding table copied to hidden_out (both or
+// neither of embed / hidden_out). workspace: int32 zeros of argmax_workspace_ints() elements, kept by the caller.
+at::Tensor argmax_advance_embed(const at::Tensor& x, at::Tensor& token, at::Tensor& step64, at::Tensor& step32,
+                                const c10::optional<at::Tensor>& embed, const c10::optional<at::Tensor>& hidden_out,
+                                at::Tensor& workspace) {
+  TORCH_CHECK(x.is_cuda() && x.is_contiguous() && x.numel() > 0, "x must be a non-empty contiguous CUDA tensor");
+  TORCH_CHECK(token.is_cuda() && token.scalar_type() == at::kLong && token.numel() == 1, "token must be one int64");
+  TORCH_CHECK(step64.is_cuda() && step64.scalar_type() == at::kLong && step64.numel() == 1, "step64 must be one int64");
+  TORCH_CHECK(step32.is_cuda() && step32.scalar_type() == at::kInt && step32.numel() == 1, "step32 must be one int32");
+  TORCH_CHECK(workspace.is_cuda() && workspace.is_contiguous() &&
+                  static_cast<size_t>(workspace.numel() * workspace.element_size()) >= llmq_argmax_workspace_bytes(),
+              "workspace must be a contiguous CUDA tensor of at least ", llmq_argmax_workspace_bytes(), " bytes");
+  const bool hand_off = embed.has_value() && embed->defined();
+  TORCH_CHECK(hand_off == (hidden_out.has_value() && hidden_out->defined()), "embed and hidden_out go together");
+  int64_t hidden = 0;
+  if (hand_off) {
+    TORCH_CHECK(embed->is_cuda() && embed->is_contiguous() && embed->dim() == 2 && embed->scalar_type() == x.scalar_type(),
+                "embed must be a contiguous [vocab, hidden] CUDA tensor of x's dtype");
+    TORCH_CHECK(embed->size(0) >= x.numel(), "embed has ", embed->size(0), " rows for ", x.numel(), " logits");
+    hidden = embed->size(1);
+    TORCH_CHECK(hidden_out->is_cuda() && hidden_out->is_contiguous() && hidden_out->numel() == hidden &&
+                    hidden_out->scalar_type() == x.scalar_type(),
+                "hidden_out must be a contiguous CUDA tensor of ", hidden, " elements of x's dtype");
+  }
+  const int dtype = dtype_code(x, "x");
+  auto out = at::empty({1}, x.options().dtype(at::kLong));
+  const c10::OptionalDeviceGuard guard(at::device_of(x));
+  check_rc(llmq_argmax_advance_embed(x.const_data_ptr(), static_cast<int>(x.numel()), out.mutable_data_ptr<int64_t>(),
+                                     token.mutable_data_ptr<int64_t>(), step64.mutable_data_ptr<int64_t>(),
+                                     step32.mutable_data_ptr<int32_t>(), hand_off ? embed->const_data_ptr() : nullptr,
+                                     hand_off ? hidden_out->mutable_data_ptr() : nullptr, static_cast<int>(hidden),
+                                     workspace.mutable_data_ptr(), dtype, current_stream(x)),
+           "argmax_advance_embed");
+  return out;
+}
+
 // argmax_row plus: token <- index, step64 += 1, step32 += 1 (one-element int64 / int64 / int32 device tensors).
 at::Tensor argmax_advance(const at::Tensor& x, at::Tensor& token, at::Tensor& step64, at::Tensor& step32) {
   TORCH_CHECK(x.is_cuda() && x.is_contiguous() && x.numel() > 0, "x must be a non-empty contiguous CUDA tensor");
@@ -1146,6 +1182,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("partials"), py::arg("n_splits"), py::arg("head_dim"), py::arg("qweight"), py::arg("wscale"),
         py::arg("out_group") = 0, py::arg("in_head_dim") = 0, py::arg("residual") = py::none(),
         py::arg("out_dtype") = at::kBFloat16);
+  m.def("argmax_advance_embed", &argmax_advance_embed,
+        "argmax_advance over 32 workgroups; with embed / hidden_out also hidden_out <- embed[index]", py::arg("x"),
+        py::arg("token"), py::arg("step64"), py::arg("step32"), py::arg("embed") = py::none(),
+        py::arg("hidden_out") = py::none(), py::arg("workspace"));
+  m.def("argmax_workspace_ints", []() { return static_cast<int64_t>((llmq_argmax_workspace_bytes() + 3) / 4); },
+        "elements of the int32 zeros tensor argmax_advance_embed takes as workspace");
   m.def("argmax_advance", &argmax_advance, "argmax_row, then token <- index, step64 += 1, step32 += 1",
         py::arg("x"), py::arg("token"), py::arg("step64"), py::arg("step32"));
   m.def("abi_version", []() { return llmq_abi_version(); });

@@ -111,6 +111,10 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_argmax_row.restype = c_int
     lib.llmq_argmax_advance.argtypes = [c_p, c_int, c_p, c_p, c_p, c_p, c_int, c_p]
     lib.llmq_argmax_advance.restype = c_int
+    lib.llmq_argmax_advance_embed.argtypes = [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_int, c_p, c_int, c_p]
+    lib.llmq_argmax_advance_embed.restype = c_int
+    lib.llmq_argmax_workspace_bytes.argtypes = []
+    lib.llmq_argmax_workspace_bytes.restype = ctypes.c_size_t
     lib.llmq_wq_gemm_a8.argtypes = [c_p] * 6 + [c_int] * 7 + [c_p]
     lib.llmq_wq_gemm_a8.restype = c_int
     lib.llmq_wq_gemm_a8_fast.argtypes = [c_p] * 7 + [ctypes.c_size_t] + [c_int] * 8 + [c_p]

@@ -122,6 +122,16 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
             raise ValueError("the fused decode step needs a kernel-mode lm_head")
         self.final_norm = model.model.norm.weight.detach().contiguous()
         self.final_eps = model.model.norm.variance_epsilon
+        # The launch that picks a step's token also looks up that token's embedding for the next step
+        # (llmq_argmax_advance_embed), so a step starts at its first GEMV. Plain nn.Embedding tables of the
+        # model's dtype only; anything else keeps the embedding module's own launch.
+        table = model.model.embed_tokens
+        plain = (type(table) is torch.nn.Embedding and table.max_norm is None and table.weight.is_contiguous()
+                 and table.weight.dtype in (torch.bfloat16, torch.float16, torch.float32)
+                 and table.weight.shape[1] % 8 == 0 and table.weight.shape[0] >= head.qdata.shape[0])
+        self._embed_table = table.weight.detach() if plain else None
+        self._hidden0 = torch.zeros(1, table.weight.shape[1], dtype=table.weight.dtype, device=self.device)
+        self._argmax_ws = torch.zeros(self._ext.argmax_workspace_ints(), dtype=torch.int32, device=self.device)
 
     # ---- the prompt pass: q|k|v and gate|up as one projection each ----------------------------------
     def _project(self, x, fused):
@@ -157,7 +167,8 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         if not decode:
             return super()._forward(token_ids, cos, sin, decode)
         ext, cache = self._ext, self.cache
-        hidden = self.model.model.embed_tokens(token_ids)  # [1, hidden]
+        # (the row _set_step_inputs or the previous step's token pick left for this token)
+        hidden = self._hidden0 if self._embed_table is not None else self.model.model.embed_tokens(token_ids)
         for index, f in enumerate(self.fused_layers):
             qkv = ext.wq_gemv_fused(hidden, f["qkv"].qdata, f["qkv"].wscale, f["qkv"].out_group, PRO_RMSNORM,
                                     f["norm1"], f["eps1"], 0, None)
@@ -189,8 +200,17 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         return ext.wq_gemv_fused(hidden, head.qdata, head.wscale, head.out_group, PRO_RMSNORM, self.final_norm,
                                  self.final_eps, 0, None)
 
+    def _set_step_inputs(self, token, position: int):
+        super()._set_step_inputs(token, position)
+        if self._embed_table is not None:
+            self._hidden0.copy_(self.model.model.embed_tokens(self.token))
+
     def _step(self):
         logits = self._forward(self.token, None, None, decode=True)
-        # greedy pick, next input token and both position counters in one launch
-        nxt = self._ext.argmax_advance(logits, self.token, self.pos_index, self.cache.position)
+        # greedy pick, next input token, both position counters and the next step's embedding row in one launch
+        if self._embed_table is not None and logits.dtype == self._embed_table.dtype:
+            nxt = self._ext.argmax_advance_embed(logits, self.token, self.pos_index, self.cache.position,
+                                                 self._embed_table, self._hidden0, self._argmax_ws)
+        else:
+            nxt = self._ext.argmax_advance(logits, self.token, self.pos_index, self.cache.position)
         return logits, nxt

@@ -229,6 +229,40 @@ def test_argmax_advance_does_the_loop_bookkeeping(ext):
     assert got.item() == want and token.item() == want and step64.item() == 43 and step32.item() == 43
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("n", [128256, 5000, 37, 8])
+def test_argmax_advance_embed_picks_the_same_token_and_hands_over_its_row(ext, dtype, n):
+    """The 32-workgroup form against the one-workgroup one and torch: first maximum among ties that fall in
+    different slices, the loop's bookkeeping, the winner's embedding row, and a workspace left ready for the
+    next call (three calls in a row on different rows)."""
+    gen = torch.Generator().manual_seed(n)
+    table = torch.randn(n, 64, generator=gen).to(dtype).cuda()
+    hidden = torch.zeros(1, 64, dtype=dtype, device="cuda")
+    ws = torch.zeros(ext.argmax_workspace_ints(), dtype=torch.int32, device="cuda")
+    token = torch.zeros(1, dtype=torch.long, device="cuda")
+    step64 = torch.tensor([7], dtype=torch.long, device="cuda")
+    step32 = torch.tensor([7], dtype=torch.int32, device="cuda")
+    for call in range(3):
+        x = torch.randn(1, n, generator=gen).to(dtype)
+        if call == 1 and n > 100:   # equal maxima far apart: the first one wins
+            x[0, [n // 3, n // 3 + 1, n - 2]] = 9.0
+        x = x.cuda()
+        got = ext.argmax_advance_embed(x, token, step64, step32, table, hidden, ws)
+        want = ext.argmax_row(x).item()
+        assert want == x.float().argmax().item() or call == 1
+        assert got.item() == want and token.item() == want
+        assert step64.item() == 8 + call and step32.item() == 8 + call
+        assert torch.equal(hidden[0], table[want])
+        assert ws[64].item() == 0   # the arrival counter, behind the 32 + 32 slice results
+    # without the hand-off: only the pick and the bookkeeping
+    got = ext.argmax_advance_embed(x, token, step64, step32, None, None, ws)
+    assert got.item() == want and step64.item() == 11
+    with pytest.raises(RuntimeError, match="go together"):
+        ext.argmax_advance_embed(x, token, step64, step32, table, None, ws)
+    with pytest.raises(RuntimeError, match="workspace"):
+        ext.argmax_advance_embed(x, token, step64, step32, None, None, ws[:8])
+
+
 def test_fused_runtime_equals_the_unfused_one():
     """Whole decode steps on a small model: fused and operation-by-operation runtimes give the
     same logits to the bit (hidden 512: the variance reduction happens to agree), the same
