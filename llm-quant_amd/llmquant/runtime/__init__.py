@@ -1,10 +1,10 @@
 """Running a quantized model: the integer KV cache, the kernel decode runtime, graphed decode."""
 
-from llmquant.runtime.graph_decode import (WARMUP_CALLS, GraphedDecoder, KernelDecoder, can_graph,
+from llmquant.runtime.graph_decode import (WARMUP_CALLS, GraphedDecoder, KernelDecoder, can_graph, drop_kept,
                                            graphed_generate, kernel_runtime)
 from llmquant.runtime.kv_cache import KernelQuantCache, make_kernel_cache_factory
 from llmquant.runtime.llama_decode import LlamaKernelRuntime
 from llmquant.runtime.llama_fused import LlamaFusedRuntime
 
 __all__ = ["WARMUP_CALLS", "GraphedDecoder", "KernelDecoder", "KernelQuantCache", "LlamaFusedRuntime", "LlamaKernelRuntime",
-           "can_graph", "graphed_generate", "kernel_runtime", "make_kernel_cache_factory"]
+           "can_graph", "drop_kept", "graphed_generate", "kernel_runtime", "make_kernel_cache_factory"]

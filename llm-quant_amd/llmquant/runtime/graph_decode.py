@@ -20,8 +20,8 @@ import torch
 from llmquant.runtime.llama_decode import WARMUP_CALLS, LlamaKernelRuntime
 from llmquant.runtime.llama_fused import LlamaFusedRuntime
 
-__all__ = ["GraphedDecoder", "KernelDecoder", "WARMUP_CALLS", "can_graph", "graphed_generate", "kept_graphed_decoder",
-           "kept_kernel_runtime", "kernel_runtime"]
+__all__ = ["GraphedDecoder", "KernelDecoder", "WARMUP_CALLS", "can_graph", "drop_kept", "graphed_generate",
+           "kept_graphed_decoder", "kept_kernel_runtime", "kernel_runtime"]
 
 
 def _on_gpu(model) -> bool:
@@ -179,6 +179,14 @@ def kept_kernel_runtime(model, max_len: int, kv_bits: int = 8):
             runtimes.pop(next(iter(runtimes)))  # the least recently used
     runtimes[key] = runtime  # most recently used last
     return runtime
+
+
+def drop_kept(model) -> None:
+    """Forget everything graphed_generate keeps on `model` (up to four runtimes per side, each with its KV cache
+    and the memory pool of its captured graph; they reference the model and the model them, so without this
+    they live until the cycle collector finds the model unreachable)."""
+    for name in ("_llmq_kept_runtimes", "_llmq_kept_decoders", "_llmq_module_tree"):
+        model.__dict__.pop(name, None)
 
 
 def kept_graphed_decoder(model, prompt_tokens: int, new_tokens: int):

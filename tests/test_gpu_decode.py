@@ -411,6 +411,11 @@ def test_a_model_with_kept_steps_can_still_be_copied():
     twin = copy.deepcopy(kernel)
     assert not twin.__dict__.get("_llmq_kept_runtimes")
     assert torch.equal(graphed_generate(twin, ids, 8, kv_bits=8), fast)
+    from llmquant.runtime import drop_kept
+
+    drop_kept(twin)
+    assert not any(name.startswith("_llmq_kept") or name == "_llmq_module_tree" for name in twin.__dict__)
+    assert torch.equal(graphed_generate(twin, ids, 8, kv_bits=8), fast)
 
 
 def test_measure_latency_reports_the_reference_keys():
