@@ -10,28 +10,27 @@
 // dtype and calls the BLAS library for M > 4, llmquant/quantizers/kernel.py:68-79,88-91: nine times the
 // int4 codes' bytes through HBM per call, and a second rounding per weight.)
 //
-// Shape. A workgroup of four waves owns a 128 (m) x 256 (n) tile of the output; every wave owns 64 of
-// the 256 columns and all 128 rows: 4 x 2 MFMA tiles of 32 x 32 (v_mfma_f32_32x32x16_bf16), eight
-// k-steps of 16 per group. What bounds a tiled GEMM on this chip is LDS bandwidth (one 16-byte operand
-// read per lane per MFMA is all the LDS delivers), so only the activation goes through LDS, shared by
-// the four waves, and each operand read feeds two MFMAs; the weights never touch LDS: a lane reads the
-// codes of its own column straight from HBM in operand layout (32 bytes of int4 or 64 of int8 per group)
-// and converts them in registers.
+// Shape. A workgroup of eight waves (two per SIMD) owns a 128 (m) x 256 (n) tile of the output; every wave owns
+// 32 of the 256 columns and all 128 rows: 4 x 1 MFMA tiles of 32 x 32 (v_mfma_f32_32x32x16_bf16), eight
+// k-steps of 16 per group. A lane converts the codes of one column only, and each converted operand feeds four
+// MFMAs (with 64 x 64 per wave two waves converted the same codes: measured 3-4 % slower on the large shapes).
+// Everything reaches LDS straight from global memory (global_load_lds_dwordx4, 1 KB per wave instruction,
+// XOR-swizzled by row so that the operand reads are conflict-free), three stages deep for int4, two for int8:
+// the activation tile, the raw codes of the 256 weight rows, the activation-sum records and the group's scales.
+// The workgroup meets once per group, before the last k-step, and the next group's operands are read from LDS
+// behind that barrier.
 //
 // Codes become bf16 without a conversion instruction: a nibble n = code + 8 placed in the mantissa of
 // 16.0 (bits 0x4180 | n << 3) IS the bf16 value 16 + n, two nibbles per AND-OR (int8: code + 128 through
 // v_cvt_f32_ubyte, whose upper half is the bf16 value). The matrix core therefore sums x * (code + B),
-// B = 24 or 128, and B * sum_k x is taken out again per group. That correction is a rank-one term,
-// -B * wscale[n, g] * xsum[m, g], and it too runs on the matrix core: both factors are cut into three
-// bf16 pieces and the six significant cross products fill one more k-step, accumulated straight into
-// the running total.
+// B = 24 or 128, and B * sum_k x is taken out again per group by one more k-step in front of the eight: the
+// group's activation sum, cut into three bf16 pieces, against the constant -B. The fp32 group sum is then
+// folded into the fp32 total with one multiply-add by the group's weight scale.
 //
-// The activation is prepared once per call by act_prep_kernel: within every 16-byte chunk the eight
-// values are reordered to (0, 4, 1, 5, 2, 6, 3, 7), the order in which the AND-OR above leaves the
-// codes (a sum does not care about the order of its terms, as long as both operands agree), and the
-// per-group sums are cut into their bf16 pieces. The GEMM then moves activation tiles from global
-// memory to LDS without passing through registers (global_load_lds_dwordx4), XOR-swizzled by row so the
-// operand reads are conflict-free.
+// The activation is prepared once per call by act_prep_kernel: rows padded to whole tiles, within every
+// 16-byte chunk the eight values reordered to (0, 4, 1, 5, 2, 6, 3, 7), the order in which the AND-OR above
+// leaves the codes (a sum does not care about the order of its terms, as long as both operands agree), and
+// the per-group sums written as records of bf16 pieces.
 //
 // Small N: a split of the reduction axis across workgroups, fp32 partial tiles in a workspace, added in a
 // fixed order by a second launch (the result does not depend on which workgroup finished first).
@@ -48,10 +47,10 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kGroup = 128;
 constexpr int kBM = 128;            // activation rows per workgroup
-constexpr int kWaveM = 64;          // activation rows per wave
-constexpr int kWaveN = 64;          // weight rows (output columns) per wave
-constexpr int kWaves = 8;           // 2 (rows) x 4 (columns)
-constexpr int kBN = kWaveN * 4;
+constexpr int kWaveM = 128;         // activation rows per wave
+constexpr int kWaveN = 32;          // weight rows (output columns) per wave
+constexpr int kWaves = 8;           // 1 (rows) x 8 (columns)
+constexpr int kBN = kWaveN * 8;
 constexpr int kThreads = kWaves * kWave;
 constexpr int kRowBytes = kGroup * 2;          // one activation row of one group
 constexpr int kTileBytes = kBM * kRowBytes;    // 32 KB
@@ -178,7 +177,7 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   const int sp = logical / (a.m_tiles * a.n_tiles);
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  const int wm = wv & 1, wn = wv >> 1;  // the wave's half of the rows, quarter of the columns
+  const int wm = 0, wn = wv;  // every wave all the rows, an eighth of the columns
   const int lm = lane & 31, lh = lane >> 5;
   const int m0 = mt * kBM, n0 = nt * kBN;
   const int g_begin = sp * a.groups_per_split;
@@ -250,8 +249,8 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   constexpr int kDmaPerWave = kXInstr + kCodeInstr + 1;   // waves 0..5; waves 6, 7: one fewer
 
   // ---- LDS -> operands ----------------------------------------------------------------------------------
-  // activation operand of k-step j, row tile mi: row wm*64 + mi*32 + lm, chunk (8 lh + j) ^ (lm & 15)
-  const uint32_t a_base = (wm * 64 + lm) * kRowBytes + (((8 * lh) ^ (lm & 15)) << 4);  // k-step j: a_base ^ (j << 4)
+  // activation operand of k-step j, row tile mi: row mi*32 + lm, chunk (8 lh + j) ^ (lm & 15)
+  const uint32_t a_base = (wm * kWaveM + lm) * kRowBytes + (((8 * lh) ^ (lm & 15)) << 4);  // k-step j: a_base ^ (j << 4)
   // this lane's codes of a group: weight row wn*64 + ni*32 + lm, k in [64 lh, 64 lh + 64): 16-byte chunks
   // lh * kRawLoads + q, at c_base ^ (q << 4)
   constexpr int kRawLoads = BITS == 4 ? 2 : 4;
@@ -292,7 +291,7 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
     const uint8_t* stage = smem + st * kStageBytes<BITS>;
 #pragma unroll
     for (int mi = 0; mi < kMT; ++mi)
-      rec[mi] = read16(stage, kTileBytes + kCodeTileBytes<BITS> + (wm * 64 + mi * 32 + lm) * 16);
+      rec[mi] = read16(stage, kTileBytes + kCodeTileBytes<BITS> + (wm * kWaveM + mi * 32 + lm) * 16);
 #pragma unroll
     for (int ni = 0; ni < kNT; ++ni)
 #pragma unroll
@@ -318,8 +317,9 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   for (int g = g_begin; g < g_end; ++g) {
     const uint8_t* stage = smem + st * kStageBytes<BITS>;
     const int st_next = st + 1 == kStages<BITS> ? 0 : st + 1;
-    const float scale_now[kNT] = {scale[0], scale[1]};
-    static_assert(kNT == 2, "scale_now");
+    float scale_now[kNT];
+#pragma unroll
+    for (int ni = 0; ni < kNT; ++ni) scale_now[ni] = scale[ni];
 
     // The group's sums start at -B * xsum[m] (one k-step: the three bf16 pieces of the activation sum
     // against the constant -B; the upper half of the wave, k' 8..15, multiplies zeros), then take the
@@ -382,7 +382,7 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
       for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          const int m = m0 + wm * kWaveM + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
           if (m < a.M && n < a.N) out[static_cast<int64_t>(m) * a.N + n] = from_float<bf16_t>(total[mi][ni][r]);
         }
     }
@@ -395,7 +395,7 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
       for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          const int m = m0 + wm * kWaveM + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
           if (m < a.M && n < a.N) part[static_cast<int64_t>(m) * a.N + n] = total[mi][ni][r];
         }
     }
