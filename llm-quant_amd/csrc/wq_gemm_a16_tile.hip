@@ -251,7 +251,7 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   // ---- LDS -> operands ----------------------------------------------------------------------------------
   // activation operand of k-step j, row tile mi: row mi*32 + lm, chunk (8 lh + j) ^ (lm & 15)
   const uint32_t a_base = (wm * kWaveM + lm) * kRowBytes + (((8 * lh) ^ (lm & 15)) << 4);  // k-step j: a_base ^ (j << 4)
-  // this lane's codes of a group: weight row wn*64 + ni*32 + lm, k in [64 lh, 64 lh + 64): 16-byte chunks
+  // this lane's codes of a group: weight row wn*32 + lm, k in [64 lh, 64 lh + 64): 16-byte chunks
   // lh * kRawLoads + q, at c_base ^ (q << 4)
   constexpr int kRawLoads = BITS == 4 ? 2 : 4;
   uint32_t c_base[kNT];
