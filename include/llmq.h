@@ -369,6 +369,16 @@ int llmq_argmax_row(const void* x, int n, int64_t* out_index, int dtype, llmq_st
 int llmq_argmax_advance(const void* x, int n, int64_t* out_index, int64_t* token_or_null,
                         int64_t* step64_or_null, int32_t* step32_or_null, int dtype,
                         llmq_stream_t stream);
+/* Causal grouped-query attention of a prompt: out[i, h, :] = softmax over j <= i of (scale * q[i, h, :] .
+ * k[h / (q_heads / kv_heads), j, :]) times v, what the reference's prompt pass gets from transformers'
+ * attention on the rotated queries and the K / V its FakeQuantCache returns (llmquant/quantizers/fake.py:39-55;
+ * the reference has no kernel of its own for it). q: [tokens, q_heads, head_dim]; k, v: [kv_heads, tokens,
+ * head_dim] (the dequantized cache values, as llmq_rope_kv_append hands them back); out: [tokens, q_heads,
+ * head_dim]. float16 or bfloat16, head_dim 64 or 128, 16-byte aligned; fp32 accumulation, probabilities rounded
+ * to `dtype` before they meet v. */
+int llmq_prefill_attention(const void* q, const void* k, const void* v, void* out, int tokens, int q_heads,
+                           int kv_heads, int head_dim, float scale, int dtype, llmq_stream_t stream);
+
 /* llmq_argmax_advance over 32 workgroups instead of one (the workgroup that finishes last picks among the
  * slices' first maxima: the same index), and, when embed_or_null is given, the next step's embedding lookup
  * as well: hidden_out[0 .. hidden_dim) = embed[index * hidden_dim ..], what the reference's loop does with

@@ -1027,6 +1027,28 @@ at::Tensor argmax_row(const at::Tensor& x) {
   return out;
 }
 
+// Causal grouped-query attention of a prompt. q [tokens, q_heads, head_dim]; k, v [kv_heads, tokens, head_dim]
+// (contiguous, fp16 / bf16, head_dim 64 or 128) -> [tokens, q_heads * head_dim].
+at::Tensor prefill_attention(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, double scale) {
+  TORCH_CHECK(q.is_cuda() && k.is_cuda() && v.is_cuda(), "q, k, v must be CUDA tensors");
+  TORCH_CHECK(q.dim() == 3 && k.dim() == 3 && v.dim() == 3, "q must be [tokens, q_heads, head_dim], k and v [kv_heads, tokens, head_dim]");
+  TORCH_CHECK(q.scalar_type() == k.scalar_type() && q.scalar_type() == v.scalar_type(), "q, k, v must share a dtype");
+  TORCH_CHECK(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, "q, k, v must be float16 or bfloat16");
+  const auto qc = q.contiguous(), kc = k.contiguous(), vc = v.contiguous();
+  const int64_t tokens = qc.size(0), q_heads = qc.size(1), head_dim = qc.size(2), kv_heads = kc.size(0);
+  TORCH_CHECK(kc.size(1) == tokens && kc.size(2) == head_dim && vc.sizes() == kc.sizes(),
+              "k and v must be [kv_heads, ", tokens, ", ", head_dim, "]");
+  auto out = at::empty({tokens, q_heads * head_dim}, qc.options());
+  if (tokens == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(qc));
+  check_rc(llmq_prefill_attention(qc.const_data_ptr(), kc.const_data_ptr(), vc.const_data_ptr(), out.mutable_data_ptr(),
+                                  static_cast<int>(tokens), static_cast<int>(q_heads), static_cast<int>(kv_heads),
+                                  static_cast<int>(head_dim), static_cast<float>(scale), dtype_code(qc, "q"),
+                                  current_stream(qc)),
+           "prefill_attention");
+  return out;
+}
+
 // argmax_advance over 32 workgroups, and the winner's row of the embedding table copied to hidden_out (both or
 // neither of embed / hidden_out). workspace: int32 zeros of argmax_workspace_ints() elements, kept by the caller.
 at::Tensor argmax_advance_embed(const at::Tensor& x, at::Tensor& token, at::Tensor& step64, at::Tensor& step32,
@@ -1182,6 +1204,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("partials"), py::arg("n_splits"), py::arg("head_dim"), py::arg("qweight"), py::arg("wscale"),
         py::arg("out_group") = 0, py::arg("in_head_dim") = 0, py::arg("residual") = py::none(),
         py::arg("out_dtype") = at::kBFloat16);
+  m.def("prefill_attention", &prefill_attention, "causal grouped-query attention of a prompt on the matrix core",
+        py::arg("q"), py::arg("k"), py::arg("v"), py::arg("scale"));
   m.def("argmax_advance_embed", &argmax_advance_embed,
         "argmax_advance over 32 workgroups; with embed / hidden_out also hidden_out <- embed[index]", py::arg("x"),
         py::arg("token"), py::arg("step64"), py::arg("step32"), py::arg("embed") = py::none(),

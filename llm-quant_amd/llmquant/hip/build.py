@@ -111,6 +111,8 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_argmax_row.restype = c_int
     lib.llmq_argmax_advance.argtypes = [c_p, c_int, c_p, c_p, c_p, c_p, c_int, c_p]
     lib.llmq_argmax_advance.restype = c_int
+    lib.llmq_prefill_attention.argtypes = [c_p, c_p, c_p, c_p, c_int, c_int, c_int, c_int, ctypes.c_float, c_int, c_p]
+    lib.llmq_prefill_attention.restype = c_int
     lib.llmq_argmax_advance_embed.argtypes = [c_p, c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_int, c_p, c_int, c_p]
     lib.llmq_argmax_advance_embed.restype = c_int
     lib.llmq_argmax_workspace_bytes.argtypes = []

@@ -33,6 +33,11 @@ def _rotate_half(x):
 class LlamaKernelRuntime:
     """Prefill + greedy decode of one sequence over a LlamaForCausalLM-shaped model."""
 
+    # Prompts of up to this many tokens x head_dim go through the package's own attention kernel, which is built
+    # for the short walk (every CU busy at 512 tokens; 1024 tokens at head_dim 64, 512 at 128); beyond it the
+    # library's flash kernel is the faster one.
+    PROMPT_ATTENTION_MAX_WORK = 65536
+
     def __init__(self, model, max_len: int, kv_bits: int = 8, exact_prefill: bool = False):
         cfg = model.config
         self.exact_prefill = exact_prefill
@@ -162,6 +167,11 @@ class LlamaKernelRuntime:
             # prompt: attention sees the fake-quantized K/V of the prompt itself, which is what
             # FakeQuantCache.update returns on an empty cache
             ctx = self._fp32_causal_attention(q, k_dq, v_dq)
+        elif (self._one_launch_ops and self.head_dim in (64, 128) and tokens * self.head_dim <= self.PROMPT_ATTENTION_MAX_WORK
+              and q.dim() == 3 and q.is_contiguous() and k_dq.is_contiguous() and v_dq.is_contiguous()):
+            # the same causal grouped-query softmax(q k^T) v as the library call below, walked by four waves
+            # per 32 queries, and written as [tokens, heads * head_dim] directly
+            ctx = self._ext.prefill_attention(q, k_dq, v_dq, self.scaling)
         else:
             ctx = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k_dq[None], v_dq[None],
                                                  is_causal=True, scale=self.scaling, enable_gqa=True)
