@@ -20,8 +20,13 @@
 // (query, half) with 16 of the block's 32 scores, so the running maximum and sum of a query are in-lane
 // reductions plus one exchange between the two halves; O^T = V^T P^T (A = head_dim x keys, B = keys x queries)
 // takes the probabilities straight out of those registers as its B operand (the k index of the MFMA is just a
-// naming of the keys, the same on both operands) and V transposed through the wave's own LDS tile. The next
-// block's K and V are requested as soon as this block's have been consumed.
+// naming of the keys, the same on both operands) and V^T from the wave's own LDS tile: the block's rows of V go
+// there as they lie in memory (global_load_lds_dwordx4, no register in between, the 16-byte pieces of odd keys
+// XOR-swizzled by four so that the reads below spread over the banks), and ds_read_b64_tr_b16 hands lane
+// (d, half) four keys of its column per read. Among the 16 lanes of a group, that instruction gives lane l, as
+// its element j, element l % 4 of what lane 4 j + l / 4 points at: with lane 4 j + i pointing at key j,
+// columns 4 i .. 4 i + 3, lane l gets column l of keys 0..3. The next block's K and V are requested as soon as
+// this block's K has been consumed, into the tile's other buffer.
 #include "llmq_device.h"
 
 namespace {
@@ -32,9 +37,9 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef short v4s __attribute__((ext_vector_type(4)));
 
 constexpr int kQueriesPerGroup = 32, kWavesPerGroup = 4, kKeysPerBlock = 32;
-constexpr int kVtStride = kKeysPerBlock + 4;   // elements: rows of the transposed V tile 72 bytes apart
 
 template <typename T> __device__ __forceinline__ v16f mfma16(u32x4 a, u32x4 b, v16f c);
 template <> __device__ __forceinline__ v16f mfma16<bf16_t>(u32x4 a, u32x4 b, v16f c) {
@@ -58,7 +63,7 @@ template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float lo, float hi)
 __device__ __forceinline__ int key_of(int lh, int r) { return 8 * (r >> 2) + 4 * lh + (r & 3); }
 
 template <int D> struct Lds {
-  static constexpr int kTile = D * kVtStride * 2;                  // bytes of one wave's transposed V tile
+  static constexpr int kTile = 2 * kKeysPerBlock * D * 2;          // bytes of one wave's V tile, two buffers
   static constexpr int kRow = D + 4;                               // floats of a row of a partial result
   static constexpr int kPartial = kQueriesPerGroup * kRow * 4;     // bytes of one wave's partial result
   static constexpr int kBody = kWavesPerGroup * (kPartial > kTile ? kPartial : kTile);
@@ -66,7 +71,7 @@ template <int D> struct Lds {
 };
 
 template <typename T, int D>
-__global__ __launch_bounds__(kWavesPerGroup * kWave) void prefill_attention_kernel(
+__global__ __launch_bounds__(kWavesPerGroup * kWave, 2) void prefill_attention_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, T* __restrict__ out, const int tokens,
     const int q_heads, const int kv_heads, const float scale_log2e) {
   constexpr int kDSteps = D / 16;    // k-steps of S^T = K Q^T
@@ -92,30 +97,43 @@ __global__ __launch_bounds__(kWavesPerGroup * kWave) void prefill_attention_kern
   }
   const int n_blocks = min(q0 + kQueriesPerGroup - 1, tokens - 1) / kKeysPerBlock + 1;   // up to the diagonal
 
-  // V of a block, as this wave moves it: lane (key = lane % 32, half) takes the 16-byte pieces 2 u + half of its
-  // key's row (so that the two halves write to different banks), and writes them out as a column of the tile
-  constexpr int kVLoads = D / 16;
-  u32x4 kreg[kDSteps], vreg[kVLoads];
-  auto request = [&](int b) {
+  // K of a block straight into the A operand's registers; V into the LDS tile: transfer i of a wave covers
+  // bytes 1024 i + 16 lane of the tile, which is piece (slot ^ 4 (key & 1)) of key (1024 i + 16 lane) / (2 D)
+  constexpr int kTileBytes = kKeysPerBlock * D * 2, kVInstr = kTileBytes / 1024, kRowBytes = 2 * D;
+  unsigned char* tile = s_mem + wv * Lds<D>::kTile;
+  uint32_t v_off[kVInstr];   // byte offsets into a block of V (before the clamp of the key to the prompt's end)
+  int v_key[kVInstr];
+#pragma unroll
+  for (int i = 0; i < kVInstr; ++i) {
+    const int at = 1024 * i + 16 * lane, key = at / kRowBytes, slot = (at % kRowBytes) / 16;
+    v_key[i] = key;
+    v_off[i] = static_cast<uint32_t>((slot ^ ((key & 1) << 2)) * 16);
+  }
+  u32x4 kreg[kDSteps];
+  auto request = [&](int b, int buf) {
     const int j0 = b * kKeysPerBlock;
     const T* row = kh + static_cast<int64_t>(min(j0 + lm, tokens - 1)) * D + 8 * lh;
 #pragma unroll
     for (int t = 0; t < kDSteps; ++t) kreg[t] = load16(row + 16 * t);
-    row = vh + static_cast<int64_t>(min(j0 + lm, tokens - 1)) * D + 8 * lh;
 #pragma unroll
-    for (int u = 0; u < kVLoads; ++u) vreg[u] = load16(row + 16 * u);
-  };
-  uint16_t* vt = reinterpret_cast<uint16_t*>(s_mem + wv * Lds<D>::kTile);
-  auto stage_v = [&]() {
-#pragma unroll
-    for (int u = 0; u < kVLoads; ++u) {
-      const uint32_t w[4] = {vreg[u].x, vreg[u].y, vreg[u].z, vreg[u].w};
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        vt[(16 * u + 8 * lh + e) * kVtStride + lm] = static_cast<uint16_t>(w[e >> 1] >> (16 * (e & 1)));
-      }
+    for (int i = 0; i < kVInstr; ++i) {
+      const unsigned char* src = reinterpret_cast<const unsigned char*>(vh) +
+                                 static_cast<int64_t>(min(j0 + v_key[i], tokens - 1)) * kRowBytes + v_off[i];
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(src),
+                                       reinterpret_cast<u32x4*>(tile + buf * kTileBytes + 1024 * i), 16, 0, 0);
     }
   };
+  // where this lane points for the transposing reads: key 4 lh + j of a group of eight, columns
+  // 32 t + 16 (g & 1) + 4 i .. + 3, with g = lane / 16, j = lane % 16 / 4, i = lane % 4
+  uint32_t tr_at[kDTiles];
+  {
+    const int g = lane >> 4, j = (lane >> 2) & 3, i = lane & 3;
+#pragma unroll
+    for (int t = 0; t < kDTiles; ++t) {
+      const int piece = 4 * t + 2 * (g & 1) + (i >> 1);
+      tr_at[t] = static_cast<uint32_t>((4 * lh + j) * kRowBytes + (piece ^ ((j & 1) << 2)) * 16 + (i & 1) * 8);
+    }
+  }
 
   v16f o[kDTiles];
 #pragma unroll
@@ -124,16 +142,19 @@ __global__ __launch_bounds__(kWavesPerGroup * kWave) void prefill_attention_kern
     for (int r = 0; r < 16; ++r) o[t][r] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;   // of this lane's query, in units of log2
 
-  if (wv < n_blocks) request(wv);
-  for (int b = wv; b < n_blocks; b += kWavesPerGroup) {
+  if (wv < n_blocks) request(wv, 0);
+  int buf = 0;
+  for (int b = wv; b < n_blocks; b += kWavesPerGroup, buf ^= 1) {
     const int j0 = b * kKeysPerBlock;
-    stage_v();
+    // this block's K and V have arrived (nothing else of this wave is in flight)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     v16f s;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.0f;
 #pragma unroll
     for (int t = 0; t < kDSteps; ++t) s = mfma16<T>(kreg[t], qreg[t], s);
-    if (b + kWavesPerGroup < n_blocks) request(b + kWavesPerGroup);
+    // (the other buffer: its last readers were the previous block's MFMAs, whose operands have long arrived)
+    if (b + kWavesPerGroup < n_blocks) request(b + kWavesPerGroup, buf ^ 1);
 
     // scores in units of log2, keys beyond the query or the prompt out
     const bool edge = j0 + kKeysPerBlock - 1 > min(q0, tokens - 1);
@@ -173,31 +194,29 @@ __global__ __launch_bounds__(kWavesPerGroup * kWave) void prefill_attention_kern
         for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
     }
 
-    // O^T += V^T P^T: k-step st covers the keys that registers 8 st .. 8 st + 7 hold (key_of). The tile was
-    // written by this wave alone, and a wave's LDS accesses complete in order.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // O^T += V^T P^T: k-step st covers the keys that registers 8 st .. 8 st + 7 hold (key_of): two transposing
+    // reads, keys 16 st + 4 lh + 0..3 and 16 st + 8 + 4 lh + 0..3
+    const unsigned char* vt = tile + buf * kTileBytes;
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
       const u32x4 pb = {p[4 * st], p[4 * st + 1], p[4 * st + 2], p[4 * st + 3]};
 #pragma unroll
       for (int t = 0; t < kDTiles; ++t) {
-        const uint16_t* row = vt + (32 * t + lm) * kVtStride + 16 * st + 4 * lh;
-        const uint2 a_lo = *reinterpret_cast<const uint2*>(row);        // keys 16 st + 4 lh + 0..3
-        const uint2 a_hi = *reinterpret_cast<const uint2*>(row + 8);    // keys 16 st + 8 + 4 lh + 0..3
+        const unsigned char* at = vt + tr_at[t] + 16 * st * kRowBytes;
+        const uint2 a_lo = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) v4s*)(at)));
+        const uint2 a_hi = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) v4s*)(at + 8 * kRowBytes)));
         o[t] = mfma16<T>(u32x4{a_lo.x, a_lo.y, a_hi.x, a_hi.y}, pb, o[t]);
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();   // (the next block's columns are written after these reads)
   }
 
   // ---- merge the four walks: m = max m_w, l = sum l_w 2^(m_w - m), O = sum O_w 2^(m_w - m), in wave order ------
   float* s_max = reinterpret_cast<float*>(s_mem + Lds<D>::kBody);
   float* s_sum = s_max + kWavesPerGroup * kQueriesPerGroup;
   if (lh == 0) s_max[wv * kQueriesPerGroup + lm] = m_run;
-  __syncthreads();   // also: every wave is done with its V tile, which the partial results overwrite
+  __syncthreads();   // also: every wave is done with its V tiles, which the partial results overwrite
   float m_all = s_max[lm];
 #pragma unroll
   for (int w = 1; w < kWavesPerGroup; ++w) m_all = fmaxf(m_all, s_max[w * kQueriesPerGroup + lm]);

@@ -33,10 +33,11 @@ def _rotate_half(x):
 class LlamaKernelRuntime:
     """Prefill + greedy decode of one sequence over a LlamaForCausalLM-shaped model."""
 
-    # Prompts of up to this many tokens x head_dim go through the package's own attention kernel, which is built
-    # for the short walk (every CU busy at 512 tokens; 1024 tokens at head_dim 64, 512 at 128); beyond it the
-    # library's flash kernel is the faster one.
-    PROMPT_ATTENTION_MAX_WORK = 65536
+    # Prompts of up to this many tokens (by head_dim) go through the package's own attention kernel, which is
+    # built for the short walk (every CU busy at 512 tokens, where it takes under half the library's time) and
+    # level with the library's flash kernel at these lengths; between them and 8192 tokens the library is 5-10 %
+    # ahead.
+    PROMPT_ATTENTION_MAX_TOKENS = {64: 2048, 128: 1536}
 
     def __init__(self, model, max_len: int, kv_bits: int = 8, exact_prefill: bool = False):
         cfg = model.config
@@ -167,7 +168,7 @@ class LlamaKernelRuntime:
             # prompt: attention sees the fake-quantized K/V of the prompt itself, which is what
             # FakeQuantCache.update returns on an empty cache
             ctx = self._fp32_causal_attention(q, k_dq, v_dq)
-        elif (self._one_launch_ops and self.head_dim in (64, 128) and tokens * self.head_dim <= self.PROMPT_ATTENTION_MAX_WORK
+        elif (self._one_launch_ops and tokens <= self.PROMPT_ATTENTION_MAX_TOKENS.get(self.head_dim, 0)
               and q.dim() == 3 and q.is_contiguous() and k_dq.is_contiguous() and v_dq.is_contiguous()):
             # the same causal grouped-query softmax(q k^T) v as the library call below, walked by four waves
             # per 32 queries, and written as [tokens, heads * head_dim] directly
