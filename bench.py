@@ -584,6 +584,33 @@ def other_kernels(torch):
                           "GBps": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)})
         del qs
     out["w4a16_fused_gemm_small_m"] = fused
+
+    # The prompt's causal grouped-query attention (Llama-3.2-1B geometry: 32 query / 8 kv heads of 64; and the
+    # 8B head size), the package's kernel beside torch's scaled_dot_product_attention + the copy that brings its
+    # output to [tokens, heads * head_dim]. Flops: 4 * tokens^2 / 2 * heads * head_dim.
+    attention = []
+    for tokens, d in ((128, 64), (512, 64), (2048, 64), (512, 128)):
+        qh, kvh = 32, 8
+        q = torch.randn(tokens, qh, d, device=dev).to(torch.bfloat16)
+        kk = torch.randn(kvh, tokens, d, device=dev).to(torch.bfloat16)
+        vv = torch.randn(kvh, tokens, d, device=dev).to(torch.bfloat16)
+
+        def ours():
+            for _ in range(10):
+                ext.prefill_attention(q, kk, vv, d ** -0.5)
+
+        def library():
+            for _ in range(10):
+                ctx = torch.nn.functional.scaled_dot_product_attention(q.transpose(0, 1)[None], kk[None], vv[None],
+                                                                       is_causal=True, scale=d ** -0.5, enable_gqa=True)
+                ctx[0].transpose(0, 1).reshape(tokens, -1)
+
+        us = _graph_time_us(torch, ours, reps=10) / 10
+        us_lib = _graph_time_us(torch, library, reps=10) / 10
+        flops = 2 * tokens * tokens * qh * d
+        attention.append({"tokens": tokens, "q_heads": qh, "kv_heads": kvh, "head_dim": d, "us": round(us, 2),
+                          "TFLOPs": round(flops / us / 1e6, 1), "torch_sdpa_us": round(us_lib, 2)})
+    out["prompt_attention_bf16"] = attention
     return out
 
 

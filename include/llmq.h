@@ -374,8 +374,8 @@ int llmq_argmax_advance(const void* x, int n, int64_t* out_index, int64_t* token
  * attention on the rotated queries and the K / V its FakeQuantCache returns (llmquant/quantizers/fake.py:39-55;
  * the reference has no kernel of its own for it). q: [tokens, q_heads, head_dim]; k, v: [kv_heads, tokens,
  * head_dim] (the dequantized cache values, as llmq_rope_kv_append hands them back); out: [tokens, q_heads,
- * head_dim]. float16 or bfloat16, head_dim 64 or 128, 16-byte aligned; fp32 accumulation, probabilities rounded
- * to `dtype` before they meet v. */
+ * head_dim]. float16 or bfloat16, head_dim 64 or 128, 16-byte aligned, scale > 0; fp32 accumulation,
+ * probabilities rounded to `dtype` before they meet v. */
 int llmq_prefill_attention(const void* q, const void* k, const void* v, void* out, int tokens, int q_heads,
                            int kv_heads, int head_dim, float scale, int dtype, llmq_stream_t stream);
 

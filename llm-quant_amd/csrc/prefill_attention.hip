@@ -78,7 +78,8 @@ __global__ __launch_bounds__(kWavesPerGroup * kWave, 2) void prefill_attention_k
   constexpr int kDTiles = D / 32;    // row tiles of O^T
   __shared__ __attribute__((aligned(16))) unsigned char s_mem[Lds<D>::kBytes];
 
-  const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1);
+  const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);   // (in a scalar register: the walk's block index, and every branch on it, is the wave's)
   const int lm = lane & 31, lh = lane >> 5;
   // the long walks (late query blocks) first
   const int qb = static_cast<int>(gridDim.x) - 1 - static_cast<int>(blockIdx.x);
@@ -156,20 +157,20 @@ __global__ __launch_bounds__(kWavesPerGroup * kWave, 2) void prefill_attention_k
     // (the other buffer: its last readers were the previous block's MFMAs, whose operands have long arrived)
     if (b + kWavesPerGroup < n_blocks) request(b + kWavesPerGroup, buf ^ 1);
 
-    // scores in units of log2, keys beyond the query or the prompt out
-    const bool edge = j0 + kKeysPerBlock - 1 > min(q0, tokens - 1);
-    float m_blk = -INFINITY;
+    // keys beyond the query or the prompt out (only the blocks on the diagonal and at the prompt's end have any)
+    if (j0 + kKeysPerBlock - 1 > min(q0, tokens - 1)) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      float x = s[r] * scale_log2e;
-      if (edge) {
+      for (int r = 0; r < 16; ++r) {
         const int key = j0 + key_of(lh, r);
-        if (key > my_query || key >= tokens) x = -INFINITY;
+        if (key > my_query || key >= tokens) s[r] = -INFINITY;
       }
-      s[r] = x;
-      m_blk = fmaxf(m_blk, x);
     }
-    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, kWave));
+    // the block's maximum in units of log2 (scale_log2e > 0: the largest score gives it), then
+    // p = 2^(s scale_log2e - m), one multiply-add per score
+    float m_blk = s[0];
+#pragma unroll
+    for (int r = 1; r < 16; ++r) m_blk = fmaxf(m_blk, s[r]);
+    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, kWave)) * scale_log2e;
     // finite: the block's first key is at or below every query of the group (rows past the prompt's end repeat
     // its last query and are not stored)
     const float m_new = fmaxf(m_run, m_blk);
@@ -178,7 +179,8 @@ __global__ __launch_bounds__(kWavesPerGroup * kWave, 2) void prefill_attention_k
     uint32_t p[8];
 #pragma unroll
     for (int r = 0; r < 16; r += 2) {
-      const float p0 = __builtin_amdgcn_exp2f(s[r] - m_new), p1 = __builtin_amdgcn_exp2f(s[r + 1] - m_new);
+      const float p0 = __builtin_amdgcn_exp2f(fmaf(s[r], scale_log2e, -m_new));
+      const float p1 = __builtin_amdgcn_exp2f(fmaf(s[r + 1], scale_log2e, -m_new));
       l_blk += p0 + p1;
       p[r >> 1] = pack2<T>(p0, p1);
     }
@@ -259,6 +261,7 @@ extern "C" int llmq_prefill_attention(const void* q, const void* k, const void* 
   if (tokens < 0 || q_heads <= 0 || kv_heads <= 0) return llmq_host::fail_invalid("bad shape: tokens=%d q_heads=%d kv_heads=%d", tokens, q_heads, kv_heads);
   if (q_heads % kv_heads != 0) return llmq_host::fail_invalid("q_heads %d is not a multiple of kv_heads %d", q_heads, kv_heads);
   if (head_dim != 64 && head_dim != 128) return llmq_host::fail_invalid("head_dim must be 64 or 128, got %d", head_dim);
+  if (!(scale > 0.0f) || scale > 3.0e38f) return llmq_host::fail_invalid("scale must be positive and finite, got %g", static_cast<double>(scale));
   if (dtype != LLMQ_F16 && dtype != LLMQ_BF16) return llmq_host::fail_invalid("q, k, v must be float16 or bfloat16, got dtype code %d", dtype);
   if (tokens == 0) return 0;
   if (!q || !k || !v || !out) return llmq_host::fail_invalid("null tensor pointer");

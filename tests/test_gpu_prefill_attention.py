@@ -69,6 +69,8 @@ def check(ext, q, k, v, scale):
     (128, 8, 2, 128),     # Llama-3-8B's head shape
     (1, 4, 4, 64), (2, 4, 1, 64), (31, 4, 2, 128), (32, 2, 2, 64), (33, 6, 2, 64), (63, 2, 1, 128),
     (64, 3, 3, 64), (65, 4, 2, 64), (97, 8, 8, 128), (200, 4, 1, 64), (257, 2, 2, 128),
+    # long walks: many blocks per wave, head counts that are no multiple of four
+    (1023, 4, 1, 64), (1024, 8, 2, 64), (1100, 6, 2, 64), (1025, 5, 5, 128), (1300, 4, 4, 128), (2048, 8, 2, 64),
 ])
 def test_matches_float64_causal_gqa(ext, dtype, tokens, q_heads, kv_heads, d):
     q, k, v = make(tokens, q_heads, kv_heads, d, dtype, seed=tokens * 7 + d)
@@ -83,7 +85,7 @@ def test_peaked_softmax_and_large_scores(ext, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("tokens,q_heads,kv_heads,d", [(512, 32, 8, 64), (300, 8, 2, 128), (77, 4, 4, 64)])
+@pytest.mark.parametrize("tokens,q_heads,kv_heads,d", [(512, 32, 8, 64), (300, 8, 2, 128), (77, 4, 4, 64), (1536, 8, 2, 64)])
 def test_no_further_from_float64_than_the_library(ext, dtype, tokens, q_heads, kv_heads, d):
     q, k, v = make(tokens, q_heads, kv_heads, d, dtype, seed=11)
     scale = 1.0 / math.sqrt(d)
@@ -108,6 +110,11 @@ def test_first_query_sees_only_the_first_key_and_rows_do_not_depend_on_later_tok
         part = ext.prefill_attention(q[:shorter].cuda(), k[:, :shorter].contiguous().cuda(),
                                      v[:, :shorter].contiguous().cuda(), 0.125)
         assert torch.equal(part, full[:shorter])
+    # the same on a long prompt
+    q, k, v = make(1500, 4, 2, 64, torch.bfloat16, seed=6)
+    full = ext.prefill_attention(q.cuda(), k.cuda(), v.cuda(), 0.125)
+    part = ext.prefill_attention(q[:1111].cuda(), k[:, :1111].contiguous().cuda(), v[:, :1111].contiguous().cuda(), 0.125)
+    assert torch.equal(part, full[:1111])
 
 
 def test_equal_keys_give_the_running_mean_of_v(ext):
@@ -134,6 +141,8 @@ def test_empty_prompt_and_argument_checks(ext):
         ext.prefill_attention(q[:, :3].contiguous(), k, v, 1.0)
     with pytest.raises(RuntimeError, match="float16 or bfloat16"):
         ext.prefill_attention(q.float(), k.float(), v.float(), 1.0)
+    with pytest.raises(RuntimeError, match="positive"):
+        ext.prefill_attention(q, k, v, -1.0)
     with pytest.raises(RuntimeError, match="k and v must be"):
         ext.prefill_attention(q, k[:, :4].contiguous(), v[:, :4].contiguous(), 1.0)
 
