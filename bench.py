@@ -314,9 +314,18 @@ def other_kernels(torch):
 
     us = _event_time_us(torch, fq, reps=48)
     nbytes = 2 * 2048 * 8192 * 2 + 2048 * 64 * 4
+    # what a plain device copy of the same tensors takes (one read + one write of the same bytes, no scales)
+    ys = [torch.empty_like(x) for x in xs]
+
+    def copy():
+        ys[i[0] % len(xs)].copy_(xs[i[0] % len(xs)])
+        i[0] += 1
+
+    us_copy = _event_time_us(torch, copy, reps=48)
     out["fake_quant_2048x8192_bf16_int4"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
-                                             "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
-    del xs
+                                             "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
+                                             "device_copy_of_the_same_tensor_us": round(us_copy, 2)}
+    del xs, ys
     # KV cache decode step, Llama-3.2-1B geometry, 2048 tokens of context + the one being decoded:
     # RoPE + quantize-and-append + attention in one launch per layer, 16 layers replayed as a graph
     # (16 layers of cache are 36 MB and would sit in the 256 MB Infinity Cache: the launches walk as many
