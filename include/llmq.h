@@ -227,6 +227,28 @@ int llmq_wq_gemm_a16_tile(const void* x, const void* qweight, const float* wscal
                           size_t workspace_bytes, int M, int N, int G, int gs, int out_group, int wformat,
                           int dtype, llmq_stream_t stream);
 
+/* gate_proj | up_proj and the activation between them and down_proj in one launch, for the prompt pass of a gated
+ * MLP (transformers' LlamaMLP: down_proj(act_fn(gate_proj(x)) * up_proj(x)), each Linear on the reference's
+ * M > 4 branch, llmquant/quantizers/kernel.py:68-79,88-91): `qweight` is gate_proj's I rows followed by up_proj's
+ * I rows ([2 I, G, gs], wscale [2 I (or tiles of out_group), G]); a workgroup multiplies 128 gate rows and the
+ * 128 up rows that belong to them, rounds both results to bfloat16 as the two Linears would, and writes
+ * silu(gate) * up (rounded where `act_fn(gate) * up` on bfloat16 tensors rounds) for its 128 x 128 block directly as
+ * the prepared activation of the next GEMM: into the first llmq_wq_gemm_a16_tile_prepared_bytes(M, I / 128) bytes
+ * of `next_workspace`, which is then the workspace of llmq_wq_gemm_a16_tile_prepared on down_proj's weight
+ * (N, G = I / 128). The bits are those of llmq_wq_gemm_a16_tile + llmq_silu_mul_rows + llmq_wq_gemm_a16_tile.
+ * I must be a multiple of 128; the reduction axis is never split (use it where ceil(M / 128) * I / 128 workgroups
+ * fill the chip). `workspace`: at least llmq_wq_gemm_a16_tile_prepared_bytes(M, G) bytes. */
+size_t llmq_wq_gemm_a16_tile_prepared_bytes(int M, int G);
+int llmq_wq_gemm_a16_tile_gate_up_silu(const void* x, const void* qweight, const float* wscale, void* workspace,
+                                       size_t workspace_bytes, void* next_workspace, size_t next_workspace_bytes,
+                                       int M, int I, int G, int gs, int out_group, int wformat, int dtype,
+                                       llmq_stream_t stream);
+/* llmq_wq_gemm_a16_tile on an activation that is already in `workspace` in prepared form (left there by
+ * llmq_wq_gemm_a16_tile_gate_up_silu): no x. workspace_bytes as for llmq_wq_gemm_a16_tile. */
+int llmq_wq_gemm_a16_tile_prepared(const void* qweight, const float* wscale, void* out, void* workspace,
+                                   size_t workspace_bytes, int M, int N, int G, int gs, int out_group, int wformat,
+                                   int dtype, llmq_stream_t stream);
+
 /* The elementwise pieces of a prompt pass, one launch each, with the rounding points of the PyTorch
  * sequences they replace (the same ones the decode kernels use). dtype: LLMQ_F32 / F16 / BF16; all
  * tensors 16-byte aligned. No counterpart in the reference, which leaves these to transformers

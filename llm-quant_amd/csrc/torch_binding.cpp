@@ -636,6 +636,75 @@ at::Tensor wq_gemm_a16_tile(const at::Tensor& x, const at::Tensor& qweight, cons
   return out;
 }
 
+// gate|up GEMM with silu(gate) * up written as the prepared activation of the next tiled GEMM (down_proj, next_n
+// rows): returns that GEMM's workspace, to be handed to wq_gemm_a16_tile_prepared.
+at::Tensor wq_gemm_a16_tile_gate_up_silu(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale,
+                                         int64_t out_group, int64_t next_n) {
+  TORCH_CHECK(x.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "x, qweight and wscale must be CUDA tensors");
+  TORCH_CHECK(x.scalar_type() == at::kBFloat16, "the tiled fused GEMM takes bfloat16 activations");
+  TORCH_CHECK(x.dim() == 2, "x must be [M, K]");
+  TORCH_CHECK(qweight.dim() == 3, "qweight must be [2 * intermediate, groups, group_size], got ", qweight.dim(), "D");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 2, "wscale must be float32 [scale_rows, groups]");
+  const auto xc = x.contiguous();
+  const auto wc = qweight.contiguous();
+  const auto sc = wscale.contiguous();
+  const int64_t M = xc.size(0), N = wc.size(0), groups = wc.size(1);
+  const int64_t group_size = packed ? wc.size(2) * 2 : wc.size(2);
+  TORCH_CHECK(group_size == 128, "the tiled fused GEMM needs group_size 128, got ", group_size);
+  TORCH_CHECK(N % 256 == 0, "gate rows followed by up rows, a multiple of 128 each: got ", N, " rows");
+  TORCH_CHECK(xc.size(1) == groups * group_size, "x last dim ", xc.size(1), " does not match qweight ", groups, "x", group_size);
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  TORCH_CHECK(sc.size(0) == scale_rows && sc.size(1) == groups, "wscale must be [", scale_rows, ", ", groups, "]");
+  TORCH_CHECK(M > 0 && next_n > 0, "empty activation");
+  const int64_t inter = N / 2, next_groups = inter / 128;
+  const c10::OptionalDeviceGuard guard(at::device_of(xc));
+  const size_t need = llmq_wq_gemm_a16_tile_prepared_bytes(static_cast<int>(M), static_cast<int>(groups));
+  const size_t next_need = llmq_wq_gemm_a16_tile_workspace_bytes(static_cast<int>(M), static_cast<int>(next_n), static_cast<int>(next_groups));
+  auto workspace = at::empty({static_cast<int64_t>((need + 3) / 4)}, xc.options().dtype(at::kFloat));
+  auto next = at::empty({static_cast<int64_t>((next_need + 3) / 4)}, xc.options().dtype(at::kFloat));
+  check_rc(llmq_wq_gemm_a16_tile_gate_up_silu(xc.const_data_ptr(), wc.const_data_ptr(), sc.const_data_ptr<float>(),
+                                              workspace.mutable_data_ptr(), need, next.mutable_data_ptr(), next_need,
+                                              static_cast<int>(M), static_cast<int>(inter), static_cast<int>(groups),
+                                              static_cast<int>(group_size), static_cast<int>(out_group),
+                                              packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype_code(xc, "x"),
+                                              current_stream(xc)),
+           "wq_gemm_a16_tile_gate_up_silu");
+  return next;
+}
+
+// The tiled GEMM on a prepared activation of `rows` rows sitting in `workspace` (from wq_gemm_a16_tile_gate_up_silu).
+at::Tensor wq_gemm_a16_tile_prepared(const at::Tensor& workspace, int64_t rows, const at::Tensor& qweight,
+                                     const at::Tensor& wscale, int64_t out_group) {
+  TORCH_CHECK(workspace.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "workspace, qweight and wscale must be CUDA tensors");
+  TORCH_CHECK(workspace.scalar_type() == at::kFloat && workspace.dim() == 1 && workspace.is_contiguous(),
+              "workspace must be the tensor wq_gemm_a16_tile_gate_up_silu returned");
+  TORCH_CHECK(qweight.dim() == 3, "qweight must be [N, groups, group_size], got ", qweight.dim(), "D");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 2, "wscale must be float32 [scale_rows, groups]");
+  const auto wc = qweight.contiguous();
+  const auto sc = wscale.contiguous();
+  const int64_t M = rows, N = wc.size(0), groups = wc.size(1);
+  const int64_t group_size = packed ? wc.size(2) * 2 : wc.size(2);
+  TORCH_CHECK(group_size == 128, "the tiled fused GEMM needs group_size 128, got ", group_size);
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  TORCH_CHECK(sc.size(0) == scale_rows && sc.size(1) == groups, "wscale must be [", scale_rows, ", ", groups, "]");
+  TORCH_CHECK(M > 0 && N > 0, "empty activation or weight");
+  const size_t need = llmq_wq_gemm_a16_tile_workspace_bytes(static_cast<int>(M), static_cast<int>(N), static_cast<int>(groups));
+  TORCH_CHECK(static_cast<size_t>(workspace.numel()) * 4 >= need, "workspace holds ", workspace.numel() * 4, " bytes, this GEMM needs ", need);
+  auto out = at::empty({M, N}, workspace.options().dtype(at::kBFloat16));
+  const c10::OptionalDeviceGuard guard(at::device_of(workspace));
+  check_rc(llmq_wq_gemm_a16_tile_prepared(wc.const_data_ptr(), sc.const_data_ptr<float>(), out.mutable_data_ptr(),
+                                          workspace.mutable_data_ptr(), static_cast<size_t>(workspace.numel()) * 4,
+                                          static_cast<int>(M), static_cast<int>(N), static_cast<int>(groups),
+                                          static_cast<int>(group_size), static_cast<int>(out_group),
+                                          packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, LLMQ_BF16, current_stream(workspace)),
+           "wq_gemm_a16_tile_prepared");
+  return out;
+}
+
 // ---- elementwise pieces of a prompt pass ----------------------------------------------------------------
 at::Tensor rmsnorm(const at::Tensor& x, const at::Tensor& weight, double eps) {
   TORCH_CHECK(x.is_cuda() && weight.is_cuda(), "x and weight must be CUDA tensors");
@@ -1146,6 +1215,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("wq_gemm_a16", &wq_gemm_a16,
         "Weight-only GEMM for a few dozen rows: fp16/bf16 activations x int4/int8 group-quantized weights, no dense copy",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("split") = false);
+  m.def("wq_gemm_a16_tile_gate_up_silu", &wq_gemm_a16_tile_gate_up_silu,
+        "gate|up tiled GEMM whose workgroups write silu(gate) * up as the next tiled GEMM's prepared activation",
+        py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("next_n"));
+  m.def("wq_gemm_a16_tile_prepared", &wq_gemm_a16_tile_prepared,
+        "the tiled GEMM on the prepared activation wq_gemm_a16_tile_gate_up_silu left in its workspace",
+        py::arg("workspace"), py::arg("rows"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0);
   m.def("wq_gemm_a16_tile", &wq_gemm_a16_tile,
         "Fused weight-only GEMM for prompt-sized bf16 activations: 128 x 256 tiles on the bf16 matrix cores, no dense weight",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0);

@@ -59,13 +59,11 @@ constexpr int kMT = kWaveM / 32, kNT = kWaveN / 32;
 template <int BITS> constexpr float kCodeBias = BITS == 4 ? 24.0f : 128.0f;
 
 // ---- activation preparation -----------------------------------------------------------------------
-// One lane per 16-byte chunk, 16 lanes per (row, group).
-__global__ __launch_bounds__(256) void act_prep_kernel(const u32x4* __restrict__ x, u32x4* __restrict__ xp,
-                                                       u32x4* __restrict__ rec, const int64_t n_chunks) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  const bool active = i < n_chunks;  // n_chunks is a multiple of 16: a row of 16 lanes is active or idle as one
-  u32x4 v = {0u, 0u, 0u, 0u};
-  if (active) v = x[i];
+// One lane per 16-byte chunk, 16 lanes per (row, group): `v` holds the chunk's eight bf16 values (zeros in a lane
+// with nothing to do; a row of 16 lanes is active or idle as one). Writes the reordered chunk, and from the row's
+// first lane the record of the group's sum.
+__device__ __forceinline__ void emit_prepared(const u32x4 v, const bool active, const bool first_of_row,
+                                              u32x4* __restrict__ chunk_out, u32x4* __restrict__ record_out) {
   float f[8];
   Pack<bf16_t>::unpack(v, f);
   float s = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
@@ -77,16 +75,25 @@ __global__ __launch_bounds__(256) void act_prep_kernel(const u32x4* __restrict__
   o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
   o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
   o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
-  xp[i] = o;
-  if ((threadIdx.x & 15) == 0) {
+  *chunk_out = o;
+  if (first_of_row) {
     // s = hi + mid + lo, each a bf16: 24 bits of the sum
     const uint32_t hi = bf16_bits_rne(s);
     const float r1 = s - __builtin_bit_cast(float, hi << 16);
     const uint32_t mid = bf16_bits_rne(r1);
     const float r2 = r1 - __builtin_bit_cast(float, mid << 16);
     const uint32_t lo = bf16_bits_rne(r2);
-    rec[i >> 4] = u32x4{hi | (mid << 16), lo, 0u, 0u};  // k' slots 0..2 of the correction step
+    *record_out = u32x4{hi | (mid << 16), lo, 0u, 0u};  // k' slots 0..2 of the correction step
   }
+}
+
+__global__ __launch_bounds__(256) void act_prep_kernel(const u32x4* __restrict__ x, u32x4* __restrict__ xp,
+                                                       u32x4* __restrict__ rec, const int64_t n_chunks) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const bool active = i < n_chunks;  // n_chunks is a multiple of 16: a row of 16 lanes is active or idle as one
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (active) v = x[i];
+  emit_prepared(v, active, (threadIdx.x & 15) == 0, xp + (active ? i : 0), rec + (active ? i >> 4 : 0));
 }
 
 struct TileArgs {
@@ -98,7 +105,19 @@ struct TileArgs {
   float* partial;      // [splits][M][N] fp32 (more)
   int M, N, G, out_group;
   int m_tiles, n_tiles, splits, groups_per_split;
+  // kEpiGateUpSilu: the prepared activation of the next GEMM (its xp and rec, next_G groups a row)
+  uint8_t* next_xp;
+  uint8_t* next_rec;
+  int next_G;
 };
+
+// What a workgroup does with its totals. kEpiStore: rounds them to bf16 into out (or leaves fp32 partial tiles).
+// kEpiGateUpSilu: the weight is gate_proj's rows followed by up_proj's (N = 2 I); a tile is 128 gate rows and the
+// 128 up rows that belong to them, and the workgroup writes act = silu(bf16 gate) * bf16 up (the rounding points of
+// `act_fn(gate) * up` on bf16 tensors) for its 128 x 128 block straight into the next GEMM's prepared activation:
+// the block is one group of 128 of that activation's reduction axis, so its chunks and records are complete.
+enum Epilogue { kEpiStore = 0, kEpiGateUpSilu = 1 };
+constexpr int kEpiRowBytes = 128 * 2 + 16;   // a row of the gate (or up) block in LDS: 16 bytes of padding per row
 
 // LDS, per buffer (two buffers): the activation tile [128 rows][16 slots of 16 bytes], the raw codes of
 // the workgroup's 256 weight rows for one group ([256][64] bytes of int4 or [256][128] of int8, slots
@@ -161,7 +180,7 @@ __device__ __forceinline__ v16f mfma(const u32x4& a, const u32x4& b, const v16f&
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
 }
 
-template <int BITS>
+template <int BITS, int EPI>
 __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const TileArgs a) {
   extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
 
@@ -179,7 +198,12 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int wm = 0, wn = wv;  // every wave all the rows, an eighth of the columns
   const int lm = lane & 31, lh = lane >> 5;
-  const int m0 = mt * kBM, n0 = nt * kBN;
+  // (kEpiGateUpSilu: n0 is the tile's first gate row; column c of the tile is weight row weight_row(c))
+  const int m0 = mt * kBM, n0 = EPI == kEpiGateUpSilu ? nt * (kBN / 2) : nt * kBN;
+  auto weight_row = [&](int c) {
+    if constexpr (EPI == kEpiGateUpSilu) return c < kBN / 2 ? n0 + c : a.N / 2 + n0 + (c - kBN / 2);
+    else return min(n0 + c, a.N - 1);
+  };
   const int g_begin = sp * a.groups_per_split;
   const int g_end = min(g_begin + a.groups_per_split, a.G);
 
@@ -207,13 +231,13 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   for (int i = 0; i < kCodeInstr; ++i) {
     const int row = (wv * kCodeInstr + i) * kRowsPerInstr + lane / kSlots;
     const int chunk = code_slot<BITS>(row, lane % kSlots);  // the swizzle is its own inverse
-    w_off[i] = static_cast<uint32_t>(min(n0 + row, a.N - 1)) * w_row_bytes + chunk * 16;
+    w_off[i] = static_cast<uint32_t>(weight_row(row)) * w_row_bytes + chunk * 16;
   }
   // records: waves 0 and 1, 64 rows each; scales: waves 2..5, 64 columns each
   const uint32_t r_off = static_cast<uint32_t>(m0 + (wv & 1) * 64 + lane) * a.G * 16;
   const float* sw_lane;
   {
-    const int n = min(n0 + ((wv - 2) & 3) * 64 + lane, a.N - 1);
+    const int n = weight_row(((wv - 2) & 3) * 64 + lane);
     sw_lane = a.sw + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * a.G;
   }
 
@@ -373,6 +397,36 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   }
 
   // ---- store: register r of a 32 x 32 tile is row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
+  if constexpr (EPI == kEpiGateUpSilu) {
+    // Waves 0..3 hold the block's gate columns, 4..7 its up columns: both go to LDS as bf16 (no wave reads a
+    // stage any more: the loop's last barrier came after every wave's last operand read), then a lane takes a
+    // 16-byte chunk of a row at a time, 16 lanes a row, as act_prep_kernel does with a tensor in memory.
+    __builtin_amdgcn_s_barrier();
+    uint8_t* block = smem + (wn >> 2) * (kBM * kEpiRowBytes);
+    const int col = (wn & 3) * 32 + lm;
+#pragma unroll
+    for (int mi = 0; mi < kMT; ++mi)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+        *reinterpret_cast<uint16_t*>(block + row * kEpiRowBytes + col * 2) = bf16_bits_rne(total[mi][0][r]);
+      }
+    __syncthreads();
+    u32x4* __restrict__ next_xp = reinterpret_cast<u32x4*>(a.next_xp);
+    u32x4* __restrict__ next_rec = reinterpret_cast<u32x4*>(a.next_rec);
+#pragma unroll
+    for (int pass = 0; pass < kBM * 16 / kThreads; ++pass) {
+      const int q = pass * kThreads + tid, row = q >> 4, chunk = q & 15;
+      float g[8], u[8];
+      Pack<bf16_t>::unpack(read16(smem, row * kEpiRowBytes + chunk * 16), g);
+      Pack<bf16_t>::unpack(read16(smem, kBM * kEpiRowBytes + row * kEpiRowBytes + chunk * 16), u);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) g[e] = round_through<bf16_t>(g[e] / (1.0f + expf(-g[e]))) * u[e];
+      const int64_t at = static_cast<int64_t>(m0 + row) * a.next_G + nt;   // (row, group) of the next activation
+      emit_prepared(Pack<bf16_t>::pack(g), true, chunk == 0, next_xp + at * 16 + chunk, next_rec + at);
+    }
+    return;
+  }
   if (a.splits == 1) {
     bf16_t* __restrict__ out = static_cast<bf16_t*>(a.out);
 #pragma unroll
@@ -427,9 +481,9 @@ __global__ __launch_bounds__(256) void add_splits_kernel(const float* __restrict
   }
 }
 
-template <int BITS>
+template <int BITS, int EPI>
 int launch_tiles(const TileArgs& a, dim3 grid, hipStream_t stream) {
-  auto kernel = wq_gemm_a16_tile_kernel<BITS>;
+  auto kernel = wq_gemm_a16_tile_kernel<BITS, EPI>;
   static bool raised = false;  // per instantiation; worst case two threads both set it
   if (!raised) {
     const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -481,9 +535,11 @@ extern "C" size_t llmq_wq_gemm_a16_tile_workspace_bytes(int M, int N, int G) {
   return p.xp_bytes + p.rec_bytes + p.partial_bytes;
 }
 
-extern "C" int llmq_wq_gemm_a16_tile(const void* x, const void* qweight, const float* wscale, void* out,
-                                     void* workspace, size_t workspace_bytes, int M, int N, int G, int gs,
-                                     int out_group, int wformat, int dtype, llmq_stream_t stream) {
+namespace {
+
+// The checks the three entry points share; `x` is null when the activation is already prepared.
+int check_common(const void* x, bool prepared, const void* qweight, const float* wscale, const void* workspace, int M,
+                 int N, int G, int gs, int out_group, int wformat, int dtype) {
   if (M < 0 || N < 0 || G < 0) return llmq_host::fail_invalid("negative dimension M=%d N=%d G=%d", M, N, G);
   if (gs != kGroup) return llmq_host::fail_invalid("the tiled fused GEMM needs group_size 128, got %d", gs);
   if (dtype != LLMQ_BF16) return llmq_host::fail_invalid("the tiled fused GEMM takes bfloat16 activations, got dtype code %d", dtype);
@@ -492,35 +548,47 @@ extern "C" int llmq_wq_gemm_a16_tile(const void* x, const void* qweight, const f
   if (out_group < 0) return llmq_host::fail_invalid("out_group must be >= 0, got %d", out_group);
   if (M == 0 || N == 0) return 0;
   if (G == 0) return llmq_host::fail_invalid("a weight with no groups has no reduction axis");
-  if (!x || !qweight || !wscale || !out || !workspace) return llmq_host::fail_invalid("null tensor pointer");
-  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(qweight) | reinterpret_cast<uintptr_t>(workspace) |
-       reinterpret_cast<uintptr_t>(out)) & 15u)
+  if ((!prepared && !x) || !qweight || !wscale || !workspace) return llmq_host::fail_invalid("null tensor pointer");
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(qweight) | reinterpret_cast<uintptr_t>(workspace)) & 15u)
     return llmq_host::fail_invalid("activation, weight, output and workspace pointers must be 16-byte aligned");
   if ((static_cast<uint64_t>(M) + kBM) * G * kRowBytes >= (1ull << 32))
     return llmq_host::fail_invalid("activation of %d x %d values is beyond the kernel's 32-bit offsets", M, G * kGroup);
-  const Plan p = plan_for(M, N, G);
-  if (workspace_bytes < p.xp_bytes + p.rec_bytes + p.partial_bytes)
-    return llmq_host::fail_invalid("workspace of %zu bytes is too small, need %zu", workspace_bytes,
-                                   p.xp_bytes + p.rec_bytes + p.partial_bytes);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  uint8_t* ws = static_cast<uint8_t*>(workspace);
-  uint8_t* xp = ws;
-  uint8_t* rec = ws + p.xp_bytes;
-  float* partial = reinterpret_cast<float*>(ws + p.xp_bytes + p.rec_bytes);
+  if (static_cast<uint64_t>(N) * G * kGroup >= (1ull << 32))
+    return llmq_host::fail_invalid("weight of %d x %d codes is beyond the kernel's 32-bit offsets", N, G * kGroup);
+  return 0;
+}
 
+int prepare(const void* x, uint8_t* xp, uint8_t* rec, int M, int G, hipStream_t s) {
   const int64_t n_chunks = static_cast<int64_t>(M) * G * 16;
   hipLaunchKernelGGL(act_prep_kernel, dim3(static_cast<unsigned>((n_chunks + 255) / 256)), dim3(256), 0, s,
                      static_cast<const u32x4*>(x), reinterpret_cast<u32x4*>(xp), reinterpret_cast<u32x4*>(rec),
                      n_chunks);
-  if (int rc = llmq_host::check_launch("act_prep_kernel")) return rc;
+  return llmq_host::check_launch("act_prep_kernel");
+}
 
+// x (or, x null, the prepared activation already in the workspace) times the weight, into out.
+int run_store(const void* x, const void* qweight, const float* wscale, void* out, void* workspace,
+              size_t workspace_bytes, int M, int N, int G, int gs, int out_group, int wformat, int dtype,
+              hipStream_t s) {
+  if (int rc = check_common(x, x == nullptr, qweight, wscale, workspace, M, N, G, gs, out_group, wformat, dtype)) return rc;
+  if (M == 0 || N == 0) return 0;
+  if (!out || (reinterpret_cast<uintptr_t>(out) & 15u)) return llmq_host::fail_invalid("out must be a 16-byte aligned pointer");
+  const Plan p = plan_for(M, N, G);
+  if (workspace_bytes < p.xp_bytes + p.rec_bytes + p.partial_bytes)
+    return llmq_host::fail_invalid("workspace of %zu bytes is too small, need %zu", workspace_bytes,
+                                   p.xp_bytes + p.rec_bytes + p.partial_bytes);
+  uint8_t* ws = static_cast<uint8_t*>(workspace);
+  uint8_t* xp = ws;
+  uint8_t* rec = ws + p.xp_bytes;
+  float* partial = reinterpret_cast<float*>(ws + p.xp_bytes + p.rec_bytes);
+  if (x != nullptr) {
+    if (int rc = prepare(x, xp, rec, M, G, s)) return rc;
+  }
   TileArgs a{xp, rec, static_cast<const uint8_t*>(qweight), wscale, out, partial, M, N, G, out_group,
-             p.m_tiles, p.n_tiles, p.splits, p.groups_per_split};
+             p.m_tiles, p.n_tiles, p.splits, p.groups_per_split, nullptr, nullptr, 0};
   const int total = p.m_tiles * p.n_tiles * p.splits;
   const dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8));
-  if (static_cast<uint64_t>(N) * G * kGroup >= (1ull << 32))
-    return llmq_host::fail_invalid("weight of %d x %d codes is beyond the kernel's 32-bit offsets", N, G * kGroup);
-  if (int rc = wformat == LLMQ_W_INT4_PACKED ? launch_tiles<4>(a, grid, s) : launch_tiles<8>(a, grid, s)) return rc;
+  if (int rc = wformat == LLMQ_W_INT4_PACKED ? launch_tiles<4, kEpiStore>(a, grid, s) : launch_tiles<8, kEpiStore>(a, grid, s)) return rc;
   if (p.splits > 1) {
     const int64_t count = static_cast<int64_t>(M) * N;
     hipLaunchKernelGGL(add_splits_kernel, dim3(static_cast<unsigned>((count / 4 + 256) / 256)), dim3(256), 0, s,
@@ -528,4 +596,61 @@ extern "C" int llmq_wq_gemm_a16_tile(const void* x, const void* qweight, const f
     return llmq_host::check_launch("add_splits_kernel");
   }
   return 0;
+}
+
+}  // namespace
+
+extern "C" int llmq_wq_gemm_a16_tile(const void* x, const void* qweight, const float* wscale, void* out,
+                                     void* workspace, size_t workspace_bytes, int M, int N, int G, int gs,
+                                     int out_group, int wformat, int dtype, llmq_stream_t stream) {
+  if (M > 0 && N > 0 && !x) return llmq_host::fail_invalid("null tensor pointer");
+  return run_store(x, qweight, wscale, out, workspace, workspace_bytes, M, N, G, gs, out_group, wformat, dtype,
+                   static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmq_wq_gemm_a16_tile_prepared(const void* qweight, const float* wscale, void* out, void* workspace,
+                                              size_t workspace_bytes, int M, int N, int G, int gs, int out_group,
+                                              int wformat, int dtype, llmq_stream_t stream) {
+  return run_store(nullptr, qweight, wscale, out, workspace, workspace_bytes, M, N, G, gs, out_group, wformat, dtype,
+                   static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t llmq_wq_gemm_a16_tile_prepared_bytes(int M, int G) {
+  if (M <= 0 || G <= 0) return 0;
+  const Plan p = plan_for(M, kBN, G);   // (the prepared part of the workspace does not depend on N)
+  return p.xp_bytes + p.rec_bytes;
+}
+
+extern "C" int llmq_wq_gemm_a16_tile_gate_up_silu(const void* x, const void* qweight, const float* wscale,
+                                                  void* workspace, size_t workspace_bytes, void* next_workspace,
+                                                  size_t next_workspace_bytes, int M, int I, int G, int gs,
+                                                  int out_group, int wformat, int dtype, llmq_stream_t stream) {
+  if (I < 0 || I > (1 << 29)) return llmq_host::fail_invalid("bad intermediate size %d", I);
+  if (int rc = check_common(x, false, qweight, wscale, workspace, M, 2 * I, G, gs, out_group, wformat, dtype)) return rc;
+  if (M == 0 || I == 0) return 0;
+  if (I % (kBN / 2)) return llmq_host::fail_invalid("the intermediate size must be a multiple of %d, got %d", kBN / 2, I);
+  if (!next_workspace || (reinterpret_cast<uintptr_t>(next_workspace) & 15u))
+    return llmq_host::fail_invalid("next_workspace must be a 16-byte aligned pointer");
+  const int next_G = I / kGroup;
+  Plan p = plan_for(M, 2 * I, G);
+  const Plan next = plan_for(M, kBN, next_G);
+  if (workspace_bytes < p.xp_bytes + p.rec_bytes)
+    return llmq_host::fail_invalid("workspace of %zu bytes is too small, need %zu", workspace_bytes, p.xp_bytes + p.rec_bytes);
+  if (next_workspace_bytes < next.xp_bytes + next.rec_bytes)
+    return llmq_host::fail_invalid("next_workspace of %zu bytes is too small, need %zu", next_workspace_bytes,
+                                   next.xp_bytes + next.rec_bytes);
+  if ((static_cast<uint64_t>(M) + kBM) * next_G * kRowBytes >= (1ull << 32))
+    return llmq_host::fail_invalid("activation of %d x %d values is beyond the next GEMM's 32-bit offsets", M, I);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint8_t* ws = static_cast<uint8_t*>(workspace);
+  uint8_t* xp = ws;
+  uint8_t* rec = ws + p.xp_bytes;
+  if (int rc = prepare(x, xp, rec, M, G, s)) return rc;
+  uint8_t* nws = static_cast<uint8_t*>(next_workspace);
+  // whole reduction axis per workgroup: a tile's epilogue needs its finished totals
+  TileArgs a{xp, rec, static_cast<const uint8_t*>(qweight), wscale, nullptr, nullptr, M, 2 * I, G, out_group,
+             p.m_tiles, I / (kBN / 2), 1, G, nws, nws + next.xp_bytes, next_G};
+  const int total = a.m_tiles * a.n_tiles;
+  const dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8));
+  return wformat == LLMQ_W_INT4_PACKED ? launch_tiles<4, kEpiGateUpSilu>(a, grid, s) : launch_tiles<8, kEpiGateUpSilu>(a, grid, s);
 }

@@ -130,6 +130,13 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_wq_gemm_a16_tile.argtypes = [c_p] * 5 + [ctypes.c_size_t] + [c_int] * 7 + [c_p]
     lib.llmq_wq_gemm_a16_tile.restype = c_int
     lib.llmq_wq_gemm_a16_tile_workspace_bytes.argtypes = [c_int] * 3
+    lib.llmq_wq_gemm_a16_tile_prepared_bytes.argtypes = [c_int] * 2
+    lib.llmq_wq_gemm_a16_tile_prepared_bytes.restype = ctypes.c_size_t
+    lib.llmq_wq_gemm_a16_tile_gate_up_silu.argtypes = ([c_p] * 4 + [ctypes.c_size_t, c_p, ctypes.c_size_t] + [c_int] * 7
+                                                       + [c_p])
+    lib.llmq_wq_gemm_a16_tile_gate_up_silu.restype = c_int
+    lib.llmq_wq_gemm_a16_tile_prepared.argtypes = [c_p] * 4 + [ctypes.c_size_t] + [c_int] * 7 + [c_p]
+    lib.llmq_wq_gemm_a16_tile_prepared.restype = c_int
     lib.llmq_wq_gemm_a16_tile_workspace_bytes.restype = ctypes.c_size_t
     lib.llmq_wq_gemm_a16_workspace_bytes.argtypes = [c_int] * 3
     lib.llmq_wq_gemm_a16_workspace_bytes.restype = ctypes.c_size_t

@@ -140,6 +140,10 @@ class LlamaKernelRuntime:
             return self._ext.silu_mul(gate, up)
         return mlp.act_fn(gate) * up
 
+    def _mlp(self, index, layer, x):
+        """down_proj(act_fn(gate_proj(x)) * up_proj(x))."""
+        return layer.mlp.down_proj(self._gated(index, layer, x))
+
     def _layer(self, index, layer, hidden, cos, sin, decode: bool, branch=None, defer: bool = False):
         """One decoder layer. `branch`: the previous layer's MLP output, still to be added to `hidden`
         (done in the launch of this layer's first norm). `defer`: hand back (hidden, MLP output) and
@@ -178,7 +182,7 @@ class LlamaKernelRuntime:
                                                  is_causal=True, scale=self.scaling, enable_gqa=True)
             ctx = ctx[0].transpose(0, 1).reshape(tokens, -1)
         hidden, x = self._add_norm(layer.post_attention_layernorm, hidden, attn.o_proj(ctx))
-        out = layer.mlp.down_proj(self._gated(index, layer, x))
+        out = self._mlp(index, layer, x)
         return (hidden, out) if defer else hidden + out
 
     def _forward(self, token_ids, cos, sin, decode: bool):

@@ -163,6 +163,27 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         half = out.shape[1] // 2
         return out[:, :half], out[:, half:]
 
+    def _mlp(self, index, layer, x):
+        """A prompt's MLP in two launches where the shapes allow: the gate|up GEMM's workgroups write
+        silu(gate) * up straight into down_proj's prepared activation (the bits of the three launches: the
+        condition on the tile count is the one under which the plain gate|up GEMM keeps its reduction axis
+        whole as well)."""
+        from llmquant.quantizers.kernel import FUSED_GEMM_MAX_ROWS, TILED_GEMM_MAX_ROWS, tiled_gemm_pays
+
+        f = self.fused_layers[index]
+        gate_up, down = f["gate_up"], f["down"]
+        rows, inter = x.shape[0], gate_up.qdata.shape[0] // 2
+        if (x.dtype == torch.bfloat16 and self._one_launch_ops and "SiLU" in type(layer.mlp.act_fn).__name__
+                and FUSED_GEMM_MAX_ROWS < rows <= TILED_GEMM_MAX_ROWS and inter % 128 == 0
+                and -(-rows // 128) * (inter // 128) >= 160
+                and tiled_gemm_pays(rows, down.out_features, down.qdata.shape[1])
+                and down.bias is None and not down._needs_padding and not down._int8_act
+                and down.qdata.shape[1] * 128 == inter):
+            workspace = self._ext.wq_gemm_a16_tile_gate_up_silu(x.contiguous(), gate_up.qdata, gate_up.wscale,
+                                                                gate_up.out_group, down.out_features)
+            return self._ext.wq_gemm_a16_tile_prepared(workspace, rows, down.qdata, down.wscale, down.out_group)
+        return super()._mlp(index, layer, x)
+
     def _forward(self, token_ids, cos, sin, decode: bool):
         if not decode:
             return super()._forward(token_ids, cos, sin, decode)

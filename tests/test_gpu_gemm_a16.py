@@ -268,3 +268,75 @@ def test_module_takes_the_tiled_gemm_for_a_prompt(ext, bits, layout):
     full_scales = np.repeat(scales, og, axis=0)[:8192] if og else scales
     exact = oracle.gemv_float64(padded, canonical[cols], full_scales[cols])
     assert rel_l2(to_np(got).reshape(m, -1)[:, cols], exact) <= 2e-3
+
+
+# ---- gate|up with silu(gate) * up written as down_proj's prepared activation ------------------------------------
+
+
+def mlp_case(m, inter, k, n_down, bits, seed, out_group=0):
+    torch.manual_seed(seed)
+    x = torch.randn(m, k).to(torch.bfloat16)
+    w_gu = (torch.randn(2 * inter, k) * 0.05).to(torch.bfloat16)
+    w_d = (torch.randn(n_down, inter) * 0.05).to(torch.bfloat16)
+    c_gu, s_gu = oracle.canonical_weight(to_np(w_gu), bits, GROUP, None, out_group or None)
+    c_d, s_d = oracle.canonical_weight(to_np(w_d), bits, GROUP, None, None)
+    pack = (lambda c: oracle.pack_int4(c)) if bits == 4 else (lambda c: c)
+    return (x.cuda(), torch.from_numpy(pack(c_gu)).cuda(), torch.from_numpy(s_gu).cuda(),
+            torch.from_numpy(pack(c_d)).cuda(), torch.from_numpy(s_d).cuda(), (to_np(x), c_gu, s_gu, c_d, s_d))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,inter,k,n_down,out_group", [
+    (512, 1024, 384, 768, 0),   # whole tiles
+    (200, 256, 256, 300, 0),    # ragged rows, ragged down_proj columns
+    (65, 128, 128, 64, 0),      # one tile, one group
+    (130, 384, 512, 2048, 64),  # gate|up scales in tiles of 64 rows
+])
+def test_gate_up_silu_epilogue_gives_the_bits_of_the_three_launches(ext, bits, m, inter, k, n_down, out_group):
+    """llmq_wq_gemm_a16_tile_gate_up_silu + llmq_wq_gemm_a16_tile_prepared against llmq_wq_gemm_a16_tile ->
+    llmq_silu_mul -> llmq_wq_gemm_a16_tile on the same operands: equal to the bit. (Reduction axes of at most
+    seven groups here: there the plain tiled GEMM does not split the axis either, so its fp32 sums run in the
+    order of the fused launch's. The rounding points are the same in any case; the longer axis is below.)"""
+    x, q_gu, s_gu, q_d, s_d, _ = mlp_case(m, inter, k, n_down, bits, seed=m + inter, out_group=out_group)
+    gate_up = ext.wq_gemm_a16_tile(x, q_gu, s_gu, out_group)
+    act = ext.silu_mul(gate_up[:, :inter], gate_up[:, inter:])
+    want = ext.wq_gemm_a16_tile(act, q_d, s_d, 0)
+    workspace = ext.wq_gemm_a16_tile_gate_up_silu(x, q_gu, s_gu, out_group, n_down)
+    got = ext.wq_gemm_a16_tile_prepared(workspace, m, q_d, s_d, 0)
+    assert got.shape == want.shape == (m, n_down) and got.dtype == torch.bfloat16
+    assert torch.equal(got, want)
+    # and the transformers form of the same thing on the same bf16 tensors
+    act_hf = torch.nn.functional.silu(gate_up[:, :inter]) * gate_up[:, inter:]
+    assert torch.equal(act, act_hf)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_gate_up_silu_epilogue_against_float64_on_a_long_axis(ext, bits):
+    """The Llama-3.2-1B MLP's reduction axes (2048 into gate|up, a cut of the 8192 into down_proj) against the
+    whole MLP in float64 on the quantized weights, with the bf16 roundings of the two Linear outputs and of the
+    activation applied where the modules apply them: rel-L2 <= 3e-3 (two chained bf16 results)."""
+    m, inter, k, n_down = 256, 2048, 2048, 512
+    x, q_gu, s_gu, q_d, s_d, (xn, c_gu, sc_gu, c_d, sc_d) = mlp_case(m, inter, k, n_down, bits, seed=3)
+    workspace = ext.wq_gemm_a16_tile_gate_up_silu(x, q_gu, s_gu, 0, n_down)
+    got = ext.wq_gemm_a16_tile_prepared(workspace, m, q_d, s_d, 0)
+    bf = lambda a: torch.from_numpy(np.asarray(a, dtype=np.float32)).to(torch.bfloat16).float().numpy().astype(np.float64)
+    gu = bf(oracle.gemv_float64(xn, c_gu, sc_gu))
+    g, u = gu[:, :inter], gu[:, inter:]
+    act = bf(bf(g / (1.0 + np.exp(-g))) * u)
+    want = oracle.gemv_float64(act.astype(np.float32), c_d, sc_d)
+    assert rel_l2(to_np(got), want) <= 3e-3
+    # the three launches on the same operands: the same roundings, sums possibly in another order
+    gate_up = ext.wq_gemm_a16_tile(x, q_gu, s_gu, 0)
+    unfused = ext.wq_gemm_a16_tile(ext.silu_mul(gate_up[:, :inter], gate_up[:, inter:]), q_d, s_d, 0)
+    assert rel_l2(to_np(got), to_np(unfused).astype(np.float64)) <= 2e-3
+
+
+def test_gate_up_silu_epilogue_argument_checks(ext):
+    x, q_gu, s_gu, q_d, s_d, _ = mlp_case(128, 128, 128, 64, 4, seed=1)
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        ext.wq_gemm_a16_tile_gate_up_silu(x, q_gu[:192], s_gu[:192], 0, 64)
+    with pytest.raises(RuntimeError, match="bfloat16"):
+        ext.wq_gemm_a16_tile_gate_up_silu(x.half(), q_gu, s_gu, 0, 64)
+    workspace = ext.wq_gemm_a16_tile_gate_up_silu(x, q_gu, s_gu, 0, 64)
+    with pytest.raises(RuntimeError, match="this GEMM needs"):
+        ext.wq_gemm_a16_tile_prepared(workspace[:16], 128, q_d, s_d, 0)
