@@ -358,3 +358,57 @@ def test_split_attention_argument_checks(ext):
         ext.wq_gemv_attn_merge(partials, 8, 64, q, s, 0, 0, None, torch.bfloat16)
     with pytest.raises(RuntimeError, match="whole number of heads"):
         ext.wq_gemv_attn_merge(torch.zeros(4096, device="cuda"), 2, 96, q, s, 0, 0, None, torch.bfloat16)
+
+
+def test_prompt_pass_with_its_own_attention_and_two_launch_mlp():
+    """A 300-token prompt through a model whose MLP is wide enough for the two-launch form (gate|up with
+    silu(gate) * up written as down_proj's prepared activation: 3 x 64 tiles) and whose attention goes through
+    llmq_prefill_attention, against the same runtime with the MLP as three launches (bit-equal: hidden states of
+    every layer, the cache, the token) and with torch's scaled_dot_product_attention for the prompt (floating
+    point: the first layer's cache codes equal, the second's within one step of each other, logits of the last position to
+    rel-L2 <= 2e-2, the bound the fused and unfused steps are held to)."""
+    from test_gpu_decode import build_model, quantized_pair
+
+    from llmquant.runtime import LlamaFusedRuntime, LlamaKernelRuntime
+
+    _, kernel = quantized_pair(build_model(512, 8192, 2, 8, 2, 4096))
+    ids = torch.randint(0, 4096, (1, 300), generator=torch.Generator().manual_seed(2)).cuda()
+    calls = {"mlp": 0, "attn": 0}
+
+    class Counting(LlamaFusedRuntime):
+        def _mlp(self, index, layer, x):
+            out = super()._mlp(index, layer, x)
+            calls["mlp"] += 1
+            return out
+
+    class ThreeLaunchMlp(LlamaFusedRuntime):
+        def _mlp(self, index, layer, x):
+            return LlamaKernelRuntime._mlp(self, index, layer, x)
+
+    class LibraryAttention(LlamaFusedRuntime):
+        PROMPT_ATTENTION_MAX_TOKENS = {}
+
+    fused = Counting(kernel, 320, 8)
+    # (the two-launch path is the one that runs: its extension call is made once per layer)
+    ext_calls = []
+    real_call = fused._ext.wq_gemm_a16_tile_gate_up_silu
+    try:
+        fused._ext.wq_gemm_a16_tile_gate_up_silu = lambda *a, **k: (ext_calls.append(1), real_call(*a, **k))[1]
+        tok = fused.prefill(ids)
+    finally:
+        fused._ext.wq_gemm_a16_tile_gate_up_silu = real_call
+    assert calls["mlp"] == 2 and len(ext_calls) == 2
+    three = ThreeLaunchMlp(kernel, 320, 8)
+    assert torch.equal(three.prefill(ids), tok)
+    for name in ("k_codes", "v_codes", "k_scale", "v_scale"):
+        assert torch.equal(getattr(three.cache, name), getattr(fused.cache, name)), name
+    logits_fused, _ = fused.eager_step(tok, 300)
+    logits_three, _ = three.eager_step(tok, 300)
+    assert torch.equal(logits_fused, logits_three)
+    library = LibraryAttention(kernel, 320, 8)
+    library.prefill(ids)
+    logits_library, _ = library.eager_step(tok, 300)
+    assert rel_l2(to_np(logits_fused), to_np(logits_library)) <= 2e-2
+    assert torch.equal(library.cache.k_codes[0, :, :300], fused.cache.k_codes[0, :, :300])
+    step = (library.cache.k_codes[1, :, :300].int() - fused.cache.k_codes[1, :, :300].int()).abs()
+    assert float((step <= 1).float().mean()) > 0.99 and int(step.max()) <= 3
