@@ -260,6 +260,7 @@ extern "C" int llmq_prefill_attention(const void* q, const void* k, const void* 
                                       int kv_heads, int head_dim, float scale, int dtype, llmq_stream_t stream) {
   if (tokens < 0 || q_heads <= 0 || kv_heads <= 0) return llmq_host::fail_invalid("bad shape: tokens=%d q_heads=%d kv_heads=%d", tokens, q_heads, kv_heads);
   if (q_heads % kv_heads != 0) return llmq_host::fail_invalid("q_heads %d is not a multiple of kv_heads %d", q_heads, kv_heads);
+  if (q_heads > 65535) return llmq_host::fail_invalid("at most 65535 query heads (one grid row each), got %d", q_heads);
   if (head_dim != 64 && head_dim != 128) return llmq_host::fail_invalid("head_dim must be 64 or 128, got %d", head_dim);
   if (!(scale > 0.0f) || scale > 3.0e38f) return llmq_host::fail_invalid("scale must be positive and finite, got %g", static_cast<double>(scale));
   if (dtype != LLMQ_F16 && dtype != LLMQ_BF16) return llmq_host::fail_invalid("q, k, v must be float16 or bfloat16, got dtype code %d", dtype);
