@@ -340,3 +340,28 @@ def test_gate_up_silu_epilogue_argument_checks(ext):
     workspace = ext.wq_gemm_a16_tile_gate_up_silu(x, q_gu, s_gu, 0, 64)
     with pytest.raises(RuntimeError, match="this GEMM needs"):
         ext.wq_gemm_a16_tile_prepared(workspace[:16], 128, q_d, s_d, 0)
+
+
+def test_gate_up_silu_epilogue_at_the_llama_1b_prompt_shape(ext):
+    """The MLP of a 512-token prompt of the Llama-3.2-1B configuration (2048 -> 2 x 8192 -> 2048, int4): 4 x 64
+    tiles, the shape the runtime takes this path on. Bit-equal to the three launches (the plain gate|up GEMM has
+    256 tiles and keeps its reduction axis whole too; down_proj's plan is the same in both), and the prepared
+    activation the epilogue leaves is, byte for byte, what the preparation pass makes of silu(gate) * up."""
+    m, inter, k, n_down = 512, 8192, 2048, 2048
+    torch.manual_seed(11)
+    x = torch.randn(m, k, device="cuda").to(torch.bfloat16)
+    q_gu = torch.randint(0, 256, (2 * inter, k // GROUP, GROUP // 2), dtype=torch.uint8, device="cuda")
+    s_gu = torch.rand(2 * inter, k // GROUP, device="cuda") * 0.004 + 0.001
+    q_d = torch.randint(0, 256, (n_down, inter // GROUP, GROUP // 2), dtype=torch.uint8, device="cuda")
+    s_d = torch.rand(n_down, inter // GROUP, device="cuda") * 0.004 + 0.001
+    gate_up = ext.wq_gemm_a16_tile(x, q_gu, s_gu, 0)
+    act = ext.silu_mul(gate_up[:, :inter], gate_up[:, inter:])
+    want = ext.wq_gemm_a16_tile(act, q_d, s_d, 0)
+    workspace = ext.wq_gemm_a16_tile_gate_up_silu(x, q_gu, s_gu, 0, n_down)
+    prepared = workspace.view(torch.uint8)[: m * inter * 2].clone()
+    got = ext.wq_gemm_a16_tile_prepared(workspace, m, q_d, s_d, 0)
+    assert torch.equal(got, want)
+    assert float(want.float().abs().mean()) > 0
+    # the chunks: eight consecutive bf16 values in the order (0, 4, 1, 5, 2, 6, 3, 7)
+    chunks = act.view(m, inter // 8, 8)[:, :, [0, 4, 1, 5, 2, 6, 3, 7]].contiguous()
+    assert torch.equal(prepared, chunks.view(torch.uint8).flatten())
