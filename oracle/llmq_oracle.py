@@ -430,3 +430,23 @@ def gqa_decode_attention(q, k, v, sm_scale, dtype="bf16"):
         p = np.exp(s - s.max())
         out[h] = (p / p.sum()) @ vv
     return round_to(out.astype(np.float32), dtype)
+
+
+def gqa_prompt_attention(q, k, v, sm_scale) -> np.ndarray:
+    """A whole prompt, causal and grouped-query: query i sees keys 0..i. q: [T, Hq, D]; k, v: [Hkv, T, D]
+    (the values FakeQuantCache.update hands back, fake.py:39-55, which is what the reference's prompt pass
+    gives transformers' attention). softmax(q k^T * sm_scale + causal mask) v in float64 -> [T, Hq * D]
+    float64 (unrounded: the tolerance anchor of the GPU kernel)."""
+    q = np.asarray(q, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    v = np.asarray(v, dtype=np.float64)
+    tokens, hq, d = q.shape
+    rep = hq // k.shape[0]
+    out = np.zeros((tokens, hq, d))
+    hidden = np.triu(np.ones((tokens, tokens), dtype=bool), 1)   # key j > query i
+    for h in range(hq):
+        s = (q[:, h] @ k[h // rep].T) * sm_scale
+        s[hidden] = -np.inf
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        out[:, h] = (p / p.sum(axis=1, keepdims=True)) @ v[h // rep]
+    return out.reshape(tokens, hq * d)

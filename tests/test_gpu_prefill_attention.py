@@ -1,6 +1,6 @@
-"""Causal grouped-query attention of a prompt (llmq_prefill_attention) against the definition computed in
-float64 on the host, and against torch's scaled_dot_product_attention, which is what the reference's prompt
-pass runs on the K / V its FakeQuantCache returns (llmquant/quantizers/fake.py:39-55).
+"""Causal grouped-query attention of a prompt (llmq_prefill_attention) against the oracle's float64
+restatement (oracle.gqa_prompt_attention), and against torch's scaled_dot_product_attention, which is what the
+reference's prompt pass runs on the K / V its FakeQuantCache returns (llmquant/quantizers/fake.py:39-55).
 
 Floating point, so a tolerance: the kernel accumulates scores and the weighted sum in fp32 and rounds the
 probabilities to the 16-bit type before they meet V, as the library's flash kernel does. Against float64 the
@@ -14,6 +14,8 @@ import numpy as np
 import pytest
 import torch
 
+import llmq_oracle as oracle
+
 pytestmark = pytest.mark.gpu
 
 
@@ -25,17 +27,9 @@ def ext():
 
 
 def causal_gqa_float64(q, k, v, scale):
-    """q [T, Hq, D]; k, v [Hkv, T, D] (any float dtype, CPU) -> [T, Hq * D] in float64."""
-    q, k, v = q.double(), k.double(), v.double()
-    tokens, q_heads, d = q.shape
-    rep = q_heads // k.shape[0]
-    out = torch.empty(tokens, q_heads, d, dtype=torch.float64)
-    mask = torch.ones(tokens, tokens, dtype=torch.bool).tril()
-    for h in range(q_heads):
-        s = (q[:, h] @ k[h // rep].T) * scale
-        s = s.masked_fill(~mask, float("-inf"))
-        out[:, h] = torch.softmax(s, dim=-1) @ v[h // rep]
-    return out.reshape(tokens, q_heads * d)
+    """q [T, Hq, D]; k, v [Hkv, T, D] (16-bit tensors on the CPU) -> [T, Hq * D] in float64: the oracle's
+    restatement of what the reference's prompt pass computes."""
+    return torch.from_numpy(oracle.gqa_prompt_attention(q.float().numpy(), k.float().numpy(), v.float().numpy(), scale))
 
 
 def make(tokens, q_heads, kv_heads, d, dtype, seed, spread=1.0):

@@ -375,6 +375,34 @@ def test_attention_matches_the_library_routines_the_reference_delegates_to():
     assert not np.allclose(wrong, eager[0, 0].numpy(), rtol=1e-2, atol=1e-2)
 
 
+def test_prompt_attention_is_the_decode_attention_of_every_prefix_and_the_library_routine():
+    """The causal form, pinned three ways: row i equals the one-token attention of query i over keys 0..i
+    (the function above, itself pinned against transformers); it equals torch's scaled_dot_product_attention
+    with is_causal and enable_gqa, the call the reference's prompt pass ends in (fp32 library arithmetic
+    against float64: 1e-5), on unequal head counts, a scale other than 1 and kv heads that all differ; and a mask
+    turned the wrong way round (queries seeing the future) is far outside that tolerance."""
+    import torch
+
+    rng = np.random.default_rng(8)
+    t, hq, hkv, d = 23, 6, 2, 16
+    q = rng.standard_normal((t, hq, d)).astype(np.float32)
+    k = rng.standard_normal((hkv, t, d)).astype(np.float32) * 1.5
+    v = rng.standard_normal((hkv, t, d)).astype(np.float32)
+    scale = 0.37
+    mine = oracle.gqa_prompt_attention(q, k, v, scale)
+    assert mine.shape == (t, hq * d) and mine.dtype == np.float64
+    for i in (0, 1, 7, t - 1):
+        row = oracle.gqa_decode_attention(q[i], k[:, : i + 1], v[:, : i + 1], scale, "f32")
+        assert np.allclose(mine[i].reshape(hq, d), row, rtol=1e-6, atol=1e-6)
+    assert np.array_equal(mine[0].reshape(hq, d)[0], v[0, 0].astype(np.float64))
+    sdpa = torch.nn.functional.scaled_dot_product_attention(
+        torch.from_numpy(q).transpose(0, 1)[None], torch.from_numpy(k)[None], torch.from_numpy(v)[None],
+        is_causal=True, scale=scale, enable_gqa=True)[0].transpose(0, 1).reshape(t, hq * d).numpy()
+    assert np.allclose(mine, sdpa, rtol=1e-5, atol=1e-5)
+    backwards = oracle.gqa_prompt_attention(q[::-1], k[:, ::-1], v[:, ::-1], scale)[::-1]
+    assert not np.allclose(backwards, sdpa, rtol=1e-2, atol=1e-2)
+
+
 # ---- the C oracle says the same ----------------------------------------------------------------------------
 
 @pytest.fixture(scope="module")
