@@ -59,7 +59,7 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the legs that report the path's other kernels and end-to-end decode")
-    ap.add_argument("--only", choices=("other", "decode", "prefill"), default=None,
+    ap.add_argument("--only", choices=("other", "decode", "prefill", "decode8b"), default=None,
                     help="profiling aid: run just that leg and print its JSON (not the bench line)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="first run a plain 256 MiB device copy three times: the known-size kernel that "
@@ -116,7 +116,8 @@ def main():
     lib = load_capi()
     torch.cuda.set_device(0)
     if opts.only:
-        leg = {"other": other_kernels, "decode": decode_leg, "prefill": prefill_leg}[opts.only](torch)
+        leg = {"other": other_kernels, "decode": decode_leg, "prefill": prefill_leg,
+               "decode8b": lambda t: decode_leg(t, arch="llama3-8b")}[opts.only](torch)
         print(json.dumps({opts.only: leg}))
         return
     if opts.copy_probe:
@@ -623,11 +624,13 @@ def other_kernels(torch):
     return out
 
 
-def decode_leg(torch):
+def decode_leg(torch, arch="llama3.2-1b"):
     """The end-to-end decode case: random-init Llama-3.2-1B architecture, attention int8 / MLP int4 /
     lm_head int8 / int8 KV cache, 512-token prompt, 256 greedy tokens, batch 1. TTFT = median
     time of generating 1 token; decode tok/s = (n - 1) / (median time of n tokens - TTFT), the
-    reference's definition (llmquant/eval/evaluate.py:209-218). Both sides replay a captured step."""
+    reference's definition (llmquant/eval/evaluate.py:209-218). Both sides replay a captured step.
+    arch "llama3-8b": the same on the Llama-3-8B architecture (the other model of the layer-shape target; not
+    part of the default run), 128 new tokens."""
     import time
 
     from transformers import LlamaConfig, LlamaForCausalLM
@@ -635,16 +638,18 @@ def decode_leg(torch):
     from llmquant import QuantConfig, oneshot
 
     torch.manual_seed(0)
-    cfg = LlamaConfig(hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, num_attention_heads=32,
-                      num_key_value_heads=8, head_dim=64, vocab_size=128256, rms_norm_eps=1e-5,
+    shape = {"llama3.2-1b": dict(hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, head_dim=64),
+             "llama3-8b": dict(hidden_size=4096, intermediate_size=14336, num_hidden_layers=32, head_dim=128)}[arch]
+    cfg = LlamaConfig(num_attention_heads=32, num_key_value_heads=8, vocab_size=128256, rms_norm_eps=1e-5,
                       rope_parameters={"rope_type": "default", "rope_theta": 500000.0},
-                      tie_word_embeddings=False, max_position_embeddings=4096)
-    model = LlamaForCausalLM(cfg)
+                      tie_word_embeddings=False, max_position_embeddings=4096, **shape)
+    with torch.device("cuda:0" if arch == "llama3-8b" else "cpu"):   # (16 GB of bf16: built where it will live)
+        model = LlamaForCausalLM(cfg)
     for p in model.parameters():
         if p.dim() > 1:
             torch.nn.init.normal_(p, 0, 0.02)
     model = model.to(torch.bfloat16).to("cuda:0").eval()
-    prompt, new = 512, 256
+    prompt, new = 512, (256 if arch == "llama3.2-1b" else 128)
     from llmquant.eval import latency_row, measure_latency, reconcile
 
     def measure(kv_bits):
@@ -652,7 +657,7 @@ def decode_leg(torch):
                               kv_bits=kv_bits)
         return lat, {"ttft_ms": round(lat["ttft_ms"], 2), "decode_tok_s": round(lat["decode_tps"], 1)}
 
-    res = {"prompt_tokens": prompt, "new_tokens": new, "hip_graph": True,
+    res = {"architecture": arch, "prompt_tokens": prompt, "new_tokens": new, "hip_graph": True,
            "paths": {"bf16": "HF LlamaForCausalLM module walk over a StaticCache, one captured step, kept between "
                              "calls (hf_static_cache_graph)",
                      "kernel": "LlamaFusedRuntime: five launches per layer, integer KV cache, one captured step, "

@@ -22,12 +22,12 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-def build_model(hidden, inter, layers, heads, kv_heads, vocab, seed=0):
+def build_model(hidden, inter, layers, heads, kv_heads, vocab, seed=0, head_dim=64):
     from transformers import LlamaConfig, LlamaForCausalLM
 
     torch.manual_seed(seed)
     cfg = LlamaConfig(hidden_size=hidden, intermediate_size=inter, num_hidden_layers=layers,
-                      num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=64, vocab_size=vocab,
+                      num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=head_dim, vocab_size=vocab,
                       rms_norm_eps=1e-5, rope_parameters={"rope_type": "default", "rope_theta": 500000.0},
                       tie_word_embeddings=False, max_position_embeddings=4096)
     model = LlamaForCausalLM(cfg)
@@ -131,6 +131,18 @@ def test_teacher_forced_margin_small(small):
     rows, _, _ = teacher_forced(real, kernel, 48, 64, 4096)
     agree = check_margin(rows, 0.05)
     print(f"teacher-forced agreement {agree}/{len(rows)}")
+    assert agree >= 0.8 * len(rows)
+
+
+@pytest.mark.parametrize("runtime", ["walk", "fused"])
+def test_teacher_forced_margin_with_heads_of_128(runtime):
+    """The Llama-3-8B head geometry (head_dim 128: no padding of heads to groups, attention kernels of the other
+    head size) on a small model, with a prompt long enough for the prompt pass's own attention kernel and, in the
+    fused runtime, the two-launch MLP: both runtimes against the real-mode model under the same margin rule."""
+    real, kernel = quantized_pair(build_model(512, 7168, 2, 4, 2, 4096, seed=3, head_dim=128))
+    rows, _, _ = teacher_forced(real, kernel, 300, 24, 4096, runtime=runtime)
+    agree = check_margin(rows, 0.05)
+    print(f"teacher-forced agreement, heads of 128, {runtime}: {agree}/{len(rows)}")
     assert agree >= 0.8 * len(rows)
 
 
