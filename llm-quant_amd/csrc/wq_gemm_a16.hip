@@ -19,10 +19,14 @@
 //   weights   16 rows x 64 B (4-bit) or 128 B (8-bit), 16 or 32 bytes per lane, straight from HBM
 //             in operand layout: lane = (row j = lane % 16, block = lane / 16) holds k = 32 block ..
 //             32 block + 31, eight of them per MFMA step
-//   x         for each tile of 16 activation rows, the same 32 k of row (lane % 16): 64 contiguous
-//             bytes per lane; x is small and stays in L2
-// and issues 4 MFMAs per activation tile. Rows past M or N are clamped for the loads and dropped
-// at the store, so the load sequence is the same for every lane.
+//   x         the group's 128 values of every activation row, through the wave's own LDS tile: whole rows
+//             go there straight from L2 (global_load_lds_dwordx4: four rows of 256 bytes per instruction, eight
+//             cache lines; as operand loads, 64 bytes per lane at a row each, the same bytes were 64 lines per
+//             instruction and the address unit, not memory, set the pace), 16-byte slots XOR-swizzled by row,
+//             and come out as operands: the 32 k of row (lane % 16) that the lane's codes belong to
+// and issues 4 MFMAs per activation tile. The next group's transfer and codes are requested once this group's
+// operands are in registers. Rows past M or N are clamped for the loads and dropped at the store, so the load
+// sequence is the same for every lane.
 #include "llmq_device.h"
 
 namespace {
@@ -108,11 +112,29 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void wq_gemm_a16_kernel(const A1
     wrow[nt] = a.qw + static_cast<int64_t>(n) * a.row_bytes + blk * (BITS == 4 ? 16 : 32);
     srow[nt] = a.ws + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * G;
   }
-  const T* xrow[MT];
+  // ---- x of one group: [16 MT rows][16 slots of 16 bytes], slot p of row r holds chunk p ^ (r & 15) ------------
+  // transfer i of the wave covers rows 4 i .. 4 i + 3; lane = (row 4 i + lane / 16, slot lane % 16)
+  constexpr int kXInstr = MT * 4;
+  constexpr int kXTileBytes = MT * kTileM * kGroup * 2;
+  unsigned char* xtile = smem + wv * kXTileBytes;
+  const unsigned char* xsrc[kXInstr];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    xrow[mt] = static_cast<const T*>(a.x) + static_cast<int64_t>(min(mt * kTileM + j, a.M - 1)) * K + blk * 32;
+  for (int i = 0; i < kXInstr; ++i) {
+    const int row = 4 * i + (lane >> 4), chunk = (lane & 15) ^ (row & 15);
+    xsrc[i] = reinterpret_cast<const unsigned char*>(static_cast<const T*>(a.x) + static_cast<int64_t>(min(row, a.M - 1)) * K +
+                                                     chunk * 8);
   }
+  auto request_rows = [&](int g) {
+#pragma unroll
+    for (int i = 0; i < kXInstr; ++i) {
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(xsrc[i] + static_cast<int64_t>(g) * (kGroup * 2)),
+                                       reinterpret_cast<u32x4*>(xtile + 1024 * i), 16, 0, 0);
+    }
+  };
+  // operand of step s, tile mt: row 16 mt + j, chunk 4 blk + s
+  uint32_t x_at[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) x_at[mt] = static_cast<uint32_t>((mt * kTileM + j) * (kGroup * 2));
 
   struct Weights {
     uint32_t raw[NT][kRaw];
@@ -133,11 +155,13 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void wq_gemm_a16_kernel(const A1
       W.scale[nt] = srow[nt][g];
     }
   };
-  auto load_rows = [&](int g, Rows& X) {
+  auto read_rows = [&](Rows& X) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
-      for (int s = 0; s < 4; ++s) X.xa[mt][s] = load16(xrow[mt] + static_cast<int64_t>(g) * kGroup + 8 * s);
+      for (int s = 0; s < 4; ++s) {
+        X.xa[mt][s] = *reinterpret_cast<const u32x4*>(xtile + x_at[mt] + (((4 * blk + s) ^ j) << 4));
+      }
     }
   };
 
@@ -165,17 +189,30 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void wq_gemm_a16_kernel(const A1
     }
   };
 
-  // The wave's groups wv, wv + wk, ... Loads are written next to their use: the compiler would sink
-  // them there anyway, and on this kernel that order measured faster than register sets filled a
-  // group or several ahead; the latency is covered by the other waves of the CU (60-130 registers:
-  // three to six waves per SIMD).
-  for (int g = wv; g < G; g += wk) {
-    Weights W;
-    Rows X;
-    load_weights(g, W);
-    load_rows(g, X);
-    multiply(W, X);
+  // The wave's groups wv, wv + wk, ...: this group's rows and codes have arrived (nothing else of the wave is in
+  // flight), the rows go from the tile to registers, and with the tile free again the next group's transfer
+  // and codes are requested, to arrive under this group's multiplications.
+  Weights W0, W1;
+  if (wv < G) {
+    request_rows(wv);
+    load_weights(wv, W0);
   }
+  auto step = [&](int g, const Weights& now, Weights& next) {
+    Rows X;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    read_rows(X);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (g + wk < G) {
+      request_rows(g + wk);
+      load_weights(g + wk, next);
+    }
+    multiply(now, X);
+  };
+  for (int g = wv; g < G; g += 2 * wk) {   // (two groups a round: the register sets swap by name)
+    step(g, W0, W1);
+    if (g + wk < G) step(g + wk, W1, W0);
+  }
+  __syncthreads();   // every wave is done with its tile: the partial sums take the same memory
 
   // ---- waves meet: part[wave][m][n], summed in wave order ---------------------------------------
 #pragma unroll
@@ -200,8 +237,24 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void wq_gemm_a16_kernel(const A1
 template <typename T, int BITS, int MT, int NT>
 int launch_tile(const A16Args& a, int wk, hipStream_t stream) {
   const int grid = (a.N + NT * kTileN - 1) / (NT * kTileN);
-  const int lds = wk * MT * kTileM * NT * kTileN * static_cast<int>(sizeof(float));
-  hipLaunchKernelGGL((wq_gemm_a16_kernel<T, BITS, MT, NT>), dim3(grid), dim3(wk * kWave), lds, stream, a);
+  // the waves' activation tiles, then (the same memory) their partial sums
+  const int part = wk * MT * kTileM * NT * kTileN * static_cast<int>(sizeof(float));
+  const int tiles = wk * MT * kTileM * kGroup * 2;
+  const int lds = part > tiles ? part : tiles;
+  auto kernel = wq_gemm_a16_kernel<T, BITS, MT, NT>;
+  if (lds > 64 * 1024) {
+    static bool raised = false;  // per instantiation; worst case two threads both set it
+    if (!raised) {
+      const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kMaxWaves * MT * kTileM * kGroup * 2);
+      if (err != hipSuccess) {
+        llmq_host::set_error("raising the LDS limit failed: %s", hipGetErrorString(err));
+        return static_cast<int>(err);
+      }
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(wk * kWave), lds, stream, a);
   return llmq_host::check_launch("wq_gemm_a16_kernel");
 }
 
