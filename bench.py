@@ -586,7 +586,7 @@ def other_kernels(torch):
             us_whole = _graph_time_us(torch, fused_sweep, reps=5) / copies
             us_split = _graph_time_us(torch, split_sweep, reps=5) / copies
             us_dense = _graph_time_us(torch, dense_sweep, reps=5) / copies
-            us = us_split if (m > 16 or k // GROUP >= 64) else us_whole  # KernelQuantLinear's choice (fused_gemm_splits)
+            us = us_whole  # KernelQuantLinear's choice (fused_gemm_splits: the whole-rows form everywhere)
             nbytes = nbytes_w + m * k * 2 + m * n * 2
             fused.append({"M": m, "N": n, "K": k, "weights": "int4", "us": round(us, 2),
                           "whole_rows_form_us": round(us_whole, 2), "split_form_us": round(us_split, 2),

@@ -235,6 +235,77 @@ __device__ __forceinline__ void merge_partials8(const float* rec, int n_splits, 
   for (int e = 0; e < 8; ++e) f[e] *= inv;
 }
 
+// ---- codes as 16-bit matrix-core operands without a conversion instruction -------------------------------
+// A 4-bit code is stored with a bias of 8 (n = code + 8, 0..15); placed in the mantissa of 16.0 it IS the value
+// 16 + n in bf16 (0x4180 | n << 3) and in fp16 (0x4c00 | n << 6), two codes per AND-OR. An 8-bit code with its
+// sign bit flipped is b = code + 128 (0..255): fp16 holds 256 + b as 0x5c00 | b << 2 (a byte permute and a
+// shift-OR per two codes); bf16 has seven mantissa bits, so there b goes through v_cvt_f32_ubyte, whose upper
+// half is the bf16 value. What the matrix core then sums is x (code + kBias); kBias sum x comes out again per
+// group (the products are exact in fp32 either way). Operand element order: the eight codes of a 32-bit word of
+// int4 (two of int8) as (0, 4, 1, 5, 2, 6, 3, 7): the other operand's 16-byte chunks must be in the same
+// order (interleave_halves), which a sum over k does not mind.
+__device__ __forceinline__ uint32_t and_or(uint32_t value, uint32_t mask_scalar, uint32_t bits) {
+  // (value & mask) | bits in one instruction; the compiler leaves it as two. One operand of a VOP3 may come
+  // from a scalar register on this chip, so the mask is scalar and the bits sit in a vector register.
+  uint32_t d;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(value), "s"(mask_scalar), "v"(bits));
+  return d;
+}
+// (x0 x1)(x2 x3)(x4 x5)(x6 x7) -> (x0 x4)(x1 x5)(x2 x6)(x3 x7), 16-bit elements
+__device__ __forceinline__ u32x4 interleave_halves(const u32x4 v) {
+  u32x4 o;
+  o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+  o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+  o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+  o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+  return o;
+}
+template <typename T, int BITS> struct BiasedCodes;
+template <> struct BiasedCodes<bf16_t, 4> {
+  static constexpr float kBias = 24.0f;
+  static constexpr uint32_t kMagic = 0x41804180u;   // keep it in a vector register: asm volatile("" : "+v"(magic))
+  // raw: the lane's codes of a group; step: which eight of them
+  static __device__ __forceinline__ u32x4 operand(const uint32_t* raw, int step, uint32_t magic) {
+    const uint32_t w = raw[step];
+    return u32x4{and_or(w << 3, 0x00780078u, magic), and_or(w >> 1, 0x00780078u, magic),
+                 and_or(w >> 5, 0x00780078u, magic), and_or(w >> 9, 0x00780078u, magic)};
+  }
+};
+template <> struct BiasedCodes<f16_t, 4> {
+  static constexpr float kBias = 24.0f;
+  static constexpr uint32_t kMagic = 0x4c004c00u;
+  static __device__ __forceinline__ u32x4 operand(const uint32_t* raw, int step, uint32_t magic) {
+    const uint32_t w = raw[step];
+    return u32x4{and_or(w << 6, 0x03c003c0u, magic), and_or(w << 2, 0x03c003c0u, magic),
+                 and_or(w >> 2, 0x03c003c0u, magic), and_or(w >> 6, 0x03c003c0u, magic)};
+  }
+};
+template <> struct BiasedCodes<bf16_t, 8> {
+  static constexpr float kBias = 128.0f;
+  static constexpr uint32_t kMagic = 0u;
+  static __device__ __forceinline__ u32x4 operand(const uint32_t* raw, int step, uint32_t) {
+    const uint32_t w0 = raw[2 * step] ^ 0x80808080u, w1 = raw[2 * step + 1] ^ 0x80808080u;   // codes 0..3, 4..7
+    uint32_t out[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float lo = static_cast<float>((w0 >> (8 * i)) & 0xffu), hi = static_cast<float>((w1 >> (8 * i)) & 0xffu);
+      // integers below 256: the upper half of the float is the bf16 value, exactly
+      out[i] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, hi), __builtin_bit_cast(uint32_t, lo), 0x07060302u);
+    }
+    return u32x4{out[0], out[1], out[2], out[3]};
+  }
+};
+template <> struct BiasedCodes<f16_t, 8> {
+  static constexpr float kBias = 384.0f;
+  static constexpr uint32_t kMagic = 0x5c005c00u;
+  static __device__ __forceinline__ u32x4 operand(const uint32_t* raw, int step, uint32_t magic) {
+    const uint32_t w0 = raw[2 * step] ^ 0x80808080u, w1 = raw[2 * step + 1] ^ 0x80808080u;
+    // byte i of w0 into the low half, byte i of w1 into the high half, zeros above each
+    return u32x4{(__builtin_amdgcn_perm(w1, w0, 0x0c040c00u) << 2) | magic, (__builtin_amdgcn_perm(w1, w0, 0x0c050c01u) << 2) | magic,
+                 (__builtin_amdgcn_perm(w1, w0, 0x0c060c02u) << 2) | magic, (__builtin_amdgcn_perm(w1, w0, 0x0c070c03u) << 2) | magic};
+  }
+};
+
 }  // namespace llmq
 
 // ---- host-side error plumbing -----------------------------------------------------------------

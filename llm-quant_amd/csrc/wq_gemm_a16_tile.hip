@@ -138,14 +138,7 @@ template <int BITS> __device__ __forceinline__ int code_slot(int row, int c) {
   return BITS == 4 ? c ^ ((row >> 2) & 3) : c ^ ((row >> 1) & 7);
 }
 
-// (value & mask) | bits in one instruction; the compiler leaves it as two. One operand of a VOP3 may
-// come from a scalar register on this chip, so the mask is scalar and the bits sit in a vector register.
-constexpr uint32_t kNibbleMask = 0x00780078u;
-__device__ __forceinline__ uint32_t and_or(uint32_t value, uint32_t mask_scalar, uint32_t bits) {
-  uint32_t d;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(value), "s"(mask_scalar), "v"(bits));
-  return d;
-}
+constexpr uint32_t kNibbleMask = 0x00780078u;   // (and_or: (value & mask) | bits in one instruction)
 
 // Two of the four operand words of a k-step: a k-step's eight codes are one 32-bit word of int4 or two of
 // int8; operand word i pairs codes i and i + 4. `half` selects words (0, 1) or (2, 3).

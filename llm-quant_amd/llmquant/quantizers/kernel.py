@@ -23,16 +23,17 @@ from llmquant.quantizers.real import quantize_weight
 KERNEL_MAX_ROWS = 4
 #: ... except that up to this many rows of a 16-bit activation go to the fused GEMM, which reads
 #: the codes once and builds no dense weight (the measured crossover with dequantize + matmul).
-#: Up to FUSED_GEMM_WHOLE_ROWS rows in its one-launch form (a workgroup owns whole weight rows),
-#: above that, and for rows of FUSED_GEMM_SPLIT_GROUPS groups or more (down_proj), in the form
-#: that splits the reduction axis across workgroups (two launches, flat in the row count).
+#: In its one-launch form (a workgroup owns whole weight rows) at every row count: since the activation
+#: reaches the matrix core through LDS that form is the faster one on every shape measured (Llama-3.2-1B and
+#: Llama-3-8B layers, lm_head), by 5-40 %; the form that splits the reduction axis across workgroups (two
+#: launches) stays available through the extension (`split=True`).
 FUSED_GEMM_MAX_ROWS = 64
-FUSED_GEMM_WHOLE_ROWS = 16
+FUSED_GEMM_WHOLE_ROWS = FUSED_GEMM_MAX_ROWS
 #: ... and from this many rows on it is also faster than the GEMV kernel, which multiplies its rows
 #: as int8 digit planes and slows down with each row (14336 x 4096 int4, graph replay: GEMV 9.6 /
 #: 13.0 / 14.8 / 21.0 us for 1-4 rows, the fused GEMM 13.4-14.3 us for any of them)
 FUSED_GEMM_MIN_ROWS = 3
-FUSED_GEMM_SPLIT_GROUPS = 64
+FUSED_GEMM_SPLIT_GROUPS = 1 << 30   # (no row is long enough for the split form to win)
 
 
 #: Prompt-sized bf16 activations: the tiled fused GEMM (128 x 256 output tiles, no dense weight) up to this
