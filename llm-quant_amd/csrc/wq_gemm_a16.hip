@@ -128,8 +128,12 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void wq_gemm_a16_kernel(const A1
   auto request_rows = [&](int g) {
 #pragma unroll
     for (int i = 0; i < kXInstr; ++i) {
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(xsrc[i] + static_cast<int64_t>(g) * (kGroup * 2)),
-                                       reinterpret_cast<u32x4*>(xtile + 1024 * i), 16, 0, 0);
+      // (four rows past the activation's end are not fetched: what the tile holds there feeds only result rows
+      // that are dropped at the store)
+      if (4 * i < a.M) {
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(xsrc[i] + static_cast<int64_t>(g) * (kGroup * 2)),
+                                         reinterpret_cast<u32x4*>(xtile + 1024 * i), 16, 0, 0);
+      }
     }
   };
   // operand of step s, tile mt: row 16 mt + j, chunk 4 blk + s
