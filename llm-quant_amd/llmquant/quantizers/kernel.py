@@ -49,9 +49,25 @@ def tiled_gemm_pays(rows: int, out_features: int, groups: int) -> bool:
     return FUSED_GEMM_MAX_ROWS < rows <= TILED_GEMM_MAX_ROWS and (out_features >= 8192 or groups >= 64)
 
 
+#: Narrow, short weights (N * groups up to 4096 x 32: q|k|v and o_proj of the 1B and 8B models) keep the fused GEMM up
+#: to this many rows, 64 at a time: two launches of it beat both dequantize + matmul and the tiled GEMM there
+#: (3072 x 2048 int8, M = 128: 14.1 us against 21.7 and 21.2; 4096 x 4096: 24.4 against 32.0 and 27.4).
+FUSED_GEMM_SLAB_MAX_ROWS = 128
+FUSED_GEMM_SLAB_MAX_GROUP_ROWS = 4096 * 32
+
+
+def fused_gemm_takes(rows: int, out_features: int, groups: int) -> bool:
+    """Whether this many rows of a 16-bit activation go to the fused GEMM for a few dozen rows."""
+    if FUSED_GEMM_MIN_ROWS <= rows <= FUSED_GEMM_MAX_ROWS:
+        return True
+    return (FUSED_GEMM_MAX_ROWS < rows <= FUSED_GEMM_SLAB_MAX_ROWS and not tiled_gemm_pays(rows, out_features, groups)
+            and out_features * groups <= FUSED_GEMM_SLAB_MAX_GROUP_ROWS)
+
+
 def fused_gemm_splits(rows: int, groups: int) -> bool:
-    """Which form of the fused GEMM is faster for this many activation rows and groups per weight row."""
-    return rows > FUSED_GEMM_WHOLE_ROWS or groups >= FUSED_GEMM_SPLIT_GROUPS
+    """Which form of the fused GEMM is faster for this many activation rows and groups per weight row: the
+    whole-rows form (False) at every row count, the split form only from FUSED_GEMM_SPLIT_GROUPS groups a row."""
+    return groups >= FUSED_GEMM_SPLIT_GROUPS
 
 
 def pad_activation(flat: torch.Tensor, args) -> torch.Tensor:
@@ -194,7 +210,9 @@ class KernelQuantLinear(nn.Module):
 
     def forward(self, x):
         rows = x.reshape(-1, x.shape[-1])
-        fused = (FUSED_GEMM_MIN_ROWS <= rows.shape[0] <= self._fused_max_rows
+        # (heads padded to groups: above 64 rows the dense branch on the real width reads half the codes)
+        fused = (self._fused_max_rows > 0 and fused_gemm_takes(rows.shape[0], self.out_features, self.qdata.shape[1])
+                 and (rows.shape[0] <= self._fused_max_rows or not self._head_keep)
                  and rows.dtype in (torch.bfloat16, torch.float16) and not self._int8_act)
         tiled = (self._fused_max_rows > 0 and rows.dtype == torch.bfloat16 and not self._int8_act
                  and tiled_gemm_pays(rows.shape[0], self.out_features, self.qdata.shape[1]))

@@ -138,11 +138,11 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         """x [tokens, K] times a concatenated weight: what KernelQuantLinear.forward would pick for this
         many rows, once for the whole concatenation (three or two matmuls and dequantize passes fewer
         per layer, and the host's matmul dispatch is the longest part of a prompt pass)."""
-        from llmquant.quantizers.kernel import (FUSED_GEMM_MAX_ROWS, FUSED_GEMM_MIN_ROWS, KERNEL_MAX_ROWS,
-                                                fused_gemm_splits, tiled_gemm_pays)
+        from llmquant.quantizers.kernel import KERNEL_MAX_ROWS, fused_gemm_splits, fused_gemm_takes, tiled_gemm_pays
 
         rows = x.shape[0]
-        if FUSED_GEMM_MIN_ROWS <= rows <= FUSED_GEMM_MAX_ROWS and x.dtype in (torch.bfloat16, torch.float16):
+        if (fused_gemm_takes(rows, fused.qdata.shape[0], fused.qdata.shape[1])
+                and x.dtype in (torch.bfloat16, torch.float16)):
             return self._ext.wq_gemm_a16(x, fused.qdata, fused.wscale, fused.out_group,
                                          fused_gemm_splits(rows, fused.qdata.shape[1]))
         if rows <= KERNEL_MAX_ROWS:

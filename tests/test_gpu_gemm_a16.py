@@ -270,6 +270,46 @@ def test_module_takes_the_tiled_gemm_for_a_prompt(ext, bits, layout):
     assert rel_l2(to_np(got).reshape(m, -1)[:, cols], exact) <= 2e-3
 
 
+@pytest.mark.parametrize("bits,layout", [(8, {"out_group": 64}), (4, {})])
+def test_module_keeps_the_fused_gemm_for_100_rows_of_a_narrow_weight(ext, bits, layout):
+    """KernelQuantLinear on 100 rows against a q|k|v-sized weight (3072 x 2048): two launches of the fused GEMM for a
+    few dozen rows run (the dense branch and the tiled GEMM are made to fail loudly), and the result is the
+    real-mode sum; with heads padded to groups the dense branch on the real width keeps such a batch."""
+    import torch.nn as nn
+
+    from llmquant.core.scheme import QuantizationArgs, QuantizationScheme
+    from llmquant.quantizers import KernelQuantLinear
+
+    torch.manual_seed(22)
+    linear = nn.Linear(2048, 3072, bias=False).to(torch.bfloat16).cuda()
+    scheme = QuantizationScheme(weights=QuantizationArgs(num_bits=bits, strategy="group", group_size=GROUP, **layout),
+                                input_activations=None)
+    module = KernelQuantLinear.from_linear(linear, scheme)
+    module._dequantized_weight = module._dense = None
+    m = 100
+    x = torch.randn(m, 2048).to(torch.bfloat16)
+    real_tile = module._ext.wq_gemm_a16_tile
+    try:
+        module._ext.wq_gemm_a16_tile = None
+        got = module(x.cuda())
+    finally:
+        module._ext.wq_gemm_a16_tile = real_tile
+    assert got.shape == (m, 3072) and got.dtype == torch.bfloat16
+    canonical, scales = oracle.canonical_weight(to_np(linear.weight), bits, GROUP, None, layout.get("out_group"))
+    og = layout.get("out_group")
+    full_scales = np.repeat(scales, og, axis=0)[:3072] if og else scales
+    exact = oracle.gemv_float64(to_np(x), canonical, full_scales)
+    assert rel_l2(to_np(got), exact) <= 2e-3
+    assert torch.equal(got[:64], module(x[:64].cuda())) and torch.equal(got[64:], module(x[64:].cuda()))
+    padded = KernelQuantLinear.from_linear(nn.Linear(2048, 2048, bias=False).to(torch.bfloat16).cuda(), QuantizationScheme(
+        weights=QuantizationArgs(num_bits=8, strategy="group", group_size=GROUP, head_dim=64), input_activations=None))
+    calls = []
+    dense = padded._dense
+    padded._dense = lambda rows, real_width=False: (calls.append(real_width), dense(rows, real_width))[1]
+    padded(torch.randn(m, 2048).to(torch.bfloat16).cuda())
+    assert calls == [True]
+
+
 # ---- gate|up with silu(gate) * up written as down_proj's prepared activation ------------------------------------
 
 

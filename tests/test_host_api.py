@@ -152,9 +152,22 @@ def test_row_count_routing_of_the_kernel_mode_linear():
     assert FUSED_GEMM_WHOLE_ROWS == FUSED_GEMM_MAX_ROWS == 64
     # the whole-rows form at every row count and row length (gate/up and down_proj of Llama-3-8B: 32 and 112
     # groups per row): it is the faster one everywhere since its activation goes through LDS
-    for rows in (3, 16, 17, 64):
+    for rows in (3, 16, 17, 64, 100, 128):
         for groups in (16, 32, 63, 64, 112):
             assert not fused_gemm_splits(rows, groups)
+
+
+def test_narrow_short_weights_keep_the_fused_gemm_up_to_128_rows():
+    from llmquant.quantizers.kernel import fused_gemm_takes, tiled_gemm_pays
+
+    # q|k|v and o_proj of Llama-3.2-1B (16 groups a row) and Llama-3-8B's o_proj (4096 x 32 groups)
+    for n, g in ((3072, 16), (2048, 16), (4096, 32)):
+        assert fused_gemm_takes(3, n, g) and fused_gemm_takes(64, n, g) and fused_gemm_takes(65, n, g) and fused_gemm_takes(128, n, g)
+        assert not fused_gemm_takes(129, n, g) and not fused_gemm_takes(2, n, g)
+    # wider or longer weights: 64 rows, then the tiled GEMM or the dense branch
+    assert fused_gemm_takes(64, 6144, 32) and not fused_gemm_takes(65, 6144, 32)
+    assert fused_gemm_takes(64, 16384, 16) and not fused_gemm_takes(100, 16384, 16) and tiled_gemm_pays(100, 16384, 16)
+    assert not fused_gemm_takes(100, 2048, 64) and tiled_gemm_pays(100, 2048, 64)
 
 
 # ---- layout ---------------------------------------------------------------------------------------------
