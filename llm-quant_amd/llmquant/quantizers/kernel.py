@@ -46,7 +46,13 @@ def tiled_gemm_pays(rows: int, out_features: int, groups: int) -> bool:
     """Whether the tiled fused GEMM beats dequantize + matmul for this many activation rows: wide outputs
     (enough 128 x 256 tiles to fill the chip) or long rows (the reduction axis is split instead). Narrow,
     short weights (q|k|v, o_proj of a 1B model) have too few tiles either way and stay with the library."""
-    return FUSED_GEMM_MAX_ROWS < rows <= TILED_GEMM_MAX_ROWS and (out_features >= 8192 or groups >= 64)
+    if not FUSED_GEMM_MAX_ROWS < rows <= TILED_GEMM_MAX_ROWS:
+        return False
+    if out_features >= 8192 or groups >= 64:
+        return True
+    # one tile of rows on a mid-sized weight (Llama-3-8B's q|k|v, 6144 x 4096 int8, M = 65-128: 24.8-27.1 us against
+    # 32.7-36.0 for dequantize + matmul); smaller weights take the fused GEMM for a few dozen rows twice instead
+    return rows <= 128 and out_features * groups > FUSED_GEMM_SLAB_MAX_GROUP_ROWS
 
 
 #: Narrow, short weights (N * groups up to 4096 x 32: q|k|v and o_proj of the 1B and 8B models) keep the fused GEMM up

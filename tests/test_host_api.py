@@ -168,6 +168,9 @@ def test_narrow_short_weights_keep_the_fused_gemm_up_to_128_rows():
     assert fused_gemm_takes(64, 6144, 32) and not fused_gemm_takes(65, 6144, 32)
     assert fused_gemm_takes(64, 16384, 16) and not fused_gemm_takes(100, 16384, 16) and tiled_gemm_pays(100, 16384, 16)
     assert not fused_gemm_takes(100, 2048, 64) and tiled_gemm_pays(100, 2048, 64)
+    # a mid-sized weight (Llama-3-8B's q|k|v): one tile of rows goes to the tiled GEMM, more to the dense branch
+    assert tiled_gemm_pays(100, 6144, 32) and tiled_gemm_pays(128, 6144, 32) and not tiled_gemm_pays(129, 6144, 32)
+    assert not tiled_gemm_pays(100, 4096, 32) and not tiled_gemm_pays(100, 3072, 16)
 
 
 # ---- layout ---------------------------------------------------------------------------------------------
