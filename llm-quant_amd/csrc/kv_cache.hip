@@ -639,6 +639,56 @@ constexpr int kSplitThreads = kSplitWaves * kWave;
 constexpr int kSplitSlab = kSplitWaves * kTokPerIter;  // 64 tokens per workgroup step
 constexpr int kSplitPrefetch = 2;  // steps of cache rows a wave requests before it knows the position
 
+// Phase A of a split attention step: the workgroup's waves rotate its query heads into s_q (times the softmax
+// scale in log2 units; one head: wave 0), and in the last split waves 1 / 2 quantize the new token's K / V: the
+// dequantized values go to s_new for the workgroup's own attention, the codes and scales (writer only: one
+// workgroup per kv head) into the cache at `pos`.
+template <typename T, int BITS, int D, int HEADS>
+__device__ __forceinline__ void split_phase_a(const T* __restrict__ qkv, const T* __restrict__ cos_row,
+                                              const T* __restrict__ sin_row, uint8_t* __restrict__ k_codes,
+                                              uint8_t* __restrict__ v_codes, float* __restrict__ k_scale,
+                                              float* __restrict__ v_scale, const float sm_scale_log2, const int q_heads,
+                                              const int kv_heads, const int t_max, const int pos, const int qh0,
+                                              const int kvh, const bool last_split, const bool writer, const int lane,
+                                              const int wv, float (*s_q)[D], float (*s_new)[D]) {
+  for (int h = wv; h < HEADS; h += kSplitWaves) {
+    const T* q = qkv + static_cast<int64_t>(qh0 + h) * D;
+    for (int i = lane; i < D; i += kWave) s_q[h][i] = rope_element<T, D>(q, cos_row, sin_row, i) * sm_scale_log2;
+  }
+  if (wv >= 1 && wv <= 2 && last_split) {
+    const bool is_v = wv == 2;
+    const T* src = qkv + (static_cast<int64_t>(q_heads) + (is_v ? kv_heads : 0) + kvh) * D;
+    const float qmax = static_cast<float>((1 << (BITS - 1)) - 1);
+    const float qmin = -qmax - 1.0f;
+    float f[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int d = lane + e * kWave;
+      f[e] = 0.0f;
+      if (d < D) f[e] = is_v ? to_float(src[d]) : rope_element<T, D>(src, cos_row, sin_row, d);
+    }
+    const float amax = group_max<kWave>(fmaxf(fabsf(f[0]), fabsf(f[1])));
+    const float scale = scale_from_amax(amax, qmax);
+    const int64_t slot = static_cast<int64_t>(kvh) * t_max + pos;
+    if (writer && lane == 0) (is_v ? v_scale : k_scale)[slot] = scale;
+    uint8_t* codes = is_v ? v_codes : k_codes;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int d = lane + e * kWave;
+      const float qv = quant_code(f[e], scale, qmin, qmax);
+      if (d < D) s_new[is_v ? 1 : 0][d] = round_through<T>(qv * scale);
+      const int code = static_cast<int>(qv);
+      if constexpr (BITS == 8) {
+        if (writer && d < D) codes[slot * D + d] = static_cast<uint8_t>(code);
+      } else {
+        const int mine = (code + 8) & 0xf;
+        const int other = dpp<kDppXor1>(mine);
+        if (writer && (lane & 1) == 0 && d < D) codes[slot * (D / 2) + d / 2] = static_cast<uint8_t>(mine | (other << 4));
+      }
+    }
+  }
+}
+
 // HEADS: query heads of one kv head that a workgroup takes together (1, or 4 under grouped-query
 // attention with long caches). Every cache row is then read and dequantized once for the four of
 // them: beyond a few thousand tokens the step is bound by exactly that arithmetic, which one
@@ -687,42 +737,8 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
 
   // ---- phase A: the waves rotate the query heads (one head: wave 0); in the last split wave 1 / 2 also
   // prepare the new K / V ----------------------------------------------------------------------------
-  for (int h = wv; h < HEADS; h += kSplitWaves) {
-    const T* q = qkv + static_cast<int64_t>(qh0 + h) * D;
-    for (int i = lane; i < D; i += kWave) s_q[h][i] = rope_element<T, D>(q, cos_row, sin_row, i) * sm_scale_log2;
-  }
-  if (wv >= 1 && wv <= 2 && last_split) {
-    const bool is_v = wv == 2;
-    const T* src = qkv + (static_cast<int64_t>(q_heads) + (is_v ? kv_heads : 0) + kvh) * D;
-    const float qmax = static_cast<float>((1 << (BITS - 1)) - 1);
-    const float qmin = -qmax - 1.0f;
-    float f[2];
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const int d = lane + e * kWave;
-      f[e] = 0.0f;
-      if (d < D) f[e] = is_v ? to_float(src[d]) : rope_element<T, D>(src, cos_row, sin_row, d);
-    }
-    const float amax = group_max<kWave>(fmaxf(fabsf(f[0]), fabsf(f[1])));
-    const float scale = scale_from_amax(amax, qmax);
-    const int64_t slot = static_cast<int64_t>(kvh) * t_max + pos;
-    if (writer && lane == 0) (is_v ? v_scale : k_scale)[slot] = scale;
-    uint8_t* codes = is_v ? v_codes : k_codes;
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const int d = lane + e * kWave;
-      const float qv = quant_code(f[e], scale, qmin, qmax);
-      if (d < D) s_new[is_v ? 1 : 0][d] = round_through<T>(qv * scale);
-      const int code = static_cast<int>(qv);
-      if constexpr (BITS == 8) {
-        if (writer && d < D) codes[slot * D + d] = static_cast<uint8_t>(code);
-      } else {
-        const int mine = (code + 8) & 0xf;
-        const int other = dpp<kDppXor1>(mine);
-        if (writer && (lane & 1) == 0 && d < D) codes[slot * (D / 2) + d / 2] = static_cast<uint8_t>(mine | (other << 4));
-      }
-    }
-  }
+  split_phase_a<T, BITS, D, HEADS>(qkv, cos_row, sin_row, k_codes, v_codes, k_scale, v_scale, sm_scale_log2, q_heads,
+                                   kv_heads, t_max, pos, qh0, kvh, last_split, writer, lane, wv, s_q, s_new);
   __syncthreads();
 
   // ---- phase B: this split's slabs of tokens 0 .. pos-1, and (last split) token pos from LDS ------------
@@ -783,6 +799,265 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
       rec[1] = ll;
     }
     rec[kAttnRecordHeader + d] = oo;
+  }
+}
+
+// ---- the same step for long caches under grouped-query attention, on the int8 matrix core ---------------------
+// Beyond a few thousand tokens the step above is bound by the vector ALU: every code is converted to a float and
+// multiplied there (~500 instructions per 16 tokens and four heads, 2.6 TB/s of cache bytes at best). Here the int8
+// codes are matrix-core operands as they lie in the cache (v_mfma_i32_16x16x64_i8), for the four query heads of a
+// kv head at once, and the vector ALU is left with the softmax: ~2 instructions per token and head.
+//
+//   scores   S[(head, digit)][token] = sum_d Q[(head, digit)][d] * Kcode[token][d]: the rotated, scaled query of a
+//            head as a block-floating-point integer (22 bits below the head's abs-max) cut in three signed base-256
+//            digits, one operand row each (the GEMV's trick); a lane ends up with the three digit sums of one
+//            (token, head) and combines them: score = (S0 + 256 S1 + 65536 S2) * 2^-sh * kscale[token].
+//   values   O[(head, digit)][d] = sum_t W[(head, digit)][t] * Vcode[t][d] with W = p * vscale[t], p the softmax
+//            weight relative to the running maximum, as a 14-bit integer below the largest W of the head in the
+//            64-token step, in two digits. The weights reach operand layout (tokens along a lane's 16 bytes)
+//            through 1 KB of LDS per wave; V's codes, token-major in the cache, are read from LDS transposed
+//            (ds_read_b64_tr_b8: in a group of 16 lanes, byte j of result lane l is byte l % 8 of what lane
+//            2 j + l / 8 points at).
+//
+// Both sums are exact integers; what differs from the step above is that K and V enter as code * scale without the
+// rounding to the model's dtype in between, and the 2^-14 resolution of the weights: within the tolerance the
+// attention output is held to (checked against the float64 oracle like the other kernels).
+// A wave walks 64-token slabs (wave w of split s: slabs 4 s + w, 4 s + w + 4 S, ...) through two LDS stages of its
+// own, filled by DMA (codes of K and V with their 16-byte pieces XOR-swizzled by row so that the operand reads and
+// the transposed reads meet no bank conflict, and the two scale vectors): no barrier inside the loop. The records
+// it leaves are those of the kernel above.
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+typedef int v2i32 __attribute__((ext_vector_type(2)));
+
+constexpr int kMfD = 64;                                   // head_dim this kernel is written for
+constexpr int kMfHeads = 4;                                // query heads of one kv head per workgroup
+constexpr int kMfSlab = 64;                                // tokens of one wave step
+constexpr int kMfCodes = kMfSlab * kMfD;                   // bytes of a slab's K (or V) codes
+constexpr int kMfStage = 2 * kMfCodes + 2 * kMfSlab * 4;   // K codes, V codes, K scales, V scales
+constexpr int kMfP = 16 * kMfSlab;                         // the weights as operand rows: [16 rows][64 tokens] bytes
+constexpr int kMfWaveBytes = 2 * kMfStage + kMfP + 64;     // two stages, the weights, 2^-sh per head
+constexpr int kMfRec = kMfD + 2;                           // a wave's (max, sum, output) per head
+constexpr int kMfHeaderFloats = kMfHeads * kMfD + 2 * kMfD + kSplitWaves * kMfHeads * kMfRec + kMfHeads;
+constexpr int kMfHeaderBytes = (kMfHeaderFloats * 4 + 255) / 256 * 256;
+constexpr int kMfLdsBytes = kMfHeaderBytes + kSplitWaves * kMfWaveBytes;   // 80 KB: two workgroups a CU
+// caches shorter than this keep the vector-ALU form, whose K and V pass through the model's dtype as the reference's
+// cache holds them; the step is bound by latency there whichever form runs
+constexpr int kMfMinCache = 4096;
+
+template <typename T>
+__global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_mfma_kernel(
+    const T* __restrict__ qkv, const T* __restrict__ cos_table, const T* __restrict__ sin_table,
+    uint8_t* __restrict__ k_codes, uint8_t* __restrict__ v_codes, float* __restrict__ k_scale,
+    float* __restrict__ v_scale, float* __restrict__ partials, const int32_t* __restrict__ pos_dev,
+    const float sm_scale_log2, const int q_heads, const int kv_heads, const int t_max) {
+  constexpr int D = kMfD, HEADS = kMfHeads;
+  constexpr int GREC = D + kAttnRecordHeader;
+  extern __shared__ __attribute__((aligned(16))) unsigned char mf_smem[];
+  float (*s_q)[D] = reinterpret_cast<float (*)[D]>(mf_smem);
+  float (*s_new)[D] = reinterpret_cast<float (*)[D]>(mf_smem + HEADS * D * 4);
+  float* s_rec = reinterpret_cast<float*>(mf_smem + (HEADS + 2) * D * 4);   // [waves][HEADS][kMfRec]
+  float* s_new_score = s_rec + kSplitWaves * HEADS * kMfRec;
+
+  const int qh0 = blockIdx.x * HEADS, split = blockIdx.y, n_splits = gridDim.y;
+  const bool last_split = split == n_splits - 1;
+  const int rep = q_heads / kv_heads;  // a multiple of HEADS
+  const int kvh = qh0 / rep;
+  const bool writer = last_split && qh0 % rep == 0;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int j = lane & 15, g = lane >> 4;   // (column, row block) of the matrix core's lanes
+
+  unsigned char* mine = mf_smem + kMfHeaderBytes + wv * kMfWaveBytes;
+  unsigned char* pbuf = mine + 2 * kMfStage;
+  float* qinv_of = reinterpret_cast<float*>(pbuf + kMfP);
+
+  const uint8_t* kbase = k_codes + static_cast<int64_t>(kvh) * t_max * D;
+  const uint8_t* vbase = v_codes + static_cast<int64_t>(kvh) * t_max * D;
+  const float* ksc = k_scale + static_cast<int64_t>(kvh) * t_max;
+  const float* vsc = v_scale + static_cast<int64_t>(kvh) * t_max;
+  // transfer i of a slab's codes lands in LDS bytes 1024 i + 16 lane: row 16 i + lane / 4, slot lane % 4; the slot
+  // holds the row's 16-byte piece (slot ^ f(row)), f chosen per tensor for the way it is read back
+  const int row_in_transfer = lane >> 2;
+  const int piece_k = (lane & 3) ^ ((row_in_transfer >> 2) & 3);     // f_K(row) = (row / 4) % 4
+  const int swz_v_lane = (lane >> 4) & 1;                            // f_V(row) = (row / 4) % 2 + 2 * ((row / 16) % 2)
+  auto request = [&](const int t0, const int stage) {
+    unsigned char* st = mine + stage * kMfStage;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t t = min(t0 + 16 * i + row_in_transfer, t_max - 1);   // (rows past the cache's end: the last row again)
+      const int piece_v = (lane & 3) ^ (swz_v_lane | ((i & 1) << 1));
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(kbase + t * D + 16 * piece_k),
+                                       reinterpret_cast<u32x4*>(st + 1024 * i), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(vbase + t * D + 16 * piece_v),
+                                       reinterpret_cast<u32x4*>(st + kMfCodes + 1024 * i), 16, 0, 0);
+    }
+    const int64_t ts = min(t0 + lane, t_max - 1);
+    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(ksc + ts),
+                                     reinterpret_cast<uint32_t*>(st + 2 * kMfCodes), 4, 0, 0);
+    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(vsc + ts),
+                                     reinterpret_cast<uint32_t*>(st + 2 * kMfCodes + kMfSlab * 4), 4, 0, 0);
+  };
+  constexpr int kRequestLoads = 10;
+
+  // the wave's first slab does not depend on the position (rows up to t_max - 1 exist; what lies at or beyond the
+  // position is masked later): requested first, so that the position's round trip and phase A run under it
+  int t0 = (split * kSplitWaves + wv) * kMfSlab;
+  const int t_step = n_splits * kSplitWaves * kMfSlab;
+  request(t0, 0);
+
+  const int pos = min(max(pos_dev[0], 0), t_max - 1);
+  const T* cos_row = cos_table + static_cast<int64_t>(pos) * D;
+  const T* sin_row = sin_table + static_cast<int64_t>(pos) * D;
+  split_phase_a<T, 8, D, HEADS>(qkv, cos_row, sin_row, k_codes, v_codes, k_scale, v_scale, sm_scale_log2, q_heads,
+                                kv_heads, t_max, pos, qh0, kvh, last_split, writer, lane, wv, s_q, s_new);
+  // operand rows the weights never reach (two of a head's four) stay zero
+  for (int i = lane; i < kMfP / 4; i += kWave) reinterpret_cast<uint32_t*>(pbuf)[i] = 0u;
+  __syncthreads();
+
+  // ---- the query heads as operand rows: lane (row = j = 4 head + digit, block g) holds d = 16 g .. 16 g + 15 ----
+  v4i32 qa;
+  {
+    const int h = j >> 2, digit = j & 3;
+    float amax = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) amax = fmaxf(amax, fabsf(s_q[h][d]));
+    const uint32_t e = __builtin_bit_cast(uint32_t, amax) >> 23;   // amax = f 2^(e - 126), f in [0.5, 1)
+    const bool usable = e >= 22u && e < 255u;                       // (below 2^-105 the head counts as zero)
+    const float up = __builtin_bit_cast(float, (275u - e) << 23);  // 2^(148 - e): amax * up in [2^21, 2^22)
+    const float down = __builtin_bit_cast(float, (e - 21u) << 23); // 2^(e - 148)
+    uint32_t words[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int b = 0; b < 16; ++b) {
+      const int qi = usable ? static_cast<int>(rintf(s_q[h][16 * g + b] * up)) : 0;
+      const int d0 = static_cast<int8_t>(qi);
+      const int r1 = (qi - d0) >> 8;
+      const int d1 = static_cast<int8_t>(r1);
+      const int d2 = (r1 - d1) >> 8;
+      const int digit_value = digit == 0 ? d0 : digit == 1 ? d1 : digit == 2 ? d2 : 0;
+      words[b >> 2] |= static_cast<uint32_t>(digit_value & 0xff) << (8 * (b & 3));
+    }
+    qa = v4i32{static_cast<int>(words[0]), static_cast<int>(words[1]), static_cast<int>(words[2]), static_cast<int>(words[3])};
+    if (digit == 0 && g == 0) qinv_of[h] = usable ? down : 0.0f;
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  const float qinv = qinv_of[g];   // in the score tiles a lane's head is its row block
+
+  const int swz_v_read = ((j >> 3) & 1) | ((g & 1) << 1);   // f_V of the rows this lane points at in a transposed read
+  float m_run = -INFINITY, l_part = 0.0f;
+  float o_acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};               // head g, d = 16 tile + j
+  int stage = 0;
+  for (; t0 < pos; t0 += t_step, stage ^= 1) {
+    if (t0 + t_step < pos) {
+      request(t0 + t_step, stage ^ 1);
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kRequestLoads) : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    const unsigned char* st = mine + stage * kMfStage;
+    const float* ks_of = reinterpret_cast<const float*>(st + 2 * kMfCodes);
+    const float* vs_of = ks_of + kMfSlab;
+    // ---- scores of the slab's four tiles of 16 tokens: lane = (token 16 c + j, head g)
+    float sc[4], w[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int r = 16 * c + j;
+      const v4i32 kb = *reinterpret_cast<const v4i32*>(st + r * D + 16 * (g ^ ((r >> 2) & 3)));
+      const v4i32 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qa, kb, v4i32{0, 0, 0, 0}, 0, 0, 0);
+      const float dot = fmaf(static_cast<float>(acc[2]), 65536.0f,
+                             fmaf(static_cast<float>(acc[1]), 256.0f, static_cast<float>(acc[0])));
+      sc[c] = t0 + r < pos ? dot * (ks_of[r] * qinv) : -INFINITY;
+    }
+    const float m_new = fmaxf(m_run, group_max<16>(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]))));
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);   // (the slab's first token is below pos: m_new is finite)
+    float p_sum = 0.0f, w_max = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int r = 16 * c + j;
+      const float p = __builtin_amdgcn_exp2f(sc[c] - m_new);
+      p_sum += p;
+      w[c] = t0 + r < pos ? p * vs_of[r] : 0.0f;
+      w_max = fmaxf(w_max, w[c]);
+    }
+    l_part = fmaf(l_part, alpha, p_sum);
+    m_run = m_new;
+    // ---- the weights as 14-bit integers below the head's largest in this slab, two digits
+    w_max = group_max<16>(w_max);
+    const uint32_t we = max(__builtin_bit_cast(uint32_t, w_max) >> 23, 13u);   // w_max = f 2^(we - 126)
+    const float w_up = __builtin_bit_cast(float, (267u - we) << 23);            // 2^(140 - we): w * w_up < 2^14
+    const float w_down = __builtin_bit_cast(float, (we - 13u) << 23);           // 2^(we - 140)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int wi = static_cast<int>(rintf(w[c] * w_up));
+      const int d0 = static_cast<int8_t>(wi);
+      const int d1 = (wi - d0) >> 8;
+      pbuf[(4 * g) * kMfSlab + 16 * c + j] = static_cast<unsigned char>(d0);
+      pbuf[(4 * g + 1) * kMfSlab + 16 * c + j] = static_cast<unsigned char>(d1);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const v4i32 pa = *reinterpret_cast<const v4i32*>(pbuf + j * kMfSlab + 16 * g);   // row j, tokens 16 g .. 16 g + 15
+    // ---- weighted values, 16 of the head's dimensions per tile: lane = (d = 16 tile + j, head g)
+    const unsigned char* vrow = st + kMfCodes + (16 * g + (j >> 1)) * D + 8 * (j & 1);
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      const int at = 16 * (dt ^ swz_v_read);
+      const v2i32 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (__attribute__((address_space(3))) v2i32*)(vrow + at));                // tokens 16 g .. 16 g + 7
+      const v2i32 hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (__attribute__((address_space(3))) v2i32*)(vrow + 8 * D + at));        // 16 g + 8 .. 16 g + 15
+      const v4i32 vb = v4i32{lo[0], lo[1], hi[0], hi[1]};
+      const v4i32 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(pa, vb, v4i32{0, 0, 0, 0}, 0, 0, 0);
+      const float sum = fmaf(static_cast<float>(acc[1]), 256.0f, static_cast<float>(acc[0]));
+      o_acc[dt] = fmaf(o_acc[dt], alpha, sum * w_down);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // (the stage and the weights are free for the next round)
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // (a wave with no slab below pos: its first request lands before it leaves)
+
+  // ---- the waves meet: (max, sum, output) per wave and head, then the new token, then the split's record --------
+  {
+    const float l_row = row16_sum(l_part);
+    float* rec = s_rec + (wv * HEADS + g) * kMfRec;
+    if (j == 0) {
+      rec[0] = m_run;
+      rec[1] = l_row;
+    }
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) rec[2 + 16 * dt + j] = o_acc[dt];
+  }
+  if (wv == kSplitWaves - 1) {
+    // the new token is a record of its own: its scores here, its value is s_new[1]
+    float dot = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dot = fmaf(s_q[g][4 * j + i], s_new[0][4 * j + i], dot);
+    dot = row16_sum(dot);
+    if (j == 0) s_new_score[g] = last_split ? dot : -INFINITY;
+  }
+  __syncthreads();
+  for (int item = threadIdx.x; item < HEADS * D; item += kSplitThreads) {
+    const int h = item / D, d = item - h * D;
+    const float new_score = s_new_score[h];
+    float mm = new_score;
+#pragma unroll
+    for (int w2 = 0; w2 < kSplitWaves; ++w2) mm = fmaxf(mm, s_rec[(w2 * HEADS + h) * kMfRec]);
+    float ll = 0.0f, oo = 0.0f;
+#pragma unroll
+    for (int w2 = 0; w2 < kSplitWaves; ++w2) {
+      const float* rec = s_rec + (w2 * HEADS + h) * kMfRec;
+      const float a = rec[0] == -INFINITY ? 0.0f : exp2f(rec[0] - mm);
+      ll += rec[1] * a;
+      oo += rec[2 + d] * a;
+    }
+    if (new_score != -INFINITY) {
+      const float b = exp2f(new_score - mm);
+      ll += b;
+      oo = fmaf(b, s_new[1][d], oo);
+    }
+    float* out_rec = partials + (static_cast<int64_t>(qh0 + h) * n_splits + split) * GREC;
+    if (d == 0) {
+      out_rec[0] = mm;
+      out_rec[1] = ll;
+    }
+    out_rec[kAttnRecordHeader + d] = oo;
   }
 }
 
@@ -1342,6 +1617,36 @@ extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos
   const int rep_heads = q_heads / kv_heads;
   const bool grouped = rep_heads % 4 == 0 && n_splits >= 32;
   const dim3 grid(grouped ? q_heads / 4 : q_heads, n_splits), block(kSplitThreads);
+  if (grouped && bits == 8 && head_dim == kMfD && t_max >= kMfMinCache) {
+    // int8 codes of 64-wide heads: the matrix-core form (ctx 8 K / 32 K / 131 K, 32 heads on 8 kv heads: see the
+    // kernel's comment for what it changes in the arithmetic)
+#define LLMQ_SPLIT_MFMA(T)                                                                                        \
+  do {                                                                                                            \
+    auto kernel = kv_rope_append_attend_split_mfma_kernel<T>;                                                     \
+    static bool raised = false; /* per instantiation; worst case two threads both set it */                       \
+    if (!raised) {                                                                                                \
+      const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                           \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kMfLdsBytes);        \
+      if (err != hipSuccess) {                                                                                    \
+        llmq_host::set_error("raising the LDS limit failed: %s", hipGetErrorString(err));                         \
+        return static_cast<int>(err);                                                                             \
+      }                                                                                                           \
+      raised = true;                                                                                              \
+    }                                                                                                             \
+    hipLaunchKernelGGL(kernel, grid, block, kMfLdsBytes, s, static_cast<const T*>(qkv),                           \
+                       static_cast<const T*>(cos_table), static_cast<const T*>(sin_table),                        \
+                       static_cast<uint8_t*>(k_codes), static_cast<uint8_t*>(v_codes), k_scale, v_scale, partials, \
+                       pos_dev, scale_log2, q_heads, kv_heads, t_max);                                            \
+  } while (0)
+    switch (dtype) {
+      case LLMQ_F32: LLMQ_SPLIT_MFMA(float); break;
+      case LLMQ_F16: LLMQ_SPLIT_MFMA(f16_t); break;
+      case LLMQ_BF16: LLMQ_SPLIT_MFMA(bf16_t); break;
+      default: return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
+    }
+#undef LLMQ_SPLIT_MFMA
+    return llmq_host::check_launch("kv_rope_append_attend_split_mfma_kernel");
+  }
 #define LLMQ_SPLIT(T, B, D)                                                                            \
   do {                                                                                                 \
     if (grouped) {                                                                                     \

@@ -226,7 +226,7 @@ def rope_oracle(x, cos, sin):
     return oracle.round_to(a + b, "bf16")
 
 
-def decode_step_case(ext, bits, ctx, q_heads=32, kv_heads=8, d=64, seed=0):
+def decode_step_case(ext, bits, ctx, q_heads=32, kv_heads=8, d=64, seed=0, t_max=None):
     """KV-cache quantization in decode attention, Llama-3.2-1B geometry: a cache of `ctx` tokens with
     per-channel scale variance, one new token through RoPE -> quantize-append -> attention. Returns the
     device-side cache, the q|k|v row and tables, and the oracle's attention output [Hq, D] (bf16 values)."""
@@ -236,7 +236,7 @@ def decode_step_case(ext, bits, ctx, q_heads=32, kv_heads=8, d=64, seed=0):
     v = (torch.randn(kv_heads, ctx, d, generator=gen) * channel).to(torch.bfloat16)
     qkv = torch.randn(1, (q_heads + 2 * kv_heads) * d, generator=gen).to(torch.bfloat16)
     qkv[:, q_heads * d:] *= channel.repeat(2 * kv_heads).to(torch.bfloat16)
-    t_max = ctx + 1
+    t_max = ctx + 1 if t_max is None else t_max
     inv_freq = 1.0 / (500000.0 ** (torch.arange(0, d, 2).float() / d))
     emb = torch.outer(torch.arange(t_max).float(), inv_freq)
     emb = torch.cat((emb, emb), -1)
@@ -302,3 +302,40 @@ def test_decode_step_attention_against_the_oracle(ext, bits, ctx, splits):
         padded = oracle.pad_activation(want.reshape(1, -1), 128, d)
         exact = oracle.gemv_float64(padded, canonical, scales) + to_np(res).astype(np.float64)
         assert rel_l2(to_np(out), exact) <= 1e-2
+
+
+@pytest.mark.parametrize("ctx,splits,t_max,q_heads,kv_heads", [
+    (2048, 32, 4096, 32, 8), (640, 32, 4096, 32, 8), (0, 32, 4096, 32, 8), (1, 32, 4096, 32, 8), (63, 32, 4096, 32, 8),
+    (64, 32, 4096, 32, 8), (65, 32, 4096, 32, 8), (4094, 32, 4096, 32, 8), (5002, 32, 5004, 32, 8),
+    (9000, 64, 9216, 32, 8), (3000, 48, 4100, 8, 2), (20000, 32, 20001, 16, 2)])
+def test_long_cache_decode_step_on_the_matrix_core_against_the_oracle(ext, ctx, splits, t_max, q_heads, kv_heads):
+    """Caches of 4096 rows and more under grouped-query attention with int8 codes and 64-wide heads take the
+    matrix-core form of the split step (codes as int8 operands, the query in three digits, the softmax weights
+    in two): the same checks as the vector-ALU form gets, against the same oracle (appended codes and scales bit
+    for bit, output rel-L2 <= 1e-2 and <= 2e-2 per head), at contexts around the 64-token slab boundaries, with
+    one token and none, up to the cache's last row, with cache lengths that are not whole slabs. Rows beyond the
+    position hold random codes and NaN scales: nothing of them may reach the result."""
+    d, bits = 64, 8
+    cache, qkv, cos_t, sin_t, want, (kq, ks, vq, vs) = decode_step_case(ext, bits, ctx, q_heads, kv_heads, seed=ctx,
+                                                                        t_max=t_max)
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    for name in ("k_codes", "v_codes"):
+        cache[name][:, ctx + 1:] = torch.randint(-128, 128, cache[name][:, ctx + 1:].shape, generator=gen,
+                                                 device="cuda").to(cache[name].dtype)
+    for name in ("k_scale", "v_scale"):
+        cache[name][:, ctx + 1:] = float("nan")
+    position = torch.tensor([ctx], dtype=torch.int32, device="cuda")
+    partials = torch.full((ext.kv_attend_partials_floats(q_heads, d, splits),), float("nan"), device="cuda")
+    ext.kv_rope_append_attend_split(qkv, cos_t, sin_t, cache["k_codes"], cache["v_codes"], cache["k_scale"],
+                                    cache["v_scale"], partials, position, d ** -0.5, q_heads, splits)
+    merged = ext.kv_attend_merge(partials, q_heads, d, splits, torch.bfloat16)
+    assert np.array_equal(codes_np(cache["k_codes"], bits)[:, : ctx + 1], kq)
+    assert np.array_equal(codes_np(cache["v_codes"], bits)[:, : ctx + 1], vq)
+    assert np.array_equal(to_np(cache["k_scale"])[:, : ctx + 1], ks)
+    assert np.array_equal(to_np(cache["v_scale"])[:, : ctx + 1], vs)
+    got = to_np(merged).reshape(q_heads, d)
+    assert np.isfinite(got).all()
+    assert rel_l2(got, want) <= 1e-2
+    per_head = np.linalg.norm(got - want, axis=1) / np.linalg.norm(want, axis=1)
+    assert per_head.max() <= 2e-2, per_head.argmax()
+    print(f"ctx {ctx} splits {splits}: rel-L2 {rel_l2(got, want):.2e}, worst head {per_head.max():.2e}")
