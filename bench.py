@@ -398,6 +398,27 @@ def other_kernels(torch):
     entry["frac_hbm"] = round(entry["GBps"] / HBM_PEAK_GBPS, 4)
     out["kv_int8_rope_append_attention_ctx32000_per_layer"] = entry
     del kc, vc, ks, vs
+    # and for heads of 128 (the Llama-3-8B geometry), 5 layers = 350 MB
+    layers, d = 5, 128
+    kc = torch.randint(0, 100, (layers, kvh, t_max, d), device=dev).to(torch.int8)
+    vc = torch.randint(0, 100, (layers, kvh, t_max, d), device=dev).to(torch.int8)
+    ks = torch.rand(layers, kvh, t_max, device=dev) * 0.05
+    vs = torch.rand(layers, kvh, t_max, device=dev) * 0.05
+    qkv = torch.randn(1, (qh + 2 * kvh) * d, device=dev).to(torch.bfloat16)
+    table = torch.randn(t_max, d, device=dev).to(torch.bfloat16)
+    partials = torch.zeros(ext.kv_attend_partials_floats(qh, d, 32), device=dev)
+
+    def long_step_128():
+        for layer in range(layers):
+            ext.kv_rope_append_attend_split(qkv, table, table, kc[layer], vc[layer], ks[layer], vs[layer], partials,
+                                            pos, d ** -0.5, qh, 32)
+
+    nbytes = 2 * kvh * (ctx + 1) * d + 2 * kvh * (ctx + 1) * 4
+    us = round(_graph_time_us(torch, long_step_128, reps=20) / layers, 2)
+    out["kv_int8_rope_append_attention_ctx32000_head_dim128_per_layer"] = {
+        "bytes": nbytes, "four_heads_matrix_core_32_splits_us": us, "GBps": round(nbytes / us / 1e3, 1),
+        "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    del kc, vc, ks, vs
     # the GEMV on Llama-3-8B's linears (M = 1): random codes, buffers rotated over > 600 MB so that
     # every launch streams from HBM; the launches of one rotation replayed as a HIP graph
     shapes_8b = []

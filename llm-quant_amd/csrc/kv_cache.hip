@@ -829,34 +829,48 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
 typedef int v4i32 __attribute__((ext_vector_type(4)));
 typedef int v2i32 __attribute__((ext_vector_type(2)));
 
-constexpr int kMfD = 64;                                   // head_dim this kernel is written for
-constexpr int kMfHeads = 4;                                // query heads of one kv head per workgroup
-constexpr int kMfSlab = 64;                                // tokens of one wave step
-constexpr int kMfCodes = kMfSlab * kMfD;                   // bytes of a slab's K (or V) codes
-constexpr int kMfStage = 2 * kMfCodes + 2 * kMfSlab * 4;   // K codes, V codes, K scales, V scales
-constexpr int kMfP = 16 * kMfSlab;                         // the weights as operand rows: [16 rows][64 tokens] bytes
-constexpr int kMfWaveBytes = 2 * kMfStage + kMfP + 64;     // two stages, the weights, 2^-sh per head
-constexpr int kMfRec = kMfD + 2;                           // a wave's (max, sum, output) per head
-constexpr int kMfHeaderFloats = kMfHeads * kMfD + 2 * kMfD + kSplitWaves * kMfHeads * kMfRec + kMfHeads;
-constexpr int kMfHeaderBytes = (kMfHeaderFloats * 4 + 255) / 256 * 256;
-constexpr int kMfLdsBytes = kMfHeaderBytes + kSplitWaves * kMfWaveBytes;   // 80 KB: two workgroups a CU
+constexpr int kMfHeads = 4;   // query heads of one kv head per workgroup
+constexpr int kMfSlab = 64;   // tokens of one wave step
 // caches shorter than this keep the vector-ALU form, whose K and V pass through the model's dtype as the reference's
 // cache holds them; the step is bound by latency there whichever form runs
 constexpr int kMfMinCache = 4096;
 
-template <typename T>
+template <int D> struct MfLds {
+  static constexpr int kPieces = D / 16;                          // 16-byte pieces of a row of codes
+  static constexpr int kTransfers = kMfSlab * D / 1024;           // 1 KB DMA instructions per tensor and slab
+  static constexpr int kCodes = kMfSlab * D;                      // bytes of a slab's K (or V) codes
+  static constexpr int kStage = 2 * kCodes + 2 * kMfSlab * 4;     // K codes, V codes, K scales, V scales
+  static constexpr int kP = 16 * kMfSlab;                         // the weights as operand rows: [16 rows][64 tokens] bytes
+  static constexpr int kWaveBytes = 2 * kStage + kP + 64;         // two stages, the weights, 2^-sh per head
+  static constexpr int kRec = D + 2;                              // a wave's (max, sum, output) per head
+  static constexpr int kHeaderFloats = kMfHeads * D + 2 * D + kSplitWaves * kMfHeads * kRec + kMfHeads;
+  static constexpr int kHeaderBytes = (kHeaderFloats * 4 + 255) / 256 * 256;
+  static constexpr int kBytes = kHeaderBytes + kSplitWaves * kWaveBytes;   // 80 KB (D = 64), 148 KB (D = 128)
+  // Slot of a row's 16-byte piece p in LDS is p ^ swizzle(row). K is read as operands: 16 lanes read the same piece
+  // of 16 consecutive rows and have to land in 16 different bank quads. V is read transposed: a lane points at 8
+  // bytes of row 16 g + 8 half + s / 2 (s its index among its 16 lanes), two such groups of lanes go together.
+  static __device__ __forceinline__ int swizzle_k(int row) { return D == 64 ? (row >> 2) & 3 : (row >> 1) & 7; }
+  static __device__ __forceinline__ int swizzle_v(int row) {
+    return D == 64 ? ((row >> 2) & 1) | (((row >> 4) & 1) << 1) : ((row >> 1) & 3) | (((row >> 4) & 1) << 2);
+  }
+};
+
+template <typename T, int D>
 __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_mfma_kernel(
     const T* __restrict__ qkv, const T* __restrict__ cos_table, const T* __restrict__ sin_table,
     uint8_t* __restrict__ k_codes, uint8_t* __restrict__ v_codes, float* __restrict__ k_scale,
     float* __restrict__ v_scale, float* __restrict__ partials, const int32_t* __restrict__ pos_dev,
     const float sm_scale_log2, const int q_heads, const int kv_heads, const int t_max) {
-  constexpr int D = kMfD, HEADS = kMfHeads;
+  using L = MfLds<D>;
+  constexpr int HEADS = kMfHeads;
   constexpr int GREC = D + kAttnRecordHeader;
+  constexpr int kKSteps = D / 64;    // matrix-core steps along a head's dimensions
+  constexpr int kDTiles = D / 16;    // tiles of 16 dimensions of the output
   extern __shared__ __attribute__((aligned(16))) unsigned char mf_smem[];
   float (*s_q)[D] = reinterpret_cast<float (*)[D]>(mf_smem);
   float (*s_new)[D] = reinterpret_cast<float (*)[D]>(mf_smem + HEADS * D * 4);
-  float* s_rec = reinterpret_cast<float*>(mf_smem + (HEADS + 2) * D * 4);   // [waves][HEADS][kMfRec]
-  float* s_new_score = s_rec + kSplitWaves * HEADS * kMfRec;
+  float* s_rec = reinterpret_cast<float*>(mf_smem + (HEADS + 2) * D * 4);   // [waves][HEADS][kRec]
+  float* s_new_score = s_rec + kSplitWaves * HEADS * L::kRec;
 
   const int qh0 = blockIdx.x * HEADS, split = blockIdx.y, n_splits = gridDim.y;
   const bool last_split = split == n_splits - 1;
@@ -867,37 +881,34 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
   const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int j = lane & 15, g = lane >> 4;   // (column, row block) of the matrix core's lanes
 
-  unsigned char* mine = mf_smem + kMfHeaderBytes + wv * kMfWaveBytes;
-  unsigned char* pbuf = mine + 2 * kMfStage;
-  float* qinv_of = reinterpret_cast<float*>(pbuf + kMfP);
+  unsigned char* mine = mf_smem + L::kHeaderBytes + wv * L::kWaveBytes;
+  unsigned char* pbuf = mine + 2 * L::kStage;
+  float* qinv_of = reinterpret_cast<float*>(pbuf + L::kP);
 
   const uint8_t* kbase = k_codes + static_cast<int64_t>(kvh) * t_max * D;
   const uint8_t* vbase = v_codes + static_cast<int64_t>(kvh) * t_max * D;
   const float* ksc = k_scale + static_cast<int64_t>(kvh) * t_max;
   const float* vsc = v_scale + static_cast<int64_t>(kvh) * t_max;
-  // transfer i of a slab's codes lands in LDS bytes 1024 i + 16 lane: row 16 i + lane / 4, slot lane % 4; the slot
-  // holds the row's 16-byte piece (slot ^ f(row)), f chosen per tensor for the way it is read back
-  const int row_in_transfer = lane >> 2;
-  const int piece_k = (lane & 3) ^ ((row_in_transfer >> 2) & 3);     // f_K(row) = (row / 4) % 4
-  const int swz_v_lane = (lane >> 4) & 1;                            // f_V(row) = (row / 4) % 2 + 2 * ((row / 16) % 2)
+  // transfer i of a slab's codes lands in LDS bytes 1024 i + 16 lane: row (1024 / D) i + lane / pieces, slot
+  // lane % pieces
   auto request = [&](const int t0, const int stage) {
-    unsigned char* st = mine + stage * kMfStage;
+    unsigned char* st = mine + stage * L::kStage;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int64_t t = min(t0 + 16 * i + row_in_transfer, t_max - 1);   // (rows past the cache's end: the last row again)
-      const int piece_v = (lane & 3) ^ (swz_v_lane | ((i & 1) << 1));
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(kbase + t * D + 16 * piece_k),
+    for (int i = 0; i < L::kTransfers; ++i) {
+      const int row = (1024 / D) * i + lane / L::kPieces, slot = lane % L::kPieces;
+      const int64_t t = min(t0 + row, t_max - 1);   // (rows past the cache's end: the last row again)
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(kbase + t * D + 16 * (slot ^ L::swizzle_k(row))),
                                        reinterpret_cast<u32x4*>(st + 1024 * i), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(vbase + t * D + 16 * piece_v),
-                                       reinterpret_cast<u32x4*>(st + kMfCodes + 1024 * i), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(vbase + t * D + 16 * (slot ^ L::swizzle_v(row))),
+                                       reinterpret_cast<u32x4*>(st + L::kCodes + 1024 * i), 16, 0, 0);
     }
     const int64_t ts = min(t0 + lane, t_max - 1);
     __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(ksc + ts),
-                                     reinterpret_cast<uint32_t*>(st + 2 * kMfCodes), 4, 0, 0);
+                                     reinterpret_cast<uint32_t*>(st + 2 * L::kCodes), 4, 0, 0);
     __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(vsc + ts),
-                                     reinterpret_cast<uint32_t*>(st + 2 * kMfCodes + kMfSlab * 4), 4, 0, 0);
+                                     reinterpret_cast<uint32_t*>(st + 2 * L::kCodes + kMfSlab * 4), 4, 0, 0);
   };
-  constexpr int kRequestLoads = 10;
+  constexpr int kRequestLoads = 2 * L::kTransfers + 2;
 
   // the wave's first slab does not depend on the position (rows up to t_max - 1 exist; what lies at or beyond the
   // position is masked later): requested first, so that the position's round trip and phase A run under it
@@ -911,11 +922,11 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
   split_phase_a<T, 8, D, HEADS>(qkv, cos_row, sin_row, k_codes, v_codes, k_scale, v_scale, sm_scale_log2, q_heads,
                                 kv_heads, t_max, pos, qh0, kvh, last_split, writer, lane, wv, s_q, s_new);
   // operand rows the weights never reach (two of a head's four) stay zero
-  for (int i = lane; i < kMfP / 4; i += kWave) reinterpret_cast<uint32_t*>(pbuf)[i] = 0u;
+  for (int i = lane; i < L::kP / 4; i += kWave) reinterpret_cast<uint32_t*>(pbuf)[i] = 0u;
   __syncthreads();
 
-  // ---- the query heads as operand rows: lane (row = j = 4 head + digit, block g) holds d = 16 g .. 16 g + 15 ----
-  v4i32 qa;
+  // ---- the query heads as operand rows: lane (row = j = 4 head + digit, block g) holds d = 64 step + 16 g .. + 15
+  v4i32 qa[kKSteps];
   {
     const int h = j >> 2, digit = j & 3;
     float amax = 0.0f;
@@ -925,26 +936,33 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
     const bool usable = e >= 22u && e < 255u;                       // (below 2^-105 the head counts as zero)
     const float up = __builtin_bit_cast(float, (275u - e) << 23);  // 2^(148 - e): amax * up in [2^21, 2^22)
     const float down = __builtin_bit_cast(float, (e - 21u) << 23); // 2^(e - 148)
-    uint32_t words[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-    for (int b = 0; b < 16; ++b) {
-      const int qi = usable ? static_cast<int>(rintf(s_q[h][16 * g + b] * up)) : 0;
-      const int d0 = static_cast<int8_t>(qi);
-      const int r1 = (qi - d0) >> 8;
-      const int d1 = static_cast<int8_t>(r1);
-      const int d2 = (r1 - d1) >> 8;
-      const int digit_value = digit == 0 ? d0 : digit == 1 ? d1 : digit == 2 ? d2 : 0;
-      words[b >> 2] |= static_cast<uint32_t>(digit_value & 0xff) << (8 * (b & 3));
+    for (int ks = 0; ks < kKSteps; ++ks) {
+      uint32_t words[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int b = 0; b < 16; ++b) {
+        const int qi = usable ? static_cast<int>(rintf(s_q[h][64 * ks + 16 * g + b] * up)) : 0;
+        const int d0 = static_cast<int8_t>(qi);
+        const int r1 = (qi - d0) >> 8;
+        const int d1 = static_cast<int8_t>(r1);
+        const int d2 = (r1 - d1) >> 8;
+        const int digit_value = digit == 0 ? d0 : digit == 1 ? d1 : digit == 2 ? d2 : 0;
+        words[b >> 2] |= static_cast<uint32_t>(digit_value & 0xff) << (8 * (b & 3));
+      }
+      qa[ks] = v4i32{static_cast<int>(words[0]), static_cast<int>(words[1]), static_cast<int>(words[2]),
+                     static_cast<int>(words[3])};
     }
-    qa = v4i32{static_cast<int>(words[0]), static_cast<int>(words[1]), static_cast<int>(words[2]), static_cast<int>(words[3])};
     if (digit == 0 && g == 0) qinv_of[h] = usable ? down : 0.0f;
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   const float qinv = qinv_of[g];   // in the score tiles a lane's head is its row block
 
-  const int swz_v_read = ((j >> 3) & 1) | ((g & 1) << 1);   // f_V of the rows this lane points at in a transposed read
+  // the rows this lane points at in a transposed read are 16 g + 8 half + j / 2: one swizzle for both halves
+  const int swz_v_read = L::swizzle_v(16 * g + (j >> 1));
   float m_run = -INFINITY, l_part = 0.0f;
-  float o_acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};               // head g, d = 16 tile + j
+  float o_acc[kDTiles];   // head g, d = 16 tile + j
+#pragma unroll
+  for (int dt = 0; dt < kDTiles; ++dt) o_acc[dt] = 0.0f;
   int stage = 0;
   for (; t0 < pos; t0 += t_step, stage ^= 1) {
     if (t0 + t_step < pos) {
@@ -953,16 +971,20 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    const unsigned char* st = mine + stage * kMfStage;
-    const float* ks_of = reinterpret_cast<const float*>(st + 2 * kMfCodes);
+    const unsigned char* st = mine + stage * L::kStage;
+    const float* ks_of = reinterpret_cast<const float*>(st + 2 * L::kCodes);
     const float* vs_of = ks_of + kMfSlab;
     // ---- scores of the slab's four tiles of 16 tokens: lane = (token 16 c + j, head g)
     float sc[4], w[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int r = 16 * c + j;
-      const v4i32 kb = *reinterpret_cast<const v4i32*>(st + r * D + 16 * (g ^ ((r >> 2) & 3)));
-      const v4i32 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qa, kb, v4i32{0, 0, 0, 0}, 0, 0, 0);
+      v4i32 acc = v4i32{0, 0, 0, 0};
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks) {
+        const v4i32 kb = *reinterpret_cast<const v4i32*>(st + r * D + 16 * ((4 * ks + g) ^ L::swizzle_k(r)));
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qa[ks], kb, acc, 0, 0, 0);
+      }
       const float dot = fmaf(static_cast<float>(acc[2]), 65536.0f,
                              fmaf(static_cast<float>(acc[1]), 256.0f, static_cast<float>(acc[0])));
       sc[c] = t0 + r < pos ? dot * (ks_of[r] * qinv) : -INFINITY;
@@ -996,9 +1018,9 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     const v4i32 pa = *reinterpret_cast<const v4i32*>(pbuf + j * kMfSlab + 16 * g);   // row j, tokens 16 g .. 16 g + 15
     // ---- weighted values, 16 of the head's dimensions per tile: lane = (d = 16 tile + j, head g)
-    const unsigned char* vrow = st + kMfCodes + (16 * g + (j >> 1)) * D + 8 * (j & 1);
+    const unsigned char* vrow = st + L::kCodes + (16 * g + (j >> 1)) * D + 8 * (j & 1);
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt) {
+    for (int dt = 0; dt < kDTiles; ++dt) {
       const int at = 16 * (dt ^ swz_v_read);
       const v2i32 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
           (__attribute__((address_space(3))) v2i32*)(vrow + at));                // tokens 16 g .. 16 g + 7
@@ -1016,19 +1038,19 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
   // ---- the waves meet: (max, sum, output) per wave and head, then the new token, then the split's record --------
   {
     const float l_row = row16_sum(l_part);
-    float* rec = s_rec + (wv * HEADS + g) * kMfRec;
+    float* rec = s_rec + (wv * HEADS + g) * L::kRec;
     if (j == 0) {
       rec[0] = m_run;
       rec[1] = l_row;
     }
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt) rec[2 + 16 * dt + j] = o_acc[dt];
+    for (int dt = 0; dt < kDTiles; ++dt) rec[2 + 16 * dt + j] = o_acc[dt];
   }
   if (wv == kSplitWaves - 1) {
     // the new token is a record of its own: its scores here, its value is s_new[1]
     float dot = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dot = fmaf(s_q[g][4 * j + i], s_new[0][4 * j + i], dot);
+    for (int i = 0; i < D / 16; ++i) dot = fmaf(s_q[g][(D / 16) * j + i], s_new[0][(D / 16) * j + i], dot);
     dot = row16_sum(dot);
     if (j == 0) s_new_score[g] = last_split ? dot : -INFINITY;
   }
@@ -1038,11 +1060,11 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
     const float new_score = s_new_score[h];
     float mm = new_score;
 #pragma unroll
-    for (int w2 = 0; w2 < kSplitWaves; ++w2) mm = fmaxf(mm, s_rec[(w2 * HEADS + h) * kMfRec]);
+    for (int w2 = 0; w2 < kSplitWaves; ++w2) mm = fmaxf(mm, s_rec[(w2 * HEADS + h) * L::kRec]);
     float ll = 0.0f, oo = 0.0f;
 #pragma unroll
     for (int w2 = 0; w2 < kSplitWaves; ++w2) {
-      const float* rec = s_rec + (w2 * HEADS + h) * kMfRec;
+      const float* rec = s_rec + (w2 * HEADS + h) * L::kRec;
       const float a = rec[0] == -INFINITY ? 0.0f : exp2f(rec[0] - mm);
       ll += rec[1] * a;
       oo += rec[2 + d] * a;
@@ -1617,12 +1639,12 @@ extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos
   const int rep_heads = q_heads / kv_heads;
   const bool grouped = rep_heads % 4 == 0 && n_splits >= 32;
   const dim3 grid(grouped ? q_heads / 4 : q_heads, n_splits), block(kSplitThreads);
-  if (grouped && bits == 8 && head_dim == kMfD && t_max >= kMfMinCache) {
-    // int8 codes of 64-wide heads: the matrix-core form (ctx 8 K / 32 K / 131 K, 32 heads on 8 kv heads: see the
-    // kernel's comment for what it changes in the arithmetic)
-#define LLMQ_SPLIT_MFMA(T)                                                                                        \
+  if (grouped && bits == 8 && t_max >= kMfMinCache) {
+    // int8 codes: the matrix-core form (see the kernel's comment for what it changes in the arithmetic)
+#define LLMQ_SPLIT_MFMA(T, D)                                                                                     \
   do {                                                                                                            \
-    auto kernel = kv_rope_append_attend_split_mfma_kernel<T>;                                                     \
+    auto kernel = kv_rope_append_attend_split_mfma_kernel<T, D>;                                                  \
+    constexpr int kMfLdsBytes = MfLds<D>::kBytes;                                                                 \
     static bool raised = false; /* per instantiation; worst case two threads both set it */                       \
     if (!raised) {                                                                                                \
       const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                           \
@@ -1638,12 +1660,16 @@ extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos
                        static_cast<uint8_t*>(k_codes), static_cast<uint8_t*>(v_codes), k_scale, v_scale, partials, \
                        pos_dev, scale_log2, q_heads, kv_heads, t_max);                                            \
   } while (0)
+#define LLMQ_SPLIT_MFMA_D(T)                                           \
+  if (head_dim == 64) LLMQ_SPLIT_MFMA(T, 64); else LLMQ_SPLIT_MFMA(T, 128); \
+  break;
     switch (dtype) {
-      case LLMQ_F32: LLMQ_SPLIT_MFMA(float); break;
-      case LLMQ_F16: LLMQ_SPLIT_MFMA(f16_t); break;
-      case LLMQ_BF16: LLMQ_SPLIT_MFMA(bf16_t); break;
+      case LLMQ_F32: LLMQ_SPLIT_MFMA_D(float)
+      case LLMQ_F16: LLMQ_SPLIT_MFMA_D(f16_t)
+      case LLMQ_BF16: LLMQ_SPLIT_MFMA_D(bf16_t)
       default: return llmq_host::fail_invalid("unsupported dtype code %d", dtype);
     }
+#undef LLMQ_SPLIT_MFMA_D
 #undef LLMQ_SPLIT_MFMA
     return llmq_host::check_launch("kv_rope_append_attend_split_mfma_kernel");
   }
