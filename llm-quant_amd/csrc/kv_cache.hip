@@ -826,6 +826,10 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
 // own, filled by DMA (codes of K and V with their 16-byte pieces XOR-swizzled by row so that the operand reads and
 // the transposed reads meet no bank conflict, and the two scale vectors): no barrier inside the loop. The records
 // it leaves are those of the kernel above.
+// 4-bit codes: a lane's eight packed bytes (16 codes) become two operand halves, the low nibbles (even dimensions) and
+// the high ones (odd), with the query's digits laid out in the same order; V's packed bytes go through the same
+// transposed read and split into the operand of an even and of an odd dimension. The nibbles are code + 8: the 8
+// leaves through the C operand of the multiply (- 8 * the sum of the other operand's row, an integer the lane has).
 typedef int v4i32 __attribute__((ext_vector_type(4)));
 typedef int v2i32 __attribute__((ext_vector_type(2)));
 
@@ -835,34 +839,42 @@ constexpr int kMfSlab = 64;   // tokens of one wave step
 // cache holds them; the step is bound by latency there whichever form runs
 constexpr int kMfMinCache = 4096;
 
-template <int D> struct MfLds {
-  static constexpr int kPieces = D / 16;                          // 16-byte pieces of a row of codes
-  static constexpr int kTransfers = kMfSlab * D / 1024;           // 1 KB DMA instructions per tensor and slab
-  static constexpr int kCodes = kMfSlab * D;                      // bytes of a slab's K (or V) codes
+template <int BITS, int D> struct MfLds {
+  static constexpr int kRowBytes = D * BITS / 8;                  // a token's codes: 32, 64 or 128 bytes
+  static constexpr int kPieces = kRowBytes / 16;                  // 16-byte pieces of a row of codes
+  static constexpr int kTransfers = kMfSlab * kRowBytes / 1024;   // 1 KB DMA instructions per tensor and slab
+  static constexpr int kCodes = kMfSlab * kRowBytes;              // bytes of a slab's K (or V) codes
   static constexpr int kStage = 2 * kCodes + 2 * kMfSlab * 4;     // K codes, V codes, K scales, V scales
   static constexpr int kP = 16 * kMfSlab;                         // the weights as operand rows: [16 rows][64 tokens] bytes
-  static constexpr int kWaveBytes = 2 * kStage + kP + 64;         // two stages, the weights, 2^-sh per head
+  static constexpr int kWaveBytes = 2 * kStage + kP + 512;        // two stages, the weights, per-head constants
   static constexpr int kRec = D + 2;                              // a wave's (max, sum, output) per head
   static constexpr int kHeaderFloats = kMfHeads * D + 2 * D + kSplitWaves * kMfHeads * kRec + kMfHeads;
   static constexpr int kHeaderBytes = (kHeaderFloats * 4 + 255) / 256 * 256;
-  static constexpr int kBytes = kHeaderBytes + kSplitWaves * kWaveBytes;   // 80 KB (D = 64), 148 KB (D = 128)
-  // Slot of a row's 16-byte piece p in LDS is p ^ swizzle(row). K is read as operands: 16 lanes read the same piece
-  // of 16 consecutive rows and have to land in 16 different bank quads. V is read transposed: a lane points at 8
-  // bytes of row 16 g + 8 half + s / 2 (s its index among its 16 lanes), two such groups of lanes go together.
-  static __device__ __forceinline__ int swizzle_k(int row) { return D == 64 ? (row >> 2) & 3 : (row >> 1) & 7; }
+  static constexpr int kBytes = kHeaderBytes + kSplitWaves * kWaveBytes;   // int8: 82 KB (D = 64), 150 KB (D = 128)
+  // Slot of a row's 16-byte piece p in LDS is p ^ swizzle(row); both depend on the row's bytes only. K is read as
+  // operands: 16 lanes read the same piece (or, 4-bit, the same eight bytes) of 16 consecutive rows and have to land
+  // in different banks. V is read transposed: a lane points at 8 bytes of row 16 g + 8 half + s / 2 (s its index
+  // among its 16 lanes), two such groups of lanes go together.
+  static __device__ __forceinline__ int swizzle_k(int row) {
+    return kRowBytes == 32 ? (row >> 3) & 1 : kRowBytes == 64 ? (row >> 2) & 3 : (row >> 1) & 7;
+  }
   static __device__ __forceinline__ int swizzle_v(int row) {
-    return D == 64 ? ((row >> 2) & 1) | (((row >> 4) & 1) << 1) : ((row >> 1) & 3) | (((row >> 4) & 1) << 2);
+    return kRowBytes == 32   ? (row >> 4) & 1
+           : kRowBytes == 64 ? ((row >> 2) & 1) | (((row >> 4) & 1) << 1)
+                             : ((row >> 1) & 3) | (((row >> 4) & 1) << 2);
   }
 };
 
-template <typename T, int D>
+template <typename T, int BITS, int D>
 __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_mfma_kernel(
     const T* __restrict__ qkv, const T* __restrict__ cos_table, const T* __restrict__ sin_table,
     uint8_t* __restrict__ k_codes, uint8_t* __restrict__ v_codes, float* __restrict__ k_scale,
     float* __restrict__ v_scale, float* __restrict__ partials, const int32_t* __restrict__ pos_dev,
     const float sm_scale_log2, const int q_heads, const int kv_heads, const int t_max) {
-  using L = MfLds<D>;
+  using L = MfLds<BITS, D>;
   constexpr int HEADS = kMfHeads;
+  constexpr int RB = L::kRowBytes;
+  constexpr uint32_t kNibbles = 0x0f0f0f0fu;
   constexpr int GREC = D + kAttnRecordHeader;
   constexpr int kKSteps = D / 64;    // matrix-core steps along a head's dimensions
   constexpr int kDTiles = D / 16;    // tiles of 16 dimensions of the output
@@ -883,23 +895,24 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
 
   unsigned char* mine = mf_smem + L::kHeaderBytes + wv * L::kWaveBytes;
   unsigned char* pbuf = mine + 2 * L::kStage;
-  float* qinv_of = reinterpret_cast<float*>(pbuf + L::kP);
+  float* qinv_of = reinterpret_cast<float*>(pbuf + L::kP);        // [4]: 2^-sh per head
+  int* qpart_of = reinterpret_cast<int*>(pbuf + L::kP + 64);       // [4 blocks][16 rows]: sums of the query's digits
 
-  const uint8_t* kbase = k_codes + static_cast<int64_t>(kvh) * t_max * D;
-  const uint8_t* vbase = v_codes + static_cast<int64_t>(kvh) * t_max * D;
+  const uint8_t* kbase = k_codes + static_cast<int64_t>(kvh) * t_max * RB;
+  const uint8_t* vbase = v_codes + static_cast<int64_t>(kvh) * t_max * RB;
   const float* ksc = k_scale + static_cast<int64_t>(kvh) * t_max;
   const float* vsc = v_scale + static_cast<int64_t>(kvh) * t_max;
-  // transfer i of a slab's codes lands in LDS bytes 1024 i + 16 lane: row (1024 / D) i + lane / pieces, slot
+  // transfer i of a slab's codes lands in LDS bytes 1024 i + 16 lane: row (1024 / row bytes) i + lane / pieces, slot
   // lane % pieces
   auto request = [&](const int t0, const int stage) {
     unsigned char* st = mine + stage * L::kStage;
 #pragma unroll
     for (int i = 0; i < L::kTransfers; ++i) {
-      const int row = (1024 / D) * i + lane / L::kPieces, slot = lane % L::kPieces;
+      const int row = (1024 / RB) * i + lane / L::kPieces, slot = lane % L::kPieces;
       const int64_t t = min(t0 + row, t_max - 1);   // (rows past the cache's end: the last row again)
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(kbase + t * D + 16 * (slot ^ L::swizzle_k(row))),
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(kbase + t * RB + 16 * (slot ^ L::swizzle_k(row))),
                                        reinterpret_cast<u32x4*>(st + 1024 * i), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(vbase + t * D + 16 * (slot ^ L::swizzle_v(row))),
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(vbase + t * RB + 16 * (slot ^ L::swizzle_v(row))),
                                        reinterpret_cast<u32x4*>(st + L::kCodes + 1024 * i), 16, 0, 0);
     }
     const int64_t ts = min(t0 + lane, t_max - 1);
@@ -919,14 +932,16 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
   const int pos = min(max(pos_dev[0], 0), t_max - 1);
   const T* cos_row = cos_table + static_cast<int64_t>(pos) * D;
   const T* sin_row = sin_table + static_cast<int64_t>(pos) * D;
-  split_phase_a<T, 8, D, HEADS>(qkv, cos_row, sin_row, k_codes, v_codes, k_scale, v_scale, sm_scale_log2, q_heads,
+  split_phase_a<T, BITS, D, HEADS>(qkv, cos_row, sin_row, k_codes, v_codes, k_scale, v_scale, sm_scale_log2, q_heads,
                                 kv_heads, t_max, pos, qh0, kvh, last_split, writer, lane, wv, s_q, s_new);
   // operand rows the weights never reach (two of a head's four) stay zero
   for (int i = lane; i < L::kP / 4; i += kWave) reinterpret_cast<uint32_t*>(pbuf)[i] = 0u;
   __syncthreads();
 
   // ---- the query heads as operand rows: lane (row = j = 4 head + digit, block g) holds d = 64 step + 16 g .. + 15
+  // (4-bit codes: in the order the nibbles of eight bytes come apart, the even dimensions, then the odd ones)
   v4i32 qa[kKSteps];
+  v4i32 q_bias = v4i32{0, 0, 0, 0};   // 4-bit: - 8 * (sum of the digits of rows 4 g .. 4 g + 3), the scores' C operand
   {
     const int h = j >> 2, digit = j & 3;
     float amax = 0.0f;
@@ -936,26 +951,37 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
     const bool usable = e >= 22u && e < 255u;                       // (below 2^-105 the head counts as zero)
     const float up = __builtin_bit_cast(float, (275u - e) << 23);  // 2^(148 - e): amax * up in [2^21, 2^22)
     const float down = __builtin_bit_cast(float, (e - 21u) << 23); // 2^(e - 148)
+    int digit_sum = 0;
 #pragma unroll
     for (int ks = 0; ks < kKSteps; ++ks) {
       uint32_t words[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
       for (int b = 0; b < 16; ++b) {
-        const int qi = usable ? static_cast<int>(rintf(s_q[h][64 * ks + 16 * g + b] * up)) : 0;
+        const int d_in_block = BITS == 8 ? b : (b < 8 ? 2 * b : 2 * (b - 8) + 1);
+        const int qi = usable ? static_cast<int>(rintf(s_q[h][64 * ks + 16 * g + d_in_block] * up)) : 0;
         const int d0 = static_cast<int8_t>(qi);
         const int r1 = (qi - d0) >> 8;
         const int d1 = static_cast<int8_t>(r1);
         const int d2 = (r1 - d1) >> 8;
         const int digit_value = digit == 0 ? d0 : digit == 1 ? d1 : digit == 2 ? d2 : 0;
         words[b >> 2] |= static_cast<uint32_t>(digit_value & 0xff) << (8 * (b & 3));
+        digit_sum += digit_value;
       }
       qa[ks] = v4i32{static_cast<int>(words[0]), static_cast<int>(words[1]), static_cast<int>(words[2]),
                      static_cast<int>(words[3])};
     }
     if (digit == 0 && g == 0) qinv_of[h] = usable ? down : 0.0f;
+    if constexpr (BITS == 4) qpart_of[16 * g + j] = digit_sum;
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   const float qinv = qinv_of[g];   // in the score tiles a lane's head is its row block
+  if constexpr (BITS == 4) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = 4 * g + r;
+      q_bias[r] = -8 * ((qpart_of[row] + qpart_of[16 + row]) + (qpart_of[32 + row] + qpart_of[48 + row]));
+    }
+  }
 
   // the rows this lane points at in a transposed read are 16 g + 8 half + j / 2: one swizzle for both halves
   const int swz_v_read = L::swizzle_v(16 * g + (j >> 1));
@@ -979,10 +1005,19 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int r = 16 * c + j;
-      v4i32 acc = v4i32{0, 0, 0, 0};
+      v4i32 acc = q_bias;
 #pragma unroll
       for (int ks = 0; ks < kKSteps; ++ks) {
-        const v4i32 kb = *reinterpret_cast<const v4i32*>(st + r * D + 16 * ((4 * ks + g) ^ L::swizzle_k(r)));
+        v4i32 kb;
+        if constexpr (BITS == 8) {
+          kb = *reinterpret_cast<const v4i32*>(st + r * RB + 16 * ((4 * ks + g) ^ L::swizzle_k(r)));
+        } else {
+          // the lane's 16 codes are bytes 32 ks + 8 g .. + 7 of the row
+          const u32x2 raw = *reinterpret_cast<const u32x2*>(st + r * RB + 16 * ((2 * ks + (g >> 1)) ^ L::swizzle_k(r)) +
+                                                            8 * (g & 1));
+          kb = v4i32{static_cast<int>(raw.x & kNibbles), static_cast<int>(raw.y & kNibbles),
+                     static_cast<int>((raw.x >> 4) & kNibbles), static_cast<int>((raw.y >> 4) & kNibbles)};
+        }
         acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qa[ks], kb, acc, 0, 0, 0);
       }
       const float dot = fmaf(static_cast<float>(acc[2]), 65536.0f,
@@ -1007,6 +1042,7 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
     const uint32_t we = max(__builtin_bit_cast(uint32_t, w_max) >> 23, 13u);   // w_max = f 2^(we - 126)
     const float w_up = __builtin_bit_cast(float, (267u - we) << 23);            // 2^(140 - we): w * w_up < 2^14
     const float w_down = __builtin_bit_cast(float, (we - 13u) << 23);           // 2^(we - 140)
+    int w_sum0 = 0, w_sum1 = 0;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int wi = static_cast<int>(rintf(w[c] * w_up));
@@ -1014,22 +1050,38 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
       const int d1 = (wi - d0) >> 8;
       pbuf[(4 * g) * kMfSlab + 16 * c + j] = static_cast<unsigned char>(d0);
       pbuf[(4 * g + 1) * kMfSlab + 16 * c + j] = static_cast<unsigned char>(d1);
+      w_sum0 += d0;
+      w_sum1 += d1;
     }
+    v4i32 w_bias = v4i32{0, 0, 0, 0};   // 4-bit: - 8 * (sum over the slab of the head's digits), the values' C operand
+    if constexpr (BITS == 4) w_bias = v4i32{-8 * row16_sum(w_sum0), -8 * row16_sum(w_sum1), 0, 0};
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     const v4i32 pa = *reinterpret_cast<const v4i32*>(pbuf + j * kMfSlab + 16 * g);   // row j, tokens 16 g .. 16 g + 15
-    // ---- weighted values, 16 of the head's dimensions per tile: lane = (d = 16 tile + j, head g)
-    const unsigned char* vrow = st + L::kCodes + (16 * g + (j >> 1)) * D + 8 * (j & 1);
+    // ---- weighted values, 16 of the head's dimensions per tile: lane = (head g, d = 16 tile + j; 4-bit: tiles come
+    // in pairs from 16 packed bytes a token, d = 32 pair + 2 j and + 1)
+    const unsigned char* vrow = st + L::kCodes + (16 * g + (j >> 1)) * RB + 8 * (j & 1);
 #pragma unroll
-    for (int dt = 0; dt < kDTiles; ++dt) {
-      const int at = 16 * (dt ^ swz_v_read);
+    for (int bt = 0; bt < RB / 16; ++bt) {
+      const int at = 16 * (bt ^ swz_v_read);
       const v2i32 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
           (__attribute__((address_space(3))) v2i32*)(vrow + at));                // tokens 16 g .. 16 g + 7
       const v2i32 hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-          (__attribute__((address_space(3))) v2i32*)(vrow + 8 * D + at));        // 16 g + 8 .. 16 g + 15
+          (__attribute__((address_space(3))) v2i32*)(vrow + 8 * RB + at));       // 16 g + 8 .. 16 g + 15
       const v4i32 vb = v4i32{lo[0], lo[1], hi[0], hi[1]};
-      const v4i32 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(pa, vb, v4i32{0, 0, 0, 0}, 0, 0, 0);
-      const float sum = fmaf(static_cast<float>(acc[1]), 256.0f, static_cast<float>(acc[0]));
-      o_acc[dt] = fmaf(o_acc[dt], alpha, sum * w_down);
+      if constexpr (BITS == 8) {
+        const v4i32 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(pa, vb, w_bias, 0, 0, 0);
+        const float sum = fmaf(static_cast<float>(acc[1]), 256.0f, static_cast<float>(acc[0]));
+        o_acc[bt] = fmaf(o_acc[bt], alpha, sum * w_down);
+      } else {
+        const v4i32 even = vb & static_cast<int>(kNibbles);
+        const v4i32 odd = (vb >> 4) & static_cast<int>(kNibbles);
+        const v4i32 acc_e = __builtin_amdgcn_mfma_i32_16x16x64_i8(pa, even, w_bias, 0, 0, 0);
+        const v4i32 acc_o = __builtin_amdgcn_mfma_i32_16x16x64_i8(pa, odd, w_bias, 0, 0, 0);
+        const float sum_e = fmaf(static_cast<float>(acc_e[1]), 256.0f, static_cast<float>(acc_e[0]));
+        const float sum_o = fmaf(static_cast<float>(acc_o[1]), 256.0f, static_cast<float>(acc_o[0]));
+        o_acc[2 * bt] = fmaf(o_acc[2 * bt], alpha, sum_e * w_down);
+        o_acc[2 * bt + 1] = fmaf(o_acc[2 * bt + 1], alpha, sum_o * w_down);
+      }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // (the stage and the weights are free for the next round)
   }
@@ -1044,7 +1096,10 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
       rec[1] = l_row;
     }
 #pragma unroll
-    for (int dt = 0; dt < kDTiles; ++dt) rec[2 + 16 * dt + j] = o_acc[dt];
+    for (int dt = 0; dt < kDTiles; ++dt) {
+      const int d = BITS == 8 ? 16 * dt + j : 32 * (dt >> 1) + 2 * j + (dt & 1);
+      rec[2 + d] = o_acc[dt];
+    }
   }
   if (wv == kSplitWaves - 1) {
     // the new token is a record of its own: its scores here, its value is s_new[1]
@@ -1639,12 +1694,12 @@ extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos
   const int rep_heads = q_heads / kv_heads;
   const bool grouped = rep_heads % 4 == 0 && n_splits >= 32;
   const dim3 grid(grouped ? q_heads / 4 : q_heads, n_splits), block(kSplitThreads);
-  if (grouped && bits == 8 && t_max >= kMfMinCache) {
-    // int8 codes: the matrix-core form (see the kernel's comment for what it changes in the arithmetic)
-#define LLMQ_SPLIT_MFMA(T, D)                                                                                     \
+  if (grouped && t_max >= kMfMinCache) {
+    // long caches: the matrix-core form (see the kernel's comment for what it changes in the arithmetic)
+#define LLMQ_SPLIT_MFMA(T, B, D)                                                                                  \
   do {                                                                                                            \
-    auto kernel = kv_rope_append_attend_split_mfma_kernel<T, D>;                                                  \
-    constexpr int kMfLdsBytes = MfLds<D>::kBytes;                                                                 \
+    auto kernel = kv_rope_append_attend_split_mfma_kernel<T, B, D>;                                               \
+    constexpr int kMfLdsBytes = MfLds<B, D>::kBytes;                                                              \
     static bool raised = false; /* per instantiation; worst case two threads both set it */                       \
     if (!raised) {                                                                                                \
       const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                           \
@@ -1660,8 +1715,9 @@ extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos
                        static_cast<uint8_t*>(k_codes), static_cast<uint8_t*>(v_codes), k_scale, v_scale, partials, \
                        pos_dev, scale_log2, q_heads, kv_heads, t_max);                                            \
   } while (0)
-#define LLMQ_SPLIT_MFMA_D(T)                                           \
-  if (head_dim == 64) LLMQ_SPLIT_MFMA(T, 64); else LLMQ_SPLIT_MFMA(T, 128); \
+#define LLMQ_SPLIT_MFMA_D(T)                                                        \
+  if (bits == 8) { if (head_dim == 64) LLMQ_SPLIT_MFMA(T, 8, 64); else LLMQ_SPLIT_MFMA(T, 8, 128); } \
+  else { if (head_dim == 64) LLMQ_SPLIT_MFMA(T, 4, 64); else LLMQ_SPLIT_MFMA(T, 4, 128); }           \
   break;
     switch (dtype) {
       case LLMQ_F32: LLMQ_SPLIT_MFMA_D(float)

@@ -310,20 +310,21 @@ def test_decode_step_attention_against_the_oracle(ext, bits, ctx, splits):
     (5002, 32, 5004, 32, 8, 64), (9000, 64, 9216, 32, 8, 64), (3000, 48, 4100, 8, 2, 64), (20000, 32, 20001, 16, 2, 64),
     (2048, 32, 4096, 32, 8, 128), (0, 32, 4096, 32, 8, 128), (65, 32, 4096, 32, 8, 128), (4094, 32, 4096, 32, 8, 128),
     (5002, 32, 5004, 32, 8, 128), (9000, 64, 9216, 8, 2, 128)])
-def test_long_cache_decode_step_on_the_matrix_core_against_the_oracle(ext, ctx, splits, t_max, q_heads, kv_heads, d):
-    """Caches of 4096 rows and more under grouped-query attention with int8 codes take the
+@pytest.mark.parametrize("bits", [8, 4])
+def test_long_cache_decode_step_on_the_matrix_core_against_the_oracle(ext, bits, ctx, splits, t_max, q_heads, kv_heads,
+                                                                      d):
+    """Caches of 4096 rows and more under grouped-query attention take the
     matrix-core form of the split step (codes as int8 operands, the query in three digits, the softmax weights
     in two): the same checks as the vector-ALU form gets, against the same oracle (appended codes and scales bit
     for bit, output rel-L2 <= 1e-2 and <= 2e-2 per head), at contexts around the 64-token slab boundaries, with
     one token and none, up to the cache's last row, with cache lengths that are not whole slabs. Rows beyond the
     position hold random codes and NaN scales: nothing of them may reach the result."""
-    bits = 8
     cache, qkv, cos_t, sin_t, want, (kq, ks, vq, vs) = decode_step_case(ext, bits, ctx, q_heads, kv_heads, d, seed=ctx,
                                                                         t_max=t_max)
     gen = torch.Generator(device="cuda").manual_seed(1)
     for name in ("k_codes", "v_codes"):
-        cache[name][:, ctx + 1:] = torch.randint(-128, 128, cache[name][:, ctx + 1:].shape, generator=gen,
-                                                 device="cuda").to(cache[name].dtype)
+        cache[name][:, ctx + 1:] = torch.randint(0, 256, cache[name][:, ctx + 1:].shape, generator=gen,
+                                                 device="cuda").to(torch.uint8).view(cache[name].dtype)
     for name in ("k_scale", "v_scale"):
         cache[name][:, ctx + 1:] = float("nan")
     position = torch.tensor([ctx], dtype=torch.int32, device="cuda")
@@ -340,4 +341,4 @@ def test_long_cache_decode_step_on_the_matrix_core_against_the_oracle(ext, ctx, 
     assert rel_l2(got, want) <= 1e-2
     per_head = np.linalg.norm(got - want, axis=1) / np.linalg.norm(want, axis=1)
     assert per_head.max() <= 2e-2, per_head.argmax()
-    print(f"ctx {ctx} splits {splits} d {d}: rel-L2 {rel_l2(got, want):.2e}, worst head {per_head.max():.2e}")
+    print(f"int{bits} ctx {ctx} splits {splits} d {d}: rel-L2 {rel_l2(got, want):.2e}, worst head {per_head.max():.2e}")
