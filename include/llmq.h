@@ -367,7 +367,12 @@ int llmq_kv_rope_append_attend(const void* qkv, const void* cos_table, const voi
  * dtype(merge(partials)) (o_proj of a decoder layer; in_head_dim / residual as there).
  * With n_splits >= 32 and q_heads / kv_heads a multiple of 4 a workgroup takes four query heads of
  * a kv head together, so every cache row is read and dequantized once for the four (long caches:
- * the step is bound by that arithmetic); the records and their layout are the same. */
+ * the step is bound by that arithmetic); the records and their layout are the same. When in
+ * addition t_max >= 4096, the four heads' scores and weighted values are computed on the int8 matrix
+ * core with the cache's codes as operands (the query in three base-256 digits, the softmax weights
+ * times the value scales in two): exact integer sums of code * scale, without the rounding of the
+ * dequantized K and V to `dtype` that the other forms make as the reference's cache does; the
+ * output agrees with them to ~1e-3 relative. */
 size_t llmq_kv_attend_partials_floats(int q_heads, int head_dim, int n_splits);
 int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos_table, const void* sin_table,
                                      void* k_codes, void* v_codes, float* k_scale, float* v_scale,
