@@ -247,6 +247,14 @@ class LlamaKernelRuntime:
             self.logits, self.next_token = self._step()
         self._set_step_inputs(token, position)
 
+    def _ensure_graph(self, token, position: int):
+        """A captured step that starts from (token, position): captured now, or, on a kept runtime, the one it has
+        (it reads token and position from the device)."""
+        if self.graph is None:
+            self.capture(token, position)
+        else:
+            self._set_step_inputs(token, position)
+
     @torch.no_grad()
     def step(self):
         """Replay one step; the token fed is the previous step's argmax, already on the device."""
@@ -272,10 +280,7 @@ class LlamaKernelRuntime:
         out = [nxt.reshape(1, 1)]
         if max_new_tokens > 1:
             if use_graph:
-                if self.graph is None:
-                    self.capture(nxt, prompt)
-                else:  # a kept runtime: the captured step reads token and position from the device
-                    self._set_step_inputs(nxt, prompt)
+                self._ensure_graph(nxt, prompt)
                 for _ in range(max_new_tokens - 1):
                     out.append(self.step().clone().reshape(1, 1))
             else:

@@ -44,6 +44,12 @@ def _fusable(*mods) -> bool:
     return True
 
 
+# cached tokens from which a long cache's decode step takes its many-split, matrix-core attention launch: measured on
+# the 1B architecture in a 32 K-row cache, us a token with 8 / 32 splits: 600 tokens 551 / 636, 2000: 578 / 637,
+# 5000: 636 / 636, 7000: 673 / 639, 31000: 1104 / 728
+LONG_CONTEXT_FROM = 5120
+
+
 class _Fused:
     """Concatenated storage of Linears that read the same activation."""
 
@@ -78,16 +84,25 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         hands o_proj a finished attention output instead of partial records."""
         super().__init__(model, max_len, kv_bits, exact_prefill)
         self._ext = load_extension()
+        # A cache of many thousand rows is often mostly empty: the split count (and with it the kernel form) a step
+        # runs with follows the tokens the cache holds, in two regimes with a captured step each.
+        self.short_splits = None     # split count below `long_from` cached tokens; None: one regime
+        self.long_from = LONG_CONTEXT_FROM
         if attn_splits is None:
             # one workgroup per CU at least, four more splits per 2048 tokens of cache up to 16; from
             # ~12 K tokens on 32 splits, where the kernel takes the four query heads of a kv head
-            # together (grouped-query models) and dequantizes every cache row once for all of them
+            # together (grouped-query models) with the cache's codes as matrix-core operands
             grouped = self.kv_heads > 0 and (self.q_heads // self.kv_heads) % 4 == 0
+            short = max(1, 256 // max(self.q_heads, 1))
             if max_len >= 12288 and grouped:
                 attn_splits = 32
+                if short < attn_splits:
+                    self.short_splits = short
             else:
-                attn_splits = max(1, 256 // max(self.q_heads, 1), min(16, (max_len + 2047) // 2048 * 4))
+                attn_splits = max(short, min(16, (max_len + 2047) // 2048 * 4))
         self.attn_splits = int(attn_splits)
+        self._splits_now = self.attn_splits
+        self._graphs = {}            # split count -> (graph, logits, next_token)
         self._partials = torch.zeros(self._ext.kv_attend_partials_floats(self.q_heads, self.head_dim,
                                                                          self.attn_splits),
                                      dtype=torch.float32, device=self.device) if self.attn_splits > 1 else None
@@ -187,19 +202,19 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
     def _forward(self, token_ids, cos, sin, decode: bool):
         if not decode:
             return super()._forward(token_ids, cos, sin, decode)
-        ext, cache = self._ext, self.cache
+        ext, cache, splits = self._ext, self.cache, self._splits_now
         # (the row _set_step_inputs or the previous step's token pick left for this token)
         hidden = self._hidden0 if self._embed_table is not None else self.model.model.embed_tokens(token_ids)
         for index, f in enumerate(self.fused_layers):
             qkv = ext.wq_gemv_fused(hidden, f["qkv"].qdata, f["qkv"].wscale, f["qkv"].out_group, PRO_RMSNORM,
                                     f["norm1"], f["eps1"], 0, None)
-            if self.attn_splits > 1:
+            if splits > 1:
                 # partial records per (head, split), merged by o_proj while it stages its activation
                 ext.kv_rope_append_attend_split(qkv, self.cos_table, self.sin_table, cache.k_codes[index],
                                                 cache.v_codes[index], cache.k_scale[index], cache.v_scale[index],
                                                 self._partials, cache.position, self.scaling, self.q_heads,
-                                                self.attn_splits)
-                hidden = ext.wq_gemv_attn_merge(self._partials, self.attn_splits, self.head_dim, f["o"].qdata,
+                                                splits)
+                hidden = ext.wq_gemv_attn_merge(self._partials, splits, self.head_dim, f["o"].qdata,
                                                 f["o"].wscale, f["o"].out_group, f["o_head_dim"], hidden,
                                                 hidden.dtype)
             else:
@@ -221,10 +236,46 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         return ext.wq_gemv_fused(hidden, head.qdata, head.wscale, head.out_group, PRO_RMSNORM, self.final_norm,
                                  self.final_eps, 0, None)
 
+    def _splits_for(self, cached_tokens: int) -> int:
+        """Split count of the attention launch for a cache that holds this many tokens."""
+        if self.short_splits is not None and cached_tokens < self.long_from:
+            return self.short_splits
+        return self.attn_splits
+
     def _set_step_inputs(self, token, position: int):
         super()._set_step_inputs(token, position)
+        self._splits_now = self._splits_for(position)
         if self._embed_table is not None:
             self._hidden0.copy_(self.model.model.embed_tokens(self.token))
+
+    def _use_graph_of(self, splits: int) -> bool:
+        kept = self._graphs.get(splits)
+        if kept is None:
+            return False
+        self.graph, self.logits, self.next_token = kept
+        self._splits_now = splits
+        return True
+
+    @torch.no_grad()
+    def capture(self, token, position: int):
+        """One captured step per regime: the one `position` falls in is captured (or, if it has been, made current)."""
+        if self._use_graph_of(self._splits_for(position)):
+            self._set_step_inputs(token, position)
+            return
+        super().capture(token, position)
+        self._graphs[self._splits_now] = (self.graph, self.logits, self.next_token)
+
+    def _ensure_graph(self, token, position: int):
+        self.capture(token, position)
+
+    @torch.no_grad()
+    def step(self):
+        # the cache has grown (or been rewound) into the other regime: its captured step takes over, from the token
+        # and position the previous step left on the device
+        position = self.cache.get_seq_length()
+        if self.short_splits is not None and self._splits_for(position) != self._splits_now:
+            self.capture(self.token.clone(), position)
+        return super().step()
 
     def _step(self):
         logits = self._forward(self.token, None, None, decode=True)

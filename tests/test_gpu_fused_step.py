@@ -412,3 +412,42 @@ def test_prompt_pass_with_its_own_attention_and_two_launch_mlp():
     assert torch.equal(library.cache.k_codes[0, :, :300], fused.cache.k_codes[0, :, :300])
     step = (library.cache.k_codes[1, :, :300].int() - fused.cache.k_codes[1, :, :300].int()).abs()
     assert float((step <= 1).float().mean()) > 0.99 and int(step.max()) <= 3
+
+
+def test_decode_step_follows_the_tokens_the_cache_holds_through_two_regimes():
+    """A long cache that is mostly empty: below `long_from` cached tokens the step runs the attention launch with
+    the short cache's split count, from there on with the many-split form (here: the matrix-core kernel, the cache
+    has 12288 rows), each regime with a captured step of its own. Graph replay and eager steps pick the same
+    launches at the same positions, so their tokens are equal; a second generation reuses both captured steps."""
+    from test_gpu_decode import build_model, quantized_pair
+
+    from llmquant.runtime import LlamaFusedRuntime
+
+    _, kernel = quantized_pair(build_model(512, 1024, 3, 8, 2, 4096))
+    ids = torch.randint(0, 4096, (1, 40), generator=torch.Generator().manual_seed(5)).cuda()
+
+    def runtime():
+        rt = LlamaFusedRuntime(kernel, 12288, 8)
+        assert rt.attn_splits == 32
+        rt.short_splits, rt.long_from = 8, 48   # (8 heads: the automatic choice has one regime; forced here)
+        return rt
+
+    eager, graphed = runtime(), runtime()
+    seen = []
+    real = eager._ext.kv_rope_append_attend_split
+    try:
+        eager._ext.kv_rope_append_attend_split = lambda *a: (seen.append((eager.cache.get_seq_length(), a[11])), real(*a))[1]
+        out_eager = eager.generate(ids, 24, use_graph=False)
+    finally:
+        eager._ext.kv_rope_append_attend_split = real
+    by_position = dict(seen)
+    assert all(by_position[p] == (8 if p < 48 else 32) for p in range(40, 63)), by_position
+    out_graphed = graphed.generate(ids, 24, use_graph=True)
+    assert torch.equal(out_graphed, out_eager)
+    assert sorted(graphed._graphs) == [8, 32]
+    kept = dict(graphed._graphs)
+    assert torch.equal(graphed.generate(ids, 24, use_graph=True), out_eager)
+    assert all(graphed._graphs[k][0] is kept[k][0] for k in kept)   # no step was captured again
+    # a prompt that already lies in the long regime starts there
+    long_ids = torch.randint(0, 4096, (1, 60), generator=torch.Generator().manual_seed(6)).cuda()
+    assert torch.equal(graphed.generate(long_ids, 8, use_graph=True), eager.generate(long_ids, 8, use_graph=False))
