@@ -44,10 +44,12 @@ def _fusable(*mods) -> bool:
     return True
 
 
-# cached tokens from which a long cache's decode step takes its many-split, matrix-core attention launch: measured on
-# the 1B architecture in a 32 K-row cache, us a token with 8 / 32 splits: 600 tokens 551 / 636, 2000: 578 / 637,
-# 5000: 636 / 636, 7000: 673 / 639, 31000: 1104 / 728
-LONG_CONTEXT_FROM = 5120
+# Cached tokens from which a grouped-query model's decode step takes the matrix-core attention launch with 16 splits, and
+# with 32. Measured on the 1B architecture in a 32 K-row cache, us a token by cached tokens, for 8 splits on the vector
+# ALU / 16 / 32 splits on the matrix core: 600: 551 / 599 / 636; 2000: 578 / 599 / 637; 3500: 595 / 600 / 639;
+# 5000: 636 / 620 / 638; 7000: 673 / 625 / 640; 15000: 791 / 671 / 671; 31000: 1104 / 755 / 729
+MID_CONTEXT_FROM = 4096
+LONG_CONTEXT_FROM = 16384
 
 
 class _Fused:
@@ -85,26 +87,29 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         super().__init__(model, max_len, kv_bits, exact_prefill)
         self._ext = load_extension()
         # A cache of many thousand rows is often mostly empty: the split count (and with it the kernel form) a step
-        # runs with follows the tokens the cache holds, in two regimes with a captured step each.
-        self.short_splits = None     # split count below `long_from` cached tokens; None: one regime
-        self.long_from = LONG_CONTEXT_FROM
+        # runs with follows the tokens the cache holds, through regimes [(from this many cached tokens, splits)] with
+        # a captured step each.
+        self.regimes = None          # None: one regime, attn_splits
         if attn_splits is None:
-            # one workgroup per CU at least, four more splits per 2048 tokens of cache up to 16; from
-            # ~12 K tokens on 32 splits, where the kernel takes the four query heads of a kv head
-            # together (grouped-query models) with the cache's codes as matrix-core operands
+            # one workgroup per CU at least; grouped-query models on caches beyond 4096 rows: 16 splits from 4096
+            # cached tokens and 32 from 16384, where the kernel takes the four query heads of a kv head together
+            # with the cache's codes as matrix-core operands; others: four more splits per 2048 rows of cache up to 16
             grouped = self.kv_heads > 0 and (self.q_heads // self.kv_heads) % 4 == 0
             short = max(1, 256 // max(self.q_heads, 1))
-            if max_len >= 12288 and grouped:
+            if grouped and short < 16 and max_len > MID_CONTEXT_FROM:
+                self.regimes = [(0, short), (MID_CONTEXT_FROM, 16)]
+                if max_len > LONG_CONTEXT_FROM:
+                    self.regimes.append((LONG_CONTEXT_FROM, 32))
+                attn_splits = self.regimes[-1][1]
+            elif grouped and max_len >= 12288:
                 attn_splits = 32
-                if short < attn_splits:
-                    self.short_splits = short
             else:
                 attn_splits = max(short, min(16, (max_len + 2047) // 2048 * 4))
         self.attn_splits = int(attn_splits)
         self._splits_now = self.attn_splits
         self._graphs = {}            # split count -> (graph, logits, next_token)
         self._partials = torch.zeros(self._ext.kv_attend_partials_floats(self.q_heads, self.head_dim,
-                                                                         self.attn_splits),
+                                                                         max([self.attn_splits] + [c for _, c in self.regimes or []])),
                                      dtype=torch.float32, device=self.device) if self.attn_splits > 1 else None
         self.fused_layers = []
         for layer in self.layers:
@@ -238,9 +243,13 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
 
     def _splits_for(self, cached_tokens: int) -> int:
         """Split count of the attention launch for a cache that holds this many tokens."""
-        if self.short_splits is not None and cached_tokens < self.long_from:
-            return self.short_splits
-        return self.attn_splits
+        if not self.regimes:
+            return self.attn_splits
+        splits = self.regimes[0][1]
+        for start, count in self.regimes:
+            if cached_tokens >= start:
+                splits = count
+        return splits
 
     def _set_step_inputs(self, token, position: int):
         super()._set_step_inputs(token, position)
@@ -273,7 +282,7 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         # the cache has grown (or been rewound) into the other regime: its captured step takes over, from the token
         # and position the previous step left on the device
         position = self.cache.get_seq_length()
-        if self.short_splits is not None and self._splits_for(position) != self._splits_now:
+        if self.regimes and self._splits_for(position) != self._splits_now:
             self.capture(self.token.clone(), position)
         return super().step()
 

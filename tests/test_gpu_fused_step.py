@@ -415,7 +415,7 @@ def test_prompt_pass_with_its_own_attention_and_two_launch_mlp():
 
 
 def test_decode_step_follows_the_tokens_the_cache_holds_through_two_regimes():
-    """A long cache that is mostly empty: below `long_from` cached tokens the step runs the attention launch with
+    """A long cache that is mostly empty: below a threshold of cached tokens the step runs the attention launch with
     the short cache's split count, from there on with the many-split form (here: the matrix-core kernel, the cache
     has 12288 rows), each regime with a captured step of its own. Graph replay and eager steps pick the same
     launches at the same positions, so their tokens are equal; a second generation reuses both captured steps."""
@@ -428,8 +428,8 @@ def test_decode_step_follows_the_tokens_the_cache_holds_through_two_regimes():
 
     def runtime():
         rt = LlamaFusedRuntime(kernel, 12288, 8)
-        assert rt.attn_splits == 32
-        rt.short_splits, rt.long_from = 8, 48   # (8 heads: the automatic choice has one regime; forced here)
+        assert rt.attn_splits == 32 and rt.regimes is None
+        rt.regimes = [(0, 8), (48, 32)]   # (8 heads: the automatic choice has one regime; forced here)
         return rt
 
     eager, graphed = runtime(), runtime()
@@ -451,3 +451,24 @@ def test_decode_step_follows_the_tokens_the_cache_holds_through_two_regimes():
     # a prompt that already lies in the long regime starts there
     long_ids = torch.randint(0, 4096, (1, 60), generator=torch.Generator().manual_seed(6)).cuda()
     assert torch.equal(graphed.generate(long_ids, 8, use_graph=True), eager.generate(long_ids, 8, use_graph=False))
+
+
+def test_regimes_the_fused_runtime_picks():
+    """32 query heads on 8 kv heads: caches up to 4096 rows have one regime (8 splits: a workgroup per CU); longer ones
+    go to 16 splits from 4096 cached tokens and, beyond 16384 rows, to 32 from 16384. An explicit split count is one
+    regime; a model without grouped heads keeps the split count that grows with the cache."""
+    from test_gpu_decode import build_model, quantized_pair
+
+    from llmquant.runtime import LlamaFusedRuntime
+
+    _, kernel = quantized_pair(build_model(2048, 1024, 1, 32, 8, 4096))
+    assert LlamaFusedRuntime(kernel, 2048, 8).regimes is None and LlamaFusedRuntime(kernel, 4096, 8).attn_splits == 8
+    mid = LlamaFusedRuntime(kernel, 8192, 8)
+    assert mid.regimes == [(0, 8), (4096, 16)] and mid.attn_splits == 16
+    assert [mid._splits_for(n) for n in (0, 4095, 4096, 8000)] == [8, 8, 16, 16]
+    long = LlamaFusedRuntime(kernel, 32768, 8)
+    assert long.regimes == [(0, 8), (4096, 16), (16384, 32)] and long.attn_splits == 32
+    assert [long._splits_for(n) for n in (100, 5000, 16383, 16384, 32000)] == [8, 16, 16, 32, 32]
+    assert LlamaFusedRuntime(kernel, 32768, 8, attn_splits=12).regimes is None
+    _, plain = quantized_pair(build_model(512, 1024, 1, 8, 8, 4096))
+    assert LlamaFusedRuntime(plain, 8192, 8).regimes is None and LlamaFusedRuntime(plain, 8192, 8).attn_splits == 32
