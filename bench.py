@@ -373,8 +373,8 @@ def other_kernels(torch):
         entry["GBps"] = round(nbytes / entry["split_us"] / 1e3, 1)
         out[f"kv_int{bits}_rope_append_attention_ctx2048_per_layer"] = entry
     # the same step on a long cache (32 000 tokens, int8; 10 layers = 350 MB, so that every launch reads HBM): one
-    # query head per workgroup on the vector ALU at its best split count against the form long caches take, four
-    # heads of a kv head per workgroup with the int8 codes as matrix-core operands
+    # query head per workgroup on the vector ALU (12 splits; from 16 on the entry point takes the other form) against
+    # the form long caches take, four heads of a kv head per workgroup with the int8 codes as matrix-core operands
     layers, kvh, qh, d, t_max, ctx = 10, 8, 32, 64, 32768, 32000
     kc = torch.randint(0, 100, (layers, kvh, t_max, d), device=dev).to(torch.int8)
     vc = torch.randint(0, 100, (layers, kvh, t_max, d), device=dev).to(torch.int8)
@@ -385,7 +385,7 @@ def other_kernels(torch):
     pos = torch.tensor([ctx], dtype=torch.int32, device=dev)
     nbytes = 2 * kvh * (ctx + 1) * d + 2 * kvh * (ctx + 1) * 4
     entry = {"bytes": nbytes}
-    for name, splits in (("one_head_per_workgroup_16_splits_us", 16), ("four_heads_matrix_core_32_splits_us", 32)):
+    for name, splits in (("one_head_per_workgroup_vector_alu_12_splits_us", 12), ("four_heads_matrix_core_32_splits_us", 32)):
         partials = torch.zeros(ext.kv_attend_partials_floats(qh, d, splits), device=dev)
 
         def long_step():
