@@ -837,7 +837,7 @@ constexpr int kMfHeads = 4;   // query heads of one kv head per workgroup
 constexpr int kMfSlab = 64;   // tokens of one wave step
 // caches shorter than this keep the vector-ALU form, whose K and V pass through the model's dtype as the reference's
 // cache holds them; the step is bound by latency there whichever form runs
-constexpr int kMfMinCache = 4096;
+constexpr int kMfMinCache = 2048;
 
 template <int BITS, int D> struct MfLds {
   static constexpr int kRowBytes = D * BITS / 8;                  // a token's codes: 32, 64 or 128 bytes
@@ -848,7 +848,7 @@ template <int BITS, int D> struct MfLds {
   static constexpr int kP = 16 * kMfSlab;                         // the weights as operand rows: [16 rows][64 tokens] bytes
   static constexpr int kWaveBytes = 2 * kStage + kP + 512;        // two stages, the weights, per-head constants
   static constexpr int kRec = D + 2;                              // a wave's (max, sum, output) per head
-  static constexpr int kHeaderFloats = kMfHeads * D + 2 * D + kSplitWaves * kMfHeads * kRec + kMfHeads;
+  static constexpr int kHeaderFloats = kMfHeads * D + 2 * D + kSplitWaves * kMfHeads * kRec + 2 * kMfHeads;
   static constexpr int kHeaderBytes = (kHeaderFloats * 4 + 255) / 256 * 256;
   static constexpr int kBytes = kHeaderBytes + kSplitWaves * kWaveBytes;   // int8: 82 KB (D = 64), 150 KB (D = 128)
   // Slot of a row's 16-byte piece p in LDS is p ^ swizzle(row); both depend on the row's bytes only. K is read as
@@ -883,6 +883,7 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
   float (*s_new)[D] = reinterpret_cast<float (*)[D]>(mf_smem + HEADS * D * 4);
   float* s_rec = reinterpret_cast<float*>(mf_smem + (HEADS + 2) * D * 4);   // [waves][HEADS][kRec]
   float* s_new_score = s_rec + kSplitWaves * HEADS * L::kRec;
+  float* s_qmax = s_new_score + HEADS;   // abs-max of each rotated, scaled query head
 
   const int qh0 = blockIdx.x * HEADS, split = blockIdx.y, n_splits = gridDim.y;
   const bool last_split = split == n_splits - 1;
@@ -936,6 +937,16 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
                                 kv_heads, t_max, pos, qh0, kvh, last_split, writer, lane, wv, s_q, s_new);
   // operand rows the weights never reach (two of a head's four) stay zero
   for (int i = lane; i < L::kP / 4; i += kWave) reinterpret_cast<uint32_t*>(pbuf)[i] = 0u;
+  {
+    // the head this wave has just rotated (one per wave): its abs-max, for the digits below
+    static_assert(HEADS == kSplitWaves, "a head per wave");
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    float a = 0.0f;
+#pragma unroll
+    for (int i = 0; i < D / kWave; ++i) a = fmaxf(a, fabsf(s_q[wv][lane + i * kWave]));
+    a = group_max<kWave>(a);
+    if (lane == 0) s_qmax[wv] = a;
+  }
   __syncthreads();
 
   // ---- the query heads as operand rows: lane (row = j = 4 head + digit, block g) holds d = 64 step + 16 g .. + 15
@@ -944,13 +955,15 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
   v4i32 q_bias = v4i32{0, 0, 0, 0};   // 4-bit: - 8 * (sum of the digits of rows 4 g .. 4 g + 3), the scores' C operand
   {
     const int h = j >> 2, digit = j & 3;
-    float amax = 0.0f;
-#pragma unroll
-    for (int d = 0; d < D; ++d) amax = fmaxf(amax, fabsf(s_q[h][d]));
+    const float amax = s_qmax[h];
     const uint32_t e = __builtin_bit_cast(uint32_t, amax) >> 23;   // amax = f 2^(e - 126), f in [0.5, 1)
     const bool usable = e >= 22u && e < 255u;                       // (below 2^-105 the head counts as zero)
     const float up = __builtin_bit_cast(float, (275u - e) << 23);  // 2^(148 - e): amax * up in [2^21, 2^22)
     const float down = __builtin_bit_cast(float, (e - 21u) << 23); // 2^(e - 148)
+    // digit k of q = d0 + 256 d1 + 65536 d2 (each in [-128, 127]) is the sign-extended low byte of
+    // (q + 128 + ... + 128 * 256^(k-1)) >> 8 k; the fourth row of a head is empty
+    const int digit_add = digit == 1 ? 128 : digit == 2 ? 32896 : 0;
+    const int digit_shift = 8 * (digit & 3);
     int digit_sum = 0;
 #pragma unroll
     for (int ks = 0; ks < kKSteps; ++ks) {
@@ -958,12 +971,8 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
 #pragma unroll
       for (int b = 0; b < 16; ++b) {
         const int d_in_block = BITS == 8 ? b : (b < 8 ? 2 * b : 2 * (b - 8) + 1);
-        const int qi = usable ? static_cast<int>(rintf(s_q[h][64 * ks + 16 * g + d_in_block] * up)) : 0;
-        const int d0 = static_cast<int8_t>(qi);
-        const int r1 = (qi - d0) >> 8;
-        const int d1 = static_cast<int8_t>(r1);
-        const int d2 = (r1 - d1) >> 8;
-        const int digit_value = digit == 0 ? d0 : digit == 1 ? d1 : digit == 2 ? d2 : 0;
+        const int qi = static_cast<int>(rintf(s_q[h][64 * ks + 16 * g + d_in_block] * up));
+        const int digit_value = usable && digit < 3 ? static_cast<int>(static_cast<int8_t>((qi + digit_add) >> digit_shift)) : 0;
         words[b >> 2] |= static_cast<uint32_t>(digit_value & 0xff) << (8 * (b & 3));
         digit_sum += digit_value;
       }
@@ -1688,7 +1697,7 @@ extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos
   const float scale_log2 = sm_scale * 1.4426950408889634f;
   hipStream_t s = static_cast<hipStream_t>(stream);
   // Four query heads of a kv head per workgroup once the caller asks for 32 splits or more (or for 16 on a cache of
-  // 4096 rows or more, which then takes the matrix-core form below): measured on the vector ALU at 32 splits, ctx
+  // 2048 rows or more, which then takes the matrix-core form below): measured on the vector ALU at 32 splits, ctx
   // 8 K / 16 K / 32 K: 9.7 / 13.6 / 20.9 us per layer against 13.0 / 19.7 / 32.0 us for one head per workgroup at
   // its best split count; below that the one-head form, which puts more workgroups on the chip, is as fast or faster.
   const int rep_heads = q_heads / kv_heads;

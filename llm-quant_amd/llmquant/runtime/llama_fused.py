@@ -46,9 +46,9 @@ def _fusable(*mods) -> bool:
 
 # Cached tokens from which a grouped-query model's decode step takes the matrix-core attention launch with 16 splits, and
 # with 32. Measured on the 1B architecture in a 32 K-row cache, us a token by cached tokens, for 8 splits on the vector
-# ALU / 16 / 32 splits on the matrix core: 600: 551 / 599 / 636; 2000: 578 / 599 / 637; 3500: 595 / 600 / 639;
-# 5000: 636 / 620 / 638; 7000: 673 / 625 / 640; 15000: 791 / 671 / 671; 31000: 1104 / 755 / 729
-MID_CONTEXT_FROM = 4096
+# ALU / 16 / 32 splits on the matrix core: 600: 551 / 576 / 615; 2000: 578 / 576 / 615; 3500: 595 / 577 / 616;
+# 7000: 673 / 601 / 616; 15000: 791 / 646 / 644; 31000: 1104 / 732 / 706
+MID_CONTEXT_FROM = 2048
 LONG_CONTEXT_FROM = 16384
 
 
@@ -91,7 +91,7 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         # a captured step each.
         self.regimes = None          # None: one regime, attn_splits
         if attn_splits is None:
-            # one workgroup per CU at least; grouped-query models on caches beyond 4096 rows: 16 splits from 4096
+            # one workgroup per CU at least; grouped-query models on caches beyond 2048 rows: 16 splits from 2048
             # cached tokens and 32 from 16384, where the kernel takes the four query heads of a kv head together
             # with the cache's codes as matrix-core operands; others: four more splits per 2048 rows of cache up to 16
             grouped = self.kv_heads > 0 and (self.q_heads // self.kv_heads) % 4 == 0
