@@ -367,8 +367,16 @@ def other_kernels(torch):
         nbytes = 2 * kvh * (ctx + 1) * width + 2 * kvh * (ctx + 1) * 4
         entry = {"bytes": nbytes, "splits": splits, "layers_of_cache_walked": layers,
                  "cache_bytes_touched_per_replay": nbytes * layers}
+        partials16 = torch.zeros(ext.kv_attend_partials_floats(qh, d, 16), device=dev)
+
+        def matrix_core_16_splits():  # the form the runtime's step takes from 2048 cached tokens on (four heads a workgroup)
+            for layer in range(layers):
+                ext.kv_rope_append_attend_split(qkv, table, table, kc[layer], vc[layer], ks[layer], vs[layer],
+                                                partials16, pos, d ** -0.5, qh, 16)
+
         for name, fn in (("one_workgroup_per_head_us", one_workgroup_per_head), ("split_us", split_only),
-                         ("split_plus_merge_kernel_us", split_and_merge)):
+                         ("split_plus_merge_kernel_us", split_and_merge),
+                         ("matrix_core_16_splits_us", matrix_core_16_splits)):
             entry[name] = round(_graph_time_us(torch, fn, reps=5) / layers, 2)
         entry["GBps"] = round(nbytes / entry["split_us"] / 1e3, 1)
         out[f"kv_int{bits}_rope_append_attention_ctx2048_per_layer"] = entry
