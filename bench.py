@@ -367,21 +367,23 @@ def other_kernels(torch):
         nbytes = 2 * kvh * (ctx + 1) * width + 2 * kvh * (ctx + 1) * 4
         entry = {"bytes": nbytes, "splits": splits, "layers_of_cache_walked": layers,
                  "cache_bytes_touched_per_replay": nbytes * layers}
-        partials16 = torch.zeros(ext.kv_attend_partials_floats(qh, d, 16), device=dev)
+        partials7 = torch.zeros(ext.kv_attend_partials_floats(qh, d, 7), device=dev)
 
-        def matrix_core_16_splits():  # the form the runtime's step takes from 2048 cached tokens on (four heads a workgroup)
+        def vector_alu_7_splits():  # (below 8 splits the entry point keeps one head a workgroup on the vector ALU)
             for layer in range(layers):
                 ext.kv_rope_append_attend_split(qkv, table, table, kc[layer], vc[layer], ks[layer], vs[layer],
-                                                partials16, pos, d ** -0.5, qh, 16)
+                                                partials7, pos, d ** -0.5, qh, 7)
 
+        # split_us: what the runtime's step runs on a cache of this size, 8 splits, four heads of a kv head a workgroup
+        # with the cache's codes as matrix-core operands
         for name, fn in (("one_workgroup_per_head_us", one_workgroup_per_head), ("split_us", split_only),
                          ("split_plus_merge_kernel_us", split_and_merge),
-                         ("matrix_core_16_splits_us", matrix_core_16_splits)):
+                         ("vector_alu_7_splits_us", vector_alu_7_splits)):
             entry[name] = round(_graph_time_us(torch, fn, reps=5) / layers, 2)
         entry["GBps"] = round(nbytes / entry["split_us"] / 1e3, 1)
         out[f"kv_int{bits}_rope_append_attention_ctx2048_per_layer"] = entry
     # the same step on a long cache (32 000 tokens, int8; 10 layers = 350 MB, so that every launch reads HBM): one
-    # query head per workgroup on the vector ALU (12 splits; from 16 on the entry point takes the other form) against
+    # query head per workgroup on the vector ALU (7 splits; from 8 on the entry point takes the other form) against
     # the form long caches take, four heads of a kv head per workgroup with the int8 codes as matrix-core operands
     layers, kvh, qh, d, t_max, ctx = 10, 8, 32, 64, 32768, 32000
     kc = torch.randint(0, 100, (layers, kvh, t_max, d), device=dev).to(torch.int8)
@@ -393,7 +395,7 @@ def other_kernels(torch):
     pos = torch.tensor([ctx], dtype=torch.int32, device=dev)
     nbytes = 2 * kvh * (ctx + 1) * d + 2 * kvh * (ctx + 1) * 4
     entry = {"bytes": nbytes}
-    for name, splits in (("one_head_per_workgroup_vector_alu_12_splits_us", 12), ("four_heads_matrix_core_32_splits_us", 32)):
+    for name, splits in (("one_head_per_workgroup_vector_alu_7_splits_us", 7), ("four_heads_matrix_core_32_splits_us", 32)):
         partials = torch.zeros(ext.kv_attend_partials_floats(qh, d, splits), device=dev)
 
         def long_step():

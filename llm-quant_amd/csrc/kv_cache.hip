@@ -1696,12 +1696,12 @@ extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos
     return llmq_host::fail_invalid("cache code and record pointers must be 16-byte aligned");
   const float scale_log2 = sm_scale * 1.4426950408889634f;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // Four query heads of a kv head per workgroup once the caller asks for 32 splits or more (or for 16 on a cache of
+  // Four query heads of a kv head per workgroup once the caller asks for 32 splits or more (or for 8 on a cache of
   // 2048 rows or more, which then takes the matrix-core form below): measured on the vector ALU at 32 splits, ctx
   // 8 K / 16 K / 32 K: 9.7 / 13.6 / 20.9 us per layer against 13.0 / 19.7 / 32.0 us for one head per workgroup at
   // its best split count; below that the one-head form, which puts more workgroups on the chip, is as fast or faster.
   const int rep_heads = q_heads / kv_heads;
-  const bool grouped = rep_heads % 4 == 0 && (n_splits >= 32 || (n_splits >= 16 && t_max >= kMfMinCache));
+  const bool grouped = rep_heads % 4 == 0 && (n_splits >= 32 || (n_splits >= 8 && t_max >= kMfMinCache));
   const dim3 grid(grouped ? q_heads / 4 : q_heads, n_splits), block(kSplitThreads);
   if (grouped && t_max >= kMfMinCache) {
     // long caches: the matrix-core form (see the kernel's comment for what it changes in the arithmetic)

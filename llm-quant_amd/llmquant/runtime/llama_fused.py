@@ -44,11 +44,13 @@ def _fusable(*mods) -> bool:
     return True
 
 
-# Cached tokens from which a grouped-query model's decode step takes the matrix-core attention launch with 16 splits, and
-# with 32. Measured on the 1B architecture in a 32 K-row cache, us a token by cached tokens, for 8 splits on the vector
-# ALU / 16 / 32 splits on the matrix core: 600: 551 / 576 / 615; 2000: 578 / 576 / 615; 3500: 595 / 577 / 616;
-# 7000: 673 / 601 / 616; 15000: 791 / 646 / 644; 31000: 1104 / 732 / 706
-MID_CONTEXT_FROM = 2048
+# Cached tokens from which a grouped-query model's decode step runs its attention launch with 16 splits, and with 32 (a
+# cache of 2048 rows or more takes the matrix-core form of the launch from 8 splits on). Measured on the 1B architecture
+# in a 32 K-row cache, us a token by cached tokens, for 8 / 16 / 32 splits: 600: 560 / 576 / 615; 1000: 551 / - / -;
+# 2000: 562 / 576 / 615; 3500: 574 / 577 / 616; 7000: - / 601 / 616; 15000: - / 646 / 644; 31000: - / 732 / 706
+# (the vector-ALU form, which caches below 2048 rows keep, with 8 splits: 546-551 / 555 / 578 / 595 at 600 / 1000 / 2000 /
+# 3500, 673 at 7000)
+MID_CONTEXT_FROM = 5120
 LONG_CONTEXT_FROM = 16384
 
 
@@ -91,9 +93,9 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         # a captured step each.
         self.regimes = None          # None: one regime, attn_splits
         if attn_splits is None:
-            # one workgroup per CU at least; grouped-query models on caches beyond 2048 rows: 16 splits from 2048
-            # cached tokens and 32 from 16384, where the kernel takes the four query heads of a kv head together
-            # with the cache's codes as matrix-core operands; others: four more splits per 2048 rows of cache up to 16
+            # one workgroup per CU at least; grouped-query models on long caches: 16 splits from 5120 cached tokens and
+            # 32 from 16384 (the kernel takes the four query heads of a kv head together with the cache's codes as
+            # matrix-core operands); others: four more splits per 2048 rows of cache up to 16
             grouped = self.kv_heads > 0 and (self.q_heads // self.kv_heads) % 4 == 0
             short = max(1, 256 // max(self.q_heads, 1))
             if grouped and short < 16 and max_len > MID_CONTEXT_FROM:
@@ -101,6 +103,8 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
                 if max_len > LONG_CONTEXT_FROM:
                     self.regimes.append((LONG_CONTEXT_FROM, 32))
                 attn_splits = self.regimes[-1][1]
+            elif grouped and short < 16:
+                attn_splits = short
             elif grouped and max_len >= 12288:
                 attn_splits = 32
             else:

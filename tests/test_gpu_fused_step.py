@@ -454,21 +454,21 @@ def test_decode_step_follows_the_tokens_the_cache_holds_through_two_regimes():
 
 
 def test_regimes_the_fused_runtime_picks():
-    """32 query heads on 8 kv heads: caches up to 2048 rows have one regime (8 splits: a workgroup per CU); longer ones
-    go to 16 splits from 2048 cached tokens and, beyond 16384 rows, to 32 from 16384. An explicit split count is one
-    regime; a model without grouped heads keeps the split count that grows with the cache."""
+    """32 query heads on 8 kv heads: caches up to 5120 rows have one regime (8 splits); longer ones go to 16 splits from
+    5120 cached tokens and, beyond 16384 rows, to 32 from 16384. An explicit split count is one regime; a model
+    without grouped heads keeps the split count that grows with the cache."""
     from test_gpu_decode import build_model, quantized_pair
 
     from llmquant.runtime import LlamaFusedRuntime
 
     _, kernel = quantized_pair(build_model(2048, 1024, 1, 32, 8, 4096))
-    assert LlamaFusedRuntime(kernel, 769, 8).regimes is None and LlamaFusedRuntime(kernel, 2048, 8).attn_splits == 8
+    assert LlamaFusedRuntime(kernel, 769, 8).regimes is None and LlamaFusedRuntime(kernel, 4096, 8).attn_splits == 8
     mid = LlamaFusedRuntime(kernel, 8192, 8)
-    assert mid.regimes == [(0, 8), (2048, 16)] and mid.attn_splits == 16
-    assert [mid._splits_for(n) for n in (0, 2047, 2048, 8000)] == [8, 8, 16, 16]
+    assert mid.regimes == [(0, 8), (5120, 16)] and mid.attn_splits == 16
+    assert [mid._splits_for(n) for n in (0, 5119, 5120, 8000)] == [8, 8, 16, 16]
     long = LlamaFusedRuntime(kernel, 32768, 8)
-    assert long.regimes == [(0, 8), (2048, 16), (16384, 32)] and long.attn_splits == 32
-    assert [long._splits_for(n) for n in (100, 5000, 16383, 16384, 32000)] == [8, 16, 16, 32, 32]
+    assert long.regimes == [(0, 8), (5120, 16), (16384, 32)] and long.attn_splits == 32
+    assert [long._splits_for(n) for n in (100, 6000, 16383, 16384, 32000)] == [8, 16, 16, 32, 32]
     assert LlamaFusedRuntime(kernel, 32768, 8, attn_splits=12).regimes is None
     _, plain = quantized_pair(build_model(512, 1024, 1, 8, 8, 4096))
     assert LlamaFusedRuntime(plain, 8192, 8).regimes is None and LlamaFusedRuntime(plain, 8192, 8).attn_splits == 32
