@@ -86,7 +86,7 @@ def test_graph_replay_equals_eager_bit_for_bit(small):
     assert seq_a.shape == (1, 64) and torch.equal(seq_a, seq_b)
 
 
-def teacher_forced(real, kernel, prompt, new_tokens, vocab, runtime="walk"):
+def teacher_forced(real, kernel, prompt, new_tokens, vocab, runtime="walk", max_len=None):
     """Both models fed the oracle's own greedy stream. Rows: (same argmax, oracle top-2 gap, max logit
     error, relative logit error); also the oracle's stream (its free-running greedy tokens) and the prompt.
     runtime: "walk" = the operation-by-operation LlamaKernelRuntime, "fused" = LlamaFusedRuntime, the
@@ -99,7 +99,7 @@ def teacher_forced(real, kernel, prompt, new_tokens, vocab, runtime="walk"):
     with torch.no_grad():
         want = real(ids, past_key_values=cache, use_cache=True).logits[0, -1]
     cls = LlamaFusedRuntime if runtime == "fused" else LlamaKernelRuntime
-    rt = cls(kernel, prompt + new_tokens + 2, 8)
+    rt = cls(kernel, max_len or prompt + new_tokens + 2, 8)
     first = rt.prefill(ids)
     rows = [(first.item() == want.argmax().item(), 0.0, 0.0, 0.0)]
     tok = want.argmax().reshape(1)
@@ -144,6 +144,59 @@ def test_teacher_forced_margin_with_heads_of_128(runtime):
     agree = check_margin(rows, 0.05)
     print(f"teacher-forced agreement, heads of 128, {runtime}: {agree}/{len(rows)}")
     assert agree >= 0.8 * len(rows)
+
+
+@pytest.mark.parametrize("head_dim,kv_bits", [(64, 8), (128, 8), (64, 4)])
+def test_teacher_forced_margin_on_a_long_cache(head_dim, kv_bits):
+    """A cache of 2304 rows: the fused runtime's decode step takes the matrix-core form of the attention launch (the
+    cache's codes as int8 operands, four query heads of a kv head a workgroup). The whole step against the real-mode
+    model under the same margin rule as the short caches, for both head sizes and for an int4 cache."""
+    from llmquant import QuantConfig, oneshot
+    from llmquant.hip.build import load_extension
+
+    model = build_model(512, 1024, 2, 512 // head_dim, 512 // head_dim // 4, 4096, seed=5, head_dim=head_dim)
+    # (the recipe names the weights; the cache width is the runtime's and the reference cache's argument)
+    recipe = QuantConfig(attn_weight="int8", mlp_weight="int4", head_weight="int8", kv_cache="int8")
+    real = oneshot(copy.deepcopy(model), recipe.to_modifier("real"))
+    kernel = oneshot(copy.deepcopy(model), recipe.to_modifier("kernel"))
+    calls = []
+    ext = load_extension()
+    split = ext.kv_rope_append_attend_split
+    try:
+        ext.kv_rope_append_attend_split = lambda *a: (calls.append((a[3].shape[1], a[11])), split(*a))[1]
+        rows, _, _ = teacher_forced_bits(real, kernel, 200, 24, 4096, kv_bits, max_len=2304)
+    finally:
+        ext.kv_rope_append_attend_split = split
+    # (the launches ran on the 2304-row cache with the split count whose form is the matrix core's)
+    assert calls and all(rows_of_cache == 2304 and splits >= 8 for rows_of_cache, splits in calls)
+    agree = check_margin(rows, 0.05)
+    print(f"teacher-forced agreement, cache of 2304 rows, heads of {head_dim}, int{kv_bits} cache: {agree}/{len(rows)}")
+    assert agree >= 0.8 * len(rows)
+
+
+def teacher_forced_bits(real, kernel, prompt, new_tokens, vocab, kv_bits, max_len):
+    """teacher_forced for the fused runtime with a cache of `kv_bits` on both sides."""
+    from llmquant.quantizers import make_cache_factory
+    from llmquant.runtime import LlamaFusedRuntime
+
+    ids = torch.randint(0, vocab, (1, prompt), generator=torch.Generator().manual_seed(1)).cuda()
+    cache = make_cache_factory(kv_bits)()
+    with torch.no_grad():
+        want = real(ids, past_key_values=cache, use_cache=True).logits[0, -1]
+    rt = LlamaFusedRuntime(kernel, max_len, kv_bits)
+    first = rt.prefill(ids)
+    rows = [(first.item() == want.argmax().item(), 0.0, 0.0, 0.0)]
+    tok = want.argmax().reshape(1)
+    for i in range(new_tokens):
+        with torch.no_grad():
+            want = real(tok.reshape(1, 1), past_key_values=cache, use_cache=True).logits[0, -1].float()
+        logits, nxt = rt.eager_step(tok, prompt + i)
+        got = logits[0].float()
+        top2 = want.topk(2).values
+        rows.append((nxt.item() == want.argmax().item(), (top2[0] - top2[1]).item(),
+                     (got - want).abs().max().item(), ((got - want).norm() / want.norm()).item()))
+        tok = want.argmax().reshape(1)
+    return rows, None, ids
 
 
 def identical_prefix(a, b) -> int:
