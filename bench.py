@@ -408,6 +408,27 @@ def other_kernels(torch):
     entry["frac_hbm"] = round(entry["GBps"] / HBM_PEAK_GBPS, 4)
     out["kv_int8_rope_append_attention_ctx32000_per_layer"] = entry
     del kc, vc, ks, vs
+    # 131 000 tokens (3 layers = 430 MB): the cache's bytes are most of the launch
+    layers, t_long, ctx_long = 3, 131072, 131000
+    kc = torch.randint(0, 100, (layers, kvh, t_long, d), device=dev).to(torch.int8)
+    vc = torch.randint(0, 100, (layers, kvh, t_long, d), device=dev).to(torch.int8)
+    ks = torch.rand(layers, kvh, t_long, device=dev) * 0.05
+    vs = torch.rand(layers, kvh, t_long, device=dev) * 0.05
+    table_long = torch.randn(t_long, d, device=dev).to(torch.bfloat16)
+    pos_long = torch.tensor([ctx_long], dtype=torch.int32, device=dev)
+    partials = torch.zeros(ext.kv_attend_partials_floats(qh, d, 64), device=dev)
+
+    def longest_step():
+        for layer in range(layers):
+            ext.kv_rope_append_attend_split(qkv, table_long, table_long, kc[layer], vc[layer], ks[layer], vs[layer],
+                                            partials, pos_long, d ** -0.5, qh, 64)
+
+    nbytes = 2 * kvh * (ctx_long + 1) * d + 2 * kvh * (ctx_long + 1) * 4
+    us = round(_graph_time_us(torch, longest_step, reps=20) / layers, 2)
+    out["kv_int8_rope_append_attention_ctx131000_per_layer"] = {
+        "bytes": nbytes, "four_heads_matrix_core_64_splits_us": us, "GBps": round(nbytes / us / 1e3, 1),
+        "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    del kc, vc, ks, vs, table_long
     # and for heads of 128 (the Llama-3-8B geometry), 5 layers = 350 MB
     layers, d = 5, 128
     kc = torch.randint(0, 100, (layers, kvh, t_max, d), device=dev).to(torch.int8)
