@@ -802,7 +802,7 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
   }
 }
 
-// ---- the same step for long caches under grouped-query attention, on the int8 matrix core ---------------------
+// ---- the same step under grouped-query attention on the int8 matrix core (caches of 2048 rows and more) --------
 // Beyond a few thousand tokens the step above is bound by the vector ALU: every code is converted to a float and
 // multiplied there (~500 instructions per 16 tokens and four heads, 2.6 TB/s of cache bytes at best). Here the int8
 // codes are matrix-core operands as they lie in the cache (v_mfma_i32_16x16x64_i8), for the four query heads of a
@@ -823,9 +823,10 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
 // rounding to the model's dtype in between, and the 2^-14 resolution of the weights: within the tolerance the
 // attention output is held to (checked against the float64 oracle like the other kernels).
 // A wave walks 64-token slabs (wave w of split s: slabs 4 s + w, 4 s + w + 4 S, ...) through two LDS stages of its
-// own, filled by DMA (codes of K and V with their 16-byte pieces XOR-swizzled by row so that the operand reads and
-// the transposed reads meet no bank conflict, and the two scale vectors): no barrier inside the loop. The records
-// it leaves are those of the kernel above.
+// own, filled by DMA (codes of K and V with their 16-byte pieces XOR-swizzled by row for the operand reads and the
+// transposed reads, and the two scale vectors): no barrier inside the loop. The records it leaves are those of the
+// kernel above. Measured, 32 heads on 8 kv heads of 64, int8, per layer: 5.7 us at 2048 cached tokens (8 splits; the
+// step above 6.6), 12 us at 32 000 (32 splits; 20.7), 33 us at 131 000 (64 splits; 55).
 // 4-bit codes: a lane's eight packed bytes (16 codes) become two operand halves, the low nibbles (even dimensions) and
 // the high ones (odd), with the query's digits laid out in the same order; V's packed bytes go through the same
 // transposed read and split into the operand of an even and of an odd dimension. The nibbles are code + 8: the 8
