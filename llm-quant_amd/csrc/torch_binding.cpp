@@ -221,6 +221,7 @@ struct DensePlan {
   hipblasLtMatmulDesc_t desc = nullptr;
   hipblasLtMatrixLayout_t w = nullptr, x = nullptr, out = nullptr;
   hipblasLtMatmulAlgo_t algo;
+  bool usable = true;   // false: the heuristic had nothing for this shape within the workspace; torch's matmul takes it
 };
 struct DenseState {
   hipblasLtHandle_t handle = nullptr;
@@ -279,8 +280,11 @@ const DensePlan& dense_plan(DenseState& st, bool bf16, int64_t M, int64_t N, int
   for (int i = 0; i < n_results && pick < 0; ++i) {
     if (results[i].state == HIPBLAS_STATUS_SUCCESS && results[i].workspaceSize <= cap) pick = i;
   }
-  TORCH_CHECK(pick >= 0, "hipBLASLt offers no algorithm for a ", M, " x ", N, " x ", K, " matmul");
-  p.algo = results[pick].algo;
+  if (pick >= 0) {
+    p.algo = results[pick].algo;
+  } else {
+    p.usable = false;   // (seen for 31000 x 16384 x 2048: remembered, so that the heuristic is not asked again per call)
+  }
   return st.plans.emplace(key, p).first->second;
 }
 
@@ -309,6 +313,7 @@ at::Tensor dense_linear(const at::Tensor& x, const at::Tensor& w) {
   at::Tensor& workspace = st.workspaces[static_cast<void*>(stream.stream())];
   if (!workspace.defined()) workspace = at::empty({kDenseWorkspaceBytes}, x.options().dtype(at::kByte));
   const DensePlan& plan = dense_plan(st, x.scalar_type() == at::kBFloat16, M, N, K);
+  if (!plan.usable) return at::mm(x, w.t());
   const float one = 1.0f, zero = 0.0f;
   check_lt(hipblasLtMatmul(st.handle, plan.desc, &one, w.const_data_ptr(), plan.w, x.const_data_ptr(), plan.x, &zero,
                            out.const_data_ptr(), plan.out, out.mutable_data_ptr(), plan.out, &plan.algo,

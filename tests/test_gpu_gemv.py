@@ -566,6 +566,24 @@ def test_dense_linear_is_the_library_matmul_with_a_kept_plan(dtype):
         ext.dense_linear(x.cpu(), w)
 
 
+def test_dense_linear_takes_a_shape_the_library_has_no_plan_for():
+    """31000 x 16384 x 2048 (the gate|up projection of a 31000-token prompt on the 1B architecture): the library's
+    heuristic offers no algorithm within the workspace, and the call goes to torch's matmul instead of failing; the
+    second call does not ask the heuristic again and gives the same bits."""
+    from llmquant.hip import load_extension
+
+    ext = load_extension()
+    gen = torch.Generator(device="cuda").manual_seed(22)
+    x = torch.randn(31000, 2048, generator=gen, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(16384, 2048, generator=gen, device="cuda") * 0.05).to(torch.bfloat16)
+    first = ext.dense_linear(x, w)
+    assert first.shape == (31000, 16384)
+    rows = torch.tensor([0, 1, 77, 15499, 30999], device="cuda")
+    want = (x[rows].double() @ w.double().T).cpu().numpy()
+    assert rel_l2(to_np(first[rows]), want) <= 1e-2
+    assert torch.equal(ext.dense_linear(x, w), first)
+
+
 @pytest.mark.parametrize("bits", [8, 4])
 def test_wq_dense_linear_is_dequantize_then_matmul(bits):
     """One call for the dense branch: the dequantized matrix (bit-exact, tested above) times x, whole
