@@ -813,17 +813,18 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
 //            digits, one operand row each (the GEMV's trick); a lane ends up with the three digit sums of one
 //            (token, head) and combines them: score = (S0 + 256 S1 + 65536 S2) * 2^-sh * kscale[token].
 //   values   O[(head, digit)][d] = sum_t W[(head, digit)][t] * Vcode[t][d] with W = p * vscale[t], p the softmax
-//            weight relative to the running maximum, as a 14-bit integer below the largest W of the head in the
-//            64-token step, in two digits. The weights reach operand layout (tokens along a lane's 16 bytes)
+//            weight relative to the running maximum, as an integer below the largest W of the head in the 64-token
+//            step: 14 bits in two digits (fp32 models: 22 in three). The weights reach operand layout (tokens along a lane's 16 bytes)
 //            through 1 KB of LDS per wave; V's codes, token-major in the cache, are read from LDS transposed
 //            (ds_read_b64_tr_b8: in a group of 16 lanes, byte j of result lane l is byte l % 8 of what lane
 //            2 j + l / 8 points at).
 //
 // Both sums are exact integers; what differs from the step above is that K and V enter as code * scale without the
-// rounding to the model's dtype in between, and the 2^-14 resolution of the weights: within the tolerance the
-// attention output is held to (checked against the float64 oracle like the other kernels).
+// rounding to the model's dtype in between, and the resolution of the weights (2^-14 beside a 16-bit output's 2^-8 or
+// 2^-11; 2^-22, fp32's own, for fp32 models): within the tolerance the attention output is held to, and for fp32
+// models at fp32's rounding level (rel-L2 1e-6 against the float64 oracle).
 // A wave walks 64-token slabs (wave w of split s: slabs 4 s + w, 4 s + w + 4 S, ...) through two LDS stages of its
-// own, filled by DMA (codes of K and V with their 16-byte pieces XOR-swizzled by row for the operand reads and the
+// own, both in flight while it computes, filled by DMA (codes of K and V with their 16-byte pieces XOR-swizzled by row for the operand reads and the
 // transposed reads, and the two scale vectors): no barrier inside the loop. The records it leaves are those of the
 // kernel above. Measured, 32 heads on 8 kv heads of 64, int8, per layer: 5.7 us at 2048 cached tokens (8 splits; the
 // step above 6.6), 12 us at 32 000 (32 splits; 20.7), 33 us at 131 000 (64 splits; 55).
@@ -878,6 +879,7 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
   constexpr uint32_t kNibbles = 0x0f0f0f0fu;
   constexpr int GREC = D + kAttnRecordHeader;
   constexpr int kKSteps = D / 64;    // matrix-core steps along a head's dimensions
+  constexpr int kWDigits = sizeof(T) == 4 ? 3 : 2;   // base-256 digits of the softmax weights (see the loop)
   constexpr int kDTiles = D / 16;    // tiles of 16 dimensions of the output
   extern __shared__ __attribute__((aligned(16))) unsigned char mf_smem[];
   float (*s_q)[D] = reinterpret_cast<float (*)[D]>(mf_smem);
@@ -934,9 +936,11 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
   const int pos = min(max(pos_dev[0], 0), t_max - 1);
   const T* cos_row = cos_table + static_cast<int64_t>(pos) * D;
   const T* sin_row = sin_table + static_cast<int64_t>(pos) * D;
+  // two slabs in flight per wave from here on: the second goes out as soon as the position says it exists
+  if (t0 + t_step < pos) request(t0 + t_step, 1);
   split_phase_a<T, BITS, D, HEADS>(qkv, cos_row, sin_row, k_codes, v_codes, k_scale, v_scale, sm_scale_log2, q_heads,
                                 kv_heads, t_max, pos, qh0, kvh, last_split, writer, lane, wv, s_q, s_new);
-  // operand rows the weights never reach (two of a head's four) stay zero
+  // operand rows the weights never reach (one or two of a head's four) stay zero
   for (int i = lane; i < L::kP / 4; i += kWave) reinterpret_cast<uint32_t*>(pbuf)[i] = 0u;
   {
     // the head this wave has just rotated (one per wave): its abs-max, for the digits below
@@ -1001,8 +1005,8 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
   for (int dt = 0; dt < kDTiles; ++dt) o_acc[dt] = 0.0f;
   int stage = 0;
   for (; t0 < pos; t0 += t_step, stage ^= 1) {
+    // this slab is in `stage`; the next one, if there is one, has been requested into the other stage
     if (t0 + t_step < pos) {
-      request(t0 + t_step, stage ^ 1);
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kRequestLoads) : "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -1047,24 +1051,34 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
     }
     l_part = fmaf(l_part, alpha, p_sum);
     m_run = m_new;
-    // ---- the weights as 14-bit integers below the head's largest in this slab, two digits
+    // ---- the weights as integers below the head's largest in this slab: 14 bits in two digits for 16-bit models (whose
+    // output keeps 8 or 11 bits), 22 bits in three digits, like the query's, for fp32 ones
+    constexpr uint32_t kWBits = kWDigits == 3 ? 22u : 14u;
     w_max = group_max<16>(w_max);
-    const uint32_t we = max(__builtin_bit_cast(uint32_t, w_max) >> 23, 13u);   // w_max = f 2^(we - 126)
-    const float w_up = __builtin_bit_cast(float, (267u - we) << 23);            // 2^(140 - we): w * w_up < 2^14
-    const float w_down = __builtin_bit_cast(float, (we - 13u) << 23);           // 2^(we - 140)
-    int w_sum0 = 0, w_sum1 = 0;
+    const uint32_t we = max(__builtin_bit_cast(uint32_t, w_max) >> 23, kWBits - 1u);   // w_max = f 2^(we - 126)
+    const float w_up = __builtin_bit_cast(float, (253u + kWBits - we) << 23);   // 2^(126 + bits - we): w * w_up < 2^bits
+    const float w_down = __builtin_bit_cast(float, (we + 1u - kWBits) << 23);   // 2^(we - 126 - bits)
+    int w_sum0 = 0, w_sum1 = 0, w_sum2 = 0;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int wi = static_cast<int>(rintf(w[c] * w_up));
       const int d0 = static_cast<int8_t>(wi);
-      const int d1 = (wi - d0) >> 8;
+      const int r1 = (wi + 128) >> 8;   // (wi - d0) / 256
+      const int d1 = kWDigits == 3 ? static_cast<int>(static_cast<int8_t>(r1)) : r1;
       pbuf[(4 * g) * kMfSlab + 16 * c + j] = static_cast<unsigned char>(d0);
       pbuf[(4 * g + 1) * kMfSlab + 16 * c + j] = static_cast<unsigned char>(d1);
       w_sum0 += d0;
       w_sum1 += d1;
+      if constexpr (kWDigits == 3) {
+        const int d2 = (wi + 32896) >> 16;
+        pbuf[(4 * g + 2) * kMfSlab + 16 * c + j] = static_cast<unsigned char>(d2);
+        w_sum2 += d2;
+      }
     }
     v4i32 w_bias = v4i32{0, 0, 0, 0};   // 4-bit: - 8 * (sum over the slab of the head's digits), the values' C operand
-    if constexpr (BITS == 4) w_bias = v4i32{-8 * row16_sum(w_sum0), -8 * row16_sum(w_sum1), 0, 0};
+    if constexpr (BITS == 4) {
+      w_bias = v4i32{-8 * row16_sum(w_sum0), -8 * row16_sum(w_sum1), kWDigits == 3 ? -8 * row16_sum(w_sum2) : 0, 0};
+    }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     const v4i32 pa = *reinterpret_cast<const v4i32*>(pbuf + j * kMfSlab + 16 * g);   // row j, tokens 16 g .. 16 g + 15
     // ---- weighted values, 16 of the head's dimensions per tile: lane = (head g, d = 16 tile + j; 4-bit: tiles come
@@ -1080,20 +1094,26 @@ __global__ __launch_bounds__(kSplitThreads, 2) void kv_rope_append_attend_split_
       const v4i32 vb = v4i32{lo[0], lo[1], hi[0], hi[1]};
       if constexpr (BITS == 8) {
         const v4i32 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(pa, vb, w_bias, 0, 0, 0);
-        const float sum = fmaf(static_cast<float>(acc[1]), 256.0f, static_cast<float>(acc[0]));
+        float sum = fmaf(static_cast<float>(acc[1]), 256.0f, static_cast<float>(acc[0]));
+        if constexpr (kWDigits == 3) sum = fmaf(static_cast<float>(acc[2]), 65536.0f, sum);
         o_acc[bt] = fmaf(o_acc[bt], alpha, sum * w_down);
       } else {
         const v4i32 even = vb & static_cast<int>(kNibbles);
         const v4i32 odd = (vb >> 4) & static_cast<int>(kNibbles);
         const v4i32 acc_e = __builtin_amdgcn_mfma_i32_16x16x64_i8(pa, even, w_bias, 0, 0, 0);
         const v4i32 acc_o = __builtin_amdgcn_mfma_i32_16x16x64_i8(pa, odd, w_bias, 0, 0, 0);
-        const float sum_e = fmaf(static_cast<float>(acc_e[1]), 256.0f, static_cast<float>(acc_e[0]));
-        const float sum_o = fmaf(static_cast<float>(acc_o[1]), 256.0f, static_cast<float>(acc_o[0]));
+        float sum_e = fmaf(static_cast<float>(acc_e[1]), 256.0f, static_cast<float>(acc_e[0]));
+        float sum_o = fmaf(static_cast<float>(acc_o[1]), 256.0f, static_cast<float>(acc_o[0]));
+        if constexpr (kWDigits == 3) {
+          sum_e = fmaf(static_cast<float>(acc_e[2]), 65536.0f, sum_e);
+          sum_o = fmaf(static_cast<float>(acc_o[2]), 65536.0f, sum_o);
+        }
         o_acc[2 * bt] = fmaf(o_acc[2 * bt], alpha, sum_e * w_down);
         o_acc[2 * bt + 1] = fmaf(o_acc[2 * bt + 1], alpha, sum_o * w_down);
       }
     }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // (the stage and the weights are free for the next round)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // (the stage and the weights are free again)
+    if (t0 + 2 * t_step < pos) request(t0 + 2 * t_step, stage);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // (a wave with no slab below pos: its first request lands before it leaves)
 

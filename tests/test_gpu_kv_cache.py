@@ -216,31 +216,35 @@ def test_argument_checks(ext):
 # ---- the kernels the decode step runs, straight against the oracle -------------------------------------
 
 
-def rope_oracle(x, cos, sin):
-    """transformers' apply_rotary_pos_emb on bf16 values, every product and the sum rounded to bf16
+def rope_oracle(x, cos, sin, tag="bf16"):
+    """transformers' apply_rotary_pos_emb on values of the model's dtype, every product and the sum rounded to it
     (x [H, D]; cos, sin [D]): x * cos + rotate_half(x) * sin."""
     half = x.shape[-1] // 2
     rot = np.concatenate((-x[..., half:], x[..., :half]), axis=-1)
-    a = oracle.round_to(x * cos, "bf16")
-    b = oracle.round_to(rot * sin, "bf16")
-    return oracle.round_to(a + b, "bf16")
+    a = oracle.round_to(x * cos, tag)
+    b = oracle.round_to(rot * sin, tag)
+    return oracle.round_to(a + b, tag)
 
 
-def decode_step_case(ext, bits, ctx, q_heads=32, kv_heads=8, d=64, seed=0, t_max=None):
+DTYPE_OF_TAG = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}
+
+
+def decode_step_case(ext, bits, ctx, q_heads=32, kv_heads=8, d=64, seed=0, t_max=None, tag="bf16"):
     """KV-cache quantization in decode attention, Llama-3.2-1B geometry: a cache of `ctx` tokens with
     per-channel scale variance, one new token through RoPE -> quantize-append -> attention. Returns the
     device-side cache, the q|k|v row and tables, and the oracle's attention output [Hq, D] (bf16 values)."""
+    dtype = DTYPE_OF_TAG[tag]
     gen = torch.Generator().manual_seed(seed)
     channel = torch.exp(0.5 * torch.randn(d, generator=gen))
-    k = (torch.randn(kv_heads, ctx, d, generator=gen) * channel).to(torch.bfloat16)
-    v = (torch.randn(kv_heads, ctx, d, generator=gen) * channel).to(torch.bfloat16)
-    qkv = torch.randn(1, (q_heads + 2 * kv_heads) * d, generator=gen).to(torch.bfloat16)
-    qkv[:, q_heads * d:] *= channel.repeat(2 * kv_heads).to(torch.bfloat16)
+    k = (torch.randn(kv_heads, ctx, d, generator=gen) * channel).to(dtype)
+    v = (torch.randn(kv_heads, ctx, d, generator=gen) * channel).to(dtype)
+    qkv = torch.randn(1, (q_heads + 2 * kv_heads) * d, generator=gen).to(dtype)
+    qkv[:, q_heads * d:] *= channel.repeat(2 * kv_heads).to(dtype)
     t_max = ctx + 1 if t_max is None else t_max
     inv_freq = 1.0 / (500000.0 ** (torch.arange(0, d, 2).float() / d))
     emb = torch.outer(torch.arange(t_max).float(), inv_freq)
     emb = torch.cat((emb, emb), -1)
-    cos_t, sin_t = emb.cos().to(torch.bfloat16), emb.sin().to(torch.bfloat16)
+    cos_t, sin_t = emb.cos().to(dtype), emb.sin().to(dtype)
 
     cache = new_cache(kv_heads, t_max, d, bits)
     if ctx:
@@ -251,13 +255,13 @@ def decode_step_case(ext, bits, ctx, q_heads=32, kv_heads=8, d=64, seed=0, t_max
     k_new = row[q_heads * d: (q_heads + kv_heads) * d].reshape(kv_heads, d)
     v_new = row[(q_heads + kv_heads) * d:].reshape(kv_heads, d)
     cos, sin = to_np(cos_t)[ctx], to_np(sin_t)[ctx]
-    q_rot, k_rot = rope_oracle(q_new, cos, sin), rope_oracle(k_new, cos, sin)
+    q_rot, k_rot = rope_oracle(q_new, cos, sin, tag), rope_oracle(k_new, cos, sin, tag)
     k_all = np.concatenate((to_np(k), k_rot[:, None]), axis=1)
     v_all = np.concatenate((to_np(v), v_new[:, None]), axis=1)
     kq, ks = oracle.kv_quant(k_all, bits)
     vq, vs = oracle.kv_quant(v_all, bits)
-    want = oracle.gqa_decode_attention(q_rot, oracle.kv_dequant(kq, ks, "bf16"), oracle.kv_dequant(vq, vs, "bf16"),
-                                       d ** -0.5, "bf16")
+    want = oracle.gqa_decode_attention(q_rot, oracle.kv_dequant(kq, ks, tag), oracle.kv_dequant(vq, vs, tag),
+                                       d ** -0.5, tag)
     return cache, qkv.cuda(), cos_t.cuda(), sin_t.cuda(), want, (kq, ks, vq, vs)
 
 
@@ -342,3 +346,29 @@ def test_long_cache_decode_step_on_the_matrix_core_against_the_oracle(ext, bits,
     per_head = np.linalg.norm(got - want, axis=1) / np.linalg.norm(want, axis=1)
     assert per_head.max() <= 2e-2, per_head.argmax()
     print(f"int{bits} ctx {ctx} splits {splits} d {d}: rel-L2 {rel_l2(got, want):.2e}, worst head {per_head.max():.2e}")
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("tag,tol", [("f16", 2e-3), ("f32", 1e-3)])
+@pytest.mark.parametrize("t_max,d", [(701, 64), (2304, 64), (2304, 128)])
+def test_decode_step_attention_in_the_other_dtypes(ext, bits, tag, tol, t_max, d):
+    """fp16 and fp32 models through the split step, on a cache short enough for the vector-ALU form (701 rows) and on
+    one that takes the matrix-core form (2304 rows; heads of 64 and of 128), 700 cached tokens, against the oracle with
+    that dtype's rounding points: the appended codes and scales bit for bit, the output within the dtype's share of
+    the tolerance (fp32: what the kernels' own arithmetic leaves)."""
+    q_heads, kv_heads, ctx, splits = 32, 8, 700, 8
+    cache, qkv, cos_t, sin_t, want, (kq, ks, vq, vs) = decode_step_case(ext, bits, ctx, q_heads, kv_heads, d, seed=11,
+                                                                        t_max=t_max, tag=tag)
+    position = torch.tensor([ctx], dtype=torch.int32, device="cuda")
+    partials = torch.full((ext.kv_attend_partials_floats(q_heads, d, splits),), float("nan"), device="cuda")
+    ext.kv_rope_append_attend_split(qkv, cos_t, sin_t, cache["k_codes"], cache["v_codes"], cache["k_scale"],
+                                    cache["v_scale"], partials, position, d ** -0.5, q_heads, splits)
+    merged = ext.kv_attend_merge(partials, q_heads, d, splits, DTYPE_OF_TAG[tag])
+    assert np.array_equal(codes_np(cache["k_codes"], bits)[:, : ctx + 1], kq)
+    assert np.array_equal(codes_np(cache["v_codes"], bits)[:, : ctx + 1], vq)
+    assert np.array_equal(to_np(cache["k_scale"])[:, : ctx + 1], ks)
+    assert np.array_equal(to_np(cache["v_scale"])[:, : ctx + 1], vs)
+    got = to_np(merged).reshape(q_heads, d)
+    err = rel_l2(got, want)
+    print(f"{tag} int{bits} cache of {t_max} rows, heads of {d}: rel-L2 {err:.2e}")
+    assert err <= tol
