@@ -146,7 +146,7 @@ def test_teacher_forced_margin_with_heads_of_128(runtime):
     assert agree >= 0.8 * len(rows)
 
 
-@pytest.mark.parametrize("head_dim,kv_bits", [(64, 8), (128, 8), (64, 4)])
+@pytest.mark.parametrize("head_dim,kv_bits", [(64, 8), (128, 8), (64, 4), (128, 4)])
 def test_teacher_forced_margin_on_a_long_cache(head_dim, kv_bits):
     """A cache of 2304 rows: the fused runtime's decode step takes the matrix-core form of the attention launch (the
     cache's codes as int8 operands, four query heads of a kv head a workgroup). The whole step against the real-mode
