@@ -365,10 +365,10 @@ int llmq_kv_rope_append_attend(const void* qkv, const void* cos_table, const voi
  * by llmq_kv_attend_merge (out: [q_heads * head_dim] `dtype`), or for free by the GEMV that
  * consumes the attention output: llmq_wq_gemv_attn_merge is llmq_wq_gemv_fused whose activation is
  * dtype(merge(partials)) (o_proj of a decoder layer; in_head_dim / residual as there).
- * With n_splits >= 32 (or >= 8 and t_max >= 2048) and q_heads / kv_heads a multiple of 4 a workgroup takes four query heads of
+ * With n_splits >= 32 (or >= 8 and t_max >= 2048; heads of 128: >= 8 at any t_max) and q_heads / kv_heads a multiple of 4 a workgroup takes four query heads of
  * a kv head together, so every cache row is read and dequantized once for the four (long caches:
  * the step is bound by that arithmetic); the records and their layout are the same. When in
- * addition t_max >= 2048, the four heads' scores and weighted values are computed on the int8 matrix
+ * addition t_max >= 2048 (heads of 128: at any t_max), the four heads' scores and weighted values are computed on the int8 matrix
  * core with the cache's codes as operands (the query in three base-256 digits, the softmax weights
  * times the value scales in two): exact integer sums of code * scale, without the rounding of the
  * dequantized K and V to `dtype` that the other forms make as the reference's cache does; the

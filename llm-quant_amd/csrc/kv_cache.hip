@@ -1722,9 +1722,12 @@ extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos
   // 8 K / 16 K / 32 K: 9.7 / 13.6 / 20.9 us per layer against 13.0 / 19.7 / 32.0 us for one head per workgroup at
   // its best split count; below that the one-head form, which puts more workgroups on the chip, is as fast or faster.
   const int rep_heads = q_heads / kv_heads;
-  const bool grouped = rep_heads % 4 == 0 && (n_splits >= 32 || (n_splits >= 8 && t_max >= kMfMinCache));
+  // (heads of 128: the vector-ALU form has twice the arithmetic per cache row, and the matrix-core form is ahead at every
+  // cache length: the Llama-3-8B architecture's step at 600 cached tokens, 1968 us a token against 2038)
+  const int mf_min_cache = head_dim == 128 ? 0 : kMfMinCache;
+  const bool grouped = rep_heads % 4 == 0 && (n_splits >= 32 || (n_splits >= 8 && t_max >= mf_min_cache));
   const dim3 grid(grouped ? q_heads / 4 : q_heads, n_splits), block(kSplitThreads);
-  if (grouped && t_max >= kMfMinCache) {
+  if (grouped && t_max >= mf_min_cache) {
     // long caches: the matrix-core form (see the kernel's comment for what it changes in the arithmetic)
 #define LLMQ_SPLIT_MFMA(T, B, D)                                                                                  \
   do {                                                                                                            \
