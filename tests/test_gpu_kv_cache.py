@@ -372,3 +372,32 @@ def test_decode_step_attention_in_the_other_dtypes(ext, bits, tag, tol, t_max, d
     err = rel_l2(got, want)
     print(f"{tag} int{bits} cache of {t_max} rows, heads of {d}: rel-L2 {err:.2e}")
     assert err <= tol
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("ctx,t_max,splits,q_heads,kv_heads", [(0, 1, 8, 32, 8), (1, 2, 8, 32, 8), (63, 64, 8, 32, 8),
+                                                            (64, 65, 8, 32, 8), (300, 301, 8, 32, 8), (300, 512, 32, 8, 2),
+                                                            (700, 769, 16, 16, 4)])
+def test_heads_of_128_take_the_matrix_core_form_on_short_caches_too(ext, bits, ctx, t_max, splits, q_heads, kv_heads):
+    """With heads of 128 the entry point takes the matrix-core form of the split step whatever the cache's size (eight
+    splits or more, four query heads per kv head): caches of one row, of exactly one slab and of a few hundred rows
+    against the oracle, the checks of the long caches."""
+    d = 128
+    cache, qkv, cos_t, sin_t, want, (kq, ks, vq, vs) = decode_step_case(ext, bits, ctx, q_heads, kv_heads, d,
+                                                                        seed=100 + ctx, t_max=t_max)
+    for name in ("k_scale", "v_scale"):
+        cache[name][:, ctx + 1:] = float("nan")
+    position = torch.tensor([ctx], dtype=torch.int32, device="cuda")
+    partials = torch.full((ext.kv_attend_partials_floats(q_heads, d, splits),), float("nan"), device="cuda")
+    ext.kv_rope_append_attend_split(qkv, cos_t, sin_t, cache["k_codes"], cache["v_codes"], cache["k_scale"],
+                                    cache["v_scale"], partials, position, d ** -0.5, q_heads, splits)
+    merged = ext.kv_attend_merge(partials, q_heads, d, splits, torch.bfloat16)
+    assert np.array_equal(codes_np(cache["k_codes"], bits)[:, : ctx + 1], kq)
+    assert np.array_equal(codes_np(cache["v_codes"], bits)[:, : ctx + 1], vq)
+    assert np.array_equal(to_np(cache["k_scale"])[:, : ctx + 1], ks)
+    assert np.array_equal(to_np(cache["v_scale"])[:, : ctx + 1], vs)
+    got = to_np(merged).reshape(q_heads, d)
+    assert np.isfinite(got).all()
+    assert rel_l2(got, want) <= 1e-2
+    per_head = np.linalg.norm(got - want, axis=1) / np.linalg.norm(want, axis=1)
+    assert per_head.max() <= 2e-2, per_head.argmax()
