@@ -466,7 +466,10 @@ __global__ __launch_bounds__(256) void add_splits_kernel(const float* __restrict
     }
     *reinterpret_cast<u32x2*>(out + i4) = u32x2{bf16_pair_rne(s[0], s[1]), bf16_pair_rne(s[2], s[3])};
   } else {
-    for (int64_t i = i4; i < count; ++i) {
+    // a count that is not a multiple of four leaves the later slices off 16-byte alignment: this lane's own
+    // (up to) four values one at a time
+    const int64_t end = i4 + 4 < count ? i4 + 4 : count;
+    for (int64_t i = i4; i < end; ++i) {
       float s = partial[i];
       for (int k = 1; k < splits; ++k) s = s + partial[k * count + i];
       out[i] = from_float<bf16_t>(s);

@@ -23,6 +23,11 @@ What pins each function (the tests that do so live in tests/test_oracle_*.py):
                        (reference tests/test_moe.py:310-333)
   moe_experts_real     per expert == real_linear; tracks transformers' MixtralExperts in bf16
                        (reference tests/test_moe.py:77-117, 336-345)
+  llama_rmsnorm, llama_gated_act, llama_residual_add
+                       the elementwise steps of transformers' LlamaDecoderLayer around the Linears
+                       (third-party arithmetic the reference delegates to); pinned against the library's own
+                       LlamaRMSNorm / LlamaMLP modules and torch's bf16/fp16 adds on the CPU, and by closed
+                       forms (a constant row normalises to +-weight, silu(0) = 0)
   gqa_decode_attention the reference delegates attention to HF transformers and holds no test of its
                        arithmetic; pinned against the routines it delegates to (transformers'
                        eager_attention_forward and torch's scaled_dot_product_attention, grouped-query,
@@ -343,6 +348,35 @@ def moe_experts_real(hidden, top_k_index, top_k_weights, qgate_up, sgate_up, qdo
         final[token] = round_to(final[token] + out, dtype)
     assert final.shape[1] == h_dim
     return final
+
+
+# ---------------------------------------------------------------------------------------------
+# The elementwise steps of a decoder layer around the quantized Linears. The reference runs them through HF
+# transformers (LlamaDecoderLayer; installed transformers/models/llama/modeling_llama.py: LlamaRMSNorm.forward,
+# LlamaMLP.forward, the residual adds of LlamaDecoderLayer.forward). Rounding points are the library's.
+# ---------------------------------------------------------------------------------------------
+
+
+def llama_rmsnorm(x, weight, eps, dtype="bf16"):
+    """LlamaRMSNorm.forward: x to fp32, variance = mean(x^2) over the last axis, x * rsqrt(variance + eps),
+    rounded to `dtype`, then weight * that, rounded to `dtype` again. The mean is taken in float64 and
+    rounded to fp32 once (torch leaves its order to the reduction kernel)."""
+    xf = np.asarray(x, dtype=np.float32)
+    variance = (xf.astype(np.float64) ** 2).mean(axis=-1, keepdims=True).astype(np.float32)
+    inv = (1.0 / np.sqrt((variance + np.float32(eps)).astype(np.float64))).astype(np.float32)
+    normed = round_to(xf * inv, dtype)
+    return round_to(np.asarray(weight, dtype=np.float32) * normed, dtype)
+
+
+def llama_gated_act(gate, up, dtype="bf16"):
+    """LlamaMLP.forward's act_fn(gate_proj(x)) * up_proj(x) on `dtype` tensors: silu rounded to `dtype`, the
+    product rounded to `dtype`."""
+    return round_to(silu(gate, dtype) * np.asarray(up, dtype=np.float32), dtype)
+
+
+def llama_residual_add(residual, branch, dtype="bf16"):
+    """residual + branch on `dtype` tensors (LlamaDecoderLayer.forward): one rounding of the exact sum."""
+    return round_to(np.asarray(residual, dtype=np.float32) + np.asarray(branch, dtype=np.float32), dtype)
 
 
 # ---------------------------------------------------------------------------------------------

@@ -2,16 +2,23 @@
 weights int8, MLP int4, lm_head int8, int8 KV cache (the end-to-end decode case, at reduced and at
 full size).
 
-What is asserted, and why it is not plain token equality with the oracle model: the oracle
-model is HF transformers driven with mode="real" Linears and FakeQuantCache. A random-init
-network amplifies any difference in fp32 summation order (one bf16 ulp in one Linear output)
-into ~2-4 % logit noise after 16 layers, while the oracle's own top-2 logit gaps have a median
-of ~0.1 and reach 0: free-running greedy streams of two correct implementations part at the
-first near-tie. So the checks are (a) replay == eager, bit for bit (the reference's own
-criterion, tests/test_graph_decode.py:92-136); (b) under teacher forcing, the logits stay within
-a relative error bound and every disagreeing argmax sits at an oracle top-2 gap smaller than
-the measured logit error; (c) each runtime layer equals the HF layer it walks, to bf16
-resolution, on identical inputs.
+The oracle model is HF transformers driven with mode="real" Linears and FakeQuantCache.
+
+Token identity (the first 64 greedy tokens, free-running on both sides, equal to the oracle model's) is
+asserted on float32 models, at full size and on two small geometries, for graphed_generate (fused step under
+HIP graph replay), the fused step run eagerly and the operation-by-operation walk: there the two
+implementations differ by fp32 summation order only (~1e-6 of a logit) while the oracle's top-2 gaps stay
+above 5e-4, so equality is what a correct implementation gives.
+
+On bfloat16 models the same criterion cannot be asserted against an implementation whose Linears are not
+bit-identical to torch's bf16 arithmetic: a random-init network amplifies one bf16 ulp in one Linear output
+into ~2-4 % logit noise after 16 layers, while the oracle's own top-2 logit gaps (bf16 logits) have a median
+of ~0.1 and reach exactly 0, so free-running streams of two correct implementations part at the first
+near-tie. There the checks are (a) replay == eager, bit for bit (the reference's own criterion,
+tests/test_graph_decode.py:92-136); (b) under teacher forcing, the logits stay within a relative error
+bound and every disagreeing argmax sits at an oracle top-2 gap smaller than twice the measured logit error;
+(c) each runtime layer equals the HF layer it walks, to bf16 resolution, on identical inputs; and the
+plain 64-token identity is kept as an expected failure so that its state is on record in every run.
 """
 
 import copy
@@ -22,7 +29,7 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-def build_model(hidden, inter, layers, heads, kv_heads, vocab, seed=0, head_dim=64):
+def build_model(hidden, inter, layers, heads, kv_heads, vocab, seed=0, head_dim=64, dtype=torch.bfloat16):
     from transformers import LlamaConfig, LlamaForCausalLM
 
     torch.manual_seed(seed)
@@ -34,7 +41,7 @@ def build_model(hidden, inter, layers, heads, kv_heads, vocab, seed=0, head_dim=
     for p in model.parameters():
         if p.dim() > 1:
             torch.nn.init.normal_(p, 0, 0.02)
-    return model.to(torch.bfloat16).cuda().eval()
+    return model.to(dtype).cuda().eval()
 
 
 def quantized_pair(model):
@@ -226,9 +233,11 @@ def llama_1b():
     return pair
 
 
-#: teacher-forced relative logit error allowed at full size. A random-init 16-layer network turns
-#: one-ulp bf16 differences between two correct implementations (summation order of the projections, the
-#: attention's rounding points) into a few per cent of logit noise: measured 0.02-0.05 on this model.
+#: teacher-forced relative logit error allowed at full size in bfloat16: a guard against a broken layer, not a
+#: parity tolerance (no tolerance is stated for logits after 16 bf16 layers; the stated fp32 bound, rel-L2 1e-3,
+#: is applied to the float32 models in test_first_64_greedy_tokens_identical_fp32). A random-init 16-layer
+#: network turns one-ulp bf16 differences between two correct implementations (summation order of the
+#: projections, the attention's rounding points) into a few per cent of logit noise: measured 0.02-0.05 here.
 FULL_SIZE_REL_BOUND = 0.08
 
 
@@ -255,35 +264,114 @@ def test_teacher_forced_margin_llama_1b_config(llama_1b, runtime):
     assert agree >= 0.85 * len(rows)
 
 
-#: identical-prefix length of the free-running streams measured on this model and prompt (64 = the whole
-#: window). The assertion below allows it to move only where the oracle itself is at a near-tie.
-MEASURED_FREE_RUNNING_PREFIX = 2
+_FREE_RUNNING = {}
 
 
-def test_free_running_prefix_llama_1b_config(llama_1b):
-    """The first 64 greedy tokens, free-running on both sides: the real-mode model's own stream against
-    graphed_generate's (fused step, HIP graph replay). Reports the identical-prefix length and asserts
-    (a) it is at least the length recorded above, and (b) where the streams part, they part at a token
-    whose top-2 logit gap in the oracle is within twice the logit error measured at that very step under
-    teacher forcing, i.e. at a near-tie that arithmetic noise decides, never at a clear margin. Up to the
-    parting point both sides have seen the same tokens, so the teacher-forced row describes that step."""
+def free_running_bf16(llama_1b):
+    """graphed_generate's and the eager fused runtime's first 64 free-running tokens at full size (bf16)."""
     from llmquant.runtime import LlamaFusedRuntime, graphed_generate
 
-    real, kernel = llama_1b
-    rows, oracle_stream, ids = full_size_rows(llama_1b, "fused")
-    kernel.__dict__.pop("_llmq_kept_runtimes", None)
-    free = graphed_generate(kernel, ids, 65, kv_bits=8)[0, 512:].tolist()
-    eager = LlamaFusedRuntime(kernel, 512 + 65 + 1, 8).generate(ids, 65, use_graph=False)[0, 512:].tolist()
-    kernel.__dict__.pop("_llmq_kept_runtimes", None)
+    if not _FREE_RUNNING:
+        _, kernel = llama_1b
+        _, _, ids = full_size_rows(llama_1b, "fused")
+        kernel.__dict__.pop("_llmq_kept_runtimes", None)
+        _FREE_RUNNING["replay"] = graphed_generate(kernel, ids, 65, kv_bits=8)[0, 512:].tolist()
+        _FREE_RUNNING["eager"] = LlamaFusedRuntime(kernel, 512 + 65 + 1, 8).generate(ids, 65, use_graph=False)[0, 512:].tolist()
+        kernel.__dict__.pop("_llmq_kept_runtimes", None)
+    return _FREE_RUNNING["replay"], _FREE_RUNNING["eager"]
+
+
+def test_free_running_streams_part_only_at_a_near_tie_llama_1b_config_bf16(llama_1b):
+    """bfloat16, full size, free-running on both sides: the real-mode model's own stream against
+    graphed_generate's (fused step, HIP graph replay). Asserts that replay and eager runs give the same
+    tokens, and that where the streams part, they part at a token whose top-2 logit gap in the oracle is
+    within twice the logit error measured at that very step under teacher forcing, i.e. at a near-tie
+    that arithmetic noise decides, never at a clear margin. Up to the parting point both sides have seen
+    the same tokens, so the teacher-forced row describes that step. (The identity of all 64 tokens is
+    the next test's subject; for float32 models it is asserted further down.)"""
+    rows, oracle_stream, _ = full_size_rows(llama_1b, "fused")
+    free, eager = free_running_bf16(llama_1b)
     assert free == eager  # replay == eager at full size, bit for bit in the tokens
     prefix = identical_prefix(free[:64], oracle_stream[:64])
     agree = sum(a == b for a, b in zip(free[:64], oracle_stream[:64]))
-    print(f"free-running: identical prefix {prefix}/64 tokens, {agree}/64 positions equal")
+    print(f"free-running, bf16: identical prefix {prefix}/64 tokens, {agree}/64 positions equal")
     if prefix < 64:
         ok, gap, err, rel = rows[prefix]
         print(f"streams part at token {prefix}: oracle top-2 gap {gap:.4f}, logit error there {err:.4f}")
         assert not ok and gap <= 2 * err
-    assert prefix >= MEASURED_FREE_RUNNING_PREFIX
+
+
+@pytest.mark.xfail(strict=False, reason="bfloat16 random-init model: the oracle's own bf16 logits tie exactly (top-2 gap "
+                   "0.0) at the third token while two correct bf16 implementations differ by ~0.05-0.15 of a logit "
+                   "there; identity of the 64 tokens is asserted on the float32 models below")
+def test_first_64_greedy_tokens_identical_llama_1b_config_bf16(llama_1b):
+    _, oracle_stream, _ = full_size_rows(llama_1b, "fused")
+    free, _ = free_running_bf16(llama_1b)
+    assert free[:64] == oracle_stream[:64]
+
+
+def oracle_greedy_stream(real, ids, new_tokens, kv_bits=8):
+    """The real-mode model's own free-running greedy tokens under HF transformers with FakeQuantCache, and
+    the top-2 logit gap at each pick."""
+    from llmquant.quantizers import make_cache_factory
+
+    cache = make_cache_factory(kv_bits)()
+    stream, gaps, rows = [], [], []
+    with torch.no_grad():
+        logits = real(ids, past_key_values=cache, use_cache=True).logits[0, -1].float()
+        for _ in range(new_tokens):
+            rows.append(logits)
+            top2 = logits.topk(2).values
+            gaps.append((top2[0] - top2[1]).item())
+            tok = logits.argmax().reshape(1, 1)
+            stream.append(tok.item())
+            logits = real(tok, past_key_values=cache, use_cache=True).logits[0, -1].float()
+    return stream, gaps, rows
+
+
+FP32_MODELS = {
+    # name: (build_model arguments, keyword arguments, vocabulary, prompt tokens)
+    "llama-1b architecture, full size": ((2048, 8192, 16, 32, 8, 128256), dict(), 128256, 512),
+    "3 layers, heads of 64": ((512, 1024, 3, 8, 2, 4096), dict(), 4096, 48),
+    "2 layers, heads of 128, wide MLP": ((512, 7168, 2, 4, 2, 4096), dict(seed=3, head_dim=128), 4096, 300),
+}
+
+
+@pytest.mark.parametrize("name", list(FP32_MODELS))
+def test_first_64_greedy_tokens_identical_fp32(name):
+    """The token criterion itself, where arithmetic noise cannot decide a pick: the same architecture,
+    seed and recipe (attention int8, MLP int4, lm_head int8, int8 KV) built in float32. Free-running on
+    both sides, the first 64 greedy tokens of graphed_generate (the fused five-launch step under HIP
+    graph replay: what the benchmark runs), of the fused step run eagerly and of the operation-by-
+    operation walk all equal the real-mode model's under HF transformers with FakeQuantCache(8).
+    The kernel side differs from the oracle by fp32 summation order and the GEMV's 2^-22 block
+    exponent (~1e-6 of a logit); the oracle's smallest top-2 gap over the 64 picks is asserted to be
+    above 1e-4, so the equality does not hang on a tie. The logits of every one of the 64 steps are
+    held to the oracle's within rel-L2 1e-3, the bound stated for fp32 accumulation, through all layers."""
+    from llmquant.runtime import LlamaFusedRuntime, LlamaKernelRuntime, graphed_generate
+
+    shape, extra, vocab, prompt = FP32_MODELS[name]
+    real, kernel = quantized_pair(build_model(*shape, dtype=torch.float32, **extra))
+    torch.cuda.empty_cache()
+    ids = torch.randint(0, vocab, (1, prompt), generator=torch.Generator().manual_seed(1)).cuda()
+    want, gaps, want_logits = oracle_greedy_stream(real, ids, 64)
+    print(f"{name}: oracle top-2 gaps over 64 picks: min {min(gaps):.2e}, median {sorted(gaps)[32]:.3f}")
+    assert min(gaps) > 1e-4
+    replay = graphed_generate(kernel, ids, 64, kv_bits=8)[0, prompt:].tolist()
+    kernel.__dict__.pop("_llmq_kept_runtimes", None)
+    assert replay == want, f"graph replay parts from the oracle at token {identical_prefix(replay, want)}"
+    rt = LlamaFusedRuntime(kernel, prompt + 66, 8)
+    tok, eager, worst = rt.prefill(ids), [], 0.0
+    for i in range(64):
+        eager.append(tok.item())
+        logits, tok = rt.eager_step(tok, prompt + i)
+        if i + 1 < 64 and eager == want[:i + 1]:  # (same tokens seen so far: the same step on both sides)
+            worst = max(worst, ((logits[0].float() - want_logits[i + 1]).norm() / want_logits[i + 1].norm()).item())
+    print(f"{name}: largest relative logit error over the steps {worst:.2e}")
+    assert eager == want, f"the eager fused step parts from the oracle at token {identical_prefix(eager, want)}"
+    assert worst <= 1e-3
+    walk = LlamaKernelRuntime(kernel, prompt + 66, 8).generate(ids, 64, use_graph=False)[0, prompt:].tolist()
+    assert walk == want, f"the walk parts from the oracle at token {identical_prefix(walk, want)}"
 
 
 def test_runtime_layer_equals_the_hf_layer(small):

@@ -1,9 +1,16 @@
-"""The fused decode-step kernels against the operation-by-operation forms they replace.
+"""The fused decode-step kernels: against the CPU oracle, and against the operation-by-operation forms
+they replace.
 
 Each fused op must reproduce the PyTorch sequence of transformers' LlamaDecoderLayer with its
 rounding points: RMSNorm -> Linear, SiLU(gate)*up -> Linear, head-padded input -> Linear,
-Linear -> + residual, RoPE -> cache append -> attention, argmax. The unfused side uses the
-same GEMV / cache kernels (themselves checked against the oracle elsewhere), so equality here is
+Linear -> + residual, RoPE -> cache append -> attention, argmax.
+
+The oracle tests (`*_against_the_oracle`) build the staged activation in numpy with the library's rounding
+points (oracle.llama_rmsnorm / llama_gated_act / pad_activation / llama_residual_add, themselves pinned
+against transformers' modules on the CPU) and hold the kernel's output to the float64 closed form of the
+real-mode Linear (llmquant/quantizers/real.py:76-103) at the Llama-3.2-1B and Llama-3-8B layer shapes, int8
+and int4: rel-L2 <= 1e-2 for bf16 outputs and <= 1e-3 for fp32 (the stated bars; measured ~2e-3 and ~1e-7).
+The remaining tests compare with the unfused sequence over the same GEMV / cache kernels, where equality is
 expected to the bit except where a reduction order differs (RMSNorm's variance).
 """
 
@@ -31,6 +38,110 @@ def weights(n, k, bits, out_group=0, head_dim=None, seed=0):
     canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP, head_dim, out_group or None)
     q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
     return q, torch.from_numpy(scales).cuda()
+
+
+def oracle_weights(n, k, bits, out_group=0, head_dim=None, seed=0):
+    """(device codes, device scales, canonical codes, scales): the weight on both sides of a comparison."""
+    torch.manual_seed(seed)
+    w = (torch.randn(n, k) * 0.02).to(torch.bfloat16)
+    canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP, head_dim, out_group or None)
+    q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
+    return q, torch.from_numpy(scales).cuda(), canonical, scales
+
+
+#: the projections a decode step runs behind an RMSNorm, (N, K, out_group): q|k|v with one scale row per head,
+#: gate|up, lm_head -- of the Llama-3.2-1B and the Llama-3-8B architecture
+NORM_THEN_LINEAR = {
+    "1B q|k|v": (3072, 2048, 64), "1B gate|up": (16384, 2048, 0), "1B lm_head": (128256, 2048, 0),
+    "8B q|k|v": (6144, 4096, 128), "8B gate|up": (28672, 4096, 0),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("name", list(NORM_THEN_LINEAR))
+def test_rmsnorm_prologue_against_the_oracle(ext, name, bits, dtype):
+    """llmq_wq_gemv_fused with the RMSNorm prologue == real-mode Linear over LlamaRMSNorm's output, both in
+    numpy: the norm with the library's rounding points, the Linear as the float64 closed form."""
+    n, k, out_group = NORM_THEN_LINEAR[name]
+    q, s, canonical, scales = oracle_weights(n, k, bits, out_group, seed=21)
+    tag = "bf16" if dtype == torch.bfloat16 else "f32"
+    torch.manual_seed(22)
+    x = (torch.randn(1, k) * 3).to(dtype)
+    norm = (1 + 0.1 * torch.randn(k)).to(dtype)
+    got = ext.wq_gemv_fused(x.cuda(), q, s, out_group, 1, norm.cuda(), 1e-5, 0, None)
+    assert got.shape == (1, n) and got.dtype == dtype
+    staged = oracle.llama_rmsnorm(to_np(x), to_np(norm), 1e-5, tag)
+    exact = oracle.gemv_float64(staged, canonical, scales, out_group or None)
+    err = rel_l2(to_np(got), exact)
+    assert err <= (1e-2 if tag == "bf16" else 1e-3)
+    assert err <= (2.5e-3 if tag == "bf16" else 1e-5)   # measured: the output's own rounding and little else
+    if tag == "bf16":
+        want = oracle.round_to(exact.astype(np.float32), "bf16")
+        assert (to_np(got) == want).mean() > 0.98
+
+
+#: down_proj of the two architectures: (N, K)
+GATED_THEN_LINEAR = {"1B down": (2048, 8192), "8B down": (4096, 14336)}
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("name", list(GATED_THEN_LINEAR))
+def test_silu_mul_prologue_and_residual_against_the_oracle(ext, name, bits):
+    """llmq_wq_gemv_fused with the SiLU(gate) * up prologue and the residual epilogue == LlamaMLP's elementwise
+    step, the real-mode Linear and LlamaDecoderLayer's add, each with its bf16 rounding, in numpy."""
+    n, k = GATED_THEN_LINEAR[name]
+    q, s, canonical, scales = oracle_weights(n, k, bits, seed=23)
+    torch.manual_seed(24)
+    gate_up = (torch.randn(1, 2 * k) * 2).to(torch.bfloat16)
+    res = torch.randn(1, n).to(torch.bfloat16)
+    got = ext.wq_gemv_fused(gate_up.cuda(), q, s, 0, 2, None, 0.0, 0, res.cuda())
+    act = oracle.llama_gated_act(to_np(gate_up)[:, :k], to_np(gate_up)[:, k:], "bf16")
+    branch = oracle.gemv_float64(act, canonical, scales)
+    want = oracle.llama_residual_add(to_np(res), oracle.round_to(branch.astype(np.float32), "bf16"), "bf16")
+    assert rel_l2(to_np(got), want) <= 1e-2
+    assert rel_l2(to_np(got), to_np(res).astype(np.float64) + branch) <= 3e-3   # (unrounded: the tolerance anchor)
+    assert (to_np(got) == want).mean() > 0.98
+    # and with nothing in front of it but the residual behind: the plain activation
+    plain = ext.wq_gemv_fused(torch.from_numpy(act).to(torch.bfloat16).cuda(), q, s, 0, 0, None, 0.0, 0, res.cuda())
+    assert rel_l2(to_np(plain), want) <= 1e-2 and (to_np(plain) == want).mean() > 0.98
+
+
+@pytest.mark.parametrize("prologue", [0, 1], ids=["plain", "rmsnorm"])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("inter,k", [(8192, 2048), (14336, 4096)], ids=["1B gate|up", "8B gate|up"])
+def test_gate_up_silu_against_the_oracle(ext, inter, k, bits, prologue):
+    """llmq_wq_gemv_gate_up_silu (the gate|up GEMV that stores act(gate) * up) == [RMSNorm ->] the two real-mode
+    Linears -> LlamaMLP's elementwise step, in numpy: gate and up rounded to bf16 as the Linears' outputs are,
+    silu rounded, the product rounded."""
+    q, s, canonical, scales = oracle_weights(2 * inter, k, bits, seed=25)
+    torch.manual_seed(26)
+    x = (torch.randn(1, k) * 2).to(torch.bfloat16)
+    norm = (1 + 0.1 * torch.randn(k)).to(torch.bfloat16) if prologue else None
+    got = ext.wq_gemv_gate_up_silu(x.cuda(), q, s, prologue, norm.cuda() if prologue else None, 1e-5)
+    staged = oracle.llama_rmsnorm(to_np(x), to_np(norm), 1e-5, "bf16") if prologue else to_np(x)
+    both = oracle.round_to(oracle.gemv_float64(staged, canonical, scales).astype(np.float32), "bf16")
+    want = oracle.llama_gated_act(both[:, :inter], both[:, inter:], "bf16")
+    assert got.shape == (1, inter)
+    assert rel_l2(to_np(got), want) <= 1e-2
+    assert (to_np(got) == want).mean() > 0.97
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("n,k,head_dim", [(2048, 2048, 64), (4096, 4096, 128)], ids=["1B o_proj", "8B o_proj"])
+def test_head_padding_and_residual_against_the_oracle(ext, n, k, head_dim, bits):
+    """o_proj in the decode step: the attention output's heads padded to groups while staging (heads of 64 in
+    groups of 128; heads of 128 need none), the real-mode Linear, the residual add -- against numpy."""
+    padded_heads = head_dim if head_dim < GROUP else None
+    q, s, canonical, scales = oracle_weights(n, k, bits, head_dim=padded_heads, seed=27)
+    torch.manual_seed(28)
+    x = torch.randn(1, k).to(torch.bfloat16)
+    res = torch.randn(1, n).to(torch.bfloat16)
+    got = ext.wq_gemv_fused(x.cuda(), q, s, 0, 0, None, 0.0, padded_heads or 0, res.cuda())
+    branch = oracle.gemv_float64(oracle.pad_activation(to_np(x), GROUP, padded_heads), canonical, scales)
+    want = oracle.llama_residual_add(to_np(res), oracle.round_to(branch.astype(np.float32), "bf16"), "bf16")
+    assert rel_l2(to_np(got), want) <= 1e-2
+    assert (to_np(got) == want).mean() > 0.98
 
 
 @pytest.mark.parametrize("bits", [8, 4])

@@ -157,11 +157,13 @@ def tile_case(ext, m, n, k, bits, out_group=0, head_dim=None, seed=0, scale=1.0,
 
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("m,n,k", [(128, 256, 128), (65, 256, 256), (130, 300, 768), (512, 512, 2048), (300, 70, 384),
-                                   (129, 257, 1152), (1, 16, 128), (256, 1024, 8192)])
+                                   (129, 257, 1152), (1, 16, 128), (256, 1024, 8192), (65, 70, 1024),
+                                   (1023, 66, 2048)])
 def test_tiled_gemm_against_the_oracle(ext, bits, m, n, k):
     """Whole outputs against the float64 closed form and the real-mode forward: full tiles, ragged M and N
     (rows and columns past the end are clamped for the loads and dropped at the store), one group, rows long
-    enough that the reduction axis is split across workgroups."""
+    enough that the reduction axis is split across workgroups, and split outputs whose element count is not a
+    multiple of four (the slice addition then walks its values one at a time)."""
     got, x, canonical, scales = tile_case(ext, m, n, k, bits, seed=m + n)
     assert got.shape == (m, n) and got.dtype == torch.bfloat16
     exact = oracle.gemv_float64(x, canonical, scales)

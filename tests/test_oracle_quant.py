@@ -375,6 +375,63 @@ def test_attention_matches_the_library_routines_the_reference_delegates_to():
     assert not np.allclose(wrong, eager[0, 0].numpy(), rtol=1e-2, atol=1e-2)
 
 
+def _bf16_ulps(a, b):
+    ia = (np.ascontiguousarray(a, dtype=np.float32).view(np.uint32) >> 16).astype(np.int64)
+    ib = (np.ascontiguousarray(b, dtype=np.float32).view(np.uint32) >> 16).astype(np.int64)
+    ia = np.where(ia & 0x8000, 0x8000 - ia, ia)
+    ib = np.where(ib & 0x8000, 0x8000 - ib, ib)
+    return np.abs(ia - ib)
+
+
+def test_decoder_layer_elementwise_steps_match_the_library_modules():
+    """llama_rmsnorm / llama_gated_act / llama_residual_add against transformers' own LlamaRMSNorm and
+    LlamaMLP (driven with identity projections) and torch's 16-bit adds, on the CPU. A rounding point
+    moved (fp32 product kept past the cast, the weight applied before the cast, silu left unrounded)
+    fails the equality; the variance's summation order may move a normalised value by one unit of the
+    last place at most, and rarely."""
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaMLP, LlamaRMSNorm
+
+    torch.manual_seed(0)
+    for dtype, tag in ((torch.bfloat16, "bf16"), (torch.float16, "f16"), (torch.float32, "f32")):
+        x = (torch.randn(3, 2048) * 3).to(dtype)
+        norm = LlamaRMSNorm(2048, eps=1e-5).to(dtype)
+        with torch.no_grad():
+            norm.weight.copy_((1 + 0.1 * torch.randn(2048)).to(dtype))
+            theirs = norm(x).float().numpy()
+        mine = oracle.llama_rmsnorm(x.float().numpy(), norm.weight.detach().float().numpy(), 1e-5, tag)
+        if tag == "bf16":
+            ulps = _bf16_ulps(mine, theirs)
+            assert ulps.max() <= 1 and (ulps == 0).mean() > 0.999
+        else:
+            np.testing.assert_allclose(mine, theirs, rtol=2e-3 if tag == "f16" else 1e-6, atol=0)
+            assert (mine == theirs).mean() > 0.99
+        gate, up = (torch.randn(3, 512) * 2).to(dtype), torch.randn(3, 512).to(dtype)
+        cfg = LlamaConfig(hidden_size=512, intermediate_size=512, hidden_act="silu")
+        mlp = LlamaMLP(cfg).to(dtype)
+        with torch.no_grad():
+            theirs = (mlp.act_fn(gate) * up).float().numpy()
+        mine = oracle.llama_gated_act(gate.float().numpy(), up.float().numpy(), tag)
+        if tag == "f32":
+            np.testing.assert_allclose(mine, theirs, rtol=1e-6, atol=1e-12)
+        else:
+            assert np.array_equal(mine, theirs)
+        a, b = torch.randn(3, 512).to(dtype), torch.randn(3, 512).to(dtype)
+        assert np.array_equal(oracle.llama_residual_add(a.float().numpy(), b.float().numpy(), tag),
+                              (a + b).float().numpy())
+    # closed forms: a constant row normalises to +-weight (eps = 0), silu(0) * up = 0
+    w = np.linspace(0.5, 1.5, 64, dtype=np.float32)
+    assert np.array_equal(oracle.llama_rmsnorm(np.full((1, 64), -4.0, np.float32), w, 0.0, "f32"), -w[None])
+    assert np.array_equal(oracle.llama_gated_act(np.zeros((1, 8), np.float32), np.ones((1, 8), np.float32)), np.zeros((1, 8)))
+    # a rounding point moved must show: the weight applied in fp32 before the cast differs from the library
+    x = (torch.randn(4, 2048) * 3).to(torch.bfloat16)
+    wt = (1 + 0.1 * torch.randn(2048)).to(torch.bfloat16)
+    xf = x.float().numpy()
+    inv = 1.0 / np.sqrt((xf.astype(np.float64) ** 2).mean(-1, keepdims=True) + 1e-5)
+    moved = oracle.round_to((wt.float().numpy() * (xf * inv)).astype(np.float32), "bf16")
+    assert (moved != oracle.llama_rmsnorm(xf, wt.float().numpy(), 1e-5, "bf16")).mean() > 0.05
+
+
 def test_prompt_attention_is_the_decode_attention_of_every_prefix_and_the_library_routine():
     """The causal form, pinned three ways: row i equals the one-token attention of query i over keys 0..i
     (the function above, itself pinned against transformers); it equals torch's scaled_dot_product_attention
