@@ -221,6 +221,23 @@ def main():
 
     dom_graph_us = _graph_time_us(torch, dominant_burst, reps=5) / 12
 
+    # ---- configs[0]: the single down_proj int4 GEMV (2048 x 8192, M = 1) on its own line: the launch under graph
+    # replay, weights rotated over > 600 MB (72 copies of 8.9 MB) so that every launch reads HBM
+    down4 = next(c for c in cases if c["name"] == "down" and c["bits"] == 4)
+    rot = [(torch.roll(down4["bufs"][0][0], i, 0).contiguous(), torch.roll(down4["bufs"][0][1], i, 0).contiguous())
+           for i in range(72)]
+
+    def config1_burst():
+        here = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for q, s in rot:
+            rc = lib.llmq_wq_gemv(down4["x"].data_ptr(), q.data_ptr(), s.data_ptr(), down4["out"].data_ptr(),
+                                  1, down4["n"], down4["k"] // GROUP, GROUP, 0, 4, BF16, here)
+            if rc:
+                raise RuntimeError(lib.llmq_last_error().decode())
+
+    config1_us = _graph_time_us(torch, config1_burst, reps=5) / len(rot)
+    del rot
+
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     achieved = dominant["bytes"] / (dom_avg_ms * 1e-3) / 1e9
     result = {
@@ -251,6 +268,13 @@ def main():
                      "box_streaming_read_GBps": round(read_ceiling, 1),
                      "frac_of_box_streaming_read": round(achieved / read_ceiling, 4)},
         "shapes": shapes,
+        "config1_down_proj_int4_gemv": {
+            "workload": "configs[0]: N=2048, K=8192, M=1, int4 g128, bf16 activation, fp32 accumulation",
+            "bytes": down4["bytes"], "graph_replay_launch_us": round(config1_us, 2),
+            "GBps": round(down4["bytes"] / config1_us / 1e3, 1),
+            "frac_hbm": round(down4["bytes"] / config1_us / 1e3 / HBM_PEAK_GBPS, 4),
+            "note": "8.9 MB at 8 TB/s is 1.1 us, under the 2.0 us an empty kernel takes under graph replay: this "
+                    "launch is bound by its fixed cost (launch, activation staging, first-byte latency), not by HBM"},
     }
 
     del cases
@@ -712,45 +736,110 @@ def decode_leg(torch, arch="llama3.2-1b"):
         return lat, {"ttft_ms": round(lat["ttft_ms"], 2), "decode_tok_s": round(lat["decode_tps"], 1)}
 
     res = {"architecture": arch, "prompt_tokens": prompt, "new_tokens": new, "hip_graph": True,
-           "paths": {"bf16": "HF LlamaForCausalLM module walk over a StaticCache, one captured step, kept between "
-                             "calls (hf_static_cache_graph)",
+           "paths": {"bf16_fused_runtime": "the bf16 model through the same five-launch step as the quantized one: "
+                                           "LlamaDenseFusedRuntime (llmq_dense_gemv_fused over the bf16 weights, "
+                                           "unquantized bf16 KV cache), one captured step, kept between calls",
+                     "bf16_hf_walk": "HF LlamaForCausalLM module walk over a StaticCache, one captured step, kept "
+                                     "between calls (hf_static_cache_graph)",
                      "kernel": "LlamaFusedRuntime: five launches per layer, integer KV cache, one captured step, "
                                "kept between calls (fused_runtime_graph)",
-                     "kernel, kv_cache=bf16": "the kernel-mode model under the HF module walk over a StaticCache "
-                                              "(the reference's arrangement for a weight-only recipe)"},
-           "note": "speedup_vs_bf16 compares two runtimes as well as two precisions: the bf16 side is the HF module "
-                   "walk (about 40 launches per layer), the kernel side the fused runtime. The kv_cache=bf16 row "
-                   "is the quantized weights under the same HF walk as the baseline: what quantization alone buys."}
+                     "kernel_kv_bf16_fused_runtime": "the kernel-mode model under the same fused runtime with its "
+                                                     "cache left at bf16 (the kv_cache=bf16 ablation)",
+                     "kernel_kv_bf16_hf_walk": "the kernel-mode model under the HF module walk over a StaticCache "
+                                               "(the reference's arrangement for a weight-only recipe)"},
+           "note": "speedup_vs_bf16 is kernel / bf16_fused_runtime: both sides run the same five-launch step under "
+                   "graph replay, so it prices the quantization alone. speedup_vs_bf16_hf_walk compares against the "
+                   "HF module walk (about 40 launches per layer) and is mostly the runtime."}
     from llmquant.eval import deployed_cost
 
-    lat_bf16, res["bf16"] = measure(None)
+    lat_bf16_walk, res["bf16_hf_walk"] = measure(None)
+    lat_bf16, res["bf16_fused_runtime"] = measure(16)
     cost_bf16 = deployed_cost(model, None)
+    from llmquant.runtime import drop_kept
+
+    drop_kept(model)
     recipe = QuantConfig(attn_weight="int8", mlp_weight="int4", head_weight="int8", kv_cache="int8")
     oneshot(model, recipe.to_modifier("kernel"))
+    torch.cuda.empty_cache()
     cost_kernel, cost_abl = deployed_cost(model, 8), deployed_cost(model, None)
     lat_kernel, res["kernel"] = measure(8)
-    # ablation row of the verification plan: the selected recipe with the KV cache back at bf16
-    lat_abl, res["kernel_kv_bf16_hf_walk"] = measure(None)
+    # ablation row of the verification plan: the selected recipe with the KV cache back at bf16, under the same
+    # fused runtime, and under the HF walk as the reference arranges it
+    lat_abl, res["kernel_kv_bf16_fused_runtime"] = measure(16)
+    lat_abl_walk, res["kernel_kv_bf16_hf_walk"] = measure(None)
     res["config"] = recipe.describe()
-    res["speedup_vs_bf16"] = round(res["kernel"]["decode_tok_s"] / res["bf16"]["decode_tok_s"], 3)
-    res["speedup_vs_bf16_same_runtime"] = round(res["kernel_kv_bf16_hf_walk"]["decode_tok_s"]
-                                                / res["bf16"]["decode_tok_s"], 3)
-    # the same runs as rows of the reference's report format (eval/run.py, eval/verify.py)
+    res["speedup_vs_bf16"] = round(res["kernel"]["decode_tok_s"] / res["bf16_fused_runtime"]["decode_tok_s"], 3)
+    res["speedup_vs_bf16_hf_walk"] = round(res["kernel"]["decode_tok_s"] / res["bf16_hf_walk"]["decode_tok_s"], 3)
+    res["hf_walk_speedup_of_the_weights_alone"] = round(res["kernel_kv_bf16_hf_walk"]["decode_tok_s"]
+                                                        / res["bf16_hf_walk"]["decode_tok_s"], 3)
+    # the same runs as rows of the reference's report format (eval/run.py, eval/verify.py): the plan's three rows
+    # all under the fused runtime, the two HF-walk runs beside them
     from dataclasses import replace
 
     from llmquant.eval import verification_plan
 
     plan = verification_plan(recipe)
-    measured = {"bf16 baseline": (None, "hf_static_cache_graph", lat_bf16, cost_bf16),
+    measured = {"bf16 baseline": (None, "fused_runtime_graph", lat_bf16, cost_bf16),
                 "selected": (recipe, "fused_runtime_graph", lat_kernel, cost_kernel),
-                "selected, kv_cache=bf16": (replace(recipe, kv_cache="bf16"), "hf_static_cache_graph", lat_abl, cost_abl)}
+                "selected, kv_cache=bf16": (replace(recipe, kv_cache="bf16"), "fused_runtime_graph", lat_abl, cost_abl)}
     rows = [dict(latency_row(*measured[label][:3], cost=measured[label][3]), verify_label=label)
             for label, _ in plan if label in measured]
-    res["verify_rows"] = [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in row.items()} for row in rows]
     res["verify"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in reconcile(rows).items()}
+    rows.append(dict(latency_row(None, "hf_static_cache_graph", lat_bf16_walk, cost=cost_bf16),
+                     verify_label="bf16 baseline, HF module walk"))
+    rows.append(dict(latency_row(replace(recipe, kv_cache="bf16"), "hf_static_cache_graph", lat_abl_walk, cost=cost_abl),
+                     verify_label="selected, kv_cache=bf16, HF module walk"))
+    res["verify_rows"] = [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in row.items()} for row in rows]
     del model
     torch.cuda.empty_cache()
+    if arch == "llama3.2-1b":
+        res["token_identity_first_64"] = token_identity(torch, cfg, recipe, prompt)
     return res
+
+
+def token_identity(torch, cfg, recipe, prompt):
+    """The first 64 greedy tokens, free-running on both sides: graphed_generate (the fused step under graph
+    replay, what the tok/s above is measured on) against the same weights in the package's real mode under HF
+    transformers with the PyTorch-side quantized cache -- on the architecture built in float32 (where the two
+    differ by fp32 summation order only and the streams must be identical) and in bfloat16 (where a random-init
+    model's own logits tie and two correct implementations part at the first near-tie)."""
+    import copy
+
+    from transformers import LlamaForCausalLM
+
+    from llmquant import oneshot
+    from llmquant.quantizers import make_cache_factory
+    from llmquant.runtime import graphed_generate
+
+    out = {}
+    ids = torch.randint(0, cfg.vocab_size, (1, prompt), generator=torch.Generator().manual_seed(1)).to("cuda:0")
+    for tag, dtype in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+        torch.manual_seed(0)
+        model = LlamaForCausalLM(cfg)
+        for p in model.parameters():
+            if p.dim() > 1:
+                torch.nn.init.normal_(p, 0, 0.02)
+        model = model.to(dtype).to("cuda:0").eval()
+        real = oneshot(copy.deepcopy(model), recipe.to_modifier("real"))
+        kernel = oneshot(model, recipe.to_modifier("kernel"))
+        cache = make_cache_factory(8)()
+        want, gaps = [], []
+        with torch.no_grad():
+            logits = real(ids, past_key_values=cache, use_cache=True).logits[0, -1].float()
+            for _ in range(64):
+                top2 = logits.topk(2).values
+                gaps.append((top2[0] - top2[1]).item())
+                tok = logits.argmax().reshape(1, 1)
+                want.append(tok.item())
+                logits = real(tok, past_key_values=cache, use_cache=True).logits[0, -1].float()
+        got = graphed_generate(kernel, ids, 64, kv_bits=8)[0, prompt:].tolist()
+        prefix = next((i for i, (a, b) in enumerate(zip(got, want)) if a != b), 64)
+        out[tag] = {"identical_prefix": prefix, "positions_equal": sum(a == b for a, b in zip(got, want)),
+                    "oracle_min_top2_gap": round(min(gaps), 6),
+                    "oracle_top2_gap_where_the_streams_part": round(gaps[prefix], 6) if prefix < 64 else None}
+        del model, real, kernel, cache
+        torch.cuda.empty_cache()
+    return out
 
 
 def prefill_leg(torch):
@@ -841,9 +930,52 @@ def cpu_baseline(torch, cases, budget_s: float):
               "sample": f"{steps} full steps of the same sweep (same operands) in {elapsed:.1f} s, "
                         f"OpenMP over output rows",
               "cpu": model, "os_cpu_count": os.cpu_count()}
+    result["fake"] = cpu_fake_sweep(torch, cases, min(6.0, budget_s))
     result["w4a8_gemm"] = cpu_w4a8_gemm(torch, olib)
     result["decode"] = cpu_decode(torch)
     return result
+
+
+def cpu_fake_sweep(torch, cases, budget_s: float):
+    """The reference's fake path (llmquant/quantizers/fake.py:18-36: weights quantize-dequantized once and kept
+    in bf16, then F.linear) on the host cores, on the same sweep and the same operands: the package's
+    FakeQuantLinear over the dequantized weight of every shape, torch CPU, all threads torch is given. `value` is
+    in the unit of the GPU figure (the sweep's algorithmic bytes in their quantized form per second); what the
+    host actually streams is the bf16 weight, reported beside it."""
+    from llmquant.core.scheme import QuantizationArgs, QuantizationScheme
+    from llmquant.quantizers import FakeQuantLinear
+
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    layers, bf16_bytes = [], 0
+    for case in cases:
+        q, s = case["bufs"][0]
+        from llmquant.packing.packing import unpack_int4
+
+        codes = unpack_int4(q) if case["bits"] == 4 else q
+        weight = (codes.float() * s[:, :, None]).reshape(case["n"], case["k"]).to(torch.bfloat16).cpu()
+        scheme = QuantizationScheme(weights=QuantizationArgs(case["bits"], "group", group_size=GROUP),
+                                    input_activations=None)
+        layers.append((FakeQuantLinear(weight, None, scheme), case["x"].cpu()))
+        bf16_bytes += weight.numel() * 2
+    step_bytes = sum(c["bytes"] for c in cases)
+
+    def one_step():
+        with torch.no_grad():
+            for layer, x in layers:
+                layer(x)
+
+    one_step()
+    t0 = time.perf_counter()
+    steps = 0
+    while time.perf_counter() - t0 < budget_s:
+        one_step()
+        steps += 1
+    elapsed = time.perf_counter() - t0
+    return {"value": round(step_bytes * steps / elapsed / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "bf16_weight_GBps": round(bf16_bytes * steps / elapsed / 1e9, 2),
+            "sample": f"{steps} full steps of the same sweep through FakeQuantLinear (dequantized bf16 weights + "
+                      f"F.linear, torch CPU) in {elapsed:.1f} s"}
 
 
 def cpu_w4a8_gemm(torch, olib):

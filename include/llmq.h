@@ -338,7 +338,9 @@ int llmq_kv_decode_attention(const void* q, const void* k_codes, const void* v_c
  * t_max as for llmq_kv_decode_attention). Calls no hipMalloc / hipFree and no allocating routine. Every
  * call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams) race; calls on one
  * stream, and calls on different GPUs, are fine. Each call clears the counters first with a one-workgroup
- * fill kernel (not a memset node, so the call can be captured). */
+ * fill kernel (not a memset node, so the call can be captured). The FIRST call on a device looks the array's
+ * address up (hipGetDevice, hipGetSymbolAddress: they may load the code object) and must be made outside
+ * stream capture; every later call on that device launches two kernels and nothing else. */
 int llmq_kv_decode_attention_static(const void* q, const void* k_codes, const void* v_codes,
                                     const float* k_scale, const float* v_scale, void* out,
                                     const int32_t* len_dev, float sm_scale, int q_heads, int kv_heads,
@@ -372,7 +374,10 @@ int llmq_kv_rope_append_attend(const void* qkv, const void* cos_table, const voi
  * core with the cache's codes as operands (the query in three base-256 digits, the softmax weights
  * times the value scales in two): exact integer sums of code * scale, without the rounding of the
  * dequantized K and V to `dtype` that the other forms make as the reference's cache does; the
- * output agrees with them to ~1e-3 relative. */
+ * output agrees with them to ~1e-3 relative.
+ * bits == 16 (this entry point only; dtype fp16 / bf16): an UNQUANTIZED cache, k_codes / v_codes holding
+ * [kv_heads, t_max, head_dim] values of `dtype` (the rotated key and the value as they are; scales written
+ * as 1): the 16-bit baseline's cache under the same step, one query head per workgroup. */
 size_t llmq_kv_attend_partials_floats(int q_heads, int head_dim, int n_splits);
 int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos_table, const void* sin_table,
                                      void* k_codes, void* v_codes, float* k_scale, float* v_scale,
@@ -385,6 +390,19 @@ int llmq_wq_gemv_attn_merge(const float* partials, int n_splits, int head_dim, c
                             const float* wscale, void* out, int N, int G, int out_group, int wformat,
                             int dtype, int in_head_dim, const void* residual_or_null,
                             llmq_stream_t stream);
+
+/* The same decode-step GEMV over an UNQUANTIZED fp16 / bf16 weight [N, K] (row-major), one activation row:
+ *   out[n] = sum_k x'[k] * weight[n, k], fp32 accumulation,
+ * with llmq_wq_gemv_fused's RMSNorm prologue and residual epilogue, llmq_wq_gemv_gate_up_silu's store
+ * (pair_half > 0: weight is gate rows over up rows, N = 2 * pair_half, out [pair_half] = act(gate) * up) and
+ * llmq_wq_gemv_attn_merge's prologue (LLMQ_PRO_ATTN_MERGE: x is the split attention's records, attn_splits per
+ * head of attn_head_dim), each with the same rounding points. It has no counterpart among the reference's
+ * kernels: it is what lets the 16-bit baseline run through the same five-launch decode step as the quantized
+ * model, as the reference times both sides under one runtime (llmquant/eval/verify.py:44-47).
+ * K a multiple of 8, at most 28672; pointers 16-byte aligned; dtype LLMQ_F16 or LLMQ_BF16. */
+int llmq_dense_gemv_fused(const void* x, const void* weight, void* out, int N, int K, int dtype, int prologue,
+                          const void* norm_weight, float eps, const void* residual, int pair_half,
+                          int attn_splits, int attn_head_dim, llmq_stream_t stream);
 
 /* Index of the first maximum of a row of n elements, written to *out_index on the device: the
  * greedy sampler of the decode loop (the reference calls logits.argmax(-1),

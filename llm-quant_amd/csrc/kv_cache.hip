@@ -236,6 +236,25 @@ __device__ __forceinline__ void decode_raw(const RawCodes<BITS, DPL>& r, float* 
   }
 }
 
+// BITS == 16: the cache holds the values themselves in the model's 16-bit type T (the unquantized cache of a
+// 16-bit baseline run through the same step); "decoding" is the conversion to float and the scale is 1.
+template <typename T, int DPL>
+__device__ __forceinline__ void decode_values16(const RawCodes<16, DPL>& r, float* c) {
+#pragma unroll
+  for (int i = 0; i < DPL / 8; ++i) {
+    Pack<T>::unpack(u32x4{r.w[4 * i], r.w[4 * i + 1], r.w[4 * i + 2], r.w[4 * i + 3]}, c + 8 * i);
+  }
+}
+template <typename T, int BITS, int DPL>
+__device__ __forceinline__ void decode_cache_row(const RawCodes<BITS, DPL>& r, float* c) {
+  if constexpr (BITS == 16) {
+    static_assert(sizeof(T) == 2, "an unquantized cache holds 16-bit values");
+    decode_values16<T, DPL>(r, c);
+  } else {
+    decode_raw<BITS, DPL>(r, c);
+  }
+}
+
 // One step's operands of attend_range, for callers that can request the first steps early.
 template <int BITS, int DPL> struct AttnPrefetch {
   RawCodes<BITS, DPL> k, v;
@@ -274,7 +293,6 @@ __device__ __forceinline__ void attend_range(const float (*qf)[D / 4], const uin
                                              float* m, float* l, float (*o)[D / 4],
                                              const AttnPrefetch<BITS, D / 4>* first = nullptr, int t_clamp = -1) {
   constexpr int DPL = D / 4;
-  constexpr int ROWB = BITS == 8 ? D : D / 2;
 #pragma unroll
   for (int h = 0; h < REP; ++h) {
     m[h] = -INFINITY;
@@ -305,8 +323,8 @@ __device__ __forceinline__ void attend_range(const float (*qf)[D / 4], const uin
       ring[r] = attn_prefetch<BITS, DPL>(kbase, vbase, ksc, vsc, min(t0 + NPRE * t_step + tk, t_clamp), dq);
     }
     float kc[DPL], vc[DPL];
-    decode_raw<BITS, DPL>(k_now, kc);
-    decode_raw<BITS, DPL>(v_now, vc);
+    decode_cache_row<T, BITS, DPL>(k_now, kc);
+    decode_cache_row<T, BITS, DPL>(v_now, vc);
     float s[REP];
 #pragma unroll
     for (int h = 0; h < REP; ++h) s[h] = 0.0f;
@@ -557,11 +575,24 @@ __global__ __launch_bounds__(kFusedThreads) void kv_rope_append_attend_kernel(
       f[e] = 0.0f;
       if (d < D) f[e] = is_v ? to_float(src[d]) : rope_element<T, D>(src, cos_row, sin_row, d);
     }
+    const int64_t slot = static_cast<int64_t>(kvh) * t_max + pos;
+    uint8_t* codes = is_v ? v_codes : k_codes;
+    if constexpr (BITS == 16) {
+      // the unquantized cache: the rotated key / the value as the model's dtype holds them, scale 1
+      if (writer && lane == 0) (is_v ? v_scale : k_scale)[slot] = 1.0f;
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int d = lane + e * kWave;
+        if (d < D) {
+          s_new[is_v ? 1 : 0][d] = f[e];   // (already a value of T: RoPE rounds its result, V is read as T)
+          if (writer) reinterpret_cast<T*>(codes)[slot * D + d] = from_float<T>(f[e]);
+        }
+      }
+      return;
+    }
     const float amax = group_max<kWave>(fmaxf(fabsf(f[0]), fabsf(f[1])));
     const float scale = scale_from_amax(amax, qmax);
-    const int64_t slot = static_cast<int64_t>(kvh) * t_max + pos;
     if (writer && lane == 0) (is_v ? v_scale : k_scale)[slot] = scale;
-    uint8_t* codes = is_v ? v_codes : k_codes;
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
       const int d = lane + e * kWave;
@@ -570,7 +601,7 @@ __global__ __launch_bounds__(kFusedThreads) void kv_rope_append_attend_kernel(
       const int code = static_cast<int>(qv);
       if constexpr (BITS == 8) {
         if (writer && d < D) codes[slot * D + d] = static_cast<uint8_t>(code);
-      } else {
+      } else if constexpr (BITS == 4) {
         const int mine = (code + 8) & 0xf;
         const int other = dpp<kDppXor1>(mine);
         if (writer && (lane & 1) == 0 && d < D) codes[slot * (D / 2) + d / 2] = static_cast<uint8_t>(mine | (other << 4));
@@ -667,11 +698,24 @@ __device__ __forceinline__ void split_phase_a(const T* __restrict__ qkv, const T
       f[e] = 0.0f;
       if (d < D) f[e] = is_v ? to_float(src[d]) : rope_element<T, D>(src, cos_row, sin_row, d);
     }
+    const int64_t slot = static_cast<int64_t>(kvh) * t_max + pos;
+    uint8_t* codes = is_v ? v_codes : k_codes;
+    if constexpr (BITS == 16) {
+      // the unquantized cache: the rotated key / the value as the model's dtype holds them, scale 1
+      if (writer && lane == 0) (is_v ? v_scale : k_scale)[slot] = 1.0f;
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int d = lane + e * kWave;
+        if (d < D) {
+          s_new[is_v ? 1 : 0][d] = f[e];   // (already a value of T: RoPE rounds its result, V is read as T)
+          if (writer) reinterpret_cast<T*>(codes)[slot * D + d] = from_float<T>(f[e]);
+        }
+      }
+      return;
+    }
     const float amax = group_max<kWave>(fmaxf(fabsf(f[0]), fabsf(f[1])));
     const float scale = scale_from_amax(amax, qmax);
-    const int64_t slot = static_cast<int64_t>(kvh) * t_max + pos;
     if (writer && lane == 0) (is_v ? v_scale : k_scale)[slot] = scale;
-    uint8_t* codes = is_v ? v_codes : k_codes;
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
       const int d = lane + e * kWave;
@@ -680,7 +724,7 @@ __device__ __forceinline__ void split_phase_a(const T* __restrict__ qkv, const T
       const int code = static_cast<int>(qv);
       if constexpr (BITS == 8) {
         if (writer && d < D) codes[slot * D + d] = static_cast<uint8_t>(code);
-      } else {
+      } else if constexpr (BITS == 4) {
         const int mine = (code + 8) & 0xf;
         const int other = dpp<kDppXor1>(mine);
         if (writer && (lane & 1) == 0 && d < D) codes[slot * (D / 2) + d / 2] = static_cast<uint8_t>(mine | (other << 4));
@@ -700,7 +744,7 @@ __global__ __launch_bounds__(kSplitThreads) void kv_rope_append_attend_split_ker
     float* __restrict__ v_scale, float* __restrict__ partials, const int32_t* __restrict__ pos_dev,
     const float sm_scale_log2, const int q_heads, const int kv_heads, const int t_max) {
   constexpr int DPL = D / 4;
-  constexpr int ROWB = BITS == 8 ? D : D / 2;
+  constexpr int ROWB = D * BITS / 8;
   constexpr int REC = D + 2;                    // per-wave record in LDS
   constexpr int GREC = D + kAttnRecordHeader;  // per-split record in global memory
   __shared__ float s_q[HEADS][D];
@@ -1516,9 +1560,9 @@ constexpr int kStaticCounters = 256;  // >= kStaticMaxQHeads, and a whole number
 constexpr size_t kStaticPartFloats = static_cast<size_t>(kStaticMaxQHeads) * 64 * (128 + 2);
 static __device__ __align__(256) float g_attn_scratch[kStaticCounters + kStaticPartFloats];
 
+namespace {
 __global__ void clear_counters_kernel(int* __restrict__ count) { count[threadIdx.x] = 0; }
 
-namespace {
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 float* g_scratch_ptr[kMaxDevices] = {};
@@ -1704,7 +1748,10 @@ extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos
                                                 float* partials, const int32_t* pos_dev, float sm_scale,
                                                 int q_heads, int kv_heads, int head_dim, int t_max, int bits,
                                                 int n_splits, int dtype, llmq_stream_t stream) {
-  if (bits != 8 && bits != 4) return llmq_host::fail_invalid("KV cache bits must be 8 or 4, got %d", bits);
+  if (bits != 8 && bits != 4 && bits != 16)
+    return llmq_host::fail_invalid("KV cache bits must be 8 or 4 (or 16: an unquantized cache of the model's dtype), got %d", bits);
+  if (bits == 16 && dtype != LLMQ_F16 && dtype != LLMQ_BF16)
+    return llmq_host::fail_invalid("an unquantized cache (bits 16) holds float16 or bfloat16 values, got dtype code %d", dtype);
   if (head_dim != 64 && head_dim != 128) return llmq_host::fail_invalid("head_dim must be 64 or 128, got %d", head_dim);
   if (kv_heads <= 0 || q_heads <= 0 || q_heads % kv_heads)
     return llmq_host::fail_invalid("q_heads %d must be a positive multiple of kv_heads %d", q_heads, kv_heads);
@@ -1725,7 +1772,8 @@ extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos
   // (heads of 128: the vector-ALU form has twice the arithmetic per cache row, and the matrix-core form is ahead at every
   // cache length: the Llama-3-8B architecture's step at 600 cached tokens, 1968 us a token against 2038)
   const int mf_min_cache = head_dim == 128 ? 0 : kMfMinCache;
-  const bool grouped = rep_heads % 4 == 0 && (n_splits >= 32 || (n_splits >= 8 && t_max >= mf_min_cache));
+  // (the unquantized cache keeps the one-head form: it is the baseline's step, not a path to tune)
+  const bool grouped = bits != 16 && rep_heads % 4 == 0 && (n_splits >= 32 || (n_splits >= 8 && t_max >= mf_min_cache));
   const dim3 grid(grouped ? q_heads / 4 : q_heads, n_splits), block(kSplitThreads);
   if (grouped && t_max >= mf_min_cache) {
     // long caches: the matrix-core form (see the kernel's comment for what it changes in the arithmetic)
@@ -1782,6 +1830,27 @@ extern "C" int llmq_kv_rope_append_attend_split(const void* qkv, const void* cos
   if (bits == 8) { if (head_dim == 64) LLMQ_SPLIT(T, 8, 64); else LLMQ_SPLIT(T, 8, 128); }             \
   else { if (head_dim == 64) LLMQ_SPLIT(T, 4, 64); else LLMQ_SPLIT(T, 4, 128); }                       \
   break;
+#define LLMQ_SPLIT_16(T)                                                                               \
+  do {                                                                                                 \
+    if (head_dim == 64) {                                                                              \
+      hipLaunchKernelGGL((kv_rope_append_attend_split_kernel<T, 16, 64, 1>), grid, block, 0, s,        \
+                         static_cast<const T*>(qkv), static_cast<const T*>(cos_table),                 \
+                         static_cast<const T*>(sin_table), static_cast<uint8_t*>(k_codes),             \
+                         static_cast<uint8_t*>(v_codes), k_scale, v_scale, partials, pos_dev,          \
+                         scale_log2, q_heads, kv_heads, t_max);                                        \
+    } else {                                                                                           \
+      hipLaunchKernelGGL((kv_rope_append_attend_split_kernel<T, 16, 128, 1>), grid, block, 0, s,       \
+                         static_cast<const T*>(qkv), static_cast<const T*>(cos_table),                 \
+                         static_cast<const T*>(sin_table), static_cast<uint8_t*>(k_codes),             \
+                         static_cast<uint8_t*>(v_codes), k_scale, v_scale, partials, pos_dev,          \
+                         scale_log2, q_heads, kv_heads, t_max);                                        \
+    }                                                                                                  \
+  } while (0)
+  if (bits == 16) {
+    if (dtype == LLMQ_F16) LLMQ_SPLIT_16(f16_t); else LLMQ_SPLIT_16(bf16_t);
+    return llmq_host::check_launch("kv_rope_append_attend_split_kernel");
+  }
+#undef LLMQ_SPLIT_16
   switch (dtype) {
     case LLMQ_F32: LLMQ_SPLIT_BD(float)
     case LLMQ_F16: LLMQ_SPLIT_BD(f16_t)

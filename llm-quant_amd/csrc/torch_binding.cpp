@@ -813,12 +813,14 @@ CacheGeometry cache_geometry(const at::Tensor& codes, const at::Tensor& scale, c
   TORCH_CHECK(codes.is_cuda() && scale.is_cuda(), what, " cache tensors must be CUDA");
   TORCH_CHECK(codes.dim() == 3 && codes.is_contiguous(), what, " codes must be contiguous [kv_heads, t_max, head_dim]");
   const bool packed = codes.scalar_type() == at::kByte;
-  TORCH_CHECK(packed || codes.scalar_type() == at::kChar, what, " codes must be int8, or uint8 for 4-bit");
+  // (fp16 / bf16 "codes": an unquantized cache, bits 16, which only the split attention step takes)
+  const bool unquantized = codes.scalar_type() == at::kHalf || codes.scalar_type() == at::kBFloat16;
+  TORCH_CHECK(packed || unquantized || codes.scalar_type() == at::kChar, what, " codes must be int8, or uint8 for 4-bit");
   TORCH_CHECK(scale.scalar_type() == at::kFloat && scale.is_contiguous() && scale.dim() == 2 &&
                   scale.size(0) == codes.size(0) && scale.size(1) == codes.size(1),
               what, " scales must be contiguous float32 [kv_heads, t_max]");
   return {static_cast<int>(codes.size(0)), static_cast<int>(codes.size(1)),
-          static_cast<int>(packed ? codes.size(2) * 2 : codes.size(2)), packed ? 4 : 8};
+          static_cast<int>(packed ? codes.size(2) * 2 : codes.size(2)), unquantized ? 16 : (packed ? 4 : 8)};
 }
 
 void check_position(const at::Tensor& position) {
@@ -1012,6 +1014,8 @@ at::Tensor kv_rope_append_attend_split(const at::Tensor& qkv, const at::Tensor& 
                 "cos/sin tables must be contiguous [>= t_max, head_dim] tensors of qkv's dtype");
   }
   check_position(position);
+  TORCH_CHECK(g.bits != 16 || k_codes.scalar_type() == qkv.scalar_type(),
+              "an unquantized cache must hold values of qkv's dtype");
   TORCH_CHECK(n_splits >= 1 && n_splits <= 256, "n_splits must be in [1, 256], got ", n_splits);
   const auto need = static_cast<int64_t>(llmq_kv_attend_partials_floats(static_cast<int>(q_heads), g.head_dim,
                                                                         static_cast<int>(n_splits)));
@@ -1086,6 +1090,57 @@ at::Tensor wq_gemv_attn_merge(const at::Tensor& partials, int64_t n_splits, int6
                                    packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype, static_cast<int>(in_head_dim),
                                    res_ptr, current_stream(partials)),
            "wq_gemv_attn_merge");
+  return out;
+}
+
+// The decode-step GEMV over an unquantized fp16 / bf16 weight [N, K] (the 16-bit baseline's kernel).
+// prologue 0 / 1 (RMSNorm): x is [1, K]; prologue 3 (attention merge): x is the fp32 records of split
+// attention, n_splits per head of head_dim. pair_half > 0: weight is gate rows over up rows, out [1, pair_half].
+at::Tensor dense_gemv_fused(const at::Tensor& x, const at::Tensor& weight, int64_t prologue,
+                            const c10::optional<at::Tensor>& norm_weight, double eps,
+                            const c10::optional<at::Tensor>& residual, int64_t pair_half, int64_t n_splits,
+                            int64_t head_dim) {
+  TORCH_CHECK(x.is_cuda() && weight.is_cuda(), "x and weight must be CUDA tensors");
+  TORCH_CHECK(weight.dim() == 2 && weight.is_contiguous(), "weight must be contiguous [N, K]");
+  TORCH_CHECK(weight.scalar_type() == at::kHalf || weight.scalar_type() == at::kBFloat16,
+              "weight must be float16 or bfloat16");
+  TORCH_CHECK(x.is_contiguous(), "x must be contiguous");
+  const int64_t N = weight.size(0), K = weight.size(1);
+  const bool merge = prologue == LLMQ_PRO_ATTN_MERGE;
+  if (merge) {
+    TORCH_CHECK(x.scalar_type() == at::kFloat && head_dim > 0 && K % head_dim == 0 && n_splits >= 1 &&
+                    x.numel() >= static_cast<int64_t>(llmq_kv_attend_partials_floats(
+                                     static_cast<int>(K / head_dim), static_cast<int>(head_dim), static_cast<int>(n_splits))),
+                "the attention-merge prologue takes the float32 records of ", K / std::max<int64_t>(head_dim, 1), " heads x ",
+                n_splits, " splits");
+  } else {
+    TORCH_CHECK(x.scalar_type() == weight.scalar_type() && x.numel() == K, "x must be [1, ", K, "] of the weight's dtype");
+  }
+  const void* norm_ptr = nullptr;
+  if (prologue == LLMQ_PRO_RMSNORM) {
+    TORCH_CHECK(norm_weight.has_value() && norm_weight->defined() && norm_weight->is_cuda() &&
+                    norm_weight->is_contiguous() && norm_weight->numel() == K &&
+                    norm_weight->scalar_type() == weight.scalar_type(),
+                "the RMSNorm prologue needs norm_weight [", K, "] of the weight's dtype");
+    norm_ptr = norm_weight->const_data_ptr();
+  }
+  const int64_t n_out = pair_half > 0 ? pair_half : N;
+  const void* res_ptr = nullptr;
+  if (residual.has_value() && residual->defined()) {
+    TORCH_CHECK(residual->is_cuda() && residual->is_contiguous() && residual->numel() == n_out &&
+                    residual->scalar_type() == weight.scalar_type(),
+                "residual must be a contiguous tensor of the weight's dtype with ", n_out, " elements");
+    res_ptr = residual->const_data_ptr();
+  }
+  auto out = at::empty({1, n_out}, weight.options());
+  const int dtype = dtype_code(weight, "weight");
+  if (N == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(weight));
+  check_rc(llmq_dense_gemv_fused(x.const_data_ptr(), weight.const_data_ptr(), out.mutable_data_ptr(),
+                                 static_cast<int>(N), static_cast<int>(K), dtype, static_cast<int>(prologue), norm_ptr,
+                                 static_cast<float>(eps), res_ptr, static_cast<int>(pair_half),
+                                 static_cast<int>(n_splits), static_cast<int>(head_dim), current_stream(weight)),
+           "dense_gemv_fused");
   return out;
 }
 
@@ -1272,6 +1327,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     return static_cast<int64_t>(llmq_kv_attend_partials_floats(static_cast<int>(q_heads), static_cast<int>(head_dim),
                                                                static_cast<int>(n_splits)));
   }, py::arg("q_heads"), py::arg("head_dim"), py::arg("n_splits"));
+  m.def("dense_gemv_fused", &dense_gemv_fused, py::arg("x"), py::arg("weight"), py::arg("prologue") = 0,
+        py::arg("norm_weight") = py::none(), py::arg("eps") = 0.0, py::arg("residual") = py::none(),
+        py::arg("pair_half") = 0, py::arg("n_splits") = 0, py::arg("head_dim") = 0,
+        "Decode-step GEMV over an unquantized fp16 / bf16 weight with the fused step's prologues and epilogues");
   m.def("kv_rope_append_attend_split", &kv_rope_append_attend_split,
         "RoPE + quantize-append + attention spread over n_splits workgroups per head; fills and returns partials",
         py::arg("qkv"), py::arg("cos_table"), py::arg("sin_table"), py::arg("k_codes"), py::arg("v_codes"),

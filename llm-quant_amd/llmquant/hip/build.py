@@ -107,6 +107,8 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_kv_attend_merge.restype = c_int
     lib.llmq_wq_gemv_attn_merge.argtypes = [c_p, c_int, c_int, c_p, c_p, c_p] + [c_int] * 6 + [c_p, c_p]
     lib.llmq_wq_gemv_attn_merge.restype = c_int
+    lib.llmq_dense_gemv_fused.argtypes = [c_p, c_p, c_p, c_int, c_int, c_int, c_int, c_p, c_f, c_p, c_int, c_int, c_int, c_p]
+    lib.llmq_dense_gemv_fused.restype = c_int
     lib.llmq_argmax_row.argtypes = [c_p, c_int, c_p, c_int, c_p]
     lib.llmq_argmax_row.restype = c_int
     lib.llmq_argmax_advance.argtypes = [c_p, c_int, c_p, c_p, c_p, c_p, c_int, c_p]

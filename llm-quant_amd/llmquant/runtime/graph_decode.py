@@ -18,7 +18,7 @@ from __future__ import annotations
 import torch
 
 from llmquant.runtime.llama_decode import WARMUP_CALLS, LlamaKernelRuntime
-from llmquant.runtime.llama_fused import LlamaFusedRuntime
+from llmquant.runtime.llama_fused import LlamaDenseFusedRuntime, LlamaFusedRuntime
 
 __all__ = ["GraphedDecoder", "KernelDecoder", "WARMUP_CALLS", "can_graph", "drop_kept", "graphed_generate",
            "kept_graphed_decoder", "kept_kernel_runtime", "kernel_runtime"]
@@ -101,6 +101,13 @@ class GraphedDecoder:
 def kernel_runtime(model, max_len: int, kv_bits: int = 8):
     """The fastest runtime the model qualifies for: the five-launches-per-layer fused step when
     every Linear is a weight-only kernel-mode module, else the operation-by-operation walk."""
+    if kv_bits == 16:
+        # an unquantized cache: the 16-bit baseline through the same fused step (plain nn.Linear modules), or
+        # a kernel-mode model with its cache left at the model's dtype (the kv_cache=bf16 ablation)
+        try:
+            return LlamaDenseFusedRuntime(model, max_len, 16)
+        except ValueError:
+            return LlamaFusedRuntime(model, max_len, 16)
     try:
         return LlamaFusedRuntime(model, max_len, kv_bits)
     except ValueError:

@@ -20,25 +20,29 @@ from llmquant.hip.build import load_extension
 class KernelQuantCache:
     """K/V codes and scales for every layer of one sequence (batch 1).
 
-    num_bits   8 (int8 codes) or 4 (nibble-packed)
+    num_bits   8 (int8 codes) or 4 (nibble-packed); 16: an unquantized cache of `dtype` values (the 16-bit
+               baseline run through the same decode step; only the fused step's attention launch reads it)
     position   device int32 [1]: where the next token is written
     length     device int32 [1]: tokens valid for attention (position + tokens being added)
     """
 
     def __init__(self, num_layers: int, kv_heads: int, head_dim: int, max_len: int, num_bits: int = 8,
-                 q_heads: int | None = None, device="cuda"):
-        if num_bits not in (4, 8):
-            raise ValueError(f"KV cache bits must be 4 or 8, got {num_bits}")
+                 q_heads: int | None = None, device="cuda", dtype=torch.bfloat16):
+        if num_bits not in (4, 8, 16):
+            raise ValueError(f"KV cache bits must be 4 or 8 (or 16 for an unquantized cache), got {num_bits}")
+        if num_bits == 16 and dtype not in (torch.bfloat16, torch.float16):
+            raise ValueError("an unquantized cache holds bfloat16 or float16 values")
         self.num_bits, self.num_layers = num_bits, num_layers
         self.kv_heads, self.head_dim, self.max_len = kv_heads, head_dim, max_len
         self._ext = load_extension()
-        width = head_dim if num_bits == 8 else head_dim // 2
-        code_dtype = torch.int8 if num_bits == 8 else torch.uint8
+        width = head_dim // 2 if num_bits == 4 else head_dim
+        code_dtype = {8: torch.int8, 4: torch.uint8, 16: dtype}[num_bits]
         shape = (num_layers, kv_heads, max_len, width)
         self.k_codes = torch.zeros(shape, dtype=code_dtype, device=device)
         self.v_codes = torch.zeros(shape, dtype=code_dtype, device=device)
-        self.k_scale = torch.zeros(num_layers, kv_heads, max_len, dtype=torch.float32, device=device)
-        self.v_scale = torch.zeros(num_layers, kv_heads, max_len, dtype=torch.float32, device=device)
+        fill = torch.ones if num_bits == 16 else torch.zeros
+        self.k_scale = fill(num_layers, kv_heads, max_len, dtype=torch.float32, device=device)
+        self.v_scale = fill(num_layers, kv_heads, max_len, dtype=torch.float32, device=device)
         self.position = torch.zeros(1, dtype=torch.int32, device=device)
         self.length = torch.zeros(1, dtype=torch.int32, device=device)
         q_heads = q_heads or kv_heads
@@ -65,6 +69,8 @@ class KernelQuantCache:
 
     def bytes_per_token(self) -> int:
         """Codes + scales stored per cached token over all layers, K and V."""
+        if self.num_bits == 16:
+            return 2 * self.num_layers * self.kv_heads * self.head_dim * 2
         width = self.head_dim if self.num_bits == 8 else self.head_dim // 2
         return 2 * self.num_layers * self.kv_heads * (width + 4)
 
@@ -73,6 +79,13 @@ class KernelQuantCache:
         """key / value: [kv_heads, n_new, head_dim] (any strides with a contiguous last axis).
         Writes at position .. position + n_new - 1. With return_dequantized, hands back what
         FakeQuantCache.update would have returned for these tokens."""
+        if self.num_bits == 16:
+            # the unquantized cache: a copy at the host-side position (prompt passes only; the fused decode step
+            # appends inside its attention launch)
+            start, stop = self._host_length, self._host_length + key.shape[1]
+            self.k_codes[layer][:, start:stop] = key
+            self.v_codes[layer][:, start:stop] = value
+            return (key.contiguous(), value.contiguous()) if return_dequantized else (None, None)
         return self._ext.kv_append(key, value, self.k_codes[layer], self.v_codes[layer], self.k_scale[layer],
                                    self.v_scale[layer], self.position, return_dequantized)
 

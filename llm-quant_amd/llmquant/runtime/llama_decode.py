@@ -55,7 +55,8 @@ class LlamaKernelRuntime:
         # RMSNorm, RoPE and SiLU * up as one launch each (16-bit models); False walks the PyTorch modules
         self._one_launch_ops = self.dtype in (torch.bfloat16, torch.float16)
         self.cache = KernelQuantCache(len(self.layers), self.kv_heads, self.head_dim, max_len, kv_bits,
-                                      q_heads=self.q_heads, device=self.device)
+                                      q_heads=self.q_heads, device=self.device,
+                                      **({"dtype": self.dtype} if kv_bits == 16 else {}))
         # cos / sin for every position, computed the way LlamaRotaryEmbedding.forward does
         # (fp32 outer product, cat, cos/sin, attention_scaling, cast) so lookups equal recomputation
         rope = model.model.rotary_emb
@@ -119,7 +120,8 @@ class LlamaKernelRuntime:
     def _rope_append_in_one_launch(self, q, k, v, cos):
         """RoPE and the cache append of a prompt as one launch (llmq_rope_kv_append): stock rotation,
         heads of 64 or 128, rows of the projections with a contiguous last axis."""
-        return (self._one_launch_ops and self.head_dim in (64, 128) and q.dtype == cos.dtype and cos.is_contiguous()
+        return (self._one_launch_ops and self.cache.num_bits != 16 and self.head_dim in (64, 128)
+                and q.dtype == cos.dtype and cos.is_contiguous()
                 and all(t.dim() == 2 and t.stride(1) == 1 for t in (q, k, v)))
 
     def _qkv(self, index, layer, x):

@@ -27,7 +27,7 @@ from llmquant.hip.build import load_extension
 from llmquant.quantizers.kernel import KernelQuantLinear
 from llmquant.runtime.llama_decode import LlamaKernelRuntime
 
-PRO_NONE, PRO_RMSNORM, PRO_SILU_MUL = 0, 1, 2
+PRO_NONE, PRO_RMSNORM, PRO_SILU_MUL, PRO_ATTN_MERGE = 0, 1, 2, 3
 
 
 def _fusable(*mods) -> bool:
@@ -109,6 +109,13 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
                 attn_splits = 32
             else:
                 attn_splits = max(short, min(16, (max_len + 2047) // 2048 * 4))
+        if kv_bits == 16:
+            # an unquantized cache of the model's dtype (the kv_cache=bf16 ablation under this runtime): only the
+            # split attention launch reads it, one regime
+            if self.dtype not in (torch.bfloat16, torch.float16):
+                raise ValueError("an unquantized cache needs a bfloat16 or float16 model")
+            self.regimes = None
+            attn_splits = max(2, min(int(attn_splits), 16))
         self.attn_splits = int(attn_splits)
         self._splits_now = self.attn_splits
         self._graphs = {}            # split count -> (graph, logits, next_token)
@@ -144,15 +151,21 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         head = model.lm_head
         if not _fusable(head):
             raise ValueError("the fused decode step needs a kernel-mode lm_head")
+        self._init_token_pick(model, head.qdata.shape[0])
+
+    def _init_token_pick(self, model, head_rows: int):
+        """The final norm's weight and what the token pick at the end of a step needs."""
         self.final_norm = model.model.norm.weight.detach().contiguous()
         self.final_eps = model.model.norm.variance_epsilon
         # The launch that picks a step's token also looks up that token's embedding for the next step
         # (llmq_argmax_advance_embed), so a step starts at its first GEMV. Plain nn.Embedding tables of the
         # model's dtype only; anything else keeps the embedding module's own launch.
         table = model.model.embed_tokens
+        # (and of the logits' dtype, which is the model's: _forward and _step must take the same branch)
         plain = (type(table) is torch.nn.Embedding and table.max_norm is None and table.weight.is_contiguous()
                  and table.weight.dtype in (torch.bfloat16, torch.float16, torch.float32)
-                 and table.weight.shape[1] % 8 == 0 and table.weight.shape[0] >= head.qdata.shape[0])
+                 and table.weight.dtype == self.dtype
+                 and table.weight.shape[1] % 8 == 0 and table.weight.shape[0] >= head_rows)
         self._embed_table = table.weight.detach() if plain else None
         self._hidden0 = torch.zeros(1, table.weight.shape[1], dtype=table.weight.dtype, device=self.device)
         self._argmax_ws = torch.zeros(self._ext.argmax_workspace_ints(), dtype=torch.int32, device=self.device)
@@ -293,9 +306,87 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
     def _step(self):
         logits = self._forward(self.token, None, None, decode=True)
         # greedy pick, next input token, both position counters and the next step's embedding row in one launch
-        if self._embed_table is not None and logits.dtype == self._embed_table.dtype:
+        if self._embed_table is not None:
             nxt = self._ext.argmax_advance_embed(logits, self.token, self.pos_index, self.cache.position,
                                                  self._embed_table, self._hidden0, self._argmax_ws)
         else:
             nxt = self._ext.argmax_advance(logits, self.token, self.pos_index, self.cache.position)
         return logits, nxt
+
+
+class LlamaDenseFusedRuntime(LlamaFusedRuntime):
+    """The same five-launch decode step for a model whose Linears are plain 16-bit nn.Linear modules, over an
+    unquantized cache of the model's dtype (kv_bits 16): the baseline's runtime. The reference times the
+    bf16 model and the quantized one under one runtime (llmquant/eval/verify.py:44-47); this is what makes
+    that possible here, where the quantized side's runtime is the fused step. Launch for launch it is
+    LlamaFusedRuntime's step with llmq_dense_gemv_fused in place of the quantized GEMVs; the prompt pass is the
+    walk's, with the library's matmuls over the concatenated weights."""
+
+    def __init__(self, model, max_len: int, kv_bits: int = 16, exact_prefill: bool = False, attn_splits=None):
+        if kv_bits != 16:
+            raise ValueError("the 16-bit baseline's fused step runs over an unquantized cache (kv_bits 16)")
+        LlamaKernelRuntime.__init__(self, model, max_len, 16, exact_prefill)
+        if self.dtype not in (torch.bfloat16, torch.float16):
+            raise ValueError("the dense fused decode step takes bfloat16 or float16 models")
+        self._ext = load_extension()
+        self.regimes = None
+        # (the o_proj launch merges split-attention records: at least two splits)
+        self.attn_splits = int(attn_splits or max(2, 256 // max(self.q_heads, 1)))
+        self._splits_now = self.attn_splits
+        self._graphs = {}
+        self._partials = torch.zeros(self._ext.kv_attend_partials_floats(self.q_heads, self.head_dim, self.attn_splits),
+                                     dtype=torch.float32, device=self.device)
+
+        def plain(*mods):
+            return all(type(m) is torch.nn.Linear and m.bias is None and m.weight.dtype == self.dtype
+                       and m.weight.shape[1] % 8 == 0 for m in mods)
+
+        self.fused_layers = []
+        for layer in self.layers:
+            attn, mlp = layer.self_attn, layer.mlp
+            if not plain(attn.q_proj, attn.k_proj, attn.v_proj, attn.o_proj, mlp.gate_proj, mlp.up_proj, mlp.down_proj):
+                raise ValueError("the dense fused decode step needs plain 16-bit nn.Linear modules without bias")
+            if "SiLU" not in type(mlp.act_fn).__name__:
+                raise ValueError("the dense fused decode step computes SiLU(gate) * up")
+            cat = lambda *mods: torch.cat([m.weight.detach() for m in mods], dim=0).contiguous()
+            self.fused_layers.append(dict(
+                qkv=cat(attn.q_proj, attn.k_proj, attn.v_proj), gate_up=cat(mlp.gate_proj, mlp.up_proj),
+                o=attn.o_proj.weight.detach().contiguous(), down=mlp.down_proj.weight.detach().contiguous(),
+                inter=mlp.gate_proj.weight.shape[0],
+                norm1=layer.input_layernorm.weight.detach().contiguous(), eps1=layer.input_layernorm.variance_epsilon,
+                norm2=layer.post_attention_layernorm.weight.detach().contiguous(),
+                eps2=layer.post_attention_layernorm.variance_epsilon))
+        if not plain(model.lm_head):
+            raise ValueError("the dense fused decode step needs a plain 16-bit lm_head")
+        self.head_weight = model.lm_head.weight.detach().contiguous()
+        self._init_token_pick(model, self.head_weight.shape[0])
+
+    # the prompt pass: the library's matmuls, q|k|v and gate|up over the concatenated weights
+    def _qkv(self, index, layer, x):
+        out = x @ self.fused_layers[index]["qkv"].T
+        q_width, kv_width = self.q_heads * self.head_dim, self.kv_heads * self.head_dim
+        return out[:, :q_width], out[:, q_width:q_width + kv_width], out[:, q_width + kv_width:]
+
+    def _gate_up(self, index, layer, x):
+        out = x @ self.fused_layers[index]["gate_up"].T
+        half = out.shape[1] // 2
+        return out[:, :half], out[:, half:]
+
+    def _mlp(self, index, layer, x):
+        return LlamaKernelRuntime._mlp(self, index, layer, x)
+
+    def _forward(self, token_ids, cos, sin, decode: bool):
+        if not decode:
+            return LlamaKernelRuntime._forward(self, token_ids, cos, sin, decode)
+        ext, cache, splits = self._ext, self.cache, self._splits_now
+        gemv = ext.dense_gemv_fused
+        hidden = self._hidden0 if self._embed_table is not None else self.model.model.embed_tokens(token_ids)
+        for index, f in enumerate(self.fused_layers):
+            qkv = gemv(hidden, f["qkv"], PRO_RMSNORM, f["norm1"], f["eps1"])
+            ext.kv_rope_append_attend_split(qkv, self.cos_table, self.sin_table, cache.k_codes[index],
+                                            cache.v_codes[index], cache.k_scale[index], cache.v_scale[index],
+                                            self._partials, cache.position, self.scaling, self.q_heads, splits)
+            hidden = gemv(self._partials, f["o"], PRO_ATTN_MERGE, None, 0.0, hidden, 0, splits, self.head_dim)
+            act = gemv(hidden, f["gate_up"], PRO_RMSNORM, f["norm2"], f["eps2"], None, f["inter"])
+            hidden = gemv(act, f["down"], PRO_NONE, None, 0.0, hidden)
+        return gemv(hidden, self.head_weight, PRO_RMSNORM, self.final_norm, self.final_eps)

@@ -12,6 +12,7 @@ import torch
 pytestmark = pytest.mark.gpu
 
 DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+_WARMED = []   # non-empty once the entry point has run on the device
 
 
 def make_case(ext, q_heads, kv_heads, d, t_max, length, bits, dtype, seed):
@@ -42,9 +43,15 @@ def both_ways(lib, ext, q_heads, kv_heads, d, t_max, length, bits, dtype, seed):
     rc = lib.llmq_kv_decode_attention(*tensors, want.data_ptr(), workspace.data_ptr(), len_dev.data_ptr(), scale,
                                       *sizes, stream)
     assert rc == 0, lib.llmq_last_error()
+    torch.cuda.synchronize()
+    free_before, reserved_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
     rc = lib.llmq_kv_decode_attention_static(*tensors, got.data_ptr(), len_dev.data_ptr(), scale, *sizes, stream)
     assert rc == 0, lib.llmq_last_error()
     torch.cuda.synchronize()
+    if _WARMED:  # (the first call on the device may load the code object that holds the array)
+        # the device's free memory (hipMemGetInfo) and torch's pool are what they were: the call allocated nothing
+        assert torch.cuda.mem_get_info()[0] == free_before and torch.cuda.memory_reserved() == reserved_before
+    _WARMED.append(True)
     assert torch.isfinite(want.float()).all()
     assert torch.equal(got.view(torch.int16 if dtype != torch.float32 else torch.int32),
                        want.view(torch.int16 if dtype != torch.float32 else torch.int32))
