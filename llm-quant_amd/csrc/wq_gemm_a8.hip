@@ -27,6 +27,8 @@
 // the same exact integer group sums, folded in with fewer vector instructions: 1: fma((float)isum * sw, sx,
 // total), three per output and group instead of four; 2: one activation scale per token (sx[M]), which
 // leaves the sum over groups: fma((float)isum, sw, total), two, and the token's scale once at the store.
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "llmq_device.h"
@@ -41,6 +43,9 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 constexpr int kGroup = 128;
 constexpr int kThreads = 256;
 constexpr int kRowStride = kGroup + 16;  // bytes; padding keeps 16-byte reads off the same banks
+// the group-parallel kernel (exact form) takes outputs of up to this many 32 x 32 tiles per round of 256 of the
+// tiled kernel's 64 x 64 tiles
+constexpr int kGroupsTilesPerRound = 640;
 
 struct GemmArgs {
   const int8_t* a;     // [M, G*128]
@@ -314,10 +319,38 @@ int launch_tile(const GemmArgs& g, int wformat, hipStream_t stream) {
   return llmq_host::check_launch("wq_gemm_a8_kernel");
 }
 
+// LLMQ_A8_FORM=tile / groups in the environment pins the exact GEMM to the tiled kernels or to the group-parallel
+// kernel (wq_gemm_a8_groups.hip) whatever the shape: the two are bit-identical, and the tests run every shape
+// through both. Read per call.
+int forced_form() {
+  const char* v = getenv("LLMQ_A8_FORM");
+  if (v == nullptr) return 0;
+  return v[0] == 't' ? 1 : (v[0] == 'g' ? 2 : 0);
+}
+
 template <typename T, int MODE>
 int launch_typed(const GemmArgs& g, int wformat, hipStream_t stream) {
   // 128 x 128 tiles when there is at least one for every CU, else 64 x 64
   const int64_t big_tiles = static_cast<int64_t>((g.N + 127) / 128) * ((g.M + 127) / 128);
+  if constexpr (MODE == 0) {
+    // The exact form: a tile's groups are a chain of dependent steps, and with few tiles the chip waits on few
+    // chains. The group-parallel kernel computes eight groups of a 32 x 64 tile at once and only orders the
+    // additions (same bits).
+    // Which is faster, measured on 32-group and 112-group rows at M = 128 ... 2048 (int4): the tiled kernel takes
+    // ~0.57 us per group and round of 256 of its 64 x 64 tiles, this one ~0.7 ns per group and 32 x 32 tile (it pays
+    // for staging and unpacking per wave): it wins where the output is a few hundred 32 x 32 tiles and the rows are
+    // long -- 128 x 4096 x 14336: 41 us against 65; 128 x 14336 x 4096: 49 against 30, which stays tiled.
+    const int form = forced_form();
+    const int64_t tiles32 = static_cast<int64_t>((g.N + 31) / 32) * ((g.M + 31) / 32);
+    const int64_t tiles64 = static_cast<int64_t>((g.N + 63) / 64) * ((g.M + 63) / 64);
+    const bool pays = big_tiles < 256 && g.G >= 16 && tiles32 <= kGroupsTilesPerRound * ((tiles64 + 255) / 256);
+    const bool groups = form == 2 || (form == 0 && pays);
+    if (groups && llmq_host::gemm_a8_groups_supported(g.M, g.N, g.G)) {
+      const int dtype = sizeof(T) == 4 ? LLMQ_F32 : (std::is_same<T, f16_t>::value ? LLMQ_F16 : LLMQ_BF16);
+      return llmq_host::gemm_a8_groups(g.a, g.sx, g.qw, g.sw, g.bias, g.out, g.M, g.N, g.G, g.out_group, wformat, dtype,
+                                       stream);
+    }
+  }
   return big_tiles >= 256 ? launch_tile<T, 2, MODE>(g, wformat, stream) : launch_tile<T, 1, MODE>(g, wformat, stream);
 }
 

@@ -1,0 +1,332 @@
+// The exact integer prefill GEMM for outputs with too few tiles to fill the chip, gfx950.
+//
+//   out[m, n] = sum over groups g, IN ORDER, of  ((float)(sum_k a[m,g,k] * q[n,g,k]) * sw[sr(n),g]) * sx[m,g]
+//
+// -- the A8 branch of RealQuantLinear.forward (llmquant/quantizers/real.py:76-103), bit for bit, as
+// wq_gemm_a8.hip computes it. What is fixed by that arithmetic is the order of the fp32 ADDITIONS; the terms
+//   p[m, n, g] = fl(fl(float(isum) * sw) * sx)
+// do not depend on one another. A workgroup that walks the groups of its tile one after the other (as the tiled
+// kernel does) is a chain of G dependent steps, each a load -> multiply -> scale round trip, and with few tiles
+// (M = 128 against a weight of a few thousand rows) the chip waits on 128 such chains: 64 us for 112 groups.
+//
+// Here the eight waves of a workgroup take DIFFERENT groups of the same 32 x 32 output tile: in round r, wave w
+// computes p for group 8 r + w (operands of its own, nothing shared, no barrier: loaded as whole rows a round
+// ahead and turned into matrix-core operand layout through the wave's LDS slot), leaves the 32 x 32 fp32 terms
+// in that slot, and after a barrier every wave adds, for
+// its eighth of the tile, slot 0, slot 1, ... slot 7 onto its running totals: the additions happen in group
+// order, one at a time, exactly as in the serial walk. A tile's chain is G / 8 rounds long; the next round's
+// operands are in flight across the barriers. Cost: every term crosses LDS once (8 bytes per output and group).
+//
+// Operand layout. v_mfma_i32_32x32x32_i8 takes from lane l: row l % 32, sixteen k-values of half l / 32. A lane
+// owns one half of a group's 128 k-values (64 contiguous bytes of a row of activations, 32 bytes of packed
+// weights); a sum over k does not care about the order inside the half as long as both operands agree on it.
+// Packed int4: a 32-bit word w of eight codes gives (w << 4 & 0xf0f0f0f0) ^ 0x80808080 = the even codes and
+// (w & 0xf0f0f0f0) ^ 0x80808080 = the odd codes as signed bytes 16 * code (the 16 leaves through the weight
+// scale, a power of two: no rounding changes); the activation bytes are brought into the same even / odd order
+// with one byte permute per word.
+#include "llmq_device.h"
+
+namespace {
+
+using namespace llmq;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int kGroup = 128;
+constexpr int kWaysLog2 = 3;
+constexpr int kWays = 1 << kWaysLog2;       // waves of a workgroup = groups of a round
+constexpr int kThreads = kWays * kWave;
+constexpr int kTM = 32, kTN = 32;           // output tile of a workgroup (and of every wave)
+constexpr int kSlotFloats = kTM * kTN;      // one wave's terms of one group
+
+struct GroupArgs {
+  const int8_t* a;     // [M, G*128]
+  const float* sx;     // [M, G]
+  const uint8_t* qw;   // [N, G, 128] int8 or [N, G, 64] packed
+  const float* sw;     // [scale_rows, G]
+  const float* bias;   // [N] or null
+  void* out;           // [M, N]
+  int M, N, G, out_group;
+};
+
+// What a wave holds of one group between its loads and its multiply: the 16-byte packets of its operand tiles as
+// they lie in memory. Packet p = 64 i + lane of the activation tile is row p / 8, piece p % 8 (eight whole rows of
+// 128 bytes per load instruction); of the weight tile, row p / 4, piece p % 4 (int4: 64 bytes a row) or row p / 8,
+// piece p % 8 (int8). Loading straight in operand layout instead (lane = row, 16 bytes of it) touches 32 cache
+// lines per instruction, and the address unit then sets the pace (measured: 4x slower).
+template <int BITS> struct Operands {
+  u32x4 ra[4];
+  u32x4 rb[BITS == 8 ? 4 : 2];
+};
+
+constexpr int kChunkGroups = 32;   // groups whose scales sit in LDS at a time
+
+
+
+template <typename T, int BITS>
+__device__ __forceinline__ void groups_body(const GroupArgs& g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* slots = reinterpret_cast<float*>(smem);                       // [kWays][kSlotFloats]
+  float* s_sx = slots + kWays * kSlotFloats;                           // [kChunkGroups][kTM]
+  float* s_sw = s_sx + kChunkGroups * kTM;                             // [kChunkGroups][kTN]
+
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid >> 6;
+  const int col = lane & 31, half = lane >> 5;
+  const int m0 = blockIdx.y * kTM, n0 = blockIdx.x * kTN;
+  const uint32_t k_total = static_cast<uint32_t>(g.G) * kGroup;
+  const uint32_t w_row_bytes = BITS == 8 ? k_total : k_total / 2;
+  constexpr int kBPackets = BITS == 8 ? 4 : 2;
+  constexpr int kGroupBytesB = BITS == 8 ? kGroup : kGroup / 2;
+
+  // byte offsets of the lane's packets in group 0 (rows past the end clamped: loaded, never stored); the host
+  // has checked that both operands are smaller than 4 GB
+  uint32_t a_off[4], b_off[kBPackets];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int p = i * kWave + lane;
+    a_off[i] = static_cast<uint32_t>(min(m0 + (p >> 3), g.M - 1)) * k_total + (p & 7) * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < kBPackets; ++i) {
+    const int p = i * kWave + lane;
+    const int row = BITS == 8 ? p >> 3 : p >> 2, piece = BITS == 8 ? p & 7 : p & 3;
+    b_off[i] = static_cast<uint32_t>(min(n0 + row, g.N - 1)) * w_row_bytes + piece * 16;
+  }
+  auto load = [&](Operands<BITS>& o, int grp) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o.ra[i] = load16(g.a + (a_off[i] + static_cast<uint32_t>(grp) * kGroup));
+#pragma unroll
+    for (int i = 0; i < kBPackets; ++i) o.rb[i] = load16(g.qw + (b_off[i] + static_cast<uint32_t>(grp) * kGroupBytesB));
+  };
+
+  // The tile's scales, kChunkGroups groups at a time, as [group][row] and [group][column]: a thread reads four of
+  // them a chunk ahead (32 consecutive groups of a row are one cache line) and puts them into LDS between the two
+  // barriers of the chunk's last round.
+  float pre_sx[2], pre_sw[2];
+  auto load_chunk = [&](int chunk) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      // (groups past the end: clamped, so that the loads are unconditional; those values are never multiplied with)
+      const int idx = tid + kThreads * i, row = idx >> 5, grp = min(chunk * kChunkGroups + (idx & 31), g.G - 1);
+      const int n = min(n0 + row, g.N - 1);
+      pre_sx[i] = g.sx[static_cast<int64_t>(min(m0 + row, g.M - 1)) * g.G + grp];
+      pre_sw[i] = g.sw[static_cast<int64_t>(g.out_group > 0 ? n / g.out_group : n) * g.G + grp];
+    }
+  };
+  auto store_chunk = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int idx = tid + kThreads * i;
+      s_sx[(idx & 31) * kTM + (idx >> 5)] = pre_sx[i];
+      // (the unpacked nibbles are 16 x their codes: the 16 leaves here, exactly)
+      s_sw[(idx & 31) * kTN + (idx >> 5)] = BITS == 4 ? pre_sw[i] * 0.0625f : pre_sw[i];
+    }
+  };
+
+  // One group's terms into this wave's slot. The slot (4 KB) first serves as the wave's staging area, for the
+  // activations and then for the weights: the packets go in as whole rows (16-byte pieces XOR-swizzled by row, so
+  // that neither the writes nor the operand reads collide on banks) and come back out in operand layout: lane
+  // (row or column `col`, k-half `half`) reads its pieces. LDS serves a wave's accesses in order; the wave
+  // barriers keep the compiler from moving them.
+  // Result register r of the 32 x 32 product is row 8 (r / 4) + 4 half + r % 4, column col; the slot keeps the
+  // terms as [r / 4][lane][r % 4].
+  auto produce = [&](const Operands<BITS>& o, int grp) {
+    unsigned char* stage = reinterpret_cast<unsigned char*>(slots + wv * kSlotFloats);
+    // piece `piece` of 128-byte line `line`, XOR-swizzled
+    auto piece_at = [](int line, int piece) { return line * 128 + ((piece ^ (line & 7)) << 4); };
+    // packet 64 i + lane is piece lane % 8 of line 8 i + lane / 8: one address, the rest are constant offsets
+    unsigned char* put = stage + piece_at(lane >> 3, lane & 7);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) store16(put + i * 1024, o.ra[i]);
+    __builtin_amdgcn_wave_barrier();
+    v4i fa[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const u32x4 d = load16(stage + piece_at(col, 4 * half + ks));
+      if constexpr (BITS == 8) {
+        fa[ks] = v4i{static_cast<int>(d.x), static_cast<int>(d.y), static_cast<int>(d.z), static_cast<int>(d.w)};
+      } else {
+        // even bytes, odd bytes of each pair of words: the order the unpacked nibbles come in
+        fa[ks] = v4i{static_cast<int>(__builtin_amdgcn_perm(d.y, d.x, 0x06040200u)),
+                     static_cast<int>(__builtin_amdgcn_perm(d.y, d.x, 0x07050301u)),
+                     static_cast<int>(__builtin_amdgcn_perm(d.w, d.z, 0x06040200u)),
+                     static_cast<int>(__builtin_amdgcn_perm(d.w, d.z, 0x07050301u))};
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < kBPackets; ++i) store16(put + i * 1024, o.rb[i]);   // int4: 64-byte rows, two to a line
+    __builtin_amdgcn_wave_barrier();
+    v4i fb[4];
+    if constexpr (BITS == 8) {
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const u32x4 w = load16(stage + piece_at(col, 4 * half + ks));
+        fb[ks] = v4i{static_cast<int>(w.x), static_cast<int>(w.y), static_cast<int>(w.z), static_cast<int>(w.w)};
+      }
+    } else {
+      // the lane's column: packets 4 col + 2 half + {0, 1} of the staged tile (neighbours in one line: the second
+      // address is the first with bit 4 flipped)
+      const int q = col * 4 + 2 * half;
+      const int at = piece_at(q >> 3, q & 7);
+      const u32x4 lo = load16(stage + at), hi = load16(stage + (at ^ 16));
+      const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const uint32_t w0 = w[2 * ks], w1 = w[2 * ks + 1];
+        fb[ks] = v4i{static_cast<int>(((w0 << 4) & 0xf0f0f0f0u) ^ 0x80808080u), static_cast<int>((w0 & 0xf0f0f0f0u) ^ 0x80808080u),
+                     static_cast<int>(((w1 << 4) & 0xf0f0f0f0u) ^ 0x80808080u), static_cast<int>((w1 & 0xf0f0f0f0u) ^ 0x80808080u)};
+      }
+    }
+    // every operand is in registers: the staging area becomes the slot
+    __builtin_amdgcn_wave_barrier();
+    v16i d = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) d = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks], fb[ks], d, 0, 0, 0);
+    float* slot = slots + wv * kSlotFloats;
+    const int gl = grp & (kChunkGroups - 1);
+    const float sw = s_sw[gl * kTN + col];
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      const u32x4 s4 = *reinterpret_cast<const u32x4*>(&s_sx[gl * kTM + 8 * r4 + 4 * half]);
+      const float sx4[4] = {__builtin_bit_cast(float, s4.x), __builtin_bit_cast(float, s4.y),
+                            __builtin_bit_cast(float, s4.z), __builtin_bit_cast(float, s4.w)};
+      float p[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float f = static_cast<float>(d[4 * r4 + i]);
+        f = f * sw;
+        p[i] = f * sx4[i];
+      }
+      store16(slot + (r4 * kWave + lane) * 4, Pack<float>::pack(p));
+    }
+  };
+
+  // this wave's eighth of the tile in the additions: result registers 4 (wv / 2) + 2 (wv % 2) + {0, 1} of every lane
+  float total[2] = {0.0f, 0.0f};
+  const int my_pair = ((wv >> 1) * kWave + lane) * 4 + 2 * (wv & 1);
+  auto add_round = [&](int valid) {
+    for (int s = 0; s < valid; ++s) {
+      const u32x2 v = *reinterpret_cast<const u32x2*>(slots + s * kSlotFloats + my_pair);
+      total[0] = total[0] + __builtin_bit_cast(float, v.x);
+      total[1] = total[1] + __builtin_bit_cast(float, v.y);
+    }
+  };
+
+  const int rounds = (g.G + kWays - 1) >> kWaysLog2;
+  const int full = g.G >> kWaysLog2;   // rounds in which every wave has a group
+  constexpr int kRoundsPerChunk = kChunkGroups / kWays;
+  Operands<BITS> cur, nxt;
+  if (wv < g.G) load(cur, wv);
+  load_chunk(0);
+  store_chunk();
+  load_chunk(1);   // (past the last group: clamped loads whose values are never stored)
+  __syncthreads();   // the first chunk's scales are in place
+  // between the two barriers of a chunk's last round nobody multiplies with its scales any more, and the next
+  // round does not start before the second barrier: the next chunk goes in, and the one after it is requested
+  auto turn_chunk = [&](int r) {
+    if ((r + 1) % kRoundsPerChunk == 0 && r + 1 < rounds) {
+      store_chunk();
+      load_chunk((r + 1) / kRoundsPerChunk + 1);
+    }
+  };
+  int r = 0;
+  // Steady state: this round's and the next round's group exist for every wave, so nothing branches around the
+  // loads and the compiler's waits before the staging stores count exactly the loads that may stay in flight
+  // (a branch around them makes it drain the next round's loads before this round's multiply). The operand set
+  // is copied at the end of a round (two rounds per trip with the sets swapping roles needs 57 more registers).
+  for (; r + 1 < full; ++r) {
+    const int grp = r * kWays + wv;
+    load(nxt, grp + kWays);
+    produce(cur, grp);
+    __syncthreads();
+    turn_chunk(r);
+    add_round(kWays);
+    __syncthreads();
+    cur = nxt;
+  }
+  for (; r < rounds; ++r) {
+    const int grp = r * kWays + wv;
+    const bool more = grp + kWays < g.G;
+    if (more) load(nxt, grp + kWays);
+    if (grp < g.G) produce(cur, grp);
+    __syncthreads();
+    turn_chunk(r);
+    add_round(min(kWays, g.G - r * kWays));
+    __syncthreads();
+    if (more) cur = nxt;
+  }
+
+  T* __restrict__ out = static_cast<T*>(g.out);
+  const int n = n0 + col;
+  if (n < g.N) {
+    const float b = g.bias != nullptr ? g.bias[n] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int m = m0 + 8 * (wv >> 1) + 4 * half + 2 * (wv & 1) + i;
+      if (m < g.M) {
+        const float v = g.bias != nullptr ? total[i] + b : total[i];
+        out[static_cast<int64_t>(m) * g.N + n] = from_float<T>(v);
+      }
+    }
+  }
+}
+
+// Packed int4 weights: held to 128 registers (eight spilled, all outside the steady loop's multiply), so that two
+// workgroups (sixteen waves) share a CU and one's additions run under the other's multiplies: 128 x 4096 x 14336
+// in 41 us against 47 us with one workgroup a CU. int8 weights would spill 31: that form runs one workgroup a CU.
+template <typename T>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void wq_gemm_a8_groups_kernel4(const GroupArgs g) {
+  groups_body<T, 4>(g);
+}
+template <typename T>
+__global__ __launch_bounds__(kThreads) void wq_gemm_a8_groups_kernel8(const GroupArgs g) {
+  groups_body<T, 8>(g);
+}
+
+constexpr size_t kLdsBytes = (static_cast<size_t>(kWays) * kSlotFloats + kChunkGroups * (kTM + kTN)) * sizeof(float);
+
+template <typename T, int BITS>
+int launch(const GroupArgs& g, hipStream_t stream) {
+  auto kernel = BITS == 4 ? wq_gemm_a8_groups_kernel4<T> : wq_gemm_a8_groups_kernel8<T>;
+  static bool raised = false;  // per instantiation; worst case two threads both set it
+  if (!raised) {
+    const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (err != hipSuccess) {
+      llmq_host::set_error("raising the LDS limit failed: %s", hipGetErrorString(err));
+      return static_cast<int>(err);
+    }
+    raised = true;
+  }
+  const dim3 grid((g.N + kTN - 1) / kTN, (g.M + kTM - 1) / kTM), block(kThreads);
+  hipLaunchKernelGGL(kernel, grid, block, kLdsBytes, stream, g);
+  return llmq_host::check_launch("wq_gemm_a8_groups_kernel");
+}
+
+}  // namespace
+
+namespace llmq_host {
+
+// Whether the group-parallel form can take the problem: it addresses both operands with 32-bit byte offsets.
+bool gemm_a8_groups_supported(int M, int N, int G) {
+  const uint64_t k_total = static_cast<uint64_t>(G) * kGroup;
+  return static_cast<uint64_t>(M) * k_total < (1ull << 32) && static_cast<uint64_t>(N) * k_total < (1ull << 32);
+}
+
+int gemm_a8_groups(const int8_t* a, const float* sx, const void* qweight, const float* wscale,
+                   const float* bias_or_null, void* out, int M, int N, int G, int out_group, int wformat, int dtype,
+                   hipStream_t stream) {
+  GroupArgs g{a, sx, static_cast<const uint8_t*>(qweight), wscale, bias_or_null, out, M, N, G, out_group};
+#define LLMQ_GO(T) (wformat == LLMQ_W_INT8 ? launch<T, 8>(g, stream) : launch<T, 4>(g, stream))
+  switch (dtype) {
+    case LLMQ_F32: return LLMQ_GO(float);
+    case LLMQ_F16: return LLMQ_GO(f16_t);
+    case LLMQ_BF16: return LLMQ_GO(bf16_t);
+  }
+#undef LLMQ_GO
+  return fail_invalid("out must be float32, float16 or bfloat16, got dtype code %d", dtype);
+}
+
+}  // namespace llmq_host

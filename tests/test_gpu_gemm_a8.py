@@ -25,7 +25,27 @@ def ext():
     return load_extension()
 
 
-def run_case(ext, m, n, k, bits, dtype, out_group=0, bias=False, seed=0, outliers=False):
+#: The exact GEMM has two bit-identical forms: tiled kernels that walk a tile's groups one after the other, and a
+#: group-parallel kernel (eight groups of a 32 x 64 tile at once, additions in group order) for outputs of few
+#: tiles. LLMQ_A8_FORM pins one whatever the shape; None is the library's own choice.
+FORMS = pytest.mark.parametrize("form", ["tile", "groups", None], ids=["tiled", "group-parallel", "own choice"])
+
+
+@pytest.fixture(autouse=True)
+def no_form_left_pinned():
+    import os
+
+    yield
+    os.environ.pop("LLMQ_A8_FORM", None)
+
+
+def run_case(ext, m, n, k, bits, dtype, out_group=0, bias=False, seed=0, outliers=False, form=None):
+    import os
+
+    if form is None:
+        os.environ.pop("LLMQ_A8_FORM", None)
+    else:
+        os.environ["LLMQ_A8_FORM"] = form
     torch.manual_seed(seed)
     w = (torch.randn(n, k) * 0.015).to(torch.bfloat16)
     x = torch.randn(m, k)
@@ -44,19 +64,24 @@ def run_case(ext, m, n, k, bits, dtype, out_group=0, bias=False, seed=0, outlier
     return got, (x, canonical, scales, b)
 
 
+@FORMS
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("m,n,k", [(32, 256, 512), (1, 128, 128), (37, 200, 384), (130, 129, 256), (4, 512, 2048)])
-def test_bit_exact_against_real_mode(ext, bits, dtype, m, n, k):
-    got, (x, canonical, scales, _) = run_case(ext, m, n, k, bits, dtype)
+@pytest.mark.parametrize("m,n,k", [(32, 256, 512), (1, 128, 128), (37, 200, 384), (130, 129, 256), (4, 512, 2048),
+                                   (65, 70, 1152), (33, 64, 2176)])
+def test_bit_exact_against_real_mode(ext, bits, dtype, m, n, k, form):
+    """(1152 and 2176: nine and seventeen groups, a last round of the group-parallel form with one group in it.)"""
+    got, (x, canonical, scales, _) = run_case(ext, m, n, k, bits, dtype, form=form)
     want = oracle.real_linear(to_np(x), canonical, scales, tag_of(dtype), None, 8)
     assert got.shape == (m, n) and got.dtype == dtype
     assert np.array_equal(to_np(got).view(np.uint32), want.view(np.uint32))
 
 
+@FORMS
 @pytest.mark.parametrize("bits", [4, 8])
-def test_bias_and_head_scales(ext, bits):
-    got, (x, canonical, scales, b) = run_case(ext, 70, 192, 512, bits, torch.bfloat16, out_group=64, bias=True, seed=1)
+def test_bias_and_head_scales(ext, bits, form):
+    got, (x, canonical, scales, b) = run_case(ext, 70, 192, 512, bits, torch.bfloat16, out_group=64, bias=True, seed=1,
+                                              form=form)
     want = oracle.real_linear(to_np(x), canonical, scales, "bf16", 64, 8, to_np(b))
     assert np.array_equal(to_np(got), want)
 
@@ -70,12 +95,13 @@ def test_matches_the_float64_closed_form(ext):
     assert rel_l2(to_np(got), exact) <= 1e-6
 
 
+@pytest.mark.parametrize("form", ["tile", "groups"], ids=["tiled", "group-parallel"])
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
 @pytest.mark.parametrize("m", [128, 512, 2048])
-def test_llama_8b_mlp_shapes_on_sampled_entries(ext, n, k, m):
+def test_llama_8b_mlp_shapes_on_sampled_entries(ext, n, k, m, form):
     """The 512-token prefill case at full size (1% outlier channels x20): 64 x 64 sampled outputs,
-    bit-exact against the oracle restricted to those rows and columns."""
-    got, (x, canonical, scales, _) = run_case(ext, m, n, k, 4, torch.bfloat16, seed=3, outliers=True)
+    bit-exact against the oracle restricted to those rows and columns, through both forms of the kernel."""
+    got, (x, canonical, scales, _) = run_case(ext, m, n, k, 4, torch.bfloat16, seed=3, outliers=True, form=form)
     rng = np.random.default_rng(0)
     rows = np.sort(rng.choice(m, 64, replace=False))
     cols = np.sort(rng.choice(n, 64, replace=False))
