@@ -34,6 +34,8 @@
 //
 // Small N: a split of the reduction axis across workgroups, fp32 partial tiles in a workspace, added in a
 // fixed order by a second launch (the result does not depend on which workgroup finished first).
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "llmq_device.h"
@@ -46,15 +48,43 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kGroup = 128;
-constexpr int kBM = 128;            // activation rows per workgroup
-constexpr int kWaveM = 128;         // activation rows per wave
-constexpr int kWaveN = 32;          // weight rows (output columns) per wave
-constexpr int kWaves = 8;           // 1 (rows) x 8 (columns)
-constexpr int kBN = kWaveN * 8;
-constexpr int kThreads = kWaves * kWave;
 constexpr int kRowBytes = kGroup * 2;          // one activation row of one group
-constexpr int kTileBytes = kBM * kRowBytes;    // 32 KB
-constexpr int kMT = kWaveM / 32, kNT = kWaveN / 32;
+template <int BITS> constexpr int kCodeRowBytes = BITS == 4 ? kGroup / 2 : kGroup;
+
+// The workgroup's tile: BM activation rows x 32 COLS weight rows; a wave owns 32 of the columns, all the rows and
+// one KH-th of every group's k-steps. Wide (128 x 256, eight waves, two per SIMD) is the throughput shape. Narrow
+// (64 x 128) is for outputs that have too few wide tiles to occupy the chip (a 512-token prompt against a 3072-row
+// weight: 48 wide tiles, 192 narrow ones): its eight waves are four column blocks times two halves of the group
+// (still two waves per SIMD, so that one converts codes while the other multiplies), the halves' totals are added
+// through LDS once, at the end, and the smaller stages leave LDS for four of them in flight.
+template <int BM, int COLS, int KH> struct Shape {
+  static constexpr int kBM = BM;                 // activation rows per workgroup
+  static constexpr int kWaveM = BM;              // ... and per wave
+  static constexpr int kWaveN = 32;              // weight rows (output columns) per wave
+  static constexpr int kColWaves = COLS;         // column blocks
+  static constexpr int kKH = KH;                 // waves that share a column block, each with 8 / KH k-steps of a group
+  static constexpr int kWaves = COLS * KH;
+  static constexpr int kBN = kWaveN * COLS;
+  static constexpr int kThreads = kWaves * kWave;
+  static constexpr int kTileBytes = BM * kRowBytes;
+  static constexpr int kMT = BM / 32, kNT = kWaveN / 32;
+  static constexpr int kRecTileBytes = BM * 16;
+  static constexpr int kScaleTileBytes = kBN * 4;
+  static constexpr int kRecWaves = BM / 64;      // waves that fetch the activation-sum records (64 rows each)
+  static constexpr int kScaleWaves = kBN / 64;   // ... and, after them, the scales (64 columns each)
+  template <int BITS> static constexpr int kCodeTileBytes = kBN * kCodeRowBytes<BITS>;
+  template <int BITS>
+  static constexpr int kStageBytes = kTileBytes + kCodeTileBytes<BITS> + kRecTileBytes + kScaleTileBytes;
+  // as many stages as fit the 160 KB of LDS, at most four: a group's transfers are requested kStages - 1 groups
+  // before it is multiplied (wide: three for int4, 153 KB, two for int8; narrow: four)
+  template <int BITS>
+  static constexpr int kStages = (160 * 1024 / kStageBytes<BITS>) >= 4 ? 4 : (160 * 1024 / kStageBytes<BITS>);
+  template <int BITS> static constexpr int kLdsBytes = kStages<BITS> * kStageBytes<BITS>;
+};
+using Wide = Shape<128, 8, 1>;
+using Narrow = Shape<64, 4, 2>;
+// (what the host side sizes for when it does not say which: the wide tile)
+constexpr int kBM = Wide::kBM, kBN = Wide::kBN;
 
 template <int BITS> constexpr float kCodeBias = BITS == 4 ? 24.0f : 128.0f;
 
@@ -119,19 +149,9 @@ struct TileArgs {
 enum Epilogue { kEpiStore = 0, kEpiGateUpSilu = 1 };
 constexpr int kEpiRowBytes = 128 * 2 + 16;   // a row of the gate (or up) block in LDS: 16 bytes of padding per row
 
-// LDS, per buffer (two buffers): the activation tile [128 rows][16 slots of 16 bytes], the raw codes of
-// the workgroup's 256 weight rows for one group ([256][64] bytes of int4 or [256][128] of int8, slots
-// XOR-swizzled by row like the activation), and the 128 activation-sum records.
-template <int BITS> constexpr int kCodeRowBytes = BITS == 4 ? kGroup / 2 : kGroup;
-template <int BITS> constexpr int kCodeTileBytes = kBN * kCodeRowBytes<BITS>;
-constexpr int kRecTileBytes = kBM * 16;
-constexpr int kScaleTileBytes = kBN * 4;
-template <int BITS> constexpr int kStageBytes = kTileBytes + kCodeTileBytes<BITS> + kRecTileBytes + kScaleTileBytes;
-// three stages where they fit the 160 KB of LDS (int4: 153 KB): a group's transfers are requested two
-// groups before it is multiplied; int8 codes leave room for two
-template <int BITS> constexpr int kStages = BITS == 4 ? 3 : 2;
-template <int BITS> constexpr int kLdsBytes = kStages<BITS> * kStageBytes<BITS>;
-
+// LDS, per stage: the activation tile [BM rows][16 slots of 16 bytes], the raw codes of the workgroup's weight rows
+// for one group ([BN][64] bytes of int4 or [BN][128] of int8, slots XOR-swizzled by row like the activation), the
+// activation-sum records and the group's scales.
 // slot of chunk c in weight row `row`: 16 consecutive rows read the same chunk at once and must land in
 // 16 different bank quads
 template <int BITS> __device__ __forceinline__ int code_slot(int row, int c) {
@@ -141,12 +161,12 @@ template <int BITS> __device__ __forceinline__ int code_slot(int row, int c) {
 constexpr uint32_t kNibbleMask = 0x00780078u;   // (and_or: (value & mask) | bits in one instruction)
 
 // Two of the four operand words of a k-step: a k-step's eight codes are one 32-bit word of int4 or two of
-// int8; operand word i pairs codes i and i + 4. `half` selects words (0, 1) or (2, 3).
+// int8 (`raw`: the wave's k-steps one after the other); operand word i pairs codes i and i + 4. `half` selects
+// words (0, 1) or (2, 3).
 template <int BITS>
-__device__ __forceinline__ void code_words(const u32x4* raw, int step, int half, uint32_t sixteen, uint32_t* out) {
+__device__ __forceinline__ void code_words(const uint32_t* raw, int step, int half, uint32_t sixteen, uint32_t* out) {
   if constexpr (BITS == 4) {
-    const u32x4 q = raw[step >> 2];
-    const uint32_t w = (step & 3) == 0 ? q.x : (step & 3) == 1 ? q.y : (step & 3) == 2 ? q.z : q.w;
+    const uint32_t w = raw[step];
     if (half == 0) {
       out[0] = and_or(w << 3, kNibbleMask, sixteen);  // nibbles 0 and 4
       out[1] = and_or(w >> 1, kNibbleMask, sixteen);  // 1 and 5
@@ -155,9 +175,8 @@ __device__ __forceinline__ void code_words(const u32x4* raw, int step, int half,
       out[1] = and_or(w >> 9, kNibbleMask, sixteen);  // 3 and 7
     }
   } else {
-    const u32x4 q = raw[step >> 1];
-    const uint32_t w0 = ((step & 1) ? q.z : q.x) ^ 0x80808080u;  // codes 0..3 of the step, + 128
-    const uint32_t w1 = ((step & 1) ? q.w : q.y) ^ 0x80808080u;  // codes 4..7
+    const uint32_t w0 = raw[2 * step] ^ 0x80808080u;      // codes 0..3 of the step, + 128
+    const uint32_t w1 = raw[2 * step + 1] ^ 0x80808080u;  // codes 4..7
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int e = 2 * half + i;
@@ -173,9 +192,16 @@ __device__ __forceinline__ v16f mfma(const u32x4& a, const u32x4& b, const v16f&
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
 }
 
-template <int BITS, int EPI>
-__global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const TileArgs a) {
+template <int BITS, int EPI, typename S>
+__global__ __launch_bounds__(S::kThreads, 1) void wq_gemm_a16_tile_kernel(const TileArgs a) {
   extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
+  static_assert(EPI == kEpiStore || std::is_same<S, Wide>::value, "the gate|up epilogue is laid out for the wide tile");
+  constexpr int kBM = S::kBM, kBN = S::kBN, kWaveM = S::kWaveM, kWaveN = S::kWaveN, kWaves = S::kWaves;
+  constexpr int kThreads = S::kThreads, kTileBytes = S::kTileBytes, kMT = S::kMT, kNT = S::kNT;
+  constexpr int kRecTileBytes = S::kRecTileBytes, kRecWaves = S::kRecWaves, kScaleWaves = S::kScaleWaves;
+  constexpr int kCodeTileB = S::template kCodeTileBytes<BITS>, kStageB = S::template kStageBytes<BITS>;
+  constexpr int kStagesN = S::template kStages<BITS>;
+  constexpr int kKH = S::kKH, kSteps = 8 / kKH;   // k-steps of a group that one wave multiplies
 
   // Workgroups are dealt to the 8 XCDs round-robin by their index; a run of consecutive logical tiles
   // (the m-tiles of one n-tile first: they read the same weights) is put on one XCD, so the codes come
@@ -189,7 +215,10 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   const int sp = logical / (a.m_tiles * a.n_tiles);
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  const int wm = 0, wn = wv;  // every wave all the rows, an eighth of the columns
+  // every wave all the rows, 32 of the columns, and half kh of every group's k-steps (kKH == 1: all of them)
+  const int wm = 0, wn = wv % S::kColWaves;
+  const int kh = kKH == 1 ? 0 : __builtin_amdgcn_readfirstlane(wv / S::kColWaves);
+  static_assert(kKH == 1 || (kKH == kMT && kNT == 1), "the waves of a column block keep one 32 x 32 row tile each");
   const int lm = lane & 31, lh = lane >> 5;
   // (kEpiGateUpSilu: n0 is the tile's first gate row; column c of the tile is weight row weight_row(c))
   const int m0 = mt * kBM, n0 = EPI == kEpiGateUpSilu ? nt * (kBN / 2) : nt * kBN;
@@ -214,28 +243,35 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
     const int row = wv * (kBM / kWaves) + i * 4 + (lane >> 4);
     x_off[i] = static_cast<uint32_t>(m0 + row) * x_row_bytes + (((lane & 15) ^ (row & 15)) << 4);
   }
-  // codes: 2 (int4) or 4 (int8) instructions per wave; 16 or 8 weight rows each
-  constexpr int kCodeInstr = kCodeTileBytes<BITS> / 1024 / kWaves;
+  // codes: instructions of 16 (int4) or 8 (int8) weight rows each; kCodeInstr per wave (wide: 2 / 4), and where
+  // that does not come out even, one more from each of the first kLeftCodes waves
+  constexpr int kCodeInstr = kCodeTileB / 1024 / kWaves, kLeftCodes = kCodeTileB / 1024 % kWaves;
   constexpr int kRowsPerInstr = 1024 / kCodeRowBytes<BITS>;
   constexpr int kSlots = kCodeRowBytes<BITS> / 16;
   const uint32_t w_row_bytes = static_cast<uint32_t>(a.G) * kCodeRowBytes<BITS>;
-  uint32_t w_off[kCodeInstr];
+  uint32_t w_off[kCodeInstr + 1];
 #pragma unroll
-  for (int i = 0; i < kCodeInstr; ++i) {
-    const int row = (wv * kCodeInstr + i) * kRowsPerInstr + lane / kSlots;
+  for (int i = 0; i < kCodeInstr + 1; ++i) {
+    const int instr = i < kCodeInstr ? wv * kCodeInstr + i : kWaves * kCodeInstr + wv % (kLeftCodes ? kLeftCodes : 1);
+    const int row = instr * kRowsPerInstr + lane / kSlots;
     const int chunk = code_slot<BITS>(row, lane % kSlots);  // the swizzle is its own inverse
     w_off[i] = static_cast<uint32_t>(weight_row(row)) * w_row_bytes + chunk * 16;
   }
-  // records: waves 0 and 1, 64 rows each; scales: waves 2..5, 64 columns each
-  const uint32_t r_off = static_cast<uint32_t>(m0 + (wv & 1) * 64 + lane) * a.G * 16;
+  // One further instruction from the waves after those: the records (kRecWaves waves, 64 rows each), then the
+  // scales (kScaleWaves waves, 64 columns each).
+  constexpr int kExtraWaves = kLeftCodes + kRecWaves + kScaleWaves;
+  static_assert(kExtraWaves <= kWaves, "at most one transfer instruction per wave beyond the even share");
+  const int rec_wave = (wv + kWaves - kLeftCodes) % kWaves % kRecWaves;
+  const int scale_wave = (wv + kWaves - kLeftCodes - kRecWaves) % kWaves % kScaleWaves;
+  const uint32_t r_off = static_cast<uint32_t>(m0 + rec_wave * 64 + lane) * a.G * 16;
   const float* sw_lane;
   {
-    const int n = weight_row(((wv - 2) & 3) * 64 + lane);
+    const int n = weight_row(scale_wave * 64 + lane);
     sw_lane = a.sw + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * a.G;
   }
 
   auto request = [&](int g, int buf) {
-    uint8_t* stage = smem + buf * kStageBytes<BITS>;
+    uint8_t* stage = smem + buf * kStageB;
     const uint8_t* xg = a.xp + static_cast<uint32_t>(g) * kRowBytes;
 #pragma unroll
     for (int i = 0; i < kXInstr; ++i) {
@@ -250,32 +286,41 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
                                        reinterpret_cast<u32x4*>(stage + kTileBytes + (wv * kCodeInstr + i) * 1024), 16,
                                        0, 0);
     }
-    if (wv < 2) {
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(a.rec + r_off + static_cast<uint32_t>(g) * 16),
-                                       reinterpret_cast<u32x4*>(stage + kTileBytes + kCodeTileBytes<BITS> + wv * 1024),
+    if (wv < kLeftCodes) {
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(wg + w_off[kCodeInstr]),
+                                       reinterpret_cast<u32x4*>(stage + kTileBytes + (kWaves * kCodeInstr + wv) * 1024),
                                        16, 0, 0);
-    } else if (wv < 6) {
+    } else if (wv < kLeftCodes + kRecWaves) {
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(a.rec + r_off + static_cast<uint32_t>(g) * 16),
+                                       reinterpret_cast<u32x4*>(stage + kTileBytes + kCodeTileB + rec_wave * 1024),
+                                       16, 0, 0);
+    } else if (wv < kExtraWaves) {
       // the scales of 64 columns, one float per lane
       __builtin_amdgcn_global_load_lds(
-          sw_lane + g, reinterpret_cast<float*>(stage + kTileBytes + kCodeTileBytes<BITS> + kRecTileBytes + (wv - 2) * 256),
+          sw_lane + g, reinterpret_cast<float*>(stage + kTileBytes + kCodeTileB + kRecTileBytes + scale_wave * 256),
           4, 0, 0);
     }
   };
   // transfer instructions per wave and group (a compile-time count per branch: the waits below name how many
   // of the youngest may still be in flight)
-  constexpr int kDmaPerWave = kXInstr + kCodeInstr + 1;   // waves 0..5; waves 6, 7: one fewer
+  constexpr int kDmaPerWave = kXInstr + kCodeInstr + 1;   // the first kExtraWaves waves; the others: one fewer
 
   // ---- LDS -> operands ----------------------------------------------------------------------------------
   // activation operand of k-step j, row tile mi: row mi*32 + lm, chunk (8 lh + j) ^ (lm & 15)
-  const uint32_t a_base = (wm * kWaveM + lm) * kRowBytes + (((8 * lh) ^ (lm & 15)) << 4);  // k-step j: a_base ^ (j << 4)
-  // this lane's codes of a group: weight row wn*32 + lm, k in [64 lh, 64 lh + 64): 16-byte chunks
-  // lh * kRawLoads + q, at c_base ^ (q << 4)
-  constexpr int kRawLoads = BITS == 4 ? 2 : 4;
+  // (the wave's own k-steps are kh * kSteps + j, j < kSteps: its step j is at a_base ^ (j << 4))
+  const uint32_t a_base = (wm * kWaveM + lm) * kRowBytes + (((8 * lh + kh * kSteps) ^ (lm & 15)) << 4);
+  // this lane's codes of a group: weight row wn*32 + lm, k in [64 lh, 64 lh + 64), of which the wave's k-steps are
+  // kRawBytes bytes: the 16-byte chunks (lh kKH + kh) kRawLoads + q, at c_base ^ (q << 4), or (8 bytes) one half
+  // of a chunk
+  constexpr int kRawBytes = kSteps * (BITS == 4 ? 4 : 8);
+  constexpr int kRawLoads = kRawBytes / 16, kRawWords = kRawBytes / 4;
+  static_assert(kRawBytes == 8 || kRawBytes % 16 == 0, "a wave's codes of a group: 16-byte chunks, or half of one");
   uint32_t c_base[kNT];
 #pragma unroll
   for (int ni = 0; ni < kNT; ++ni) {
     const int row = wn * kWaveN + ni * 32 + lm;
-    c_base[ni] = kTileBytes + row * kCodeRowBytes<BITS> + code_slot<BITS>(row, lh * kRawLoads) * 16;
+    const int first = (lh * kKH + kh) * kRawBytes;   // byte of the lane's row
+    c_base[ni] = kTileBytes + row * kCodeRowBytes<BITS> + code_slot<BITS>(row, first >> 4) * 16 + (first & 15);
   }
   auto read16 = [&](const uint8_t* stage, uint32_t offset) { return *reinterpret_cast<const u32x4*>(stage + offset); };
 
@@ -289,33 +334,49 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   uint32_t sixteen = 0x41804180u;  // bf16 16.0 twice; kept in a vector register (see and_or)
   asm volatile("" : "+v"(sixteen));
   const uint32_t nb = bf16_bits_rne(-kCodeBias<BITS>);  // exact
-  const uint32_t nb2 = lh ? 0u : (nb | (nb << 16));
+  const uint32_t nb2 = (lh || kh) ? 0u : (nb | (nb << 16));   // (the correction step belongs to the group's first k-steps)
   const u32x4 bias_operand = {nb2, nb2, 0u, 0u};
 
   // ---- prologue: the first groups on their way, the first one's operands in registers ---------------------
 #pragma unroll
-  for (int st = 0; st < kStages<BITS>; ++st) {
+  for (int st = 0; st < kStagesN; ++st) {
     if (g_begin + st < g_end) request(g_begin + st, st);
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // (the first group's transfers only, where all kStages batches exist: the loop waits for each later one in turn)
+  if (g_end - g_begin >= kStagesN) {
+    if (wv < kExtraWaves) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStagesN - 1) * kDmaPerWave) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStagesN - 1) * (kDmaPerWave - 1)) : "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
   __builtin_amdgcn_s_barrier();
 
   // What a lane holds of the group it is about to multiply: the records (operand of the correction
   // step), its raw codes, its columns' scales and the activation operands of k-step 0.
-  u32x4 raw[kNT][kRawLoads], rec[kMT], fa[2][kMT];
+  u32x4 rec[kMT], fa[2][kMT];
+  uint32_t raw[kNT][kRawWords];
   float scale[kNT];
   auto fetch_group_operands = [&](int st) {
-    const uint8_t* stage = smem + st * kStageBytes<BITS>;
+    const uint8_t* stage = smem + st * kStageB;
 #pragma unroll
     for (int mi = 0; mi < kMT; ++mi)
-      rec[mi] = read16(stage, kTileBytes + kCodeTileBytes<BITS> + (wm * kWaveM + mi * 32 + lm) * 16);
+      rec[mi] = read16(stage, kTileBytes + kCodeTileB + (wm * kWaveM + mi * 32 + lm) * 16);
+#pragma unroll
+    for (int ni = 0; ni < kNT; ++ni) {
+      if constexpr (kRawBytes == 8) {
+        const u32x2 v = *reinterpret_cast<const u32x2*>(stage + c_base[ni]);
+        raw[ni][0] = v.x, raw[ni][1] = v.y;
+      } else {
+#pragma unroll
+        for (int q = 0; q < kRawLoads; ++q) {
+          const u32x4 v = read16(stage, c_base[ni] ^ (q << 4));
+          raw[ni][4 * q] = v.x, raw[ni][4 * q + 1] = v.y, raw[ni][4 * q + 2] = v.z, raw[ni][4 * q + 3] = v.w;
+        }
+      }
+    }
 #pragma unroll
     for (int ni = 0; ni < kNT; ++ni)
-#pragma unroll
-      for (int q = 0; q < kRawLoads; ++q) raw[ni][q] = read16(stage, c_base[ni] ^ (q << 4));
-#pragma unroll
-    for (int ni = 0; ni < kNT; ++ni)
-      scale[ni] = *reinterpret_cast<const float*>(stage + kTileBytes + kCodeTileBytes<BITS> + kRecTileBytes +
+      scale[ni] = *reinterpret_cast<const float*>(stage + kTileBytes + kCodeTileB + kRecTileBytes +
                                                   (wn * kWaveN + ni * 32 + lm) * 4);
 #pragma unroll
     for (int mi = 0; mi < kMT; ++mi) fa[0][mi] = read16(stage, mi * 32 * kRowBytes + a_base);
@@ -332,8 +393,8 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
   // next group's operands come out of it, and no wave starts a group waiting for memory or LDS.
   int st = 0;  // the stage of group g
   for (int g = g_begin; g < g_end; ++g) {
-    const uint8_t* stage = smem + st * kStageBytes<BITS>;
-    const int st_next = st + 1 == kStages<BITS> ? 0 : st + 1;
+    const uint8_t* stage = smem + st * kStageB;
+    const int st_next = st + 1 == kStagesN ? 0 : st + 1;
     float scale_now[kNT];
 #pragma unroll
     for (int ni = 0; ni < kNT; ++ni) scale_now[ni] = scale[ni];
@@ -347,10 +408,10 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
 #pragma unroll
       for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < kNT; ++ni) acc[mi][ni] = mfma(rec[mi], bias_operand, zero);
+        for (int ni = 0; ni < kNT; ++ni) acc[mi][ni] = kh == 0 ? mfma(rec[mi], bias_operand, zero) : zero;
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < kSteps; ++j) {
       u32x4 fb[kNT];
 #pragma unroll
       for (int ni = 0; ni < kNT; ++ni) {
@@ -359,21 +420,21 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
         code_words<BITS>(raw[ni], j, 1, sixteen, hi);
         fb[ni] = u32x4{lo[0], lo[1], hi[0], hi[1]};
       }
-      if (j < 7) {
+      if (j < kSteps - 1) {
 #pragma unroll
         for (int mi = 0; mi < kMT; ++mi) fa[(j + 1) & 1][mi] = read16(stage, mi * 32 * kRowBytes + (a_base ^ ((j + 1) << 4)));
       } else {
         // own transfers of the next group have landed (the youngest kStages - 2 batches may stay in flight)
-        if (kStages<BITS> == 3 && g + 2 < g_end) {  // (the batch of group g + 2 exists and is younger)
-          if (wv < 6) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDmaPerWave) : "memory");
-          else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDmaPerWave - 1) : "memory");
+        if (kStagesN >= 3 && g + kStagesN - 1 < g_end) {  // (the batches of groups g + 2 .. exist and are younger)
+          if (wv < kExtraWaves) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStagesN - 2) * kDmaPerWave) : "memory");
+          else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStagesN - 2) * (kDmaPerWave - 1)) : "memory");
         } else {
           asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
-        if (g + kStages<BITS> < g_end) request(g + kStages<BITS>, st);
-        if (g + 1 < g_end) fetch_group_operands(st_next);  // (fa[0]: step 7 multiplies out of fa[1])
+        if (g + kStagesN < g_end) request(g + kStagesN, st);
+        if (g + 1 < g_end) fetch_group_operands(st_next);  // (fa[0]: the last step multiplies out of fa[1])
       }
 #pragma unroll
       for (int mi = 0; mi < kMT; ++mi)
@@ -420,32 +481,59 @@ __global__ __launch_bounds__(kThreads, 1) void wq_gemm_a16_tile_kernel(const Til
     }
     return;
   }
-  if (a.splits == 1) {
-    bf16_t* __restrict__ out = static_cast<bf16_t*>(a.out);
+  // one 32 x 32 tile of totals, whose first row is m_first and whose column (this lane's) is n
+  auto store_tile = [&](const float (&v)[16], int m_first, int n) {
+    if (a.splits == 1) {
+      bf16_t* __restrict__ out = static_cast<bf16_t*>(a.out);
 #pragma unroll
-    for (int ni = 0; ni < kNT; ++ni) {
-      const int n = n0 + wn * kWaveN + ni * 32 + lm;
+      for (int r = 0; r < 16; ++r) {
+        const int m = m_first + 8 * (r >> 2) + 4 * lh + (r & 3);
+        if (m < a.M && n < a.N) out[static_cast<int64_t>(m) * a.N + n] = from_float<bf16_t>(v[r]);
+      }
+    } else {
+      float* __restrict__ part = a.partial + static_cast<int64_t>(sp) * a.M * a.N;
 #pragma unroll
-      for (int mi = 0; mi < kMT; ++mi)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm * kWaveM + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-          if (m < a.M && n < a.N) out[static_cast<int64_t>(m) * a.N + n] = from_float<bf16_t>(total[mi][ni][r]);
-        }
+      for (int r = 0; r < 16; ++r) {
+        const int m = m_first + 8 * (r >> 2) + 4 * lh + (r & 3);
+        if (m < a.M && n < a.N) part[static_cast<int64_t>(m) * a.N + n] = v[r];
+      }
     }
+  };
+  if constexpr (kKH > 1) {
+    // The kKH waves of a column block hold the totals of their parts of every group. Wave kh keeps row tile kh and
+    // hands the others over through LDS (4 KB a tile, [register][lane]; the stages are free: the loop's last
+    // barrier came after every wave's last operand read and its last transfer), then adds the parts of its tile in
+    // the order of the waves, its own in its place.
+    float* exchange = reinterpret_cast<float*>(smem);
+    auto slot = [&](int from, int tile) { return ((from * S::kColWaves + wn) * (kKH - 1) + (tile - (tile > from))) * 1024; };
+    float own[16];
+#pragma unroll
+    for (int t = 0; t < kKH; ++t) {
+      if (t == kh) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) own[r] = total[t][0][r];
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) exchange[slot(kh, t) + r * 64 + lane] = total[t][0][r];
+      }
+    }
+    __syncthreads();
+    float sum[16];
+#pragma unroll
+    for (int from = 0; from < kKH; ++from) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float part = from == kh ? own[r] : exchange[slot(from, kh) + r * 64 + lane];
+        sum[r] = from == 0 ? part : sum[r] + part;
+      }
+    }
+    store_tile(sum, m0 + kh * 32, n0 + wn * kWaveN + lm);
   } else {
-    float* __restrict__ part = a.partial + static_cast<int64_t>(sp) * a.M * a.N;
 #pragma unroll
-    for (int ni = 0; ni < kNT; ++ni) {
-      const int n = n0 + wn * kWaveN + ni * 32 + lm;
+    for (int ni = 0; ni < kNT; ++ni)
 #pragma unroll
       for (int mi = 0; mi < kMT; ++mi)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm * kWaveM + mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-          if (m < a.M && n < a.N) part[static_cast<int64_t>(m) * a.N + n] = total[mi][ni][r];
-        }
-    }
+        store_tile(total[mi][ni], m0 + wm * kWaveM + mi * 32, n0 + wn * kWaveN + ni * 32 + lm);
   }
 }
 
@@ -477,23 +565,26 @@ __global__ __launch_bounds__(256) void add_splits_kernel(const float* __restrict
   }
 }
 
-template <int BITS, int EPI>
+template <int BITS, int EPI, typename S = Wide>
 int launch_tiles(const TileArgs& a, dim3 grid, hipStream_t stream) {
-  auto kernel = wq_gemm_a16_tile_kernel<BITS, EPI>;
+  auto kernel = wq_gemm_a16_tile_kernel<BITS, EPI, S>;
+  constexpr int kLds = S::template kLdsBytes<BITS>;
   static bool raised = false;  // per instantiation; worst case two threads both set it
   if (!raised) {
     const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes<BITS>);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (err != hipSuccess) {
       llmq_host::set_error("raising the LDS limit failed: %s", hipGetErrorString(err));
       return static_cast<int>(err);
     }
     raised = true;
   }
-  hipLaunchKernelGGL(kernel, grid, dim3(kThreads), kLdsBytes<BITS>, stream, a);
+  hipLaunchKernelGGL(kernel, grid, dim3(S::kThreads), kLds, stream, a);
   return llmq_host::check_launch("wq_gemm_a16_tile_kernel");
 }
 
+// rows of up to this many groups take the narrow tile when the wide one would have to cut the reduction axis
+constexpr int kNarrowMaxGroups = 16;
 constexpr size_t kAlign = 256;
 size_t aligned(size_t bytes) { return (bytes + kAlign - 1) / kAlign * kAlign; }
 
@@ -502,23 +593,46 @@ struct Plan {
   size_t xp_bytes, rec_bytes, partial_bytes;
 };
 
-Plan plan_for(int M, int N, int G) {
+// LLMQ_A16_TILE=wide / narrow in the environment pins the tile shape whatever the problem (read per call; the
+// tests run shapes through both).
+int forced_shape() {
+  const char* v = getenv("LLMQ_A16_TILE");
+  if (v == nullptr) return 0;
+  return v[0] == 'w' ? 1 : (v[0] == 'n' ? 2 : 0);
+}
+
+// Whether the 64 x 128 tile is the faster one: outputs whose narrow tiles run in one round (a workgroup has a CU
+// to itself) and rows short enough that cutting the reduction axis of the wide tile instead (fp32 partial tiles,
+// a second launch) does not pay. Measured on int8, M x N x K: 512 x 3072 x 2048 24.4 us against 29.3,
+// 256 x 3072 x 2048 18.5 / 23.3, 512 x 3072 x 3072 34.0 / 30.3, 512 x 2048 x 4096 30.9 / 30.2,
+// 512 x 4096 x 4096 41.2 / 37.2.
+bool narrow_tile(int M, int N, int G) {
+  const int forced = forced_shape();
+  if (forced) return forced == 2;
+  const int narrow_tiles = ((M + Narrow::kBM - 1) / Narrow::kBM) * ((N + Narrow::kBN - 1) / Narrow::kBN);
+  return narrow_tiles <= 256 && G <= kNarrowMaxGroups;
+}
+
+Plan plan_for(int M, int N, int G, bool narrow = false) {
   Plan p{};
-  p.m_tiles = (M + kBM - 1) / kBM;
-  p.n_tiles = (N + kBN - 1) / kBN;
+  p.m_tiles = narrow ? (M + Narrow::kBM - 1) / Narrow::kBM : (M + kBM - 1) / kBM;
+  p.n_tiles = narrow ? (N + Narrow::kBN - 1) / Narrow::kBN : (N + kBN - 1) / kBN;
   const int tiles = p.m_tiles * p.n_tiles;
-  // fewer tiles than would occupy most CUs: cut the reduction axis, at least four groups per slice
+  // fewer tiles than would occupy most CUs: cut the reduction axis, at least four groups per slice and no more
+  // workgroups than CUs (a workgroup has a CU's LDS to itself: one over is a second round)
   int splits = 1;
   if (tiles < 160) {
-    splits = (256 + tiles - 1) / tiles;
+    splits = 256 / tiles;
     if (splits > G / 4) splits = G / 4;
     if (splits < 1) splits = 1;
   }
   p.groups_per_split = (G + splits - 1) / splits;
   p.splits = (G + p.groups_per_split - 1) / p.groups_per_split;  // every slice holds at least one group
-  // (rows padded to whole tiles: the kernel reads them without clamping; what the pad rows hold is never stored)
-  p.xp_bytes = aligned(static_cast<size_t>(p.m_tiles) * kBM * G * kRowBytes);
-  p.rec_bytes = aligned(static_cast<size_t>(p.m_tiles) * kBM * G * 16);
+  // (rows padded to whole wide tiles, which covers whole narrow ones: the kernel reads them without clamping; what
+  // the pad rows hold is never stored)
+  const size_t padded_rows = static_cast<size_t>((M + kBM - 1) / kBM) * kBM;
+  p.xp_bytes = aligned(padded_rows * G * kRowBytes);
+  p.rec_bytes = aligned(padded_rows * G * 16);
   p.partial_bytes = p.splits > 1 ? aligned(static_cast<size_t>(p.splits) * M * N * sizeof(float)) : 0;
   return p;
 }
@@ -527,8 +641,9 @@ Plan plan_for(int M, int N, int G) {
 
 extern "C" size_t llmq_wq_gemm_a16_tile_workspace_bytes(int M, int N, int G) {
   if (M <= 0 || N <= 0 || G <= 0) return 0;
-  const Plan p = plan_for(M, N, G);
-  return p.xp_bytes + p.rec_bytes + p.partial_bytes;
+  // (the larger of the two shapes' needs: the shape is chosen per call, and may be pinned from the environment)
+  const Plan w = plan_for(M, N, G, false), n = plan_for(M, N, G, true);
+  return w.xp_bytes + w.rec_bytes + (w.partial_bytes > n.partial_bytes ? w.partial_bytes : n.partial_bytes);
 }
 
 namespace {
@@ -569,7 +684,8 @@ int run_store(const void* x, const void* qweight, const float* wscale, void* out
   if (int rc = check_common(x, x == nullptr, qweight, wscale, workspace, M, N, G, gs, out_group, wformat, dtype)) return rc;
   if (M == 0 || N == 0) return 0;
   if (!out || (reinterpret_cast<uintptr_t>(out) & 15u)) return llmq_host::fail_invalid("out must be a 16-byte aligned pointer");
-  const Plan p = plan_for(M, N, G);
+  const bool narrow = narrow_tile(M, N, G);
+  const Plan p = plan_for(M, N, G, narrow);
   if (workspace_bytes < p.xp_bytes + p.rec_bytes + p.partial_bytes)
     return llmq_host::fail_invalid("workspace of %zu bytes is too small, need %zu", workspace_bytes,
                                    p.xp_bytes + p.rec_bytes + p.partial_bytes);
@@ -584,7 +700,10 @@ int run_store(const void* x, const void* qweight, const float* wscale, void* out
              p.m_tiles, p.n_tiles, p.splits, p.groups_per_split, nullptr, nullptr, 0};
   const int total = p.m_tiles * p.n_tiles * p.splits;
   const dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8));
-  if (int rc = wformat == LLMQ_W_INT4_PACKED ? launch_tiles<4, kEpiStore>(a, grid, s) : launch_tiles<8, kEpiStore>(a, grid, s)) return rc;
+  int rc;
+  if (narrow) rc = wformat == LLMQ_W_INT4_PACKED ? launch_tiles<4, kEpiStore, Narrow>(a, grid, s) : launch_tiles<8, kEpiStore, Narrow>(a, grid, s);
+  else rc = wformat == LLMQ_W_INT4_PACKED ? launch_tiles<4, kEpiStore>(a, grid, s) : launch_tiles<8, kEpiStore>(a, grid, s);
+  if (rc) return rc;
   if (p.splits > 1) {
     const int64_t count = static_cast<int64_t>(M) * N;
     hipLaunchKernelGGL(add_splits_kernel, dim3(static_cast<unsigned>((count / 4 + 256) / 256)), dim3(256), 0, s,

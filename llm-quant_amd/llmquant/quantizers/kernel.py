@@ -42,13 +42,27 @@ FUSED_GEMM_SPLIT_GROUPS = 1 << 30   # (no row is long enough for the split form 
 TILED_GEMM_MAX_ROWS = 1024
 
 
+#: The tiled GEMM's 64 x 128 tile: outputs it covers in one round of workgroups (one per CU) on rows of at most
+#: this many groups (csrc/wq_gemm_a16_tile.hip, narrow_tile)
+TILED_GEMM_NARROW_MAX_GROUPS = 16
+TILED_GEMM_NARROW_MAX_TILES = 256
+#: ... and from this many of those tiles (measured down to 192 x 3072: 72 tiles; smaller outputs stay with the library)
+TILED_GEMM_NARROW_MIN_TILES = 64
+
+
 def tiled_gemm_pays(rows: int, out_features: int, groups: int) -> bool:
     """Whether the tiled fused GEMM beats dequantize + matmul for this many activation rows: wide outputs
-    (enough 128 x 256 tiles to fill the chip) or long rows (the reduction axis is split instead). Narrow,
-    short weights (q|k|v, o_proj of a 1B model) have too few tiles either way and stay with the library."""
+    (enough 128 x 256 tiles to fill the chip), long rows (the reduction axis is split instead), or short rows on an
+    output that 64 x 128 tiles cover in one round (q|k|v of a 1B model at a 512-token prompt: 192 tiles)."""
     if not FUSED_GEMM_MAX_ROWS < rows <= TILED_GEMM_MAX_ROWS:
         return False
     if out_features >= 8192 or groups >= 64:
+        return True
+    # 512 x 3072 x 2048 int8 24.4 us against 24.4 for dequantize + matmul (int4 21.1 / 24.6), 512 x 4096 x 2048
+    # 23.6 / 26.6, 192 x 3072 x 2048 16.9 / 24.4; at most 5 % behind where it is behind (384 x 3072, 1024 x 2048)
+    narrow_tiles = -(-rows // 64) * -(-out_features // 128)
+    if (rows > FUSED_GEMM_SLAB_MAX_ROWS and groups <= TILED_GEMM_NARROW_MAX_GROUPS
+            and TILED_GEMM_NARROW_MIN_TILES <= narrow_tiles <= TILED_GEMM_NARROW_MAX_TILES):
         return True
     # one tile of rows on a mid-sized weight (Llama-3-8B's q|k|v, 6144 x 4096 int8, M = 65-128: 24.8-27.1 us against
     # 32.7-36.0 for dequantize + matmul); smaller weights take the fused GEMM for a few dozen rows twice instead

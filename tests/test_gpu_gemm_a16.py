@@ -141,9 +141,28 @@ def test_split_form_repeats_itself_and_checks_its_workspace(ext):
 # ---- the tiled form for prompt-sized M ---------------------------------------------------------------------
 
 
-def tile_case(ext, m, n, k, bits, out_group=0, head_dim=None, seed=0, scale=1.0, offset=0.0):
+#: The tiled GEMM has two tile shapes with the same arithmetic: 128 x 256 (eight waves) and 64 x 128 (four waves,
+#: for outputs of few wide tiles). LLMQ_A16_TILE pins one whatever the problem; None is the library's own choice.
+SHAPES = pytest.mark.parametrize("tile", ["wide", "narrow", None], ids=["128x256", "64x128", "own choice"])
+
+
+@pytest.fixture(autouse=True)
+def no_tile_shape_left_pinned():
+    import os
+
+    yield
+    os.environ.pop("LLMQ_A16_TILE", None)
+
+
+def tile_case(ext, m, n, k, bits, out_group=0, head_dim=None, seed=0, scale=1.0, offset=0.0, tile=None):
     """x [m, k] bf16 against a quantized [n, k] weight through wq_gemm_a16_tile; returns the result and the
     oracle's operands (activation padded the way the weight was)."""
+    import os
+
+    if tile is None:
+        os.environ.pop("LLMQ_A16_TILE", None)
+    else:
+        os.environ["LLMQ_A16_TILE"] = tile
     torch.manual_seed(seed)
     w = (torch.randn(n, k) * 0.02).to(torch.bfloat16)
     x = (torch.randn(m, k) * scale + offset).to(torch.bfloat16)
@@ -159,12 +178,13 @@ def tile_case(ext, m, n, k, bits, out_group=0, head_dim=None, seed=0, scale=1.0,
 @pytest.mark.parametrize("m,n,k", [(128, 256, 128), (65, 256, 256), (130, 300, 768), (512, 512, 2048), (300, 70, 384),
                                    (129, 257, 1152), (1, 16, 128), (256, 1024, 8192), (65, 70, 1024),
                                    (1023, 66, 2048)])
-def test_tiled_gemm_against_the_oracle(ext, bits, m, n, k):
+@SHAPES
+def test_tiled_gemm_against_the_oracle(ext, bits, m, n, k, tile):
     """Whole outputs against the float64 closed form and the real-mode forward: full tiles, ragged M and N
     (rows and columns past the end are clamped for the loads and dropped at the store), one group, rows long
     enough that the reduction axis is split across workgroups, and split outputs whose element count is not a
     multiple of four (the slice addition then walks its values one at a time)."""
-    got, x, canonical, scales = tile_case(ext, m, n, k, bits, seed=m + n)
+    got, x, canonical, scales = tile_case(ext, m, n, k, bits, seed=m + n, tile=tile)
     assert got.shape == (m, n) and got.dtype == torch.bfloat16
     exact = oracle.gemv_float64(x, canonical, scales)
     assert rel_l2(to_np(got), exact) <= 2e-3
@@ -196,14 +216,15 @@ PREFILL_SHAPES = {
 }
 
 
+@SHAPES
 @pytest.mark.parametrize("name", list(PREFILL_SHAPES))
-def test_tiled_gemm_at_the_prompt_pass_shapes(ext, name):
+def test_tiled_gemm_at_the_prompt_pass_shapes(ext, name, tile):
     """The four projections of a 512-token prompt pass of the Llama-3.2-1B configuration, on 96 x 128 sampled
     outputs (and the last rows and columns) against the float64 closed form, rel-L2 <= 2e-3, and against the
     real-mode forward restricted to the sample."""
     spec = dict(PREFILL_SHAPES[name])
     m, n, k, bits = 512, spec.pop("n"), spec.pop("k"), spec.pop("bits")
-    got, x, canonical, scales = tile_case(ext, m, n, k, bits, seed=11, **spec)
+    got, x, canonical, scales = tile_case(ext, m, n, k, bits, seed=11, tile=tile, **spec)
     out_group = spec.get("out_group")
     rng = np.random.default_rng(3)
     rows = np.unique(np.concatenate([rng.choice(m, 96, replace=False), [m - 1]]))
@@ -338,7 +359,12 @@ def test_gate_up_silu_epilogue_gives_the_bits_of_the_three_launches(ext, bits, m
     """llmq_wq_gemm_a16_tile_gate_up_silu + llmq_wq_gemm_a16_tile_prepared against llmq_wq_gemm_a16_tile ->
     llmq_silu_mul -> llmq_wq_gemm_a16_tile on the same operands: equal to the bit. (Reduction axes of at most
     seven groups here: there the plain tiled GEMM does not split the axis either, so its fp32 sums run in the
-    order of the fused launch's. The rounding points are the same in any case; the longer axis is below.)"""
+    order of the fused launch's. The rounding points are the same in any case; the longer axis is below. The
+    128 x 256 tile is pinned for the three launches: the epilogue is laid out for it, and the 64 x 128 tile adds
+    the two halves of every group separately.)"""
+    import os
+
+    os.environ["LLMQ_A16_TILE"] = "wide"
     x, q_gu, s_gu, q_d, s_d, _ = mlp_case(m, inter, k, n_down, bits, seed=m + inter, out_group=out_group)
     gate_up = ext.wq_gemm_a16_tile(x, q_gu, s_gu, out_group)
     act = ext.silu_mul(gate_up[:, :inter], gate_up[:, inter:])

@@ -171,6 +171,10 @@ def test_narrow_short_weights_keep_the_fused_gemm_up_to_128_rows():
     # a mid-sized weight (Llama-3-8B's q|k|v): one tile of rows goes to the tiled GEMM, more to the dense branch
     assert tiled_gemm_pays(100, 6144, 32) and tiled_gemm_pays(128, 6144, 32) and not tiled_gemm_pays(129, 6144, 32)
     assert not tiled_gemm_pays(100, 4096, 32) and not tiled_gemm_pays(100, 3072, 16)
+    # short rows on an output that 64 x 128 tiles cover in one round: q|k|v of Llama-3.2-1B at a 512-token prompt
+    assert tiled_gemm_pays(512, 3072, 16) and tiled_gemm_pays(192, 3072, 16) and tiled_gemm_pays(512, 4096, 16)
+    assert not tiled_gemm_pays(512, 3072, 24) and not tiled_gemm_pays(512, 2048, 32)   # longer rows: the library
+    assert not tiled_gemm_pays(1024, 3072, 16) and not tiled_gemm_pays(136, 512, 16)   # two rounds; a dozen tiles
 
 
 # ---- layout ---------------------------------------------------------------------------------------------
