@@ -243,8 +243,25 @@ int llmq_wq_gemm_a16_tile_gate_up_silu(const void* x, const void* qweight, const
                                        size_t workspace_bytes, void* next_workspace, size_t next_workspace_bytes,
                                        int M, int I, int G, int gs, int out_group, int wformat, int dtype,
                                        llmq_stream_t stream);
+/* llmq_wq_gemm_a16_tile_gate_up_silu on an activation that is already in `workspace` in prepared form (left there
+ * by llmq_add_rmsnorm_prepared): no x. */
+int llmq_wq_gemm_a16_tile_gate_up_silu_prepared(const void* qweight, const float* wscale, void* workspace,
+                                                size_t workspace_bytes, void* next_workspace,
+                                                size_t next_workspace_bytes, int M, int I, int G, int gs, int out_group,
+                                                int wformat, int dtype, llmq_stream_t stream);
+/* llmq_add_rmsnorm (below) whose normed rows are written in the tiled GEMM's prepared form into the first
+ * llmq_wq_gemm_a16_tile_prepared_bytes(rows, hidden / 128) bytes of `workspace` instead of as a tensor: what
+ * llmq_wq_gemm_a16_tile would make of that tensor, bit for bit, without the tensor and without the preparation
+ * launch; `workspace` is then the workspace of llmq_wq_gemm_a16_tile_prepared (q|k|v) or
+ * llmq_wq_gemm_a16_tile_gate_up_silu_prepared with M = rows, G = hidden / 128. LLMQ_BF16 only; hidden a multiple
+ * of 128; delta_or_null and sum_out_or_null as in llmq_add_rmsnorm. No counterpart in the reference (transformers'
+ * LlamaRMSNorm.forward followed by the Linear's M > 4 branch, llmquant/quantizers/kernel.py:68-79). */
+int llmq_add_rmsnorm_prepared(const void* x, const void* delta_or_null, const void* weight, void* sum_out_or_null,
+                              void* workspace, size_t workspace_bytes, int rows, int hidden, float eps, int dtype,
+                              llmq_stream_t stream);
 /* llmq_wq_gemm_a16_tile on an activation that is already in `workspace` in prepared form (left there by
- * llmq_wq_gemm_a16_tile_gate_up_silu): no x. workspace_bytes as for llmq_wq_gemm_a16_tile. */
+ * llmq_wq_gemm_a16_tile_gate_up_silu or llmq_add_rmsnorm_prepared): no x. workspace_bytes as for
+ * llmq_wq_gemm_a16_tile. */
 int llmq_wq_gemm_a16_tile_prepared(const void* qweight, const float* wscale, void* out, void* workspace,
                                    size_t workspace_bytes, int M, int N, int G, int gs, int out_group, int wformat,
                                    int dtype, llmq_stream_t stream);

@@ -679,12 +679,48 @@ at::Tensor wq_gemm_a16_tile_gate_up_silu(const at::Tensor& x, const at::Tensor& 
   return next;
 }
 
+// The same launch on an activation that is already in prepared form in `workspace` (from add_rmsnorm_prepared).
+at::Tensor wq_gemm_a16_tile_gate_up_silu_prepared(const at::Tensor& workspace, int64_t rows, const at::Tensor& qweight,
+                                                  const at::Tensor& wscale, int64_t out_group, int64_t next_n) {
+  TORCH_CHECK(workspace.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "workspace, qweight and wscale must be CUDA tensors");
+  TORCH_CHECK(workspace.scalar_type() == at::kFloat && workspace.dim() == 1 && workspace.is_contiguous(),
+              "workspace must be the tensor add_rmsnorm_prepared returned");
+  TORCH_CHECK(qweight.dim() == 3, "qweight must be [2 * intermediate, groups, group_size], got ", qweight.dim(), "D");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 2, "wscale must be float32 [scale_rows, groups]");
+  const auto wc = qweight.contiguous();
+  const auto sc = wscale.contiguous();
+  const int64_t M = rows, N = wc.size(0), groups = wc.size(1);
+  const int64_t group_size = packed ? wc.size(2) * 2 : wc.size(2);
+  TORCH_CHECK(group_size == 128, "the tiled fused GEMM needs group_size 128, got ", group_size);
+  TORCH_CHECK(N % 256 == 0, "gate rows followed by up rows, a multiple of 128 each: got ", N, " rows");
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  TORCH_CHECK(sc.size(0) == scale_rows && sc.size(1) == groups, "wscale must be [", scale_rows, ", ", groups, "]");
+  TORCH_CHECK(M > 0 && next_n > 0, "empty activation");
+  const int64_t inter = N / 2, next_groups = inter / 128;
+  const c10::OptionalDeviceGuard guard(at::device_of(workspace));
+  const size_t need = llmq_wq_gemm_a16_tile_prepared_bytes(static_cast<int>(M), static_cast<int>(groups));
+  TORCH_CHECK(static_cast<size_t>(workspace.numel()) * 4 >= need, "workspace holds ", workspace.numel() * 4, " bytes, this GEMM needs ", need);
+  const size_t next_need = llmq_wq_gemm_a16_tile_workspace_bytes(static_cast<int>(M), static_cast<int>(next_n), static_cast<int>(next_groups));
+  auto next = at::empty({static_cast<int64_t>((next_need + 3) / 4)}, workspace.options());
+  check_rc(llmq_wq_gemm_a16_tile_gate_up_silu_prepared(wc.const_data_ptr(), sc.const_data_ptr<float>(),
+                                                       workspace.mutable_data_ptr(), static_cast<size_t>(workspace.numel()) * 4,
+                                                       next.mutable_data_ptr(), next_need, static_cast<int>(M),
+                                                       static_cast<int>(inter), static_cast<int>(groups),
+                                                       static_cast<int>(group_size), static_cast<int>(out_group),
+                                                       packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, LLMQ_BF16,
+                                                       current_stream(workspace)),
+           "wq_gemm_a16_tile_gate_up_silu_prepared");
+  return next;
+}
+
 // The tiled GEMM on a prepared activation of `rows` rows sitting in `workspace` (from wq_gemm_a16_tile_gate_up_silu).
 at::Tensor wq_gemm_a16_tile_prepared(const at::Tensor& workspace, int64_t rows, const at::Tensor& qweight,
                                      const at::Tensor& wscale, int64_t out_group) {
   TORCH_CHECK(workspace.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "workspace, qweight and wscale must be CUDA tensors");
   TORCH_CHECK(workspace.scalar_type() == at::kFloat && workspace.dim() == 1 && workspace.is_contiguous(),
-              "workspace must be the tensor wq_gemm_a16_tile_gate_up_silu returned");
+              "workspace must be the tensor wq_gemm_a16_tile_gate_up_silu or add_rmsnorm_prepared returned");
   TORCH_CHECK(qweight.dim() == 3, "qweight must be [N, groups, group_size], got ", qweight.dim(), "D");
   const bool packed = qweight.scalar_type() == at::kByte;
   TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
@@ -749,6 +785,37 @@ std::tuple<at::Tensor, at::Tensor> add_rmsnorm(const at::Tensor& x, const at::Te
                             static_cast<float>(eps), dtype_code(xc, "x"), current_stream(xc)),
            "add_rmsnorm");
   return {sum, out};
+}
+
+// LlamaRMSNorm(x + delta) (delta None: of x) written as the prepared activation of a tiled GEMM on a weight of
+// next_n rows: returns (x + delta or x, that GEMM's workspace), the workspace to be handed to
+// wq_gemm_a16_tile_prepared or wq_gemm_a16_tile_gate_up_silu_prepared with rows = the rows of x.
+std::tuple<at::Tensor, at::Tensor> add_rmsnorm_prepared(const at::Tensor& x, const c10::optional<at::Tensor>& delta,
+                                                        const at::Tensor& weight, double eps, int64_t next_n) {
+  TORCH_CHECK(x.is_cuda() && weight.is_cuda(), "x and weight must be CUDA tensors");
+  TORCH_CHECK(x.scalar_type() == at::kBFloat16, "the prepared form is of bfloat16 activations");
+  TORCH_CHECK(x.dim() == 2 && weight.dim() == 1 && weight.size(0) == x.size(1), "x must be [rows, hidden], weight [hidden]");
+  TORCH_CHECK(weight.scalar_type() == x.scalar_type(), "weight must have x's dtype");
+  TORCH_CHECK(x.size(0) > 0 && next_n > 0, "empty activation");
+  const auto xc = x.contiguous();
+  const auto wc = weight.contiguous();
+  at::Tensor dc, sum = xc;
+  if (delta.has_value()) {
+    TORCH_CHECK(delta->is_cuda() && delta->sizes() == x.sizes() && delta->scalar_type() == x.scalar_type(), "x and delta must match");
+    dc = delta->contiguous();
+    sum = at::empty_like(xc);
+  }
+  const int64_t rows = xc.size(0), hidden = xc.size(1);
+  TORCH_CHECK(hidden % 128 == 0, "hidden must be a multiple of 128, got ", hidden);
+  const c10::OptionalDeviceGuard guard(at::device_of(xc));
+  const size_t need = llmq_wq_gemm_a16_tile_workspace_bytes(static_cast<int>(rows), static_cast<int>(next_n), static_cast<int>(hidden / 128));
+  auto workspace = at::empty({static_cast<int64_t>((need + 3) / 4)}, xc.options().dtype(at::kFloat));
+  check_rc(llmq_add_rmsnorm_prepared(xc.const_data_ptr(), delta.has_value() ? dc.const_data_ptr() : nullptr,
+                                     wc.const_data_ptr(), delta.has_value() ? sum.mutable_data_ptr() : nullptr,
+                                     workspace.mutable_data_ptr(), need, static_cast<int>(rows), static_cast<int>(hidden),
+                                     static_cast<float>(eps), LLMQ_BF16, current_stream(xc)),
+           "add_rmsnorm_prepared");
+  return {sum, workspace};
 }
 
 // q [tokens, q_heads * D], k [tokens, kv_heads * D] (rows may be strided), cos / sin [tokens, D].
@@ -1278,6 +1345,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("wq_gemm_a16_tile_gate_up_silu", &wq_gemm_a16_tile_gate_up_silu,
         "gate|up tiled GEMM whose workgroups write silu(gate) * up as the next tiled GEMM's prepared activation",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("next_n"));
+  m.def("wq_gemm_a16_tile_gate_up_silu_prepared", &wq_gemm_a16_tile_gate_up_silu_prepared,
+        "wq_gemm_a16_tile_gate_up_silu on the prepared activation add_rmsnorm_prepared left in its workspace",
+        py::arg("workspace"), py::arg("rows"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0,
+        py::arg("next_n"));
+  m.def("add_rmsnorm_prepared", &add_rmsnorm_prepared,
+        "(x + delta, workspace): LlamaRMSNorm(x + delta) written as the prepared activation of a tiled GEMM, one launch",
+        py::arg("x"), py::arg("delta"), py::arg("weight"), py::arg("eps"), py::arg("next_n"));
   m.def("wq_gemm_a16_tile_prepared", &wq_gemm_a16_tile_prepared,
         "the tiled GEMM on the prepared activation wq_gemm_a16_tile_gate_up_silu left in its workspace",
         py::arg("workspace"), py::arg("rows"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0);

@@ -126,6 +126,58 @@ __global__ __launch_bounds__(256) void act_prep_kernel(const u32x4* __restrict__
   emit_prepared(v, active, (threadIdx.x & 15) == 0, xp + (active ? i : 0), rec + (active ? i >> 4 : 0));
 }
 
+// LlamaRMSNorm (optionally on x + delta, the residual add in front of it, which is stored as well) whose result
+// goes straight into prepared form: what act_prep_kernel would make of llmq_add_rmsnorm's output, without that
+// tensor and without the second launch. One workgroup per row, the arithmetic and rounding points of
+// rmsnorm_kernel (csrc/prefill_ops.hip): out = w * bf16(x_f32 * rsqrt(mean(x_f32^2) + eps)), rounded to bf16.
+// hidden is a multiple of 128, so the 16 lanes of a (row, group) are in the loop together.
+constexpr int kNormThreads = 256;
+template <bool ADD>
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_prep_kernel(const bf16_t* __restrict__ x,
+                                                                   const bf16_t* __restrict__ delta,
+                                                                   const bf16_t* __restrict__ w,
+                                                                   bf16_t* __restrict__ sum_out, u32x4* __restrict__ xp,
+                                                                   u32x4* __restrict__ rec, const int hidden,
+                                                                   const float eps) {
+  __shared__ float red[kNormThreads / kWave];
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * hidden;
+  const bf16_t* row = x + base;
+  const int tid = threadIdx.x;
+  float ss = 0.0f;
+  for (int i = tid * 8; i < hidden; i += kNormThreads * 8) {
+    float f[8];
+    Pack<bf16_t>::unpack(load16(row + i), f);
+    if constexpr (ADD) {
+      float d[8];
+      Pack<bf16_t>::unpack(load16(delta + base + i), d);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = round_through<bf16_t>(f[e] + d[e]);
+      store16(sum_out + base + i, Pack<bf16_t>::pack(f));
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss = fmaf(f[e], f[e], ss);
+  }
+  ss = wave_sum(ss);
+  if ((tid & (kWave - 1)) == 0) red[tid / kWave] = ss;
+  __syncthreads();
+  float total = 0.0f;
+#pragma unroll
+  for (int k = 0; k < kNormThreads / kWave; ++k) total += red[k];
+  const float inv_rms = rsqrtf(total / static_cast<float>(hidden) + eps);
+  // (with ADD a thread reads back exactly the packets it stored above)
+  const bf16_t* src = ADD ? sum_out + base : row;
+  const int64_t chunk0 = base >> 3;   // the row's first chunk; 16 chunks a group
+  for (int i = tid * 8; i < hidden; i += kNormThreads * 8) {
+    float f[8], g[8];
+    Pack<bf16_t>::unpack(load16(src + i), f);
+    Pack<bf16_t>::unpack(load16(w + i), g);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = g[e] * round_through<bf16_t>(f[e] * inv_rms);
+    const int64_t chunk = chunk0 + (i >> 3);
+    emit_prepared(Pack<bf16_t>::pack(f), true, (tid & 15) == 0, xp + chunk, rec + (chunk >> 4));
+  }
+}
+
 struct TileArgs {
   const uint8_t* xp;   // [M, G*128] bf16, chunks reordered
   const uint8_t* rec;  // [M, G] records of 16 bytes
@@ -214,7 +266,8 @@ __global__ __launch_bounds__(S::kThreads, 1) void wq_gemm_a16_tile_kernel(const 
   const int nt = (logical / a.m_tiles) % a.n_tiles;
   const int sp = logical / (a.m_tiles * a.n_tiles);
 
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  // (the wave's index as a scalar: LDS addresses of the transfers are then scalar arithmetic into M0)
+  const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
   // every wave all the rows, 32 of the columns, and half kh of every group's k-steps (kKH == 1: all of them)
   const int wm = 0, wn = wv % S::kColWaves;
   const int kh = kKH == 1 ? 0 : __builtin_amdgcn_readfirstlane(wv / S::kColWaves);
@@ -270,28 +323,35 @@ __global__ __launch_bounds__(S::kThreads, 1) void wq_gemm_a16_tile_kernel(const 
     sw_lane = a.sw + static_cast<int64_t>(a.out_group > 0 ? n / a.out_group : n) * a.G;
   }
 
+  // (a lane's 32-bit offset goes through an empty asm where it is used: the compiler then adds it to the scalar
+  // base inside the instruction, scalar base + 32-bit lane offset, instead of keeping a 64-bit address per lane
+  // and transfer across the loop and adding the group's step to each with the vector ALU)
+  auto here = [](uint32_t offset) {
+    asm volatile("" : "+v"(offset));
+    return offset;
+  };
   auto request = [&](int g, int buf) {
     uint8_t* stage = smem + buf * kStageB;
     const uint8_t* xg = a.xp + static_cast<uint32_t>(g) * kRowBytes;
 #pragma unroll
     for (int i = 0; i < kXInstr; ++i) {
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(xg + x_off[i]),
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(xg + here(x_off[i])),
                                        reinterpret_cast<u32x4*>(stage + (wv * (kBM / kWaves) + i * 4) * kRowBytes), 16,
                                        0, 0);
     }
     const uint8_t* wg = a.qw + static_cast<uint32_t>(g) * kCodeRowBytes<BITS>;
 #pragma unroll
     for (int i = 0; i < kCodeInstr; ++i) {
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(wg + w_off[i]),
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(wg + here(w_off[i])),
                                        reinterpret_cast<u32x4*>(stage + kTileBytes + (wv * kCodeInstr + i) * 1024), 16,
                                        0, 0);
     }
     if (wv < kLeftCodes) {
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(wg + w_off[kCodeInstr]),
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(wg + here(w_off[kCodeInstr])),
                                        reinterpret_cast<u32x4*>(stage + kTileBytes + (kWaves * kCodeInstr + wv) * 1024),
                                        16, 0, 0);
     } else if (wv < kLeftCodes + kRecWaves) {
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(a.rec + r_off + static_cast<uint32_t>(g) * 16),
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4*>(a.rec + static_cast<uint32_t>(g) * 16 + here(r_off)),
                                        reinterpret_cast<u32x4*>(stage + kTileBytes + kCodeTileB + rec_wave * 1024),
                                        16, 0, 0);
     } else if (wv < kExtraWaves) {
@@ -583,8 +643,6 @@ int launch_tiles(const TileArgs& a, dim3 grid, hipStream_t stream) {
   return llmq_host::check_launch("wq_gemm_a16_tile_kernel");
 }
 
-// rows of up to this many groups take the narrow tile when the wide one would have to cut the reduction axis
-constexpr int kNarrowMaxGroups = 16;
 constexpr size_t kAlign = 256;
 size_t aligned(size_t bytes) { return (bytes + kAlign - 1) / kAlign * kAlign; }
 
@@ -599,18 +657,6 @@ int forced_shape() {
   const char* v = getenv("LLMQ_A16_TILE");
   if (v == nullptr) return 0;
   return v[0] == 'w' ? 1 : (v[0] == 'n' ? 2 : 0);
-}
-
-// Whether the 64 x 128 tile is the faster one: outputs whose narrow tiles run in one round (a workgroup has a CU
-// to itself) and rows short enough that cutting the reduction axis of the wide tile instead (fp32 partial tiles,
-// a second launch) does not pay. Measured on int8, M x N x K: 512 x 3072 x 2048 24.4 us against 29.3,
-// 256 x 3072 x 2048 18.5 / 23.3, 512 x 3072 x 3072 34.0 / 30.3, 512 x 2048 x 4096 30.9 / 30.2,
-// 512 x 4096 x 4096 41.2 / 37.2.
-bool narrow_tile(int M, int N, int G) {
-  const int forced = forced_shape();
-  if (forced) return forced == 2;
-  const int narrow_tiles = ((M + Narrow::kBM - 1) / Narrow::kBM) * ((N + Narrow::kBN - 1) / Narrow::kBN);
-  return narrow_tiles <= 256 && G <= kNarrowMaxGroups;
 }
 
 Plan plan_for(int M, int N, int G, bool narrow = false) {
@@ -635,6 +681,31 @@ Plan plan_for(int M, int N, int G, bool narrow = false) {
   p.rec_bytes = aligned(padded_rows * G * 16);
   p.partial_bytes = p.splits > 1 ? aligned(static_cast<size_t>(p.splits) * M * N * sizeof(float)) : 0;
   return p;
+}
+
+// What a plan costs, in microseconds, from the measured shape of a launch: rounds of 256 workgroups, each a fixed
+// part (first transfers from memory, the store) plus a time per group of the reduction axis (wide 8 + 1.93 / 2.1 a
+// group for int4 / int8, narrow 6 + 0.75 / 1.0), and where the axis is cut the partial tiles' way through memory
+// and the second launch (3 us + 8 bytes per partial value at 9 TB/s: most of it overlaps the tiles). Within a
+// tenth of the measured launches.
+double plan_cost(const Plan& p, int M, int N, bool narrow, bool int4) {
+  const double fixed = narrow ? 6.0 : 8.0;
+  const double per_group = narrow ? (int4 ? 0.75 : 1.0) : (int4 ? 1.93 : 2.1);
+  const int workgroups = p.m_tiles * p.n_tiles * p.splits;
+  const double rounds = static_cast<double>((workgroups + 255) / 256);
+  double cost = rounds * (fixed + p.groups_per_split * per_group);
+  if (p.splits > 1) cost += 3.0 + static_cast<double>(p.splits) * M * N * 8.0 / 9.0e6;
+  return cost;
+}
+
+// Whether the 64 x 128 tile is the faster one: outputs of few 128 x 256 tiles, where the narrow tile fills the
+// chip without cutting the reduction axis (512 x 3072 x 2048 int8: 24.4 us against 29.3; 128 x 14336 x 4096 int4:
+// 31.7 / 36.4), and not where its tiles need a second round (1024 x 3072 x 2048: 42.6 / 33.0) or the rows are long
+// enough for the wide tile's slices to pay for their partial sums (512 x 4096 x 4096: 41.2 / 37.2).
+bool narrow_tile(int M, int N, int G, bool int4) {
+  const int forced = forced_shape();
+  if (forced) return forced == 2;
+  return plan_cost(plan_for(M, N, G, true), M, N, true, int4) < plan_cost(plan_for(M, N, G, false), M, N, false, int4);
 }
 
 }  // namespace
@@ -684,7 +755,7 @@ int run_store(const void* x, const void* qweight, const float* wscale, void* out
   if (int rc = check_common(x, x == nullptr, qweight, wscale, workspace, M, N, G, gs, out_group, wformat, dtype)) return rc;
   if (M == 0 || N == 0) return 0;
   if (!out || (reinterpret_cast<uintptr_t>(out) & 15u)) return llmq_host::fail_invalid("out must be a 16-byte aligned pointer");
-  const bool narrow = narrow_tile(M, N, G);
+  const bool narrow = narrow_tile(M, N, G, wformat == LLMQ_W_INT4_PACKED);
   const Plan p = plan_for(M, N, G, narrow);
   if (workspace_bytes < p.xp_bytes + p.rec_bytes + p.partial_bytes)
     return llmq_host::fail_invalid("workspace of %zu bytes is too small, need %zu", workspace_bytes,
@@ -736,12 +807,14 @@ extern "C" size_t llmq_wq_gemm_a16_tile_prepared_bytes(int M, int G) {
   return p.xp_bytes + p.rec_bytes;
 }
 
-extern "C" int llmq_wq_gemm_a16_tile_gate_up_silu(const void* x, const void* qweight, const float* wscale,
-                                                  void* workspace, size_t workspace_bytes, void* next_workspace,
-                                                  size_t next_workspace_bytes, int M, int I, int G, int gs,
-                                                  int out_group, int wformat, int dtype, llmq_stream_t stream) {
+namespace {
+
+// x null: the activation is already in `workspace` in prepared form.
+int run_gate_up_silu(const void* x, const void* qweight, const float* wscale, void* workspace, size_t workspace_bytes,
+                     void* next_workspace, size_t next_workspace_bytes, int M, int I, int G, int gs, int out_group,
+                     int wformat, int dtype, llmq_stream_t stream) {
   if (I < 0 || I > (1 << 29)) return llmq_host::fail_invalid("bad intermediate size %d", I);
-  if (int rc = check_common(x, false, qweight, wscale, workspace, M, 2 * I, G, gs, out_group, wformat, dtype)) return rc;
+  if (int rc = check_common(x, x == nullptr, qweight, wscale, workspace, M, 2 * I, G, gs, out_group, wformat, dtype)) return rc;
   if (M == 0 || I == 0) return 0;
   if (I % (kBN / 2)) return llmq_host::fail_invalid("the intermediate size must be a multiple of %d, got %d", kBN / 2, I);
   if (!next_workspace || (reinterpret_cast<uintptr_t>(next_workspace) & 15u))
@@ -760,7 +833,9 @@ extern "C" int llmq_wq_gemm_a16_tile_gate_up_silu(const void* x, const void* qwe
   uint8_t* ws = static_cast<uint8_t*>(workspace);
   uint8_t* xp = ws;
   uint8_t* rec = ws + p.xp_bytes;
-  if (int rc = prepare(x, xp, rec, M, G, s)) return rc;
+  if (x != nullptr) {
+    if (int rc = prepare(x, xp, rec, M, G, s)) return rc;
+  }
   uint8_t* nws = static_cast<uint8_t*>(next_workspace);
   // whole reduction axis per workgroup: a tile's epilogue needs its finished totals
   TileArgs a{xp, rec, static_cast<const uint8_t*>(qweight), wscale, nullptr, nullptr, M, 2 * I, G, out_group,
@@ -768,4 +843,59 @@ extern "C" int llmq_wq_gemm_a16_tile_gate_up_silu(const void* x, const void* qwe
   const int total = a.m_tiles * a.n_tiles;
   const dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8));
   return wformat == LLMQ_W_INT4_PACKED ? launch_tiles<4, kEpiGateUpSilu>(a, grid, s) : launch_tiles<8, kEpiGateUpSilu>(a, grid, s);
+}
+
+}  // namespace
+
+extern "C" int llmq_wq_gemm_a16_tile_gate_up_silu(const void* x, const void* qweight, const float* wscale,
+                                                  void* workspace, size_t workspace_bytes, void* next_workspace,
+                                                  size_t next_workspace_bytes, int M, int I, int G, int gs,
+                                                  int out_group, int wformat, int dtype, llmq_stream_t stream) {
+  if (M > 0 && I > 0 && !x) return llmq_host::fail_invalid("null tensor pointer");
+  return run_gate_up_silu(x, qweight, wscale, workspace, workspace_bytes, next_workspace, next_workspace_bytes, M, I,
+                          G, gs, out_group, wformat, dtype, stream);
+}
+
+extern "C" int llmq_wq_gemm_a16_tile_gate_up_silu_prepared(const void* qweight, const float* wscale, void* workspace,
+                                                           size_t workspace_bytes, void* next_workspace,
+                                                           size_t next_workspace_bytes, int M, int I, int G, int gs,
+                                                           int out_group, int wformat, int dtype,
+                                                           llmq_stream_t stream) {
+  return run_gate_up_silu(nullptr, qweight, wscale, workspace, workspace_bytes, next_workspace, next_workspace_bytes,
+                          M, I, G, gs, out_group, wformat, dtype, stream);
+}
+
+extern "C" int llmq_add_rmsnorm_prepared(const void* x, const void* delta_or_null, const void* weight,
+                                         void* sum_out_or_null, void* workspace, size_t workspace_bytes, int rows,
+                                         int hidden, float eps, int dtype, llmq_stream_t stream) {
+  if (rows < 0 || hidden <= 0) return llmq_host::fail_invalid("bad dimension rows=%d hidden=%d", rows, hidden);
+  if (dtype != LLMQ_BF16) return llmq_host::fail_invalid("the prepared form is of bfloat16 activations, got dtype code %d", dtype);
+  if (hidden % kGroup) return llmq_host::fail_invalid("hidden must be a multiple of %d, got %d", kGroup, hidden);
+  if (rows == 0) return 0;
+  if (!x || !weight || !workspace) return llmq_host::fail_invalid("null tensor pointer");
+  if ((delta_or_null == nullptr) != (sum_out_or_null == nullptr))
+    return llmq_host::fail_invalid("delta and sum_out go together");
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(workspace) |
+       reinterpret_cast<uintptr_t>(delta_or_null) | reinterpret_cast<uintptr_t>(sum_out_or_null)) & 15u)
+    return llmq_host::fail_invalid("tensors and the workspace must be 16-byte aligned");
+  const int G = hidden / kGroup;
+  if ((static_cast<uint64_t>(rows) + kBM) * G * kRowBytes >= (1ull << 32))
+    return llmq_host::fail_invalid("activation of %d x %d values is beyond the tiled GEMM's 32-bit offsets", rows, hidden);
+  const Plan p = plan_for(rows, kBN, G);
+  if (workspace_bytes < p.xp_bytes + p.rec_bytes)
+    return llmq_host::fail_invalid("workspace of %zu bytes is too small, need %zu", workspace_bytes, p.xp_bytes + p.rec_bytes);
+  uint8_t* ws = static_cast<uint8_t*>(workspace);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (delta_or_null) {
+    hipLaunchKernelGGL(rmsnorm_prep_kernel<true>, dim3(rows), dim3(kNormThreads), 0, s, static_cast<const bf16_t*>(x),
+                       static_cast<const bf16_t*>(delta_or_null), static_cast<const bf16_t*>(weight),
+                       static_cast<bf16_t*>(sum_out_or_null), reinterpret_cast<u32x4*>(ws),
+                       reinterpret_cast<u32x4*>(ws + p.xp_bytes), hidden, eps);
+  } else {
+    hipLaunchKernelGGL(rmsnorm_prep_kernel<false>, dim3(rows), dim3(kNormThreads), 0, s, static_cast<const bf16_t*>(x),
+                       static_cast<const bf16_t*>(nullptr), static_cast<const bf16_t*>(weight),
+                       static_cast<bf16_t*>(nullptr), reinterpret_cast<u32x4*>(ws),
+                       reinterpret_cast<u32x4*>(ws + p.xp_bytes), hidden, eps);
+  }
+  return llmq_host::check_launch("rmsnorm_prep_kernel");
 }

@@ -137,6 +137,11 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_wq_gemm_a16_tile_gate_up_silu.argtypes = ([c_p] * 4 + [ctypes.c_size_t, c_p, ctypes.c_size_t] + [c_int] * 7
                                                        + [c_p])
     lib.llmq_wq_gemm_a16_tile_gate_up_silu.restype = c_int
+    lib.llmq_wq_gemm_a16_tile_gate_up_silu_prepared.argtypes = ([c_p] * 3 + [ctypes.c_size_t, c_p, ctypes.c_size_t]
+                                                                + [c_int] * 7 + [c_p])
+    lib.llmq_wq_gemm_a16_tile_gate_up_silu_prepared.restype = c_int
+    lib.llmq_add_rmsnorm_prepared.argtypes = [c_p] * 5 + [ctypes.c_size_t, c_int, c_int, ctypes.c_float, c_int, c_p]
+    lib.llmq_add_rmsnorm_prepared.restype = c_int
     lib.llmq_wq_gemm_a16_tile_prepared.argtypes = [c_p] * 4 + [ctypes.c_size_t] + [c_int] * 7 + [c_p]
     lib.llmq_wq_gemm_a16_tile_prepared.restype = c_int
     lib.llmq_wq_gemm_a16_tile_workspace_bytes.restype = ctypes.c_size_t

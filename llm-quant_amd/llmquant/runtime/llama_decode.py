@@ -98,9 +98,10 @@ class LlamaKernelRuntime:
             return self._ext.rmsnorm(x, module.weight, module.variance_epsilon)
         return module(x)
 
-    def _add_norm(self, module, hidden, branch):
+    def _add_norm(self, module, hidden, branch, consumer=None):
         """(hidden + branch, norm(hidden + branch)): the residual add in the launch of the norm after it.
-        branch None: (hidden, norm(hidden))."""
+        branch None: (hidden, norm(hidden)). `consumer`: ("qkv" | "mlp", layer index) when the normed rows go
+        to that projection of a prompt pass and nowhere else (a runtime may then hand them over in another form)."""
         if branch is None:
             return hidden, self._norm(module, hidden)
         if (self._one_launch_ops and type(module).__name__.endswith("RMSNorm") and hasattr(module, "variance_epsilon")
@@ -152,7 +153,7 @@ class LlamaKernelRuntime:
         leave the last add to the caller's next norm; otherwise the layer's output."""
         attn = layer.self_attn
         tokens = hidden.shape[0]
-        hidden, x = self._add_norm(layer.input_layernorm, hidden, branch)
+        hidden, x = self._add_norm(layer.input_layernorm, hidden, branch, None if decode else ("qkv", index))
         q, k, v = self._qkv(index, layer, x)
         k_dq = v_dq = None
         if not decode and self._rope_append_in_one_launch(q, k, v, cos):
@@ -183,7 +184,8 @@ class LlamaKernelRuntime:
             ctx = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k_dq[None], v_dq[None],
                                                  is_causal=True, scale=self.scaling, enable_gqa=True)
             ctx = ctx[0].transpose(0, 1).reshape(tokens, -1)
-        hidden, x = self._add_norm(layer.post_attention_layernorm, hidden, attn.o_proj(ctx))
+        hidden, x = self._add_norm(layer.post_attention_layernorm, hidden, attn.o_proj(ctx),
+                                   None if decode else ("mlp", index))
         out = self._mlp(index, layer, x)
         return (hidden, out) if defer else hidden + out
 

@@ -54,6 +54,14 @@ MID_CONTEXT_FROM = 5120
 LONG_CONTEXT_FROM = 16384
 
 
+class PreparedRows:
+    """Normed rows of a prompt in the tiled fused GEMM's prepared form (operand order, per-group sums) inside that
+    GEMM's workspace, in place of the tensor: what llmq_add_rmsnorm_prepared leaves."""
+
+    def __init__(self, workspace, rows, dtype):
+        self.workspace, self.rows, self.dtype = workspace, rows, dtype
+
+
 class _Fused:
     """Concatenated storage of Linears that read the same activation."""
 
@@ -171,12 +179,57 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         self._argmax_ws = torch.zeros(self._ext.argmax_workspace_ints(), dtype=torch.int32, device=self.device)
 
     # ---- the prompt pass: q|k|v and gate|up as one projection each ----------------------------------
+    def _takes_tile(self, rows, dtype, fused):
+        """Whether _project sends this many rows of this dtype to the tiled fused GEMM."""
+        from llmquant.quantizers.kernel import KERNEL_MAX_ROWS, fused_gemm_takes, tiled_gemm_pays
+
+        n, groups = fused.qdata.shape[0], fused.qdata.shape[1]
+        return (dtype == torch.bfloat16 and rows > KERNEL_MAX_ROWS and not fused_gemm_takes(rows, n, groups)
+                and tiled_gemm_pays(rows, n, groups))
+
+    def _mlp_in_two_launches(self, rows, dtype, index, layer):
+        """Whether _mlp runs this many rows as gate|up with the activation in its store + down_proj."""
+        from llmquant.quantizers.kernel import FUSED_GEMM_MAX_ROWS, TILED_GEMM_MAX_ROWS, tiled_gemm_pays
+
+        f = self.fused_layers[index]
+        gate_up, down = f["gate_up"], f["down"]
+        inter = gate_up.qdata.shape[0] // 2
+        return (dtype == torch.bfloat16 and self._one_launch_ops and "SiLU" in type(layer.mlp.act_fn).__name__
+                and FUSED_GEMM_MAX_ROWS < rows <= TILED_GEMM_MAX_ROWS and inter % 128 == 0
+                and -(-rows // 128) * (inter // 128) >= 160
+                and tiled_gemm_pays(rows, down.out_features, down.qdata.shape[1])
+                and down.bias is None and not down._needs_padding and not down._int8_act
+                and down.qdata.shape[1] * 128 == inter)
+
+    def _add_norm(self, module, hidden, branch, consumer=None):
+        """The base class's, except that rows on their way to a tiled fused GEMM leave the norm in that GEMM's
+        prepared form (llmq_add_rmsnorm_prepared: the bits of norm + preparation, one launch and one tensor
+        fewer): the second value is then a PreparedRows for _project / _mlp."""
+        if (consumer is not None and self._one_launch_ops and hidden.dim() == 2 and hidden.dtype == torch.bfloat16
+                and type(module).__name__.endswith("RMSNorm") and hasattr(module, "variance_epsilon")
+                and hidden.shape[-1] % 128 == 0 and module.weight.dtype == hidden.dtype
+                and (branch is None or branch.dtype == hidden.dtype)):
+            kind, index = consumer
+            rows, f = hidden.shape[0], self.fused_layers[index]
+            fused = f["qkv"] if kind == "qkv" else f["gate_up"]
+            direct = isinstance(fused, _Fused) and fused.qdata.shape[1] * 128 == hidden.shape[-1]
+            if direct and (self._takes_tile(rows, hidden.dtype, fused)
+                           or (kind == "mlp" and self._mlp_in_two_launches(rows, hidden.dtype, index,
+                                                                          self.layers[index]))):
+                next_n = max(fused.qdata.shape[0], f["down"].out_features if kind == "mlp" else 0)
+                hidden, workspace = self._ext.add_rmsnorm_prepared(hidden, branch, module.weight,
+                                                                   module.variance_epsilon, next_n)
+                return hidden, PreparedRows(workspace, rows, hidden.dtype)
+        return super()._add_norm(module, hidden, branch, consumer)
+
     def _project(self, x, fused):
         """x [tokens, K] times a concatenated weight: what KernelQuantLinear.forward would pick for this
         many rows, once for the whole concatenation (three or two matmuls and dequantize passes fewer
         per layer, and the host's matmul dispatch is the longest part of a prompt pass)."""
         from llmquant.quantizers.kernel import KERNEL_MAX_ROWS, fused_gemm_splits, fused_gemm_takes, tiled_gemm_pays
 
+        if isinstance(x, PreparedRows):   # (_add_norm found that these rows take the tiled GEMM)
+            return self._ext.wq_gemm_a16_tile_prepared(x.workspace, x.rows, fused.qdata, fused.wscale, fused.out_group)
         rows = x.shape[0]
         if (fused_gemm_takes(rows, fused.qdata.shape[0], fused.qdata.shape[1])
                 and x.dtype in (torch.bfloat16, torch.float16)):
@@ -205,19 +258,17 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         silu(gate) * up straight into down_proj's prepared activation (the bits of the three launches: the
         condition on the tile count is the one under which the plain gate|up GEMM keeps its reduction axis
         whole as well)."""
-        from llmquant.quantizers.kernel import FUSED_GEMM_MAX_ROWS, TILED_GEMM_MAX_ROWS, tiled_gemm_pays
-
         f = self.fused_layers[index]
         gate_up, down = f["gate_up"], f["down"]
-        rows, inter = x.shape[0], gate_up.qdata.shape[0] // 2
-        if (x.dtype == torch.bfloat16 and self._one_launch_ops and "SiLU" in type(layer.mlp.act_fn).__name__
-                and FUSED_GEMM_MAX_ROWS < rows <= TILED_GEMM_MAX_ROWS and inter % 128 == 0
-                and -(-rows // 128) * (inter // 128) >= 160
-                and tiled_gemm_pays(rows, down.out_features, down.qdata.shape[1])
-                and down.bias is None and not down._needs_padding and not down._int8_act
-                and down.qdata.shape[1] * 128 == inter):
-            workspace = self._ext.wq_gemm_a16_tile_gate_up_silu(x.contiguous(), gate_up.qdata, gate_up.wscale,
-                                                                gate_up.out_group, down.out_features)
+        rows = x.rows if isinstance(x, PreparedRows) else x.shape[0]
+        if self._mlp_in_two_launches(rows, x.dtype, index, layer):
+            if isinstance(x, PreparedRows):
+                workspace = self._ext.wq_gemm_a16_tile_gate_up_silu_prepared(x.workspace, rows, gate_up.qdata,
+                                                                             gate_up.wscale, gate_up.out_group,
+                                                                             down.out_features)
+            else:
+                workspace = self._ext.wq_gemm_a16_tile_gate_up_silu(x.contiguous(), gate_up.qdata, gate_up.wscale,
+                                                                    gate_up.out_group, down.out_features)
             return self._ext.wq_gemm_a16_tile_prepared(workspace, rows, down.qdata, down.wscale, down.out_group)
         return super()._mlp(index, layer, x)
 

@@ -502,12 +502,13 @@ def test_prompt_pass_with_its_own_attention_and_two_launch_mlp():
     fused = Counting(kernel, 320, 8)
     # (the two-launch path is the one that runs: its extension call is made once per layer)
     ext_calls = []
-    real_call = fused._ext.wq_gemm_a16_tile_gate_up_silu
+    # (on rows that the norm in front of it left in prepared form: llmq_add_rmsnorm_prepared)
+    real_call = fused._ext.wq_gemm_a16_tile_gate_up_silu_prepared
     try:
-        fused._ext.wq_gemm_a16_tile_gate_up_silu = lambda *a, **k: (ext_calls.append(1), real_call(*a, **k))[1]
+        fused._ext.wq_gemm_a16_tile_gate_up_silu_prepared = lambda *a, **k: (ext_calls.append(1), real_call(*a, **k))[1]
         tok = fused.prefill(ids)
     finally:
-        fused._ext.wq_gemm_a16_tile_gate_up_silu = real_call
+        fused._ext.wq_gemm_a16_tile_gate_up_silu_prepared = real_call
     assert calls["mlp"] == 2 and len(ext_calls) == 2
     three = ThreeLaunchMlp(kernel, 320, 8)
     assert torch.equal(three.prefill(ids), tok)

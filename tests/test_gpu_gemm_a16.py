@@ -410,6 +410,71 @@ def test_gate_up_silu_epilogue_argument_checks(ext):
         ext.wq_gemm_a16_tile_prepared(workspace[:16], 128, q_d, s_d, 0)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("with_delta", [False, True], ids=["norm", "add+norm"])
+@pytest.mark.parametrize("m,k,n", [(512, 2048, 3072), (200, 384, 520), (65, 128, 64), (130, 4096, 1024)])
+def test_rmsnorm_into_prepared_form_gives_the_bits_of_norm_then_gemm(ext, m, k, n, with_delta, bits):
+    """llmq_add_rmsnorm_prepared + llmq_wq_gemm_a16_tile_prepared against llmq_add_rmsnorm -> llmq_wq_gemm_a16_tile:
+    the residual sum, the prepared chunks (eight consecutive normed values in the order 0, 4, 1, 5, 2, 6, 3, 7) and
+    the GEMM's output equal to the bit; the norm itself against the oracle's LlamaRMSNorm (the mean of squares is
+    summed in another order on the GPU: a last-place difference in 1 / rms moves a few results by one bf16 step)."""
+    torch.manual_seed(m + k)
+    x = (torch.randn(m, k, device="cuda") * 1.5).to(torch.bfloat16)
+    delta = torch.randn(m, k, device="cuda").to(torch.bfloat16) if with_delta else None
+    weight = (1 + 0.1 * torch.randn(k, device="cuda")).to(torch.bfloat16)
+    width = GROUP if bits == 8 else GROUP // 2
+    q = torch.randint(0, 256, (n, k // GROUP, width), dtype=torch.uint8, device="cuda")
+    q = q.view(torch.int8) if bits == 8 else q
+    sw = torch.rand(n, k // GROUP, device="cuda") * 0.004 + 0.001
+    if with_delta:
+        want_sum, normed = ext.add_rmsnorm(x, delta, weight, 1e-5)
+    else:
+        want_sum, normed = x, ext.rmsnorm(x, weight, 1e-5)
+    want = ext.wq_gemm_a16_tile(normed, q, sw, 0)
+    got_sum, workspace = ext.add_rmsnorm_prepared(x, delta, weight, 1e-5, n)
+    prepared = workspace.view(torch.uint8)[: m * k * 2].clone()
+    got = ext.wq_gemm_a16_tile_prepared(workspace, m, q, sw, 0)
+    assert torch.equal(got_sum, want_sum) and torch.equal(got, want)
+    chunks = normed.view(m, k // 8, 8)[:, :, [0, 4, 1, 5, 2, 6, 3, 7]].contiguous()
+    assert torch.equal(prepared, chunks.view(torch.uint8).flatten())
+    summed = to_np(x).astype(np.float32) + (to_np(delta).astype(np.float32) if with_delta else 0)
+    summed = oracle.round_to(summed, "bf16") if with_delta else summed
+    want_normed = oracle.llama_rmsnorm(summed, to_np(weight), 1e-5, "bf16")
+    assert (to_np(normed) == want_normed).mean() > 0.99 and rel_l2(to_np(normed), want_normed) <= 1e-3
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_gate_up_silu_epilogue_on_prepared_rows(ext, bits):
+    """The gated MLP of a prompt from the norm on: add_rmsnorm_prepared -> gate_up_silu_prepared -> prepared against
+    add_rmsnorm -> gate_up_silu -> prepared, equal to the bit."""
+    m, inter, k, n_down = 300, 2560, 512, 640
+    x, q_gu, s_gu, q_d, s_d, _ = mlp_case(m, inter, k, n_down, bits, seed=5)
+    delta = torch.randn_like(x)
+    weight = (1 + 0.1 * torch.randn(k, device="cuda")).to(torch.bfloat16)
+    hidden, normed = ext.add_rmsnorm(x, delta, weight, 1e-6)
+    want = ext.wq_gemm_a16_tile_prepared(ext.wq_gemm_a16_tile_gate_up_silu(normed, q_gu, s_gu, 0, n_down), m, q_d, s_d, 0)
+    got_hidden, workspace = ext.add_rmsnorm_prepared(x, delta, weight, 1e-6, max(2 * inter, n_down))
+    down_ws = ext.wq_gemm_a16_tile_gate_up_silu_prepared(workspace, m, q_gu, s_gu, 0, n_down)
+    got = ext.wq_gemm_a16_tile_prepared(down_ws, m, q_d, s_d, 0)
+    assert torch.equal(got_hidden, hidden) and torch.equal(got, want)
+    assert float(want.float().abs().mean()) > 0
+
+
+def test_rmsnorm_into_prepared_form_argument_checks(ext):
+    x = torch.randn(64, 256, device="cuda").to(torch.bfloat16)
+    weight = torch.ones(256, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="bfloat16"):
+        ext.add_rmsnorm_prepared(x.half(), None, weight.half(), 1e-5, 128)
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        ext.add_rmsnorm_prepared(x[:, :200].contiguous(), None, weight[:200].contiguous(), 1e-5, 128)
+    with pytest.raises(RuntimeError, match="must match"):
+        ext.add_rmsnorm_prepared(x, x[:32], weight, 1e-5, 128)
+    _, workspace = ext.add_rmsnorm_prepared(x, None, weight, 1e-5, 128)
+    q = torch.randint(0, 256, (512, 2, 64), dtype=torch.uint8, device="cuda")
+    with pytest.raises(RuntimeError, match="this GEMM needs"):
+        ext.wq_gemm_a16_tile_gate_up_silu_prepared(workspace[:16], 64, q, torch.ones(512, 2, device="cuda"), 0, 64)
+
+
 def test_gate_up_silu_epilogue_at_the_llama_1b_prompt_shape(ext):
     """The MLP of a 512-token prompt of the Llama-3.2-1B configuration (2048 -> 2 x 8192 -> 2048, int4): 4 x 64
     tiles, the shape the runtime takes this path on. Bit-equal to the three launches (the plain gate|up GEMM has
