@@ -607,11 +607,12 @@ at::Tensor wq_gemm_a16(const at::Tensor& x, const at::Tensor& qweight, const at:
   return out;
 }
 
-// The fused GEMM for prompt-sized M (bf16): 128 x 256 tiles, no dense weight.
+// The fused GEMM for prompt-sized M (bf16 / fp16): 128 x 256 or 64 x 128 tiles, no dense weight.
 at::Tensor wq_gemm_a16_tile(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale, int64_t out_group) {
   TORCH_CHECK(x.is_cuda(), "x must be a CUDA tensor");
   TORCH_CHECK(qweight.is_cuda() && wscale.is_cuda(), "qweight and wscale must be CUDA tensors");
-  TORCH_CHECK(x.scalar_type() == at::kBFloat16, "the tiled fused GEMM takes bfloat16 activations");
+  TORCH_CHECK(x.scalar_type() == at::kBFloat16 || x.scalar_type() == at::kHalf,
+              "the tiled fused GEMM takes bfloat16 or float16 activations");
   TORCH_CHECK(x.dim() == 2, "x must be [M, K]");
   TORCH_CHECK(qweight.dim() == 3, "qweight must be [N, groups, group_size], got ", qweight.dim(), "D");
   const bool packed = qweight.scalar_type() == at::kByte;
@@ -646,7 +647,8 @@ at::Tensor wq_gemm_a16_tile(const at::Tensor& x, const at::Tensor& qweight, cons
 at::Tensor wq_gemm_a16_tile_gate_up_silu(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale,
                                          int64_t out_group, int64_t next_n) {
   TORCH_CHECK(x.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "x, qweight and wscale must be CUDA tensors");
-  TORCH_CHECK(x.scalar_type() == at::kBFloat16, "the tiled fused GEMM takes bfloat16 activations");
+  TORCH_CHECK(x.scalar_type() == at::kBFloat16 || x.scalar_type() == at::kHalf,
+              "the tiled fused GEMM takes bfloat16 or float16 activations");
   TORCH_CHECK(x.dim() == 2, "x must be [M, K]");
   TORCH_CHECK(qweight.dim() == 3, "qweight must be [2 * intermediate, groups, group_size], got ", qweight.dim(), "D");
   const bool packed = qweight.scalar_type() == at::kByte;
@@ -681,7 +683,9 @@ at::Tensor wq_gemm_a16_tile_gate_up_silu(const at::Tensor& x, const at::Tensor& 
 
 // The same launch on an activation that is already in prepared form in `workspace` (from add_rmsnorm_prepared).
 at::Tensor wq_gemm_a16_tile_gate_up_silu_prepared(const at::Tensor& workspace, int64_t rows, const at::Tensor& qweight,
-                                                  const at::Tensor& wscale, int64_t out_group, int64_t next_n) {
+                                                  const at::Tensor& wscale, int64_t out_group, int64_t next_n,
+                                                  at::ScalarType dtype) {
+  TORCH_CHECK(dtype == at::kBFloat16 || dtype == at::kHalf, "dtype must be bfloat16 or float16");
   TORCH_CHECK(workspace.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "workspace, qweight and wscale must be CUDA tensors");
   TORCH_CHECK(workspace.scalar_type() == at::kFloat && workspace.dim() == 1 && workspace.is_contiguous(),
               "workspace must be the tensor add_rmsnorm_prepared returned");
@@ -709,15 +713,16 @@ at::Tensor wq_gemm_a16_tile_gate_up_silu_prepared(const at::Tensor& workspace, i
                                                        next.mutable_data_ptr(), next_need, static_cast<int>(M),
                                                        static_cast<int>(inter), static_cast<int>(groups),
                                                        static_cast<int>(group_size), static_cast<int>(out_group),
-                                                       packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, LLMQ_BF16,
-                                                       current_stream(workspace)),
+                                                       packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8,
+                                                       dtype == at::kHalf ? LLMQ_F16 : LLMQ_BF16, current_stream(workspace)),
            "wq_gemm_a16_tile_gate_up_silu_prepared");
   return next;
 }
 
 // The tiled GEMM on a prepared activation of `rows` rows sitting in `workspace` (from wq_gemm_a16_tile_gate_up_silu).
 at::Tensor wq_gemm_a16_tile_prepared(const at::Tensor& workspace, int64_t rows, const at::Tensor& qweight,
-                                     const at::Tensor& wscale, int64_t out_group) {
+                                     const at::Tensor& wscale, int64_t out_group, at::ScalarType dtype) {
+  TORCH_CHECK(dtype == at::kBFloat16 || dtype == at::kHalf, "dtype must be bfloat16 or float16");
   TORCH_CHECK(workspace.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "workspace, qweight and wscale must be CUDA tensors");
   TORCH_CHECK(workspace.scalar_type() == at::kFloat && workspace.dim() == 1 && workspace.is_contiguous(),
               "workspace must be the tensor wq_gemm_a16_tile_gate_up_silu or add_rmsnorm_prepared returned");
@@ -735,13 +740,14 @@ at::Tensor wq_gemm_a16_tile_prepared(const at::Tensor& workspace, int64_t rows, 
   TORCH_CHECK(M > 0 && N > 0, "empty activation or weight");
   const size_t need = llmq_wq_gemm_a16_tile_workspace_bytes(static_cast<int>(M), static_cast<int>(N), static_cast<int>(groups));
   TORCH_CHECK(static_cast<size_t>(workspace.numel()) * 4 >= need, "workspace holds ", workspace.numel() * 4, " bytes, this GEMM needs ", need);
-  auto out = at::empty({M, N}, workspace.options().dtype(at::kBFloat16));
+  auto out = at::empty({M, N}, workspace.options().dtype(dtype));
   const c10::OptionalDeviceGuard guard(at::device_of(workspace));
   check_rc(llmq_wq_gemm_a16_tile_prepared(wc.const_data_ptr(), sc.const_data_ptr<float>(), out.mutable_data_ptr(),
                                           workspace.mutable_data_ptr(), static_cast<size_t>(workspace.numel()) * 4,
                                           static_cast<int>(M), static_cast<int>(N), static_cast<int>(groups),
                                           static_cast<int>(group_size), static_cast<int>(out_group),
-                                          packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, LLMQ_BF16, current_stream(workspace)),
+                                          packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8,
+                                          dtype == at::kHalf ? LLMQ_F16 : LLMQ_BF16, current_stream(workspace)),
            "wq_gemm_a16_tile_prepared");
   return out;
 }
@@ -793,7 +799,8 @@ std::tuple<at::Tensor, at::Tensor> add_rmsnorm(const at::Tensor& x, const at::Te
 std::tuple<at::Tensor, at::Tensor> add_rmsnorm_prepared(const at::Tensor& x, const c10::optional<at::Tensor>& delta,
                                                         const at::Tensor& weight, double eps, int64_t next_n) {
   TORCH_CHECK(x.is_cuda() && weight.is_cuda(), "x and weight must be CUDA tensors");
-  TORCH_CHECK(x.scalar_type() == at::kBFloat16, "the prepared form is of bfloat16 activations");
+  TORCH_CHECK(x.scalar_type() == at::kBFloat16 || x.scalar_type() == at::kHalf,
+              "the prepared form is of bfloat16 or float16 activations");
   TORCH_CHECK(x.dim() == 2 && weight.dim() == 1 && weight.size(0) == x.size(1), "x must be [rows, hidden], weight [hidden]");
   TORCH_CHECK(weight.scalar_type() == x.scalar_type(), "weight must have x's dtype");
   TORCH_CHECK(x.size(0) > 0 && next_n > 0, "empty activation");
@@ -813,7 +820,7 @@ std::tuple<at::Tensor, at::Tensor> add_rmsnorm_prepared(const at::Tensor& x, con
   check_rc(llmq_add_rmsnorm_prepared(xc.const_data_ptr(), delta.has_value() ? dc.const_data_ptr() : nullptr,
                                      wc.const_data_ptr(), delta.has_value() ? sum.mutable_data_ptr() : nullptr,
                                      workspace.mutable_data_ptr(), need, static_cast<int>(rows), static_cast<int>(hidden),
-                                     static_cast<float>(eps), LLMQ_BF16, current_stream(xc)),
+                                     static_cast<float>(eps), dtype_code(xc, "x"), current_stream(xc)),
            "add_rmsnorm_prepared");
   return {sum, workspace};
 }
@@ -1348,13 +1355,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("wq_gemm_a16_tile_gate_up_silu_prepared", &wq_gemm_a16_tile_gate_up_silu_prepared,
         "wq_gemm_a16_tile_gate_up_silu on the prepared activation add_rmsnorm_prepared left in its workspace",
         py::arg("workspace"), py::arg("rows"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0,
-        py::arg("next_n"));
+        py::arg("next_n"), py::arg("dtype") = at::kBFloat16);
   m.def("add_rmsnorm_prepared", &add_rmsnorm_prepared,
         "(x + delta, workspace): LlamaRMSNorm(x + delta) written as the prepared activation of a tiled GEMM, one launch",
         py::arg("x"), py::arg("delta"), py::arg("weight"), py::arg("eps"), py::arg("next_n"));
   m.def("wq_gemm_a16_tile_prepared", &wq_gemm_a16_tile_prepared,
         "the tiled GEMM on the prepared activation wq_gemm_a16_tile_gate_up_silu left in its workspace",
-        py::arg("workspace"), py::arg("rows"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0);
+        py::arg("workspace"), py::arg("rows"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0,
+        py::arg("dtype") = at::kBFloat16);
   m.def("wq_gemm_a16_tile", &wq_gemm_a16_tile,
         "Fused weight-only GEMM for prompt-sized bf16 activations: 128 x 256 tiles on the bf16 matrix cores, no dense weight",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0);

@@ -1,6 +1,6 @@
 // Weight-only quantized GEMM for prompt-sized activations (M in the hundreds and thousands), gfx950:
-// bf16 activations times int4 / int8 group-quantized weights on the bf16 matrix core, with no dense
-// copy of the weight anywhere.
+// bf16 (or fp16) activations times int4 / int8 group-quantized weights on the 16-bit matrix core, with no dense
+// copy of the weight anywhere. The text below describes the bf16 form; what differs for fp16 is said at kBiased.
 //
 //   out[m, n] = sum over g of  wscale[sr(n), g] * sum_k x[m, g*128 + k] * code[n, g, k]
 //
@@ -45,6 +45,14 @@ namespace {
 using namespace llmq;
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+// bfloat16: the matrix core sums x * (code + B) and B * sum x is taken out again (below). float16 has the mantissa
+// to hold B + code as well, but the pieces of a group's activation sum do not fit its exponent range (128 values of
+// up to 65504, and pieces of a small sum fall below its smallest step), so there the bias is subtracted from the
+// operand itself, exactly, with one packed add per two codes, and there is no correction step.
+template <typename T> constexpr bool kBiased = std::is_same<T, bf16_t>::value;
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kGroup = 128;
@@ -86,14 +94,21 @@ using Narrow = Shape<64, 4, 2>;
 // (what the host side sizes for when it does not say which: the wide tile)
 constexpr int kBM = Wide::kBM, kBN = Wide::kBN;
 
-template <int BITS> constexpr float kCodeBias = BITS == 4 ? 24.0f : 128.0f;
 
 // ---- activation preparation -----------------------------------------------------------------------
 // One lane per 16-byte chunk, 16 lanes per (row, group): `v` holds the chunk's eight bf16 values (zeros in a lane
 // with nothing to do; a row of 16 lanes is active or idle as one). Writes the reordered chunk, and from the row's
 // first lane the record of the group's sum.
+template <typename T>
 __device__ __forceinline__ void emit_prepared(const u32x4 v, const bool active, const bool first_of_row,
                                               u32x4* __restrict__ chunk_out, u32x4* __restrict__ record_out) {
+  if constexpr (!kBiased<T>) {
+    // (no correction step: the records stay part of the layout and are zeros)
+    if (!active) return;
+    *chunk_out = interleave_halves(v);
+    if (first_of_row) *record_out = u32x4{0u, 0u, 0u, 0u};
+    return;
+  }
   float f[8];
   Pack<bf16_t>::unpack(v, f);
   float s = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
@@ -117,13 +132,14 @@ __device__ __forceinline__ void emit_prepared(const u32x4 v, const bool active, 
   }
 }
 
+template <typename T>
 __global__ __launch_bounds__(256) void act_prep_kernel(const u32x4* __restrict__ x, u32x4* __restrict__ xp,
                                                        u32x4* __restrict__ rec, const int64_t n_chunks) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   const bool active = i < n_chunks;  // n_chunks is a multiple of 16: a row of 16 lanes is active or idle as one
   u32x4 v = {0u, 0u, 0u, 0u};
   if (active) v = x[i];
-  emit_prepared(v, active, (threadIdx.x & 15) == 0, xp + (active ? i : 0), rec + (active ? i >> 4 : 0));
+  emit_prepared<T>(v, active, (threadIdx.x & 15) == 0, xp + (active ? i : 0), rec + (active ? i >> 4 : 0));
 }
 
 // LlamaRMSNorm (optionally on x + delta, the residual add in front of it, which is stored as well) whose result
@@ -132,27 +148,27 @@ __global__ __launch_bounds__(256) void act_prep_kernel(const u32x4* __restrict__
 // rmsnorm_kernel (csrc/prefill_ops.hip): out = w * bf16(x_f32 * rsqrt(mean(x_f32^2) + eps)), rounded to bf16.
 // hidden is a multiple of 128, so the 16 lanes of a (row, group) are in the loop together.
 constexpr int kNormThreads = 256;
-template <bool ADD>
-__global__ __launch_bounds__(kNormThreads) void rmsnorm_prep_kernel(const bf16_t* __restrict__ x,
-                                                                   const bf16_t* __restrict__ delta,
-                                                                   const bf16_t* __restrict__ w,
-                                                                   bf16_t* __restrict__ sum_out, u32x4* __restrict__ xp,
+template <typename T, bool ADD>
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_prep_kernel(const T* __restrict__ x,
+                                                                   const T* __restrict__ delta,
+                                                                   const T* __restrict__ w,
+                                                                   T* __restrict__ sum_out, u32x4* __restrict__ xp,
                                                                    u32x4* __restrict__ rec, const int hidden,
                                                                    const float eps) {
   __shared__ float red[kNormThreads / kWave];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * hidden;
-  const bf16_t* row = x + base;
+  const T* row = x + base;
   const int tid = threadIdx.x;
   float ss = 0.0f;
   for (int i = tid * 8; i < hidden; i += kNormThreads * 8) {
     float f[8];
-    Pack<bf16_t>::unpack(load16(row + i), f);
+    Pack<T>::unpack(load16(row + i), f);
     if constexpr (ADD) {
       float d[8];
-      Pack<bf16_t>::unpack(load16(delta + base + i), d);
+      Pack<T>::unpack(load16(delta + base + i), d);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) f[e] = round_through<bf16_t>(f[e] + d[e]);
-      store16(sum_out + base + i, Pack<bf16_t>::pack(f));
+      for (int e = 0; e < 8; ++e) f[e] = round_through<T>(f[e] + d[e]);
+      store16(sum_out + base + i, Pack<T>::pack(f));
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) ss = fmaf(f[e], f[e], ss);
@@ -165,16 +181,16 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_prep_kernel(const bf16_t
   for (int k = 0; k < kNormThreads / kWave; ++k) total += red[k];
   const float inv_rms = rsqrtf(total / static_cast<float>(hidden) + eps);
   // (with ADD a thread reads back exactly the packets it stored above)
-  const bf16_t* src = ADD ? sum_out + base : row;
+  const T* src = ADD ? sum_out + base : row;
   const int64_t chunk0 = base >> 3;   // the row's first chunk; 16 chunks a group
   for (int i = tid * 8; i < hidden; i += kNormThreads * 8) {
     float f[8], g[8];
-    Pack<bf16_t>::unpack(load16(src + i), f);
-    Pack<bf16_t>::unpack(load16(w + i), g);
+    Pack<T>::unpack(load16(src + i), f);
+    Pack<T>::unpack(load16(w + i), g);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) f[e] = g[e] * round_through<bf16_t>(f[e] * inv_rms);
+    for (int e = 0; e < 8; ++e) f[e] = g[e] * round_through<T>(f[e] * inv_rms);
     const int64_t chunk = chunk0 + (i >> 3);
-    emit_prepared(Pack<bf16_t>::pack(f), true, (tid & 15) == 0, xp + chunk, rec + (chunk >> 4));
+    emit_prepared<T>(Pack<T>::pack(f), true, (tid & 15) == 0, xp + chunk, rec + (chunk >> 4));
   }
 }
 
@@ -210,41 +226,34 @@ template <int BITS> __device__ __forceinline__ int code_slot(int row, int c) {
   return BITS == 4 ? c ^ ((row >> 2) & 3) : c ^ ((row >> 1) & 7);
 }
 
-constexpr uint32_t kNibbleMask = 0x00780078u;   // (and_or: (value & mask) | bits in one instruction)
 
-// Two of the four operand words of a k-step: a k-step's eight codes are one 32-bit word of int4 or two of
-// int8 (`raw`: the wave's k-steps one after the other); operand word i pairs codes i and i + 4. `half` selects
-// words (0, 1) or (2, 3).
-template <int BITS>
-__device__ __forceinline__ void code_words(const uint32_t* raw, int step, int half, uint32_t sixteen, uint32_t* out) {
-  if constexpr (BITS == 4) {
-    const uint32_t w = raw[step];
-    if (half == 0) {
-      out[0] = and_or(w << 3, kNibbleMask, sixteen);  // nibbles 0 and 4
-      out[1] = and_or(w >> 1, kNibbleMask, sixteen);  // 1 and 5
-    } else {
-      out[0] = and_or(w >> 5, kNibbleMask, sixteen);  // 2 and 6
-      out[1] = and_or(w >> 9, kNibbleMask, sixteen);  // 3 and 7
-    }
-  } else {
-    const uint32_t w0 = raw[2 * step] ^ 0x80808080u;      // codes 0..3 of the step, + 128
-    const uint32_t w1 = raw[2 * step + 1] ^ 0x80808080u;  // codes 4..7
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int e = 2 * half + i;
-      const float lo = static_cast<float>((w0 >> (8 * e)) & 0xffu);
-      const float hi = static_cast<float>((w1 >> (8 * e)) & 0xffu);
-      // integers below 256: the upper half of the float is the bf16 value, exactly
-      out[i] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, hi), __builtin_bit_cast(uint32_t, lo), 0x07060302u);
-    }
+// The four operand words of a k-step of the wave (`raw`: its k-steps' codes one after the other, one 32-bit word
+// of int4 or two of int8 a step); operand word i pairs codes i and i + 4.
+template <typename T, int BITS>
+__device__ __forceinline__ u32x4 operand_words(const uint32_t* raw, int step, uint32_t magic) {
+  u32x4 w = BiasedCodes<T, BITS>::operand(raw, step, magic);
+  if constexpr (!kBiased<T>) {
+    const _Float16 b = static_cast<_Float16>(BiasedCodes<T, BITS>::kBias);
+    const h2 bias = {b, b};
+    w.x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, w.x) - bias);
+    w.y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, w.y) - bias);
+    w.z = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, w.z) - bias);
+    w.w = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, w.w) - bias);
   }
+  return w;
 }
 
-__device__ __forceinline__ v16f mfma(const u32x4& a, const u32x4& b, const v16f& c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+template <typename T> __device__ __forceinline__ v16f mfma(const u32x4& a, const u32x4& b, const v16f& c) {
+  if constexpr (std::is_same<T, bf16_t>::value)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+}
+template <typename T> __device__ __forceinline__ uint16_t bits16(float v) {
+  return __builtin_bit_cast(uint16_t, from_float<T>(v));
 }
 
-template <int BITS, int EPI, typename S>
+template <typename T, int BITS, int EPI, typename S>
 __global__ __launch_bounds__(S::kThreads, 1) void wq_gemm_a16_tile_kernel(const TileArgs a) {
   extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
   static_assert(EPI == kEpiStore || std::is_same<S, Wide>::value, "the gate|up epilogue is laid out for the wide tile");
@@ -391,9 +400,9 @@ __global__ __launch_bounds__(S::kThreads, 1) void wq_gemm_a16_tile_kernel(const 
     for (int ni = 0; ni < kNT; ++ni)
 #pragma unroll
       for (int r = 0; r < 16; ++r) total[mi][ni][r] = 0.0f;
-  uint32_t sixteen = 0x41804180u;  // bf16 16.0 twice; kept in a vector register (see and_or)
+  uint32_t sixteen = BiasedCodes<T, BITS>::kMagic;  // 16.0 (int8 in float16: 256.0) twice; kept in a vector register (see and_or)
   asm volatile("" : "+v"(sixteen));
-  const uint32_t nb = bf16_bits_rne(-kCodeBias<BITS>);  // exact
+  const uint32_t nb = bf16_bits_rne(-BiasedCodes<T, BITS>::kBias);  // exact (read where kBiased<T> only)
   const uint32_t nb2 = (lh || kh) ? 0u : (nb | (nb << 16));   // (the correction step belongs to the group's first k-steps)
   const u32x4 bias_operand = {nb2, nb2, 0u, 0u};
 
@@ -418,9 +427,11 @@ __global__ __launch_bounds__(S::kThreads, 1) void wq_gemm_a16_tile_kernel(const 
   float scale[kNT];
   auto fetch_group_operands = [&](int st) {
     const uint8_t* stage = smem + st * kStageB;
+    if constexpr (kBiased<T>) {
 #pragma unroll
-    for (int mi = 0; mi < kMT; ++mi)
-      rec[mi] = read16(stage, kTileBytes + kCodeTileB + (wm * kWaveM + mi * 32 + lm) * 16);
+      for (int mi = 0; mi < kMT; ++mi)
+        rec[mi] = read16(stage, kTileBytes + kCodeTileB + (wm * kWaveM + mi * 32 + lm) * 16);
+    }
 #pragma unroll
     for (int ni = 0; ni < kNT; ++ni) {
       if constexpr (kRawBytes == 8) {
@@ -468,18 +479,13 @@ __global__ __launch_bounds__(S::kThreads, 1) void wq_gemm_a16_tile_kernel(const 
 #pragma unroll
       for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < kNT; ++ni) acc[mi][ni] = kh == 0 ? mfma(rec[mi], bias_operand, zero) : zero;
+        for (int ni = 0; ni < kNT; ++ni) acc[mi][ni] = kBiased<T> && kh == 0 ? mfma<T>(rec[mi], bias_operand, zero) : zero;
     }
 #pragma unroll
     for (int j = 0; j < kSteps; ++j) {
       u32x4 fb[kNT];
 #pragma unroll
-      for (int ni = 0; ni < kNT; ++ni) {
-        uint32_t lo[2], hi[2];
-        code_words<BITS>(raw[ni], j, 0, sixteen, lo);
-        code_words<BITS>(raw[ni], j, 1, sixteen, hi);
-        fb[ni] = u32x4{lo[0], lo[1], hi[0], hi[1]};
-      }
+      for (int ni = 0; ni < kNT; ++ni) fb[ni] = operand_words<T, BITS>(raw[ni], j, sixteen);
       if (j < kSteps - 1) {
 #pragma unroll
         for (int mi = 0; mi < kMT; ++mi) fa[(j + 1) & 1][mi] = read16(stage, mi * 32 * kRowBytes + (a_base ^ ((j + 1) << 4)));
@@ -499,7 +505,7 @@ __global__ __launch_bounds__(S::kThreads, 1) void wq_gemm_a16_tile_kernel(const 
 #pragma unroll
       for (int mi = 0; mi < kMT; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < kNT; ++ni) acc[mi][ni] = mfma(fa[j & 1][mi], fb[ni], acc[mi][ni]);
+        for (int ni = 0; ni < kNT; ++ni) acc[mi][ni] = mfma<T>(fa[j & 1][mi], fb[ni], acc[mi][ni]);
     }
 #pragma unroll
     for (int mi = 0; mi < kMT; ++mi)
@@ -523,7 +529,7 @@ __global__ __launch_bounds__(S::kThreads, 1) void wq_gemm_a16_tile_kernel(const 
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = mi * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-        *reinterpret_cast<uint16_t*>(block + row * kEpiRowBytes + col * 2) = bf16_bits_rne(total[mi][0][r]);
+        *reinterpret_cast<uint16_t*>(block + row * kEpiRowBytes + col * 2) = bits16<T>(total[mi][0][r]);
       }
     __syncthreads();
     u32x4* __restrict__ next_xp = reinterpret_cast<u32x4*>(a.next_xp);
@@ -532,23 +538,23 @@ __global__ __launch_bounds__(S::kThreads, 1) void wq_gemm_a16_tile_kernel(const 
     for (int pass = 0; pass < kBM * 16 / kThreads; ++pass) {
       const int q = pass * kThreads + tid, row = q >> 4, chunk = q & 15;
       float g[8], u[8];
-      Pack<bf16_t>::unpack(read16(smem, row * kEpiRowBytes + chunk * 16), g);
-      Pack<bf16_t>::unpack(read16(smem, kBM * kEpiRowBytes + row * kEpiRowBytes + chunk * 16), u);
+      Pack<T>::unpack(read16(smem, row * kEpiRowBytes + chunk * 16), g);
+      Pack<T>::unpack(read16(smem, kBM * kEpiRowBytes + row * kEpiRowBytes + chunk * 16), u);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) g[e] = round_through<bf16_t>(g[e] / (1.0f + expf(-g[e]))) * u[e];
+      for (int e = 0; e < 8; ++e) g[e] = round_through<T>(g[e] / (1.0f + expf(-g[e]))) * u[e];
       const int64_t at = static_cast<int64_t>(m0 + row) * a.next_G + nt;   // (row, group) of the next activation
-      emit_prepared(Pack<bf16_t>::pack(g), true, chunk == 0, next_xp + at * 16 + chunk, next_rec + at);
+      emit_prepared<T>(Pack<T>::pack(g), true, chunk == 0, next_xp + at * 16 + chunk, next_rec + at);
     }
     return;
   }
   // one 32 x 32 tile of totals, whose first row is m_first and whose column (this lane's) is n
   auto store_tile = [&](const float (&v)[16], int m_first, int n) {
     if (a.splits == 1) {
-      bf16_t* __restrict__ out = static_cast<bf16_t*>(a.out);
+      T* __restrict__ out = static_cast<T*>(a.out);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m_first + 8 * (r >> 2) + 4 * lh + (r & 3);
-        if (m < a.M && n < a.N) out[static_cast<int64_t>(m) * a.N + n] = from_float<bf16_t>(v[r]);
+        if (m < a.M && n < a.N) out[static_cast<int64_t>(m) * a.N + n] = from_float<T>(v[r]);
       }
     } else {
       float* __restrict__ part = a.partial + static_cast<int64_t>(sp) * a.M * a.N;
@@ -598,7 +604,8 @@ __global__ __launch_bounds__(S::kThreads, 1) void wq_gemm_a16_tile_kernel(const 
 }
 
 // out[i] = bf16(partial[0][i] + partial[1][i] + ...), slices added in order; four values per lane.
-__global__ __launch_bounds__(256) void add_splits_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
+template <typename T>
+__global__ __launch_bounds__(256) void add_splits_kernel(const float* __restrict__ partial, T* __restrict__ out,
                                                          const int64_t count, const int splits) {
   const int64_t i4 = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
   if (i4 >= count) return;
@@ -612,7 +619,9 @@ __global__ __launch_bounds__(256) void add_splits_kernel(const float* __restrict
 #pragma unroll
       for (int e = 0; e < 4; ++e) s[e] = s[e] + t[e];
     }
-    *reinterpret_cast<u32x2*>(out + i4) = u32x2{bf16_pair_rne(s[0], s[1]), bf16_pair_rne(s[2], s[3])};
+    *reinterpret_cast<u32x2*>(out + i4) =
+        u32x2{static_cast<uint32_t>(bits16<T>(s[0])) | static_cast<uint32_t>(bits16<T>(s[1])) << 16,
+              static_cast<uint32_t>(bits16<T>(s[2])) | static_cast<uint32_t>(bits16<T>(s[3])) << 16};
   } else {
     // a count that is not a multiple of four leaves the later slices off 16-byte alignment: this lane's own
     // (up to) four values one at a time
@@ -620,14 +629,14 @@ __global__ __launch_bounds__(256) void add_splits_kernel(const float* __restrict
     for (int64_t i = i4; i < end; ++i) {
       float s = partial[i];
       for (int k = 1; k < splits; ++k) s = s + partial[k * count + i];
-      out[i] = from_float<bf16_t>(s);
+      out[i] = from_float<T>(s);
     }
   }
 }
 
-template <int BITS, int EPI, typename S = Wide>
+template <typename T, int BITS, int EPI, typename S = Wide>
 int launch_tiles(const TileArgs& a, dim3 grid, hipStream_t stream) {
-  auto kernel = wq_gemm_a16_tile_kernel<BITS, EPI, S>;
+  auto kernel = wq_gemm_a16_tile_kernel<T, BITS, EPI, S>;
   constexpr int kLds = S::template kLdsBytes<BITS>;
   static bool raised = false;  // per instantiation; worst case two threads both set it
   if (!raised) {
@@ -724,7 +733,8 @@ int check_common(const void* x, bool prepared, const void* qweight, const float*
                  int N, int G, int gs, int out_group, int wformat, int dtype) {
   if (M < 0 || N < 0 || G < 0) return llmq_host::fail_invalid("negative dimension M=%d N=%d G=%d", M, N, G);
   if (gs != kGroup) return llmq_host::fail_invalid("the tiled fused GEMM needs group_size 128, got %d", gs);
-  if (dtype != LLMQ_BF16) return llmq_host::fail_invalid("the tiled fused GEMM takes bfloat16 activations, got dtype code %d", dtype);
+  if (dtype != LLMQ_BF16 && dtype != LLMQ_F16)
+    return llmq_host::fail_invalid("the tiled fused GEMM takes bfloat16 or float16 activations, got dtype code %d", dtype);
   if (wformat != LLMQ_W_INT8 && wformat != LLMQ_W_INT4_PACKED)
     return llmq_host::fail_invalid("unsupported weight format %d, expected 8 or 4", wformat);
   if (out_group < 0) return llmq_host::fail_invalid("out_group must be >= 0, got %d", out_group);
@@ -740,12 +750,25 @@ int check_common(const void* x, bool prepared, const void* qweight, const float*
   return 0;
 }
 
-int prepare(const void* x, uint8_t* xp, uint8_t* rec, int M, int G, hipStream_t s) {
+int prepare(const void* x, uint8_t* xp, uint8_t* rec, int M, int G, int dtype, hipStream_t s) {
   const int64_t n_chunks = static_cast<int64_t>(M) * G * 16;
-  hipLaunchKernelGGL(act_prep_kernel, dim3(static_cast<unsigned>((n_chunks + 255) / 256)), dim3(256), 0, s,
-                     static_cast<const u32x4*>(x), reinterpret_cast<u32x4*>(xp), reinterpret_cast<u32x4*>(rec),
-                     n_chunks);
+  const dim3 grid(static_cast<unsigned>((n_chunks + 255) / 256));
+  if (dtype == LLMQ_BF16) {
+    hipLaunchKernelGGL(act_prep_kernel<bf16_t>, grid, dim3(256), 0, s, static_cast<const u32x4*>(x),
+                       reinterpret_cast<u32x4*>(xp), reinterpret_cast<u32x4*>(rec), n_chunks);
+  } else {
+    hipLaunchKernelGGL(act_prep_kernel<f16_t>, grid, dim3(256), 0, s, static_cast<const u32x4*>(x),
+                       reinterpret_cast<u32x4*>(xp), reinterpret_cast<u32x4*>(rec), n_chunks);
+  }
   return llmq_host::check_launch("act_prep_kernel");
+}
+
+// The kernel for a weight format, an epilogue and a tile shape, by activation dtype.
+template <int EPI, typename S>
+int launch_by_type(const TileArgs& a, dim3 grid, int wformat, int dtype, hipStream_t s) {
+  const bool int4 = wformat == LLMQ_W_INT4_PACKED;
+  if (dtype == LLMQ_BF16) return int4 ? launch_tiles<bf16_t, 4, EPI, S>(a, grid, s) : launch_tiles<bf16_t, 8, EPI, S>(a, grid, s);
+  return int4 ? launch_tiles<f16_t, 4, EPI, S>(a, grid, s) : launch_tiles<f16_t, 8, EPI, S>(a, grid, s);
 }
 
 // x (or, x null, the prepared activation already in the workspace) times the weight, into out.
@@ -765,20 +788,23 @@ int run_store(const void* x, const void* qweight, const float* wscale, void* out
   uint8_t* rec = ws + p.xp_bytes;
   float* partial = reinterpret_cast<float*>(ws + p.xp_bytes + p.rec_bytes);
   if (x != nullptr) {
-    if (int rc = prepare(x, xp, rec, M, G, s)) return rc;
+    if (int rc = prepare(x, xp, rec, M, G, dtype, s)) return rc;
   }
   TileArgs a{xp, rec, static_cast<const uint8_t*>(qweight), wscale, out, partial, M, N, G, out_group,
              p.m_tiles, p.n_tiles, p.splits, p.groups_per_split, nullptr, nullptr, 0};
   const int total = p.m_tiles * p.n_tiles * p.splits;
   const dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8));
-  int rc;
-  if (narrow) rc = wformat == LLMQ_W_INT4_PACKED ? launch_tiles<4, kEpiStore, Narrow>(a, grid, s) : launch_tiles<8, kEpiStore, Narrow>(a, grid, s);
-  else rc = wformat == LLMQ_W_INT4_PACKED ? launch_tiles<4, kEpiStore>(a, grid, s) : launch_tiles<8, kEpiStore>(a, grid, s);
+  const int rc = narrow ? launch_by_type<kEpiStore, Narrow>(a, grid, wformat, dtype, s)
+                        : launch_by_type<kEpiStore, Wide>(a, grid, wformat, dtype, s);
   if (rc) return rc;
   if (p.splits > 1) {
     const int64_t count = static_cast<int64_t>(M) * N;
-    hipLaunchKernelGGL(add_splits_kernel, dim3(static_cast<unsigned>((count / 4 + 256) / 256)), dim3(256), 0, s,
-                       partial, static_cast<bf16_t*>(out), count, p.splits);
+    const dim3 add_grid(static_cast<unsigned>((count / 4 + 256) / 256));
+    if (dtype == LLMQ_BF16) {
+      hipLaunchKernelGGL(add_splits_kernel<bf16_t>, add_grid, dim3(256), 0, s, partial, static_cast<bf16_t*>(out), count, p.splits);
+    } else {
+      hipLaunchKernelGGL(add_splits_kernel<f16_t>, add_grid, dim3(256), 0, s, partial, static_cast<f16_t*>(out), count, p.splits);
+    }
     return llmq_host::check_launch("add_splits_kernel");
   }
   return 0;
@@ -834,7 +860,7 @@ int run_gate_up_silu(const void* x, const void* qweight, const float* wscale, vo
   uint8_t* xp = ws;
   uint8_t* rec = ws + p.xp_bytes;
   if (x != nullptr) {
-    if (int rc = prepare(x, xp, rec, M, G, s)) return rc;
+    if (int rc = prepare(x, xp, rec, M, G, dtype, s)) return rc;
   }
   uint8_t* nws = static_cast<uint8_t*>(next_workspace);
   // whole reduction axis per workgroup: a tile's epilogue needs its finished totals
@@ -842,7 +868,7 @@ int run_gate_up_silu(const void* x, const void* qweight, const float* wscale, vo
              p.m_tiles, I / (kBN / 2), 1, G, nws, nws + next.xp_bytes, next_G};
   const int total = a.m_tiles * a.n_tiles;
   const dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8));
-  return wformat == LLMQ_W_INT4_PACKED ? launch_tiles<4, kEpiGateUpSilu>(a, grid, s) : launch_tiles<8, kEpiGateUpSilu>(a, grid, s);
+  return launch_by_type<kEpiGateUpSilu, Wide>(a, grid, wformat, dtype, s);
 }
 
 }  // namespace
@@ -869,7 +895,8 @@ extern "C" int llmq_add_rmsnorm_prepared(const void* x, const void* delta_or_nul
                                          void* sum_out_or_null, void* workspace, size_t workspace_bytes, int rows,
                                          int hidden, float eps, int dtype, llmq_stream_t stream) {
   if (rows < 0 || hidden <= 0) return llmq_host::fail_invalid("bad dimension rows=%d hidden=%d", rows, hidden);
-  if (dtype != LLMQ_BF16) return llmq_host::fail_invalid("the prepared form is of bfloat16 activations, got dtype code %d", dtype);
+  if (dtype != LLMQ_BF16 && dtype != LLMQ_F16)
+    return llmq_host::fail_invalid("the prepared form is of bfloat16 or float16 activations, got dtype code %d", dtype);
   if (hidden % kGroup) return llmq_host::fail_invalid("hidden must be a multiple of %d, got %d", kGroup, hidden);
   if (rows == 0) return 0;
   if (!x || !weight || !workspace) return llmq_host::fail_invalid("null tensor pointer");
@@ -886,16 +913,17 @@ extern "C" int llmq_add_rmsnorm_prepared(const void* x, const void* delta_or_nul
     return llmq_host::fail_invalid("workspace of %zu bytes is too small, need %zu", workspace_bytes, p.xp_bytes + p.rec_bytes);
   uint8_t* ws = static_cast<uint8_t*>(workspace);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (delta_or_null) {
-    hipLaunchKernelGGL(rmsnorm_prep_kernel<true>, dim3(rows), dim3(kNormThreads), 0, s, static_cast<const bf16_t*>(x),
-                       static_cast<const bf16_t*>(delta_or_null), static_cast<const bf16_t*>(weight),
-                       static_cast<bf16_t*>(sum_out_or_null), reinterpret_cast<u32x4*>(ws),
-                       reinterpret_cast<u32x4*>(ws + p.xp_bytes), hidden, eps);
+  u32x4* xp = reinterpret_cast<u32x4*>(ws);
+  u32x4* rec = reinterpret_cast<u32x4*>(ws + p.xp_bytes);
+#define LLMQ_NORM_PREP(T, ADD)                                                                                      \
+  hipLaunchKernelGGL((rmsnorm_prep_kernel<T, ADD>), dim3(rows), dim3(kNormThreads), 0, s, static_cast<const T*>(x), \
+                     static_cast<const T*>(delta_or_null), static_cast<const T*>(weight),                           \
+                     static_cast<T*>(sum_out_or_null), xp, rec, hidden, eps)
+  if (dtype == LLMQ_BF16) {
+    if (delta_or_null) LLMQ_NORM_PREP(bf16_t, true); else LLMQ_NORM_PREP(bf16_t, false);
   } else {
-    hipLaunchKernelGGL(rmsnorm_prep_kernel<false>, dim3(rows), dim3(kNormThreads), 0, s, static_cast<const bf16_t*>(x),
-                       static_cast<const bf16_t*>(nullptr), static_cast<const bf16_t*>(weight),
-                       static_cast<bf16_t*>(nullptr), reinterpret_cast<u32x4*>(ws),
-                       reinterpret_cast<u32x4*>(ws + p.xp_bytes), hidden, eps);
+    if (delta_or_null) LLMQ_NORM_PREP(f16_t, true); else LLMQ_NORM_PREP(f16_t, false);
   }
+#undef LLMQ_NORM_PREP
   return llmq_host::check_launch("rmsnorm_prep_kernel");
 }

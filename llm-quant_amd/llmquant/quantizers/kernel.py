@@ -36,37 +36,63 @@ FUSED_GEMM_MIN_ROWS = 3
 FUSED_GEMM_SPLIT_GROUPS = 1 << 30   # (no row is long enough for the split form to win)
 
 
-#: Prompt-sized bf16 activations: the tiled fused GEMM (128 x 256 output tiles, no dense weight) up to this
-#: many rows, where it runs level with or ahead of dequantize + the BLAS library's matmul (measured at 128
-#: and 512 rows; at 2048 rows the library's 1.1-1.2 PFLOP/s kernels win by more than the dequantize pass costs)
+#: Prompt-sized bf16 / fp16 activations: the tiled fused GEMM (128 x 256 or 64 x 128 output tiles, no dense weight) up
+#: to this many rows where its estimated time is within 5 % of the estimate for dequantize + the BLAS library's matmul
+#: (beyond 1024 rows the library's 1.2-1.4 PFLOP/s kernels win by more than the dequantize pass costs)
 TILED_GEMM_MAX_ROWS = 1024
 
 
-#: The tiled GEMM's 64 x 128 tile: outputs it covers in one round of workgroups (one per CU) on rows of at most
-#: this many groups (csrc/wq_gemm_a16_tile.hip, narrow_tile)
-TILED_GEMM_NARROW_MAX_GROUPS = 16
-TILED_GEMM_NARROW_MAX_TILES = 256
-#: ... and from this many of those tiles (measured down to 192 x 3072: 72 tiles; smaller outputs stay with the library)
-TILED_GEMM_NARROW_MIN_TILES = 64
+def _tile_plan_cost(rows: int, out_features: int, groups: int, narrow: bool, int4: bool) -> float:
+    """Microseconds of the tiled GEMM's launch for one tile shape: the plan and the cost figures of
+    csrc/wq_gemm_a16_tile.hip (plan_for, plan_cost), which chooses the cheaper shape itself."""
+    tile_m, tile_n = (64, 128) if narrow else (128, 256)
+    tiles = -(-rows // tile_m) * -(-out_features // tile_n)
+    splits = max(1, min(256 // tiles, groups // 4)) if tiles < 160 else 1
+    per_split = -(-groups // splits)
+    splits = -(-groups // per_split)
+    fixed = 6.0 if narrow else 8.0
+    per_group = (0.75 if int4 else 1.0) if narrow else (1.93 if int4 else 2.1)
+    cost = -(-(tiles * splits) // 256) * (fixed + per_split * per_group)
+    if splits > 1:
+        cost += 3.0 + splits * rows * out_features * 8.0 / 9.0e6
+    return cost
 
 
-def tiled_gemm_pays(rows: int, out_features: int, groups: int) -> bool:
-    """Whether the tiled fused GEMM beats dequantize + matmul for this many activation rows: wide outputs
-    (enough 128 x 256 tiles to fill the chip), long rows (the reduction axis is split instead), or short rows on an
-    output that 64 x 128 tiles cover in one round (q|k|v of a 1B model at a 512-token prompt: 192 tiles)."""
+def tiled_gemm_cost(rows: int, out_features: int, groups: int, bits: int = 8, prepared: bool = False) -> float:
+    """Estimated microseconds of llmq_wq_gemm_a16_tile (within a tenth of the measured launches, 128-2048 rows on
+    weights of 2048-28672 rows): rounds of 256 workgroups, each a fixed part plus a time per group, the partial sums'
+    way through memory where the reduction axis is cut, and 3.5 us for the activation's preparation unless the rows
+    arrive prepared (llmq_add_rmsnorm_prepared, the gate|up epilogue)."""
+    launch = min(_tile_plan_cost(rows, out_features, groups, narrow, bits == 4) for narrow in (False, True))
+    return launch + (0.0 if prepared else 3.5)
+
+
+def dense_branch_cost(rows: int, out_features: int, groups: int, bits: int = 8) -> float:
+    """Estimated microseconds of dequantize + the BLAS library's matmul: 16 us of fixed cost (two launches, the
+    library's dispatch), the dequantize pass at 4 TB/s (codes in, 16-bit values out), the matmul at 1.5 PFLOP/s
+    (less below 400 rows and on reduction axes beyond 4096). Fitted to the same measurements; the library's kernels vary
+    more with shape than this."""
+    weights = out_features * groups * 128
+    matmul = 2.0 * rows * weights / 1.5e9 / min(1.0, rows / 400) * (1.0 + max(0, groups * 128 - 4096) / 32768)
+    return 16.0 + weights * (bits / 8 + 2) / 4.0e6 + matmul
+
+
+def tiled_gemm_pays(rows: int, out_features: int, groups: int, bits: int = 8, prepared: bool = False) -> bool:
+    """Whether the tiled fused GEMM is the branch for this many activation rows. Up to 128 rows: wide or long
+    weights, and mid-sized ones (the fused GEMM for a few dozen rows keeps the narrow short ones). Beyond: where its
+    estimated time is within 5 % of dequantize + matmul's (a tie goes to the branch that builds no dense weight).
+    Measured, M x N x K int4, tiled / dense us: 512 x 16384 x 2048 46 / 54, 640 x 16384 x 2048 77 / 59 (320 tiles:
+    a second round), 512 x 28672 x 4096 143 / 164, 640 x 4096 x 14336 102 / 120, 1024 x 14336 x 4096 149 / 122;
+    int8: 512 x 3072 x 2048 24.2 / 24.9, 192 x 3072 x 2048 17.1 / 24.4, 1024 x 3072 x 2048 33.0 / 28.7,
+    136 x 512 x 2048 12.6 / 13.8."""
     if not FUSED_GEMM_MAX_ROWS < rows <= TILED_GEMM_MAX_ROWS:
         return False
-    if out_features >= 8192 or groups >= 64:
-        return True
-    # 512 x 3072 x 2048 int8 24.4 us against 24.4 for dequantize + matmul (int4 21.1 / 24.6), 512 x 4096 x 2048
-    # 23.6 / 26.6, 192 x 3072 x 2048 16.9 / 24.4; at most 5 % behind where it is behind (384 x 3072, 1024 x 2048)
-    narrow_tiles = -(-rows // 64) * -(-out_features // 128)
-    if (rows > FUSED_GEMM_SLAB_MAX_ROWS and groups <= TILED_GEMM_NARROW_MAX_GROUPS
-            and TILED_GEMM_NARROW_MIN_TILES <= narrow_tiles <= TILED_GEMM_NARROW_MAX_TILES):
-        return True
-    # one tile of rows on a mid-sized weight (Llama-3-8B's q|k|v, 6144 x 4096 int8, M = 65-128: 24.8-27.1 us against
-    # 32.7-36.0 for dequantize + matmul); smaller weights take the fused GEMM for a few dozen rows twice instead
-    return rows <= 128 and out_features * groups > FUSED_GEMM_SLAB_MAX_GROUP_ROWS
+    if rows <= FUSED_GEMM_SLAB_MAX_ROWS:
+        # one tile of rows on a mid-sized weight (Llama-3-8B's q|k|v, 6144 x 4096 int8, M = 65-128: 24.8-27.1 us
+        # against 32.7-36.0 for dequantize + matmul); smaller weights take the fused GEMM for a few dozen rows twice
+        return out_features >= 8192 or groups >= 64 or out_features * groups > FUSED_GEMM_SLAB_MAX_GROUP_ROWS
+    return (tiled_gemm_cost(rows, out_features, groups, bits, prepared)
+            <= 1.05 * dense_branch_cost(rows, out_features, groups, bits))
 
 
 #: Narrow, short weights (N * groups up to 4096 x 32: q|k|v and o_proj of the 1B and 8B models) keep the fused GEMM up
@@ -234,8 +260,9 @@ class KernelQuantLinear(nn.Module):
         fused = (self._fused_max_rows > 0 and fused_gemm_takes(rows.shape[0], self.out_features, self.qdata.shape[1])
                  and (rows.shape[0] <= self._fused_max_rows or not self._head_keep)
                  and rows.dtype in (torch.bfloat16, torch.float16) and not self._int8_act)
-        tiled = (self._fused_max_rows > 0 and rows.dtype == torch.bfloat16 and not self._int8_act
-                 and tiled_gemm_pays(rows.shape[0], self.out_features, self.qdata.shape[1]))
+        tiled = (self._fused_max_rows > 0 and rows.dtype in (torch.bfloat16, torch.float16) and not self._int8_act
+                 and tiled_gemm_pays(rows.shape[0], self.out_features, self.qdata.shape[1],
+                                     4 if self.qdata.dtype == torch.uint8 else 8))
         if rows.shape[0] > KERNEL_MAX_ROWS and not self._int8_act and self._head_keep and not fused and not tiled:
             # dense branch on the real width: neither the activation nor the weight is padded
             out = self._dense(rows, real_width=True)

@@ -54,6 +54,10 @@ MID_CONTEXT_FROM = 5120
 LONG_CONTEXT_FROM = 16384
 
 
+def _code_bits(qdata) -> int:
+    return 4 if qdata.dtype == torch.uint8 else 8
+
+
 class PreparedRows:
     """Normed rows of a prompt in the tiled fused GEMM's prepared form (operand order, per-group sums) inside that
     GEMM's workspace, in place of the tensor: what llmq_add_rmsnorm_prepared leaves."""
@@ -179,33 +183,40 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         self._argmax_ws = torch.zeros(self._ext.argmax_workspace_ints(), dtype=torch.int32, device=self.device)
 
     # ---- the prompt pass: q|k|v and gate|up as one projection each ----------------------------------
-    def _takes_tile(self, rows, dtype, fused):
-        """Whether _project sends this many rows of this dtype to the tiled fused GEMM."""
+    def _takes_tile(self, rows, dtype, fused, prepared=False):
+        """Whether _project sends this many rows of this dtype to the tiled fused GEMM (`prepared`: when the norm in
+        front of it can write them in the GEMM's prepared form, which saves the preparation launch)."""
         from llmquant.quantizers.kernel import KERNEL_MAX_ROWS, fused_gemm_takes, tiled_gemm_pays
 
         n, groups = fused.qdata.shape[0], fused.qdata.shape[1]
-        return (dtype == torch.bfloat16 and rows > KERNEL_MAX_ROWS and not fused_gemm_takes(rows, n, groups)
-                and tiled_gemm_pays(rows, n, groups))
+        return (dtype in (torch.bfloat16, torch.float16) and rows > KERNEL_MAX_ROWS and not fused_gemm_takes(rows, n, groups)
+                and tiled_gemm_pays(rows, n, groups, _code_bits(fused.qdata), prepared))
 
     def _mlp_in_two_launches(self, rows, dtype, index, layer):
         """Whether _mlp runs this many rows as gate|up with the activation in its store + down_proj."""
-        from llmquant.quantizers.kernel import FUSED_GEMM_MAX_ROWS, TILED_GEMM_MAX_ROWS, tiled_gemm_pays
+        from llmquant.quantizers.kernel import (FUSED_GEMM_MAX_ROWS, TILED_GEMM_MAX_ROWS, dense_branch_cost,
+                                                tiled_gemm_cost)
 
         f = self.fused_layers[index]
         gate_up, down = f["gate_up"], f["down"]
         inter = gate_up.qdata.shape[0] // 2
-        return (dtype == torch.bfloat16 and self._one_launch_ops and "SiLU" in type(layer.mlp.act_fn).__name__
+        # down_proj on rows that the gate|up launch left prepared, against the dense branch behind a SiLU * up launch
+        # (6 us) of its own
+        down_n, down_groups, down_bits = down.out_features, down.qdata.shape[1], _code_bits(down.qdata)
+        down_pays = (tiled_gemm_cost(rows, down_n, down_groups, down_bits, prepared=True)
+                     <= 1.05 * (dense_branch_cost(rows, down_n, down_groups, down_bits) + 6.0))
+        return (dtype in (torch.bfloat16, torch.float16) and self._one_launch_ops and "SiLU" in type(layer.mlp.act_fn).__name__
                 and FUSED_GEMM_MAX_ROWS < rows <= TILED_GEMM_MAX_ROWS and inter % 128 == 0
                 and -(-rows // 128) * (inter // 128) >= 160
-                and tiled_gemm_pays(rows, down.out_features, down.qdata.shape[1])
-                and down.bias is None and not down._needs_padding and not down._int8_act
+                and down_pays and down.bias is None and not down._needs_padding and not down._int8_act
                 and down.qdata.shape[1] * 128 == inter)
 
     def _add_norm(self, module, hidden, branch, consumer=None):
         """The base class's, except that rows on their way to a tiled fused GEMM leave the norm in that GEMM's
         prepared form (llmq_add_rmsnorm_prepared: the bits of norm + preparation, one launch and one tensor
         fewer): the second value is then a PreparedRows for _project / _mlp."""
-        if (consumer is not None and self._one_launch_ops and hidden.dim() == 2 and hidden.dtype == torch.bfloat16
+        if (consumer is not None and self._one_launch_ops and hidden.dim() == 2
+                and hidden.dtype in (torch.bfloat16, torch.float16)
                 and type(module).__name__.endswith("RMSNorm") and hasattr(module, "variance_epsilon")
                 and hidden.shape[-1] % 128 == 0 and module.weight.dtype == hidden.dtype
                 and (branch is None or branch.dtype == hidden.dtype)):
@@ -213,7 +224,7 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
             rows, f = hidden.shape[0], self.fused_layers[index]
             fused = f["qkv"] if kind == "qkv" else f["gate_up"]
             direct = isinstance(fused, _Fused) and fused.qdata.shape[1] * 128 == hidden.shape[-1]
-            if direct and (self._takes_tile(rows, hidden.dtype, fused)
+            if direct and (self._takes_tile(rows, hidden.dtype, fused, prepared=True)
                            or (kind == "mlp" and self._mlp_in_two_launches(rows, hidden.dtype, index,
                                                                           self.layers[index]))):
                 next_n = max(fused.qdata.shape[0], f["down"].out_features if kind == "mlp" else 0)
@@ -229,7 +240,8 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
         from llmquant.quantizers.kernel import KERNEL_MAX_ROWS, fused_gemm_splits, fused_gemm_takes, tiled_gemm_pays
 
         if isinstance(x, PreparedRows):   # (_add_norm found that these rows take the tiled GEMM)
-            return self._ext.wq_gemm_a16_tile_prepared(x.workspace, x.rows, fused.qdata, fused.wscale, fused.out_group)
+            return self._ext.wq_gemm_a16_tile_prepared(x.workspace, x.rows, fused.qdata, fused.wscale, fused.out_group,
+                                                       x.dtype)
         rows = x.shape[0]
         if (fused_gemm_takes(rows, fused.qdata.shape[0], fused.qdata.shape[1])
                 and x.dtype in (torch.bfloat16, torch.float16)):
@@ -237,7 +249,7 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
                                          fused_gemm_splits(rows, fused.qdata.shape[1]))
         if rows <= KERNEL_MAX_ROWS:
             return self._ext.wq_gemv(x, fused.qdata, fused.wscale, fused.out_group)
-        if x.dtype == torch.bfloat16 and tiled_gemm_pays(rows, fused.qdata.shape[0], fused.qdata.shape[1]):
+        if self._takes_tile(rows, x.dtype, fused):
             return self._ext.wq_gemm_a16_tile(x.contiguous(), fused.qdata, fused.wscale, fused.out_group)
         if x.dtype in (torch.bfloat16, torch.float16):
             return self._ext.wq_dense_linear(x.contiguous(), fused.qdata, fused.wscale, fused.out_group, 0)
@@ -265,11 +277,11 @@ class LlamaFusedRuntime(LlamaKernelRuntime):
             if isinstance(x, PreparedRows):
                 workspace = self._ext.wq_gemm_a16_tile_gate_up_silu_prepared(x.workspace, rows, gate_up.qdata,
                                                                              gate_up.wscale, gate_up.out_group,
-                                                                             down.out_features)
+                                                                             down.out_features, x.dtype)
             else:
                 workspace = self._ext.wq_gemm_a16_tile_gate_up_silu(x.contiguous(), gate_up.qdata, gate_up.wscale,
                                                                     gate_up.out_group, down.out_features)
-            return self._ext.wq_gemm_a16_tile_prepared(workspace, rows, down.qdata, down.wscale, down.out_group)
+            return self._ext.wq_gemm_a16_tile_prepared(workspace, rows, down.qdata, down.wscale, down.out_group, x.dtype)
         return super()._mlp(index, layer, x)
 
     def _forward(self, token_ids, cos, sin, decode: bool):

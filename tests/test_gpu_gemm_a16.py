@@ -154,9 +154,10 @@ def no_tile_shape_left_pinned():
     os.environ.pop("LLMQ_A16_TILE", None)
 
 
-def tile_case(ext, m, n, k, bits, out_group=0, head_dim=None, seed=0, scale=1.0, offset=0.0, tile=None):
-    """x [m, k] bf16 against a quantized [n, k] weight through wq_gemm_a16_tile; returns the result and the
-    oracle's operands (activation padded the way the weight was)."""
+def tile_case(ext, m, n, k, bits, out_group=0, head_dim=None, seed=0, scale=1.0, offset=0.0, tile=None,
+              dtype=torch.bfloat16):
+    """x [m, k] bf16 (or fp16) against a quantized [n, k] weight through wq_gemm_a16_tile; returns the result and
+    the oracle's operands (activation padded the way the weight was)."""
     import os
 
     if tile is None:
@@ -164,13 +165,13 @@ def tile_case(ext, m, n, k, bits, out_group=0, head_dim=None, seed=0, scale=1.0,
     else:
         os.environ["LLMQ_A16_TILE"] = tile
     torch.manual_seed(seed)
-    w = (torch.randn(n, k) * 0.02).to(torch.bfloat16)
-    x = (torch.randn(m, k) * scale + offset).to(torch.bfloat16)
+    w = (torch.randn(n, k) * 0.02).to(dtype)
+    x = (torch.randn(m, k) * scale + offset).to(dtype)
     canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP, head_dim, out_group or None)
     q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
     s = torch.from_numpy(scales).cuda()
     padded = oracle.pad_activation(to_np(x), GROUP, head_dim)
-    got = ext.wq_gemm_a16_tile(torch.from_numpy(padded).to(torch.bfloat16).cuda(), q, s, out_group)
+    got = ext.wq_gemm_a16_tile(torch.from_numpy(padded).to(dtype).cuda(), q, s, out_group)
     return got, padded, canonical, scales
 
 
@@ -191,6 +192,56 @@ def test_tiled_gemm_against_the_oracle(ext, bits, m, n, k, tile):
     real = oracle.real_linear(x, canonical, scales, "bf16")
     assert ulp_distance(to_np(got), real, torch.bfloat16) <= 1
     assert (to_np(got) == real).mean() > 0.99
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,n,k", [(128, 256, 128), (130, 300, 768), (512, 512, 2048), (300, 70, 384), (256, 1024, 8192),
+                                   (65, 70, 1024), (512, 3072, 2048)])
+@SHAPES
+def test_tiled_gemm_float16_against_the_oracle(ext, bits, m, n, k, tile):
+    """float16 activations: the codes enter the matrix core as themselves (the bias of the bf16 form is taken off
+    the operand, exactly), so there is no correction term; same bars as the bf16 form, with float16's rounding of
+    the output. A second case with activations near float16's largest values: products and sums are fp32, nothing
+    overflows on the way."""
+    got, x, canonical, scales = tile_case(ext, m, n, k, bits, seed=m + n, tile=tile, dtype=torch.float16)
+    assert got.shape == (m, n) and got.dtype == torch.float16
+    exact = oracle.gemv_float64(x, canonical, scales)
+    assert rel_l2(to_np(got), exact) <= 3e-4
+    real = oracle.real_linear(x, canonical, scales, "f16")
+    assert ulp_distance(to_np(got), real, torch.float16) <= 1
+    assert (to_np(got) == real).mean() > 0.99
+    if (m, n, k) == (130, 300, 768):
+        got, x, canonical, scales = tile_case(ext, m, n, k, bits, seed=2, tile=tile, dtype=torch.float16, scale=2000.0,
+                                              offset=30000.0)
+        assert np.abs(x).max() > 30000 and torch.isfinite(got).all()
+        assert rel_l2(to_np(got), oracle.gemv_float64(x, canonical, scales)) <= 3e-4
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_gate_up_silu_epilogue_float16(ext, bits):
+    """The two-launch MLP on float16 activations against the three launches, equal to the bit (wide tile pinned, as
+    for bf16), and the norm in front of it written as prepared rows."""
+    import os
+
+    os.environ["LLMQ_A16_TILE"] = "wide"
+    m, inter, k, n_down = 200, 256, 256, 300
+    x, q_gu, s_gu, q_d, s_d, _ = mlp_case(m, inter, k, n_down, bits, seed=9)
+    x = (x.float() * 0.5).half()
+    gate_up = ext.wq_gemm_a16_tile(x, q_gu, s_gu, 0)
+    act = ext.silu_mul(gate_up[:, :inter], gate_up[:, inter:])
+    want = ext.wq_gemm_a16_tile(act, q_d, s_d, 0)
+    workspace = ext.wq_gemm_a16_tile_gate_up_silu(x, q_gu, s_gu, 0, n_down)
+    got = ext.wq_gemm_a16_tile_prepared(workspace, m, q_d, s_d, 0, torch.float16)
+    assert got.dtype == torch.float16 and torch.equal(got, want)
+    weight = (1 + 0.1 * torch.randn(k, device="cuda")).half()
+    delta = torch.randn_like(x)
+    hidden, normed = ext.add_rmsnorm(x, delta, weight, 1e-5)
+    want = ext.wq_gemm_a16_tile_prepared(ext.wq_gemm_a16_tile_gate_up_silu(normed, q_gu, s_gu, 0, n_down), m, q_d, s_d, 0,
+                                         torch.float16)
+    got_hidden, ws = ext.add_rmsnorm_prepared(x, delta, weight, 1e-5, max(2 * inter, n_down))
+    got = ext.wq_gemm_a16_tile_prepared(ext.wq_gemm_a16_tile_gate_up_silu_prepared(ws, m, q_gu, s_gu, 0, n_down, torch.float16),
+                                        m, q_d, s_d, 0, torch.float16)
+    assert torch.equal(got_hidden, hidden) and torch.equal(got, want)
 
 
 @pytest.mark.parametrize("bits", [4, 8])
@@ -251,8 +302,8 @@ def test_tiled_gemm_at_llama_8b_mlp_shapes(ext, n, k, m):
 def test_tiled_gemm_argument_checks(ext):
     x, q, s, _, _ = make_case(128, 256, 256, 4, torch.bfloat16)
     assert ext.wq_gemm_a16_tile(x.cuda(), q, s, 0).shape == (128, 256)
-    with pytest.raises(RuntimeError, match="bfloat16"):
-        ext.wq_gemm_a16_tile(x.cuda().half(), q, s, 0)
+    with pytest.raises(RuntimeError, match="bfloat16 or float16"):
+        ext.wq_gemm_a16_tile(x.cuda().float(), q, s, 0)
     with pytest.raises(RuntimeError, match="does not match qweight"):
         ext.wq_gemm_a16_tile(x.cuda()[:, :128].contiguous(), q, s, 0)
     with pytest.raises(RuntimeError, match="wscale must be"):
@@ -403,8 +454,8 @@ def test_gate_up_silu_epilogue_argument_checks(ext):
     x, q_gu, s_gu, q_d, s_d, _ = mlp_case(128, 128, 128, 64, 4, seed=1)
     with pytest.raises(RuntimeError, match="multiple of 128"):
         ext.wq_gemm_a16_tile_gate_up_silu(x, q_gu[:192], s_gu[:192], 0, 64)
-    with pytest.raises(RuntimeError, match="bfloat16"):
-        ext.wq_gemm_a16_tile_gate_up_silu(x.half(), q_gu, s_gu, 0, 64)
+    with pytest.raises(RuntimeError, match="bfloat16 or float16"):
+        ext.wq_gemm_a16_tile_gate_up_silu(x.float(), q_gu, s_gu, 0, 64)
     workspace = ext.wq_gemm_a16_tile_gate_up_silu(x, q_gu, s_gu, 0, 64)
     with pytest.raises(RuntimeError, match="this GEMM needs"):
         ext.wq_gemm_a16_tile_prepared(workspace[:16], 128, q_d, s_d, 0)
@@ -463,8 +514,8 @@ def test_gate_up_silu_epilogue_on_prepared_rows(ext, bits):
 def test_rmsnorm_into_prepared_form_argument_checks(ext):
     x = torch.randn(64, 256, device="cuda").to(torch.bfloat16)
     weight = torch.ones(256, device="cuda", dtype=torch.bfloat16)
-    with pytest.raises(RuntimeError, match="bfloat16"):
-        ext.add_rmsnorm_prepared(x.half(), None, weight.half(), 1e-5, 128)
+    with pytest.raises(RuntimeError, match="bfloat16 or float16"):
+        ext.add_rmsnorm_prepared(x.float(), None, weight.float(), 1e-5, 128)
     with pytest.raises(RuntimeError, match="multiple of 128"):
         ext.add_rmsnorm_prepared(x[:, :200].contiguous(), None, weight[:200].contiguous(), 1e-5, 128)
     with pytest.raises(RuntimeError, match="must match"):

@@ -342,10 +342,10 @@ def test_shape_and_dtype_checks(linear):
 
 def test_dense_branch_lands_where_fake_quant_does(linear):
     from llmquant.quantizers import FakeQuantLinear, KernelQuantLinear, RealQuantLinear
-    from llmquant.quantizers.kernel import FUSED_GEMM_SLAB_MAX_ROWS, fused_gemm_takes, tiled_gemm_pays
+    from llmquant.quantizers.kernel import TILED_GEMM_MAX_ROWS, fused_gemm_takes, tiled_gemm_pays
 
     lin = linear.cuda()
-    rows = FUSED_GEMM_SLAB_MAX_ROWS + 8   # past every fused form for a weight of this size
+    rows = TILED_GEMM_MAX_ROWS + 8   # past every fused form
     assert not fused_gemm_takes(rows, N, K // 128) and not tiled_gemm_pays(rows, N, K // 128)
     for name, spec in LAYOUTS.items():
         spec = dict(spec)

@@ -168,13 +168,30 @@ def test_narrow_short_weights_keep_the_fused_gemm_up_to_128_rows():
     assert fused_gemm_takes(64, 6144, 32) and not fused_gemm_takes(65, 6144, 32)
     assert fused_gemm_takes(64, 16384, 16) and not fused_gemm_takes(100, 16384, 16) and tiled_gemm_pays(100, 16384, 16)
     assert not fused_gemm_takes(100, 2048, 64) and tiled_gemm_pays(100, 2048, 64)
-    # a mid-sized weight (Llama-3-8B's q|k|v): one tile of rows goes to the tiled GEMM, more to the dense branch
-    assert tiled_gemm_pays(100, 6144, 32) and tiled_gemm_pays(128, 6144, 32) and not tiled_gemm_pays(129, 6144, 32)
+    # a mid-sized weight (Llama-3-8B's q|k|v): one tile of rows goes to the tiled GEMM; more, as long as the estimate
+    # says so (at 512 rows the library is ahead: 48.7 us against 46.5 measured)
+    assert tiled_gemm_pays(100, 6144, 32) and tiled_gemm_pays(128, 6144, 32) and tiled_gemm_pays(129, 6144, 32)
     assert not tiled_gemm_pays(100, 4096, 32) and not tiled_gemm_pays(100, 3072, 16)
+    # beyond 128 rows: by the estimated times of the two branches (measured cases on both sides of the line)
     # short rows on an output that 64 x 128 tiles cover in one round: q|k|v of Llama-3.2-1B at a 512-token prompt
     assert tiled_gemm_pays(512, 3072, 16) and tiled_gemm_pays(192, 3072, 16) and tiled_gemm_pays(512, 4096, 16)
     assert not tiled_gemm_pays(512, 3072, 24) and not tiled_gemm_pays(512, 2048, 32)   # longer rows: the library
-    assert not tiled_gemm_pays(1024, 3072, 16) and not tiled_gemm_pays(136, 512, 16)   # two rounds; a dozen tiles
+    assert not tiled_gemm_pays(1024, 3072, 16) and tiled_gemm_pays(136, 512, 16)   # two rounds; a dozen tiles (12.6 us / 13.8)
+    # wide int4 weights: one round of 128 x 256 tiles pays, a half-empty second round does not
+    assert tiled_gemm_pays(512, 14336, 32, 4) and not tiled_gemm_pays(640, 14336, 32, 4)
+    assert tiled_gemm_pays(512, 16384, 16, 4) and not tiled_gemm_pays(768, 16384, 16, 4)
+    assert not tiled_gemm_pays(1024, 14336, 32, 4) and not tiled_gemm_pays(1025, 2048, 64, 4)
+    # a weight whose dequantize pass alone is 73 us keeps the tiled GEMM through its second round; long rows are cut
+    assert tiled_gemm_pays(512, 28672, 32, 4) and not tiled_gemm_pays(896, 28672, 32, 4)
+    assert tiled_gemm_pays(640, 4096, 112, 4) and tiled_gemm_pays(1024, 2048, 64, 4) and tiled_gemm_pays(768, 2048, 64, 4)
+    from llmquant.quantizers.kernel import dense_branch_cost, tiled_gemm_cost
+
+    # the estimates against launches measured on an MI355X (us): within a tenth for the tiled GEMM
+    for (m, n, g, bits), measured in {(512, 3072, 16, 8): 24.2, (512, 16384, 16, 4): 46.1, (640, 14336, 32, 4): 139.6,
+                                      (2048, 14336, 32, 4): 278.5, (128, 14336, 32, 4): 31.7}.items():
+        assert abs(tiled_gemm_cost(m, n, g, bits) / measured - 1) <= 0.1, (m, n, g, bits)
+    assert abs(dense_branch_cost(512, 28672, 32, 4) / 163.6 - 1) <= 0.1
+    assert tiled_gemm_cost(512, 3072, 16, 8, prepared=True) == tiled_gemm_cost(512, 3072, 16, 8) - 3.5
 
 
 # ---- layout ---------------------------------------------------------------------------------------------
