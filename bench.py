@@ -588,18 +588,25 @@ def other_kernels(torch):
                          "weights_rotated_over_bytes": copies * (n * k // 2)})
         del q4s
     out["w4a8_gemm"] = gemm
-    # prompt-sized bf16 activations: the tiled fused GEMM (no dense weight) against the branch it replaces
-    # (one-pass dequantize + the BLAS library's matmul), weights rotated the same way
+    # prompt-sized bf16 (one row: fp16) activations: the tiled fused GEMM (no dense weight) against the branch it
+    # replaces (one-pass dequantize + the BLAS library's matmul), weights rotated the same way; `routed_to` is what
+    # KernelQuantLinear.forward picks for the shape (tiled_gemm_pays: the estimated times of the two branches)
+    from llmquant.quantizers.kernel import tiled_gemm_pays
+
     tiled = []
-    for m, n, k, bits in ((512, 16384, 2048, 4), (512, 2048, 8192, 4), (512, 3072, 2048, 8), (128, 14336, 4096, 4),
-                          (512, 14336, 4096, 4), (2048, 14336, 4096, 4), (2048, 4096, 14336, 4)):
+    for m, n, k, bits, dtype in ((512, 16384, 2048, 4, torch.bfloat16), (512, 2048, 8192, 4, torch.bfloat16),
+                                 (512, 3072, 2048, 8, torch.bfloat16), (512, 3072, 2048, 4, torch.bfloat16),
+                                 (192, 3072, 2048, 8, torch.bfloat16), (128, 14336, 4096, 4, torch.bfloat16),
+                                 (512, 14336, 4096, 4, torch.bfloat16), (512, 14336, 4096, 4, torch.float16),
+                                 (640, 14336, 4096, 4, torch.bfloat16), (1024, 2048, 8192, 4, torch.bfloat16),
+                                 (2048, 14336, 4096, 4, torch.bfloat16), (2048, 4096, 14336, 4, torch.bfloat16)):
         copies = min(24, (300 << 20) // (n * k * bits // 8) + 1)
         width = GROUP if bits == 8 else GROUP // 2
         qs = [torch.randint(0, 255, (n, k // GROUP, width), dtype=torch.uint8, device=dev) for _ in range(copies)]
         if bits == 8:
             qs = [q.view(torch.int8) for q in qs]
         sw = torch.rand(n, k // GROUP, device=dev) * 0.01 + 1e-3
-        x = torch.randn(m, k, device=dev).to(torch.bfloat16)
+        x = torch.randn(m, k, device=dev).to(dtype)
         turn = [0]
 
         def fused_call():
@@ -612,10 +619,12 @@ def other_kernels(torch):
 
         us_f = _event_time_us(torch, fused_call, reps=2 * copies)
         us_d = _event_time_us(torch, dense_call, reps=2 * copies)
-        tiled.append({"M": m, "N": n, "K": k, "weights": f"int{bits}", "us": round(us_f, 1),
+        tiled.append({"M": m, "N": n, "K": k, "weights": f"int{bits}",
+                      "activations": "bf16" if dtype == torch.bfloat16 else "fp16", "us": round(us_f, 1),
                       "TFLOPs": round(2 * m * n * k / us_f / 1e6, 1),
                       "frac_bf16_mfma_peak": round(2 * m * n * k / us_f / 1e6 / 2500.0, 4),
-                      "dequant_plus_matmul_us": round(us_d, 1)})
+                      "dequant_plus_matmul_us": round(us_d, 1),
+                      "routed_to": "tiled" if tiled_gemm_pays(m, n, k // GROUP, bits) else "dequant_plus_matmul"})
         del qs
     out["w4a16_tiled_gemm_prompt_m"] = tiled
     # a few dozen rows of a 16-bit activation: the fused GEMM (codes straight from HBM to the matrix cores)
