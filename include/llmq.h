@@ -215,11 +215,12 @@ int llmq_wq_gemm_a16_split(const void* x, const void* qweight, const float* wsca
 
 /* The same GEMM for prompt-sized activations (M in the hundreds and thousands), the reference's M > 4 branch
  * (dequantize the whole weight to the activation dtype, then the BLAS library: llmquant/quantizers/kernel.py:
- * 68-79, 88-91) without the dense weight: 128 x 256 output tiles, bf16 matrix cores, codes turned into bf16
- * operands in registers, the reduction axis split across workgroups (fp32 partial tiles, added in a fixed
- * order by a second launch) when the output has too few tiles to occupy the chip. Same sum as
+ * 68-79, 88-91) without the dense weight: 128 x 256 output tiles (64 x 128 where the output has few of those; the
+ * cheaper plan by an estimate of both, LLMQ_A16_TILE=wide / narrow in the environment pins one), 16-bit matrix
+ * cores, codes turned into operands in registers, the reduction axis split across workgroups (fp32 partial tiles,
+ * added in a fixed order by a second launch) when the output has too few tiles to occupy the chip. Same sum as
  * llmq_wq_gemm_a16: products exact, fp32 accumulation, one scale per group.
- * x, out: LLMQ_BF16 only, 16-byte aligned; gs must be 128. `workspace`: llmq_wq_gemm_a16_tile_workspace_bytes
+ * x, out: LLMQ_BF16 or LLMQ_F16, 16-byte aligned; gs must be 128. `workspace`: llmq_wq_gemm_a16_tile_workspace_bytes
  * (M, N, G) bytes, 16-byte aligned, contents irrelevant before and after (it holds the activation in operand
  * order, its per-group sums, and the partial tiles). Calls that share a workspace must not overlap. */
 size_t llmq_wq_gemm_a16_tile_workspace_bytes(int M, int N, int G);
@@ -253,7 +254,7 @@ int llmq_wq_gemm_a16_tile_gate_up_silu_prepared(const void* qweight, const float
  * llmq_wq_gemm_a16_tile_prepared_bytes(rows, hidden / 128) bytes of `workspace` instead of as a tensor: what
  * llmq_wq_gemm_a16_tile would make of that tensor, bit for bit, without the tensor and without the preparation
  * launch; `workspace` is then the workspace of llmq_wq_gemm_a16_tile_prepared (q|k|v) or
- * llmq_wq_gemm_a16_tile_gate_up_silu_prepared with M = rows, G = hidden / 128. LLMQ_BF16 only; hidden a multiple
+ * llmq_wq_gemm_a16_tile_gate_up_silu_prepared with M = rows, G = hidden / 128. LLMQ_BF16 or LLMQ_F16; hidden a multiple
  * of 128; delta_or_null and sum_out_or_null as in llmq_add_rmsnorm. No counterpart in the reference (transformers'
  * LlamaRMSNorm.forward followed by the Linear's M > 4 branch, llmquant/quantizers/kernel.py:68-79). */
 int llmq_add_rmsnorm_prepared(const void* x, const void* delta_or_null, const void* weight, void* sum_out_or_null,

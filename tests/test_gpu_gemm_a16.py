@@ -210,6 +210,13 @@ def test_tiled_gemm_float16_against_the_oracle(ext, bits, m, n, k, tile):
     real = oracle.real_linear(x, canonical, scales, "f16")
     assert ulp_distance(to_np(got), real, torch.float16) <= 1
     assert (to_np(got) == real).mean() > 0.99
+    if (m, n, k) == (512, 512, 2048):
+        # one scale row per 64 weight rows, and heads of 64 padded to groups
+        for spec in (dict(out_group=64), dict(head_dim=64)):
+            got, x, canonical, scales = tile_case(ext, m, n, k, bits, seed=4, tile=tile, dtype=torch.float16, **spec)
+            og = spec.get("out_group")
+            full = np.repeat(scales, og, axis=0)[:n] if og else scales
+            assert rel_l2(to_np(got), oracle.gemv_float64(x, canonical, full)) <= 3e-4
     if (m, n, k) == (130, 300, 768):
         got, x, canonical, scales = tile_case(ext, m, n, k, bits, seed=2, tile=tile, dtype=torch.float16, scale=2000.0,
                                               offset=30000.0)
