@@ -11,11 +11,12 @@
 //
 // Here the eight waves of a workgroup take DIFFERENT groups of the same 32 x 32 output tile: in round r, wave w
 // computes p for group 8 r + w (operands of its own, nothing shared, no barrier: loaded as whole rows a round
-// ahead and turned into matrix-core operand layout through the wave's LDS slot), leaves the 32 x 32 fp32 terms
-// in that slot, and after a barrier every wave adds, for
-// its eighth of the tile, slot 0, slot 1, ... slot 7 onto its running totals: the additions happen in group
-// order, one at a time, exactly as in the serial walk. A tile's chain is G / 8 rounds long; the next round's
-// operands are in flight across the barriers. Cost: every term crosses LDS once (8 bytes per output and group).
+// ahead and turned into matrix-core operand layout through the wave's LDS slot) and leaves the 32 x 32 fp32 terms
+// in that slot; the round ends with one barrier, and during the NEXT round (whose terms go to a second set of
+// slots) every wave adds, for its eighth of the tile, slot 0, slot 1, ... slot 7 of the round before onto its
+// running totals: the additions happen in group order, one at a time, exactly as in the serial walk, under the
+// next round's loads and multiplies. A tile's chain is G / 8 rounds long. Cost: every term crosses LDS once
+// (8 bytes per output and group).
 //
 // Operand layout. v_mfma_i32_32x32x32_i8 takes from lane l: row l % 32, sixteen k-values of half l / 32. A lane
 // owns one half of a group's 128 k-values (64 contiguous bytes of a row of activations, 32 bytes of packed
@@ -60,16 +61,16 @@ template <int BITS> struct Operands {
   u32x4 rb[BITS == 8 ? 4 : 2];
 };
 
-constexpr int kChunkGroups = 32;   // groups whose scales sit in LDS at a time
+constexpr int kChunkGroups = 16;   // groups whose scales sit in LDS at a time (two such chunks: one in use, one coming)
 
 
 
 template <typename T, int BITS>
 __device__ __forceinline__ void groups_body(const GroupArgs& g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  float* slots = reinterpret_cast<float*>(smem);                       // [kWays][kSlotFloats]
-  float* s_sx = slots + kWays * kSlotFloats;                           // [kChunkGroups][kTM]
-  float* s_sw = s_sx + kChunkGroups * kTM;                             // [kChunkGroups][kTN]
+  float* slots = reinterpret_cast<float*>(smem);                       // [2][kWays][kSlotFloats]: rounds alternate
+  float* s_sx = slots + 2 * kWays * kSlotFloats;                       // [2][kChunkGroups][kTM]: chunks alternate
+  float* s_sw = s_sx + 2 * kChunkGroups * kTM;                         // [2][kChunkGroups][kTN]
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid >> 6;
   const int col = lane & 31, half = lane >> 5;
@@ -100,28 +101,24 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
     for (int i = 0; i < kBPackets; ++i) o.rb[i] = load16(g.qw + (b_off[i] + static_cast<uint32_t>(grp) * kGroupBytesB));
   };
 
-  // The tile's scales, kChunkGroups groups at a time, as [group][row] and [group][column]: a thread reads four of
-  // them a chunk ahead (32 consecutive groups of a row are one cache line) and puts them into LDS between the two
-  // barriers of the chunk's last round.
-  float pre_sx[2], pre_sw[2];
+  // The tile's scales, kChunkGroups groups at a time, as [group][row] and [group][column]: a thread reads one of
+  // each a chunk ahead (16 consecutive groups of a row are half a cache line) and puts them into the buffer that
+  // the chunk before the current one used, during the current chunk's last round (a barrier after every round
+  // separates that from the buffer's last reader and from its first).
+  static_assert(kThreads == kChunkGroups * kTM && kTM == kTN, "one activation scale and one weight scale a thread");
+  float pre_sx, pre_sw;
   auto load_chunk = [&](int chunk) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      // (groups past the end: clamped, so that the loads are unconditional; those values are never multiplied with)
-      const int idx = tid + kThreads * i, row = idx >> 5, grp = min(chunk * kChunkGroups + (idx & 31), g.G - 1);
-      const int n = min(n0 + row, g.N - 1);
-      pre_sx[i] = g.sx[static_cast<int64_t>(min(m0 + row, g.M - 1)) * g.G + grp];
-      pre_sw[i] = g.sw[static_cast<int64_t>(g.out_group > 0 ? n / g.out_group : n) * g.G + grp];
-    }
+    // (groups past the end: clamped, so that the loads are unconditional; those values are never multiplied with)
+    const int row = tid / kChunkGroups, grp = min(chunk * kChunkGroups + tid % kChunkGroups, g.G - 1);
+    const int n = min(n0 + row, g.N - 1);
+    pre_sx = g.sx[static_cast<int64_t>(min(m0 + row, g.M - 1)) * g.G + grp];
+    pre_sw = g.sw[static_cast<int64_t>(g.out_group > 0 ? n / g.out_group : n) * g.G + grp];
   };
-  auto store_chunk = [&]() {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int idx = tid + kThreads * i;
-      s_sx[(idx & 31) * kTM + (idx >> 5)] = pre_sx[i];
-      // (the unpacked nibbles are 16 x their codes: the 16 leaves here, exactly)
-      s_sw[(idx & 31) * kTN + (idx >> 5)] = BITS == 4 ? pre_sw[i] * 0.0625f : pre_sw[i];
-    }
+  auto store_chunk = [&](int chunk) {
+    const int at = (chunk & 1) * kChunkGroups * kTM + (tid % kChunkGroups) * kTM + tid / kChunkGroups;
+    s_sx[at] = pre_sx;
+    // (the unpacked nibbles are 16 x their codes: the 16 leaves here, exactly)
+    s_sw[at] = BITS == 4 ? pre_sw * 0.0625f : pre_sw;
   };
 
   // One group's terms into this wave's slot. The slot (4 KB) first serves as the wave's staging area, for the
@@ -131,8 +128,8 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
   // barriers keep the compiler from moving them.
   // Result register r of the 32 x 32 product is row 8 (r / 4) + 4 half + r % 4, column col; the slot keeps the
   // terms as [r / 4][lane][r % 4].
-  auto produce = [&](const Operands<BITS>& o, int grp) {
-    unsigned char* stage = reinterpret_cast<unsigned char*>(slots + wv * kSlotFloats);
+  auto produce = [&](const Operands<BITS>& o, int grp, float* round_slots) {
+    unsigned char* stage = reinterpret_cast<unsigned char*>(round_slots + wv * kSlotFloats);
     // piece `piece` of 128-byte line `line`, XOR-swizzled
     auto piece_at = [](int line, int piece) { return line * 128 + ((piece ^ (line & 7)) << 4); };
     // packet 64 i + lane is piece lane % 8 of line 8 i + lane / 8: one address, the rest are constant offsets
@@ -184,8 +181,8 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
     v16i d = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) d = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks], fb[ks], d, 0, 0, 0);
-    float* slot = slots + wv * kSlotFloats;
-    const int gl = grp & (kChunkGroups - 1);
+    float* slot = round_slots + wv * kSlotFloats;
+    const int gl = grp & (2 * kChunkGroups - 1);   // (chunk parity, group in the chunk)
     const float sw = s_sw[gl * kTN + col];
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
@@ -206,9 +203,9 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
   // this wave's eighth of the tile in the additions: result registers 4 (wv / 2) + 2 (wv % 2) + {0, 1} of every lane
   float total[2] = {0.0f, 0.0f};
   const int my_pair = ((wv >> 1) * kWave + lane) * 4 + 2 * (wv & 1);
-  auto add_round = [&](int valid) {
+  auto add_round = [&](const float* round_slots, int valid) {
     for (int s = 0; s < valid; ++s) {
-      const u32x2 v = *reinterpret_cast<const u32x2*>(slots + s * kSlotFloats + my_pair);
+      const u32x2 v = *reinterpret_cast<const u32x2*>(round_slots + s * kSlotFloats + my_pair);
       total[0] = total[0] + __builtin_bit_cast(float, v.x);
       total[1] = total[1] + __builtin_bit_cast(float, v.y);
     }
@@ -220,29 +217,39 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
   Operands<BITS> cur, nxt;
   if (wv < g.G) load(cur, wv);
   load_chunk(0);
-  store_chunk();
+  store_chunk(0);
   load_chunk(1);   // (past the last group: clamped loads whose values are never stored)
   __syncthreads();   // the first chunk's scales are in place
-  // between the two barriers of a chunk's last round nobody multiplies with its scales any more, and the next
-  // round does not start before the second barrier: the next chunk goes in, and the one after it is requested
+  // in the last round of a chunk the next chunk goes into the other buffer, and the one after it is requested
   auto turn_chunk = [&](int r) {
     if ((r + 1) % kRoundsPerChunk == 0 && r + 1 < rounds) {
-      store_chunk();
+      store_chunk((r + 1) / kRoundsPerChunk);
       load_chunk((r + 1) / kRoundsPerChunk + 1);
     }
   };
+  auto slots_of = [&](int r) { return slots + (r & 1) * kWays * kSlotFloats; };
   int r = 0;
+  // Round r: request the next round's operands, multiply this round's group into slots_of(r), add the terms of
+  // round r - 1 out of slots_of(r - 1), one barrier. (The barrier publishes this round's terms and ends the reads of
+  // the other set, which the next round overwrites.)
   // Steady state: this round's and the next round's group exist for every wave, so nothing branches around the
   // loads and the compiler's waits before the staging stores count exactly the loads that may stay in flight
   // (a branch around them makes it drain the next round's loads before this round's multiply). The operand set
   // is copied at the end of a round (two rounds per trip with the sets swapping roles needs 57 more registers).
+  if (r + 1 < full) {   // the first round has nothing to add yet
+    load(nxt, wv + kWays);
+    produce(cur, wv, slots_of(0));
+    turn_chunk(0);
+    __syncthreads();
+    cur = nxt;
+    r = 1;
+  }
   for (; r + 1 < full; ++r) {
     const int grp = r * kWays + wv;
     load(nxt, grp + kWays);
-    produce(cur, grp);
-    __syncthreads();
+    produce(cur, grp, slots_of(r));
+    add_round(slots_of(r - 1), kWays);
     turn_chunk(r);
-    add_round(kWays);
     __syncthreads();
     cur = nxt;
   }
@@ -250,13 +257,13 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
     const int grp = r * kWays + wv;
     const bool more = grp + kWays < g.G;
     if (more) load(nxt, grp + kWays);
-    if (grp < g.G) produce(cur, grp);
-    __syncthreads();
+    if (grp < g.G) produce(cur, grp, slots_of(r));
+    if (r > 0) add_round(slots_of(r - 1), kWays);   // (a round before the last is a full one)
     turn_chunk(r);
-    add_round(min(kWays, g.G - r * kWays));
     __syncthreads();
     if (more) cur = nxt;
   }
+  if (rounds > 0) add_round(slots_of(rounds - 1), min(kWays, g.G - (rounds - 1) * kWays));
 
   T* __restrict__ out = static_cast<T*>(g.out);
   const int n = n0 + col;
@@ -285,7 +292,7 @@ __global__ __launch_bounds__(kThreads) void wq_gemm_a8_groups_kernel8(const Grou
   groups_body<T, 8>(g);
 }
 
-constexpr size_t kLdsBytes = (static_cast<size_t>(kWays) * kSlotFloats + kChunkGroups * (kTM + kTN)) * sizeof(float);
+constexpr size_t kLdsBytes = 2 * (static_cast<size_t>(kWays) * kSlotFloats + kChunkGroups * (kTM + kTN)) * sizeof(float);
 
 template <typename T, int BITS>
 int launch(const GroupArgs& g, hipStream_t stream) {
