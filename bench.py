@@ -574,11 +574,26 @@ def other_kernels(torch):
                 turn[0] += 1
                 return ext.wq_gemm_a8(a, sx_token, q4s[turn[0] % copies], sw, None, 0, torch.bfloat16, False)
 
-            us = _event_time_us(torch, one, reps=2 * copies)
+            us_natural = _event_time_us(torch, one, reps=2 * copies)
             us_f = _event_time_us(torch, fast, reps=2 * copies)
             us_t = _event_time_us(torch, fast_token, reps=2 * copies)
             us_q = _event_time_us(torch, lambda: ext.quant_group_codes(x, 8, GROUP, False), reps=10)
+            # what KernelQuantLinear calls for the shape: where the exact form runs its group-parallel kernel, the
+            # quantizer writes the codes in that kernel's operand order (same codes, same result bit for bit)
+            operand_order = bool(ext.wq_gemm_a8_takes_groups(m, n, k // GROUP))
+            us = us_natural
+            if operand_order:
+                a_tiled, sx_tiled = ext.quant_act_codes_tiled(x, 4)
+
+                def tiled_call():
+                    turn[0] += 1
+                    return ext.wq_gemm_a8_tiled(a_tiled, sx_tiled, m, q4s[turn[0] % copies], sw)
+
+                us = _event_time_us(torch, tiled_call, reps=2 * copies)
+                us_q = _event_time_us(torch, lambda: ext.quant_act_codes_tiled(x, 4), reps=10)
             gemm.append({"M": m, "N": n, "K": k, "weights": "int4", "gemm_us": round(us, 1),
+                         "codes": "operand order (llmq_wq_gemm_a8_tiled)" if operand_order else "[M, K] (llmq_wq_gemm_a8)",
+                         "gemm_us_on_codes_in_natural_order": round(us_natural, 1),
                          "act_quant_us": round(us_q, 1), "TOPS": round(2 * m * n * k / us / 1e6, 1),
                          "frac_int8_mfma_peak": round(2 * m * n * k / us / 1e6 / 5000.0, 4),
                          "fast_form_us": round(us_f, 1), "fast_form_TOPS": round(2 * m * n * k / us_f / 1e6, 1),

@@ -173,6 +173,25 @@ int llmq_wq_gemm_a8(const int8_t* a, const float* sx, const void* qweight, const
                     const float* bias_or_null, void* out, int M, int N, int G, int gs,
                     int out_group, int wformat, int dtype, llmq_stream_t stream);
 
+/* llmq_wq_gemm_a8 with the activation codes in operand order, for the shapes where it runs its group-parallel
+ * kernel (few output tiles, long rows; llmq_wq_gemm_a8_takes_groups(M, N, G) != 0 says where this call is the
+ * faster one; LLMQ_A8_FORM in the environment pins the answer): the same result bit for bit, without the pass that turns activation rows into matrix-core operand
+ * layout inside the kernel (128 x 4096 x 14336 int4: 38 -> 31 us). llmq_quant_act_codes_tiled is llmq_quant_group_codes
+ * (int8 codes, groups of 128, the same arithmetic: scales [M, K / 128] equal) writing the codes where the kernel's
+ * waves read them: blocks of 32 rows x one group, [ceil(M / 32)][K / 128][4096] bytes, inside a block [k-step 0..3]
+ * [row % 32 + 32 * (k / 64)][16], and for packed int4 weights (wformat 4) every eight bytes as even k then odd k;
+ * `codes`: llmq_act_codes_tiled_bytes(M, K) bytes, 16-byte aligned; x: LLMQ_BF16 or LLMQ_F16 [M, K] contiguous.
+ * llmq_wq_gemm_a8_tiled takes any shape (arguments as for llmq_wq_gemm_a8, `codes_tiled` made for the same wformat).
+ * No counterpart in the reference, whose real mode keeps the codes inside RealQuantLinear.forward
+ * (llmquant/quantizers/real.py:76-88). */
+size_t llmq_act_codes_tiled_bytes(int M, int K);
+int llmq_quant_act_codes_tiled(const void* x, void* codes, float* scale, int M, int K, int wformat, int dtype,
+                               llmq_stream_t stream);
+int llmq_wq_gemm_a8_tiled(const void* codes_tiled, const float* sx, const void* qweight, const float* wscale,
+                          const float* bias_or_null, void* out, int M, int N, int G, int gs, int out_group,
+                          int wformat, int dtype, llmq_stream_t stream);
+int llmq_wq_gemm_a8_takes_groups(int M, int N, int G);
+
 /* The same GEMM in its fast form: the same exact integer group sums, folded into the total as
  * fma((float)isum * sw, sx, total) (one instruction and one rounding fewer than RealQuantLinear's
  * ((float)isum * sw) * sx followed by an add, llmquant/quantizers/real.py:94-99). Where the output has too few

@@ -322,9 +322,10 @@ int gemm_a8_relaxed(const int8_t* a, const float* sx, const void* qweight, const
                     int wformat, int dtype, hipStream_t stream);
 // The exact integer GEMM with a tile's groups computed eight at a time and added in order (wq_gemm_a8_groups.hip).
 bool gemm_a8_groups_supported(int M, int N, int G);
+// (tiled_a: the activation codes are in operand order, as llmq_quant_act_codes_tiled writes them)
 int gemm_a8_groups(const int8_t* a, const float* sx, const void* qweight, const float* wscale,
                    const float* bias_or_null, void* out, int M, int N, int G, int out_group, int wformat, int dtype,
-                   hipStream_t stream);
+                   hipStream_t stream, bool tiled_a = false);
 // Matrix-core GEMV (wq_gemv_mfma.hip): whether it can take a problem, and its launch.
 bool gemv_mfma_supported(const void* x, const void* qw, const float* ws, int M, int G, int gs,
                          int wformat);

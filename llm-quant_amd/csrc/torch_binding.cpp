@@ -563,6 +563,70 @@ at::Tensor wq_gemm_a8(const at::Tensor& a, const at::Tensor& sx, const at::Tenso
   return out;
 }
 
+// x [M, K] bf16 / fp16 -> (int8 codes in the operand order of the exact integer GEMM's group-parallel kernel, for
+// weights of `weight_bits` bits; scales [M, K / 128]): quant_group_codes(x, 8, 128) with the codes laid out for
+// wq_gemm_a8_tiled.
+std::tuple<at::Tensor, at::Tensor> quant_act_codes_tiled(const at::Tensor& x, int64_t weight_bits) {
+  TORCH_CHECK(x.is_cuda() && x.dim() == 2, "x must be a CUDA tensor [M, K]");
+  TORCH_CHECK(x.scalar_type() == at::kBFloat16 || x.scalar_type() == at::kHalf, "x must be bfloat16 or float16");
+  TORCH_CHECK(weight_bits == 4 || weight_bits == 8, "weight_bits must be 4 or 8, got ", weight_bits);
+  const auto xc = x.contiguous();
+  const int64_t M = xc.size(0), K = xc.size(1);
+  TORCH_CHECK(K % 128 == 0, "last dim ", K, " is not a multiple of 128");
+  const c10::OptionalDeviceGuard guard(at::device_of(xc));
+  auto codes = at::empty({static_cast<int64_t>(llmq_act_codes_tiled_bytes(static_cast<int>(M), static_cast<int>(K)))},
+                         xc.options().dtype(at::kChar));
+  auto scale = at::empty({M, K / 128}, xc.options().dtype(at::kFloat));
+  if (xc.numel() == 0) return std::make_tuple(codes, scale);
+  check_rc(llmq_quant_act_codes_tiled(xc.const_data_ptr(), codes.mutable_data_ptr(), scale.mutable_data_ptr<float>(),
+                                      static_cast<int>(M), static_cast<int>(K),
+                                      weight_bits == 4 ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype_code(xc, "x"),
+                                      current_stream(xc)),
+           "quant_act_codes_tiled");
+  return std::make_tuple(codes, scale);
+}
+
+// wq_gemm_a8 (exact form) on the codes of quant_act_codes_tiled for `rows` activation rows.
+at::Tensor wq_gemm_a8_tiled(const at::Tensor& codes, const at::Tensor& sx, int64_t rows, const at::Tensor& qweight,
+                            const at::Tensor& wscale, const c10::optional<at::Tensor>& bias, int64_t out_group,
+                            at::ScalarType out_dtype) {
+  TORCH_CHECK(codes.is_cuda() && sx.is_cuda() && qweight.is_cuda() && wscale.is_cuda(), "all tensors must be CUDA");
+  TORCH_CHECK(codes.scalar_type() == at::kChar && codes.dim() == 1 && codes.is_contiguous(),
+              "codes must be the tensor quant_act_codes_tiled returned");
+  TORCH_CHECK(qweight.dim() == 3, "qweight must be [N, groups, group_size], got ", qweight.dim(), "D");
+  const bool packed = qweight.scalar_type() == at::kByte;
+  TORCH_CHECK(packed || qweight.scalar_type() == at::kChar, "qweight must be int8, or uint8 for nibble-packed int4");
+  TORCH_CHECK(wscale.scalar_type() == at::kFloat && wscale.dim() == 2, "wscale must be float32 [scale_rows, groups]");
+  const auto sxc = sx.contiguous();
+  const auto wc = qweight.contiguous();
+  const auto sc = wscale.contiguous();
+  const int64_t M = rows, N = wc.size(0), groups = wc.size(1);
+  const int64_t group_size = packed ? wc.size(2) * 2 : wc.size(2);
+  TORCH_CHECK(group_size == 128, "the integer GEMM needs group_size 128, got ", group_size);
+  TORCH_CHECK(sxc.scalar_type() == at::kFloat && sxc.dim() == 2 && sxc.size(0) == M && sxc.size(1) == groups,
+              "sx must be float32 [", M, ", ", groups, "]");
+  TORCH_CHECK(static_cast<size_t>(codes.numel()) >= llmq_act_codes_tiled_bytes(static_cast<int>(M), static_cast<int>(groups * 128)),
+              "codes hold ", codes.numel(), " bytes: not the codes of ", M, " rows of ", groups * 128);
+  const int64_t scale_rows = out_group > 0 ? (N + out_group - 1) / out_group : N;
+  TORCH_CHECK(sc.size(0) == scale_rows && sc.size(1) == groups, "wscale must be [", scale_rows, ", ", groups, "]");
+  at::Tensor bias_f;
+  if (bias.has_value() && bias->defined()) {
+    TORCH_CHECK(bias->numel() == N, "bias must have ", N, " elements");
+    bias_f = bias->to(at::kFloat).contiguous();
+  }
+  auto out = at::empty({M, N}, codes.options().dtype(out_dtype));
+  const int dtype = dtype_code(out, "output dtype");
+  if (M == 0 || N == 0) return out;
+  const c10::OptionalDeviceGuard guard(at::device_of(codes));
+  check_rc(llmq_wq_gemm_a8_tiled(codes.const_data_ptr(), sxc.const_data_ptr<float>(), wc.const_data_ptr(),
+                                 sc.const_data_ptr<float>(), bias_f.defined() ? bias_f.const_data_ptr<float>() : nullptr,
+                                 out.mutable_data_ptr(), static_cast<int>(M), static_cast<int>(N), static_cast<int>(groups),
+                                 static_cast<int>(group_size), static_cast<int>(out_group),
+                                 packed ? LLMQ_W_INT4_PACKED : LLMQ_W_INT8, dtype, current_stream(codes)),
+           "wq_gemm_a8_tiled");
+  return out;
+}
+
 // Weight-only GEMM for a few dozen rows: x fp16/bf16 [M, K]; qweight / wscale as for wq_gemv.
 at::Tensor wq_gemm_a16(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& wscale, int64_t out_group,
                        bool split) {
@@ -1346,6 +1410,17 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "Integer GEMM: int8 activations x int4/int8 group-quantized weights, real-mode rounding order",
         py::arg("a"), py::arg("sx"), py::arg("qweight"), py::arg("wscale"), py::arg("bias") = py::none(),
         py::arg("out_group") = 0, py::arg("out_dtype") = at::kBFloat16, py::arg("exact") = true);
+  m.def("quant_act_codes_tiled", &quant_act_codes_tiled,
+        "int8 activation codes (groups of 128) in the operand order of wq_gemm_a8_tiled, and their scales",
+        py::arg("x"), py::arg("weight_bits"));
+  m.def("wq_gemm_a8_tiled", &wq_gemm_a8_tiled,
+        "the exact integer GEMM on the codes of quant_act_codes_tiled (group-parallel kernel, no operand staging pass)",
+        py::arg("codes"), py::arg("sx"), py::arg("rows"), py::arg("qweight"), py::arg("wscale"),
+        py::arg("bias") = py::none(), py::arg("out_group") = 0, py::arg("out_dtype") = at::kBFloat16);
+  m.def("wq_gemm_a8_takes_groups", [](int64_t m_rows, int64_t n, int64_t groups) {
+          return llmq_wq_gemm_a8_takes_groups(static_cast<int>(m_rows), static_cast<int>(n), static_cast<int>(groups)) != 0;
+        }, "whether wq_gemm_a8 (exact) runs its group-parallel kernel for the shape: then wq_gemm_a8_tiled is the faster call",
+        py::arg("rows"), py::arg("out_features"), py::arg("groups"));
   m.def("wq_gemm_a16", &wq_gemm_a16,
         "Weight-only GEMM for a few dozen rows: fp16/bf16 activations x int4/int8 group-quantized weights, no dense copy",
         py::arg("x"), py::arg("qweight"), py::arg("wscale"), py::arg("out_group") = 0, py::arg("split") = false);

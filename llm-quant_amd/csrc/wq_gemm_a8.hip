@@ -46,6 +46,7 @@ constexpr int kRowStride = kGroup + 16;  // bytes; padding keeps 16-byte reads o
 // the group-parallel kernel (exact form) takes outputs of up to this many 32 x 32 tiles per round of 256 of the
 // tiled kernel's 64 x 64 tiles
 constexpr int kGroupsTilesPerRound = 640;
+constexpr int kGroupsTilesOperandOrder = 1100;   // (512 x 4096 x 14336, 2048 tiles: 101 us against 82 tiled)
 
 struct GemmArgs {
   const int8_t* a;     // [M, G*128]
@@ -328,24 +329,32 @@ int forced_form() {
   return v[0] == 't' ? 1 : (v[0] == 'g' ? 2 : 0);
 }
 
+// The exact form: a tile's groups are a chain of dependent steps, and with few tiles the chip waits on few
+// chains. The group-parallel kernel computes eight groups of a 32 x 32 tile at once and only orders the
+// additions (same bits).
+// Which is faster, measured on 32-group and 112-group rows at M = 128 ... 2048 (int4): the tiled kernel takes
+// ~0.57 us per group and round of 256 of its 64 x 64 tiles, this one ~0.7 ns per group and 32 x 32 tile (it pays
+// for staging and unpacking per wave): it wins where the output is a few hundred 32 x 32 tiles and the rows are
+// long -- 128 x 4096 x 14336: 38 us against 61; 128 x 14336 x 4096: 38 against 27, which stays tiled.
+// operand_order: the activation codes come in the group-parallel kernel's operand order (llmq_wq_gemm_a8_tiled):
+// ~0.5 ns per group and tile then, 128 x 4096 x 14336 in 30 us, and on long rows it stays ahead up to about a
+// thousand tiles (256 x 4096 x 14336: 55 us against 64).
+bool takes_groups(int M, int N, int G, bool operand_order = false) {
+  const int form = forced_form();
+  const int64_t big_tiles = static_cast<int64_t>((N + 127) / 128) * ((M + 127) / 128);
+  const int64_t tiles32 = static_cast<int64_t>((N + 31) / 32) * ((M + 31) / 32);
+  const int64_t tiles64 = static_cast<int64_t>((N + 63) / 64) * ((M + 63) / 64);
+  bool pays = big_tiles < 256 && G >= 16 && tiles32 <= kGroupsTilesPerRound * ((tiles64 + 255) / 256);
+  if (operand_order && G >= 64 && tiles32 <= kGroupsTilesOperandOrder) pays = true;
+  return (form == 2 || (form == 0 && pays)) && llmq_host::gemm_a8_groups_supported(M, N, G);
+}
+
 template <typename T, int MODE>
 int launch_typed(const GemmArgs& g, int wformat, hipStream_t stream) {
   // 128 x 128 tiles when there is at least one for every CU, else 64 x 64
   const int64_t big_tiles = static_cast<int64_t>((g.N + 127) / 128) * ((g.M + 127) / 128);
   if constexpr (MODE == 0) {
-    // The exact form: a tile's groups are a chain of dependent steps, and with few tiles the chip waits on few
-    // chains. The group-parallel kernel computes eight groups of a 32 x 64 tile at once and only orders the
-    // additions (same bits).
-    // Which is faster, measured on 32-group and 112-group rows at M = 128 ... 2048 (int4): the tiled kernel takes
-    // ~0.57 us per group and round of 256 of its 64 x 64 tiles, this one ~0.7 ns per group and 32 x 32 tile (it pays
-    // for staging and unpacking per wave): it wins where the output is a few hundred 32 x 32 tiles and the rows are
-    // long -- 128 x 4096 x 14336: 41 us against 65; 128 x 14336 x 4096: 49 against 30, which stays tiled.
-    const int form = forced_form();
-    const int64_t tiles32 = static_cast<int64_t>((g.N + 31) / 32) * ((g.M + 31) / 32);
-    const int64_t tiles64 = static_cast<int64_t>((g.N + 63) / 64) * ((g.M + 63) / 64);
-    const bool pays = big_tiles < 256 && g.G >= 16 && tiles32 <= kGroupsTilesPerRound * ((tiles64 + 255) / 256);
-    const bool groups = form == 2 || (form == 0 && pays);
-    if (groups && llmq_host::gemm_a8_groups_supported(g.M, g.N, g.G)) {
+    if (takes_groups(g.M, g.N, g.G)) {
       const int dtype = sizeof(T) == 4 ? LLMQ_F32 : (std::is_same<T, f16_t>::value ? LLMQ_F16 : LLMQ_BF16);
       return llmq_host::gemm_a8_groups(g.a, g.sx, g.qw, g.sw, g.bias, g.out, g.M, g.N, g.G, g.out_group, wformat, dtype,
                                        stream);
@@ -382,6 +391,10 @@ extern "C" int llmq_wq_gemm_a8(const int8_t* a, const float* sx, const void* qwe
     return llmq_host::fail_invalid("activation and weight pointers must be 16-byte aligned");
   GemmArgs g{a, sx, static_cast<const uint8_t*>(qweight), wscale, bias_or_null, out, M, N, G, out_group};
   return launch_mode<0>(g, wformat, dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmq_wq_gemm_a8_takes_groups(int M, int N, int G) {
+  return M > 0 && N > 0 && G > 0 && takes_groups(M, N, G, true) ? 1 : 0;
 }
 
 // The tolerance forms of the same kernel (arguments already checked by llmq_wq_gemm_a8_fast).

@@ -25,6 +25,13 @@
 // (w & 0xf0f0f0f0) ^ 0x80808080 = the odd codes as signed bytes 16 * code (the 16 leaves through the weight
 // scale, a power of two: no rounding changes); the activation bytes are brought into the same even / odd order
 // with one byte permute per word.
+//
+// Activation codes in operand order (TILED_A). Turning the activation rows into operand layout through LDS is two
+// fifths of a round's LDS traffic and, for packed weights, sixteen byte permutes per wave. The quantizer that makes
+// the codes can write them where the matrix core wants them instead (act_quant_tiled_kernel): blocks of 32 rows x
+// one group (4 KB) in the order [m-tile][group], inside a block [k-step 0..3][lane 0..63][16 bytes], lane = row %
+// 32 + 32 * k-half, and for packed weights every eight bytes as even k, then odd k. A wave then loads its operand
+// with four contiguous 1 KB instructions and multiplies it as it comes.
 #include "llmq_device.h"
 
 namespace {
@@ -41,8 +48,10 @@ constexpr int kThreads = kWays * kWave;
 constexpr int kTM = 32, kTN = 32;           // output tile of a workgroup (and of every wave)
 constexpr int kSlotFloats = kTM * kTN;      // one wave's terms of one group
 
+constexpr int kBlockBytes = kTM * kGroup;   // activation codes of 32 rows x one group
+
 struct GroupArgs {
-  const int8_t* a;     // [M, G*128]
+  const int8_t* a;     // [M, G*128], or (TILED_A) [ceil(M / 32)][G][4096] in operand order
   const float* sx;     // [M, G]
   const uint8_t* qw;   // [N, G, 128] int8 or [N, G, 64] packed
   const float* sw;     // [scale_rows, G]
@@ -65,7 +74,7 @@ constexpr int kChunkGroups = 16;   // groups whose scales sit in LDS at a time (
 
 
 
-template <typename T, int BITS>
+template <typename T, int BITS, bool TILED_A>
 __device__ __forceinline__ void groups_body(const GroupArgs& g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float* slots = reinterpret_cast<float*>(smem);                       // [2][kWays][kSlotFloats]: rounds alternate
@@ -94,9 +103,13 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
     const int row = BITS == 8 ? p >> 3 : p >> 2, piece = BITS == 8 ? p & 7 : p & 3;
     b_off[i] = static_cast<uint32_t>(min(n0 + row, g.N - 1)) * w_row_bytes + piece * 16;
   }
+  const uint32_t a_block0 = static_cast<uint32_t>(blockIdx.y) * g.G * kBlockBytes + lane * 16;   // (TILED_A)
   auto load = [&](Operands<BITS>& o, int grp) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o.ra[i] = load16(g.a + (a_off[i] + static_cast<uint32_t>(grp) * kGroup));
+    for (int i = 0; i < 4; ++i) {
+      if constexpr (TILED_A) o.ra[i] = load16(g.a + (a_block0 + static_cast<uint32_t>(grp) * kBlockBytes + i * 1024));
+      else o.ra[i] = load16(g.a + (a_off[i] + static_cast<uint32_t>(grp) * kGroup));
+    }
 #pragma unroll
     for (int i = 0; i < kBPackets; ++i) o.rb[i] = load16(g.qw + (b_off[i] + static_cast<uint32_t>(grp) * kGroupBytesB));
   };
@@ -134,10 +147,15 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
     auto piece_at = [](int line, int piece) { return line * 128 + ((piece ^ (line & 7)) << 4); };
     // packet 64 i + lane is piece lane % 8 of line 8 i + lane / 8: one address, the rest are constant offsets
     unsigned char* put = stage + piece_at(lane >> 3, lane & 7);
+    v4i fa[4];
+    if constexpr (TILED_A) {
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+        fa[ks] = v4i{static_cast<int>(o.ra[ks].x), static_cast<int>(o.ra[ks].y), static_cast<int>(o.ra[ks].z), static_cast<int>(o.ra[ks].w)};
+    } else {
 #pragma unroll
     for (int i = 0; i < 4; ++i) store16(put + i * 1024, o.ra[i]);
     __builtin_amdgcn_wave_barrier();
-    v4i fa[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       const u32x4 d = load16(stage + piece_at(col, 4 * half + ks));
@@ -152,6 +170,7 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
       }
     }
     __builtin_amdgcn_wave_barrier();
+    }
 #pragma unroll
     for (int i = 0; i < kBPackets; ++i) store16(put + i * 1024, o.rb[i]);   // int4: 64-byte rows, two to a line
     __builtin_amdgcn_wave_barrier();
@@ -283,20 +302,63 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
 // Packed int4 weights: held to 128 registers (eight spilled, all outside the steady loop's multiply), so that two
 // workgroups (sixteen waves) share a CU and one's additions run under the other's multiplies: 128 x 4096 x 14336
 // in 41 us against 47 us with one workgroup a CU. int8 weights would spill 31: that form runs one workgroup a CU.
-template <typename T>
+template <typename T, bool TILED_A>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void wq_gemm_a8_groups_kernel4(const GroupArgs g) {
-  groups_body<T, 4>(g);
+  groups_body<T, 4, TILED_A>(g);
 }
-template <typename T>
+template <typename T, bool TILED_A>
 __global__ __launch_bounds__(kThreads) void wq_gemm_a8_groups_kernel8(const GroupArgs g) {
-  groups_body<T, 8>(g);
+  groups_body<T, 8, TILED_A>(g);
+}
+
+// The activation quantizer of llmq_quant_group_codes (int8 codes, group 128: csrc/fake_quant.hip, quant_lanes_kernel:
+// the same abs-max butterfly, IEEE division and round-half-even per group of 16 lanes) writing its codes in operand
+// order. A lane holds eight consecutive values of a (row, group); EVEN_ODD: for packed int4 weights.
+template <typename T, bool EVEN_ODD>
+__global__ __launch_bounds__(256) void act_quant_tiled_kernel(const T* __restrict__ x, int8_t* __restrict__ codes,
+                                                              float* __restrict__ scale_out, const int64_t total,
+                                                              const uint32_t K) {
+  const int64_t e0 = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 8;
+  const bool active = e0 < total;   // total is a multiple of 128: the 16 lanes of a group are active or idle as one
+  float f[8];
+  if (active) {
+    Pack<T>::unpack(load16(x + e0), f);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = 0.0f;
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(f[i]));
+  amax = group_max<16>(amax);
+  const float scale = scale_from_amax(amax, 127.0f);
+  if (!active) return;
+  const uint32_t G = K / kGroup;
+  const uint32_t row = static_cast<uint32_t>(e0 / K), in_row = static_cast<uint32_t>(e0 - static_cast<int64_t>(row) * K);
+  const uint32_t grp = in_row / kGroup, j = (in_row % kGroup) / 8;   // j: which eight of the group's 128
+  if (j == 0) scale_out[static_cast<int64_t>(row) * G + grp] = scale;
+  uint32_t c[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) c[i] = static_cast<uint32_t>(static_cast<int>(quant_code(f[i], scale, -128.0f, 127.0f))) & 0xffu;
+  u32x2 w;
+  if constexpr (EVEN_ODD) {
+    w.x = c[0] | c[2] << 8 | c[4] << 16 | c[6] << 24;
+    w.y = c[1] | c[3] << 8 | c[5] << 16 | c[7] << 24;
+  } else {
+    w.x = c[0] | c[1] << 8 | c[2] << 16 | c[3] << 24;
+    w.y = c[4] | c[5] << 8 | c[6] << 16 | c[7] << 24;
+  }
+  // k = 8 j .. 8 j + 7: k-half j / 8, k-step (j % 8) / 2, first or second eight bytes of the lane's sixteen
+  const int64_t block = (static_cast<int64_t>(row / kTM) * G + grp) * kBlockBytes;
+  const uint32_t at = ((j & 7) >> 1) * 1024 + ((row % kTM) + 32 * (j >> 3)) * 16 + (j & 1) * 8;
+  *reinterpret_cast<u32x2*>(codes + block + at) = w;
 }
 
 constexpr size_t kLdsBytes = 2 * (static_cast<size_t>(kWays) * kSlotFloats + kChunkGroups * (kTM + kTN)) * sizeof(float);
 
-template <typename T, int BITS>
+template <typename T, int BITS, bool TILED_A>
 int launch(const GroupArgs& g, hipStream_t stream) {
-  auto kernel = BITS == 4 ? wq_gemm_a8_groups_kernel4<T> : wq_gemm_a8_groups_kernel8<T>;
+  auto kernel = BITS == 4 ? wq_gemm_a8_groups_kernel4<T, TILED_A> : wq_gemm_a8_groups_kernel8<T, TILED_A>;
   static bool raised = false;  // per instantiation; worst case two threads both set it
   if (!raised) {
     const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -324,9 +386,11 @@ bool gemm_a8_groups_supported(int M, int N, int G) {
 
 int gemm_a8_groups(const int8_t* a, const float* sx, const void* qweight, const float* wscale,
                    const float* bias_or_null, void* out, int M, int N, int G, int out_group, int wformat, int dtype,
-                   hipStream_t stream) {
+                   hipStream_t stream, bool tiled_a) {
   GroupArgs g{a, sx, static_cast<const uint8_t*>(qweight), wscale, bias_or_null, out, M, N, G, out_group};
-#define LLMQ_GO(T) (wformat == LLMQ_W_INT8 ? launch<T, 8>(g, stream) : launch<T, 4>(g, stream))
+#define LLMQ_GO(T)                                                                                       \
+  (tiled_a ? (wformat == LLMQ_W_INT8 ? launch<T, 8, true>(g, stream) : launch<T, 4, true>(g, stream))   \
+           : (wformat == LLMQ_W_INT8 ? launch<T, 8, false>(g, stream) : launch<T, 4, false>(g, stream)))
   switch (dtype) {
     case LLMQ_F32: return LLMQ_GO(float);
     case LLMQ_F16: return LLMQ_GO(f16_t);
@@ -337,3 +401,55 @@ int gemm_a8_groups(const int8_t* a, const float* sx, const void* qweight, const 
 }
 
 }  // namespace llmq_host
+
+extern "C" size_t llmq_act_codes_tiled_bytes(int M, int K) {
+  if (M <= 0 || K <= 0) return 0;
+  return static_cast<size_t>((M + kTM - 1) / kTM) * kTM * static_cast<size_t>(K);
+}
+
+extern "C" int llmq_quant_act_codes_tiled(const void* x, void* codes, float* scale, int M, int K, int wformat,
+                                          int dtype, llmq_stream_t stream) {
+  if (M < 0 || K <= 0 || K % kGroup) return llmq_host::fail_invalid("bad shape M=%d K=%d (K a multiple of %d)", M, K, kGroup);
+  if (wformat != LLMQ_W_INT8 && wformat != LLMQ_W_INT4_PACKED)
+    return llmq_host::fail_invalid("unsupported weight format %d, expected 8 or 4", wformat);
+  if (dtype != LLMQ_BF16 && dtype != LLMQ_F16)
+    return llmq_host::fail_invalid("x must be bfloat16 or float16, got dtype code %d", dtype);
+  if (M == 0) return 0;
+  if (!x || !codes || !scale) return llmq_host::fail_invalid("null tensor pointer");
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(codes)) & 15u)
+    return llmq_host::fail_invalid("x and codes must be 16-byte aligned");
+  if (!llmq_host::gemm_a8_groups_supported(M + kTM, 1, K / kGroup))
+    return llmq_host::fail_invalid("activation of %d x %d codes is beyond the kernel's 32-bit offsets", M, K);
+  const int64_t total = static_cast<int64_t>(M) * K;
+  const dim3 grid(static_cast<unsigned>((total / 8 + 255) / 256)), block(256);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool even_odd = wformat == LLMQ_W_INT4_PACKED;
+#define LLMQ_GO(T)                                                                                               \
+  if (even_odd) hipLaunchKernelGGL((act_quant_tiled_kernel<T, true>), grid, block, 0, s, static_cast<const T*>(x), \
+                                   static_cast<int8_t*>(codes), scale, total, static_cast<uint32_t>(K));          \
+  else hipLaunchKernelGGL((act_quant_tiled_kernel<T, false>), grid, block, 0, s, static_cast<const T*>(x),         \
+                          static_cast<int8_t*>(codes), scale, total, static_cast<uint32_t>(K))
+  if (dtype == LLMQ_BF16) { LLMQ_GO(bf16_t); } else { LLMQ_GO(f16_t); }
+#undef LLMQ_GO
+  return llmq_host::check_launch("act_quant_tiled_kernel");
+}
+
+extern "C" int llmq_wq_gemm_a8_tiled(const void* codes_tiled, const float* sx, const void* qweight, const float* wscale,
+                                     const float* bias_or_null, void* out, int M, int N, int G, int gs, int out_group,
+                                     int wformat, int dtype, llmq_stream_t stream) {
+  if (M < 0 || N < 0 || G < 0) return llmq_host::fail_invalid("negative dimension M=%d N=%d G=%d", M, N, G);
+  if (gs != kGroup) return llmq_host::fail_invalid("the integer GEMM needs group_size 128, got %d", gs);
+  if (wformat != LLMQ_W_INT8 && wformat != LLMQ_W_INT4_PACKED)
+    return llmq_host::fail_invalid("unsupported weight format %d, expected 8 or 4", wformat);
+  if (out_group < 0) return llmq_host::fail_invalid("out_group must be >= 0, got %d", out_group);
+  if (M == 0 || N == 0) return 0;
+  if (G == 0) return llmq_host::fail_invalid("a weight with no groups has no reduction axis");
+  if (!codes_tiled || !sx || !qweight || !wscale || !out) return llmq_host::fail_invalid("null tensor pointer");
+  if ((reinterpret_cast<uintptr_t>(codes_tiled) | reinterpret_cast<uintptr_t>(qweight)) & 15u)
+    return llmq_host::fail_invalid("codes and qweight must be 16-byte aligned");
+  if (!llmq_host::gemm_a8_groups_supported(M + kTM, N, G))
+    return llmq_host::fail_invalid("operands of %d x %d and %d x %d codes are beyond the kernel's 32-bit offsets", M,
+                                   G * kGroup, N, G * kGroup);
+  return llmq_host::gemm_a8_groups(static_cast<const int8_t*>(codes_tiled), sx, qweight, wscale, bias_or_null, out, M, N,
+                                   G, out_group, wformat, dtype, static_cast<hipStream_t>(stream), true);
+}

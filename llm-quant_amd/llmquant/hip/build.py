@@ -125,6 +125,14 @@ def load_capi() -> ctypes.CDLL:
     lib.llmq_wq_gemm_a8_fast.restype = c_int
     lib.llmq_wq_gemm_a8_fast_workspace_bytes.argtypes = [c_int] * 3
     lib.llmq_wq_gemm_a8_fast_workspace_bytes.restype = ctypes.c_size_t
+    lib.llmq_act_codes_tiled_bytes.argtypes = [c_int] * 2
+    lib.llmq_act_codes_tiled_bytes.restype = ctypes.c_size_t
+    lib.llmq_quant_act_codes_tiled.argtypes = [c_p] * 3 + [c_int] * 4 + [c_p]
+    lib.llmq_quant_act_codes_tiled.restype = c_int
+    lib.llmq_wq_gemm_a8_tiled.argtypes = [c_p] * 6 + [c_int] * 7 + [c_p]
+    lib.llmq_wq_gemm_a8_tiled.restype = c_int
+    lib.llmq_wq_gemm_a8_takes_groups.argtypes = [c_int] * 3
+    lib.llmq_wq_gemm_a8_takes_groups.restype = c_int
     lib.llmq_wq_gemm_a16.argtypes = [c_p] * 4 + [c_int] * 7 + [c_p]
     lib.llmq_wq_gemm_a16.restype = c_int
     lib.llmq_wq_gemm_a16_split.argtypes = [c_p] * 5 + [ctypes.c_size_t] + [c_int] * 7 + [c_p]

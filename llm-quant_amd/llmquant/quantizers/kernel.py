@@ -272,6 +272,15 @@ class KernelQuantLinear(nn.Module):
         if self._needs_padding:
             rows = pad_activation(rows, self._weight_args)
         if self._int8_act:
+            if (self.a8_exact and rows.dtype in (torch.bfloat16, torch.float16) and x.dtype == rows.dtype
+                    and self._ext.wq_gemm_a8_takes_groups(rows.shape[0], self.out_features, self.qdata.shape[1])):
+                # few output tiles, long rows: the group-parallel kernel, with the codes written in its operand order
+                # by the quantizer (the same codes and scales, the same result bit for bit)
+                codes, act_scale = self._ext.quant_act_codes_tiled(rows.contiguous(),
+                                                                   4 if self.qdata.dtype == torch.uint8 else 8)
+                out = self._ext.wq_gemm_a8_tiled(codes, act_scale, rows.shape[0], self.qdata, self.wscale, self.bias,
+                                                 self.out_group, x.dtype)
+                return out.reshape(*x.shape[:-1], self.out_features)
             codes, act_scale = self._ext.quant_group_codes(rows, 8, 128, False)
             out = self._ext.wq_gemm_a8(codes, act_scale, self.qdata, self.wscale, self.bias, self.out_group,
                                        x.dtype, self.a8_exact)

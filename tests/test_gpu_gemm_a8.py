@@ -86,6 +86,96 @@ def test_bias_and_head_scales(ext, bits, form):
     assert np.array_equal(to_np(got), want)
 
 
+def untile_codes(tiled, m, k, even_odd):
+    """The [m, k] codes out of llmq_quant_act_codes_tiled's layout: blocks of 32 rows x one group, inside a block
+    [k-step][row % 32 + 32 * k-half][16 bytes], with packed weights every eight bytes as even k then odd k."""
+    padded = -(-m // 32) * 32
+    t = tiled.reshape(padded // 32, k // GROUP, 4, 2, 32, 2, 8)      # m-tile, group, k-step, k-half, row, run, byte
+    if even_odd:
+        t = t[..., [0, 4, 1, 5, 2, 6, 3, 7]]
+    t = t.transpose(0, 4, 1, 3, 2, 5, 6)                             # m-tile, row, group, k-half, k-step, run, byte
+    return t.reshape(padded, k)[:m]
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,n,k", [(32, 256, 512), (1, 128, 128), (37, 200, 384), (130, 129, 256), (65, 70, 1152),
+                                   (33, 64, 2176), (128, 512, 4096)])
+def test_operand_order_codes_give_the_same_bits(ext, bits, dtype, m, n, k):
+    """llmq_quant_act_codes_tiled + llmq_wq_gemm_a8_tiled: the scales and (taken out of the layout again) the codes of
+    llmq_quant_group_codes, which are the oracle's; the product bit for bit the real-mode forward, with a bias and
+    one weight scale row per 64 rows as well; rows of the last block of 32 that do not exist are never written."""
+    torch.manual_seed(m + k)
+    w = (torch.randn(n, k) * 0.015).to(torch.bfloat16)
+    x = torch.randn(m, k).to(dtype)
+    b = torch.randn(n)
+    want_codes, want_sx = oracle.quant_group_codes(to_np(x), 8, GROUP)
+    tiled, sx = ext.quant_act_codes_tiled(x.cuda(), bits)
+    assert tiled.numel() == -(-m // 32) * 32 * k and np.array_equal(to_np(sx), want_sx)
+    assert np.array_equal(untile_codes(tiled.cpu().numpy(), m, k, bits == 4), want_codes)
+    for out_group, bias in ((0, None), (64, b)):
+        canonical, scales = oracle.canonical_weight(to_np(w), bits, GROUP, None, out_group or None)
+        q = torch.from_numpy(oracle.pack_int4(canonical) if bits == 4 else canonical).cuda()
+        s = torch.from_numpy(scales).cuda()
+        got = ext.wq_gemm_a8_tiled(tiled, sx, m, q, s, None if bias is None else bias.cuda(), out_group, dtype)
+        want = oracle.real_linear(to_np(x), canonical, scales, tag_of(dtype), out_group or None, 8,
+                                  None if bias is None else to_np(bias))
+        assert got.shape == (m, n) and got.dtype == dtype
+        assert np.array_equal(to_np(got), want)
+        natural, _ = ext.quant_group_codes(x.cuda(), 8, GROUP, False)
+        assert torch.equal(got, ext.wq_gemm_a8(natural, sx, q, s, None if bias is None else bias.cuda(), out_group, dtype))
+
+
+def test_operand_order_at_the_long_row_shape_and_through_the_module(ext):
+    """128 x 4096 x 14336 int4 (the shape the group-parallel kernel is for) on sampled entries against the oracle,
+    and KernelQuantLinear with int8 activations taking that pair of calls for it (the natural-order calls are made
+    to fail loudly), equal to RealQuantLinear's forward."""
+    got, (x, canonical, scales, _) = run_case(ext, 128, 4096, 14336, 4, torch.bfloat16, seed=3, outliers=True)
+    tiled, sx = ext.quant_act_codes_tiled(x.cuda(), 4)
+    q = torch.from_numpy(oracle.pack_int4(canonical)).cuda()
+    fast = ext.wq_gemm_a8_tiled(tiled, sx, 128, q, torch.from_numpy(scales).cuda(), None, 0, torch.bfloat16)
+    assert torch.equal(fast, got) and ext.wq_gemm_a8_takes_groups(128, 4096, 112)
+    assert not ext.wq_gemm_a8_takes_groups(2048, 4096, 112) and not ext.wq_gemm_a8_takes_groups(128, 14336, 32)
+    import torch.nn as nn
+
+    from llmquant.core.scheme import QuantizationArgs, QuantizationScheme
+    from llmquant.quantizers import KernelQuantLinear, RealQuantLinear
+
+    torch.manual_seed(5)
+    linear = nn.Linear(4096, 1024, bias=True).to(torch.bfloat16).cuda()
+    scheme = QuantizationScheme(weights=QuantizationArgs(num_bits=4, strategy="group", group_size=GROUP),
+                                input_activations=QuantizationArgs(num_bits=8, strategy="group", group_size=GROUP))
+    module, real = KernelQuantLinear.from_linear(linear, scheme), RealQuantLinear.from_linear(linear, scheme)
+    xs = torch.randn(3, 40, 4096, device="cuda").to(torch.bfloat16)
+    assert ext.wq_gemm_a8_takes_groups(120, 1024, 32)
+    want = real(xs)
+
+    class OnlyTiled:
+        def __getattr__(self, name):
+            if name in ("quant_group_codes", "wq_gemm_a8"):
+                raise AssertionError(f"{name} called: the operand-order pair should have run")
+            return getattr(ext, name)
+
+    module._ext = OnlyTiled()
+    assert torch.equal(module(xs), want)
+
+
+def test_operand_order_argument_checks(ext):
+    x = torch.randn(40, 256, device="cuda").to(torch.bfloat16)
+    with pytest.raises(RuntimeError, match="bfloat16 or float16"):
+        ext.quant_act_codes_tiled(x.float(), 4)
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        ext.quant_act_codes_tiled(x[:, :200].contiguous(), 4)
+    tiled, sx = ext.quant_act_codes_tiled(x, 4)
+    q = torch.randint(0, 256, (64, 2, 64), dtype=torch.uint8, device="cuda")
+    s = torch.ones(64, 2, device="cuda")
+    with pytest.raises(RuntimeError, match="not the codes of"):
+        ext.wq_gemm_a8_tiled(tiled[:1024], sx, 40, q, s)
+    with pytest.raises(RuntimeError, match="sx must be"):
+        ext.wq_gemm_a8_tiled(tiled, sx[:, :1].contiguous(), 40, q, s)
+    assert ext.wq_gemm_a8_tiled(tiled, sx, 40, q, s).shape == (40, 64)
+
+
 def test_matches_the_float64_closed_form(ext):
     """Independent of the accumulation order: y = sum_g sx sw sum_k a q, in float64."""
     got, (x, canonical, scales, _) = run_case(ext, 64, 256, 1024, 4, torch.float32, seed=2)
