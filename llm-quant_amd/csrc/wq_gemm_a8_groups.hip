@@ -140,7 +140,8 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
   // (row or column `col`, k-half `half`) reads its pieces. LDS serves a wave's accesses in order; the wave
   // barriers keep the compiler from moving them.
   // Result register r of the 32 x 32 product is row 8 (r / 4) + 4 half + r % 4, column col; the slot keeps the
-  // terms as [r / 4][lane][r % 4].
+  // terms as [r / 2][lane][r % 2]: the pair of registers that one wave adds lies contiguous over the lanes, so
+  // that both the stores here and the adders' 8-byte reads spread over all banks.
   auto produce = [&](const Operands<BITS>& o, int grp, float* round_slots) {
     unsigned char* stage = reinterpret_cast<unsigned char*>(round_slots + wv * kSlotFloats);
     // piece `piece` of 128-byte line `line`, XOR-swizzled
@@ -215,13 +216,16 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
         f = f * sw;
         p[i] = f * sx4[i];
       }
-      store16(slot + (r4 * kWave + lane) * 4, Pack<float>::pack(p));
+      *reinterpret_cast<u32x2*>(slot + ((2 * r4) * kWave + lane) * 2) =
+          u32x2{__builtin_bit_cast(uint32_t, p[0]), __builtin_bit_cast(uint32_t, p[1])};
+      *reinterpret_cast<u32x2*>(slot + ((2 * r4 + 1) * kWave + lane) * 2) =
+          u32x2{__builtin_bit_cast(uint32_t, p[2]), __builtin_bit_cast(uint32_t, p[3])};
     }
   };
 
   // this wave's eighth of the tile in the additions: result registers 4 (wv / 2) + 2 (wv % 2) + {0, 1} of every lane
   float total[2] = {0.0f, 0.0f};
-  const int my_pair = ((wv >> 1) * kWave + lane) * 4 + 2 * (wv & 1);
+  const int my_pair = (wv * kWave + lane) * 2;
   auto add_round = [&](const float* round_slots, int valid) {
     for (int s = 0; s < valid; ++s) {
       const u32x2 v = *reinterpret_cast<const u32x2*>(round_slots + s * kSlotFloats + my_pair);
