@@ -145,9 +145,12 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
   auto produce = [&](const Operands<BITS>& o, int grp, float* round_slots) {
     unsigned char* stage = reinterpret_cast<unsigned char*>(round_slots + wv * kSlotFloats);
     // piece `piece` of 128-byte line `line`, XOR-swizzled
-    auto piece_at = [](int line, int piece) { return line * 128 + ((piece ^ (line & 7)) << 4); };
-    // packet 64 i + lane is piece lane % 8 of line 8 i + lane / 8: one address, the rest are constant offsets
-    unsigned char* put = stage + piece_at(lane >> 3, lane & 7);
+    // (by line / 2: the sixteen lanes that LDS serves together read one piece of sixteen different lines, or of
+    // eight lines and two pieces four apart (packed weights), and a line's parity is already a bank bit)
+    auto piece_at = [](int line, int piece) { return line * 128 + ((piece ^ ((line >> 1) & 7)) << 4); };
+    // packet 64 i + lane is piece lane % 8 of line 8 i + lane / 8: one address; eight lines on, the swizzle's third
+    // bit has flipped
+    auto put_at = [&](int i) { return stage + ((piece_at(lane >> 3, lane & 7) ^ ((i & 1) << 6)) + i * 1024); };
     v4i fa[4];
     if constexpr (TILED_A) {
 #pragma unroll
@@ -155,7 +158,7 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
         fa[ks] = v4i{static_cast<int>(o.ra[ks].x), static_cast<int>(o.ra[ks].y), static_cast<int>(o.ra[ks].z), static_cast<int>(o.ra[ks].w)};
     } else {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) store16(put + i * 1024, o.ra[i]);
+    for (int i = 0; i < 4; ++i) store16(put_at(i), o.ra[i]);
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
@@ -173,7 +176,7 @@ __device__ __forceinline__ void groups_body(const GroupArgs& g) {
     __builtin_amdgcn_wave_barrier();
     }
 #pragma unroll
-    for (int i = 0; i < kBPackets; ++i) store16(put + i * 1024, o.rb[i]);   // int4: 64-byte rows, two to a line
+    for (int i = 0; i < kBPackets; ++i) store16(put_at(i), o.rb[i]);   // int4: 64-byte rows, two to a line
     __builtin_amdgcn_wave_barrier();
     v4i fb[4];
     if constexpr (BITS == 8) {
