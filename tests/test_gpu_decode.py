@@ -153,6 +153,18 @@ def test_teacher_forced_margin_with_heads_of_128(runtime):
     assert agree >= 0.8 * len(rows)
 
 
+@pytest.mark.parametrize("runtime", ["walk", "fused"])
+def test_teacher_forced_margin_on_a_float16_model(runtime):
+    """A float16 model end to end: the prompt pass through the tiled matrix-core kernels' float16 form (codes made
+    exact by a packed add, no Σx records used), the prepared RMSNorm, and the decode step's float16 kernels, against
+    the real-mode float16 model under the margin rule."""
+    real, kernel = quantized_pair(build_model(512, 2048, 2, 8, 2, 4096, seed=7, dtype=torch.float16))
+    rows, _, _ = teacher_forced(real, kernel, 300, 24, 4096, runtime=runtime)
+    agree = check_margin(rows, 0.05)
+    print(f"teacher-forced agreement, float16 model, {runtime}: {agree}/{len(rows)}")
+    assert agree >= 0.8 * len(rows)
+
+
 @pytest.mark.parametrize("head_dim,kv_bits", [(64, 8), (128, 8), (64, 4), (128, 4)])
 def test_teacher_forced_margin_on_a_long_cache(head_dim, kv_bits):
     """A cache of 2304 rows: the fused runtime's decode step takes the matrix-core form of the attention launch (the
