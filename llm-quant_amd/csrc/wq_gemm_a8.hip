@@ -58,6 +58,14 @@ struct GemmArgs {
   int M, N, G, out_group;
 };
 
+// a 32-bit offset the compiler must take as it is, inside the loop: the load then has the form scalar base +
+// vector offset, and the base moves from group to group with two scalar additions instead of one 64-bit vector
+// addition per load
+__device__ __forceinline__ uint32_t here(uint32_t& v) {
+  asm volatile("" : "+v"(v));  // (in place: a copy would cost a move per load)
+  return v;
+}
+
 // W: the wave's quadrant is (32 W) x (32 W), the workgroup's tile (64 W) x (64 W). W = 2 is the
 // throughput shape; W = 1 gives four times as many workgroups when the problem is too small to
 // fill the chip with 128 x 128 tiles.
@@ -66,25 +74,60 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
   constexpr int kBM = 64 * W, kBN = 64 * W;
   __shared__ __attribute__((aligned(16))) int8_t s_a[2][kBM * kRowStride];
   __shared__ __attribute__((aligned(16))) int8_t s_b[2][kBN * kRowStride];
-  __shared__ __attribute__((aligned(16))) float s_sx[2][kBM];
-  __shared__ __attribute__((aligned(16))) float s_sw[2][kBN];
+  __shared__ __attribute__((aligned(16))) float s_scale[2][kBM + kBN];  // activation scales, then weight scales
 
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wv >> 1, wn = wv & 1;  // quadrant of the tile
   const int m0 = blockIdx.y * kBM, n0 = blockIdx.x * kBN;
   const int64_t k_total = static_cast<int64_t>(g.G) * kGroup;
   const int64_t w_row_bytes = BITS == 8 ? k_total : k_total / 2;
+  constexpr int kWGroupBytes = BITS == 8 ? kGroup : kGroup / 2;
 
   // ---- staging: who loads what ------------------------------------------------------------------
   // A tile: kBM rows x 128 B = 8 kBM 16-byte packets. Thread t: packets t + 256*i:
   // row = p / 8, piece = p % 8.
   // B tile int8: same. B tile int4: kBN rows x 64 B = 4 kBN packets: row = p / 4.
+  // Addresses are the tile's first row (the same in every lane) plus an offset per thread that does not change
+  // from group to group (at most 128 rows: 32 bits hold it, the host checks the row length).
   constexpr int kAPackets = kBM * 8 / kThreads;
   constexpr int kBPackets = (BITS == 8 ? kBN * 8 : kBN * 4) / kThreads;
+  const int8_t* a_tile = g.a + static_cast<int64_t>(m0) * k_total;
+  const uint8_t* b_tile = g.qw + static_cast<int64_t>(n0) * w_row_bytes;
+  uint32_t a_off[kAPackets], b_off[kBPackets];
+#pragma unroll
+  for (int i = 0; i < kAPackets; ++i) {
+    const int p = tid + kThreads * i;
+    a_off[i] = static_cast<uint32_t>(min(p >> 3, g.M - 1 - m0)) * static_cast<uint32_t>(k_total) + (p & 7) * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < kBPackets; ++i) {
+    const int p = tid + kThreads * i;
+    const int row = min(BITS == 8 ? p >> 3 : p >> 2, g.N - 1 - n0);
+    b_off[i] = static_cast<uint32_t>(row) * static_cast<uint32_t>(w_row_bytes) + (BITS == 8 ? (p & 7) : (p & 3)) * 16;
+  }
+  // One scale per thread and group: the first kBM / 64 waves load activation scales, the others weight scales
+  // (waves past the tile's rows and columns, and the first ones in MODE 2, which has no activation scale per
+  // group, repeat a weight scale's address): a fixed number of loads per group lets the waits before the LDS
+  // stores count the loads that may stay in flight instead of draining them all.
+  const bool sx_wave = MODE != 2 && wv < kBM / 64;
+  const int sc_idx = wv < kBM / 64 ? tid : (tid - kBM) & (kBN - 1);
+  auto scale_row = [&](int n) { return g.out_group > 0 ? n / g.out_group : n; };
+  const char* sc_tile = sx_wave ? reinterpret_cast<const char*>(g.sx + static_cast<int64_t>(m0) * g.G)
+                                : reinterpret_cast<const char*>(g.sw + static_cast<int64_t>(scale_row(n0)) * g.G);
+  uint32_t sc_off =
+      static_cast<uint32_t>(sx_wave ? min(sc_idx, g.M - 1 - m0) : scale_row(min(n0 + sc_idx, g.N - 1)) - scale_row(n0)) *
+      static_cast<uint32_t>(g.G) * 4u;
+  const float scale_factor = BITS == 4 && wv >= kBM / 64 ? 0.0625f : 1.0f;  // see the unpack of packed weights
+  // LDS addresses of a thread's first packets; the others are whole rows further on
+  const int a_lds = (tid >> 3) * kRowStride + (tid & 7) * 16;
+  const int b_lds = BITS == 8 ? a_lds : (tid >> 2) * kRowStride + (tid & 3) * 32;
+  constexpr int kARowsPerPass = kThreads / 8, kBRowsPerPass = BITS == 8 ? kThreads / 8 : kThreads / 4;
+
   // what a thread holds of one group between its global loads and its LDS stores
   struct Staged {
     u32x4 ra[kAPackets], rb[kBPackets];
-    float r_sx, r_sw;
+    float r_s;
   };
   // The small tile has little work per group, so with one group in flight its loop runs at one
   // memory round trip per iteration: it keeps two register sets and requests a group three
@@ -92,78 +135,32 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
   // next group at the top of an iteration and moves it to LDS at the bottom.
   constexpr int kAhead = W == 1 ? 2 : 0;
   constexpr int kSets = kAhead > 0 ? kAhead : 1;
-  // A steady-state copy of the loop with no branch around its loads and stores (and the same number
-  // of loads in every thread) lets the compiler wait for exactly the loads an LDS store needs
-  // instead of draining everything in flight: measured, M = 2048: int8 weights 346 -> 240 us at
-  // 4096 x 14336, 382 -> 310 us at 14336 x 4096; the small tile 75 -> 64 us at M = 128. The large
-  // tile with int4 weights is the one variant it slows (its unpack leaves no registers for the
-  // second copy's live ranges: 18 spilled), so that one keeps the plain loop.
-  constexpr bool kBranchFreeLoop = !(W == 2 && BITS == 4);
   Staged st[kSets];
 
   auto load_group = [&](int grp, Staged& t) {
-    u32x4* ra = t.ra;
-    u32x4* rb = t.rb;
-    float& r_sx = t.r_sx;
-    float& r_sw = t.r_sw;
+    const int8_t* ag = a_tile + static_cast<uint32_t>(grp) * kGroup;
 #pragma unroll
-    for (int i = 0; i < kAPackets; ++i) {
-      const int p = tid + kThreads * i;
-      const int row = min(m0 + (p >> 3), g.M - 1);
-      ra[i] = load16(g.a + static_cast<int64_t>(row) * k_total + static_cast<int64_t>(grp) * kGroup + (p & 7) * 16);
-    }
+    for (int i = 0; i < kAPackets; ++i) t.ra[i] = load16(ag + here(a_off[i]));
+    const uint8_t* bg = b_tile + static_cast<uint32_t>(grp) * kWGroupBytes;
 #pragma unroll
-    for (int i = 0; i < kBPackets; ++i) {
-      const int p = tid + kThreads * i;
-      if constexpr (BITS == 8) {
-        const int row = min(n0 + (p >> 3), g.N - 1);
-        rb[i] = load16(g.qw + static_cast<int64_t>(row) * w_row_bytes + static_cast<int64_t>(grp) * kGroup + (p & 7) * 16);
-      } else {
-        const int row = min(n0 + (p >> 2), g.N - 1);
-        rb[i] = load16(g.qw + static_cast<int64_t>(row) * w_row_bytes + static_cast<int64_t>(grp) * (kGroup / 2) + (p & 3) * 16);
-      }
-    }
-    // every thread loads one scale, kept or not (threads past the tile's rows and columns repeat an
-    // address): a fixed number of loads per group lets the waits before the LDS stores count the
-    // loads that may stay in flight instead of draining them all
-    if constexpr (!kBranchFreeLoop) {
-      if (tid < kBM) {
-        if constexpr (MODE != 2) r_sx = g.sx[static_cast<int64_t>(min(m0 + tid, g.M - 1)) * g.G + grp];
-      } else if (tid < kBM + kBN) {
-        const int n = min(n0 + tid - kBM, g.N - 1);
-        r_sw = g.sw[static_cast<int64_t>(g.out_group > 0 ? n / g.out_group : n) * g.G + grp];
-      }
-    } else {
-      const int idx = tid < kBM ? tid : (tid - kBM) & (kBN - 1);
-      const int n = min(n0 + idx, g.N - 1);
-      // (MODE 2 has no activation scale per group: those threads repeat a weight scale's load)
-      const float* sp = (tid < kBM && MODE != 2) ? g.sx + static_cast<int64_t>(min(m0 + idx, g.M - 1)) * g.G
-                                                 : g.sw + static_cast<int64_t>(g.out_group > 0 ? n / g.out_group : n) * g.G;
-      const float v = sp[grp];
-      r_sx = v;
-      r_sw = v;
-    }
+    for (int i = 0; i < kBPackets; ++i) t.rb[i] = load16(bg + here(b_off[i]));
+    t.r_s = *reinterpret_cast<const float*>(sc_tile + static_cast<uint32_t>(grp) * 4 + here(sc_off));
   };
-  auto store_group = [&](int buf, const Staged& t) {
-    const u32x4* ra = t.ra;
-    const u32x4* rb = t.rb;
-    const float r_sx = t.r_sx, r_sw = t.r_sw;
+  auto store_group = [&](auto buffer, const Staged& t) {
+    constexpr int buf = decltype(buffer)::value;
 #pragma unroll
-    for (int i = 0; i < kAPackets; ++i) {
-      const int p = tid + kThreads * i;
-      store16(&s_a[buf][(p >> 3) * kRowStride + (p & 7) * 16], ra[i]);
-    }
+    for (int i = 0; i < kAPackets; ++i) store16(&s_a[buf][a_lds + i * kARowsPerPass * kRowStride], t.ra[i]);
 #pragma unroll
     for (int i = 0; i < kBPackets; ++i) {
-      const int p = tid + kThreads * i;
+      int8_t* dst = &s_b[buf][b_lds + i * kBRowsPerPass * kRowStride];
       if constexpr (BITS == 8) {
-        store16(&s_b[buf][(p >> 3) * kRowStride + (p & 7) * 16], rb[i]);
+        store16(dst, t.rb[i]);
       } else {
         // 16 packed bytes = 32 codes -> 32 signed bytes in natural k order, each 16 x its code:
         // a nibble n = code + 8 moved to the top of its byte and its top bit flipped reads, as a
         // signed byte, 16 (n - 8). The factor 16 leaves the integer sums exact (< 2^26) and is
         // taken back out of the weight scale, a power of two, so no rounding changes.
-        const uint32_t w[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
+        const uint32_t w[4] = {t.rb[i].x, t.rb[i].y, t.rb[i].z, t.rb[i].w};
         uint32_t o[8];
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
@@ -173,13 +170,11 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
           o[2 * d] = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
           o[2 * d + 1] = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
         }
-        int8_t* dst = &s_b[buf][(p >> 2) * kRowStride + (p & 3) * 32];
         store16(dst, u32x4{o[0], o[1], o[2], o[3]});
         store16(dst + 16, u32x4{o[4], o[5], o[6], o[7]});
       }
     }
-    if (tid < kBM) s_sx[buf][tid] = r_sx;
-    else if (tid < kBM + kBN) s_sw[buf][tid - kBM] = BITS == 4 ? r_sw * 0.0625f : r_sw;  // see the unpack above
+    if (kBM + kBN == kThreads || wv < (kBM + kBN) / 64) s_scale[buf][tid] = t.r_s * scale_factor;
   };
 
   float acc[W][W][16];
@@ -191,35 +186,33 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
       for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
 
   load_group(0, st[0]);
-  store_group(0, st[0]);
+  store_group(std::integral_constant<int, 0>{}, st[0]);
   __syncthreads();
 #pragma unroll
   for (int a = 0; a < kAhead; ++a) {
     if (1 + a < g.G) load_group(1 + a, st[a]);  // st[a] will hold groups 1 + a, 1 + a + kAhead, ...
   }
 
-  const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
-  // one group: multiply it from LDS buffer grp & 1, move group grp + 1 (in `next`) into the other
-  // buffer, and with kAhead > 0 request group grp + 1 + kAhead into the registers that frees
-  // `steady`: the caller guarantees that groups grp + 1 and grp + 1 + kAhead exist, so the body has
-  // no branch around its loads and stores
-  auto iterate = [&](int grp, Staged& next, auto steady) {
+  const int frag = (lane & 31) * kRowStride + (lane >> 5) * 16;  // a lane's row and k half within a 32-row block
+  // One group: multiply it from LDS buffer `buffer` (= grp & 1, a compile-time value so that every LDS address
+  // is a register plus a constant), move group grp + 1 (in `next`) into the other buffer, and with kAhead > 0
+  // request group grp + 1 + kAhead into the registers that frees. `steady`: the caller guarantees that groups
+  // grp + 1 and grp + 1 + kAhead exist, so the body has no branch around its loads and stores.
+  auto iterate = [&](int grp, Staged& next, auto buffer, auto steady) {
+    constexpr int buf = decltype(buffer)::value;
     constexpr bool kSteady = decltype(steady)::value;
-    const int buf = grp & 1;
     if (kAhead == 0 && (kSteady || grp + 1 < g.G)) load_group(grp + 1, next);  // in flight during the MFMAs below
 
-    // The four 32 x 32 sub-tiles of the quadrant, one after the other: while the matrix core
-    // works on sub-tile t + 1 the vector ALU runs the scale epilogue of sub-tile t.
     v4i fa[W][kGroup / 32], fb[kGroup / 32];
 #pragma unroll
     for (int mi = 0; mi < W; ++mi)
 #pragma unroll
       for (int ks = 0; ks < kGroup / 32; ++ks)
-        fa[mi][ks] = *reinterpret_cast<const v4i*>(&s_a[buf][((wm * W + mi) * 32 + frag_row) * kRowStride + ks * 32 + frag_k]);
+        fa[mi][ks] = *reinterpret_cast<const v4i*>(&s_a[buf][(wm * W + mi) * 32 * kRowStride + frag + ks * 32]);
     auto load_b = [&](int ni) {
 #pragma unroll
       for (int ks = 0; ks < kGroup / 32; ++ks)
-        fb[ks] = *reinterpret_cast<const v4i*>(&s_b[buf][((wn * W + ni) * 32 + frag_row) * kRowStride + ks * 32 + frag_k]);
+        fb[ks] = *reinterpret_cast<const v4i*>(&s_b[buf][(wn * W + ni) * 32 * kRowStride + frag + ks * 32]);
     };
     auto multiply = [&](int mi) {
       v16i d = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -231,12 +224,12 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
     };
     // result register r of a 32 x 32 tile is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
     auto scale_in = [&](const v16i& d, int mi, int ni) {
-      const float sw = s_sw[buf][(wn * W + ni) * 32 + (lane & 31)];
+      const float sw = s_scale[buf][kBM + (wn * W + ni) * 32 + (lane & 31)];
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         // four consecutive rows: one 128-bit LDS read of their activation scales
         const int row = (wm * W + mi) * 32 + 8 * r4 + 4 * (lane >> 5);
-        const u32x4 s4 = MODE == 2 ? u32x4{0, 0, 0, 0} : *reinterpret_cast<const u32x4*>(&s_sx[buf][row]);
+        const u32x4 s4 = MODE == 2 ? u32x4{0, 0, 0, 0} : *reinterpret_cast<const u32x4*>(&s_scale[buf][row]);
         const float sx4[4] = {__builtin_bit_cast(float, s4.x), __builtin_bit_cast(float, s4.y),
                               __builtin_bit_cast(float, s4.z), __builtin_bit_cast(float, s4.w)};
 #pragma unroll
@@ -256,36 +249,45 @@ __global__ __launch_bounds__(kThreads, 2) void wq_gemm_a8_kernel(const GemmArgs 
     };
     load_b(0);
     if constexpr (W == 2) {
+      // All sixteen multiplies of the group first, then the next group's unpacking and LDS stores (its loads
+      // were requested at the top and have had the multiplies to arrive in), then the four epilogues: the LDS
+      // stores are long done when the epilogue reaches the barrier. Measured against the epilogues between the
+      // multiplies and against the stores after the epilogues or before the multiplies: the orders differ by a
+      // few percent, this one is the best on most shapes. The empty instructions pin it: left alone the compiler
+      // arrives at the same order but runs out of registers on the way (32 spilled with int8 weights).
       v16i d0 = multiply(0);
       v16i d1 = multiply(1);
-      scale_in(d0, 0, 0);
       load_b(1);
-      d0 = multiply(0);
+      v16i d2 = multiply(0);
+      v16i d3 = multiply(1);
+      asm volatile("" : "+v"(d0), "+v"(d1), "+v"(d2), "+v"(d3));
+      if (kSteady || grp + 1 < g.G) store_group(std::integral_constant<int, buf ^ 1>{}, next);
+      asm volatile("" : "+v"(d0), "+v"(d1), "+v"(d2), "+v"(d3));
+      scale_in(d0, 0, 0);
       scale_in(d1, 1, 0);
-      d1 = multiply(1);
-      scale_in(d0, 0, 1);
-      scale_in(d1, 1, 1);
+      scale_in(d2, 0, 1);
+      scale_in(d3, 1, 1);
     } else {
       scale_in(multiply(0), 0, 0);
     }
 
-    if (kSteady || grp + 1 < g.G) store_group(buf ^ 1, next);  // nobody reads that buffer any more: see barrier below
-    if (kAhead > 0 && (kSteady || grp + 1 + kAhead < g.G)) load_group(grp + 1 + kAhead, next);
+    if constexpr (W != 2) {
+      if (kSteady || grp + 1 < g.G) store_group(std::integral_constant<int, buf ^ 1>{}, next);  // nobody reads that buffer any more: see barrier below
+      if (kAhead > 0 && (kSteady || grp + 1 + kAhead < g.G)) load_group(grp + 1 + kAhead, next);
+    }
     __syncthreads();
   };
+  // Two groups a trip, one per LDS buffer. Steady state: every group a trip touches exists (the last one is
+  // grp + 1 + 1 + kAhead), so its bodies have no branch around their loads and stores and the compiler waits
+  // for exactly the loads an LDS store needs instead of draining everything in flight.
   int grp = 0;
-  // steady state: every group a round touches exists (the last one is grp + kSets - 1 + 1 + kAhead)
-  if constexpr (kBranchFreeLoop) {
-    for (; grp + kSets + kAhead < g.G; grp += kSets) {
-#pragma unroll
-      for (int a = 0; a < kSets; ++a) iterate(grp + a, st[a], std::true_type{});
-    }
+  for (; grp + 2 + kAhead < g.G; grp += 2) {
+    iterate(grp, st[0], std::integral_constant<int, 0>{}, std::true_type{});
+    iterate(grp + 1, st[kSets - 1], std::integral_constant<int, 1>{}, std::true_type{});
   }
-  for (; grp < g.G; grp += kSets) {
-#pragma unroll
-    for (int a = 0; a < kSets; ++a) {
-      if (grp + a < g.G) iterate(grp + a, st[a], std::false_type{});
-    }
+  for (; grp < g.G; grp += 2) {
+    iterate(grp, st[0], std::integral_constant<int, 0>{}, std::false_type{});
+    if (grp + 1 < g.G) iterate(grp + 1, st[kSets - 1], std::integral_constant<int, 1>{}, std::false_type{});
   }
 
   T* __restrict__ out = static_cast<T*>(g.out);
@@ -312,6 +314,8 @@ template <typename T, int W, int MODE>
 int launch_tile(const GemmArgs& g, int wformat, hipStream_t stream) {
   constexpr int kTile = 64 * W;
   const dim3 grid((g.N + kTile - 1) / kTile, (g.M + kTile - 1) / kTile), block(kThreads);
+  // (the kernel addresses a tile's rows with 32-bit offsets from its first row)
+  if (g.G > (1 << 17)) return llmq_host::fail_invalid("rows of more than 2^24 codes are not supported, got %d groups", g.G);
   if (wformat == LLMQ_W_INT8) {
     hipLaunchKernelGGL((wq_gemm_a8_kernel<T, 8, W, MODE>), grid, block, 0, stream, g);
   } else {

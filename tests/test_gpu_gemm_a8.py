@@ -271,6 +271,14 @@ def test_argument_checks(ext):
     with pytest.raises(RuntimeError, match="group_size 128"):
         ext.wq_gemm_a8(a, torch.ones(4, 4, device="cuda"), torch.zeros(8, 4, 64, dtype=torch.int8, device="cuda"),
                        torch.ones(8, 4, device="cuda"))
+    # the tiled kernels address a tile's rows with 32-bit offsets: rows beyond 2^24 codes are refused, not wrapped
+    import os
+
+    groups = (1 << 17) + 1
+    os.environ["LLMQ_A8_FORM"] = "tile"
+    with pytest.raises(RuntimeError, match="2\\^24 codes"):
+        ext.wq_gemm_a8(torch.zeros(1, groups * 128, dtype=torch.int8, device="cuda"), torch.ones(1, groups, device="cuda"),
+                       torch.zeros(1, groups, 128, dtype=torch.int8, device="cuda"), torch.ones(1, groups, device="cuda"))
 
 
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
