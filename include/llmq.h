@@ -168,7 +168,8 @@ int llmq_dequant_weight(const void* qweight, const float* wscale, void* out, int
  *   out[m, n] = sum over g, in order, of  float(sum_k a[m,g,k]*q[n,g,k]) * sw[sr(n), g] * sx[m, g]
  * each group's term rounded to fp32 after every multiply and added sequentially, then
  * bias (fp32, nullable) added and the sum cast to `dtype`. gs must be 128.
- * a: int8 [M, G*128]; sx: fp32 [M, G]; qweight/wscale as for llmq_wq_gemv. */
+ * a: int8 [M, G*128]; sx: fp32 [M, G]; qweight/wscale as for llmq_wq_gemv. G <= 2^17 (rows of up
+ * to 2^24 codes). */
 int llmq_wq_gemm_a8(const int8_t* a, const float* sx, const void* qweight, const float* wscale,
                     const float* bias_or_null, void* out, int M, int N, int G, int gs,
                     int out_group, int wformat, int dtype, llmq_stream_t stream);
