@@ -178,6 +178,34 @@ def test_rows_longer_than_64_groups(bits, M, n, k):
 
 
 @pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("M", [1, 3])
+@pytest.mark.parametrize("n,k", [(10240, 4096), (12290, 4096), (4120, 14336), (8200, 8192)])
+def test_workgroups_that_walk_unequal_numbers_of_row_tiles(bits, M, n, k):
+    """Outputs of a round and a fraction of the resident workgroups (640 and 769 row tiles on 2 x 256 slots, 258
+    on 256, 513 on 256): where the last round would be at most half full every slot is used and some workgroups
+    walk one tile more than others; the last tile of two of the shapes is ragged. Every output row against the
+    float64 closed form."""
+    from llmquant.hip import load_extension
+
+    gen = torch.Generator().manual_seed(n + bits)
+    width = GROUP if bits == 8 else GROUP // 2
+    q = torch.randint(0, 255, (n, k // GROUP, width), generator=gen, dtype=torch.uint8)
+    scales = torch.rand(n, k // GROUP, generator=gen) * 0.01 + 1e-3
+    x = torch.randn(M, k, generator=gen)
+    codes = q.view(torch.int8).numpy() if bits == 8 else oracle.unpack_int4(q.numpy())
+    got = load_extension().wq_gemv(x.cuda(), (q.view(torch.int8) if bits == 8 else q).cuda(), scales.cuda(), 0)
+    assert got.shape == (M, n)
+    rows = torch.cat([torch.arange(0, 64), torch.randint(0, n, (384,), generator=gen), torch.arange(n - 64, n)])
+    exact = oracle.gemv_float64(to_np(x), codes[rows], to_np(scales[rows]))
+    assert rel_l2(to_np(got[:, rows]), exact) <= 1e-5
+    # (and no row anywhere is left unwritten or written twice with different values: the whole output against a
+    # float64 product on the device)
+    dense = torch.from_numpy(codes.astype("float64")).cuda() * scales.cuda().double()[:, :, None]
+    want = x.cuda().double() @ dense.reshape(n, k).T
+    assert ((got.double() - want).abs().max() / want.abs().max()).item() <= 1e-5
+
+
+@pytest.mark.parametrize("bits", [8, 4])
 def test_many_long_rows(bits):
     """N large enough for the whole-row kernel with rows of 176 groups (22528 values): the staged
     activation no longer fits the default LDS limit, so the launch has to pick a kernel that raises it."""
