@@ -212,6 +212,24 @@ def test_ragged_edges_of_the_large_tile(ext, bits):
     assert np.array_equal(to_np(got)[np.ix_(rows, cols)], want)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("groups", [1, 3, 4, 5, 8, 9])
+def test_large_tile_over_odd_and_even_group_counts(ext, bits, groups):
+    """The large-tile kernel walks two groups a trip (one per LDS buffer) in a steady loop with no branches and
+    finishes in a loop that has them: rows of 1 to 9 groups pass through every combination of the two (none, the
+    tail alone, odd and even remainders) on an output that ends inside a tile, with both weight widths. The whole
+    output must equal the group-parallel kernel's bit for bit, and sampled rows and columns the oracle's."""
+    m, n, k = 2051, 2053, groups * GROUP
+    got, (x, canonical, scales, _) = run_case(ext, m, n, k, bits, torch.bfloat16, seed=groups, form="tile")
+    other, _ = run_case(ext, m, n, k, bits, torch.bfloat16, seed=groups, form="groups")
+    assert torch.equal(got, other)
+    rng = np.random.default_rng(groups)
+    rows = np.unique(np.concatenate([rng.choice(m, 40, replace=False), np.arange(m - 4, m)]))
+    cols = np.unique(np.concatenate([rng.choice(n, 40, replace=False), np.arange(n - 6, n)]))
+    want = oracle.real_linear(to_np(x)[rows], canonical[cols], scales[cols], "bf16", None, 8)
+    assert np.array_equal(to_np(got)[np.ix_(rows, cols)], want)
+
+
 @pytest.mark.parametrize("name", ["W4A8", "W8A8"])
 @pytest.mark.parametrize("layout", [dict(), dict(head_dim=64), dict(out_group=64)])
 @pytest.mark.parametrize("m", [1, 4, 33])
