@@ -61,6 +61,7 @@ def parse():
                     help="skip the legs that report the path's other kernels and end-to-end decode")
     ap.add_argument("--only", choices=("other", "decode", "prefill", "decode8b"), default=None,
                     help="profiling aid: run just that leg and print its JSON (not the bench line)")
+    ap.add_argument("--prompt-tokens", type=int, default=512, help="prompt length of the --only prefill leg")
     ap.add_argument("--copy-probe", action="store_true",
                     help="first run a plain 256 MiB device copy three times: the known-size kernel that "
                          "hardware-counter readings of the sweep are scaled by")
@@ -116,7 +117,7 @@ def main():
     lib = load_capi()
     torch.cuda.set_device(0)
     if opts.only:
-        leg = {"other": other_kernels, "decode": decode_leg, "prefill": prefill_leg,
+        leg = {"other": other_kernels, "decode": decode_leg, "prefill": lambda t: prefill_leg(t, opts.prompt_tokens),
                "decode8b": lambda t: decode_leg(t, arch="llama3-8b")}[opts.only](torch)
         print(json.dumps({opts.only: leg}))
         return
@@ -866,8 +867,8 @@ def token_identity(torch, cfg, recipe, prompt):
     return out
 
 
-def prefill_leg(torch):
-    """The prompt pass of config 5 by itself: twelve 512-token prefills through the kernel runtime on the
+def prefill_leg(torch, prompt=512):
+    """The prompt pass of config 5 by itself: twelve prefills of `prompt` tokens through the kernel runtime on the
     random-init Llama-3.2-1B architecture (attention int8 / MLP int4 / lm_head int8 / int8 KV), wall time
     and HIP events per call. The run to profile for what a time-to-first-token is made of."""
     import time
@@ -885,7 +886,6 @@ def prefill_leg(torch):
     model = LlamaForCausalLM(cfg).to(torch.bfloat16).to("cuda:0").eval()
     oneshot(model, QuantConfig(attn_weight="int8", mlp_weight="int4", head_weight="int8",
                                kv_cache="int8").to_modifier("kernel"))
-    prompt = 512
     ids = torch.randint(0, 128256, (1, prompt), generator=torch.Generator().manual_seed(1)).to("cuda:0")
     wall, gpu, host = [], [], []
     with torch.no_grad():
