@@ -1006,9 +1006,13 @@ int launch_typed(const void* x, const void* qw, const float* ws, void* out, int 
   const int resident = 256 * per_cu;
   int grid;
   if (a.n_tiles >= 4 * resident) {
-    // long streams: twice the resident count, so that a CU always has a workgroup staging its
-    // activation while the others stream (measured on lm_head: 47.5 us against 51.5 us)
+    // long streams: more workgroups than are resident, so that a CU always has a workgroup staging its activation
+    // while the others stream, about two row tiles each (the second one's loads are requested under the first
+    // one's multiplies) and at least twice the resident count. Measured on lm_head, 8016 tiles of K = 2048, 1024
+    // resident: 51.0 us at 1x, 48.2 at 2x, 45.9 at 4x, 45.5 at 6x, 46.2 at 8x; K = 4096, 512 resident: 93.7 at 2x,
+    // 92.4 at 8x; 2048 tiles of K = 4096: 28.2 at 2x, 28.7 at 4x (one tile each), 33.6 at 8x (idle workgroups).
     grid = 2 * resident;
+    if (a.n_tiles / 2 > grid) grid = a.n_tiles / 2;
   } else {
     // Every workgroup the same number of tiles -- unless the last round would be at most half full: then all
     // resident slots are used and some workgroups walk one tile more (measured, K = 4096 int8, 2 x 256 slots:
