@@ -875,7 +875,13 @@ __global__ __launch_bounds__(256, 2) void wq_gemv_mfma_fullk_deep_kernel(const M
 #undef LLMQ_FILL
 }
 
+// The whole-row kernel (a wave owns row tiles, no barrier) takes int4 weights of at least this many row tiles and
+// bytes of codes; below, the K-split kernel's sixteen waves a CU win. Measured, replayed from a graph, whole-row /
+// K-split: K = 2048: 1024 tiles 6.8 / 6.0 us, 3072: 13.5 / 12.4, 4096: 16.5 / 16.8, 8016 (lm_head): 27.4 / 29.9;
+// K = 4096: 1024 tiles 11.5 / 9.7, 1536: 15.7 / 13.3, 2048: 16.6 / 18.1, 8016: 50.5 / 60.8; gate|up pairs with the
+// RMSNorm in front, as a decode step runs them: 8192 pairs of K = 2048 7.3 / 7.1, 14336 pairs of K = 4096 17.9 / 14.6.
 constexpr int kFullKMinTiles = 1024;
+constexpr int64_t kFullKMinBytes = 64ll << 20;
 constexpr int kLdsDefault = 64 * 1024;   // dynamic LDS a kernel may use without opting in
 constexpr int kLdsMax = 160 * 1024;      // LDS of one gfx950 CU
 
@@ -966,13 +972,14 @@ int launch_typed(const void* x, const void* qw, const float* ws, void* out, int 
   a.row_bytes = G * kGroup * BITS / 8;
   // measured on lm_head (8016 row tiles): the barrier-free kernel wins for int4 (27.7 vs 30.7 us),
   // the K-split one for int8 (46.6 vs 49.9 us)
-  // measured (graph replay): int4 lm_head 28.3 -> 27.2 us, 8B lm_head 55.0 -> 53.0, gate|up 9.5 -> 9.1 with four
-  // chunks ahead; for int8 (two chunks ahead fit) the K-split kernel below stays faster
+  // measured (graph replay): int4 lm_head 28.3 -> 27.2 us, 8B lm_head 55.0 -> 53.0 with four chunks ahead; for int8
+  // (two chunks ahead fit) the K-split kernel below stays faster
   constexpr int kDeep = 4;
   // (rows so long that the staged activation exceeds the default LDS limit go to the K-split kernel,
   // whose launch raises the limit)
-  const bool fullk_ok = M == 1 && BITS == 4 && a.n_tiles >= kFullKMinTiles && a.prologue != LLMQ_PRO_ATTN_MERGE &&
-                        LdsLayout(1, G, 0, true).part_off <= kLdsDefault;
+  const bool fullk_ok = M == 1 && BITS == 4 && a.n_tiles >= kFullKMinTiles &&
+                        static_cast<int64_t>(a.n_tiles) * kTileRows * a.row_bytes >= kFullKMinBytes &&
+                        a.prologue != LLMQ_PRO_ATTN_MERGE && LdsLayout(1, G, 0, true).part_off <= kLdsDefault;
   if (fullk_ok && (G / kGW) % kDeep == 0) {
     const LdsLayout L(1, G, 0, BITS == 4);
     auto kernel = wq_gemv_mfma_fullk_deep_kernel<T, BITS, kDeep>;
