@@ -206,6 +206,36 @@ def test_workgroups_that_walk_unequal_numbers_of_row_tiles(bits, M, n, k):
 
 
 @pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("n", [2048, 2043, 1000, 9, 1])
+def test_small_outputs_of_64_group_rows_take_eight_row_tiles(bits, n):
+    """Rows of 8192 values (sixteen waves a workgroup) and at most 128 sixteen-row tiles: the launch uses tiles of
+    eight rows so that every CU gets a workgroup; lanes 8..15 of a tile repeat rows 0..7 and store nothing. Full
+    and ragged outputs (the last tile holding 3, 8, 1 rows) against the float64 closed form, and the rows next to
+    the output in memory untouched."""
+    from llmquant.hip import load_capi
+    import ctypes
+
+    k = 8192
+    gen = torch.Generator().manual_seed(n * 7 + bits)
+    width = GROUP if bits == 8 else GROUP // 2
+    q = torch.randint(0, 255, (n, k // GROUP, width), generator=gen, dtype=torch.uint8)
+    scales = torch.rand(n, k // GROUP, generator=gen) * 0.01 + 1e-3
+    x = torch.randn(1, k, generator=gen)
+    codes = q.view(torch.int8).numpy() if bits == 8 else oracle.unpack_int4(q.numpy())
+    exact = oracle.gemv_float64(to_np(x), codes, to_np(scales))
+    # through the C ABI into the middle of a larger buffer, to see that nothing past the n outputs is written
+    lib = load_capi()
+    out = torch.full((n + 64,), 777.0, device="cuda")
+    xd, qd, sd = x.cuda(), (q.view(torch.int8) if bits == 8 else q).cuda(), scales.cuda()
+    rc = lib.llmq_wq_gemv(xd.data_ptr(), qd.data_ptr(), sd.data_ptr(), out[32:].data_ptr(), 1, n, k // GROUP, GROUP, 0,
+                          bits, 0, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, lib.llmq_last_error()
+    torch.cuda.synchronize()
+    assert rel_l2(to_np(out[32:32 + n].reshape(1, n)), exact) <= 1e-5
+    assert bool((out[:32] == 777.0).all()) and bool((out[32 + n:] == 777.0).all())
+
+
+@pytest.mark.parametrize("bits", [8, 4])
 def test_many_long_rows(bits):
     """N large enough for the whole-row kernel with rows of 176 groups (22528 values): the staged
     activation no longer fits the default LDS limit, so the launch has to pick a kernel that raises it."""
