@@ -1014,6 +1014,11 @@ int launch_typed(const void* x, const void* qw, const float* ws, void* out, int 
   // A workgroup stages the activation once and then walks row tiles, so for mid-sized N the grid
   // is sized to be resident all at once and to give every workgroup the same number of tiles.
   int per_cu = 16 / wk;
+  // With the RMSNorm in front (every workgroup reduces the whole activation row before its first multiply) three
+  // four-wave workgroups a CU do better than four: the gate|up pairs of a decode step, 1024 row tiles of K = 2048
+  // int4, replayed alone: 7.1-7.2 us on 1024 workgroups, 6.95 on 512, 6.75 on 640, 6.35-6.39 on 768, 7.4 on 896; in
+  // the step 1865 -> 1905 tok/s. (int8: 8.9 either way; eight-wave workgroups, K = 4096: two a CU stay best.)
+  if (ops.prologue == LLMQ_PRO_RMSNORM && wk == 4) per_cu = 3;
   const int by_lds = kLdsMax / L.total;
   if (per_cu > by_lds) per_cu = by_lds;
   if (per_cu < 1) per_cu = 1;
