@@ -45,6 +45,7 @@ constexpr int kThreads = 256;
 constexpr int kRowStride = kGroup + 16;  // bytes; padding keeps 16-byte reads off the same banks
 // the group-parallel kernel (exact form) takes outputs of up to this many 32 x 32 tiles per round of 256 of the
 // tiled kernel's 64 x 64 tiles
+constexpr int kLargeTileMin = 300;   // 128 x 128 tiles from this many up (256 CUs)
 constexpr int kGroupsTilesPerRound = 640;
 constexpr int kGroupsTilesOperandOrder = 1100;   // (512 x 4096 x 14336, 2048 tiles: 101 us against 82 tiled)
 
@@ -355,7 +356,7 @@ bool takes_groups(int M, int N, int G, bool operand_order = false) {
 
 template <typename T, int MODE>
 int launch_typed(const GemmArgs& g, int wformat, hipStream_t stream) {
-  // 128 x 128 tiles when there is at least one for every CU, else 64 x 64
+  // 128 x 128 tiles when there are clearly more of them than CUs, else 64 x 64
   const int64_t big_tiles = static_cast<int64_t>((g.N + 127) / 128) * ((g.M + 127) / 128);
   if constexpr (MODE == 0) {
     if (takes_groups(g.M, g.N, g.G)) {
@@ -364,7 +365,9 @@ int launch_typed(const GemmArgs& g, int wformat, hipStream_t stream) {
                                        stream);
     }
   }
-  return big_tiles >= 256 ? launch_tile<T, 2, MODE>(g, wformat, stream) : launch_tile<T, 1, MODE>(g, wformat, stream);
+  // (measured, bit-exact form, int4: 256 large tiles, one a CU: 53.7 us against 48.9 on 64 x 64 tiles at 1024 x 4096 x
+  // 4096 and 52.6 against 47.8 at 512 x 8192 x 4096; 336 large tiles: 61.1 against 68.2; 448: 77.3 against 87.5)
+  return big_tiles >= kLargeTileMin ? launch_tile<T, 2, MODE>(g, wformat, stream) : launch_tile<T, 1, MODE>(g, wformat, stream);
 }
 
 template <int MODE>

@@ -219,7 +219,7 @@ def test_large_tile_over_odd_and_even_group_counts(ext, bits, groups):
     finishes in a loop that has them: rows of 1 to 9 groups pass through every combination of the two (none, the
     tail alone, odd and even remainders) on an output that ends inside a tile, with both weight widths. The whole
     output must equal the group-parallel kernel's bit for bit, and sampled rows and columns the oracle's."""
-    m, n, k = 2051, 2053, groups * GROUP
+    m, n, k = 2051, 2309, groups * GROUP   # 17 x 19 large tiles
     got, (x, canonical, scales, _) = run_case(ext, m, n, k, bits, torch.bfloat16, seed=groups, form="tile")
     other, _ = run_case(ext, m, n, k, bits, torch.bfloat16, seed=groups, form="groups")
     assert torch.equal(got, other)
